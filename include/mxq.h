@@ -1,0 +1,137 @@
+/*
+ * mxq.h - C ABI of libmxq_hip.so: MI355X (gfx950) kernels for MXNet's INT8
+ * quantized-inference operators.
+ *
+ * This is the launcher the C++ FCompute<gpu> host functions call in place of
+ * mshadow's Kernel<OP,gpu>::Launch, broadcast::RTCReduce, cublasGemmEx and
+ * cudnnConvolutionForward.  Every entry point
+ *   - takes plain device pointers, sizes and a raw hipStream_t (as void*; NULL
+ *     is the default stream),
+ *   - only enqueues work on that stream: no allocation, no free, no device or
+ *     stream synchronisation, no retained state,
+ *   - returns 0 on success and -1 on failure with the message available from
+ *     mxq_last_error() on the calling thread (the convention of
+ *     include/mxnet/c_api_error.h:39-58 in the reference).
+ * All pointers named min / max are DEVICE pointers to one float32, exactly as the
+ * reference's min/max TBlobs of shape (1,).
+ *
+ * Reference paths are relative to the apache/mxnet tree.
+ */
+#ifndef MXQ_H_
+#define MXQ_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MXQ_ABI_VERSION 1
+
+/* element type codes = mshadow::TypeFlag (3rdparty/mshadow/mshadow/base.h:351-364) */
+#define MXQ_FLOAT32 0
+#define MXQ_UINT8 3
+#define MXQ_INT32 4
+#define MXQ_INT8 5
+
+/* Last error message of the calling thread ("" if none). */
+const char* mxq_last_error(void);
+int mxq_abi_version(void);
+
+/* ---- _contrib_quantize_v2 ------------------------------------------------
+ * Replaces QuantizeV2Operator<gpu>::Forward for fp32 input
+ * (src/operator/quantization/quantize_v2-inl.h:218-305): the
+ * Kernel<quantize_v2_zero_centered|quantize_v2_unsigned,gpu>::Launch calls and,
+ * when uncalibrated, the two broadcast::RTCReduce passes (min, max) in front
+ * of them.  out_type is MXQ_INT8 or MXQ_UINT8 (the reference's GPU build
+ * refuses uint8, :198-201; here it follows the CPU kernel :66-95 and
+ * saturates where the reference is undefined).  calibrated != 0 uses
+ * (min_calib, max_calib); otherwise the range is reduced on the device in
+ * `workspace` (>= mxq_quantize_v2_workspace(n) bytes, 16-byte aligned) and
+ * never crosses the host. */
+size_t mxq_quantize_v2_workspace(size_t n);
+int mxq_quantize_v2(void* stream, const float* in, void* out, float* omin, float* omax,
+                    size_t n, int out_type, int calibrated, float min_calib, float max_calib,
+                    void* workspace, size_t workspace_bytes);
+
+/* ---- _contrib_quantize (v1) ---------------------------------------------
+ * Replaces QuantizeCompute<gpu> (src/operator/quantization/quantize-inl.h:90-131):
+ * same kernels, the range arrives as two device scalars. */
+int mxq_quantize(void* stream, const float* in, const float* imin, const float* imax, void* out,
+                 float* omin, float* omax, size_t n, int out_type);
+
+/* Identity pass for int8/uint8 input of quantize_v2 (quantize_v2-inl.h:203-216):
+ * copies n bytes and writes the constant ranges. */
+int mxq_quantize_v2_passthrough(void* stream, const void* in, void* out, float* omin,
+                                float* omax, size_t n, int in_type, int calibrated,
+                                float min_calib, float max_calib);
+
+/* ---- _contrib_requantize -------------------------------------------------
+ * Replaces RequantizeForward<gpu> (src/operator/quantization/requantize-inl.h:127-240):
+ * int32 -> int8 with the input range (imin, imax) read from the device;
+ * calibrated uses MaxAbs(min_calib, max_calib), uncalibrated reduces the int32
+ * min and max on the device first (workspace as above). */
+size_t mxq_requantize_workspace(size_t n);
+int mxq_requantize(void* stream, const int32_t* in, const float* imin, const float* imax,
+                   int8_t* out, float* omin, float* omax, size_t n, int calibrated,
+                   float min_calib, float max_calib, void* workspace, size_t workspace_bytes);
+
+/* ---- _contrib_dequantize -------------------------------------------------
+ * Replaces DequantizeOperator<gpu>::Forward
+ * (src/operator/quantization/dequantize-inl.h:115-144); in_type MXQ_INT8 or
+ * MXQ_UINT8. */
+int mxq_dequantize(void* stream, const void* in, int in_type, const float* imin,
+                   const float* imax, float* out, size_t n);
+
+/* ---- _contrib_quantized_fully_connected ----------------------------------
+ * Replaces QuantizedFullyConnectedForwardGPU
+ * (src/operator/quantization/quantized_fully_connected.cu:58-138): cublasGemmEx
+ * (s8 x s8 -> s32, data [M,K] row-major, weight [N,K] row-major), the
+ * QuantizationRangeForS8S8MultiplicationStruct launch and QuantizedBiasAddKernel.
+ * The bias is added exactly, as the CPU operator does
+ * (quantized_fully_connected.cc:149-174: the int8 bias is rescaled to int32 once
+ * and summed in integers), not through the GPU kernel's float round trip.
+ *   bias        int8 [N] or NULL (then min_bias/max_bias are ignored)
+ *   out32       int32 [M,N] or NULL
+ *   omin, omax  output range (always written)
+ *   out8        int8 [M,N] or NULL: fused _contrib_requantize of the
+ *               accumulator with the calibrated range (min_calib, max_calib),
+ *               bit-identical to mxq_requantize on out32; relu != 0 clamps the
+ *               int8 at zero; rmin/rmax receive the requantized range.
+ * At least one of out32 / out8 must be given. */
+int mxq_quantized_fc(void* stream, const int8_t* data, const int8_t* weight, const int8_t* bias,
+                     int M, int N, int K, const float* min_data, const float* max_data,
+                     const float* min_weight, const float* max_weight, const float* min_bias,
+                     const float* max_bias, int32_t* out32, float* omin, float* omax,
+                     int8_t* out8, float* rmin, float* rmax, int relu, float min_calib,
+                     float max_calib);
+
+/* ---- _contrib_quantized_conv ----------------------------------------------
+ * Replaces QuantizedCuDNNConvOp::Forward
+ * (src/operator/quantization/quantized_conv.cu:101-219): the NHWC int8
+ * cudnnConvolutionForward, the float->int32 cast, the range kernel and the bias
+ * kernel.  Operands are NHWC here (data [N,H,W,C], weight [O,KH,KW,C], output
+ * [N,OH,OW,O]); the layout adapters below replace the three TransposeImpl calls
+ * (:147-148,183) for callers holding the operator's NCHW tensors.  Epilogue
+ * arguments as for mxq_quantized_fc. */
+int mxq_quantized_conv_nhwc(void* stream, const int8_t* data, const int8_t* weight,
+                            const int8_t* bias, int N, int H, int W, int C, int O, int KH,
+                            int KW, int stride_h, int stride_w, int pad_h, int pad_w,
+                            int dilate_h, int dilate_w, const float* min_data,
+                            const float* max_data, const float* min_weight,
+                            const float* max_weight, const float* min_bias,
+                            const float* max_bias, int32_t* out32, float* omin, float* omax,
+                            int8_t* out8, float* rmin, float* rmax, int relu, float min_calib,
+                            float max_calib);
+
+/* [N,C,H,W] int8 -> [N,H,W,C] int8 (also OIHW -> OHWI for the weight). */
+int mxq_nchw_to_nhwc_i8(void* stream, const int8_t* in, int8_t* out, int N, int C, int H, int W);
+/* [N,H,W,C] -> [N,C,H,W]; elem_bytes 1 (int8) or 4 (int32). */
+int mxq_nhwc_to_nchw(void* stream, const void* in, void* out, int N, int C, int H, int W,
+                     int elem_bytes);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MXQ_H_ */

@@ -1,0 +1,154 @@
+"""Thin torch-tensor wrappers over the C ABI (one function per entry point).
+Tensors must be contiguous CUDA(HIP) tensors; outputs are allocated with torch
+and the calls are enqueued on torch's current stream."""
+import ctypes
+
+import torch
+
+from . import _lib
+from ._lib import INT8, UINT8, check, lib
+
+_TYPE_CODE = {torch.int8: INT8, torch.uint8: UINT8}
+
+
+def _stream():
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _ptr(t):
+    if t is None:
+        return None
+    assert t.is_cuda and t.is_contiguous(), "need a contiguous device tensor"
+    return ctypes.c_void_p(t.data_ptr())
+
+
+def _scalar(dev):
+    return torch.empty(1, dtype=torch.float32, device=dev)
+
+
+def _workspace(nbytes, dev):
+    return torch.empty(nbytes, dtype=torch.uint8, device=dev)
+
+
+def quantize_v2(data, out_type="int8", min_calib_range=None, max_calib_range=None):
+    assert data.dtype == torch.float32
+    calibrated = min_calib_range is not None and max_calib_range is not None
+    if out_type == "auto":
+        out_type = "uint8" if (calibrated and min_calib_range >= 0.0) else "int8"
+    dt = {"int8": torch.int8, "uint8": torch.uint8}[out_type]
+    out = torch.empty(data.shape, dtype=dt, device=data.device)
+    omin, omax = _scalar(data.device), _scalar(data.device)
+    n = data.numel()
+    ws = None
+    wsb = 0
+    if not calibrated:
+        wsb = lib.mxq_quantize_v2_workspace(n)
+        ws = _workspace(wsb, data.device)
+    check(lib.mxq_quantize_v2(_stream(), _ptr(data), _ptr(out), _ptr(omin), _ptr(omax), n,
+                              _TYPE_CODE[dt], int(calibrated),
+                              float(min_calib_range or 0.0), float(max_calib_range or 0.0),
+                              _ptr(ws), wsb))
+    return out, omin, omax
+
+
+def quantize(data, min_range, max_range, out_type="int8"):
+    assert data.dtype == torch.float32
+    dt = {"int8": torch.int8, "uint8": torch.uint8}[out_type]
+    out = torch.empty(data.shape, dtype=dt, device=data.device)
+    omin, omax = _scalar(data.device), _scalar(data.device)
+    check(lib.mxq_quantize(_stream(), _ptr(data), _ptr(min_range), _ptr(max_range), _ptr(out),
+                           _ptr(omin), _ptr(omax), data.numel(), _TYPE_CODE[dt]))
+    return out, omin, omax
+
+
+def requantize(data, min_range, max_range, min_calib_range=None, max_calib_range=None):
+    assert data.dtype == torch.int32
+    calibrated = min_calib_range is not None and max_calib_range is not None
+    out = torch.empty(data.shape, dtype=torch.int8, device=data.device)
+    omin, omax = _scalar(data.device), _scalar(data.device)
+    n = data.numel()
+    ws = None
+    wsb = 0
+    if not calibrated:
+        wsb = lib.mxq_requantize_workspace(n)
+        ws = _workspace(wsb, data.device)
+    check(lib.mxq_requantize(_stream(), _ptr(data), _ptr(min_range), _ptr(max_range), _ptr(out),
+                             _ptr(omin), _ptr(omax), n, int(calibrated),
+                             float(min_calib_range or 0.0), float(max_calib_range or 0.0),
+                             _ptr(ws), wsb))
+    return out, omin, omax
+
+
+def dequantize(data, min_range, max_range):
+    out = torch.empty(data.shape, dtype=torch.float32, device=data.device)
+    check(lib.mxq_dequantize(_stream(), _ptr(data), _TYPE_CODE[data.dtype], _ptr(min_range),
+                             _ptr(max_range), _ptr(out), data.numel()))
+    return out
+
+
+def quantized_fc(data, weight, bias, min_data, max_data, min_weight, max_weight, min_bias=None,
+                 max_bias=None, want_int32=True, calib=None, relu=False):
+    """data int8 [M,K], weight int8 [N,K], bias int8 [N] or None.
+    Returns dict(out32, omin, omax[, out8, rmin, rmax])."""
+    M, K = data.shape
+    N, K2 = weight.shape
+    assert K == K2
+    dev = data.device
+    res = {"omin": _scalar(dev), "omax": _scalar(dev)}
+    out32 = torch.empty((M, N), dtype=torch.int32, device=dev) if want_int32 else None
+    out8 = rmin = rmax = None
+    lo = hi = 0.0
+    if calib is not None:
+        out8 = torch.empty((M, N), dtype=torch.int8, device=dev)
+        rmin, rmax = _scalar(dev), _scalar(dev)
+        lo, hi = float(calib[0]), float(calib[1])
+    check(lib.mxq_quantized_fc(_stream(), _ptr(data), _ptr(weight), _ptr(bias), M, N, K,
+                               _ptr(min_data), _ptr(max_data), _ptr(min_weight),
+                               _ptr(max_weight), _ptr(min_bias), _ptr(max_bias), _ptr(out32),
+                               _ptr(res["omin"]), _ptr(res["omax"]), _ptr(out8), _ptr(rmin),
+                               _ptr(rmax), int(relu), lo, hi))
+    res.update(out32=out32, out8=out8, rmin=rmin, rmax=rmax)
+    return res
+
+
+def quantized_conv_nhwc(data, weight, bias, min_data, max_data, min_weight, max_weight,
+                        min_bias=None, max_bias=None, stride=(1, 1), pad=(0, 0), dilate=(1, 1),
+                        want_int32=True, calib=None, relu=False):
+    """data int8 [N,H,W,C], weight int8 [O,KH,KW,C] -> out [N,OH,OW,O]."""
+    N, H, W, C = data.shape
+    O, KH, KW, C2 = weight.shape
+    assert C == C2
+    OH = (H + 2 * pad[0] - (dilate[0] * (KH - 1) + 1)) // stride[0] + 1
+    OW = (W + 2 * pad[1] - (dilate[1] * (KW - 1) + 1)) // stride[1] + 1
+    dev = data.device
+    res = {"omin": _scalar(dev), "omax": _scalar(dev)}
+    out32 = torch.empty((N, OH, OW, O), dtype=torch.int32, device=dev) if want_int32 else None
+    out8 = rmin = rmax = None
+    lo = hi = 0.0
+    if calib is not None:
+        out8 = torch.empty((N, OH, OW, O), dtype=torch.int8, device=dev)
+        rmin, rmax = _scalar(dev), _scalar(dev)
+        lo, hi = float(calib[0]), float(calib[1])
+    check(lib.mxq_quantized_conv_nhwc(_stream(), _ptr(data), _ptr(weight), _ptr(bias), N, H, W,
+                                      C, O, KH, KW, stride[0], stride[1], pad[0], pad[1],
+                                      dilate[0], dilate[1], _ptr(min_data), _ptr(max_data),
+                                      _ptr(min_weight), _ptr(max_weight), _ptr(min_bias),
+                                      _ptr(max_bias), _ptr(out32), _ptr(res["omin"]),
+                                      _ptr(res["omax"]), _ptr(out8), _ptr(rmin), _ptr(rmax),
+                                      int(relu), lo, hi))
+    res.update(out32=out32, out8=out8, rmin=rmin, rmax=rmax)
+    return res
+
+
+def nchw_to_nhwc_i8(x):
+    N, C, H, W = x.shape
+    out = torch.empty((N, H, W, C), dtype=torch.int8, device=x.device)
+    check(lib.mxq_nchw_to_nhwc_i8(_stream(), _ptr(x), _ptr(out), N, C, H, W))
+    return out
+
+
+def nhwc_to_nchw(x):
+    N, H, W, C = x.shape
+    out = torch.empty((N, C, H, W), dtype=x.dtype, device=x.device)
+    check(lib.mxq_nhwc_to_nchw(_stream(), _ptr(x), _ptr(out), N, C, H, W, x.element_size()))
+    return out

@@ -1,0 +1,714 @@
+// Bandwidth-bound kernels of the INT8 path for gfx950: quantize (v1/v2),
+// requantize, dequantize, and the single-pass min/max grid reduction the
+// uncalibrated variants need.
+//
+// Arithmetic contract (bit-exact with the reference's native CPU kernels):
+// every float operation below is one correctly rounded binary32 operation in
+// the order the reference writes it; this file is compiled with
+// -ffp-contract=off so no multiply-add is fused, and divisions are IEEE.
+//   int8 :  R = max(|lo|,|hi|); s = 127.f / R; q = trunc(sign(x) * min(|x|*s + 0.5f, 127.f))
+//           (quantization_utils.h:83-89, quantize_v2-inl.h:98-114)
+//   uint8:  s = float(255.0 / double(hi - lo)); q = trunc(double((x - lo) * s) + 0.5)
+//           (quantize_v2-inl.h:66-81; saturated to [0,255] where the reference is undefined)
+//   requantize: f = float(q32) * (max(|imin|,|imax|) / 2^31), then the int8 rule
+//           (quantization_utils.h:91-97, requantize-inl.h:89-125)
+//   dequantize: int8 y = float(q) * (max(|hi|,|lo|) / 127.f)
+//               uint8 y = float(q) * ((hi - lo) / 255.f) + lo   (dequantize-inl.h:49-75)
+//
+// Memory access pattern: a wave reads 1 KiB contiguous per load instruction
+// (lane i owns bytes 16i..16i+15), UNROLL such segments are in flight per
+// lane, loads and stores are non-temporal (the tensors are streamed once).
+#include <hip/hip_runtime.h>
+
+#include <cmath>
+#include <cstdint>
+
+#include "../../include/mxq.h"
+#include "mxq_common.h"
+
+namespace mxq {
+
+int g_cast_blocks_per_cu = 8;  // tunable through mxq_set_tuning("cast_blocks_per_cu", v)
+
+namespace {
+
+typedef float f4 __attribute__((ext_vector_type(4)));
+typedef int i4 __attribute__((ext_vector_type(4)));
+
+constexpr int kThreads = 256;
+constexpr int kUnroll = 4;             // 16-byte segments in flight per lane
+constexpr int kMaxReduceBlocks = 2048;  // partials held in the workspace
+constexpr size_t kWsHeader = 64;        // [0] lo, [4] hi, [16] ticket counter
+constexpr size_t kWsBytes = kWsHeader + size_t(kMaxReduceBlocks) * 8;
+
+__device__ __forceinline__ float maxabs(float a, float b) {
+  float x = fabsf(a), y = fabsf(b);
+  return (x < y) ? y : x;
+}
+
+template <typename T>
+__device__ __forceinline__ T nt_load(const T* p) {
+  return __builtin_nontemporal_load(p);
+}
+template <typename T>
+__device__ __forceinline__ void nt_store(T v, T* p) {
+  __builtin_nontemporal_store(v, p);
+}
+
+// ---- per-element rules -------------------------------------------------------
+
+// trunc(sign(x) * min(|x| * s + 0.5f, 127.f)); v >= 0.5 so the sign can be
+// applied after the truncation.
+__device__ __forceinline__ int quant_i8(float x, float s) {
+  float t = fabsf(x) * s;
+  float u = t + 0.5f;
+  float v = (127.0f < u) ? 127.0f : u;
+  int iv = static_cast<int>(v);
+  return (x < 0.0f) ? -iv : ((x > 0.0f) ? iv : 0);
+}
+
+__device__ __forceinline__ int quant_u8(float x, float lo, float s) {
+  float t = (x - lo) * s;
+  double u = static_cast<double>(t) + 0.5;
+  u = (u > 0.0) ? u : 0.0;
+  u = (u > 255.0) ? 255.0 : u;
+  return static_cast<int>(u);
+}
+
+__device__ __forceinline__ uint32_t pack4(int a, int b, int c, int d) {
+  return (uint32_t(a) & 0xffu) | ((uint32_t(b) & 0xffu) << 8) | ((uint32_t(c) & 0xffu) << 16) |
+         (uint32_t(d) << 24);
+}
+
+struct QuantI8 {
+  float s;
+  __device__ __forceinline__ int operator()(float x) const { return quant_i8(x, s); }
+};
+struct QuantU8 {
+  float lo, s;
+  __device__ __forceinline__ int operator()(float x) const { return quant_u8(x, lo, s); }
+};
+
+__device__ __forceinline__ float to_float(float x) { return x; }
+__device__ __forceinline__ float to_float(int32_t x) { return static_cast<float>(x); }
+
+// ---- 4-byte source -> 1-byte destination streaming body ---------------------
+// SrcT is float (quantize) or int32_t (requantize; pre scales the converted
+// value).  Each lane converts 4 consecutive elements per segment and stores one
+// dword; a wave reads 1 KiB and writes 256 B contiguous per segment.
+template <typename SrcT, typename Rule, bool PRE>
+__device__ __forceinline__ void narrow_stream(const SrcT* __restrict__ in,
+                                              uint8_t* __restrict__ out, size_t n, Rule rule,
+                                              float pre) {
+  typedef SrcT Vec4 __attribute__((ext_vector_type(4)));
+  const size_t nquad = n >> 2;  // groups of 4 elements
+  const Vec4* in4 = reinterpret_cast<const Vec4*>(in);
+  uint32_t* out4 = reinterpret_cast<uint32_t*>(out);
+  const size_t stride = size_t(gridDim.x) * kThreads;
+  size_t q = size_t(blockIdx.x) * kThreads + threadIdx.x;
+  // main loop: kUnroll segments, each `stride` quads apart
+  for (; q + size_t(kUnroll - 1) * stride < nquad; q += size_t(kUnroll) * stride) {
+    Vec4 x[kUnroll];
+#pragma unroll
+    for (int j = 0; j < kUnroll; ++j) x[j] = nt_load(in4 + q + size_t(j) * stride);
+#pragma unroll
+    for (int j = 0; j < kUnroll; ++j) {
+      float f0 = to_float(x[j].x), f1 = to_float(x[j].y), f2 = to_float(x[j].z),
+            f3 = to_float(x[j].w);
+      if (PRE) {
+        f0 = f0 * pre;
+        f1 = f1 * pre;
+        f2 = f2 * pre;
+        f3 = f3 * pre;
+      }
+      nt_store(pack4(rule(f0), rule(f1), rule(f2), rule(f3)), out4 + q + size_t(j) * stride);
+    }
+  }
+  for (; q < nquad; q += stride) {
+    Vec4 x = nt_load(in4 + q);
+    float f0 = to_float(x.x), f1 = to_float(x.y), f2 = to_float(x.z), f3 = to_float(x.w);
+    if (PRE) {
+      f0 = f0 * pre;
+      f1 = f1 * pre;
+      f2 = f2 * pre;
+      f3 = f3 * pre;
+    }
+    nt_store(pack4(rule(f0), rule(f1), rule(f2), rule(f3)), out4 + q);
+  }
+  // ragged tail (< 4 elements)
+  if (blockIdx.x == 0) {
+    size_t i = (nquad << 2) + threadIdx.x;
+    if (i < n) {
+      float f = to_float(in[i]);
+      if (PRE) f = f * pre;
+      out[i] = static_cast<uint8_t>(rule(f));
+    }
+  }
+}
+
+// Scalar fallback for pointers that are not 16-byte (source) / 4-byte
+// (destination) aligned.
+template <typename SrcT, typename Rule, bool PRE>
+__device__ __forceinline__ void narrow_scalar(const SrcT* __restrict__ in,
+                                              uint8_t* __restrict__ out, size_t n, Rule rule,
+                                              float pre) {
+  const size_t stride = size_t(gridDim.x) * kThreads;
+  for (size_t i = size_t(blockIdx.x) * kThreads + threadIdx.x; i < n; i += stride) {
+    float f = to_float(in[i]);
+    if (PRE) f = f * pre;
+    out[i] = static_cast<uint8_t>(rule(f));
+  }
+}
+
+// ---- quantize kernels ----------------------------------------------------------
+// The range is (lo, hi) by value, or read from two device scalars when dlo != NULL
+// (v1 operator inputs, or the reduced range in the workspace).
+template <bool UNSIGNED, bool VEC>
+__global__ __launch_bounds__(kThreads) void quantize_kernel(const float* __restrict__ in,
+                                                            uint8_t* __restrict__ out,
+                                                            float* __restrict__ omin,
+                                                            float* __restrict__ omax, size_t n,
+                                                            float lo, float hi,
+                                                            const float* __restrict__ dlo,
+                                                            const float* __restrict__ dhi) {
+  if (dlo != nullptr) {
+    lo = *dlo;
+    hi = *dhi;
+  }
+  if (UNSIGNED) {
+    QuantU8 rule;
+    rule.lo = lo;
+    rule.s = static_cast<float>((255.0 - 0.0) / static_cast<double>(hi - lo));
+    if (VEC)
+      narrow_stream<float, QuantU8, false>(in, out, n, rule, 0.f);
+    else
+      narrow_scalar<float, QuantU8, false>(in, out, n, rule, 0.f);
+    if (blockIdx.x == 0 && threadIdx.x == 0) {
+      *omin = lo;
+      *omax = hi;
+    }
+  } else {
+    const float r = maxabs(lo, hi);
+    QuantI8 rule;
+    rule.s = 127.0f / r;
+    if (VEC)
+      narrow_stream<float, QuantI8, false>(in, out, n, rule, 0.f);
+    else
+      narrow_scalar<float, QuantI8, false>(in, out, n, rule, 0.f);
+    if (blockIdx.x == 0 && threadIdx.x == 0) {
+      *omin = -r;
+      *omax = r;
+    }
+  }
+}
+
+// ---- requantize kernel -------------------------------------------------------
+// real range: by value (calibrated), or MaxAbs of two device scalars (the float
+// images of the int32 min and max left in the workspace by the reduction).
+template <bool VEC>
+__global__ __launch_bounds__(kThreads) void requantize_kernel(
+    const int32_t* __restrict__ in, uint8_t* __restrict__ out, float* __restrict__ omin,
+    float* __restrict__ omax, size_t n, const float* __restrict__ imin,
+    const float* __restrict__ imax, float real_range, const float* __restrict__ dlo,
+    const float* __restrict__ dhi) {
+  if (dlo != nullptr) real_range = maxabs(*dlo, *dhi);
+  const float in_scale = maxabs(*imin, *imax) / 2147483648.0f;
+  QuantI8 rule;
+  rule.s = 127.0f / maxabs(-real_range, real_range);
+  if (VEC)
+    narrow_stream<int32_t, QuantI8, true>(in, out, n, rule, in_scale);
+  else
+    narrow_scalar<int32_t, QuantI8, true>(in, out, n, rule, in_scale);
+  if (blockIdx.x == 0 && threadIdx.x == 0) {
+    *omin = -real_range;
+    *omax = real_range;
+  }
+}
+
+// ---- dequantize kernel ---------------------------------------------------------
+// Each lane reads one dword (4 quantized values) and writes one f4 per
+// segment: a wave reads 256 B and writes 1 KiB contiguous per instruction.
+template <bool UNSIGNED, bool VEC>
+__global__ __launch_bounds__(kThreads) void dequantize_kernel(const uint8_t* __restrict__ in,
+                                                              float* __restrict__ out, size_t n,
+                                                              const float* __restrict__ imin,
+                                                              const float* __restrict__ imax) {
+  const float lo = *imin, hi = *imax;
+  const float scale = UNSIGNED ? (hi - lo) / (255.0f - 0.0f) : maxabs(hi, lo) / 127.0f;
+  auto conv = [&](uint32_t byte) -> float {
+    if (UNSIGNED) {
+      float p = static_cast<float>(byte) * scale;
+      return p + lo;
+    } else {
+      return static_cast<float>(static_cast<int>(static_cast<int8_t>(byte))) * scale;
+    }
+  };
+  const size_t stride = size_t(gridDim.x) * kThreads;
+  if (VEC) {
+    const size_t nquad = n >> 2;
+    const uint32_t* in4 = reinterpret_cast<const uint32_t*>(in);
+    f4* out4 = reinterpret_cast<f4*>(out);
+    size_t q = size_t(blockIdx.x) * kThreads + threadIdx.x;
+    for (; q + size_t(kUnroll - 1) * stride < nquad; q += size_t(kUnroll) * stride) {
+      uint32_t w[kUnroll];
+#pragma unroll
+      for (int j = 0; j < kUnroll; ++j) w[j] = nt_load(in4 + q + size_t(j) * stride);
+#pragma unroll
+      for (int j = 0; j < kUnroll; ++j) {
+        f4 y;
+        y.x = conv(w[j] & 0xffu);
+        y.y = conv((w[j] >> 8) & 0xffu);
+        y.z = conv((w[j] >> 16) & 0xffu);
+        y.w = conv(w[j] >> 24);
+        nt_store(y, out4 + q + size_t(j) * stride);
+      }
+    }
+    for (; q < nquad; q += stride) {
+      uint32_t w = nt_load(in4 + q);
+      f4 y;
+      y.x = conv(w & 0xffu);
+      y.y = conv((w >> 8) & 0xffu);
+      y.z = conv((w >> 16) & 0xffu);
+      y.w = conv(w >> 24);
+      nt_store(y, out4 + q);
+    }
+    if (blockIdx.x == 0) {
+      size_t i = (nquad << 2) + threadIdx.x;
+      if (i < n) out[i] = conv(in[i]);
+    }
+  } else {
+    for (size_t i = size_t(blockIdx.x) * kThreads + threadIdx.x; i < n; i += stride)
+      out[i] = conv(in[i]);
+  }
+}
+
+// ---- single-pass min/max grid reduction -----------------------------------------
+// Wave64 reduction: DPP within each row of 16 lanes, then two cross-row
+// exchanges.  Afterwards every lane holds the wave's result.
+template <typename T, typename Op>
+__device__ __forceinline__ T wave_reduce(T v, Op op) {
+  static_assert(sizeof(T) == 4, "32-bit payload");
+  auto dpp = [](T x, auto ctrl) -> T {
+    int xi = __builtin_bit_cast(int, x);
+    int r = __builtin_amdgcn_update_dpp(xi, xi, decltype(ctrl)::value, 0xf, 0xf, false);
+    return __builtin_bit_cast(T, r);
+  };
+  v = op(v, dpp(v, std::integral_constant<int, 0xB1>{}));   // quad_perm [1,0,3,2]
+  v = op(v, dpp(v, std::integral_constant<int, 0x4E>{}));   // quad_perm [2,3,0,1]
+  v = op(v, dpp(v, std::integral_constant<int, 0x141>{}));  // row_half_mirror
+  v = op(v, dpp(v, std::integral_constant<int, 0x140>{}));  // row_mirror
+  v = op(v, __shfl_xor(v, 16, 64));
+  v = op(v, __shfl_xor(v, 32, 64));
+  return v;
+}
+
+struct MinF {
+  __device__ __forceinline__ float operator()(float a, float b) const { return fminf(a, b); }
+};
+struct MaxF {
+  __device__ __forceinline__ float operator()(float a, float b) const { return fmaxf(a, b); }
+};
+struct MinI {
+  __device__ __forceinline__ int operator()(int a, int b) const { return a < b ? a : b; }
+};
+struct MaxI {
+  __device__ __forceinline__ int operator()(int a, int b) const { return a > b ? a : b; }
+};
+struct MaxU {
+  __device__ __forceinline__ uint32_t operator()(uint32_t a, uint32_t b) const {
+    return a > b ? a : b;
+  }
+};
+
+
+// Shared finalisation: block partial -> workspace, ticket, last block folds all
+// partials.  Returns true in the last block with (mn, mx) holding the global
+// result in every thread of wave 0.
+template <typename T, typename MinOp, typename MaxOp>
+__device__ __forceinline__ bool grid_finish(T& mn, T& mx, T* partial, unsigned* counter,
+                                            T init_min, T init_max) {
+  __shared__ T s_min[kThreads / 64], s_max[kThreads / 64];
+  __shared__ bool s_last;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  mn = wave_reduce(mn, MinOp());
+  mx = wave_reduce(mx, MaxOp());
+  if (lane == 0) {
+    s_min[wave] = mn;
+    s_max[wave] = mx;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int w = 1; w < kThreads / 64; ++w) {
+      mn = MinOp()(mn, s_min[w]);
+      mx = MaxOp()(mx, s_max[w]);
+    }
+    partial[2 * blockIdx.x] = mn;
+    partial[2 * blockIdx.x + 1] = mx;
+    __threadfence();  // release the partial before taking the ticket
+    unsigned t = atomicAdd(counter, 1u);
+    s_last = (t == gridDim.x - 1);
+  }
+  __syncthreads();
+  if (!s_last) return false;
+  __threadfence();  // acquire the other blocks' partials
+  mn = init_min;
+  mx = init_max;
+  for (unsigned b = threadIdx.x; b < gridDim.x; b += kThreads) {
+    mn = MinOp()(mn, __hip_atomic_load(&partial[2 * b], __ATOMIC_RELAXED,
+                                       __HIP_MEMORY_SCOPE_AGENT));
+    mx = MaxOp()(mx, __hip_atomic_load(&partial[2 * b + 1], __ATOMIC_RELAXED,
+                                       __HIP_MEMORY_SCOPE_AGENT));
+  }
+  mn = wave_reduce(mn, MinOp());
+  mx = wave_reduce(mx, MaxOp());
+  __syncthreads();
+  if (lane == 0) {
+    s_min[wave] = mn;
+    s_max[wave] = mx;
+  }
+  __syncthreads();
+  mn = s_min[0];
+  mx = s_max[0];
+  for (int w = 1; w < kThreads / 64; ++w) {
+    mn = MinOp()(mn, s_min[w]);
+    mx = MaxOp()(mx, s_max[w]);
+  }
+  return true;
+}
+
+// fp32 min / max, NaN-propagating like mshadow's red::minimum / red::maximum
+// (3rdparty/mshadow/mshadow/base.h:1054-1115): any NaN makes both results NaN.
+// NaN is detected through the largest |x| bit pattern.
+template <bool VEC>
+__global__ __launch_bounds__(kThreads) void minmax_f32_kernel(const float* __restrict__ in,
+                                                              size_t n, float* ws_range,
+                                                              unsigned* counter,
+                                                              float* partial) {
+  float mn = INFINITY, mx = -INFINITY;
+  uint32_t amax = 0;
+  auto fold = [&](float x) {
+    mn = fminf(mn, x);
+    mx = fmaxf(mx, x);
+    uint32_t a = __builtin_bit_cast(uint32_t, x) & 0x7fffffffu;
+    amax = a > amax ? a : amax;
+  };
+  const size_t stride = size_t(gridDim.x) * kThreads;
+  if (VEC) {
+    const size_t nquad = n >> 2;
+    const f4* in4 = reinterpret_cast<const f4*>(in);
+    size_t q = size_t(blockIdx.x) * kThreads + threadIdx.x;
+    for (; q + size_t(kUnroll - 1) * stride < nquad; q += size_t(kUnroll) * stride) {
+      f4 x[kUnroll];
+#pragma unroll
+      for (int j = 0; j < kUnroll; ++j) x[j] = nt_load(in4 + q + size_t(j) * stride);
+#pragma unroll
+      for (int j = 0; j < kUnroll; ++j) {
+        fold(x[j].x);
+        fold(x[j].y);
+        fold(x[j].z);
+        fold(x[j].w);
+      }
+    }
+    for (; q < nquad; q += stride) {
+      f4 x = nt_load(in4 + q);
+      fold(x.x);
+      fold(x.y);
+      fold(x.z);
+      fold(x.w);
+    }
+    if (blockIdx.x == 0) {
+      size_t i = (nquad << 2) + threadIdx.x;
+      if (i < n) fold(in[i]);
+    }
+  } else {
+    for (size_t i = size_t(blockIdx.x) * kThreads + threadIdx.x; i < n; i += stride) fold(in[i]);
+  }
+  // A block that saw a NaN raises the flag word next to the ticket counter
+  // before it takes its ticket (same thread, ordered by the fence in
+  // grid_finish), so the last block observes it.
+  amax = wave_reduce(amax, MaxU());
+  if ((threadIdx.x & 63) == 0 && amax > 0x7f800000u) atomicOr(counter + 1, 1u);
+  __syncthreads();
+  if (grid_finish<float, MinF, MaxF>(mn, mx, partial, counter, INFINITY, -INFINITY)) {
+    if (threadIdx.x == 0) {
+      unsigned nanflag = __hip_atomic_load(counter + 1, __ATOMIC_RELAXED,
+                                           __HIP_MEMORY_SCOPE_AGENT);
+      if (nanflag) {
+        mn = NAN;
+        mx = NAN;
+      }
+      ws_range[0] = mn;
+      ws_range[1] = mx;
+    }
+  }
+}
+
+// int32 min / max; the last block converts both to their float images with the
+// input scale (QuantizedToFloatStruct, requantize-inl.h:192-227).
+template <bool VEC>
+__global__ __launch_bounds__(kThreads) void minmax_i32_kernel(const int32_t* __restrict__ in,
+                                                              size_t n,
+                                                              const float* __restrict__ imin,
+                                                              const float* __restrict__ imax,
+                                                              float* ws_range, unsigned* counter,
+                                                              int* partial) {
+  int mn = INT32_MAX, mx = INT32_MIN;
+  auto fold = [&](int x) {
+    mn = x < mn ? x : mn;
+    mx = x > mx ? x : mx;
+  };
+  const size_t stride = size_t(gridDim.x) * kThreads;
+  if (VEC) {
+    const size_t nquad = n >> 2;
+    const i4* in4 = reinterpret_cast<const i4*>(in);
+    size_t q = size_t(blockIdx.x) * kThreads + threadIdx.x;
+    for (; q + size_t(kUnroll - 1) * stride < nquad; q += size_t(kUnroll) * stride) {
+      i4 x[kUnroll];
+#pragma unroll
+      for (int j = 0; j < kUnroll; ++j) x[j] = nt_load(in4 + q + size_t(j) * stride);
+#pragma unroll
+      for (int j = 0; j < kUnroll; ++j) {
+        fold(x[j].x);
+        fold(x[j].y);
+        fold(x[j].z);
+        fold(x[j].w);
+      }
+    }
+    for (; q < nquad; q += stride) {
+      i4 x = nt_load(in4 + q);
+      fold(x.x);
+      fold(x.y);
+      fold(x.z);
+      fold(x.w);
+    }
+    if (blockIdx.x == 0) {
+      size_t i = (nquad << 2) + threadIdx.x;
+      if (i < n) fold(in[i]);
+    }
+  } else {
+    for (size_t i = size_t(blockIdx.x) * kThreads + threadIdx.x; i < n; i += stride) fold(in[i]);
+  }
+  if (grid_finish<int, MinI, MaxI>(mn, mx, partial, counter, INT32_MAX, INT32_MIN)) {
+    if (threadIdx.x == 0) {
+      const float scale = maxabs(*imin, *imax) / 2147483648.0f;
+      ws_range[0] = static_cast<float>(mn) * scale;
+      ws_range[1] = static_cast<float>(mx) * scale;
+    }
+  }
+}
+
+__global__ void passthrough_range_kernel(float* omin, float* omax, float lo, float hi) {
+  *omin = lo;
+  *omax = hi;
+}
+
+int stream_grid(size_t work_items) {
+  int dev = 0;
+  MXQ_HIP(hipGetDevice(&dev));
+  static thread_local int cached_dev = -1, cached_cus = 0;
+  if (cached_dev != dev) {
+    MXQ_HIP(hipDeviceGetAttribute(&cached_cus, hipDeviceAttributeMultiprocessorCount, dev));
+    cached_dev = dev;
+  }
+  size_t want = (work_items + kThreads - 1) / kThreads;
+  size_t cap = size_t(cached_cus) * size_t(g_cast_blocks_per_cu);
+  if (want < 1) want = 1;
+  return static_cast<int>(want < cap ? want : cap);
+}
+
+struct Ws {
+  float* range;
+  unsigned* counter;
+  void* partial;
+};
+Ws carve(void* workspace, size_t bytes) {
+  MXQ_CHECK(workspace != nullptr, "the uncalibrated path needs a workspace");
+  MXQ_CHECK(bytes >= kWsBytes, "workspace too small: " << bytes << " < " << kWsBytes);
+  MXQ_CHECK(aligned16(workspace), "workspace must be 16-byte aligned");
+  char* p = static_cast<char*>(workspace);
+  Ws w;
+  w.range = reinterpret_cast<float*>(p);
+  w.counter = reinterpret_cast<unsigned*>(p + 16);
+  w.partial = p + kWsHeader;
+  return w;
+}
+
+int reduce_grid(size_t n) {
+  int g = stream_grid((n + 3) / 4);
+  return g < kMaxReduceBlocks ? g : kMaxReduceBlocks;
+}
+
+__global__ void zero_two_kernel(unsigned* counter) {
+  counter[0] = 0u;
+  counter[1] = 0u;
+}
+
+void launch_quantize(hipStream_t s, const float* in, void* out, float* omin, float* omax,
+                     size_t n, int out_type, float lo, float hi, const float* dlo,
+                     const float* dhi) {
+  const bool vec = aligned16(in) && ((reinterpret_cast<uintptr_t>(out) & 3u) == 0);
+  const int grid = stream_grid(vec ? (n + 3) / 4 : n);
+  uint8_t* o = static_cast<uint8_t*>(out);
+#define MXQ_Q(U, V) \
+  hipLaunchKernelGGL((quantize_kernel<U, V>), dim3(grid), dim3(kThreads), 0, s, in, o, omin, \
+                     omax, n, lo, hi, dlo, dhi)
+  if (out_type == MXQ_UINT8) {
+    if (vec) MXQ_Q(true, true); else MXQ_Q(true, false);
+  } else {
+    if (vec) MXQ_Q(false, true); else MXQ_Q(false, false);
+  }
+#undef MXQ_Q
+  MXQ_LAUNCH_CHECK();
+}
+
+}  // namespace
+}  // namespace mxq
+
+using namespace mxq;
+
+extern "C" {
+
+size_t mxq_quantize_v2_workspace(size_t) { return kWsBytes; }
+size_t mxq_requantize_workspace(size_t) { return kWsBytes; }
+
+int mxq_quantize_v2(void* stream, const float* in, void* out, float* omin, float* omax,
+                    size_t n, int out_type, int calibrated, float min_calib, float max_calib,
+                    void* workspace, size_t workspace_bytes) {
+  MXQ_API_BEGIN();
+  MXQ_CHECK(out_type == MXQ_INT8 || out_type == MXQ_UINT8,
+            "quantize op only supports int8 and uint8 as output type, got " << out_type);
+  MXQ_CHECK(omin != nullptr && omax != nullptr, "null range output");
+  MXQ_CHECK(n == 0 || (in != nullptr && out != nullptr), "null data pointer");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (calibrated) {
+    if (n == 0) {
+      // Kernel<gpu>::Launch is a no-op for N == 0 (mxnet_op.h:1179): ranges untouched
+      return 0;
+    }
+    launch_quantize(s, in, out, omin, omax, n, out_type, min_calib, max_calib, nullptr, nullptr);
+  } else {
+    if (n == 0) return 0;
+    Ws w = carve(workspace, workspace_bytes);
+    hipLaunchKernelGGL(zero_two_kernel, dim3(1), dim3(1), 0, s, w.counter);
+    MXQ_LAUNCH_CHECK();
+    const bool vec = aligned16(in);
+    const int grid = reduce_grid(n);
+    if (vec)
+      hipLaunchKernelGGL((minmax_f32_kernel<true>), dim3(grid), dim3(kThreads), 0, s, in, n,
+                         w.range, w.counter, static_cast<float*>(w.partial));
+    else
+      hipLaunchKernelGGL((minmax_f32_kernel<false>), dim3(grid), dim3(kThreads), 0, s, in, n,
+                         w.range, w.counter, static_cast<float*>(w.partial));
+    MXQ_LAUNCH_CHECK();
+    launch_quantize(s, in, out, omin, omax, n, out_type, 0.f, 0.f, w.range, w.range + 1);
+  }
+  MXQ_API_END();
+}
+
+int mxq_quantize(void* stream, const float* in, const float* imin, const float* imax, void* out,
+                 float* omin, float* omax, size_t n, int out_type) {
+  MXQ_API_BEGIN();
+  MXQ_CHECK(out_type == MXQ_INT8 || out_type == MXQ_UINT8,
+            "quantize op only supports int8 and uint8 as output type, got " << out_type);
+  MXQ_CHECK(imin != nullptr && imax != nullptr && omin != nullptr && omax != nullptr,
+            "null range pointer");
+  MXQ_CHECK(n == 0 || (in != nullptr && out != nullptr), "null data pointer");
+  if (n == 0) return 0;
+  launch_quantize(static_cast<hipStream_t>(stream), in, out, omin, omax, n, out_type, 0.f, 0.f,
+                  imin, imax);
+  MXQ_API_END();
+}
+
+int mxq_quantize_v2_passthrough(void* stream, const void* in, void* out, float* omin,
+                                float* omax, size_t n, int in_type, int calibrated,
+                                float min_calib, float max_calib) {
+  MXQ_API_BEGIN();
+  MXQ_CHECK(in_type == MXQ_INT8 || in_type == MXQ_UINT8, "pass-through needs int8/uint8 input");
+  MXQ_CHECK(omin != nullptr && omax != nullptr, "null range output");
+  MXQ_CHECK(n == 0 || (in != nullptr && out != nullptr), "null data pointer");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  float lo, hi;
+  if (calibrated) {
+    lo = min_calib;
+    hi = max_calib;
+  } else if (in_type == MXQ_UINT8) {
+    lo = 0.f;
+    hi = 255.f;
+  } else {
+    lo = -127.f;
+    hi = 127.f;
+  }
+  hipLaunchKernelGGL(passthrough_range_kernel, dim3(1), dim3(1), 0, s, omin, omax, lo, hi);
+  MXQ_LAUNCH_CHECK();
+  if (n != 0 && in != out) MXQ_HIP(hipMemcpyAsync(out, in, n, hipMemcpyDeviceToDevice, s));
+  MXQ_API_END();
+}
+
+int mxq_requantize(void* stream, const int32_t* in, const float* imin, const float* imax,
+                   int8_t* out, float* omin, float* omax, size_t n, int calibrated,
+                   float min_calib, float max_calib, void* workspace, size_t workspace_bytes) {
+  MXQ_API_BEGIN();
+  MXQ_CHECK(imin != nullptr && imax != nullptr && omin != nullptr && omax != nullptr,
+            "null range pointer");
+  MXQ_CHECK(n == 0 || (in != nullptr && out != nullptr), "null data pointer");
+  if (n == 0) return 0;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const bool vec = aligned16(in) && ((reinterpret_cast<uintptr_t>(out) & 3u) == 0);
+  const int grid = stream_grid(vec ? (n + 3) / 4 : n);
+  uint8_t* o = reinterpret_cast<uint8_t*>(out);
+  float real_range = 0.f;
+  const float *dlo = nullptr, *dhi = nullptr;
+  if (calibrated) {
+    float a = fabsf(min_calib), b = fabsf(max_calib);
+    real_range = (a < b) ? b : a;
+  } else {
+    Ws w = carve(workspace, workspace_bytes);
+    hipLaunchKernelGGL(zero_two_kernel, dim3(1), dim3(1), 0, s, w.counter);
+    MXQ_LAUNCH_CHECK();
+    const int rgrid = reduce_grid(n);
+    if (aligned16(in))
+      hipLaunchKernelGGL((minmax_i32_kernel<true>), dim3(rgrid), dim3(kThreads), 0, s, in, n,
+                         imin, imax, w.range, w.counter, static_cast<int*>(w.partial));
+    else
+      hipLaunchKernelGGL((minmax_i32_kernel<false>), dim3(rgrid), dim3(kThreads), 0, s, in, n,
+                         imin, imax, w.range, w.counter, static_cast<int*>(w.partial));
+    MXQ_LAUNCH_CHECK();
+    dlo = w.range;
+    dhi = w.range + 1;
+  }
+  if (vec)
+    hipLaunchKernelGGL((requantize_kernel<true>), dim3(grid), dim3(kThreads), 0, s, in, o, omin,
+                       omax, n, imin, imax, real_range, dlo, dhi);
+  else
+    hipLaunchKernelGGL((requantize_kernel<false>), dim3(grid), dim3(kThreads), 0, s, in, o,
+                       omin, omax, n, imin, imax, real_range, dlo, dhi);
+  MXQ_LAUNCH_CHECK();
+  MXQ_API_END();
+}
+
+int mxq_dequantize(void* stream, const void* in, int in_type, const float* imin,
+                   const float* imax, float* out, size_t n) {
+  MXQ_API_BEGIN();
+  MXQ_CHECK(in_type == MXQ_INT8 || in_type == MXQ_UINT8,
+            "dequantize op only supports input type int8 or uint8, got " << in_type);
+  MXQ_CHECK(imin != nullptr && imax != nullptr, "null range pointer");
+  MXQ_CHECK(n == 0 || (in != nullptr && out != nullptr), "null data pointer");
+  if (n == 0) return 0;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const bool vec = aligned16(out) && ((reinterpret_cast<uintptr_t>(in) & 3u) == 0);
+  const int grid = stream_grid(vec ? (n + 3) / 4 : n);
+  const uint8_t* i8 = static_cast<const uint8_t*>(in);
+#define MXQ_D(U, V) \
+  hipLaunchKernelGGL((dequantize_kernel<U, V>), dim3(grid), dim3(kThreads), 0, s, i8, out, n, \
+                     imin, imax)
+  if (in_type == MXQ_UINT8) {
+    if (vec) MXQ_D(true, true); else MXQ_D(true, false);
+  } else {
+    if (vec) MXQ_D(false, true); else MXQ_D(false, false);
+  }
+#undef MXQ_D
+  MXQ_LAUNCH_CHECK();
+  MXQ_API_END();
+}
+
+}  // extern "C"

@@ -1,0 +1,300 @@
+// _contrib_quantized_conv on gfx950: implicit-GEMM int8 convolution on NHWC
+// operands with the same MFMA core and epilogue as the fully-connected kernel.
+// Replaces cudnnConvolutionForward (NHWC int8, IMPLICIT_PRECOMP_GEMM), the
+// float->int32 cast and QuantizedBiasAddKernel of the reference's GPU operator
+// (src/operator/quantization/quantized_conv.cu:101-219); the accumulator stays an
+// exact int32 and the bias is added in integers.
+//
+// GEMM view: rows m = (n, oh, ow), columns = output channel o, reduction
+// k = (kh, kw, c) with c fastest, which is the memory order of both the NHWC
+// activation pixel and the OHWI weight row.  Out-of-image taps and the K tail are
+// zero-filled by the loader, so no padded copy of the input is ever made.
+#include <hip/hip_runtime.h>
+
+#include <cmath>
+#include <cstdint>
+
+#include "../../include/mxq.h"
+#include "mxq_common.h"
+#include "mxq_gemm.cuh"
+
+namespace mxq {
+
+int g_conv_config = 0;  // 0 = choose by shape
+
+namespace {
+
+struct ConvArgs {
+  const int8_t* data;    // [N][H][W][C]
+  const int8_t* weight;  // [O][KH][KW][C]
+  int N, H, W, C, O, KH, KW;
+  int sh, sw, ph, pw, dh, dw, OH, OW;
+  int M, K;  // N*OH*OW, KH*KW*C
+  Epilogue epi;
+};
+
+// Activation loader: row = output pixel, chunk = 16 channels of one filter tap.
+template <class Cfg, int CHUNKS, bool ALIGNED>
+struct ConvFetch {
+  const int8_t* img[CHUNKS];  // start of image n
+  int ih0[CHUNKS], iw0[CHUNKS];
+  bool ok[CHUNKS];
+  int lc;
+  int C, KW, H, W, K, dh, dw;
+
+  __device__ __forceinline__ void init(const ConvArgs& args, int row0) {
+    C = args.C; KW = args.KW; H = args.H; W = args.W; K = args.K;
+    dh = args.dh; dw = args.dw;
+    lc = threadIdx.x % Cfg::CH;
+    const int lr = threadIdx.x / Cfg::CH;
+    const int ohow = args.OH * args.OW;
+#pragma unroll
+    for (int j = 0; j < CHUNKS; ++j) {
+      const int m = row0 + lr + j * Cfg::ROWS_PER_PASS;
+      ok[j] = m < args.M;
+      const int mm = ok[j] ? m : 0;
+      const int n = mm / ohow;
+      const int rem = mm - n * ohow;
+      const int oh = rem / args.OW;
+      const int ow = rem - oh * args.OW;
+      img[j] = args.data + static_cast<size_t>(n) * args.H * args.W * args.C;
+      ih0[j] = oh * args.sh - args.ph;
+      iw0[j] = ow * args.sw - args.pw;
+    }
+  }
+
+  __device__ __forceinline__ void fetch(int kt, v4i (&reg)[CHUNKS]) {
+    const int k0 = kt * Cfg::BK + lc * 16;
+    if (ALIGNED) {
+      // C % 16 == 0: the 16 bytes lie inside one tap
+      const bool k_ok = k0 < K;
+      const int tap = k0 / C;
+      const int c = k0 - tap * C;
+      const int kh = tap / KW;
+      const int kw = tap - kh * KW;
+      const int dih = kh * dh, diw = kw * dw;
+#pragma unroll
+      for (int j = 0; j < CHUNKS; ++j) {
+        const int ih = ih0[j] + dih, iw = iw0[j] + diw;
+        const bool v = ok[j] && k_ok && ih >= 0 && ih < H && iw >= 0 && iw < W;
+        v4i r = {0, 0, 0, 0};
+        if (v)
+          r = *reinterpret_cast<const v4i*>(img[j] +
+                                            (static_cast<size_t>(ih) * W + iw) * C + c);
+        reg[j] = r;
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < CHUNKS; ++j) {
+        v4i r = {0, 0, 0, 0};
+        if (ok[j]) {
+          for (int i = 0; i < 16; ++i) {
+            const int k = k0 + i;
+            if (k >= K) break;
+            const int tap = k / C;
+            const int c = k - tap * C;
+            const int kh = tap / KW;
+            const int kw = tap - kh * KW;
+            const int ih = ih0[j] + kh * dh, iw = iw0[j] + kw * dw;
+            if (ih >= 0 && ih < H && iw >= 0 && iw < W) {
+              uint32_t b =
+                  static_cast<uint8_t>(img[j][(static_cast<size_t>(ih) * W + iw) * C + c]);
+              r[i >> 2] |= static_cast<int>(b << (8 * (i & 3)));
+            }
+          }
+        }
+        reg[j] = r;
+      }
+    }
+  }
+};
+
+template <class Cfg, bool ALIGNED>
+__global__ __launch_bounds__(Cfg::kThreads) void conv_kernel(ConvArgs p) {
+  __shared__ __attribute__((aligned(16))) v4i lds[2][Cfg::STAGE_SLOTS];
+  const int wave = threadIdx.x >> 6;
+  const int wm = wave / Cfg::WN, wn = wave % Cfg::WN;
+  const int tiles_m = (p.M + Cfg::BM - 1) / Cfg::BM, tiles_n = (p.O + Cfg::BN - 1) / Cfg::BN;
+  int tm, tn;
+  tile_coords(blockIdx.x, tiles_m, tiles_n, tm, tn);
+  const int m0 = tm * Cfg::BM, n0 = tn * Cfg::BN;
+
+  ConvFetch<Cfg, Cfg::A_CHUNKS, ALIGNED> af;
+  RowFetch<Cfg, Cfg::B_CHUNKS, ALIGNED> bf;
+  af.init(p, m0);
+  bf.init(p.weight, n0, p.O, p.K);
+
+  v16i acc[Cfg::MI][Cfg::NI];
+  gemm_mainloop<Cfg>(acc, af, bf, (p.K + Cfg::BK - 1) / Cfg::BK, lds);
+
+  gemm_epilogue<Cfg>(acc, p.epi, m0 + wm * Cfg::TM, n0 + wn * Cfg::TN, p.M, p.O,
+                     static_cast<size_t>(p.O));
+  if (blockIdx.x == 0 && threadIdx.x == 0) epilogue_ranges(p.epi);
+}
+
+typedef GemmCfg<256, 256, 64, 2, 4> CfgL8;   // 8 waves, wave tile 128 x 64
+typedef GemmCfg<256, 128, 64, 4, 2> CfgW128; // 8 waves, wave tile 64 x 64
+typedef GemmCfg<256, 64, 64, 4, 1> CfgW64;   // 4 waves, wave tile 64 x 64
+typedef GemmCfg<128, 128, 64, 2, 2> CfgM;    // 4 waves, wave tile 64 x 64
+typedef GemmCfg<64, 64, 64, 2, 2> CfgS;      // 4 waves, wave tile 32 x 32
+
+template <class Cfg>
+void launch_cfg(hipStream_t s, const ConvArgs& a, bool aligned) {
+  const int tiles = ((a.M + Cfg::BM - 1) / Cfg::BM) * ((a.O + Cfg::BN - 1) / Cfg::BN);
+  if (aligned)
+    hipLaunchKernelGGL((conv_kernel<Cfg, true>), dim3(tiles), dim3(Cfg::kThreads), 0, s, a);
+  else
+    hipLaunchKernelGGL((conv_kernel<Cfg, false>), dim3(tiles), dim3(Cfg::kThreads), 0, s, a);
+  MXQ_LAUNCH_CHECK();
+}
+
+int num_cus() {
+  int dev = 0;
+  MXQ_HIP(hipGetDevice(&dev));
+  static thread_local int cached_dev = -1, cached_cus = 0;
+  if (cached_dev != dev) {
+    MXQ_HIP(hipDeviceGetAttribute(&cached_cus, hipDeviceAttributeMultiprocessorCount, dev));
+    cached_dev = dev;
+  }
+  return cached_cus;
+}
+
+// ---- layout adapters ------------------------------------------------------------
+// Batched transpose [B][R][S] -> [B][S][R] through a padded LDS tile; reads are
+// contiguous along S, writes contiguous along R.
+template <typename T>
+__global__ __launch_bounds__(256) void transpose_kernel(const T* __restrict__ in,
+                                                        T* __restrict__ out, int R, int S) {
+  __shared__ T tile[64][65];
+  const size_t b = blockIdx.z;
+  const int r0 = blockIdx.y * 64, s0 = blockIdx.x * 64;
+  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+  const T* src = in + b * static_cast<size_t>(R) * S;
+  T* dst = out + b * static_cast<size_t>(R) * S;
+  for (int i = ty; i < 64; i += 4) {
+    const int r = r0 + i, s = s0 + tx;
+    if (r < R && s < S) tile[i][tx] = src[static_cast<size_t>(r) * S + s];
+  }
+  __syncthreads();
+  for (int i = ty; i < 64; i += 4) {
+    const int s = s0 + i, r = r0 + tx;
+    if (r < R && s < S) dst[static_cast<size_t>(s) * R + r] = tile[tx][i];
+  }
+}
+
+template <typename T>
+void launch_transpose(hipStream_t s, const void* in, void* out, int B, int R, int S) {
+  if (B == 0 || R == 0 || S == 0) return;
+  MXQ_CHECK(B <= 65535 && (R + 63) / 64 <= 65535, "transpose grid too large");
+  dim3 grid((S + 63) / 64, (R + 63) / 64, B);
+  hipLaunchKernelGGL((transpose_kernel<T>), grid, dim3(256), 0, s, static_cast<const T*>(in),
+                     static_cast<T*>(out), R, S);
+  MXQ_LAUNCH_CHECK();
+}
+
+}  // namespace
+}  // namespace mxq
+
+using namespace mxq;
+
+extern "C" {
+
+int mxq_quantized_conv_nhwc(void* stream, const int8_t* data, const int8_t* weight,
+                            const int8_t* bias, int N, int H, int W, int C, int O, int KH,
+                            int KW, int stride_h, int stride_w, int pad_h, int pad_w,
+                            int dilate_h, int dilate_w, const float* min_data,
+                            const float* max_data, const float* min_weight,
+                            const float* max_weight, const float* min_bias,
+                            const float* max_bias, int32_t* out32, float* omin, float* omax,
+                            int8_t* out8, float* rmin, float* rmax, int relu, float min_calib,
+                            float max_calib) {
+  MXQ_API_BEGIN();
+  MXQ_CHECK(N >= 0 && H > 0 && W > 0 && C > 0 && O > 0 && KH > 0 && KW > 0, "bad shape");
+  MXQ_CHECK(stride_h > 0 && stride_w > 0 && dilate_h > 0 && dilate_w > 0 && pad_h >= 0 &&
+                pad_w >= 0,
+            "bad stride/dilate/pad");
+  MXQ_CHECK(min_data && max_data && min_weight && max_weight, "null input range pointer");
+  MXQ_CHECK(omin && omax, "null output range pointer");
+  MXQ_CHECK(bias == nullptr || (min_bias && max_bias), "bias given without its range");
+  MXQ_CHECK(out32 != nullptr || out8 != nullptr, "no output buffer");
+  MXQ_CHECK(out8 == nullptr || (rmin && rmax), "fused requantize needs rmin/rmax");
+  const int eh = dilate_h * (KH - 1) + 1, ew = dilate_w * (KW - 1) + 1;
+  MXQ_CHECK(H + 2 * pad_h >= eh && W + 2 * pad_w >= ew, "kernel larger than padded input");
+  ConvArgs a;
+  a.data = data;
+  a.weight = weight;
+  a.N = N; a.H = H; a.W = W; a.C = C; a.O = O; a.KH = KH; a.KW = KW;
+  a.sh = stride_h; a.sw = stride_w; a.ph = pad_h; a.pw = pad_w; a.dh = dilate_h; a.dw = dilate_w;
+  a.OH = (H + 2 * pad_h - eh) / stride_h + 1;
+  a.OW = (W + 2 * pad_w - ew) / stride_w + 1;
+  const long long M = static_cast<long long>(N) * a.OH * a.OW;
+  const long long K = static_cast<long long>(KH) * KW * C;
+  MXQ_CHECK(M < (1LL << 31) && K < (1LL << 31), "problem too large for 32-bit tile indices");
+  a.M = static_cast<int>(M);
+  a.K = static_cast<int>(K);
+  if (a.M == 0) return 0;
+  MXQ_CHECK(data != nullptr && weight != nullptr, "null operand pointer");
+  Epilogue& e = a.epi;
+  e.bias = bias;
+  e.min_data = min_data; e.max_data = max_data;
+  e.min_weight = min_weight; e.max_weight = max_weight;
+  e.min_bias = min_bias; e.max_bias = max_bias;
+  e.out32 = out32; e.out8 = out8;
+  e.omin = omin; e.omax = omax; e.rmin = rmin; e.rmax = rmax;
+  e.relu = relu;
+  float x = fabsf(min_calib), y = fabsf(max_calib);
+  e.real_range = (x < y) ? y : x;
+
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const bool aligned = (C % 16 == 0) && aligned16(data) && aligned16(weight);
+  int cfg = g_conv_config;
+  if (cfg == 0) {
+    const long cus = num_cus();
+    auto tiles = [&](int bm, int bn) {
+      return static_cast<long>((a.M + bm - 1) / bm) * ((O + bn - 1) / bn);
+    };
+    if (O > 128 && tiles(256, 256) >= cus) cfg = 1;
+    else if (O > 64 && tiles(256, 128) >= cus) cfg = 2;
+    else if (O <= 64 && tiles(256, 64) >= cus) cfg = 3;
+    else if (tiles(128, 128) >= cus) cfg = 4;
+    else cfg = 5;
+  }
+  switch (cfg) {
+    case 1: launch_cfg<CfgL8>(s, a, aligned); break;
+    case 2: launch_cfg<CfgW128>(s, a, aligned); break;
+    case 3: launch_cfg<CfgW64>(s, a, aligned); break;
+    case 4: launch_cfg<CfgM>(s, a, aligned); break;
+    case 5: launch_cfg<CfgS>(s, a, aligned); break;
+    default: MXQ_CHECK(false, "unknown conv tile configuration " << cfg);
+  }
+  MXQ_API_END();
+}
+
+int mxq_nchw_to_nhwc_i8(void* stream, const int8_t* in, int8_t* out, int N, int C, int H,
+                        int W) {
+  MXQ_API_BEGIN();
+  MXQ_CHECK(N >= 0 && C >= 0 && H >= 0 && W >= 0, "negative dimension");
+  MXQ_CHECK((static_cast<long long>(H) * W) < (1LL << 31), "image too large");
+  if (static_cast<long long>(N) * C * H * W == 0) return 0;
+  MXQ_CHECK(in != nullptr && out != nullptr, "null pointer");
+  launch_transpose<int8_t>(static_cast<hipStream_t>(stream), in, out, N, C, H * W);
+  MXQ_API_END();
+}
+
+int mxq_nhwc_to_nchw(void* stream, const void* in, void* out, int N, int C, int H, int W,
+                     int elem_bytes) {
+  MXQ_API_BEGIN();
+  MXQ_CHECK(N >= 0 && C >= 0 && H >= 0 && W >= 0, "negative dimension");
+  MXQ_CHECK(elem_bytes == 1 || elem_bytes == 4, "elem_bytes must be 1 or 4");
+  MXQ_CHECK((static_cast<long long>(H) * W) < (1LL << 31), "image too large");
+  if (static_cast<long long>(N) * C * H * W == 0) return 0;
+  MXQ_CHECK(in != nullptr && out != nullptr, "null pointer");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (elem_bytes == 1)
+    launch_transpose<int8_t>(s, in, out, N, H * W, C);
+  else
+    launch_transpose<int32_t>(s, in, out, N, H * W, C);
+  MXQ_API_END();
+}
+
+}  // extern "C"

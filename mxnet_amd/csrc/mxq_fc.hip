@@ -1,0 +1,151 @@
+// _contrib_quantized_fully_connected on gfx950: int8 data [M,K] x int8 weight
+// [N,K]^T -> int32, with the int8 bias rescaled to int32 and (optionally) the
+// calibrated requantize fused into the epilogue.  Replaces cublasGemmEx +
+// QuantizedBiasAddKernel of the reference's GPU operator
+// (src/operator/quantization/quantized_fully_connected.cu:58-138) with the exact
+// integer semantics of its CPU operator (quantized_fully_connected.cc:149-297).
+#include <hip/hip_runtime.h>
+
+#include <cmath>
+#include <cstdint>
+
+#include "../../include/mxq.h"
+#include "mxq_common.h"
+#include "mxq_gemm.cuh"
+
+namespace mxq {
+
+int g_fc_config = 0;  // 0 = choose by shape; 1.. force a tile configuration (tuning/tests)
+
+namespace {
+
+struct FcArgs {
+  const int8_t* data;    // [M][K]
+  const int8_t* weight;  // [N][K]
+  int M, N, K;
+  Epilogue epi;
+};
+
+template <class Cfg, bool ALIGNED>
+__global__ __launch_bounds__(Cfg::kThreads) void fc_kernel(FcArgs p) {
+  __shared__ __attribute__((aligned(16))) v4i lds[2][Cfg::STAGE_SLOTS];
+  const int wave = threadIdx.x >> 6;
+  const int wm = wave / Cfg::WN, wn = wave % Cfg::WN;
+  const int tiles_m = (p.M + Cfg::BM - 1) / Cfg::BM, tiles_n = (p.N + Cfg::BN - 1) / Cfg::BN;
+  int tm, tn;
+  tile_coords(blockIdx.x, tiles_m, tiles_n, tm, tn);
+  const int m0 = tm * Cfg::BM, n0 = tn * Cfg::BN;
+
+  RowFetch<Cfg, Cfg::A_CHUNKS, ALIGNED> af;
+  RowFetch<Cfg, Cfg::B_CHUNKS, ALIGNED> bf;
+  af.init(p.data, m0, p.M, p.K);
+  bf.init(p.weight, n0, p.N, p.K);
+
+  v16i acc[Cfg::MI][Cfg::NI];
+  gemm_mainloop<Cfg>(acc, af, bf, (p.K + Cfg::BK - 1) / Cfg::BK, lds);
+
+  gemm_epilogue<Cfg>(acc, p.epi, m0 + wm * Cfg::TM, n0 + wn * Cfg::TN, p.M, p.N,
+                     static_cast<size_t>(p.N));
+  if (blockIdx.x == 0 && threadIdx.x == 0) epilogue_ranges(p.epi);
+}
+
+typedef GemmCfg<256, 256, 64, 2, 4> CfgL8;  // 8 waves, wave tile 128 x 64
+typedef GemmCfg<256, 256, 64, 2, 2> CfgL4;  // 4 waves, wave tile 128 x 128
+typedef GemmCfg<128, 128, 64, 2, 2> CfgM;   // 4 waves, wave tile 64 x 64
+typedef GemmCfg<64, 64, 64, 2, 2> CfgS;     // 4 waves, wave tile 32 x 32
+
+template <class Cfg>
+void launch_cfg(hipStream_t s, const FcArgs& a, bool aligned) {
+  const int tiles = ((a.M + Cfg::BM - 1) / Cfg::BM) * ((a.N + Cfg::BN - 1) / Cfg::BN);
+  if (aligned)
+    hipLaunchKernelGGL((fc_kernel<Cfg, true>), dim3(tiles), dim3(Cfg::kThreads), 0, s, a);
+  else
+    hipLaunchKernelGGL((fc_kernel<Cfg, false>), dim3(tiles), dim3(Cfg::kThreads), 0, s, a);
+  MXQ_LAUNCH_CHECK();
+}
+
+int num_cus() {
+  int dev = 0;
+  MXQ_HIP(hipGetDevice(&dev));
+  static thread_local int cached_dev = -1, cached_cus = 0;
+  if (cached_dev != dev) {
+    MXQ_HIP(hipDeviceGetAttribute(&cached_cus, hipDeviceAttributeMultiprocessorCount, dev));
+    cached_dev = dev;
+  }
+  return cached_cus;
+}
+
+}  // namespace
+
+void launch_fc(hipStream_t s, const int8_t* data, const int8_t* weight, int M, int N, int K,
+               const Epilogue& epi) {
+  FcArgs a;
+  a.data = data;
+  a.weight = weight;
+  a.M = M;
+  a.N = N;
+  a.K = K;
+  a.epi = epi;
+  const bool aligned = (K % 16 == 0) && aligned16(data) && aligned16(weight);
+  int cfg = g_fc_config;
+  if (cfg == 0) {
+    const long cus = num_cus();
+    auto tiles = [&](int bm, int bn) {
+      return static_cast<long>((M + bm - 1) / bm) * ((N + bn - 1) / bn);
+    };
+    if (tiles(256, 256) >= cus)
+      cfg = 1;
+    else if (tiles(128, 128) >= cus)
+      cfg = 3;
+    else
+      cfg = 4;
+  }
+  switch (cfg) {
+    case 1: launch_cfg<CfgL8>(s, a, aligned); break;
+    case 2: launch_cfg<CfgL4>(s, a, aligned); break;
+    case 3: launch_cfg<CfgM>(s, a, aligned); break;
+    case 4: launch_cfg<CfgS>(s, a, aligned); break;
+    default: MXQ_CHECK(false, "unknown fc tile configuration " << cfg);
+  }
+}
+
+}  // namespace mxq
+
+using namespace mxq;
+
+extern "C" int mxq_quantized_fc(void* stream, const int8_t* data, const int8_t* weight,
+                                const int8_t* bias, int M, int N, int K, const float* min_data,
+                                const float* max_data, const float* min_weight,
+                                const float* max_weight, const float* min_bias,
+                                const float* max_bias, int32_t* out32, float* omin, float* omax,
+                                int8_t* out8, float* rmin, float* rmax, int relu,
+                                float min_calib, float max_calib) {
+  MXQ_API_BEGIN();
+  MXQ_CHECK(M >= 0 && N >= 0 && K >= 0, "negative dimension");
+  MXQ_CHECK(min_data && max_data && min_weight && max_weight, "null input range pointer");
+  MXQ_CHECK(omin && omax, "null output range pointer");
+  MXQ_CHECK(bias == nullptr || (min_bias && max_bias), "bias given without its range");
+  MXQ_CHECK(out32 != nullptr || out8 != nullptr, "no output buffer");
+  MXQ_CHECK(out8 == nullptr || (rmin && rmax), "fused requantize needs rmin/rmax");
+  if (M == 0 || N == 0) return 0;
+  MXQ_CHECK(data != nullptr && weight != nullptr, "null operand pointer");
+  Epilogue e;
+  e.bias = bias;
+  e.min_data = min_data;
+  e.max_data = max_data;
+  e.min_weight = min_weight;
+  e.max_weight = max_weight;
+  e.min_bias = min_bias;
+  e.max_bias = max_bias;
+  e.out32 = out32;
+  e.out8 = out8;
+  e.omin = omin;
+  e.omax = omax;
+  e.rmin = rmin;
+  e.rmax = rmax;
+  e.relu = relu;
+  float a = fabsf(min_calib), b = fabsf(max_calib);
+  e.real_range = (a < b) ? b : a;
+  launch_fc(static_cast<hipStream_t>(stream), data, weight, M, N, K, e);
+  MXQ_API_END();
+}

@@ -1,0 +1,278 @@
+/*
+ * CPU oracle for MXNet's INT8 quantized-inference operator path.
+ *
+ * TEST INFRASTRUCTURE ONLY.  Nothing shipped links or calls this file: it is
+ * the checker that the HIP kernels are compared against, and the timed CPU
+ * baseline of the benchmark.  It restates, operation by operation, the native
+ * (mshadow) CPU arithmetic of the reference; every function cites the
+ * reference lines it follows (paths relative to the apache/mxnet tree).
+ *
+ * Build: gcc -O2 -ffp-contract=off -fopenmp -shared -fPIC (no -mfma, no
+ * -ffast-math): every written float operation is one correctly rounded
+ * IEEE-754 binary32 operation, as in the reference's CPU build
+ * (CMakeLists.txt:244-256 uses -O3 -msse3, no FMA).
+ *
+ * How each function is pinned (tests/test_oracle_*.py):
+ *   - qref_quantize_int8 / qref_requantize / qref_dequantize_*: hand-derived
+ *     known answers, the numpy baselines of the reference's own tests
+ *     (tests/python/quantization/test_quantization.py:66-235), odd symmetry,
+ *     monotonicity, saturation, an exact rational (fractions.Fraction)
+ *     evaluation of every rounding step on small inputs.
+ *   - qref_quantize_uint8: exact rational evaluation + known answers.
+ *   - qref_minmax_*: numpy min/max (order independent), NaN propagation.
+ *   - qref_range_for_multiplication / qref_bias_i8_to_i32: known answers and
+ *     exact rational evaluation.
+ *   - qref_fc / qref_conv_nchw: numpy int64 matmul, torch int conv on the
+ *     same operands, the reference test's integer-valued fp32 Dense/Conv
+ *     construction, identity / single-tap special cases.
+ */
+#include <math.h>
+#include <stddef.h>
+#include <stdint.h>
+#include <string.h>
+
+#ifdef _OPENMP
+#include <omp.h>
+#endif
+
+/* ---- quantization_utils.h:41-81 ---------------------------------------- */
+
+/* Sign: (val > 0) - (val < 0); quantization_utils.h:41-44 */
+static inline int q_sign(float v) { return (v > 0.0f) - (v < 0.0f); }
+/* std::max / std::min argument order semantics; quantization_utils.h:55-71 */
+static inline float q_max(float a, float b) { return (a < b) ? b : a; }
+static inline float q_min(float a, float b) { return (b < a) ? b : a; }
+/* MaxAbs / MinAbs cast to float first; quantization_utils.h:73-81 */
+static inline float q_maxabs(float a, float b) { return q_max(fabsf(a), fabsf(b)); }
+
+#define Q_I8_RANGE 127.0f          /* MinAbs(MaxValue<int8>(), MinValue<int8>()) */
+#define Q_I32_RANGE 2147483648.0f  /* MinAbs(float(INT32_MIN), float(INT32_MAX)) = 2^31 */
+
+/* FloatToQuantized<int8_t>; quantization_utils.h:83-89 */
+static inline int8_t q_float_to_i8(float x, float scale) {
+  float t = fabsf(x) * scale;
+  float u = t + 0.5f;
+  float v = q_min(u, Q_I8_RANGE);
+  return (int8_t)((float)q_sign(x) * v);
+}
+
+/* QuantizedToFloat<int32_t>; quantization_utils.h:91-97 */
+static inline float q_i32_to_float(int32_t q, float min_range, float max_range) {
+  float real_range = q_maxabs(min_range, max_range);
+  float scale = real_range / Q_I32_RANGE;
+  return (float)q * scale;
+}
+
+int qref_num_threads(void) {
+#ifdef _OPENMP
+  return omp_get_max_threads();
+#else
+  return 1;
+#endif
+}
+
+/* ---- quantize_v2 -------------------------------------------------------- */
+
+/* quantize_v2_zero_centered::Map, quantize_v2-inl.h:98-114 (and the v1 twin
+ * quantize_zero_centered, quantize-inl.h:71-88).  Launched over all elements by
+ * Kernel<OP,cpu>::Launch (src/operator/mxnet_op.h:1013-1032). */
+void qref_quantize_int8(const float* in, size_t n, float imin, float imax, int8_t* out,
+                        float* omin, float* omax) {
+  float real_range = q_maxabs(imin, imax);
+  float scale = Q_I8_RANGE / real_range;
+#pragma omp parallel for schedule(static)
+  for (ptrdiff_t i = 0; i < (ptrdiff_t)n; ++i) out[i] = q_float_to_i8(in[i], scale);
+  *omin = -real_range;
+  *omax = real_range;
+}
+
+/* quantize_v2_unsigned::Map, quantize_v2-inl.h:66-81: the scale is a double
+ * division narrowed to float, the product is a float, the +0.5 is a double
+ * add, the cast truncates.  The reference has no clamp: out-of-range input is
+ * undefined there; this restatement clamps to [0,255] so it is total. */
+void qref_quantize_uint8(const float* in, size_t n, float imin, float imax, uint8_t* out,
+                         float* omin, float* omax) {
+  const double min_limit = 0.0, max_limit = 255.0;
+  const float scale = (float)((max_limit - min_limit) / (double)(imax - imin));
+#pragma omp parallel for schedule(static)
+  for (ptrdiff_t i = 0; i < (ptrdiff_t)n; ++i) {
+    float t = (in[i] - imin) * scale;
+    double u = (double)t + 0.5;
+    if (!(u > 0.0)) u = 0.0;
+    if (u > 255.0) u = 255.0;
+    out[i] = (uint8_t)u;
+  }
+  *omin = imin;
+  *omax = imax;
+}
+
+/* red::minimum / red::maximum over the whole tensor (NaN-propagating),
+ * 3rdparty/mshadow/mshadow/base.h:1054-1115, called from
+ * quantize_v2-inl.h:258-263. */
+void qref_minmax_f32(const float* in, size_t n, float* omin, float* omax) {
+  float mn = INFINITY, mx = -INFINITY;
+  int has_nan = 0;
+#pragma omp parallel for schedule(static) reduction(min : mn) reduction(max : mx) \
+    reduction(| : has_nan)
+  for (ptrdiff_t i = 0; i < (ptrdiff_t)n; ++i) {
+    float x = in[i];
+    if (x != x) has_nan = 1;
+    if (x < mn) mn = x;
+    if (x > mx) mx = x;
+  }
+  if (has_nan) mn = mx = NAN;
+  *omin = mn;
+  *omax = mx;
+}
+
+/* int32 min/max for the uncalibrated requantize, requantize-inl.h:177-191. */
+void qref_minmax_i32(const int32_t* in, size_t n, int32_t* omin, int32_t* omax) {
+  int32_t mn = INT32_MAX, mx = INT32_MIN;
+#pragma omp parallel for schedule(static) reduction(min : mn) reduction(max : mx)
+  for (ptrdiff_t i = 0; i < (ptrdiff_t)n; ++i) {
+    int32_t x = in[i];
+    if (x < mn) mn = x;
+    if (x > mx) mx = x;
+  }
+  *omin = mn;
+  *omax = mx;
+}
+
+/* ---- requantize --------------------------------------------------------- */
+
+/* RequantizeKernel::Map, requantize-inl.h:89-125; real_range is
+ * MaxAbs(min_calib, max_calib) (requantize-inl.h:144-154) or, uncalibrated,
+ * MaxAbs of the float images of the int32 min and max (:155-238). */
+void qref_requantize(const int32_t* in, size_t n, float imin, float imax, float real_range,
+                     int8_t* out, float* omin, float* omax) {
+  float in_range = q_maxabs(imin, imax);
+  float in_scale = in_range / Q_I32_RANGE;
+  /* FloatToQuantized(x, -real_range, real_range): MaxAbs(-r, r) = |r| */
+  float rr = q_maxabs(-real_range, real_range);
+  float scale = Q_I8_RANGE / rr;
+#pragma omp parallel for schedule(static)
+  for (ptrdiff_t i = 0; i < (ptrdiff_t)n; ++i) {
+    float f = (float)in[i] * in_scale;
+    out[i] = q_float_to_i8(f, scale);
+  }
+  *omin = -real_range;
+  *omax = real_range;
+}
+
+/* The range the uncalibrated requantize derives from the data,
+ * requantize-inl.h:177-227 (QuantizedToFloatStruct on the int32 min and max,
+ * then MaxAbs in RequantizeKernel::Map :107-124). */
+float qref_requantize_actual_range(const int32_t* in, size_t n, float imin, float imax) {
+  int32_t mn, mx;
+  qref_minmax_i32(in, n, &mn, &mx);
+  return q_maxabs(q_i32_to_float(mn, imin, imax), q_i32_to_float(mx, imin, imax));
+}
+
+/* ---- dequantize --------------------------------------------------------- */
+
+/* dequantize_zero_centered::Map, dequantize-inl.h:64-75 */
+void qref_dequantize_int8(const int8_t* in, size_t n, float imin, float imax, float* out) {
+  float real_range = q_maxabs(imax, imin);
+  float scale = real_range / Q_I8_RANGE;
+#pragma omp parallel for schedule(static)
+  for (ptrdiff_t i = 0; i < (ptrdiff_t)n; ++i) out[i] = (float)in[i] * scale;
+}
+
+/* dequantize_unsigned::Map, dequantize-inl.h:49-61 (limits 0 and 255) */
+void qref_dequantize_uint8(const uint8_t* in, size_t n, float imin, float imax, float* out) {
+  float scale = (imax - imin) / (255.0f - 0.0f);
+#pragma omp parallel for schedule(static)
+  for (ptrdiff_t i = 0; i < (ptrdiff_t)n; ++i) {
+    float p = (float)in[i] * scale;
+    out[i] = p + imin;
+  }
+}
+
+/* ---- quantized FC / conv ------------------------------------------------ */
+
+/* QuantizationRangeForMultiplication<int8,int8,int32>(all_sign=true),
+ * quantization_utils.h:134-157 */
+void qref_range_for_multiplication(float min_a, float max_a, float min_b, float max_b,
+                                   float* min_c, float* max_c) {
+  float a_one = q_maxabs(min_a, max_a) / Q_I8_RANGE;
+  float b_one = q_maxabs(min_b, max_b) / Q_I8_RANGE;
+  float c_one = a_one * b_one;
+  *max_c = c_one * Q_I32_RANGE;
+  *min_c = -*max_c;
+}
+
+/* QuantizedSumInitKernelWithBias::Map, quantized_fully_connected.cc:149-174 */
+void qref_bias_i8_to_i32(const int8_t* bias, size_t n, float min_out, float max_out,
+                         float min_bias, float max_bias, int32_t* bias32) {
+  float one_out = (float)((double)q_maxabs(min_out, max_out) / (double)INT32_MAX);
+  float one_bias = (float)((double)q_maxabs(min_bias, max_bias) / (double)INT8_MAX);
+  for (size_t i = 0; i < n; ++i) {
+    if (one_out != 0.0f) {
+      float p = (float)bias[i] * one_bias;
+      bias32[i] = (int32_t)(p / one_out);
+    } else {
+      bias32[i] = 0;
+    }
+  }
+}
+
+/* Net effect of QuantizedFullyConnectedForwardCPU,
+ * quantized_fully_connected.cc:218-297: the +128 shift of the data, the
+ * -128*sum_k w[n,k] correction and cblas_gemm_s8u8s32 with beta=1 cancel to
+ *   out[m,n] = bias32[n] + sum_k data[m,k] * weight[n,k]
+ * in wrap-around int32.  data [M,K] row-major, weight [N,K] row-major. */
+void qref_fc(const int8_t* data, const int8_t* weight, const int32_t* bias32, int M, int N,
+             int K, int32_t* out) {
+#pragma omp parallel for schedule(static) collapse(2)
+  for (int m = 0; m < M; ++m) {
+    for (int n = 0; n < N; ++n) {
+      const int8_t* a = data + (size_t)m * K;
+      const int8_t* b = weight + (size_t)n * K;
+      int32_t acc = 0;
+      for (int k = 0; k < K; ++k) acc += (int32_t)a[k] * (int32_t)b[k];
+      out[(size_t)m * N + n] = (int32_t)((uint32_t)acc + (uint32_t)(bias32 ? bias32[n] : 0));
+    }
+  }
+}
+
+/* Exact int32 cross-correlation with the shapes of QuantizedConvShape,
+ * quantized_conv.cc:30-131: data [N,C,H,W], weight [O,C,KH,KW], out
+ * [N,O,OH,OW], OH = (H + 2*pad - dilate*(KH-1) - 1)/stride + 1, num_group 1.
+ * bias32 (nullable) is added per output channel as in the FC. */
+void qref_conv_nchw(const int8_t* data, const int8_t* weight, const int32_t* bias32, int N,
+                    int C, int H, int W, int O, int KH, int KW, int stride_h, int stride_w,
+                    int pad_h, int pad_w, int dil_h, int dil_w, int32_t* out) {
+  const int OH = (H + 2 * pad_h - (dil_h * (KH - 1) + 1)) / stride_h + 1;
+  const int OW = (W + 2 * pad_w - (dil_w * (KW - 1) + 1)) / stride_w + 1;
+#pragma omp parallel for schedule(static) collapse(2)
+  for (int n = 0; n < N; ++n) {
+    for (int o = 0; o < O; ++o) {
+      for (int oh = 0; oh < OH; ++oh) {
+        for (int ow = 0; ow < OW; ++ow) {
+          int32_t acc = 0;
+          for (int c = 0; c < C; ++c) {
+            for (int kh = 0; kh < KH; ++kh) {
+              int ih = oh * stride_h - pad_h + kh * dil_h;
+              if (ih < 0 || ih >= H) continue;
+              for (int kw = 0; kw < KW; ++kw) {
+                int iw = ow * stride_w - pad_w + kw * dil_w;
+                if (iw < 0 || iw >= W) continue;
+                acc += (int32_t)data[(((size_t)n * C + c) * H + ih) * W + iw] *
+                       (int32_t)weight[(((size_t)o * C + c) * KH + kh) * KW + kw];
+              }
+            }
+          }
+          out[(((size_t)n * O + o) * OH + oh) * OW + ow] =
+              (int32_t)((uint32_t)acc + (uint32_t)(bias32 ? bias32[o] : 0));
+        }
+      }
+    }
+  }
+}
+
+/* quantized ReLU on int8 is max(x, 0); the min/max ranges pass through
+ * (dnnl/dnnl_quantized_act.cc:33-45).  Applied to the requantized int8. */
+void qref_relu_i8(const int8_t* in, size_t n, int8_t* out) {
+#pragma omp parallel for schedule(static)
+  for (ptrdiff_t i = 0; i < (ptrdiff_t)n; ++i) out[i] = in[i] > 0 ? in[i] : 0;
+}

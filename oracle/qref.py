@@ -1,0 +1,221 @@
+"""ctypes binding of oracle/mxq_oracle.c (the CPU restatement of the
+reference's native int8 arithmetic).  TEST INFRASTRUCTURE ONLY: the product
+never imports this module."""
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_SO = os.path.join(_HERE, "libmxq_oracle.so")
+
+
+def build(force=False):
+    """Compile the oracle with gcc (see Makefile for the flags)."""
+    if force and os.path.exists(_SO):
+        os.remove(_SO)
+    subprocess.check_call(["make", "-s", "-C", _HERE, "libmxq_oracle.so"])
+    return _SO
+
+
+def _load():
+    if not os.path.exists(_SO):
+        build()
+    return ctypes.CDLL(_SO)
+
+
+_lib = _load()
+_f = ctypes.c_float
+_sz = ctypes.c_size_t
+_i = ctypes.c_int
+_p = ctypes.c_void_p
+_pf = ctypes.POINTER(ctypes.c_float)
+
+_lib.qref_num_threads.restype = _i
+_lib.qref_quantize_int8.argtypes = [_p, _sz, _f, _f, _p, _pf, _pf]
+_lib.qref_quantize_uint8.argtypes = [_p, _sz, _f, _f, _p, _pf, _pf]
+_lib.qref_minmax_f32.argtypes = [_p, _sz, _pf, _pf]
+_lib.qref_minmax_i32.argtypes = [_p, _sz, ctypes.POINTER(ctypes.c_int32),
+                                 ctypes.POINTER(ctypes.c_int32)]
+_lib.qref_requantize.argtypes = [_p, _sz, _f, _f, _f, _p, _pf, _pf]
+_lib.qref_requantize_actual_range.argtypes = [_p, _sz, _f, _f]
+_lib.qref_requantize_actual_range.restype = _f
+_lib.qref_dequantize_int8.argtypes = [_p, _sz, _f, _f, _p]
+_lib.qref_dequantize_uint8.argtypes = [_p, _sz, _f, _f, _p]
+_lib.qref_range_for_multiplication.argtypes = [_f, _f, _f, _f, _pf, _pf]
+_lib.qref_bias_i8_to_i32.argtypes = [_p, _sz, _f, _f, _f, _f, _p]
+_lib.qref_fc.argtypes = [_p, _p, _p, _i, _i, _i, _p]
+_lib.qref_conv_nchw.argtypes = [_p, _p, _p] + [_i] * 13 + [_p]
+_lib.qref_relu_i8.argtypes = [_p, _sz, _p]
+
+
+def _c(a, dtype):
+    a = np.ascontiguousarray(a, dtype=dtype)
+    return a
+
+
+def _ptr(a):
+    return a.ctypes.data_as(ctypes.c_void_p)
+
+
+def num_threads():
+    return int(_lib.qref_num_threads())
+
+
+def minmax_f32(x):
+    x = _c(x, np.float32)
+    mn, mx = _f(), _f()
+    _lib.qref_minmax_f32(_ptr(x), x.size, ctypes.byref(mn), ctypes.byref(mx))
+    return np.float32(mn.value), np.float32(mx.value)
+
+
+def minmax_i32(x):
+    x = _c(x, np.int32)
+    mn, mx = ctypes.c_int32(), ctypes.c_int32()
+    _lib.qref_minmax_i32(_ptr(x), x.size, ctypes.byref(mn), ctypes.byref(mx))
+    return int(mn.value), int(mx.value)
+
+
+def quantize_v2(x, out_type="int8", min_calib_range=None, max_calib_range=None):
+    """_contrib_quantize_v2 on fp32 data -> (q, min, max); out_type 'auto' follows
+    GetQuantizeOutputType (quantization_utils.h:201-220)."""
+    x = _c(x, np.float32)
+    calibrated = min_calib_range is not None and max_calib_range is not None
+    if out_type == "auto":
+        out_type = "uint8" if (calibrated and min_calib_range >= 0.0) else "int8"
+    if calibrated:
+        lo, hi = np.float32(min_calib_range), np.float32(max_calib_range)
+    else:
+        lo, hi = minmax_f32(x)
+    omin, omax = _f(), _f()
+    if out_type == "int8":
+        q = np.empty(x.shape, np.int8)
+        _lib.qref_quantize_int8(_ptr(x), x.size, lo, hi, _ptr(q), ctypes.byref(omin),
+                                ctypes.byref(omax))
+    elif out_type == "uint8":
+        q = np.empty(x.shape, np.uint8)
+        _lib.qref_quantize_uint8(_ptr(x), x.size, lo, hi, _ptr(q), ctypes.byref(omin),
+                                 ctypes.byref(omax))
+    else:
+        raise ValueError(out_type)
+    return q, np.float32(omin.value), np.float32(omax.value)
+
+
+def quantize(x, min_range, max_range, out_type="int8"):
+    """v1 _contrib_quantize (quantize-inl.h:50-88): ranges are inputs."""
+    return quantize_v2(x, out_type, float(min_range), float(max_range))
+
+
+def requantize(x, min_range, max_range, min_calib_range=None, max_calib_range=None):
+    x = _c(x, np.int32)
+    imin, imax = np.float32(min_range), np.float32(max_range)
+    if min_calib_range is not None and max_calib_range is not None:
+        rr = np.float32(max(abs(np.float32(min_calib_range)), abs(np.float32(max_calib_range))))
+    else:
+        rr = np.float32(_lib.qref_requantize_actual_range(_ptr(x), x.size, imin, imax))
+    q = np.empty(x.shape, np.int8)
+    omin, omax = _f(), _f()
+    _lib.qref_requantize(_ptr(x), x.size, imin, imax, rr, _ptr(q), ctypes.byref(omin),
+                         ctypes.byref(omax))
+    return q, np.float32(omin.value), np.float32(omax.value)
+
+
+def dequantize(q, min_range, max_range):
+    q = np.ascontiguousarray(q)
+    out = np.empty(q.shape, np.float32)
+    if q.dtype == np.int8:
+        _lib.qref_dequantize_int8(_ptr(q), q.size, np.float32(min_range), np.float32(max_range),
+                                  _ptr(out))
+    elif q.dtype == np.uint8:
+        _lib.qref_dequantize_uint8(_ptr(q), q.size, np.float32(min_range),
+                                   np.float32(max_range), _ptr(out))
+    else:
+        raise TypeError(q.dtype)
+    return out
+
+
+def range_for_multiplication(min_a, max_a, min_b, max_b):
+    mn, mx = _f(), _f()
+    _lib.qref_range_for_multiplication(np.float32(min_a), np.float32(max_a), np.float32(min_b),
+                                       np.float32(max_b), ctypes.byref(mn), ctypes.byref(mx))
+    return np.float32(mn.value), np.float32(mx.value)
+
+
+def bias_i8_to_i32(bias, min_out, max_out, min_bias, max_bias):
+    bias = _c(bias, np.int8)
+    out = np.empty(bias.shape, np.int32)
+    _lib.qref_bias_i8_to_i32(_ptr(bias), bias.size, np.float32(min_out), np.float32(max_out),
+                             np.float32(min_bias), np.float32(max_bias), _ptr(out))
+    return out
+
+
+def fc_int32(data, weight, bias32=None):
+    """Raw exact contraction: data int8 [M,K], weight int8 [N,K], bias32 int32 [N]."""
+    data = _c(data, np.int8)
+    weight = _c(weight, np.int8)
+    M, K = data.shape
+    N, K2 = weight.shape
+    assert K == K2
+    out = np.empty((M, N), np.int32)
+    b = None
+    if bias32 is not None:
+        b = _c(bias32, np.int32)
+        assert b.shape == (N,)
+    _lib.qref_fc(_ptr(data), _ptr(weight), _ptr(b) if b is not None else None, M, N, K,
+                 _ptr(out))
+    return out
+
+
+def quantized_fully_connected(data, weight, bias, min_data, max_data, min_weight, max_weight,
+                              min_bias=None, max_bias=None, flatten=True):
+    """_contrib_quantized_fully_connected -> (int32 out, min_out, max_out)."""
+    data = _c(data, np.int8)
+    weight = _c(weight, np.int8)
+    if flatten:
+        d2 = data.reshape(data.shape[0], -1)
+    else:
+        d2 = data.reshape(-1, data.shape[-1])
+    mn, mx = range_for_multiplication(min_data, max_data, min_weight, max_weight)
+    b32 = None
+    if bias is not None:
+        b32 = bias_i8_to_i32(bias, mn, mx, min_bias, max_bias)
+    out = fc_int32(d2, weight, b32)
+    if not flatten:
+        out = out.reshape(data.shape[:-1] + (weight.shape[0],))
+    return out, mn, mx
+
+
+def conv_int32_nchw(data, weight, bias32=None, stride=(1, 1), pad=(0, 0), dilate=(1, 1)):
+    data = _c(data, np.int8)
+    weight = _c(weight, np.int8)
+    N, C, H, W = data.shape
+    O, C2, KH, KW = weight.shape
+    assert C == C2
+    OH = (H + 2 * pad[0] - (dilate[0] * (KH - 1) + 1)) // stride[0] + 1
+    OW = (W + 2 * pad[1] - (dilate[1] * (KW - 1) + 1)) // stride[1] + 1
+    out = np.empty((N, O, OH, OW), np.int32)
+    b = None
+    if bias32 is not None:
+        b = _c(bias32, np.int32)
+    _lib.qref_conv_nchw(_ptr(data), _ptr(weight), _ptr(b) if b is not None else None, N, C, H,
+                        W, O, KH, KW, stride[0], stride[1], pad[0], pad[1], dilate[0], dilate[1],
+                        _ptr(out))
+    return out
+
+
+def quantized_conv(data, weight, bias, min_data, max_data, min_weight, max_weight,
+                   min_bias=None, max_bias=None, stride=(1, 1), pad=(0, 0), dilate=(1, 1)):
+    """_contrib_quantized_conv (NCHW) -> (int32 out, min_out, max_out)."""
+    mn, mx = range_for_multiplication(min_data, max_data, min_weight, max_weight)
+    b32 = None
+    if bias is not None:
+        b32 = bias_i8_to_i32(bias, mn, mx, min_bias, max_bias)
+    return conv_int32_nchw(data, weight, b32, stride, pad, dilate), mn, mx
+
+
+def relu_i8(q):
+    q = _c(q, np.int8)
+    out = np.empty_like(q)
+    _lib.qref_relu_i8(_ptr(q), q.size, _ptr(out))
+    return out

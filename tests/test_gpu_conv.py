@@ -1,0 +1,115 @@
+"""Parity of the HIP implicit-GEMM quantized convolution with the CPU oracle (exact
+int32 cross-correlation), through the C ABI and the NCHW<->NHWC adapters."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from tests.data_gen import int8_uniform
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def capi():
+    import mxnet_amd
+    return mxnet_amd.capi
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def f32(v):
+    return dev(np.array([v], np.float32))
+
+
+def run_conv_nchw(capi, d, w, b, rd, rw, rb, stride, pad, dilate, calib=None, relu=False):
+    dn = capi.nchw_to_nhwc_i8(dev(d))
+    wn = capi.nchw_to_nhwc_i8(dev(w))
+    res = capi.quantized_conv_nhwc(dn, wn, None if b is None else dev(b), f32(-rd), f32(rd),
+                                   f32(-rw), f32(rw), None if b is None else f32(-rb),
+                                   None if b is None else f32(rb), stride=stride, pad=pad,
+                                   dilate=dilate, calib=calib, relu=relu)
+    res["out32_nchw"] = capi.nhwc_to_nchw(res["out32"])
+    if res["out8"] is not None:
+        res["out8_nchw"] = capi.nhwc_to_nchw(res["out8"])
+    return res
+
+
+# (N, C, H, W, O, KH, KW, stride, pad, dilate)
+CASES = [
+    (3, 4, 28, 28, 128, 3, 3, 1, 1, 1),    # the reference's test (test_quantization.py:365-367)
+    (2, 64, 56, 56, 64, 1, 1, 1, 0, 1),    # ResNet stage-1 1x1
+    (2, 64, 56, 56, 64, 3, 3, 1, 1, 1),    # ResNet stage-1 3x3
+    (2, 64, 28, 28, 256, 1, 1, 1, 0, 1),
+    (2, 256, 56, 56, 128, 1, 1, 2, 0, 1),  # stride-2 downsample
+    (2, 128, 28, 28, 128, 3, 3, 1, 1, 1),
+    (1, 512, 7, 7, 512, 3, 3, 1, 1, 1),
+    (1, 1024, 14, 14, 2048, 1, 1, 2, 0, 1),
+    (2, 32, 17, 13, 48, 3, 3, 2, 1, 1),    # odd sizes, stride 2 with pad
+    (1, 16, 12, 12, 20, 3, 3, 1, 2, 2),    # dilation
+    (2, 20, 9, 11, 36, 5, 3, 1, 2, 1),     # C % 16 != 0, rectangular kernel
+    (1, 3, 16, 16, 8, 7, 7, 2, 3, 1),      # first-layer-like, C = 3
+]
+
+
+@pytest.mark.parametrize("case", CASES)
+@pytest.mark.parametrize("use_bias", [False, True])
+def test_conv_int32(capi, case, use_bias):
+    N, C, H, W, O, KH, KW, s, p, dl = case
+    d = int8_uniform((N, C, H, W), seed=C + H)
+    w = int8_uniform((O, C, KH, KW), seed=O + KH)
+    b = int8_uniform((O,), seed=O) if use_bias else None
+    rd, rw, rb = 3.0, 0.2, 1.5
+    res = run_conv_nchw(capi, d, w, b, rd, rw, rb, (s, s), (p, p), (dl, dl))
+    ro, rmn, rmx = oracle.quantized_conv(d, w, b, -rd, rd, -rw, rw, None if b is None else -rb,
+                                         None if b is None else rb, (s, s), (p, p), (dl, dl))
+    np.testing.assert_array_equal(res["out32_nchw"].cpu().numpy(), ro)
+    assert (res["omin"].item(), res["omax"].item()) == (rmn, rmx)
+
+
+@pytest.mark.parametrize("cfg", [1, 2, 3, 4, 5])
+def test_conv_every_tile_config(capi, cfg):
+    import mxnet_amd
+    N, C, H, W, O, KH, KW, s, p, dl = (2, 32, 19, 19, 72, 3, 3, 1, 1, 1)
+    d = int8_uniform((N, C, H, W), seed=cfg)
+    w = int8_uniform((O, C, KH, KW), seed=cfg + 1)
+    b = int8_uniform((O,), seed=cfg + 2)
+    mxnet_amd._lib.set_tuning("conv_config", cfg)
+    try:
+        res = run_conv_nchw(capi, d, w, b, 1.0, 1.0, 1.0, (s, s), (p, p), (dl, dl),
+                            calib=(-0.02, 0.02), relu=True)
+        torch.cuda.synchronize()
+    finally:
+        mxnet_amd._lib.set_tuning("conv_config", 0)
+    ro, rmn, rmx = oracle.quantized_conv(d, w, b, -1.0, 1.0, -1.0, 1.0, -1.0, 1.0, (s, s),
+                                         (p, p), (dl, dl))
+    np.testing.assert_array_equal(res["out32_nchw"].cpu().numpy(), ro)
+    rq, qmn, qmx = oracle.requantize(ro, rmn, rmx, -0.02, 0.02)
+    np.testing.assert_array_equal(res["out8_nchw"].cpu().numpy(), oracle.relu_i8(rq))
+    assert (res["rmin"].item(), res["rmax"].item()) == (qmn, qmx)
+
+
+def test_layout_adapters(capi):
+    x = int8_uniform((3, 5, 7, 9), seed=1)
+    y = capi.nchw_to_nhwc_i8(dev(x))
+    np.testing.assert_array_equal(y.cpu().numpy(), x.transpose(0, 2, 3, 1))
+    z = capi.nhwc_to_nchw(y)
+    np.testing.assert_array_equal(z.cpu().numpy(), x)
+    v = np.random.default_rng(2).integers(-2**31, 2**31 - 1, size=(2, 70, 66, 130),
+                                          dtype=np.int32)
+    z = capi.nhwc_to_nchw(dev(v))
+    np.testing.assert_array_equal(z.cpu().numpy(), v.transpose(0, 3, 1, 2))
+
+
+def test_conv_1x1_equals_fc(capi):
+    """A 1x1 stride-1 convolution is the FC of the flattened pixels."""
+    N, H, W, C, O = 2, 14, 14, 256, 320
+    d = int8_uniform((N, H, W, C), seed=4)
+    w = int8_uniform((O, 1, 1, C), seed=5)
+    one = torch.ones(1, device="cuda")
+    rc = capi.quantized_conv_nhwc(dev(d), dev(w), None, -one, one, -one, one)
+    rf = capi.quantized_fc(dev(d.reshape(-1, C)), dev(w.reshape(O, C)), None, -one, one, -one,
+                           one)
+    assert torch.equal(rc["out32"].reshape(-1, O), rf["out32"])

@@ -1,0 +1,151 @@
+"""Parity of the HIP quantized fully-connected kernel with the CPU oracle through the
+C ABI: int32 accumulators and fused int8 outputs bit-exact."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from tests.data_gen import int8_uniform
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def capi():
+    import mxnet_amd
+    return mxnet_amd.capi
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def f32(v):
+    return dev(np.array([v], np.float32))
+
+
+def run_fc(capi, d, w, b, rd, rw, rb, calib=None, relu=False, want_int32=True):
+    return capi.quantized_fc(dev(d), dev(w), None if b is None else dev(b), f32(-rd), f32(rd),
+                             f32(-rw), f32(rw), None if b is None else f32(-rb),
+                             None if b is None else f32(rb), want_int32=want_int32, calib=calib,
+                             relu=relu)
+
+
+def oracle_fc(d, w, b, rd, rw, rb):
+    return oracle.quantized_fully_connected(d, w, b, -rd, rd, -rw, rw,
+                                            None if b is None else -rb,
+                                            None if b is None else rb)
+
+
+# (M, K, N): tile-aligned, ragged in each dimension, K not a multiple of 16 (scalar
+# loader), the reference's own test shapes (test_quantization.py:795-808)
+SHAPES = [(128, 1024, 1024), (256, 256, 256), (1, 16, 1), (33, 80, 100), (257, 144, 259),
+          (32, 2048, 100), (32, 444, 100), (256, 8192, 800), (256, 444, 800), (64, 64, 4096),
+          (300, 1000, 37), (512, 768, 768)]
+
+
+@pytest.mark.parametrize("M,K,N", SHAPES)
+@pytest.mark.parametrize("use_bias", [False, True])
+def test_fc_int32(capi, M, K, N, use_bias):
+    d = int8_uniform((M, K), seed=M + K)
+    w = int8_uniform((N, K), seed=N + K + 1)
+    b = int8_uniform((N,), seed=N) if use_bias else None
+    rd, rw, rb = 1.0, 0.08, 0.5
+    res = run_fc(capi, d, w, b, rd, rw, rb)
+    ro, rmn, rmx = oracle_fc(d, w, b, rd, rw, rb)
+    np.testing.assert_array_equal(res["out32"].cpu().numpy(), ro)
+    assert (res["omin"].item(), res["omax"].item()) == (rmn, rmx)
+
+
+@pytest.mark.parametrize("cfg", [1, 2, 3, 4])
+@pytest.mark.parametrize("M,K,N", [(512, 512, 512), (300, 208, 270), (70, 444, 33)])
+def test_fc_every_tile_config(capi, cfg, M, K, N):
+    import mxnet_amd
+    d = int8_uniform((M, K), seed=cfg + M)
+    w = int8_uniform((N, K), seed=cfg + N + 7)
+    b = int8_uniform((N,), seed=cfg)
+    mxnet_amd._lib.set_tuning("fc_config", cfg)
+    try:
+        res = run_fc(capi, d, w, b, 2.0, 0.1, 1.0, calib=(-30.0, 28.0))
+        torch.cuda.synchronize()
+    finally:
+        mxnet_amd._lib.set_tuning("fc_config", 0)
+    ro, rmn, rmx = oracle_fc(d, w, b, 2.0, 0.1, 1.0)
+    np.testing.assert_array_equal(res["out32"].cpu().numpy(), ro)
+    rq, qmn, qmx = oracle.requantize(ro, rmn, rmx, -30.0, 28.0)
+    np.testing.assert_array_equal(res["out8"].cpu().numpy(), rq)
+
+
+@pytest.mark.parametrize("M,K,N", [(128, 1024, 1024), (257, 144, 259), (32, 444, 100)])
+@pytest.mark.parametrize("relu", [False, True])
+def test_fc_fused_requantize_equals_unfused(capi, M, K, N, relu):
+    d = int8_uniform((M, K), seed=1)
+    w = int8_uniform((N, K), seed=2, lo=-20, hi=20)
+    b = int8_uniform((N,), seed=3)
+    rd, rw, rb = 1.0, 0.08, 0.5
+    ro, rmn, rmx = oracle_fc(d, w, b, rd, rw, rb)
+    # calibration range that clips part of the distribution
+    fl = ro.astype(np.float64) * (float(rmx) / 2147483648.0)
+    R = float(np.percentile(np.abs(fl), 99.0))
+    res = run_fc(capi, d, w, b, rd, rw, rb, calib=(-R, 0.9 * R), relu=relu, want_int32=False)
+    rq, qmn, qmx = oracle.requantize(ro, rmn, rmx, -R, 0.9 * R)
+    if relu:
+        rq = oracle.relu_i8(rq)
+    np.testing.assert_array_equal(res["out8"].cpu().numpy(), rq)
+    assert (res["rmin"].item(), res["rmax"].item()) == (qmn, qmx)
+    # and the stand-alone requantize kernel on the int32 output agrees too
+    res2 = run_fc(capi, d, w, b, rd, rw, rb)
+    q2, mn2, mx2 = capi.requantize(res2["out32"], res2["omin"], res2["omax"],
+                                   min_calib_range=-R, max_calib_range=0.9 * R)
+    if relu:
+        q2 = torch.clamp(q2, min=0)
+    assert torch.equal(q2, res["out8"])
+
+
+def test_fc_reference_test_construction(capi):
+    """The reference's own check (test_quantization.py:661-793): integer-valued data in
+    [-63,63], ranges = observed maxabs, no bias -> the int32 output equals the fp32
+    Dense output exactly."""
+    rng = np.random.default_rng(0)
+    for shape, nh in [((32, 512, 2, 2), 100), ((32, 111, 2, 2), 100), ((256, 111, 2, 2), 800)]:
+        data = rng.uniform(-63.0, 63.0, size=shape).astype(np.int32).astype(np.float32)
+        K = int(np.prod(shape[1:]))
+        weight = rng.uniform(-63.0, 63.0, size=(nh, K)).astype(np.int32).astype(np.float32)
+        want = data.reshape(shape[0], -1).astype(np.float64) @ weight.astype(np.float64).T
+        dr, wr = float(np.abs(data).max()), float(np.abs(weight).max())
+        res = run_fc(capi, data.reshape(shape[0], -1).astype(np.int8), weight.astype(np.int8),
+                     None, dr, wr, 0.0)
+        np.testing.assert_array_equal(res["out32"].cpu().numpy().astype(np.float64), want)
+
+
+def test_fc_large_linearity(capi):
+    """At the benchmark size (4096^3) check properties that need no CPU GEMM:
+    (a) rows of the output that the oracle recomputes (sampled), (b) linearity in the
+    data operand: fc(d1) + fc(d2) == fc(d1 + d2) for small-valued operands."""
+    M = K = N = 4096
+    g = torch.Generator(device="cuda").manual_seed(0)
+    d1 = torch.randint(-60, 61, (M, K), device="cuda", generator=g, dtype=torch.int8)
+    d2 = torch.randint(-60, 61, (M, K), device="cuda", generator=g, dtype=torch.int8)
+    w = torch.randint(-127, 128, (N, K), device="cuda", generator=g, dtype=torch.int8)
+    one = torch.ones(1, device="cuda")
+    r1 = capi.quantized_fc(d1, w, None, -one, one, -one, one)["out32"]
+    r2 = capi.quantized_fc(d2, w, None, -one, one, -one, one)["out32"]
+    r12 = capi.quantized_fc(d1 + d2, w, None, -one, one, -one, one)["out32"]
+    assert torch.equal(r1 + r2, r12)
+    rows = [0, 1, 255, 256, 1023, 2048, 4095]
+    want = oracle.fc_int32(d1[rows].cpu().numpy(), w.cpu().numpy())
+    np.testing.assert_array_equal(r1[rows].cpu().numpy(), want)
+    cols = [0, 31, 32, 255, 256, 4095]
+    want_c = oracle.fc_int32(d1.cpu().numpy(), w[cols].cpu().numpy())
+    np.testing.assert_array_equal(r1[:, cols].cpu().numpy(), want_c)
+
+
+def test_fc_errors(capi):
+    import mxnet_amd
+    d = torch.zeros((4, 16), dtype=torch.int8, device="cuda")
+    one = torch.ones(1, device="cuda")
+    with pytest.raises(mxnet_amd._lib.MXQError, match="no output buffer"):
+        capi.quantized_fc(d, d, None, -one, one, -one, one, want_int32=False)
+    b = torch.zeros(4, dtype=torch.int8, device="cuda")
+    with pytest.raises(mxnet_amd._lib.MXQError, match="bias given without its range"):
+        capi.quantized_fc(d, d, b, -one, one, -one, one)
