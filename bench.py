@@ -1,0 +1,351 @@
+#!/usr/bin/env python3
+"""Benchmark of the MI355X int8 operator path (one GPU).
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME]
+
+A step is one pass of the hot path over one batch of synthetic input that is
+already resident in HBM.  The default workload is the quantized fully-connected
+layer at M=K=N=4096 with the bias and the calibrated requantize-to-int8 fused in
+the epilogue; --workload selects the other headline kernels (the 64M-element
+quantize / requantize / dequantize casts, the 8192^3 FC).  One JSON line is
+printed.  `roofline` describes the workload's kernel (algorithmic bytes or ops
+per launch over the HIP-event-timed average launch); `cast_ops` lists the same
+figures for the bandwidth-bound kernels, measured in the same run;
+`cpu_baseline` is the CPU oracle (the restatement of the reference's native CPU
+operator) timed on a bounded sample on this host.
+"""
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+METRIC = "int8 FC TOPS (% MFMA peak) + quant/requant GB/s (% HBM peak), 1 GPU"
+HBM_PEAK_GBS = 8000.0    # MI355X HBM3E
+INT8_PEAK_TOPS = 5000.0  # MI355X dense int8 MFMA
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--workload", default="fc4096",
+                    choices=["fc4096", "fc8192", "quantize", "quantize_uncal", "quantize_uint8",
+                             "requantize", "requantize_uncal", "dequantize"])
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-cast-ops", action="store_true")
+    return ap.parse_args()
+
+
+class FcWorkload:
+    """BASELINE config 3: data quantized from U(-1,1) with calib (-1,1), weight from
+    N(0,0.02) with its own min/max, int8 bias, fused requantize with a calibrated range."""
+
+    def __init__(self, S, torch, capi, lib):
+        import numpy as np
+        self.S = S
+        self.name = "quantized_fully_connected M=K=N=%d, int8 bias + calibrated requantize " \
+                    "fused in the epilogue" % S
+        self.kernel = "fc_kernel"
+        self.bound = "mfma"
+        self.ops = 2.0 * S * S * S
+        g = torch.Generator(device="cuda").manual_seed(0)
+        x = torch.rand((S, S), device="cuda", generator=g) * 2.0 - 1.0
+        self.data, self.dmin, self.dmax = capi.quantize_v2(x, "int8", min_calib_range=-1.0,
+                                                           max_calib_range=1.0)
+        w = torch.randn((S, S), device="cuda", generator=g) * 0.02
+        self.weight, self.wmin, self.wmax = capi.quantize(w, w.min().reshape(1),
+                                                          w.max().reshape(1))
+        b = torch.randn((S,), device="cuda", generator=g) * 0.02
+        self.bias, self.bmin, self.bmax = capi.quantize(b, b.min().reshape(1), b.max().reshape(1))
+        del x, w
+        # calibration range of the output: max |fp32 output| over a 1-in-64 row sample
+        rows = self.data[::64].to(torch.float32) @ self.weight.to(torch.float32).t()
+        scale = (self.dmax.item() / 127.0) * (self.wmax.abs().item() / 127.0)
+        r = float(rows.abs().max().item() * scale)
+        self.calib = (-r, r)
+        self.out8 = torch.empty((S, S), dtype=torch.int8, device="cuda")
+        self.sc = [torch.empty(1, device="cuda") for _ in range(4)]
+        self.lib = lib
+        self.P = lambda t: ctypes.c_void_p(t.data_ptr())
+        self.torch = torch
+
+    def step(self):
+        P, S = self.P, self.S
+        st = ctypes.c_void_p(self.torch.cuda.current_stream().cuda_stream)
+        rc = self.lib.mxq_quantized_fc(st, P(self.data), P(self.weight), P(self.bias), S, S, S,
+                                       P(self.dmin), P(self.dmax), P(self.wmin), P(self.wmax),
+                                       P(self.bmin), P(self.bmax), None, P(self.sc[0]),
+                                       P(self.sc[1]), P(self.out8), P(self.sc[2]), P(self.sc[3]),
+                                       0, self.calib[0], self.calib[1])
+        if rc != 0:
+            raise RuntimeError(self.lib.mxq_last_error().decode())
+
+    def value(self, sec_per_step):
+        return self.ops / sec_per_step / 1e12, "TOPS"
+
+    def cpu_baseline(self, oracle, budget_s=12.0):
+        """Oracle FC on the first rows of the same operands, sized to ~budget_s."""
+        import numpy as np
+        S = self.S
+        w = self.weight.cpu().numpy()
+        d = self.data.cpu().numpy()
+        t0 = time.perf_counter()
+        oracle.fc_int32(d[:64], w)
+        t64 = time.perf_counter() - t0
+        rows = int(max(64, min(S, 64 * budget_s / max(t64, 1e-9))))
+        t0 = time.perf_counter()
+        oracle.fc_int32(d[:rows], w)
+        dt = time.perf_counter() - t0
+        tops = 2.0 * rows * S * S / dt / 1e12
+        return {"value": tops, "unit": "TOPS", "cores": oracle.num_threads(), "kind": "port",
+                "sample": "oracle qref_fc (OpenMP) on the first %d of %d data rows against the "
+                          "full [%d,%d] weight, %.1f s" % (rows, S, S, S, dt)}
+
+
+class CastWorkload:
+    """BASELINE config 2: 64M-element flat tensors, buffers rotated so that the
+    256 MB Infinity Cache cannot serve the reads."""
+    N = 1 << 26
+    NBUF = 3
+
+    def __init__(self, kind, torch, capi, lib):
+        import numpy as np
+        self.kind = kind
+        self.torch = torch
+        self.lib = lib
+        n = self.N
+        self.bound = "hbm"
+        self.P = lambda t: ctypes.c_void_p(t.data_ptr())
+        g = torch.Generator(device="cuda").manual_seed(1)
+        self.i = 0
+        self.omin = torch.empty(1, device="cuda")
+        self.omax = torch.empty(1, device="cuda")
+        self.ws = torch.empty(lib.mxq_quantize_v2_workspace(n), dtype=torch.uint8, device="cuda")
+        if kind.startswith("quantize"):
+            self.src = []
+            for _ in range(self.NBUF):
+                x = torch.randn(n, device="cuda", generator=g)
+                idx = torch.randint(0, n, (n // 10000,), device="cuda", generator=g)
+                sign = torch.randint(0, 2, (n // 10000,), device="cuda", generator=g) * 2 - 1
+                x[idx] = 50.0 * sign.to(torch.float32)
+                self.src.append(x)
+            self.dst = [torch.empty(n, dtype=torch.uint8, device="cuda")
+                        for _ in range(self.NBUF)]
+            self.bytes = (9.0 if kind == "quantize_uncal" else 5.0) * n
+            self.kernel = "quantize_kernel" + (" + minmax_f32_kernel"
+                                               if kind == "quantize_uncal" else "")
+            self.name = {"quantize": "quantize_v2 fp32->int8 calibrated (-50,50)",
+                         "quantize_uncal": "quantize_v2 fp32->int8 uncalibrated "
+                                           "(on-device min/max)",
+                         "quantize_uint8": "quantize_v2 fp32->uint8 calibrated (-50,50)"}[kind]
+        elif kind.startswith("requantize"):
+            self.src = [torch.randint(-2 ** 28, 2 ** 28, (n,), device="cuda", generator=g,
+                                      dtype=torch.int32) for _ in range(self.NBUF)]
+            self.dst = [torch.empty(n, dtype=torch.int8, device="cuda")
+                        for _ in range(self.NBUF)]
+            self.imin = torch.tensor([-1.0], device="cuda")
+            self.imax = torch.tensor([1.0], device="cuda")
+            self.bytes = (9.0 if kind == "requantize_uncal" else 5.0) * n
+            self.kernel = "requantize_kernel" + (" + minmax_i32_kernel"
+                                                 if kind == "requantize_uncal" else "")
+            self.name = ("requantize int32->int8 " +
+                         ("uncalibrated (on-device min/max)" if kind == "requantize_uncal"
+                          else "calibrated (-0.1,0.1)"))
+        elif kind == "dequantize":
+            self.src = [torch.randint(-127, 128, (n,), device="cuda", generator=g,
+                                      dtype=torch.int8) for _ in range(self.NBUF)]
+            self.dst = [torch.empty(n, dtype=torch.float32, device="cuda")
+                        for _ in range(self.NBUF)]
+            self.imin = torch.tensor([-3.0], device="cuda")
+            self.imax = torch.tensor([3.0], device="cuda")
+            self.bytes = 5.0 * n
+            self.kernel = "dequantize_kernel"
+            self.name = "dequantize int8->fp32"
+        else:
+            raise ValueError(kind)
+        self.name += ", %d elements" % n
+
+    def step(self):
+        P, n, lib = self.P, self.N, self.lib
+        k = self.i % self.NBUF
+        self.i += 1
+        st = ctypes.c_void_p(self.torch.cuda.current_stream().cuda_stream)
+        kind = self.kind
+        if kind == "quantize":
+            rc = lib.mxq_quantize_v2(st, P(self.src[k]), P(self.dst[k]), P(self.omin),
+                                     P(self.omax), n, 5, 1, -50.0, 50.0, None, 0)
+        elif kind == "quantize_uint8":
+            rc = lib.mxq_quantize_v2(st, P(self.src[k]), P(self.dst[k]), P(self.omin),
+                                     P(self.omax), n, 3, 1, -50.0, 50.0, None, 0)
+        elif kind == "quantize_uncal":
+            rc = lib.mxq_quantize_v2(st, P(self.src[k]), P(self.dst[k]), P(self.omin),
+                                     P(self.omax), n, 5, 0, 0.0, 0.0, P(self.ws),
+                                     self.ws.numel())
+        elif kind == "requantize":
+            rc = lib.mxq_requantize(st, P(self.src[k]), P(self.imin), P(self.imax),
+                                    P(self.dst[k]), P(self.omin), P(self.omax), n, 1, -0.1, 0.1,
+                                    None, 0)
+        elif kind == "requantize_uncal":
+            rc = lib.mxq_requantize(st, P(self.src[k]), P(self.imin), P(self.imax),
+                                    P(self.dst[k]), P(self.omin), P(self.omax), n, 0, 0.0, 0.0,
+                                    P(self.ws), self.ws.numel())
+        else:
+            rc = lib.mxq_dequantize(st, P(self.src[k]), 5, P(self.imin), P(self.imax),
+                                    P(self.dst[k]), n)
+        if rc != 0:
+            raise RuntimeError(lib.mxq_last_error().decode())
+
+    def value(self, sec_per_step):
+        return self.bytes / sec_per_step / 1e9, "GB/s"
+
+    def cpu_baseline(self, oracle, budget_s=12.0):
+        import numpy as np
+        n = 1 << 24
+        kind = self.kind
+        x = self.src[0][:n].cpu().numpy()
+        reps, t0 = 0, time.perf_counter()
+        while True:
+            if kind == "quantize":
+                oracle.quantize_v2(x, "int8", -50.0, 50.0)
+            elif kind == "quantize_uint8":
+                oracle.quantize_v2(x, "uint8", -50.0, 50.0)
+            elif kind == "quantize_uncal":
+                oracle.quantize_v2(x, "int8")
+            elif kind == "requantize":
+                oracle.requantize(x, -1.0, 1.0, -0.1, 0.1)
+            elif kind == "requantize_uncal":
+                oracle.requantize(x, -1.0, 1.0)
+            else:
+                oracle.dequantize(x, -3.0, 3.0)
+            reps += 1
+            dt = time.perf_counter() - t0
+            if dt > budget_s / 2 or reps >= 50:
+                break
+        gbs = self.bytes / self.N * n * reps / dt / 1e9
+        return {"value": gbs, "unit": "GB/s", "cores": oracle.num_threads(), "kind": "port",
+                "sample": "oracle (OpenMP) on the first %d elements, %d repetitions, %.1f s"
+                          % (n, reps, dt)}
+
+
+def make_workload(name, torch, capi, lib):
+    if name == "fc4096":
+        return FcWorkload(4096, torch, capi, lib)
+    if name == "fc8192":
+        return FcWorkload(8192, torch, capi, lib)
+    return CastWorkload(name, torch, capi, lib)
+
+
+def timed_run(torch, wl, steps, warmup):
+    """Returns (wall seconds for `steps` steps, HIP-event seconds for the same steps)."""
+    for _ in range(warmup):
+        wl.step()
+    torch.cuda.synchronize()
+    ev0 = torch.cuda.Event(enable_timing=True)
+    ev1 = torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    ev0.record()
+    for _ in range(steps):
+        wl.step()
+    ev1.record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    return wall, ev0.elapsed_time(ev1) / 1e3
+
+
+def roofline_of(wl, event_s_per_launch):
+    if wl.bound == "mfma":
+        achieved = wl.ops / event_s_per_launch / 1e12
+        peak, unit = INT8_PEAK_TOPS, "TOP/s"
+    else:
+        achieved = wl.bytes / event_s_per_launch / 1e9
+        peak, unit = HBM_PEAK_GBS, "GB/s"
+    return {"bound": wl.bound, "kernel": wl.kernel, "achieved": round(achieved, 1), "peak": peak,
+            "unit": unit, "frac": round(achieved / peak, 4), "traffic": None,
+            "avg_launch_us": round(event_s_per_launch * 1e6, 2)}
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (the operators "
+              "shard trivially, see DESIGN.md); run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+    import torch
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU (the HIP path has no CPU fallback)", file=sys.stderr)
+        sys.exit(2)
+    torch.cuda.set_device(0)
+    import mxnet_amd
+    from mxnet_amd import capi
+    lib = mxnet_amd._lib.lib
+
+    wl = make_workload(args.workload, torch, capi, lib)
+    wall, ev = timed_run(torch, wl, args.steps, args.warmup)
+    sec_per_step = wall / args.steps
+    value, unit = wl.value(sec_per_step)
+    line = {
+        "metric": METRIC,
+        "value": round(value, 2),
+        "unit": unit,
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(sec_per_step * 1e3, 5),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "int8",
+        "data": "synthetic",
+        "config": {"workload": wl.name},
+        "device": torch.cuda.get_device_name(0),
+        "roofline": roofline_of(wl, ev / args.steps),
+    }
+
+    if not args.no_cast_ops:
+        rows = []
+        for kind in ["quantize", "quantize_uint8", "quantize_uncal", "requantize",
+                     "requantize_uncal", "dequantize", "fc8192"]:
+            if kind == args.workload:
+                continue
+            w2 = make_workload(kind, torch, capi, lib)
+            steps2 = 20 if kind == "fc8192" else 60
+            wall2, ev2 = timed_run(torch, w2, steps2, 5)
+            r = roofline_of(w2, ev2 / steps2)
+            r["workload"] = w2.name
+            rows.append(r)
+            del w2
+            torch.cuda.empty_cache()
+        line["other_kernels"] = rows
+
+    if not args.no_cpu_baseline:
+        import oracle
+        line["cpu_baseline"] = wl.cpu_baseline(oracle)
+        try:
+            # the reference's timed CPU path is oneDNN; torch bundles a oneDNN int8 GEMM
+            if isinstance(wl, FcWorkload):
+                d = wl.data[:512].cpu()
+                w = wl.weight.cpu()
+                torch._int_mm(d, w.t())
+                t0 = time.perf_counter()
+                reps = 0
+                while time.perf_counter() - t0 < 5.0:
+                    torch._int_mm(d, w.t())
+                    reps += 1
+                dt = time.perf_counter() - t0
+                line["cpu_baseline"]["onednn_via_torch_TOPS"] = round(
+                    2.0 * 512 * wl.S * wl.S * reps / dt / 1e12, 4)
+                line["cpu_baseline"]["onednn_threads"] = torch.get_num_threads()
+        except Exception as e:  # informational only
+            line["cpu_baseline"]["onednn_via_torch_TOPS"] = "unavailable: %s" % e
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -22,13 +22,14 @@
 
 #include <cmath>
 #include <cstdint>
+#include <cstring>
 
 #include "../../include/mxq.h"
 #include "mxq_common.h"
 
 namespace mxq {
 
-int g_cast_blocks_per_cu = 8;  // tunable through mxq_set_tuning("cast_blocks_per_cu", v)
+int g_cast_blocks_per_cu = 2;  // tunable through mxq_set_tuning("cast_blocks_per_cu", v)
 
 namespace {
 
@@ -37,9 +38,13 @@ typedef int i4 __attribute__((ext_vector_type(4)));
 
 constexpr int kThreads = 256;
 constexpr int kUnroll = 4;             // 16-byte segments in flight per lane
-constexpr int kMaxReduceBlocks = 2048;  // partials held in the workspace
-constexpr size_t kWsHeader = 64;        // [0] lo, [4] hi, [16] ticket counter
-constexpr size_t kWsBytes = kWsHeader + size_t(kMaxReduceBlocks) * 8;
+// Reduction workspace: kSlots accumulator slots of 64 bytes, each {min, max, nan
+// flag} as 32-bit words.  Blocks fold their partial into slot (block % kSlots)
+// with relaxed device-scope atomics (coherent across XCDs without any fence);
+// the consuming kernel of the same stream folds the slots.
+constexpr int kSlots = 32;
+constexpr int kSlotWords = 16;
+constexpr size_t kWsBytes = size_t(kSlots) * kSlotWords * 4;
 
 __device__ __forceinline__ float maxabs(float a, float b) {
   float x = fabsf(a), y = fabsf(b);
@@ -160,9 +165,58 @@ __device__ __forceinline__ void narrow_scalar(const SrcT* __restrict__ in,
   }
 }
 
+// ---- reduced-range slots ----------------------------------------------------
+// Order-preserving map float -> uint32 (so unsigned atomic min/max order floats).
+__device__ __forceinline__ uint32_t f2ord(float f) {
+  uint32_t u = __builtin_bit_cast(uint32_t, f);
+  return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+__device__ __forceinline__ float ord2f(uint32_t o) {
+  uint32_t u = (o & 0x80000000u) ? (o & 0x7fffffffu) : ~o;
+  return __builtin_bit_cast(float, u);
+}
+
+uint32_t f2ord_host(float f) {
+  uint32_t u;
+  std::memcpy(&u, &f, 4);
+  return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+
+// Range left by the fp32 reduction, NaN-propagating like mshadow's red::minimum /
+// red::maximum (3rdparty/mshadow/mshadow/base.h:1054-1115): any NaN makes both NaN.
+__device__ __forceinline__ void load_range_f32(const uint32_t* slots, float& lo, float& hi) {
+  uint32_t mn = 0xffffffffu, mx = 0u, nan = 0u;
+#pragma unroll 8
+  for (int s = 0; s < kSlots; ++s) {
+    uint32_t a = slots[s * kSlotWords + 0], b = slots[s * kSlotWords + 1];
+    mn = a < mn ? a : mn;
+    mx = b > mx ? b : mx;
+    nan |= slots[s * kSlotWords + 2];
+  }
+  lo = ord2f(mn);
+  hi = ord2f(mx);
+  if (nan) lo = hi = NAN;
+}
+
+// Range left by the int32 reduction, converted to the float images
+// QuantizedToFloat(min), QuantizedToFloat(max) (requantize-inl.h:192-227).
+__device__ __forceinline__ void load_range_i32(const uint32_t* slots, float in_scale, float& lo,
+                                               float& hi) {
+  int mn = INT32_MAX, mx = INT32_MIN;
+#pragma unroll 8
+  for (int s = 0; s < kSlots; ++s) {
+    int a = static_cast<int>(slots[s * kSlotWords + 0]);
+    int b = static_cast<int>(slots[s * kSlotWords + 1]);
+    mn = a < mn ? a : mn;
+    mx = b > mx ? b : mx;
+  }
+  lo = static_cast<float>(mn) * in_scale;
+  hi = static_cast<float>(mx) * in_scale;
+}
+
 // ---- quantize kernels ----------------------------------------------------------
-// The range is (lo, hi) by value, or read from two device scalars when dlo != NULL
-// (v1 operator inputs, or the reduced range in the workspace).
+// The range is (lo, hi) by value, two device scalars when dlo != NULL (v1 operator
+// inputs), or the reduction slots when slots != NULL (uncalibrated v2).
 template <bool UNSIGNED, bool VEC>
 __global__ __launch_bounds__(kThreads) void quantize_kernel(const float* __restrict__ in,
                                                             uint8_t* __restrict__ out,
@@ -170,10 +224,13 @@ __global__ __launch_bounds__(kThreads) void quantize_kernel(const float* __restr
                                                             float* __restrict__ omax, size_t n,
                                                             float lo, float hi,
                                                             const float* __restrict__ dlo,
-                                                            const float* __restrict__ dhi) {
+                                                            const float* __restrict__ dhi,
+                                                            const uint32_t* __restrict__ slots) {
   if (dlo != nullptr) {
     lo = *dlo;
     hi = *dhi;
+  } else if (slots != nullptr) {
+    load_range_f32(slots, lo, hi);
   }
   if (UNSIGNED) {
     QuantU8 rule;
@@ -203,16 +260,19 @@ __global__ __launch_bounds__(kThreads) void quantize_kernel(const float* __restr
 }
 
 // ---- requantize kernel -------------------------------------------------------
-// real range: by value (calibrated), or MaxAbs of two device scalars (the float
-// images of the int32 min and max left in the workspace by the reduction).
+// real range: by value (calibrated), or MaxAbs of the float images of the int32
+// min and max left in the reduction slots.
 template <bool VEC>
 __global__ __launch_bounds__(kThreads) void requantize_kernel(
     const int32_t* __restrict__ in, uint8_t* __restrict__ out, float* __restrict__ omin,
     float* __restrict__ omax, size_t n, const float* __restrict__ imin,
-    const float* __restrict__ imax, float real_range, const float* __restrict__ dlo,
-    const float* __restrict__ dhi) {
-  if (dlo != nullptr) real_range = maxabs(*dlo, *dhi);
+    const float* __restrict__ imax, float real_range, const uint32_t* __restrict__ slots) {
   const float in_scale = maxabs(*imin, *imax) / 2147483648.0f;
+  if (slots != nullptr) {
+    float lo, hi;
+    load_range_i32(slots, in_scale, lo, hi);
+    real_range = maxabs(lo, hi);
+  }
   QuantI8 rule;
   rule.s = 127.0f / maxabs(-real_range, real_range);
   if (VEC)
@@ -321,14 +381,20 @@ struct MaxU {
 };
 
 
-// Shared finalisation: block partial -> workspace, ticket, last block folds all
-// partials.  Returns true in the last block with (mn, mx) holding the global
-// result in every thread of wave 0.
+// Slots start at the reduction identities: fp32 as ordered bits, int32 as is.
+__global__ void init_slots_kernel(uint32_t* slots, uint32_t min_id, uint32_t max_id) {
+  const int s = threadIdx.x;
+  if (s < kSlots) {
+    slots[s * kSlotWords + 0] = min_id;
+    slots[s * kSlotWords + 1] = max_id;
+    slots[s * kSlotWords + 2] = 0u;
+  }
+}
+
+// Block-level fold; thread 0 returns the block's (mn, mx).
 template <typename T, typename MinOp, typename MaxOp>
-__device__ __forceinline__ bool grid_finish(T& mn, T& mx, T* partial, unsigned* counter,
-                                            T init_min, T init_max) {
+__device__ __forceinline__ void block_fold(T& mn, T& mx) {
   __shared__ T s_min[kThreads / 64], s_max[kThreads / 64];
-  __shared__ bool s_last;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   mn = wave_reduce(mn, MinOp());
   mx = wave_reduce(mx, MaxOp());
@@ -342,48 +408,14 @@ __device__ __forceinline__ bool grid_finish(T& mn, T& mx, T* partial, unsigned* 
       mn = MinOp()(mn, s_min[w]);
       mx = MaxOp()(mx, s_max[w]);
     }
-    partial[2 * blockIdx.x] = mn;
-    partial[2 * blockIdx.x + 1] = mx;
-    __threadfence();  // release the partial before taking the ticket
-    unsigned t = atomicAdd(counter, 1u);
-    s_last = (t == gridDim.x - 1);
   }
-  __syncthreads();
-  if (!s_last) return false;
-  __threadfence();  // acquire the other blocks' partials
-  mn = init_min;
-  mx = init_max;
-  for (unsigned b = threadIdx.x; b < gridDim.x; b += kThreads) {
-    mn = MinOp()(mn, __hip_atomic_load(&partial[2 * b], __ATOMIC_RELAXED,
-                                       __HIP_MEMORY_SCOPE_AGENT));
-    mx = MaxOp()(mx, __hip_atomic_load(&partial[2 * b + 1], __ATOMIC_RELAXED,
-                                       __HIP_MEMORY_SCOPE_AGENT));
-  }
-  mn = wave_reduce(mn, MinOp());
-  mx = wave_reduce(mx, MaxOp());
-  __syncthreads();
-  if (lane == 0) {
-    s_min[wave] = mn;
-    s_max[wave] = mx;
-  }
-  __syncthreads();
-  mn = s_min[0];
-  mx = s_max[0];
-  for (int w = 1; w < kThreads / 64; ++w) {
-    mn = MinOp()(mn, s_min[w]);
-    mx = MaxOp()(mx, s_max[w]);
-  }
-  return true;
 }
 
-// fp32 min / max, NaN-propagating like mshadow's red::minimum / red::maximum
-// (3rdparty/mshadow/mshadow/base.h:1054-1115): any NaN makes both results NaN.
-// NaN is detected through the largest |x| bit pattern.
+// fp32 min / max of the whole tensor in one pass.  NaN is detected through the
+// largest |x| bit pattern (> 0x7f800000).
 template <bool VEC>
 __global__ __launch_bounds__(kThreads) void minmax_f32_kernel(const float* __restrict__ in,
-                                                              size_t n, float* ws_range,
-                                                              unsigned* counter,
-                                                              float* partial) {
+                                                              size_t n, uint32_t* slots) {
   float mn = INFINITY, mx = -INFINITY;
   uint32_t amax = 0;
   auto fold = [&](float x) {
@@ -423,35 +455,20 @@ __global__ __launch_bounds__(kThreads) void minmax_f32_kernel(const float* __res
   } else {
     for (size_t i = size_t(blockIdx.x) * kThreads + threadIdx.x; i < n; i += stride) fold(in[i]);
   }
-  // A block that saw a NaN raises the flag word next to the ticket counter
-  // before it takes its ticket (same thread, ordered by the fence in
-  // grid_finish), so the last block observes it.
+  uint32_t* slot = slots + (blockIdx.x % kSlots) * kSlotWords;
   amax = wave_reduce(amax, MaxU());
-  if ((threadIdx.x & 63) == 0 && amax > 0x7f800000u) atomicOr(counter + 1, 1u);
-  __syncthreads();
-  if (grid_finish<float, MinF, MaxF>(mn, mx, partial, counter, INFINITY, -INFINITY)) {
-    if (threadIdx.x == 0) {
-      unsigned nanflag = __hip_atomic_load(counter + 1, __ATOMIC_RELAXED,
-                                           __HIP_MEMORY_SCOPE_AGENT);
-      if (nanflag) {
-        mn = NAN;
-        mx = NAN;
-      }
-      ws_range[0] = mn;
-      ws_range[1] = mx;
-    }
+  if ((threadIdx.x & 63) == 0 && amax > 0x7f800000u) atomicOr(slot + 2, 1u);
+  block_fold<float, MinF, MaxF>(mn, mx);
+  if (threadIdx.x == 0) {
+    atomicMin(slot + 0, f2ord(mn));
+    atomicMax(slot + 1, f2ord(mx));
   }
 }
 
-// int32 min / max; the last block converts both to their float images with the
-// input scale (QuantizedToFloatStruct, requantize-inl.h:192-227).
+// int32 min / max of the whole tensor in one pass.
 template <bool VEC>
 __global__ __launch_bounds__(kThreads) void minmax_i32_kernel(const int32_t* __restrict__ in,
-                                                              size_t n,
-                                                              const float* __restrict__ imin,
-                                                              const float* __restrict__ imax,
-                                                              float* ws_range, unsigned* counter,
-                                                              int* partial) {
+                                                              size_t n, uint32_t* slots) {
   int mn = INT32_MAX, mx = INT32_MIN;
   auto fold = [&](int x) {
     mn = x < mn ? x : mn;
@@ -488,12 +505,11 @@ __global__ __launch_bounds__(kThreads) void minmax_i32_kernel(const int32_t* __r
   } else {
     for (size_t i = size_t(blockIdx.x) * kThreads + threadIdx.x; i < n; i += stride) fold(in[i]);
   }
-  if (grid_finish<int, MinI, MaxI>(mn, mx, partial, counter, INT32_MAX, INT32_MIN)) {
-    if (threadIdx.x == 0) {
-      const float scale = maxabs(*imin, *imax) / 2147483648.0f;
-      ws_range[0] = static_cast<float>(mn) * scale;
-      ws_range[1] = static_cast<float>(mx) * scale;
-    }
+  block_fold<int, MinI, MaxI>(mn, mx);
+  if (threadIdx.x == 0) {
+    int* slot = reinterpret_cast<int*>(slots + (blockIdx.x % kSlots) * kSlotWords);
+    atomicMin(slot + 0, mn);
+    atomicMax(slot + 1, mx);
   }
 }
 
@@ -516,42 +532,22 @@ int stream_grid(size_t work_items) {
   return static_cast<int>(want < cap ? want : cap);
 }
 
-struct Ws {
-  float* range;
-  unsigned* counter;
-  void* partial;
-};
-Ws carve(void* workspace, size_t bytes) {
+uint32_t* carve(void* workspace, size_t bytes) {
   MXQ_CHECK(workspace != nullptr, "the uncalibrated path needs a workspace");
   MXQ_CHECK(bytes >= kWsBytes, "workspace too small: " << bytes << " < " << kWsBytes);
   MXQ_CHECK(aligned16(workspace), "workspace must be 16-byte aligned");
-  char* p = static_cast<char*>(workspace);
-  Ws w;
-  w.range = reinterpret_cast<float*>(p);
-  w.counter = reinterpret_cast<unsigned*>(p + 16);
-  w.partial = p + kWsHeader;
-  return w;
-}
-
-int reduce_grid(size_t n) {
-  int g = stream_grid((n + 3) / 4);
-  return g < kMaxReduceBlocks ? g : kMaxReduceBlocks;
-}
-
-__global__ void zero_two_kernel(unsigned* counter) {
-  counter[0] = 0u;
-  counter[1] = 0u;
+  return static_cast<uint32_t*>(workspace);
 }
 
 void launch_quantize(hipStream_t s, const float* in, void* out, float* omin, float* omax,
                      size_t n, int out_type, float lo, float hi, const float* dlo,
-                     const float* dhi) {
+                     const float* dhi, const uint32_t* slots) {
   const bool vec = aligned16(in) && ((reinterpret_cast<uintptr_t>(out) & 3u) == 0);
   const int grid = stream_grid(vec ? (n + 3) / 4 : n);
   uint8_t* o = static_cast<uint8_t*>(out);
 #define MXQ_Q(U, V) \
   hipLaunchKernelGGL((quantize_kernel<U, V>), dim3(grid), dim3(kThreads), 0, s, in, o, omin, \
-                     omax, n, lo, hi, dlo, dhi)
+                     omax, n, lo, hi, dlo, dhi, slots)
   if (out_type == MXQ_UINT8) {
     if (vec) MXQ_Q(true, true); else MXQ_Q(true, false);
   } else {
@@ -585,22 +581,23 @@ int mxq_quantize_v2(void* stream, const float* in, void* out, float* omin, float
       // Kernel<gpu>::Launch is a no-op for N == 0 (mxnet_op.h:1179): ranges untouched
       return 0;
     }
-    launch_quantize(s, in, out, omin, omax, n, out_type, min_calib, max_calib, nullptr, nullptr);
+    launch_quantize(s, in, out, omin, omax, n, out_type, min_calib, max_calib, nullptr, nullptr,
+                    nullptr);
   } else {
     if (n == 0) return 0;
-    Ws w = carve(workspace, workspace_bytes);
-    hipLaunchKernelGGL(zero_two_kernel, dim3(1), dim3(1), 0, s, w.counter);
+    uint32_t* slots = carve(workspace, workspace_bytes);
+    hipLaunchKernelGGL(init_slots_kernel, dim3(1), dim3(64), 0, s, slots, f2ord_host(INFINITY),
+                       f2ord_host(-INFINITY));
     MXQ_LAUNCH_CHECK();
-    const bool vec = aligned16(in);
-    const int grid = reduce_grid(n);
-    if (vec)
+    const int grid = stream_grid((n + 3) / 4);
+    if (aligned16(in))
       hipLaunchKernelGGL((minmax_f32_kernel<true>), dim3(grid), dim3(kThreads), 0, s, in, n,
-                         w.range, w.counter, static_cast<float*>(w.partial));
+                         slots);
     else
       hipLaunchKernelGGL((minmax_f32_kernel<false>), dim3(grid), dim3(kThreads), 0, s, in, n,
-                         w.range, w.counter, static_cast<float*>(w.partial));
+                         slots);
     MXQ_LAUNCH_CHECK();
-    launch_quantize(s, in, out, omin, omax, n, out_type, 0.f, 0.f, w.range, w.range + 1);
+    launch_quantize(s, in, out, omin, omax, n, out_type, 0.f, 0.f, nullptr, nullptr, slots);
   }
   MXQ_API_END();
 }
@@ -615,7 +612,7 @@ int mxq_quantize(void* stream, const float* in, const float* imin, const float* 
   MXQ_CHECK(n == 0 || (in != nullptr && out != nullptr), "null data pointer");
   if (n == 0) return 0;
   launch_quantize(static_cast<hipStream_t>(stream), in, out, omin, omax, n, out_type, 0.f, 0.f,
-                  imin, imax);
+                  imin, imax, nullptr);
   MXQ_API_END();
 }
 
@@ -657,31 +654,31 @@ int mxq_requantize(void* stream, const int32_t* in, const float* imin, const flo
   const int grid = stream_grid(vec ? (n + 3) / 4 : n);
   uint8_t* o = reinterpret_cast<uint8_t*>(out);
   float real_range = 0.f;
-  const float *dlo = nullptr, *dhi = nullptr;
+  const uint32_t* slots = nullptr;
   if (calibrated) {
     float a = fabsf(min_calib), b = fabsf(max_calib);
     real_range = (a < b) ? b : a;
   } else {
-    Ws w = carve(workspace, workspace_bytes);
-    hipLaunchKernelGGL(zero_two_kernel, dim3(1), dim3(1), 0, s, w.counter);
+    uint32_t* ws = carve(workspace, workspace_bytes);
+    hipLaunchKernelGGL(init_slots_kernel, dim3(1), dim3(64), 0, s, ws,
+                       static_cast<uint32_t>(INT32_MAX), static_cast<uint32_t>(INT32_MIN));
     MXQ_LAUNCH_CHECK();
-    const int rgrid = reduce_grid(n);
+    const int rgrid = stream_grid((n + 3) / 4);
     if (aligned16(in))
       hipLaunchKernelGGL((minmax_i32_kernel<true>), dim3(rgrid), dim3(kThreads), 0, s, in, n,
-                         imin, imax, w.range, w.counter, static_cast<int*>(w.partial));
+                         ws);
     else
       hipLaunchKernelGGL((minmax_i32_kernel<false>), dim3(rgrid), dim3(kThreads), 0, s, in, n,
-                         imin, imax, w.range, w.counter, static_cast<int*>(w.partial));
+                         ws);
     MXQ_LAUNCH_CHECK();
-    dlo = w.range;
-    dhi = w.range + 1;
+    slots = ws;
   }
   if (vec)
     hipLaunchKernelGGL((requantize_kernel<true>), dim3(grid), dim3(kThreads), 0, s, in, o, omin,
-                       omax, n, imin, imax, real_range, dlo, dhi);
+                       omax, n, imin, imax, real_range, slots);
   else
     hipLaunchKernelGGL((requantize_kernel<false>), dim3(grid), dim3(kThreads), 0, s, in, o,
-                       omin, omax, n, imin, imax, real_range, dlo, dhi);
+                       omin, omax, n, imin, imax, real_range, slots);
   MXQ_LAUNCH_CHECK();
   MXQ_API_END();
 }
