@@ -49,10 +49,38 @@ __global__ __launch_bounds__(Cfg::kThreads) void fc_kernel(FcArgs p) {
   if (blockIdx.x == 0 && threadIdx.x == 0) epilogue_ranges(p.epi);
 }
 
+// Direct-to-LDS variant (see gemm_mainloop_dma); launch_fc() picks it when the
+// operands qualify.
+template <class Cfg, int NS, int PIPE>
+__global__ __launch_bounds__(Cfg::kThreads) void fc_dma_kernel(FcArgs p) {
+  __shared__ __attribute__((aligned(16))) v4i lds[NS * Cfg::STAGE_SLOTS];
+  const int tiles_m = (p.M + Cfg::BM - 1) / Cfg::BM, tiles_n = (p.N + Cfg::BN - 1) / Cfg::BN;
+  int tm, tn;
+  tile_coords(blockIdx.x, tiles_m, tiles_n, tm, tn);
+  const int m0 = tm * Cfg::BM, n0 = tn * Cfg::BN;
+
+  v16i acc[Cfg::MI][Cfg::NI];
+  gemm_mainloop_dma<Cfg, NS, PIPE>(acc, p.data, m0, p.M, p.weight, n0, p.N, p.K, lds);
+
+  static_assert(NS * Cfg::STAGE_SLOTS * 16 >=
+                    Cfg::BN * 4 + (Cfg::kThreads / 64) * Cfg::TM * (Cfg::TN + 16),
+                "stage ring too small for the epilogue transpose");
+  gemm_epilogue_lds<Cfg>(acc, p.epi, m0, n0, p.M, p.N, static_cast<size_t>(p.N), lds);
+  if (blockIdx.x == 0 && threadIdx.x == 0) epilogue_ranges(p.epi);
+}
+
 typedef GemmCfg<256, 256, 64, 2, 4> CfgL8;  // 8 waves, wave tile 128 x 64
 typedef GemmCfg<256, 256, 64, 2, 2> CfgL4;  // 4 waves, wave tile 128 x 128
 typedef GemmCfg<128, 128, 64, 2, 2> CfgM;   // 4 waves, wave tile 64 x 64
 typedef GemmCfg<64, 64, 64, 2, 2> CfgS;     // 4 waves, wave tile 32 x 32
+
+template <class Cfg, int NS, int PIPE>
+void launch_dma(hipStream_t s, const FcArgs& a) {
+  const int tiles = ((a.M + Cfg::BM - 1) / Cfg::BM) * ((a.N + Cfg::BN - 1) / Cfg::BN);
+  hipLaunchKernelGGL((fc_dma_kernel<Cfg, NS, PIPE>), dim3(tiles), dim3(Cfg::kThreads), 0, s,
+                     a);
+  MXQ_LAUNCH_CHECK();
+}
 
 template <class Cfg>
 void launch_cfg(hipStream_t s, const FcArgs& a, bool aligned) {
@@ -99,8 +127,25 @@ void launch_fc(hipStream_t s, const int8_t* data, const int8_t* weight, int M, i
       cfg = 3;
     else
       cfg = 4;
+    // large tiles that qualify go straight to LDS: 8 waves when only the int8
+    // output is written, 4 waves (128 x 128 per wave) when int32 is stored as well
+    const bool dma_shape = (K % 16 == 0) && aligned16(data) && aligned16(weight) && K >= 64 &&
+                           (K % 64 == 0) && static_cast<long long>(M) * K < (1LL << 31) &&
+                           static_cast<long long>(N) * K < (1LL << 31);
+    if (cfg == 1 && dma_shape) cfg = (epi.out32 != nullptr) ? 16 : 13;
   }
+  // direct-to-LDS kernels: K a multiple of the 64-byte stage, operands below 2 GiB
+  const bool dma_ok = aligned && K >= 64 && (K % 64 == 0) &&
+                      static_cast<long long>(M) * K < (1LL << 31) &&
+                      static_cast<long long>(N) * K < (1LL << 31);
+  if (cfg >= 11 && cfg <= 18) MXQ_CHECK(dma_ok, "shape does not qualify for the DMA kernels");
   switch (cfg) {
+    case 11: launch_dma<CfgL8, 3, 0>(s, a); break;
+    case 12: launch_dma<CfgL8, 4, 1>(s, a); break;
+    case 13: launch_dma<CfgL8, 4, 2>(s, a); break;
+    case 14: launch_dma<CfgL4, 3, 0>(s, a); break;
+    case 15: launch_dma<CfgL4, 4, 1>(s, a); break;
+    case 16: launch_dma<CfgL4, 4, 2>(s, a); break;
     case 1: launch_cfg<CfgL8>(s, a, aligned); break;
     case 2: launch_cfg<CfgL4>(s, a, aligned); break;
     case 3: launch_cfg<CfgM>(s, a, aligned); break;

@@ -92,16 +92,24 @@ __device__ __forceinline__ int epi_bias32(const Epilogue& e, const EpiScalars& s
   return static_cast<int>(p / s.foq);
 }
 
-// FloatToQuantized<int8>(float(acc) * in_scale) with the sign applied through
-// the float before the truncating convert (trunc is odd; |v| >= 0.5 rounds a
-// zero input to 0 either way).
+// FloatToQuantized<int8>(float(acc) * in_scale): trunc(sign(f) * min(|f|*s + 0.5, 127)).
+// The magnitude v is >= 0.5, so copysign(v, f) followed by the truncating convert
+// equals sign(f) * v truncated, including f == +-0 (trunc(+-0.5) = 0).
 __device__ __forceinline__ int epi_requant(int acc, const EpiScalars& s) {
   float f = static_cast<float>(acc) * s.in_scale;
   float t = fabsf(f) * s.qscale;
   float u = t + 0.5f;
-  float v = (127.0f < u) ? 127.0f : u;
-  int iv = static_cast<int>(v);
-  return (f < 0.0f) ? -iv : ((f > 0.0f) ? iv : 0);
+  float v = fminf(u, 127.0f);
+  return static_cast<int>(copysignf(v, f));
+}
+
+// {a,b,c,d} low bytes -> one dword (a in byte 0).
+__device__ __forceinline__ uint32_t pack_bytes(int a, int b, int c, int d) {
+  const uint32_t lo = __builtin_amdgcn_perm(static_cast<uint32_t>(b), static_cast<uint32_t>(a),
+                                            0x0c0c0400u);
+  const uint32_t hi = __builtin_amdgcn_perm(static_cast<uint32_t>(d), static_cast<uint32_t>(c),
+                                            0x04000c0cu);
+  return lo | hi;
 }
 
 // Bank-spreading XOR for the chunk index.  A fragment read is 32 consecutive
@@ -288,6 +296,211 @@ __device__ __forceinline__ void gemm_mainloop(v16i (&acc)[Cfg::MI][Cfg::NI], AF&
   }
 }
 
+// ---- direct-to-LDS main loop ------------------------------------------------------
+// Fast path for operands whose K is a multiple of BK, 16-byte aligned and below
+// 2 GiB: tiles go from global memory straight into LDS (global_load_lds_dwordx4,
+// no staging registers, no ds_write) through an NS-stage ring.  Each wave
+// instruction fills 64 consecutive 16-byte slots; the bank swizzle is applied on
+// the global side (lane for slot (r, c') fetches chunk c' ^ swz(r) of row r).
+// Rows past the end of the operand are clamped to its last row: they only feed
+// accumulators that the epilogue never stores.
+//
+// The loads are issued through inline assembly, so the compiler's wait-count
+// pass does not see them; completion is enforced here by hand: vmcnt counts
+// them in issue order, and a wave waits until at most the newer stages' loads
+// are outstanding before it joins the work-group barrier that publishes a stage.
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"
+__device__ __forceinline__ void lds_dma16(uint32_t lds_byte_addr, uint32_t voffset,
+                                          const int8_t* sbase) {
+#ifndef MXQ_LAB_SKIP_DMA
+  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2"
+               :
+               : "s"(lds_byte_addr), "v"(voffset), "s"(sbase)
+               : "memory", "m0");
+#endif
+}
+#pragma clang diagnostic pop
+
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+  static_assert(N >= 0 && N < 64, "vmcnt range");
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+
+// Per-thread addressing of one operand for the DMA path.
+template <class Cfg, int INSTR, int ROWS_TILE>
+struct DmaOperand {
+  uint32_t voff[INSTR];  // byte offset of this lane's chunk from the operand base at k = 0
+  __device__ __forceinline__ void init(int row0, int rows, int K, int wave, int lane) {
+    constexpr int NW = Cfg::kThreads / 64;
+#pragma unroll
+    for (int i = 0; i < INSTR; ++i) {
+      const int slot = (i * NW + wave) * 64 + lane;
+      const int r = slot / Cfg::CH;
+      const int c = (slot % Cfg::CH) ^ swz<Cfg::CH>(r);
+      int row = row0 + r;
+      row = row < rows ? row : rows - 1;
+      voff[i] = static_cast<uint32_t>(row) * static_cast<uint32_t>(K) + c * 16;
+    }
+  }
+};
+
+// PIPE selects the software pipeline of the K loop:
+//   0  wait + barrier, issue next DMA, read fragments, MFMA   (compiler scheduled)
+//   1  as 0 plus fragment double-buffering across the barrier (compiler scheduled)
+//   2  as 1 with the instruction order pinned: after every MFMA exactly one
+//      fragment read for the next k-step (and, in the first k-step, one DMA issue)
+//      is placed, so the matrix pipe is fed back-to-back while LDS and DMA work
+//      trickles in between.
+template <class Cfg, int NS, int PIPE>
+__device__ __forceinline__ void gemm_mainloop_dma(v16i (&acc)[Cfg::MI][Cfg::NI],
+                                                  const int8_t* a_base, int a_row0, int a_rows,
+                                                  const int8_t* b_base, int b_row0, int b_rows,
+                                                  int K, v4i* lds) {
+  constexpr int CH = Cfg::CH, NW = Cfg::kThreads / 64;
+  constexpr int AI = Cfg::A_CHUNKS, BI = Cfg::B_CHUNKS, CPT = AI + BI;
+  constexpr int MI = Cfg::MI, NI = Cfg::NI, KS = Cfg::KS;
+  constexpr int STAGE_BYTES = Cfg::STAGE_SLOTS * 16;
+  static_assert((Cfg::BM * CH) % (NW * 64) == 0 && (Cfg::BN * CH) % (NW * 64) == 0, "dma tiling");
+  static_assert(PIPE == 0 || NS >= 4, "cross-barrier fragment prefetch needs 4 stages");
+  static_assert(CH == 4, "fragment addressing below assumes 64-byte stage rows");
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave / Cfg::WN, wn = wave % Cfg::WN;
+
+  DmaOperand<Cfg, AI, Cfg::BM> da;
+  DmaOperand<Cfg, BI, Cfg::BN> db;
+  da.init(a_row0, a_rows, K, wave, lane);
+  db.init(b_row0, b_rows, K, wave, lane);
+  const uint32_t lds0 = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(lds));
+
+  const int KT = K / Cfg::BK;
+  // DMA instruction j (0 .. CPT-1) of a stage
+  auto issue_one = [&](int stage, int j) {
+    const int kk = stage < KT ? stage : KT - 1;  // past the end: harmless reload
+    const uint32_t sb = lds0 + static_cast<uint32_t>(stage % NS) * STAGE_BYTES;
+    if (j < AI)
+      lds_dma16(sb + (j * NW + wave) * 1024, da.voff[j],
+                a_base + static_cast<size_t>(kk) * Cfg::BK);
+    else
+      lds_dma16(sb + Cfg::BM * CH * 16 + ((j - AI) * NW + wave) * 1024, db.voff[j - AI],
+                b_base + static_cast<size_t>(kk) * Cfg::BK);
+  };
+  auto issue = [&](int stage) {
+#pragma unroll
+    for (int j = 0; j < CPT; ++j) issue_one(stage, j);
+  };
+
+  // Fragment addressing.  Row r = tile_row + 32*i + (lane & 31): 32*i does not touch
+  // the row bits swz() looks at, so fragment i sits 32*CH slots after fragment 0, and
+  // k-step ks flips bit 1 of the chunk index (chunk = 2*ks + lane/32).
+  const int frow = lane & 31, fgrp = lane >> 5;
+  const int ra = wm * Cfg::TM + frow, rb = wn * Cfg::TN + frow;
+  int fa0[KS], fb0[KS];
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) {
+    fa0[ks] = ra * CH + ((ks * 2 + fgrp) ^ swz<CH>(ra));
+    fb0[ks] = Cfg::BM * CH + rb * CH + ((ks * 2 + fgrp) ^ swz<CH>(rb));
+  }
+  // fragment f of a k-step: f < MI -> activation fragment f, else weight fragment f-MI
+  auto read_one = [&](int stage, int ks, int f, v4i (&fa)[MI], v4i (&fb)[NI]) {
+#ifndef MXQ_LAB_SKIP_LDSREAD
+    const v4i* st = lds + (stage % NS) * Cfg::STAGE_SLOTS;
+    if (f < MI)
+      fa[f] = st[fa0[ks] + f * 32 * CH];
+    else
+      fb[f - MI] = st[fb0[ks] + (f - MI) * 32 * CH];
+#endif
+  };
+  auto read_frags = [&](int stage, int ks, v4i (&fa)[MI], v4i (&fb)[NI]) {
+#pragma unroll
+    for (int f = 0; f < MI + NI; ++f) read_one(stage, ks, f, fa, fb);
+  };
+  auto mma = [&](v4i (&fa)[MI], v4i (&fb)[NI]) {
+#pragma unroll
+    for (int mi = 0; mi < MI; ++mi)
+#pragma unroll
+      for (int ni = 0; ni < NI; ++ni)
+        acc[mi][ni] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fb[ni], fa[mi], acc[mi][ni], 0, 0, 0);
+  };
+
+#pragma unroll
+  for (int mi = 0; mi < MI; ++mi)
+#pragma unroll
+    for (int ni = 0; ni < NI; ++ni)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[mi][ni][v] = 0;
+
+#pragma unroll
+  for (int s = 0; s < NS - 1; ++s) issue(s);
+
+  if (PIPE == 0) {
+    for (int kt = 0; kt < KT; ++kt) {
+      wait_vmcnt<(NS - 2) * CPT>();     // this wave's part of stage kt has landed
+      __builtin_amdgcn_s_barrier();     // ... and everybody else's; stage kt-1 is free
+      issue(kt + NS - 1);
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        v4i fa[MI], fb[NI];
+        read_frags(kt, ks, fa, fb);
+        mma(fa, fb);
+      }
+    }
+  } else {
+    static_assert(KS % 2 == 0, "fragment ping-pong assumes an even k-step count");
+    v4i fa[2][MI], fb[2][NI];
+    wait_vmcnt<(NS >= 4 ? NS - 3 : 0) * CPT>();  // stages 0 and 1 landed
+    __builtin_amdgcn_s_barrier();
+    read_frags(0, 0, fa[0], fb[0]);
+    for (int kt = 0; kt < KT; ++kt) {
+      if (PIPE == 1) {
+        issue(kt + NS - 1);  // overwrites stage kt-1, consumed before the last barrier
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+          if (ks + 1 < KS)
+            read_frags(kt, ks + 1, fa[(ks + 1) & 1], fb[(ks + 1) & 1]);
+          else
+            read_frags(kt + 1, 0, fa[(ks + 1) & 1], fb[(ks + 1) & 1]);  // published last barrier
+          mma(fa[ks & 1], fb[ks & 1]);
+        }
+      } else {
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+          constexpr int NF = MI + NI;
+          const int cur = ks & 1, nxt = cur ^ 1;
+          const int nstage = (ks + 1 < KS) ? kt : kt + 1;
+          const int nks = (ks + 1 < KS) ? ks + 1 : 0;
+#pragma unroll
+          for (int mi = 0; mi < MI; ++mi) {
+#pragma unroll
+            for (int ni = 0; ni < NI; ++ni) {
+              const int step = mi * NI + ni;
+              acc[mi][ni] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fb[cur][ni], fa[cur][mi],
+                                                                  acc[mi][ni], 0, 0, 0);
+              // spread NF fragment reads (and, in k-step 0, CPT DMA issues) over the
+              // MI*NI MFMA slots of this k-step
+              constexpr int SLOTS = MI * NI;
+#pragma unroll
+              for (int f = 0; f < NF; ++f)
+                if (f * SLOTS / NF == step) read_one(nstage, nks, f, fa[nxt], fb[nxt]);
+              if (ks == 0) {
+#pragma unroll
+                for (int j = 0; j < CPT; ++j)
+                  if (j * SLOTS / CPT == step) issue_one(kt + NS - 1, j);
+              }
+              __builtin_amdgcn_sched_barrier(0);
+            }
+          }
+        }
+      }
+      wait_vmcnt<(NS >= 4 ? NS - 3 : 0) * CPT>();  // stage kt+2 landed for this wave
+      __builtin_amdgcn_s_barrier();
+    }
+  }
+  wait_vmcnt<0>();  // drain the harmless tail loads before LDS is released
+}
+
 // Stores one wave's accumulators.  m_base/n_base: origin of the wave tile.
 template <class Cfg>
 __device__ __forceinline__ void gemm_epilogue(v16i (&acc)[Cfg::MI][Cfg::NI], const Epilogue& e,
@@ -334,9 +547,7 @@ __device__ __forceinline__ void gemm_epilogue(v16i (&acc)[Cfg::MI][Cfg::NI], con
             if (e.relu) q[i] = q[i] > 0 ? q[i] : 0;
           }
           if (full) {
-            uint32_t w = (uint32_t(q[0]) & 0xffu) | ((uint32_t(q[1]) & 0xffu) << 8) |
-                         ((uint32_t(q[2]) & 0xffu) << 16) | (uint32_t(q[3]) << 24);
-            *reinterpret_cast<uint32_t*>(e.out8 + off) = w;
+            *reinterpret_cast<uint32_t*>(e.out8 + off) = pack_bytes(q[0], q[1], q[2], q[3]);
           } else {
 #pragma unroll
             for (int i = 0; i < 4; ++i)
@@ -344,6 +555,90 @@ __device__ __forceinline__ void gemm_epilogue(v16i (&acc)[Cfg::MI][Cfg::NI], con
           }
         }
       }
+    }
+  }
+}
+
+// Epilogue of the direct-to-LDS kernels.  The stage ring is free once the K loop is
+// over, so it is reused to (a) hold the block's int32 bias once and (b) transpose
+// each wave's int8 tile: lanes own 4 adjacent columns of 32 different rows after
+// the MFMA, which would make every store instruction touch 32 cache lines with 8
+// bytes each; staged through LDS a store instruction writes whole 64..128-byte row
+// segments.  Falls back to gemm_epilogue when the output is not 16-byte friendly.
+template <class Cfg>
+__device__ __forceinline__ void gemm_epilogue_lds(v16i (&acc)[Cfg::MI][Cfg::NI],
+                                                  const Epilogue& e, int m0, int n0, int M,
+                                                  int N, size_t ldo, v4i* lds_v) {
+  constexpr int TM = Cfg::TM, TN = Cfg::TN, MI = Cfg::MI, NI = Cfg::NI;
+  constexpr int LD = TN + 16;        // staged row pitch in bytes (keeps 16-byte alignment)
+  constexpr int LPR = TN / 16;       // lanes per staged row on the way out
+  constexpr int RPI = 64 / LPR;      // rows per store instruction
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave / Cfg::WN, wn = wave % Cfg::WN;
+  const int m_base = m0 + wm * TM, n_base = n0 + wn * TN;
+  const bool fast = (N % 16 == 0) && (ldo % 16 == 0) &&
+                    ((reinterpret_cast<uintptr_t>(e.out8) & 15u) == 0);
+  if (!fast) {
+    gemm_epilogue<Cfg>(acc, e, m_base, n_base, M, N, ldo);
+    return;
+  }
+  char* lds = reinterpret_cast<char*>(lds_v);
+  int* sbias = reinterpret_cast<int*>(lds);
+  char* stage = lds + Cfg::BN * 4 + wave * (TM * LD);
+  const EpiScalars s = epi_scalars(e);
+
+  __syncthreads();  // every wave is done reading operand stages
+  for (int t = tid; t < Cfg::BN; t += Cfg::kThreads)
+    sbias[t] = (n0 + t < N) ? epi_bias32(e, s, n0 + t) : 0;
+  __syncthreads();
+
+  const int lrow = lane & 31, lgrp = lane >> 5;
+#pragma unroll
+  for (int ni = 0; ni < NI; ++ni) {
+#pragma unroll
+    for (int vq = 0; vq < 4; ++vq) {
+      const int nl = ni * 32 + 8 * vq + 4 * lgrp;  // column inside the wave tile
+      const v4i b = *reinterpret_cast<const v4i*>(sbias + wn * TN + nl);
+#pragma unroll
+      for (int mi = 0; mi < MI; ++mi) {
+        int v[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          v[i] = static_cast<int>(static_cast<uint32_t>(acc[mi][ni][4 * vq + i]) +
+                                  static_cast<uint32_t>(b[i]));
+        const int ml = mi * 32 + lrow;
+        if (e.out32 != nullptr) {
+          const int m = m_base + ml, n = n_base + nl;
+          if (m < M && n < N) {
+            v4i w = {v[0], v[1], v[2], v[3]};
+            *reinterpret_cast<v4i*>(e.out32 + static_cast<size_t>(m) * ldo + n) = w;
+          }
+        }
+        if (e.out8 != nullptr) {
+          int q[4];
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            q[i] = epi_requant(v[i], s);
+            if (e.relu) q[i] = q[i] > 0 ? q[i] : 0;
+          }
+          *reinterpret_cast<uint32_t*>(stage + ml * LD + nl) = pack_bytes(q[0], q[1], q[2], q[3]);
+        }
+      }
+    }
+  }
+  if (e.out8 != nullptr) {
+    // the wave reads back what its own lanes wrote: LDS executes a wave's
+    // instructions in order, the wait makes the writes complete first
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int it = 0; it < TM / RPI; ++it) {
+      const int rr = it * RPI + lane / LPR, c16 = lane % LPR;
+      const v4i val = *reinterpret_cast<const v4i*>(stage + rr * LD + c16 * 16);
+      const int m = m_base + rr, n = n_base + c16 * 16;
+      if (m < M && n < N)
+        *reinterpret_cast<v4i*>(e.out8 + static_cast<size_t>(m) * ldo + n) = val;
     }
   }
 }
