@@ -84,6 +84,13 @@ int mxq_requantize(void* stream, const int32_t* in, const float* imin, const flo
 int mxq_dequantize(void* stream, const void* in, int in_type, const float* imin,
                    const float* imax, float* out, size_t n);
 
+/* ---- _contrib_quantized_act (relu) -----------------------------------------
+ * int8 max(x, 0); the range passes through unchanged
+ * (src/operator/quantization/quantized_activation.cc:84-120, CPU-only in the
+ * reference through dnnl/dnnl_quantized_act.cc:33-45). */
+int mxq_quantized_relu(void* stream, const int8_t* in, const float* imin, const float* imax,
+                       int8_t* out, float* omin, float* omax, size_t n);
+
 /* ---- _contrib_quantized_fully_connected ----------------------------------
  * Replaces QuantizedFullyConnectedForwardGPU
  * (src/operator/quantization/quantized_fully_connected.cu:58-138): cublasGemmEx

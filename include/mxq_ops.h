@@ -1,0 +1,67 @@
+/*
+ * mxq_ops.h - C entry points of libmxq_ops.so, the C++ operator host library.
+ *
+ * libmxq_ops.so holds the NNVM-style registry with the INT8 operators registered
+ * under the reference's names and the FCompute<gpu> / FStatefulCompute<gpu> host
+ * functions, which call libmxq_hip.so (mxq.h).  The functions below are the small
+ * imperative front door a test harness or a language binding uses to drive one
+ * operator: they play the role of MXImperativeInvoke
+ * (src/c_api/c_api_ndarray.cc:146 in the reference: parse attributes, infer shape
+ * and type, hand TBlobs + OpContext to the registered compute function) without
+ * the engine, NDArray and storage layers around it.  The caller owns all memory.
+ * Return 0 on success, -1 on failure with the text in mxq_ops_last_error().
+ */
+#ifndef MXQ_OPS_H_
+#define MXQ_OPS_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MXQ_MAX_NDIM 8
+
+/* One tensor argument: device pointer, shape, mshadow type flag (mxq.h codes). */
+typedef struct {
+  void* data;
+  int ndim;
+  int64_t shape[MXQ_MAX_NDIM];
+  int dtype;
+} mxq_blob;
+
+const char* mxq_ops_last_error(void);
+
+/* registry introspection */
+int mxq_op_count(void);
+const char* mxq_op_name(int index);
+/* 1 if `op` (name or alias) has the attribute key, e.g. "FCompute<gpu>". */
+int mxq_op_has_attr(const char* op, const char* key);
+
+/* A node = operator + parsed attribute dict (nnvm::NodeAttrs). */
+int mxq_node_create(const char* op, const char* node_name, int num_attrs, const char** keys,
+                    const char** values, void** out_node);
+int mxq_node_free(void* node);
+int mxq_node_num_inputs(void* node, int* out);
+int mxq_node_num_outputs(void* node, int* out);
+/* comma-separated names; the string lives as long as the node */
+int mxq_node_input_names(void* node, const char** out);
+int mxq_node_output_names(void* node, const char** out);
+
+/* FInferShape / FInferType: unknown shapes have ndim -1, unknown types are -1;
+ * both arrays are updated in place. */
+int mxq_node_infer_shape(void* node, int num_in, int* in_ndim, int64_t* in_shape, int num_out,
+                         int* out_ndim, int64_t* out_shape);
+int mxq_node_infer_type(void* node, int num_in, int* in_type, int num_out, int* out_type);
+/* bytes of ResourceRequest::kTempSpace the node will ask for (0 if none) */
+int mxq_node_temp_bytes(void* node, int num_in, const mxq_blob* in, int num_out,
+                        const mxq_blob* out, size_t* bytes);
+/* runs FCompute<gpu> or FCreateOpState + FStatefulCompute<gpu> on `stream` */
+int mxq_node_forward(void* node, void* stream, int dev_id, int num_in, const mxq_blob* in,
+                     int num_out, const mxq_blob* out, void* temp_space, size_t temp_bytes);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MXQ_OPS_H_ */

@@ -7,5 +7,7 @@ include/mxq.h).  This package is the host-side mirror of the reference operator
 interface; torch is used only to own device memory and streams."""
 from . import _lib  # noqa: F401  (fails loudly if the HIP library is missing)
 from . import capi  # noqa: F401
+from . import operator  # noqa: F401  (loads the C++ operator host, libmxq_ops.so)
+from . import contrib  # noqa: F401
 
-__all__ = ["capi"]
+__all__ = ["capi", "operator", "contrib"]

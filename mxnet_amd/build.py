@@ -54,5 +54,26 @@ def build(verbose=False):
     return LIB
 
 
+OPS_LIB = os.path.join(HERE, "libmxq_ops.so")
+HOST_SOURCES = ["mxq_registry.cc", "mxq_quantization_ops.cc", "mxq_harness.cc"]
+
+
+def build_ops(verbose=False):
+    """libmxq_ops.so: the C++ operator host (registry + FCompute<gpu> functions).  Plain
+    C++17, no HIP headers: it reaches the GPU only through libmxq_hip.so's C ABI."""
+    cxx = os.environ.get("CXX", "g++")
+    srcs = [os.path.join(CSRC, "host", s) for s in HOST_SOURCES]
+    cmd = [cxx, "-O2", "-std=c++17", "-fPIC", "-shared", "-Wall", "-Wextra",
+           "-Wno-unused-parameter", "-o", OPS_LIB] + srcs + \
+          ["-L" + HERE, "-lmxq_hip", "-Wl,-rpath,$ORIGIN"]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    subprocess.check_call(cmd)
+    return OPS_LIB
+
+
 if __name__ == "__main__":
+    build(verbose="-v" in sys.argv)
+    print(build_ops(verbose="-v" in sys.argv))
+    sys.exit(0)
     print(build(verbose="-v" in sys.argv))

@@ -1,0 +1,52 @@
+"""The reference's imperative operator names: `mxnet_amd.contrib.quantize_v2(...)`
+reads like `mx.nd.contrib.quantize_v2(...)` (and the `_npx_*` aliases like
+`mx.npx.requantize`).  Same positional tensors, same keyword attributes, same
+outputs; everything runs through the C++ operator host."""
+from .operator import invoke
+
+
+def quantize(data, min_range, max_range, out_type="uint8"):
+    return invoke("_contrib_quantize", data, min_range, max_range, out_type=out_type)
+
+
+def quantize_v2(data, out_type="int8", min_calib_range=None, max_calib_range=None):
+    return invoke("_contrib_quantize_v2", data, out_type=out_type,
+                  min_calib_range=min_calib_range, max_calib_range=max_calib_range)
+
+
+def requantize(data, min_range, max_range, out_type="int8", min_calib_range=None,
+               max_calib_range=None):
+    return invoke("_contrib_requantize", data, min_range, max_range, out_type=out_type,
+                  min_calib_range=min_calib_range, max_calib_range=max_calib_range)
+
+
+def dequantize(data, min_range, max_range, out_type="float32"):
+    return invoke("_contrib_dequantize", data, min_range, max_range, out_type=out_type)
+
+
+def quantized_fully_connected(data, weight, bias=None, min_data=None, max_data=None,
+                              min_weight=None, max_weight=None, min_bias=None, max_bias=None,
+                              num_hidden=None, no_bias=False, flatten=True):
+    ins = [data, weight] + ([] if no_bias else [bias]) + [min_data, max_data, min_weight,
+                                                          max_weight]
+    if not no_bias:
+        ins += [min_bias, max_bias]
+    return invoke("_contrib_quantized_fully_connected", *ins, num_hidden=num_hidden,
+                  no_bias=no_bias, flatten=flatten)
+
+
+def quantized_conv(data, weight, bias=None, min_data=None, max_data=None, min_weight=None,
+                   max_weight=None, min_bias=None, max_bias=None, kernel=None, stride=None,
+                   dilate=None, pad=None, num_filter=None, num_group=1, no_bias=False,
+                   layout=None):
+    ins = [data, weight] + ([] if no_bias else [bias]) + [min_data, max_data, min_weight,
+                                                          max_weight]
+    if not no_bias:
+        ins += [min_bias, max_bias]
+    return invoke("_contrib_quantized_conv", *ins, kernel=kernel, stride=stride, dilate=dilate,
+                  pad=pad, num_filter=num_filter, num_group=num_group, no_bias=no_bias,
+                  layout=layout)
+
+
+def quantized_act(data, min_data, max_data, act_type="relu"):
+    return invoke("_contrib_quantized_act", data, min_data, max_data, act_type=act_type)

@@ -1,0 +1,406 @@
+// Attribute structs of the quantization operators, parsed from the string dict of
+// a node exactly as dmlc::Parameter<...>::Init does for the reference structs:
+//   QuantizeV2Param        src/operator/quantization/quantize_v2-inl.h:39-63
+//   QuantizeParam (v1)     src/operator/quantization/quantize-inl.h:39-48
+//   RequantizeParam        src/operator/quantization/requantize-inl.h:39-65
+//   DequantizeParam        src/operator/quantization/dequantize-inl.h:38-46
+//   FullyConnectedParam    src/operator/nn/fully_connected-inl.h:70-82
+//   ConvolutionParam       src/operator/nn/convolution-inl.h:56-112 (+ the defaults
+//                          ConvolutionParamParser fills, src/operator/nn/convolution.cc:366-416)
+//   ActivationParam        src/operator/nn/activation-inl.h (act_type only)
+// Same field names, defaults, enum strings and error behaviour (unknown keys are
+// errors unless they look like __hidden__ keys).
+#ifndef MXQ_PARAMS_H_
+#define MXQ_PARAMS_H_
+
+#include <cctype>
+#include <cstdlib>
+#include <map>
+#include <set>
+#include <string>
+#include <unordered_map>
+#include <vector>
+
+#include "mxq_shim.h"
+
+namespace mxnet {
+namespace op {
+
+enum QuantizeOutType { kAuto = 0, kInt8, kUint8 };
+
+namespace param_detail {
+
+typedef std::unordered_map<std::string, std::string> Dict;
+
+inline std::string trim(const std::string& s) {
+  size_t b = 0, e = s.size();
+  while (b < e && std::isspace(static_cast<unsigned char>(s[b]))) ++b;
+  while (e > b && std::isspace(static_cast<unsigned char>(s[e - 1]))) --e;
+  return s.substr(b, e - b);
+}
+
+inline bool is_hidden(const std::string& k) {
+  return k.size() > 4 && k.compare(0, 2, "__") == 0 && k.compare(k.size() - 2, 2, "__") == 0;
+}
+
+// Fails for keys that no field consumed (dmlc::Parameter::Init, kAllowHidden).
+inline void check_unknown(const Dict& d, const std::set<std::string>& known,
+                          const char* struct_name) {
+  for (const auto& kv : d) {
+    if (known.count(kv.first) || is_hidden(kv.first)) continue;
+    std::ostringstream os;
+    os << "Cannot find argument '" << kv.first << "', Possible Arguments:\n----------------\n";
+    for (const auto& k : known) os << k << "\n";
+    os << "(in " << struct_name << ")";
+    throw dmlc::ParamError(os.str());
+  }
+}
+
+inline bool parse_float(const std::string& raw, float* out) {
+  const std::string s = trim(raw);
+  if (s.empty()) return false;
+  char* end = nullptr;
+  const float v = std::strtof(s.c_str(), &end);
+  if (end == s.c_str()) return false;
+  while (*end && std::isspace(static_cast<unsigned char>(*end))) ++end;
+  if (*end == 'f' || *end == 'F') ++end;
+  if (*end) return false;
+  *out = v;
+  return true;
+}
+
+inline bool parse_int(const std::string& raw, long long* out) {
+  const std::string s = trim(raw);
+  if (s.empty()) return false;
+  char* end = nullptr;
+  const long long v = std::strtoll(s.c_str(), &end, 10);
+  if (end == s.c_str()) return false;
+  if (*end == 'L' || *end == 'l') ++end;
+  if (*end) return false;
+  *out = v;
+  return true;
+}
+
+inline void bad_value(const std::string& key, const std::string& value, const std::string& why) {
+  std::ostringstream os;
+  os << "Invalid Parameter format for " << key << " expect " << why << " but value='" << value
+     << "'";
+  throw dmlc::ParamError(os.str());
+}
+
+inline bool get_bool(const Dict& d, const std::string& key, bool def) {
+  auto it = d.find(key);
+  if (it == d.end()) return def;
+  std::string s = trim(it->second);
+  for (auto& c : s) c = static_cast<char>(std::tolower(static_cast<unsigned char>(c)));
+  if (s == "true" || s == "1") return true;
+  if (s == "false" || s == "0") return false;
+  bad_value(key, it->second, "boolean");
+  return def;
+}
+
+inline dmlc::optional<float> get_optional_float(const Dict& d, const std::string& key) {
+  auto it = d.find(key);
+  if (it == d.end()) return dmlc::optional<float>();
+  const std::string s = trim(it->second);
+  if (s == "None") return dmlc::optional<float>();
+  float v;
+  if (!parse_float(s, &v)) bad_value(key, it->second, "float or None");
+  return dmlc::optional<float>(v);
+}
+
+inline int get_enum(const Dict& d, const std::string& key,
+                    const std::vector<std::pair<std::string, int>>& names, bool has_def, int def,
+                    bool* present = nullptr) {
+  auto it = d.find(key);
+  if (present) *present = it != d.end();
+  if (it == d.end()) {
+    if (!has_def) throw dmlc::ParamError("Required parameter " + key + " is not presented");
+    return def;
+  }
+  const std::string s = trim(it->second);
+  for (const auto& n : names)
+    if (n.first == s) return n.second;
+  std::ostringstream why;
+  why << "{";
+  for (size_t i = 0; i < names.size(); ++i) why << (i ? ", " : "") << "'" << names[i].first << "'";
+  why << "}";
+  bad_value(key, it->second, why.str());
+  return def;
+}
+
+inline long long get_int(const Dict& d, const std::string& key, bool has_def, long long def,
+                         bool has_lower, long long lower) {
+  auto it = d.find(key);
+  if (it == d.end()) {
+    if (!has_def) throw dmlc::ParamError("Required parameter " + key + " is not presented");
+    return def;
+  }
+  long long v;
+  if (!parse_int(it->second, &v)) bad_value(key, it->second, "int");
+  if (has_lower && v < lower) {
+    std::ostringstream os;
+    os << "value " << v << " for Parameter " << key << " should be greater equal to " << lower;
+    throw dmlc::ParamError(os.str());
+  }
+  return v;
+}
+
+// Tuple text forms accepted by mxnet::Tuple's operator>> (include/mxnet/tuple.h:296-369):
+// "(a, b)", "[a,b]", a bare integer, "None", "()" / "[]".
+inline TShape get_shape(const Dict& d, const std::string& key, bool has_def) {
+  auto it = d.find(key);
+  if (it == d.end()) {
+    if (!has_def) throw dmlc::ParamError("Required parameter " + key + " is not presented");
+    return TShape(0, 0);
+  }
+  std::string s = trim(it->second);
+  if (s == "None") return TShape();
+  std::vector<index_t> v;
+  if (!s.empty() && (s[0] == '(' || s[0] == '[')) {
+    const char close = s[0] == '(' ? ')' : ']';
+    if (s.back() != close) bad_value(key, it->second, "Shape(tuple)");
+    s = s.substr(1, s.size() - 2);
+    size_t pos = 0;
+    while (pos <= s.size()) {
+      size_t comma = s.find(',', pos);
+      std::string tok = trim(s.substr(pos, comma == std::string::npos ? comma : comma - pos));
+      if (!tok.empty()) {
+        long long x;
+        if (!parse_int(tok, &x)) bad_value(key, it->second, "Shape(tuple)");
+        v.push_back(x);
+      }
+      if (comma == std::string::npos) break;
+      pos = comma + 1;
+    }
+  } else {
+    long long x;
+    if (!parse_int(s, &x)) bad_value(key, it->second, "Shape(tuple)");
+    v.push_back(x);
+  }
+  return TShape(v);
+}
+
+}  // namespace param_detail
+
+static const std::vector<std::pair<std::string, int>> kQuantizeOutTypeNames = {
+    {"auto", kAuto}, {"int8", kInt8}, {"uint8", kUint8}};
+
+struct QuantizeV2Param {
+  int out_type = kInt8;
+  dmlc::optional<float> min_calib_range;
+  dmlc::optional<float> max_calib_range;
+  void Init(const param_detail::Dict& d) {
+    using namespace param_detail;
+    check_unknown(d, {"out_type", "min_calib_range", "max_calib_range"}, "QuantizeV2Param");
+    out_type = get_enum(d, "out_type", kQuantizeOutTypeNames, true, kInt8);
+    min_calib_range = get_optional_float(d, "min_calib_range");
+    max_calib_range = get_optional_float(d, "max_calib_range");
+  }
+  static std::vector<nnvm::ParamFieldInfo> __FIELDS__() {
+    return {{"out_type", "{'auto', 'int8', 'uint8'},optional, default='int8'",
+             "Output data type. `auto` can be specified to automatically determine output type "
+             "according to min_calib_range."},
+            {"min_calib_range", "float or None, optional, default=None",
+             "The minimum scalar value in the form of float32. If present, it will be used to "
+             "quantize the fp32 data into int8 or uint8."},
+            {"max_calib_range", "float or None, optional, default=None",
+             "The maximum scalar value in the form of float32. If present, it will be used to "
+             "quantize the fp32 data into int8 or uint8."}};
+  }
+};
+
+struct RequantizeParam {
+  int out_type = kInt8;
+  dmlc::optional<float> min_calib_range;
+  dmlc::optional<float> max_calib_range;
+  void Init(const param_detail::Dict& d) {
+    using namespace param_detail;
+    check_unknown(d, {"out_type", "min_calib_range", "max_calib_range"}, "RequantizeParam");
+    out_type = get_enum(d, "out_type", kQuantizeOutTypeNames, true, kInt8);
+    min_calib_range = get_optional_float(d, "min_calib_range");
+    max_calib_range = get_optional_float(d, "max_calib_range");
+  }
+  static std::vector<nnvm::ParamFieldInfo> __FIELDS__() {
+    return {{"out_type", "{'auto', 'int8', 'uint8'},optional, default='int8'",
+             "Output data type. `auto` can be specified to automatically determine output type "
+             "according to min_calib_range."},
+            {"min_calib_range", "float or None, optional, default=None",
+             "The minimum scalar value in the form of float32 obtained through calibration. If "
+             "present, it will be used to requantize the int32 data into int8."},
+            {"max_calib_range", "float or None, optional, default=None",
+             "The maximum scalar value in the form of float32 obtained through calibration. If "
+             "present, it will be used to requantize the int32 data into int8."}};
+  }
+};
+
+// v1 _contrib_quantize: out_type in {int8, uint8}, default uint8
+struct QuantizeParam {
+  int out_type = mshadow::kUint8;
+  void Init(const param_detail::Dict& d) {
+    using namespace param_detail;
+    check_unknown(d, {"out_type"}, "QuantizeParam");
+    out_type = get_enum(d, "out_type", {{"int8", mshadow::kInt8}, {"uint8", mshadow::kUint8}},
+                        true, mshadow::kUint8);
+  }
+  static std::vector<nnvm::ParamFieldInfo> __FIELDS__() {
+    return {{"out_type", "{'int8', 'uint8'},optional, default='uint8'", "Output data type."}};
+  }
+};
+
+struct DequantizeParam {
+  int out_type = mshadow::kFloat32;
+  void Init(const param_detail::Dict& d) {
+    using namespace param_detail;
+    check_unknown(d, {"out_type"}, "DequantizeParam");
+    out_type = get_enum(d, "out_type", {{"float32", mshadow::kFloat32}}, true, mshadow::kFloat32);
+  }
+  static std::vector<nnvm::ParamFieldInfo> __FIELDS__() {
+    return {{"out_type", "{'float32'},optional, default='float32'", "Output data type."}};
+  }
+};
+
+struct FullyConnectedParam {
+  int num_hidden = 0;
+  bool no_bias = false;
+  bool flatten = true;
+  void Init(const param_detail::Dict& d) {
+    using namespace param_detail;
+    check_unknown(d, {"num_hidden", "no_bias", "flatten"}, "FullyConnectedParam");
+    num_hidden = static_cast<int>(get_int(d, "num_hidden", false, 0, true, 1));
+    no_bias = get_bool(d, "no_bias", false);
+    flatten = get_bool(d, "flatten", true);
+  }
+  static std::vector<nnvm::ParamFieldInfo> __FIELDS__() {
+    return {{"num_hidden", "int, required", "Number of hidden nodes of the output."},
+            {"no_bias", "boolean, optional, default=0", "Whether to disable bias parameter."},
+            {"flatten", "boolean, optional, default=1",
+             "Whether to collapse all but the first axis of the input data tensor."}};
+  }
+};
+
+struct ConvolutionParam {
+  TShape kernel, stride, dilate, pad;
+  uint32_t num_filter = 0;
+  uint32_t num_group = 1;
+  uint64_t workspace = 1024;
+  bool no_bias = false;
+  dmlc::optional<int> cudnn_tune;
+  bool cudnn_off = false;
+  dmlc::optional<int> layout;
+  void Init(const param_detail::Dict& d) {
+    using namespace param_detail;
+    check_unknown(d, {"kernel", "stride", "dilate", "pad", "num_filter", "num_group", "workspace",
+                      "no_bias", "cudnn_tune", "cudnn_off", "layout"},
+                  "ConvolutionParam");
+    kernel = get_shape(d, "kernel", false);
+    stride = get_shape(d, "stride", true);
+    dilate = get_shape(d, "dilate", true);
+    pad = get_shape(d, "pad", true);
+    num_filter = static_cast<uint32_t>(get_int(d, "num_filter", false, 0, true, 1));
+    num_group = static_cast<uint32_t>(get_int(d, "num_group", true, 1, false, 0));
+    workspace = static_cast<uint64_t>(get_int(d, "workspace", true, 1024, true, 0));
+    no_bias = get_bool(d, "no_bias", false);
+    cudnn_off = get_bool(d, "cudnn_off", false);
+    bool present = false;
+    auto none_or = [&](const std::string& key,
+                       const std::vector<std::pair<std::string, int>>& names) {
+      auto it = d.find(key);
+      if (it == d.end() || trim(it->second) == "None") return dmlc::optional<int>();
+      return dmlc::optional<int>(get_enum(d, key, names, true, 0, &present));
+    };
+    cudnn_tune = none_or("cudnn_tune", {{"off", 0}, {"limited_workspace", 1}, {"fastest", 2}});
+    layout = none_or("layout", {{"NCW", mshadow::kNCW},
+                                {"NCHW", mshadow::kNCHW},
+                                {"NCDHW", mshadow::kNCDHW},
+                                {"NWC", mshadow::kNWC},
+                                {"NHWC", mshadow::kNHWC},
+                                {"NDHWC", mshadow::kNDHWC}});
+  }
+  index_t DilatedKernelSize(int dim) const { return 1 + (kernel[dim] - 1) * dilate[dim]; }
+  static std::vector<nnvm::ParamFieldInfo> __FIELDS__() {
+    return {{"kernel", "Shape(tuple), required", "Convolution kernel size: (w,), (h, w) or (d, h, w)"},
+            {"stride", "Shape(tuple), optional, default=[]", "Convolution stride"},
+            {"dilate", "Shape(tuple), optional, default=[]", "Convolution dilate"},
+            {"pad", "Shape(tuple), optional, default=[]", "Zero pad for convolution"},
+            {"num_filter", "int (non-negative), required", "Convolution filter(channel) number"},
+            {"num_group", "int (non-negative), optional, default=1", "Number of group partitions."},
+            {"workspace", "long (non-negative), optional, default=1024",
+             "Maximum temporary workspace allowed (MB) in convolution."},
+            {"no_bias", "boolean, optional, default=0", "Whether to disable bias parameter."},
+            {"cudnn_tune", "{None, 'fastest', 'limited_workspace', 'off'},optional, default='None'",
+             "Whether to pick convolution algo by running performance test."},
+            {"cudnn_off", "boolean, optional, default=0", "Turn off cudnn for this layer."},
+            {"layout", "{None, 'NCDHW', 'NCHW', 'NCW', 'NDHWC', 'NHWC', 'NWC'},optional, "
+                       "default='None'",
+             "Set layout for input, output and weight."}};
+  }
+};
+
+namespace activation {
+enum ActivationOpType { kReLU, kSigmoid, kTanh, kSoftReLU, kSoftSign };
+}
+struct ActivationParam {
+  int act_type = activation::kReLU;
+  void Init(const param_detail::Dict& d) {
+    using namespace param_detail;
+    check_unknown(d, {"act_type"}, "ActivationParam");
+    act_type = get_enum(d, "act_type",
+                        {{"relu", activation::kReLU},
+                         {"sigmoid", activation::kSigmoid},
+                         {"tanh", activation::kTanh},
+                         {"softrelu", activation::kSoftReLU},
+                         {"softsign", activation::kSoftSign}},
+                        false, 0);
+  }
+  static std::vector<nnvm::ParamFieldInfo> __FIELDS__() {
+    return {{"act_type", "{'relu', 'sigmoid', 'softrelu', 'softsign', 'tanh'}, required",
+             "Activation function to be applied."}};
+  }
+};
+
+// src/operator/operator_common.h:478-495
+template <typename PType>
+inline void ParamParser(nnvm::NodeAttrs* attrs) {
+  PType param;
+  try {
+    param.Init(attrs->dict);
+  } catch (const dmlc::ParamError& e) {
+    std::ostringstream os;
+    os << e.what();
+    os << ", in operator " << attrs->op->name << "("
+       << "name=\"" << attrs->name << "\"";
+    for (const auto& k : attrs->dict) os << ", " << k.first << "=\"" << k.second << "\"";
+    os << ")";
+    throw dmlc::ParamError(os.str());
+  }
+  attrs->parsed = std::move(param);
+}
+
+// src/operator/nn/convolution.cc:366-416 (2-D and 1-D/3-D defaults)
+inline void ConvolutionParamParser(nnvm::NodeAttrs* attrs) {
+  ParamParser<ConvolutionParam>(attrs);
+  ConvolutionParam param_ = nnvm::get<ConvolutionParam>(attrs->parsed);
+  const int nd = param_.kernel.ndim();
+  CHECK(nd >= 1 && nd <= 3) << nd << "D convolution not supported";
+  const int def_layout = nd == 1 ? mshadow::kNCW : (nd == 2 ? mshadow::kNCHW : mshadow::kNCDHW);
+  param_.layout = param_.layout ? param_.layout.value() : def_layout;
+  if (param_.stride.ndim() == 0) param_.stride = TShape(nd, 1);
+  if (param_.dilate.ndim() == 0) param_.dilate = TShape(nd, 1);
+  if (param_.pad.ndim() == 0) param_.pad = TShape(nd, 0);
+  CHECK_EQ(param_.kernel.ndim(), param_.stride.ndim())
+      << "Stride must have the same number of dimensions with kernel_size,"
+      << "but kernel_size is set to " << param_.kernel << " while stride is " << param_.stride;
+  CHECK_EQ(param_.kernel.ndim(), param_.dilate.ndim())
+      << "Dilate must have the same number of dimensions with kernel_size,"
+      << "but kernel_size is set to " << param_.kernel << " while dilate is " << param_.dilate;
+  CHECK_EQ(param_.kernel.ndim(), param_.pad.ndim())
+      << "Padding must have the same number of dimensions with kernel_size,"
+      << "but kernel_size is set to " << param_.kernel << " while padding is " << param_.pad;
+  attrs->parsed = std::move(param_);
+}
+
+}  // namespace op
+}  // namespace mxnet
+
+#endif  // MXQ_PARAMS_H_

@@ -1,0 +1,736 @@
+// Host side of the INT8 operators for the gpu device: attribute parsing, shape /
+// type inference and the FCompute<gpu> / FStatefulCompute<gpu> functions, attached
+// to the NNVM registry under the reference's operator names.  Every compute
+// function only unpacks TBlobs, attributes, the stream and the temp space and calls
+// the C ABI of libmxq_hip.so (include/mxq.h); no kernel is launched from here.
+//
+// Reference registrations this file mirrors (names, aliases, argument order,
+// attributes, resource requests):
+//   _contrib_quantize_v2                 quantize_v2.cc:68-138, quantize_v2.cu:29-30
+//   _contrib_quantize                    quantize.cc:67-124, quantize.cu
+//   _contrib_requantize                  requantize.cc:71-124, requantize.cu:29
+//   _contrib_dequantize                  dequantize.cc:65-110, dequantize.cu:29-30
+//   _contrib_quantized_fully_connected   quantized_fully_connected.cc:317-382, .cu:141-143
+//   _contrib_quantized_conv              quantized_conv.cc:176-237, .cu:293-294
+//   _contrib_quantized_act               quantized_activation.cc:84-120
+// (all under src/operator/quantization/).  Inside MXNet only the "<gpu>" attributes
+// of this file would be compiled (the CPU .cc files already register the rest).
+#include <algorithm>
+#include <cmath>
+#include <string>
+#include <vector>
+
+#include "../../../include/mxq.h"
+#include "mxq_params.h"
+#include "mxq_shim.h"
+
+namespace mxnet {
+namespace op {
+
+using mshadow::gpu;
+
+namespace {
+
+// Non-zero return code of the launcher -> the exception MXNet's CHECK would raise.
+inline void MXQ_CALL(int rc) {
+  if (rc != 0) throw dmlc::Error(std::string("libmxq_hip: ") + mxq_last_error());
+}
+
+inline void* raw_stream(const OpContext& ctx) {
+  mshadow::Stream<gpu>* s = ctx.get_stream<gpu>();
+  return s ? s->stream_ : nullptr;
+}
+
+// quantization_utils.h:201-220
+template <typename Param>
+int GetQuantizeOutputType(const Param& param) {
+  if (param.out_type == kAuto) {
+    if (param.min_calib_range.has_value() && param.max_calib_range.has_value() &&
+        param.min_calib_range.value() >= 0.0)
+      return mshadow::kUint8;
+    return mshadow::kInt8;
+  }
+  if (param.out_type == kInt8) return mshadow::kInt8;
+  if (param.out_type == kUint8) return mshadow::kUint8;
+  LOG_FATAL << "Unsupported out_type in params: " << param.out_type;
+  return mshadow::kInt8;
+}
+
+const TShape kScalarShape{1};
+
+}  // namespace
+
+// ---- shape / type inference ---------------------------------------------------------
+
+// quantize_v2-inl.h:129-147: 1 input, outputs (data-shaped, (1,), (1,)); the batch
+// dimension flows back from the output to the input.
+static bool QuantizeV2Shape(const NodeAttrs&, ShapeVector* in, ShapeVector* out) {
+  CHECK_EQ(in->size(), 1U);
+  CHECK_EQ(out->size(), 3U);
+  TShape d = (*in)[0];
+  SHAPE_ASSIGN_CHECK(*out, 0, (*in)[0]);
+  SHAPE_ASSIGN_CHECK(*out, 1, kScalarShape);
+  SHAPE_ASSIGN_CHECK(*out, 2, kScalarShape);
+  if ((*out)[0].ndim() > 0 && d.ndim() > 0) {
+    d[0] = (*out)[0][0];
+    SHAPE_ASSIGN_CHECK(*in, 0, d);
+  }
+  return !shape_is_none((*out)[0]);
+}
+
+// quantize_v2-inl.h:149-179 (the non-oneDNN branch: fp32, uint8 or int8 input)
+static bool QuantizeV2Type(const NodeAttrs& attrs, std::vector<int>* in, std::vector<int>* out) {
+  CHECK_EQ(in->size(), 1U);
+  CHECK_EQ(out->size(), 3U);
+  const auto& param = nnvm::get<QuantizeV2Param>(attrs.parsed);
+  const int t = (*in)[0];
+  CHECK(t == mshadow::kFloat32 || t == mshadow::kUint8 || t == mshadow::kInt8 || t == -1)
+      << "quantize_v2 only supports float32, uint8 and int8 input, got " << type_string(t);
+  TYPE_ASSIGN_CHECK(*out, 0, GetQuantizeOutputType(param));
+  TYPE_ASSIGN_CHECK(*out, 1, mshadow::kFloat32);
+  TYPE_ASSIGN_CHECK(*out, 2, mshadow::kFloat32);
+  return t != -1;
+}
+
+// quantize-inl.h:133-154, shared by _contrib_quantize and _contrib_requantize
+static bool QuantizeShape(const NodeAttrs&, ShapeVector* in, ShapeVector* out) {
+  CHECK_EQ(in->size(), 3U);
+  CHECK_EQ(out->size(), 3U);
+  TShape d = (*in)[0];
+  SHAPE_ASSIGN_CHECK(*in, 1, kScalarShape);
+  SHAPE_ASSIGN_CHECK(*in, 2, kScalarShape);
+  SHAPE_ASSIGN_CHECK(*out, 0, (*in)[0]);
+  SHAPE_ASSIGN_CHECK(*out, 1, kScalarShape);
+  SHAPE_ASSIGN_CHECK(*out, 2, kScalarShape);
+  if ((*out)[0].ndim() > 0 && d.ndim() > 0) {
+    d[0] = (*out)[0][0];
+    SHAPE_ASSIGN_CHECK(*in, 0, d);
+  }
+  return shape_is_known((*out)[0]);
+}
+
+// quantize-inl.h:156-176
+static bool QuantizeType(const NodeAttrs& attrs, std::vector<int>* in, std::vector<int>* out) {
+  CHECK_EQ(in->size(), 3U);
+  CHECK_EQ(out->size(), 3U);
+  const auto& param = nnvm::get<QuantizeParam>(attrs.parsed);
+  TYPE_ASSIGN_CHECK(*in, 0, mshadow::kFloat32);
+  TYPE_ASSIGN_CHECK(*in, 1, mshadow::kFloat32);
+  TYPE_ASSIGN_CHECK(*in, 2, mshadow::kFloat32);
+  CHECK(param.out_type == mshadow::kInt8 || param.out_type == mshadow::kUint8)
+      << "quantize op only supports int8 and uint8 as output type";
+  TYPE_ASSIGN_CHECK(*out, 0, param.out_type);
+  TYPE_ASSIGN_CHECK(*out, 1, mshadow::kFloat32);
+  TYPE_ASSIGN_CHECK(*out, 2, mshadow::kFloat32);
+  return (*in)[0] != -1;
+}
+
+// requantize-inl.h:67-87
+static bool RequantizeType(const NodeAttrs& attrs, std::vector<int>* in, std::vector<int>* out) {
+  CHECK_EQ(in->size(), 3U);
+  CHECK_EQ(out->size(), 3U);
+  const auto& param = nnvm::get<RequantizeParam>(attrs.parsed);
+  TYPE_ASSIGN_CHECK(*in, 0, mshadow::kInt32);
+  TYPE_ASSIGN_CHECK(*in, 1, mshadow::kFloat32);
+  TYPE_ASSIGN_CHECK(*in, 2, mshadow::kFloat32);
+  TYPE_ASSIGN_CHECK(*out, 0, GetQuantizeOutputType(param));
+  TYPE_ASSIGN_CHECK(*out, 1, mshadow::kFloat32);
+  TYPE_ASSIGN_CHECK(*out, 2, mshadow::kFloat32);
+  return (*in)[0] != -1;
+}
+
+// dequantize-inl.h:77-96
+static bool DequantizeShape(const NodeAttrs&, ShapeVector* in, ShapeVector* out) {
+  CHECK_EQ(in->size(), 3U);
+  CHECK_EQ(out->size(), 1U);
+  TShape d = (*in)[0];
+  SHAPE_ASSIGN_CHECK(*in, 1, kScalarShape);
+  SHAPE_ASSIGN_CHECK(*in, 2, kScalarShape);
+  SHAPE_ASSIGN_CHECK(*out, 0, (*in)[0]);
+  if ((*out)[0].ndim() > 0 && d.ndim() > 0) {
+    d[0] = (*out)[0][0];
+    SHAPE_ASSIGN_CHECK(*in, 0, d);
+  }
+  return shape_is_known((*out)[0]);
+}
+
+// dequantize-inl.h:98-109
+static bool DequantizeType(const NodeAttrs&, std::vector<int>* in, std::vector<int>* out) {
+  CHECK_EQ(in->size(), 3U);
+  CHECK_EQ(out->size(), 1U);
+  CHECK((*in)[0] == mshadow::kUint8 || (*in)[0] == mshadow::kInt8)
+      << "the input data type of dequantize op must be provided, either uint8 or int8";
+  TYPE_ASSIGN_CHECK(*in, 1, mshadow::kFloat32);
+  TYPE_ASSIGN_CHECK(*in, 2, mshadow::kFloat32);
+  TYPE_ASSIGN_CHECK(*out, 0, mshadow::kFloat32);
+  return (*in)[0] != -1;
+}
+
+// quantized_fully_connected.cc:40-93
+static bool QuantizedFullyConnectedShape(const NodeAttrs& attrs, ShapeVector* in,
+                                         ShapeVector* out) {
+  const auto& param = nnvm::get<FullyConnectedParam>(attrs.parsed);
+  const uint32_t num_inputs = param.no_bias ? 2 : 3;
+  CHECK_EQ(in->size(), num_inputs * 3);
+  CHECK_EQ(out->size(), 3U);
+  TShape dshape = (*in)[0];
+  if (!ndim_is_known(dshape)) return false;
+  CHECK(dshape.ndim() >= 1) << "quantized_fully_connected needs at least 1-D data";
+  const index_t num_input =
+      param.flatten ? dshape.ProdShape(1, dshape.ndim()) : dshape[dshape.ndim() - 1];
+  SHAPE_ASSIGN_CHECK(*in, 1, Shape2(param.num_hidden, num_input));
+  if (!param.no_bias) SHAPE_ASSIGN_CHECK(*in, 2, Shape1(param.num_hidden));
+  for (size_t i = num_inputs; i < 3 * num_inputs; ++i) SHAPE_ASSIGN_CHECK(*in, i, kScalarShape);
+  if (param.flatten) {
+    SHAPE_ASSIGN_CHECK(*out, 0, Shape2(dshape[0], param.num_hidden));
+  } else {
+    TShape result(dshape);
+    result[dshape.ndim() - 1] = param.num_hidden;
+    SHAPE_ASSIGN_CHECK(*out, 0, result);
+  }
+  SHAPE_ASSIGN_CHECK(*out, 1, kScalarShape);
+  SHAPE_ASSIGN_CHECK(*out, 2, kScalarShape);
+  if ((*out)[0].ndim() > 0) {
+    dshape[0] = (*out)[0][0];
+    SHAPE_ASSIGN_CHECK(*in, 0, dshape);
+  }
+  return true;
+}
+
+// quantized_fully_connected.cc:95-120 (non-oneDNN branch: int8 data only)
+static bool QuantizedFullyConnectedType(const NodeAttrs& attrs, std::vector<int>* in,
+                                        std::vector<int>* out) {
+  const auto& param = nnvm::get<FullyConnectedParam>(attrs.parsed);
+  const uint32_t num_inputs = param.no_bias ? 2 : 3;
+  CHECK_EQ(in->size(), num_inputs * 3);
+  CHECK_EQ(out->size(), 3U);
+  for (size_t i = 0; i < num_inputs; ++i) TYPE_ASSIGN_CHECK(*in, i, mshadow::kInt8);
+  for (size_t i = num_inputs; i < 3 * num_inputs; ++i) TYPE_ASSIGN_CHECK(*in, i, mshadow::kFloat32);
+  TYPE_ASSIGN_CHECK(*out, 0, mshadow::kInt32);
+  TYPE_ASSIGN_CHECK(*out, 1, mshadow::kFloat32);
+  TYPE_ASSIGN_CHECK(*out, 2, mshadow::kFloat32);
+  return true;
+}
+
+// quantized_conv.cc:30-131 (the non-oneDNN branch: 2-D, NCHW, dilation allowed here
+// because the kernel implements it; channel multiple-of-4 rule of cuDNN dropped)
+static bool QuantizedConvShape(const NodeAttrs& attrs, ShapeVector* in, ShapeVector* out) {
+  const auto& param = nnvm::get<ConvolutionParam>(attrs.parsed);
+  CHECK_EQ(param.num_group, 1U) << "quantized_conv only supports num_group=1 for now";
+  CHECK_EQ(in->size(), param.no_bias ? 6U : 9U);
+  CHECK_EQ(out->size(), 3U);
+  if (param.layout.has_value())
+    CHECK_EQ(param.layout.value(), mshadow::kNCHW) << "quantized_conv only supports NCHW for now";
+  const TShape& dshape = (*in)[0];
+  if (dshape.ndim() <= 0) return false;
+  CHECK_EQ(param.kernel.ndim(), 2) << "quantized_conv only supports 2D convolution for now";
+  CHECK_EQ(dshape.ndim(), 4);
+  TShape wshape{static_cast<index_t>(param.num_filter), dshape[1], param.kernel[0],
+                param.kernel[1]};
+  SHAPE_ASSIGN_CHECK(*in, 1, wshape);
+  TShape oshape{dshape[0], static_cast<index_t>(param.num_filter), 1, 1};
+  oshape[2] = (dshape[2] + 2 * param.pad[0] - param.DilatedKernelSize(0)) / param.stride[0] + 1;
+  oshape[3] = (dshape[3] + 2 * param.pad[1] - param.DilatedKernelSize(1)) / param.stride[1] + 1;
+  SHAPE_ASSIGN_CHECK(*out, 0, oshape);
+  SHAPE_ASSIGN_CHECK(*out, 1, kScalarShape);
+  SHAPE_ASSIGN_CHECK(*out, 2, kScalarShape);
+  const int start = param.no_bias ? 2 : 3, end = param.no_bias ? 6 : 9;
+  for (int i = start; i < end; ++i) SHAPE_ASSIGN_CHECK(*in, i, kScalarShape);
+  if (!param.no_bias) SHAPE_ASSIGN_CHECK(*in, 2, Shape1(param.num_filter));
+  return true;
+}
+
+// quantized_conv.cc:133-156
+static bool QuantizedConvType(const NodeAttrs& attrs, std::vector<int>* in, std::vector<int>* out) {
+  const auto& param = nnvm::get<ConvolutionParam>(attrs.parsed);
+  CHECK_EQ(in->size(), param.no_bias ? 6U : 9U);
+  CHECK_EQ(out->size(), 3U);
+  TYPE_ASSIGN_CHECK(*in, 0, mshadow::kInt8);
+  TYPE_ASSIGN_CHECK(*in, 1, mshadow::kInt8);
+  if (!param.no_bias) TYPE_ASSIGN_CHECK(*in, 2, mshadow::kInt8);
+  const size_t start = param.no_bias ? 2 : 3, end = param.no_bias ? 6 : 9;
+  for (size_t i = start; i < end; ++i) TYPE_ASSIGN_CHECK(*in, i, mshadow::kFloat32);
+  TYPE_ASSIGN_CHECK(*out, 0, mshadow::kInt32);
+  TYPE_ASSIGN_CHECK(*out, 1, mshadow::kFloat32);
+  TYPE_ASSIGN_CHECK(*out, 2, mshadow::kFloat32);
+  return true;
+}
+
+// quantized_activation.cc:30-64
+static bool QuantizedActivationShape(const NodeAttrs&, ShapeVector* in, ShapeVector* out) {
+  CHECK_EQ(in->size(), 3U);
+  if (shape_is_none((*in)[0])) return false;
+  SHAPE_ASSIGN_CHECK(*in, 1, kScalarShape);
+  SHAPE_ASSIGN_CHECK(*in, 2, kScalarShape);
+  out->clear();
+  out->push_back((*in)[0]);
+  out->push_back(kScalarShape);
+  out->push_back(kScalarShape);
+  return true;
+}
+static bool QuantizedActivationType(const NodeAttrs& attrs, std::vector<int>* in,
+                                    std::vector<int>* out) {
+  const auto& param = nnvm::get<ActivationParam>(attrs.parsed);
+  CHECK_EQ(in->size(), 3U);
+  CHECK_EQ(out->size(), 3U);
+  CHECK(param.act_type == activation::kReLU)
+      << "_contrib_quantized_act only supports act_type=relu for now";
+  TYPE_ASSIGN_CHECK(*out, 0, mshadow::kInt8);
+  TYPE_ASSIGN_CHECK(*in, 1, mshadow::kFloat32);
+  TYPE_ASSIGN_CHECK(*in, 2, mshadow::kFloat32);
+  TYPE_ASSIGN_CHECK(*out, 1, mshadow::kFloat32);
+  TYPE_ASSIGN_CHECK(*out, 2, mshadow::kFloat32);
+  return true;
+}
+
+static bool DefaultStorageType(const NodeAttrs&, const int, DispatchMode* dispatch_mode,
+                               std::vector<int>* in, std::vector<int>* out) {
+  *dispatch_mode = DispatchMode::kFCompute;
+  for (int& v : *in) v = kDefaultStorage;
+  for (int& v : *out) v = kDefaultStorage;
+  return true;
+}
+
+// ---- compute: gpu ------------------------------------------------------------------
+
+// QuantizeV2Operator<gpu>::Forward, quantize_v2-inl.h:186-308
+class QuantizeV2OperatorGPU {
+ public:
+  explicit QuantizeV2OperatorGPU(const NodeAttrs& attrs) : attrs_(attrs) {}
+  void Forward(const OpContext& ctx, const std::vector<TBlob>& inputs,
+               const std::vector<OpReqType>&, const std::vector<TBlob>& outputs) {
+    const auto& param = nnvm::get<QuantizeV2Param>(attrs_.parsed);
+    const int out_type = GetQuantizeOutputType(param);
+    const bool calibrated = param.min_calib_range.has_value() && param.max_calib_range.has_value();
+    const float lo = calibrated ? param.min_calib_range.value() : 0.f;
+    const float hi = calibrated ? param.max_calib_range.value() : 0.f;
+    void* stream = raw_stream(ctx);
+    const int in_type = inputs[0].type_flag_;
+    if (in_type == mshadow::kUint8 || in_type == mshadow::kInt8) {
+      MXQ_CALL(mxq_quantize_v2_passthrough(stream, inputs[0].dptr_, outputs[0].dptr_,
+                                           outputs[1].dptr<float>(), outputs[2].dptr<float>(),
+                                           inputs[0].Size(), in_type, calibrated, lo, hi));
+      return;
+    }
+    CHECK(in_type == mshadow::kFloat32) << "quantize_v2 expects float32 data";
+    void* ws = nullptr;
+    size_t ws_bytes = 0;
+    if (!calibrated) {
+      CHECK(!ctx.requested.empty()) << "uncalibrated quantize_v2 needs its temp space resource";
+      ws_bytes = mxq_quantize_v2_workspace(inputs[0].Size());
+      ws = ctx.requested[0].get_space(ws_bytes);
+    }
+    MXQ_CALL(mxq_quantize_v2(stream, inputs[0].dptr<float>(), outputs[0].dptr_,
+                             outputs[1].dptr<float>(), outputs[2].dptr<float>(), inputs[0].Size(),
+                             out_type, calibrated, lo, hi, ws, ws_bytes));
+  }
+
+ private:
+  NodeAttrs attrs_;
+};
+
+static OpStatePtr CreateQuantizeV2State(const NodeAttrs& attrs, Context ctx, const ShapeVector&,
+                                        const std::vector<int>&) {
+  CHECK(ctx.dev_type == Context::kGPU) << "this build only provides the gpu operator";
+  return OpStatePtr::Create<QuantizeV2OperatorGPU>(attrs);
+}
+
+static void QuantizeV2ForwardGPU(const OpStatePtr& state, const OpContext& ctx,
+                                 const std::vector<TBlob>& inputs,
+                                 const std::vector<OpReqType>& req,
+                                 const std::vector<TBlob>& outputs) {
+  state.get_state<QuantizeV2OperatorGPU>().Forward(ctx, inputs, req, outputs);
+}
+
+// QuantizeCompute<gpu>, quantize-inl.h:90-131
+static void QuantizeComputeGPU(const NodeAttrs& attrs, const OpContext& ctx,
+                               const std::vector<TBlob>& inputs, const std::vector<OpReqType>&,
+                               const std::vector<TBlob>& outputs) {
+  const auto& param = nnvm::get<QuantizeParam>(attrs.parsed);
+  MXQ_CALL(mxq_quantize(raw_stream(ctx), inputs[0].dptr<float>(), inputs[1].dptr<float>(),
+                        inputs[2].dptr<float>(), outputs[0].dptr_, outputs[1].dptr<float>(),
+                        outputs[2].dptr<float>(), inputs[0].Size(), param.out_type));
+}
+
+// RequantizeForward<gpu>, requantize-inl.h:127-240
+static void RequantizeForwardGPU(const NodeAttrs& attrs, const OpContext& ctx,
+                                 const std::vector<TBlob>& inputs, const std::vector<OpReqType>&,
+                                 const std::vector<TBlob>& outputs) {
+  const auto& param = nnvm::get<RequantizeParam>(attrs.parsed);
+  const int out_type = GetQuantizeOutputType(param);
+  if (out_type == mshadow::kUint8)
+    LOG_FATAL << "currently, uint8 requantization is only supported by CPU, "
+                 "please switch to the context of CPU or int8 data type for GPU.";
+  const bool calibrated = param.min_calib_range.has_value() && param.max_calib_range.has_value();
+  void* ws = nullptr;
+  size_t ws_bytes = 0;
+  if (!calibrated) {
+    CHECK(!ctx.requested.empty()) << "uncalibrated requantize needs its temp space resource";
+    ws_bytes = mxq_requantize_workspace(inputs[0].Size());
+    ws = ctx.requested[0].get_space(ws_bytes);
+  }
+  MXQ_CALL(mxq_requantize(raw_stream(ctx), inputs[0].dptr<int32_t>(), inputs[1].dptr<float>(),
+                          inputs[2].dptr<float>(), outputs[0].dptr<int8_t>(),
+                          outputs[1].dptr<float>(), outputs[2].dptr<float>(), inputs[0].Size(),
+                          calibrated, calibrated ? param.min_calib_range.value() : 0.f,
+                          calibrated ? param.max_calib_range.value() : 0.f, ws, ws_bytes));
+}
+
+// DequantizeOperator<gpu>::Forward, dequantize-inl.h:112-148
+class DequantizeOperatorGPU {
+ public:
+  explicit DequantizeOperatorGPU(const NodeAttrs& attrs) : attrs_(attrs) {}
+  void Forward(const OpContext& ctx, const std::vector<TBlob>& inputs,
+               const std::vector<OpReqType>&, const std::vector<TBlob>& outputs) {
+    const int t = inputs[0].type_flag_;
+    if (t != mshadow::kUint8 && t != mshadow::kInt8)
+      LOG_FATAL << "dequantize op only supports input type int8 or uint8";
+    MXQ_CALL(mxq_dequantize(raw_stream(ctx), inputs[0].dptr_, t, inputs[1].dptr<float>(),
+                            inputs[2].dptr<float>(), outputs[0].dptr<float>(),
+                            outputs[0].Size()));
+  }
+
+ private:
+  NodeAttrs attrs_;
+};
+
+static OpStatePtr CreateDequantizeState(const NodeAttrs& attrs, Context ctx, const ShapeVector&,
+                                        const std::vector<int>&) {
+  CHECK(ctx.dev_type == Context::kGPU) << "this build only provides the gpu operator";
+  return OpStatePtr::Create<DequantizeOperatorGPU>(attrs);
+}
+
+static void DequantizeForwardGPU(const OpStatePtr& state, const OpContext& ctx,
+                                 const std::vector<TBlob>& inputs,
+                                 const std::vector<OpReqType>& req,
+                                 const std::vector<TBlob>& outputs) {
+  state.get_state<DequantizeOperatorGPU>().Forward(ctx, inputs, req, outputs);
+}
+
+// QuantizedFullyConnectedForwardGPU, quantized_fully_connected.cu:58-138
+static void QuantizedFullyConnectedForwardGPU(const NodeAttrs& attrs, const OpContext& ctx,
+                                              const std::vector<TBlob>& inputs,
+                                              const std::vector<OpReqType>&,
+                                              const std::vector<TBlob>& outputs) {
+  const auto& param = nnvm::get<FullyConnectedParam>(attrs.parsed);
+  const size_t num_inputs = param.no_bias ? 2 : 3;
+  CHECK_EQ(inputs.size(), num_inputs * 3);
+  CHECK_EQ(outputs.size(), 3U);
+  const TShape& dshape = inputs[0].shape_;
+  const TShape& wshape = inputs[1].shape_;
+  index_t m, k;
+  if (param.flatten || dshape.ndim() == 2) {
+    m = dshape[0];
+    k = dshape.ProdShape(1, dshape.ndim());
+  } else {
+    // flatten=false: every leading dimension is a row (the oneDNN operator's rule)
+    k = dshape[dshape.ndim() - 1];
+    m = dshape.ProdShape(0, dshape.ndim() - 1);
+  }
+  const index_t n = wshape[0];
+  CHECK_EQ(wshape[1], k);
+  const int8_t* bias = param.no_bias ? nullptr : inputs[2].dptr<int8_t>();
+  MXQ_CALL(mxq_quantized_fc(
+      raw_stream(ctx), inputs[0].dptr<int8_t>(), inputs[1].dptr<int8_t>(), bias,
+      static_cast<int>(m), static_cast<int>(n), static_cast<int>(k),
+      inputs[num_inputs].dptr<float>(), inputs[num_inputs + 1].dptr<float>(),
+      inputs[num_inputs + 2].dptr<float>(), inputs[num_inputs + 3].dptr<float>(),
+      param.no_bias ? nullptr : inputs[7].dptr<float>(),
+      param.no_bias ? nullptr : inputs[8].dptr<float>(), outputs[0].dptr<int32_t>(),
+      outputs[1].dptr<float>(), outputs[2].dptr<float>(), nullptr, nullptr, nullptr, 0, 0.f, 0.f));
+}
+
+// Temp space of the convolution: NHWC copies of data and weight plus the NHWC int32
+// result (the reference asks for the same three buffers plus cuDNN's workspace,
+// quantized_conv.cu:121-160).
+static size_t QuantizedConvTempBytes(const TShape& d, const TShape& w, const TShape& o) {
+  auto up = [](size_t x) { return (x + 255) / 256 * 256; };
+  return up(d.Size()) + up(w.Size()) + up(o.Size() * sizeof(int32_t));
+}
+
+// QuantizedConvForwardGPU, quantized_conv.cu:268-291
+static void QuantizedConvForwardGPU(const NodeAttrs& attrs, const OpContext& ctx,
+                                    const std::vector<TBlob>& inputs,
+                                    const std::vector<OpReqType>&,
+                                    const std::vector<TBlob>& outputs) {
+  const auto& param = nnvm::get<ConvolutionParam>(attrs.parsed);
+  CHECK_EQ(param.kernel.ndim(), 2) << "QuantizedConvForward<gpu> only supports 2D convolution";
+  CHECK_EQ(inputs.size(), param.no_bias ? 6U : 9U);
+  CHECK_EQ(outputs.size(), 3U);
+  const TShape& d = inputs[0].shape_;
+  const TShape& w = inputs[1].shape_;
+  const TShape& o = outputs[0].shape_;
+  CHECK(!ctx.requested.empty()) << "quantized_conv needs its temp space resource";
+  auto up = [](size_t x) { return (x + 255) / 256 * 256; };
+  char* ws = ctx.requested[0].get_space(QuantizedConvTempBytes(d, w, o));
+  int8_t* d_nhwc = reinterpret_cast<int8_t*>(ws);
+  int8_t* w_ohwi = reinterpret_cast<int8_t*>(ws + up(d.Size()));
+  int32_t* o_nhwc = reinterpret_cast<int32_t*>(ws + up(d.Size()) + up(w.Size()));
+  void* stream = raw_stream(ctx);
+  const int N = d[0], C = d[1], H = d[2], W = d[3], O = w[0], KH = w[2], KW = w[3];
+  MXQ_CALL(mxq_nchw_to_nhwc_i8(stream, inputs[0].dptr<int8_t>(), d_nhwc, N, C, H, W));
+  MXQ_CALL(mxq_nchw_to_nhwc_i8(stream, inputs[1].dptr<int8_t>(), w_ohwi, O, C, KH, KW));
+  const size_t ni = param.no_bias ? 2 : 3;
+  MXQ_CALL(mxq_quantized_conv_nhwc(
+      stream, d_nhwc, w_ohwi, param.no_bias ? nullptr : inputs[2].dptr<int8_t>(), N, H, W, C, O,
+      KH, KW, static_cast<int>(param.stride[0]), static_cast<int>(param.stride[1]),
+      static_cast<int>(param.pad[0]), static_cast<int>(param.pad[1]),
+      static_cast<int>(param.dilate[0]), static_cast<int>(param.dilate[1]),
+      inputs[ni].dptr<float>(), inputs[ni + 1].dptr<float>(), inputs[ni + 2].dptr<float>(),
+      inputs[ni + 3].dptr<float>(), param.no_bias ? nullptr : inputs[7].dptr<float>(),
+      param.no_bias ? nullptr : inputs[8].dptr<float>(), o_nhwc, outputs[1].dptr<float>(),
+      outputs[2].dptr<float>(), nullptr, nullptr, nullptr, 0, 0.f, 0.f));
+  MXQ_CALL(mxq_nhwc_to_nchw(stream, o_nhwc, outputs[0].dptr<int32_t>(), static_cast<int>(o[0]),
+                            static_cast<int>(o[1]), static_cast<int>(o[2]),
+                            static_cast<int>(o[3]), 4));
+}
+
+// _contrib_quantized_act: int8 relu, ranges pass through (dnnl_quantized_act.cc:33-45)
+static void QuantizedActivationForwardGPU(const NodeAttrs& attrs, const OpContext& ctx,
+                                          const std::vector<TBlob>& inputs,
+                                          const std::vector<OpReqType>&,
+                                          const std::vector<TBlob>& outputs) {
+  const auto& param = nnvm::get<ActivationParam>(attrs.parsed);
+  CHECK(param.act_type == activation::kReLU)
+      << "_contrib_quantized_act only supports act_type=relu for now";
+  MXQ_CALL(mxq_quantized_relu(raw_stream(ctx), inputs[0].dptr<int8_t>(), inputs[1].dptr<float>(),
+                              inputs[2].dptr<float>(), outputs[0].dptr<int8_t>(),
+                              outputs[1].dptr<float>(), outputs[2].dptr<float>(),
+                              inputs[0].Size()));
+}
+
+// Temp-space bytes the harness (or a framework without lazy resources) must provide.
+size_t MXQTempSpaceBytes(const NodeAttrs& attrs, const ShapeVector& in, const ShapeVector& out) {
+  const std::string& name = attrs.op->name;
+  if (name == "_contrib_quantize_v2") return mxq_quantize_v2_workspace(in[0].Size());
+  if (name == "_contrib_requantize") return mxq_requantize_workspace(in[0].Size());
+  if (name == "_contrib_quantized_conv") return QuantizedConvTempBytes(in[0], in[1], out[0]);
+  return 0;
+}
+
+// ---- registration ---------------------------------------------------------------------
+
+static std::vector<std::string> QuantizedFcConvInputNames(bool no_bias) {
+  if (no_bias) return {"data", "weight", "min_data", "max_data", "min_weight", "max_weight"};
+  return {"data",       "weight",     "bias",     "min_data", "max_data",
+          "min_weight", "max_weight", "min_bias", "max_bias"};
+}
+
+template <typename Param>
+static std::vector<ResourceRequest> TempSpaceUnlessCalibrated(const NodeAttrs& attrs) {
+  const auto& param = nnvm::get<Param>(attrs.parsed);
+  if (param.min_calib_range.has_value() && param.max_calib_range.has_value())
+    return std::vector<ResourceRequest>();
+  return std::vector<ResourceRequest>(1, ResourceRequest::kTempSpace);
+}
+
+NNVM_REGISTER_OP(_contrib_quantize_v2)
+    .add_alias("_npx_contrib_quantize_v2")
+    .describe("Quantize a input tensor from float to `out_type`, with user-specified "
+              "`min_calib_range` and `max_calib_range` or the input range collected at runtime.")
+    .set_attr_parser(ParamParser<QuantizeV2Param>)
+    .set_num_inputs(1)
+    .set_num_outputs(3)
+    .set_attr<nnvm::FListInputNames>("FListInputNames",
+                                     [](const NodeAttrs&) {
+                                       return std::vector<std::string>{"data"};
+                                     })
+    .set_attr<mxnet::FInferShape>("FInferShape", QuantizeV2Shape)
+    .set_attr<nnvm::FInferType>("FInferType", QuantizeV2Type)
+    .set_attr<FInferStorageType>("FInferStorageType", DefaultStorageType)
+    .set_attr<FCreateOpState>("FCreateOpState", CreateQuantizeV2State)
+    .set_attr<FStatefulCompute>("FStatefulCompute<gpu>", QuantizeV2ForwardGPU)
+    .set_attr<nnvm::FInplaceOption>("FInplaceOption",
+                                    [](const NodeAttrs&) {
+                                      return std::vector<std::pair<int, int>>{{0, 0}};
+                                    })
+    .set_attr<nnvm::FInplaceIdentity>("FInplaceIdentity",
+                                      [](const NodeAttrs&) { return std::vector<bool>{true}; })
+    .set_attr<FNeedCalibrateInput>("FNeedCalibrateInput",
+                                   [](const NodeAttrs&) { return std::vector<int>{0}; })
+    .set_attr<FResourceRequest>("FResourceRequest", TempSpaceUnlessCalibrated<QuantizeV2Param>)
+    .add_argument("data", "NDArray-or-Symbol", "A ndarray/symbol of type `float32`")
+    .add_arguments(QuantizeV2Param::__FIELDS__());
+
+NNVM_REGISTER_OP(_contrib_quantize)
+    .add_alias("_npx_contrib_quantize")
+    .describe("Quantize a input tensor from float to `out_type`, with user-specified "
+              "`min_range` and `max_range`.")
+    .set_attr_parser(ParamParser<QuantizeParam>)
+    .set_num_inputs(3)
+    .set_num_outputs(3)
+    .set_attr<nnvm::FListInputNames>("FListInputNames",
+                                     [](const NodeAttrs&) {
+                                       return std::vector<std::string>{"data", "min_range",
+                                                                       "max_range"};
+                                     })
+    .set_attr<mxnet::FInferShape>("FInferShape", QuantizeShape)
+    .set_attr<nnvm::FInferType>("FInferType", QuantizeType)
+    .set_attr<FInferStorageType>("FInferStorageType", DefaultStorageType)
+    .set_attr<FCompute>("FCompute<gpu>", QuantizeComputeGPU)
+    .add_argument("data", "NDArray-or-Symbol", "A ndarray/symbol of type `float32`")
+    .add_argument("min_range", "NDArray-or-Symbol",
+                  "The minimum scalar value possibly produced for the input")
+    .add_argument("max_range", "NDArray-or-Symbol",
+                  "The maximum scalar value possibly produced for the input")
+    .add_arguments(QuantizeParam::__FIELDS__());
+
+NNVM_REGISTER_OP(_contrib_requantize)
+    .add_alias("_npx_requantize")
+    .describe("Given data that is quantized in int32 and the corresponding thresholds, "
+              "requantize the data into int8 using min and max thresholds either calculated at "
+              "runtime or from calibration.")
+    .set_attr_parser(ParamParser<RequantizeParam>)
+    .set_num_inputs(3)
+    .set_num_outputs(3)
+    .set_attr<nnvm::FListInputNames>("FListInputNames",
+                                     [](const NodeAttrs&) {
+                                       return std::vector<std::string>{"data", "min_range",
+                                                                       "max_range"};
+                                     })
+    .set_attr<mxnet::FInferShape>("FInferShape", QuantizeShape)
+    .set_attr<nnvm::FInferType>("FInferType", RequantizeType)
+    .set_attr<FInferStorageType>("FInferStorageType", DefaultStorageType)
+    .set_attr<FCompute>("FCompute<gpu>", RequantizeForwardGPU)
+    .set_attr<FNeedCalibrateInput>("FNeedCalibrateInput",
+                                   [](const NodeAttrs&) { return std::vector<int>{0}; })
+    .set_attr<FResourceRequest>("FResourceRequest", TempSpaceUnlessCalibrated<RequantizeParam>)
+    .add_argument("data", "NDArray-or-Symbol", "A ndarray/symbol of type `int32`")
+    .add_argument("min_range", "NDArray-or-Symbol",
+                  "The original minimum scalar value in the form of float32 used for quantizing "
+                  "data into int32.")
+    .add_argument("max_range", "NDArray-or-Symbol",
+                  "The original maximum scalar value in the form of float32 used for quantizing "
+                  "data into int32.")
+    .add_arguments(RequantizeParam::__FIELDS__());
+
+NNVM_REGISTER_OP(_contrib_dequantize)
+    .describe("Dequantize the input tensor into a float tensor. min_range and max_range are "
+              "scalar floats that specify the range for the output data.")
+    .set_attr_parser(ParamParser<DequantizeParam>)
+    .set_num_inputs(3)
+    .set_num_outputs(1)
+    .set_attr<nnvm::FListInputNames>("FListInputNames",
+                                     [](const NodeAttrs&) {
+                                       return std::vector<std::string>{"data", "min_range",
+                                                                       "max_range"};
+                                     })
+    .set_attr<mxnet::FInferShape>("FInferShape", DequantizeShape)
+    .set_attr<nnvm::FInferType>("FInferType", DequantizeType)
+    .set_attr<FInferStorageType>("FInferStorageType", DefaultStorageType)
+    .set_attr<FCreateOpState>("FCreateOpState", CreateDequantizeState)
+    .set_attr<FStatefulCompute>("FStatefulCompute<gpu>", DequantizeForwardGPU)
+    .add_argument("data", "NDArray-or-Symbol", "A ndarray/symbol of type `uint8`")
+    .add_argument("min_range", "NDArray-or-Symbol",
+                  "The minimum scalar value possibly produced for the input in float32")
+    .add_argument("max_range", "NDArray-or-Symbol",
+                  "The maximum scalar value possibly produced for the input in float32")
+    .add_arguments(DequantizeParam::__FIELDS__());
+
+NNVM_REGISTER_OP(_contrib_quantized_fully_connected)
+    .add_alias("_npx_quantized_fully_connected")
+    .describe("Fully Connected operator for input, weight and bias data type of int8, and "
+              "accumulates in type int32 for the output.")
+    .set_num_inputs([](const NodeAttrs& attrs) {
+      return nnvm::get<FullyConnectedParam>(attrs.parsed).no_bias ? 6 : 9;
+    })
+    .set_num_outputs(3)
+    .set_attr_parser(ParamParser<FullyConnectedParam>)
+    .set_attr<nnvm::FListInputNames>(
+        "FListInputNames",
+        [](const NodeAttrs& attrs) {
+          return QuantizedFcConvInputNames(nnvm::get<FullyConnectedParam>(attrs.parsed).no_bias);
+        })
+    .set_attr<nnvm::FListOutputNames>("FListOutputNames",
+                                      [](const NodeAttrs&) {
+                                        return std::vector<std::string>{"output", "min_output",
+                                                                        "max_output"};
+                                      })
+    .set_attr<mxnet::FInferShape>("FInferShape", QuantizedFullyConnectedShape)
+    .set_attr<nnvm::FInferType>("FInferType", QuantizedFullyConnectedType)
+    .set_attr<FInferStorageType>("FInferStorageType", DefaultStorageType)
+    .set_attr<FNeedRequantize>("FNeedRequantize", [](const NodeAttrs&) { return true; })
+    .set_attr<FCompute>("FCompute<gpu>", QuantizedFullyConnectedForwardGPU)
+    .set_attr<FResourceRequest>("FResourceRequest",
+                                [](const NodeAttrs&) {
+                                  return std::vector<ResourceRequest>{ResourceRequest::kTempSpace};
+                                })
+    .add_argument("data", "NDArray-or-Symbol", "Input data.")
+    .add_argument("weight", "NDArray-or-Symbol", "weight.")
+    .add_argument("bias", "NDArray-or-Symbol", "bias.")
+    .add_argument("min_data", "NDArray-or-Symbol", "Minimum value of data.")
+    .add_argument("max_data", "NDArray-or-Symbol", "Maximum value of data.")
+    .add_argument("min_weight", "NDArray-or-Symbol", "Minimum value of weight.")
+    .add_argument("max_weight", "NDArray-or-Symbol", "Maximum value of weight.")
+    .add_argument("min_bias", "NDArray-or-Symbol", "Minimum value of bias.")
+    .add_argument("max_bias", "NDArray-or-Symbol", "Maximum value of bias.")
+    .add_arguments(FullyConnectedParam::__FIELDS__());
+
+NNVM_REGISTER_OP(_contrib_quantized_conv)
+    .add_alias("_npx_quantized_conv")
+    .describe("Convolution operator for input, weight and bias data type of int8, and "
+              "accumulates in type int32 for the output.")
+    .set_num_inputs([](const NodeAttrs& attrs) {
+      return nnvm::get<ConvolutionParam>(attrs.parsed).no_bias ? 6 : 9;
+    })
+    .set_num_outputs(3)
+    .set_attr_parser(ConvolutionParamParser)
+    .set_attr<nnvm::FListInputNames>(
+        "FListInputNames",
+        [](const NodeAttrs& attrs) {
+          return QuantizedFcConvInputNames(nnvm::get<ConvolutionParam>(attrs.parsed).no_bias);
+        })
+    .set_attr<nnvm::FListOutputNames>("FListOutputNames",
+                                      [](const NodeAttrs&) {
+                                        return std::vector<std::string>{"output", "min_output",
+                                                                        "max_output"};
+                                      })
+    .set_attr<mxnet::FInferShape>("FInferShape", QuantizedConvShape)
+    .set_attr<nnvm::FInferType>("FInferType", QuantizedConvType)
+    .set_attr<FInferStorageType>("FInferStorageType", DefaultStorageType)
+    .set_attr<FResourceRequest>("FResourceRequest",
+                                [](const NodeAttrs&) {
+                                  return std::vector<ResourceRequest>(1,
+                                                                      ResourceRequest::kTempSpace);
+                                })
+    .set_attr<FNeedRequantize>("FNeedRequantize", [](const NodeAttrs&) { return true; })
+    .set_attr<FCompute>("FCompute<gpu>", QuantizedConvForwardGPU)
+    .add_argument("data", "NDArray-or-Symbol", "Input data.")
+    .add_argument("weight", "NDArray-or-Symbol", "weight.")
+    .add_argument("bias", "NDArray-or-Symbol", "bias.")
+    .add_argument("min_data", "NDArray-or-Symbol", "Minimum value of data.")
+    .add_argument("max_data", "NDArray-or-Symbol", "Maximum value of data.")
+    .add_argument("min_weight", "NDArray-or-Symbol", "Minimum value of weight.")
+    .add_argument("max_weight", "NDArray-or-Symbol", "Maximum value of weight.")
+    .add_argument("min_bias", "NDArray-or-Symbol", "Minimum value of bias.")
+    .add_argument("max_bias", "NDArray-or-Symbol", "Maximum value of bias.")
+    .add_arguments(ConvolutionParam::__FIELDS__());
+
+NNVM_REGISTER_OP(_contrib_quantized_act)
+    .add_alias("_npx_quantized_act")
+    .describe("Activation operator for input and output data type of int8. Only `relu`.")
+    .set_num_inputs(3)
+    .set_num_outputs(3)
+    .set_attr_parser(ParamParser<ActivationParam>)
+    .set_attr<nnvm::FListInputNames>("FListInputNames",
+                                     [](const NodeAttrs&) {
+                                       return std::vector<std::string>{"data", "min_data",
+                                                                       "max_data"};
+                                     })
+    .set_attr<nnvm::FListOutputNames>("FListOutputNames",
+                                      [](const NodeAttrs&) {
+                                        return std::vector<std::string>{"output", "min_output",
+                                                                        "max_output"};
+                                      })
+    .set_attr<nnvm::FInferType>("FInferType", QuantizedActivationType)
+    .set_attr<mxnet::FInferShape>("FInferShape", QuantizedActivationShape)
+    .set_attr<FInferStorageType>("FInferStorageType", DefaultStorageType)
+    .set_attr<FNeedRequantize>("FNeedRequantize", [](const NodeAttrs&) { return false; })
+    .set_attr<FCompute>("FCompute<gpu>", QuantizedActivationForwardGPU)
+    .add_argument("data", "NDArray-or-Symbol", "Input data.")
+    .add_argument("min_data", "NDArray-or-Symbol", "Minimum value of data.")
+    .add_argument("max_data", "NDArray-or-Symbol", "Maximum value of data.")
+    .add_arguments(ActivationParam::__FIELDS__());
+
+}  // namespace op
+}  // namespace mxnet

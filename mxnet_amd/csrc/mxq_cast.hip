@@ -513,6 +513,41 @@ __global__ __launch_bounds__(kThreads) void minmax_i32_kernel(const int32_t* __r
   }
 }
 
+// int8 relu on packed bytes: 16 values per lane per segment.
+__global__ __launch_bounds__(kThreads) void relu_i8_kernel(const int8_t* __restrict__ in,
+                                                           int8_t* __restrict__ out, size_t n,
+                                                           const float* __restrict__ imin,
+                                                           const float* __restrict__ imax,
+                                                           float* __restrict__ omin,
+                                                           float* __restrict__ omax, bool vec) {
+  const size_t stride = size_t(gridDim.x) * kThreads;
+  const size_t t0 = size_t(blockIdx.x) * kThreads + threadIdx.x;
+  auto relu4 = [](uint32_t w) -> uint32_t {
+    // a byte is negative iff its top bit is set: build a per-byte keep mask
+    uint32_t neg = (w >> 7) & 0x01010101u;
+    uint32_t mask = (neg * 0xffu) ^ 0xffffffffu;
+    return w & mask;
+  };
+  if (vec) {
+    typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+    const size_t n16 = n >> 4;
+    const u4* in16 = reinterpret_cast<const u4*>(in);
+    u4* out16 = reinterpret_cast<u4*>(out);
+    for (size_t q = t0; q < n16; q += stride) {
+      u4 w = nt_load(in16 + q);
+      u4 r = {relu4(w.x), relu4(w.y), relu4(w.z), relu4(w.w)};
+      nt_store(r, out16 + q);
+    }
+    for (size_t i = (n16 << 4) + t0; i < n; i += stride) out[i] = in[i] > 0 ? in[i] : 0;
+  } else {
+    for (size_t i = t0; i < n; i += stride) out[i] = in[i] > 0 ? in[i] : 0;
+  }
+  if (blockIdx.x == 0 && threadIdx.x == 0) {
+    *omin = *imin;
+    *omax = *imax;
+  }
+}
+
 __global__ void passthrough_range_kernel(float* omin, float* omax, float lo, float hi) {
   *omin = lo;
   *omax = hi;
@@ -679,6 +714,20 @@ int mxq_requantize(void* stream, const int32_t* in, const float* imin, const flo
   else
     hipLaunchKernelGGL((requantize_kernel<false>), dim3(grid), dim3(kThreads), 0, s, in, o,
                        omin, omax, n, imin, imax, real_range, slots);
+  MXQ_LAUNCH_CHECK();
+  MXQ_API_END();
+}
+
+int mxq_quantized_relu(void* stream, const int8_t* in, const float* imin, const float* imax,
+                       int8_t* out, float* omin, float* omax, size_t n) {
+  MXQ_API_BEGIN();
+  MXQ_CHECK(imin != nullptr && imax != nullptr && omin != nullptr && omax != nullptr,
+            "null range pointer");
+  MXQ_CHECK(n == 0 || (in != nullptr && out != nullptr), "null data pointer");
+  const bool vec = aligned16(in) && aligned16(out);
+  const int grid = stream_grid(n == 0 ? 1 : (vec ? (n + 15) / 16 : n));
+  hipLaunchKernelGGL(relu_i8_kernel, dim3(grid), dim3(kThreads), 0,
+                     static_cast<hipStream_t>(stream), in, out, n, imin, imax, omin, omax, vec);
   MXQ_LAUNCH_CHECK();
   MXQ_API_END();
 }
