@@ -1,0 +1,156 @@
+"""The C++ operator host on the CPU: registry contents, attribute parsing, shape and
+type inference (no kernel is launched).  Expected values are read off the reference's
+registrations and inference functions (src/operator/quantization/*.cc, *-inl.h)."""
+import pytest
+import torch
+
+from mxnet_amd import operator as op
+from mxnet_amd.operator import MXNetError, Node
+
+F32, I8, U8, I32 = torch.float32, torch.int8, torch.uint8, torch.int32
+
+
+def test_registry_names_aliases_and_gpu_attributes():
+    names = op.list_operators()
+    for n in ["_contrib_quantize_v2", "_contrib_requantize", "_contrib_dequantize",
+              "_contrib_quantized_fully_connected", "_contrib_quantized_conv",
+              "_contrib_quantize", "_contrib_quantized_act"]:
+        assert n in names
+    # stateless operators carry FCompute<gpu>, the two stateful ones FStatefulCompute<gpu>
+    for n in ["_contrib_requantize", "_contrib_quantized_fully_connected",
+              "_contrib_quantized_conv", "_contrib_quantize", "_contrib_quantized_act"]:
+        assert op.has_attr(n, "FCompute<gpu>") and not op.has_attr(n, "FStatefulCompute<gpu>")
+    for n in ["_contrib_quantize_v2", "_contrib_dequantize"]:
+        assert op.has_attr(n, "FStatefulCompute<gpu>") and op.has_attr(n, "FCreateOpState")
+        assert not op.has_attr(n, "FCompute<gpu>")
+    for n in ["_contrib_quantized_fully_connected", "_contrib_quantized_conv"]:
+        assert op.has_attr(n, "FNeedRequantize") and op.has_attr(n, "FResourceRequest")
+    for n in ["_contrib_quantize_v2", "_contrib_requantize"]:
+        assert op.has_attr(n, "FNeedCalibrateInput")
+    # aliases resolve to the same operator
+    for alias, name in [("_npx_contrib_quantize_v2", "_contrib_quantize_v2"),
+                        ("_npx_requantize", "_contrib_requantize"),
+                        ("_npx_quantized_fully_connected", "_contrib_quantized_fully_connected"),
+                        ("_npx_quantized_conv", "_contrib_quantized_conv"),
+                        ("_npx_quantized_act", "_contrib_quantized_act")]:
+        assert op.has_attr(alias, "FInferShape")
+    with pytest.raises(MXNetError, match="not registered"):
+        Node("_contrib_does_not_exist")
+
+
+def test_input_output_names():
+    n = Node("_contrib_quantized_fully_connected", num_hidden=8)
+    assert n.num_inputs == 9 and n.num_outputs == 3
+    assert n.list_inputs() == ["data", "weight", "bias", "min_data", "max_data", "min_weight",
+                               "max_weight", "min_bias", "max_bias"]
+    assert n.list_outputs() == ["output", "min_output", "max_output"]
+    n = Node("_contrib_quantized_conv", kernel=(3, 3), num_filter=8, no_bias=True)
+    assert n.num_inputs == 6
+    assert n.list_inputs() == ["data", "weight", "min_data", "max_data", "min_weight",
+                               "max_weight"]
+    assert Node("_contrib_requantize").list_inputs() == ["data", "min_range", "max_range"]
+    assert Node("_contrib_quantize_v2").list_inputs() == ["data"]
+    assert Node("_contrib_dequantize").num_outputs == 1
+
+
+def test_attribute_parsing():
+    # defaults: out_type int8 for quantize_v2 and requantize, uint8 for v1 quantize
+    assert Node("_contrib_quantize_v2").infer_type([F32])[1][0] == I8
+    assert Node("_contrib_requantize").infer_type([I32, F32, F32])[1][0] == I8
+    assert Node("_contrib_quantize").infer_type([F32, F32, F32])[1][0] == U8
+    # auto: uint8 iff calibrated with a non-negative minimum (quantization_utils.h:201-220)
+    assert Node("_contrib_quantize_v2", out_type="auto", min_calib_range=0.0,
+                max_calib_range=1.0).infer_type([F32])[1][0] == U8
+    assert Node("_contrib_quantize_v2", out_type="auto", min_calib_range=-0.1,
+                max_calib_range=1.0).infer_type([F32])[1][0] == I8
+    assert Node("_contrib_quantize_v2", out_type="auto").infer_type([F32])[1][0] == I8
+    # calibration ranges arrive as std::to_string(float) text, "None" is absent
+    n = Node("_contrib_requantize", min_calib_range="-134.348999", max_calib_range="523.429993")
+    assert n.infer_type([None, None, None])[0] == [I32, F32, F32]
+    Node("_contrib_requantize", min_calib_range="None", max_calib_range="None")
+    # bool spellings
+    for v in ["True", "true", "1", True]:
+        assert Node("_contrib_quantized_fully_connected", num_hidden=4, no_bias=v).num_inputs == 6
+    for v in ["False", "false", "0", False]:
+        assert Node("_contrib_quantized_fully_connected", num_hidden=4, no_bias=v).num_inputs == 9
+    # tuple spellings
+    for k in ["(3, 3)", "[3,3]", "(3,3)"]:
+        n = Node("_contrib_quantized_conv", kernel=k, num_filter=8, no_bias=True)
+        assert n.infer_shape([(1, 4, 8, 8)] + [None] * 5)[1][0] == (1, 8, 6, 6)
+    # errors
+    with pytest.raises(MXNetError, match="Invalid Parameter format for out_type"):
+        Node("_contrib_quantize_v2", out_type="int4")
+    with pytest.raises(MXNetError, match="Cannot find argument 'foo'"):
+        Node("_contrib_dequantize", foo=1)
+    with pytest.raises(MXNetError, match="Required parameter num_hidden"):
+        Node("_contrib_quantized_fully_connected")
+    with pytest.raises(MXNetError, match="greater equal to 1"):
+        Node("_contrib_quantized_fully_connected", num_hidden=0)
+    with pytest.raises(MXNetError, match="float32"):
+        Node("_contrib_dequantize", out_type="float16")
+    with pytest.raises(MXNetError, match="in operator _contrib_quantize_v2"):
+        Node("_contrib_quantize_v2", min_calib_range="abc")
+    Node("_contrib_quantize_v2", __profiler_scope__="x")  # hidden keys are accepted
+
+
+def test_shape_inference():
+    n = Node("_contrib_quantize_v2")
+    assert n.infer_shape([(2, 3, 4)]) == ([(2, 3, 4)], [(2, 3, 4), (1,), (1,)])
+    # the batch dimension flows back from a known output (quantize_v2-inl.h:141-144)
+    assert n.infer_shape([(-1, 3)], [(2, 3), None, None])[0] == [(2, 3)]
+    with pytest.raises(MXNetError, match="Shape inconsistent"):
+        n.infer_shape([(2, 3)], [(2, 4), None, None])
+    n = Node("_contrib_requantize")
+    assert n.infer_shape([(5, 6), None, None]) == ([(5, 6), (1,), (1,)], [(5, 6), (1,), (1,)])
+    with pytest.raises(MXNetError, match="Shape inconsistent"):
+        n.infer_shape([(5, 6), (2,), None])
+    n = Node("_contrib_dequantize")
+    assert n.infer_shape([(7,), None, None]) == ([(7,), (1,), (1,)], [(7,)])
+    # quantized FC: flatten semantics (quantized_fully_connected.cc:54-78)
+    n = Node("_contrib_quantized_fully_connected", num_hidden=100)
+    ins, outs = n.infer_shape([(32, 111, 2, 2)] + [None] * 8)
+    assert ins[1] == (100, 444) and ins[2] == (100,) and ins[3:] == [(1,)] * 6
+    assert outs == [(32, 100), (1,), (1,)]
+    n = Node("_contrib_quantized_fully_connected", num_hidden=100, flatten=False, no_bias=True)
+    ins, outs = n.infer_shape([(32, 512, 2)] + [None] * 5)
+    assert ins[1] == (100, 2) and outs[0] == (32, 512, 100)
+    with pytest.raises(MXNetError, match="Shape inconsistent"):
+        Node("_contrib_quantized_fully_connected", num_hidden=8, no_bias=True).infer_shape(
+            [(4, 16), (8, 32)] + [None] * 4)
+    # quantized conv (quantized_conv.cc:30-131): OH = (H + 2p - dilated_k) / s + 1
+    n = Node("_contrib_quantized_conv", kernel=(3, 3), num_filter=128, pad=(1, 1))
+    ins, outs = n.infer_shape([(3, 4, 28, 28)] + [None] * 8)
+    assert ins[1] == (128, 4, 3, 3) and ins[2] == (128,) and outs[0] == (3, 128, 28, 28)
+    n = Node("_contrib_quantized_conv", kernel=(1, 1), num_filter=512, stride=(2, 2),
+             no_bias=True)
+    assert n.infer_shape([(64, 256, 56, 56)] + [None] * 5)[1][0] == (64, 512, 28, 28)
+    n = Node("_contrib_quantized_conv", kernel=(3, 3), num_filter=8, dilate=(2, 2), pad=(2, 2),
+             stride=(2, 2), no_bias=True)
+    assert n.infer_shape([(1, 16, 12, 13)] + [None] * 5)[1][0] == (1, 8, 6, 7)
+    with pytest.raises(MXNetError, match="num_group"):
+        Node("_contrib_quantized_conv", kernel=(3, 3), num_filter=8, num_group=2,
+             no_bias=True).infer_shape([(1, 16, 12, 13)] + [None] * 5)
+    with pytest.raises(MXNetError, match="NCHW"):
+        Node("_contrib_quantized_conv", kernel=(3, 3), num_filter=8, layout="NHWC",
+             no_bias=True).infer_shape([(1, 12, 13, 16)] + [None] * 5)
+    n = Node("_contrib_quantized_act", act_type="relu")
+    assert n.infer_shape([(4, 5), None, None])[1] == [(4, 5), (1,), (1,)]
+
+
+def test_type_inference():
+    n = Node("_contrib_quantized_fully_connected", num_hidden=4)
+    ins, outs = n.infer_type([None] * 9)
+    assert ins == [I8, I8, I8] + [F32] * 6 and outs == [I32, F32, F32]
+    with pytest.raises(MXNetError, match="Type inconsistent"):
+        n.infer_type([U8] + [None] * 8)           # gpu operator: int8 data only
+    n = Node("_contrib_quantized_conv", kernel=(1, 1), num_filter=4, no_bias=True)
+    assert n.infer_type([None] * 6) == ([I8, I8] + [F32] * 4, [I32, F32, F32])
+    n = Node("_contrib_dequantize")
+    assert n.infer_type([U8, None, None]) == ([U8, F32, F32], [F32])
+    with pytest.raises(MXNetError, match="either uint8 or int8"):
+        n.infer_type([F32, None, None])
+    with pytest.raises(MXNetError, match="Type inconsistent"):
+        Node("_contrib_requantize").infer_type([F32, None, None])
+    with pytest.raises(MXNetError, match="relu"):
+        Node("_contrib_quantized_act", act_type="tanh").infer_type([I8, None, None])
+    assert Node("_contrib_quantize_v2").infer_type([I8])[1][0] == I8   # pass-through input
