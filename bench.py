@@ -29,6 +29,15 @@ METRIC = "int8 FC TOPS (% MFMA peak) + quant/requant GB/s (% HBM peak), 1 GPU"
 HBM_PEAK_GBS = 8000.0    # MI355X HBM3E
 INT8_PEAK_TOPS = 5000.0  # MI355X dense int8 MFMA
 
+# HBM bytes per launch of the workload's kernel from `rocprofv3 --pmc FETCH_SIZE` and
+# `--pmc WRITE_SIZE` runs (FETCH_SIZE x 2.00 per the copy-kernel calibration); the
+# summaries are profiles/fc_dma_kernel_4096.md, profiles/quantize_kernel_64M.md and
+# profiles/copy_calibration_64M.md.  None = not measured.
+MEASURED_TRAFFIC_BYTES = {
+    "fc4096": 2.0 * 49309.8 * 1024 + 16384.1 * 1024,
+    "quantize": 2.0 * 131102.5 * 1024 + 65536.1 * 1024,
+}
+
 
 def parse_args():
     ap = argparse.ArgumentParser()
@@ -37,7 +46,7 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="fc4096",
                     choices=["fc4096", "fc8192", "quantize", "quantize_uncal", "quantize_uint8",
-                             "requantize", "requantize_uncal", "dequantize"])
+                             "requantize", "requantize_uncal", "dequantize", "copy"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-cast-ops", action="store_true")
     return ap.parse_args()
@@ -234,7 +243,35 @@ class CastWorkload:
                           % (n, reps, dt)}
 
 
+class CopyWorkload:
+    """A plain device copy of known size (torch's copy kernel): the yardstick the
+    FETCH_SIZE / WRITE_SIZE counters are scaled by, not a product kernel."""
+    N = 1 << 26
+
+    def __init__(self, torch):
+        self.torch = torch
+        self.bound = "hbm"
+        self.kernel = "torch elementwise copy"
+        self.name = "fp32 copy, %d elements (counter calibration)" % self.N
+        self.bytes = 8.0 * self.N
+        self.src = [torch.randn(self.N, device="cuda") for _ in range(2)]
+        self.dst = torch.empty(self.N, device="cuda")
+        self.i = 0
+
+    def step(self):
+        self.dst.copy_(self.src[self.i % 2])
+        self.i += 1
+
+    def value(self, sec_per_step):
+        return self.bytes / sec_per_step / 1e9, "GB/s"
+
+    def cpu_baseline(self, oracle, budget_s=0):
+        return None
+
+
 def make_workload(name, torch, capi, lib):
+    if name == "copy":
+        return CopyWorkload(torch)
     if name == "fc4096":
         return FcWorkload(4096, torch, capi, lib)
     if name == "fc8192":
@@ -259,7 +296,7 @@ def timed_run(torch, wl, steps, warmup):
     return wall, ev0.elapsed_time(ev1) / 1e3
 
 
-def roofline_of(wl, event_s_per_launch):
+def roofline_of(wl, event_s_per_launch, key=None):
     if wl.bound == "mfma":
         achieved = wl.ops / event_s_per_launch / 1e12
         peak, unit = INT8_PEAK_TOPS, "TOP/s"
@@ -267,7 +304,8 @@ def roofline_of(wl, event_s_per_launch):
         achieved = wl.bytes / event_s_per_launch / 1e9
         peak, unit = HBM_PEAK_GBS, "GB/s"
     return {"bound": wl.bound, "kernel": wl.kernel, "achieved": round(achieved, 1), "peak": peak,
-            "unit": unit, "frac": round(achieved / peak, 4), "traffic": None,
+            "unit": unit, "frac": round(achieved / peak, 4),
+            "traffic": MEASURED_TRAFFIC_BYTES.get(key),
             "avg_launch_us": round(event_s_per_launch * 1e6, 2)}
 
 
@@ -305,7 +343,7 @@ def main():
         "data": "synthetic",
         "config": {"workload": wl.name},
         "device": torch.cuda.get_device_name(0),
-        "roofline": roofline_of(wl, ev / args.steps),
+        "roofline": roofline_of(wl, ev / args.steps, args.workload),
     }
 
     if not args.no_cast_ops:
@@ -317,7 +355,7 @@ def main():
             w2 = make_workload(kind, torch, capi, lib)
             steps2 = 20 if kind == "fc8192" else 60
             wall2, ev2 = timed_run(torch, w2, steps2, 5)
-            r = roofline_of(w2, ev2 / steps2)
+            r = roofline_of(w2, ev2 / steps2, kind)
             r["workload"] = w2.name
             rows.append(r)
             del w2
