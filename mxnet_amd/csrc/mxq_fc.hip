@@ -139,6 +139,8 @@ void launch_fc(hipStream_t s, const int8_t* data, const int8_t* weight, int M, i
                       static_cast<long long>(M) * K < (1LL << 31) &&
                       static_cast<long long>(N) * K < (1LL << 31);
   if (cfg >= 11 && cfg <= 18) MXQ_CHECK(dma_ok, "shape does not qualify for the DMA kernels");
+  if (cfg == 17 || cfg == 18)
+    MXQ_CHECK(K % 128 == 0, "the two-stages-per-barrier kernels need K % 128 == 0");
   switch (cfg) {
     case 11: launch_dma<CfgL8, 3, 0>(s, a); break;
     case 12: launch_dma<CfgL8, 4, 1>(s, a); break;
@@ -146,6 +148,8 @@ void launch_fc(hipStream_t s, const int8_t* data, const int8_t* weight, int M, i
     case 14: launch_dma<CfgL4, 3, 0>(s, a); break;
     case 15: launch_dma<CfgL4, 4, 1>(s, a); break;
     case 16: launch_dma<CfgL4, 4, 2>(s, a); break;
+    case 17: launch_dma<CfgL8, 5, 3>(s, a); break;
+    case 18: launch_dma<CfgL4, 5, 3>(s, a); break;
     case 1: launch_cfg<CfgL8>(s, a, aligned); break;
     case 2: launch_cfg<CfgL4>(s, a, aligned); break;
     case 3: launch_cfg<CfgM>(s, a, aligned); break;

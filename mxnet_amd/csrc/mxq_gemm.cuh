@@ -433,7 +433,7 @@ __device__ __forceinline__ void gemm_mainloop_dma(v16i (&acc)[Cfg::MI][Cfg::NI],
       for (int v = 0; v < 16; ++v) acc[mi][ni][v] = 0;
 
 #pragma unroll
-  for (int s = 0; s < NS - 1; ++s) issue(s);
+  for (int s = 0; s < (PIPE == 3 ? 3 : NS - 1); ++s) issue(s);
 
   if (PIPE == 0) {
     for (int kt = 0; kt < KT; ++kt) {
@@ -447,7 +447,7 @@ __device__ __forceinline__ void gemm_mainloop_dma(v16i (&acc)[Cfg::MI][Cfg::NI],
         mma(fa, fb);
       }
     }
-  } else {
+  } else if (PIPE == 1 || PIPE == 2) {
     static_assert(KS % 2 == 0, "fragment ping-pong assumes an even k-step count");
     v4i fa[2][MI], fb[2][NI];
     wait_vmcnt<(NS >= 4 ? NS - 3 : 0) * CPT>();  // stages 0 and 1 landed
@@ -495,6 +495,55 @@ __device__ __forceinline__ void gemm_mainloop_dma(v16i (&acc)[Cfg::MI][Cfg::NI],
         }
       }
       wait_vmcnt<(NS >= 4 ? NS - 3 : 0) * CPT>();  // stage kt+2 landed for this wave
+      __builtin_amdgcn_s_barrier();
+    }
+  }
+  if (PIPE == 3) {
+    // Two stages per barrier on a 5-stage ring: during super-step (kt, kt+1) the
+    // ring holds kt, kt+1 (being consumed), kt+2 (its first fragments are fetched
+    // before the closing barrier) and receives kt+3, kt+4 in the two buffers the
+    // previous super-step freed; everything issued in a super-step must have landed
+    // at its closing barrier, so the wait is vmcnt(0).  Needs an even stage count.
+    static_assert(PIPE != 3 || NS == 5, "two stages per barrier need a 5-stage ring");
+    static_assert(KS % 2 == 0, "fragment ping-pong assumes an even k-step count");
+    constexpr int SLOTS = MI * NI;
+    constexpr int NF = MI + NI;
+    v4i fa[2][MI], fb[2][NI];
+    wait_vmcnt<0>();  // the prologue issued stages 0, 1, 2
+    __builtin_amdgcn_s_barrier();
+    read_frags(0, 0, fa[0], fb[0]);
+    for (int kt = 0; kt < KT; kt += 2) {
+#pragma unroll
+      for (int st = 0; st < 2; ++st) {
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+          const int cur = ks & 1, nxt = cur ^ 1;
+          const int nstage = (ks + 1 < KS) ? kt + st : kt + st + 1;
+          const int nks = (ks + 1 < KS) ? ks + 1 : 0;
+#pragma unroll
+          for (int mi = 0; mi < MI; ++mi) {
+#pragma unroll
+            for (int ni = 0; ni < NI; ++ni) {
+              const int step = mi * NI + ni;
+              acc[mi][ni] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fb[cur][ni], fa[cur][mi],
+                                                                  acc[mi][ni], 0, 0, 0);
+#pragma unroll
+              for (int f = 0; f < NF; ++f)
+                if (f * SLOTS / NF == step) read_one(nstage, nks, f, fa[nxt], fb[nxt]);
+              // both new stages go out during the first stage of the super-step (into
+              // the two buffers freed by the previous one): kt+3 in k-step 0, kt+4 in
+              // k-step 1
+              if (st == 0) {
+#pragma unroll
+                for (int j = 0; j < CPT; ++j)
+                  if (j * SLOTS / CPT == step) issue_one(kt + 3 + ks, j);
+              }
+              __builtin_amdgcn_sched_barrier(0);
+            }
+          }
+        }
+      }
+      wait_vmcnt<0>();
       __builtin_amdgcn_s_barrier();
     }
   }
