@@ -22,6 +22,9 @@ namespace mxq {
 
 int g_conv_config = 0;  // 0 = choose by shape
 
+void launch_fc(hipStream_t s, const int8_t* data, const int8_t* weight, int M, int N, int K,
+               int ldo, const Epilogue& epi);
+
 namespace {
 
 struct ConvArgs {
@@ -132,11 +135,109 @@ __global__ __launch_bounds__(Cfg::kThreads) void conv_kernel(ConvArgs p) {
   if (blockIdx.x == 0 && threadIdx.x == 0) epilogue_ranges(p.epi);
 }
 
+// Activation operand of the direct-to-LDS main loop: lane state for "16 channels of
+// one filter tap of one output pixel", advanced stage by stage without divisions.
+// Halo taps, rows past the last pixel and the K tail are sent to an out-of-range
+// buffer offset and arrive in LDS as zeros.  Needs C % 16 == 0.
+template <class Cfg, int INSTR>
+struct ConvIssuer {
+  int pix[INSTR];           // byte offset of pixel (n, ih0, iw0), may be negative
+  int ih0[INSTR], iw0[INSTR];
+  bool ok[INSTR];
+  int cc, kh, kw;           // position of this lane's chunk in the stage issued next
+  int dih, diw, tapoff;     // kh*dilate_h, kw*dilate_w, ((kh*dh)*W + kw*dw)*C
+  int C, H, W, KH, KW, dh, dw;
+  v4i rsrc;
+
+  __device__ __forceinline__ void init(const ConvArgs& a, int row_begin, int wave, int lane) {
+    C = a.C; H = a.H; W = a.W; KH = a.KH; KW = a.KW; dh = a.dh; dw = a.dw;
+    rsrc = make_rsrc(a.data, static_cast<uint32_t>(a.N) * a.H * a.W * a.C);
+    DmaLane<Cfg> g;
+    g.init(wave, lane);
+    const int tap = g.c16 / C;
+    cc = g.c16 - tap * C;
+    kh = tap / KW;
+    kw = tap - kh * KW;
+    retap();
+    const int ohow = a.OH * a.OW;
+#pragma unroll
+    for (int i = 0; i < INSTR; ++i) {
+      const int m = row_begin + g.row0 + i * DmaLane<Cfg>::kRowStep;
+      ok[i] = m < a.M;
+      const int mm = ok[i] ? m : 0;
+      const int n = mm / ohow;
+      const int rem = mm - n * ohow;
+      const int oh = rem / a.OW;
+      const int ow = rem - oh * a.OW;
+      ih0[i] = oh * a.sh - a.ph;
+      iw0[i] = ow * a.sw - a.pw;
+      pix[i] = ((n * H + ih0[i]) * W + iw0[i]) * C;
+    }
+  }
+  __device__ __forceinline__ void retap() {
+    dih = kh * dh;
+    diw = kw * dw;
+    tapoff = (dih * W + diw) * C;
+  }
+  __device__ __forceinline__ void issue(int i, int, uint32_t lds_addr) {
+    const int ih = ih0[i] + dih, iw = iw0[i] + diw;
+    const bool v = ok[i] && kh < KH && static_cast<unsigned>(ih) < static_cast<unsigned>(H) &&
+                   static_cast<unsigned>(iw) < static_cast<unsigned>(W);
+    const uint32_t off = v ? static_cast<uint32_t>(pix[i] + tapoff + cc) : kOutOfRange;
+    dma_buffer(lds_addr, off, rsrc);
+  }
+  __device__ __forceinline__ void stage_done() {
+    cc += Cfg::BK;
+    while (cc >= C) {
+      cc -= C;
+      if (++kw == KW) {
+        kw = 0;
+        ++kh;
+      }
+    }
+    retap();
+  }
+};
+
+template <class Cfg, int NS, int PIPE>
+__global__ __launch_bounds__(Cfg::kThreads) void conv_dma_kernel(ConvArgs p) {
+  __shared__ __attribute__((aligned(16))) v4i lds[NS * Cfg::STAGE_SLOTS];
+  const int tiles_m = (p.M + Cfg::BM - 1) / Cfg::BM, tiles_n = (p.O + Cfg::BN - 1) / Cfg::BN;
+  int tm, tn;
+  tile_coords(blockIdx.x, tiles_m, tiles_n, tm, tn);
+  const int m0 = tm * Cfg::BM, n0 = tn * Cfg::BN;
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+
+  ConvIssuer<Cfg, Cfg::A_CHUNKS> ai;
+  RowIssuerBuffer<Cfg, Cfg::B_CHUNKS> bi;
+  ai.init(p, m0, wave, lane);
+  bi.init(p.weight, n0, p.O, p.K, wave, lane);
+
+  v16i acc[Cfg::MI][Cfg::NI];
+  gemm_mainloop_dma<Cfg, NS, PIPE>(acc, ai, bi, (p.K + Cfg::BK - 1) / Cfg::BK, lds);
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+
+  static_assert(NS * Cfg::STAGE_SLOTS * 16 >=
+                    Cfg::BN * 4 + (Cfg::kThreads / 64) * Cfg::TM * (Cfg::TN + 16),
+                "stage ring too small for the epilogue transpose");
+  gemm_epilogue_lds<Cfg>(acc, p.epi, m0, n0, p.M, p.O, static_cast<size_t>(p.O), lds);
+  if (blockIdx.x == 0 && threadIdx.x == 0) epilogue_ranges(p.epi);
+}
+
 typedef GemmCfg<256, 256, 64, 2, 4> CfgL8;   // 8 waves, wave tile 128 x 64
 typedef GemmCfg<256, 128, 64, 4, 2> CfgW128; // 8 waves, wave tile 64 x 64
 typedef GemmCfg<256, 64, 64, 4, 1> CfgW64;   // 4 waves, wave tile 64 x 64
 typedef GemmCfg<128, 128, 64, 2, 2> CfgM;    // 4 waves, wave tile 64 x 64
 typedef GemmCfg<64, 64, 64, 2, 2> CfgS;      // 4 waves, wave tile 32 x 32
+typedef GemmCfg<256, 256, 64, 2, 2> CfgL4;   // 4 waves, wave tile 128 x 128
+
+template <class Cfg, int NS, int PIPE>
+void launch_dma(hipStream_t s, const ConvArgs& a) {
+  const int tiles = ((a.M + Cfg::BM - 1) / Cfg::BM) * ((a.O + Cfg::BN - 1) / Cfg::BN);
+  hipLaunchKernelGGL((conv_dma_kernel<Cfg, NS, PIPE>), dim3(tiles), dim3(Cfg::kThreads), 0, s, a);
+  MXQ_LAUNCH_CHECK();
+}
 
 template <class Cfg>
 void launch_cfg(hipStream_t s, const ConvArgs& a, bool aligned) {
@@ -247,7 +348,16 @@ int mxq_quantized_conv_nhwc(void* stream, const int8_t* data, const int8_t* weig
 
   hipStream_t s = static_cast<hipStream_t>(stream);
   const bool aligned = (C % 16 == 0) && aligned16(data) && aligned16(weight);
+  const long long data_bytes = static_cast<long long>(N) * H * W * C;
+  const bool dma_ok = aligned && data_bytes < (1LL << 31) &&
+                      static_cast<long long>(O) * a.K < (1LL << 31);
   int cfg = g_conv_config;
+  // a 1x1, unit-stride, unpadded convolution is the FC of the flattened pixels
+  if (cfg == 0 && KH == 1 && KW == 1 && stride_h == 1 && stride_w == 1 && pad_h == 0 &&
+      pad_w == 0) {
+    launch_fc(s, data, weight, a.M, O, C, O, e);
+    return 0;
+  }
   if (cfg == 0) {
     const long cus = num_cus();
     auto tiles = [&](int bm, int bn) {
@@ -258,13 +368,21 @@ int mxq_quantized_conv_nhwc(void* stream, const int8_t* data, const int8_t* weig
     else if (O <= 64 && tiles(256, 64) >= cus) cfg = 3;
     else if (tiles(128, 128) >= cus) cfg = 4;
     else cfg = 5;
+    if (dma_ok) cfg += 10;
   }
+  if (cfg > 10) MXQ_CHECK(dma_ok, "shape does not qualify for the direct-to-LDS conv kernels");
   switch (cfg) {
     case 1: launch_cfg<CfgL8>(s, a, aligned); break;
     case 2: launch_cfg<CfgW128>(s, a, aligned); break;
     case 3: launch_cfg<CfgW64>(s, a, aligned); break;
     case 4: launch_cfg<CfgM>(s, a, aligned); break;
     case 5: launch_cfg<CfgS>(s, a, aligned); break;
+    case 11: launch_dma<CfgL8, 4, 2>(s, a); break;
+    case 12: launch_dma<CfgW128, 4, 2>(s, a); break;
+    case 13: launch_dma<CfgW64, 4, 2>(s, a); break;
+    case 14: launch_dma<CfgM, 4, 2>(s, a); break;
+    case 15: launch_dma<CfgS, 4, 2>(s, a); break;
+    case 16: launch_dma<CfgL4, 4, 2>(s, a); break;
     default: MXQ_CHECK(false, "unknown conv tile configuration " << cfg);
   }
   MXQ_API_END();

@@ -23,6 +23,7 @@ struct FcArgs {
   const int8_t* data;    // [M][K]
   const int8_t* weight;  // [N][K]
   int M, N, K;
+  int ldo;               // output row pitch in elements (N for the FC)
   Epilogue epi;
 };
 
@@ -45,40 +46,59 @@ __global__ __launch_bounds__(Cfg::kThreads) void fc_kernel(FcArgs p) {
   gemm_mainloop<Cfg>(acc, af, bf, (p.K + Cfg::BK - 1) / Cfg::BK, lds);
 
   gemm_epilogue<Cfg>(acc, p.epi, m0 + wm * Cfg::TM, n0 + wn * Cfg::TN, p.M, p.N,
-                     static_cast<size_t>(p.N));
+                     static_cast<size_t>(p.ldo));
   if (blockIdx.x == 0 && threadIdx.x == 0) epilogue_ranges(p.epi);
 }
 
 // Direct-to-LDS variant (see gemm_mainloop_dma); launch_fc() picks it when the
-// operands qualify.
-template <class Cfg, int NS, int PIPE>
+// operands qualify.  BUF selects buffer loads (any K % 16 == 0, zero-filled tails)
+// over global loads (K % 64 == 0, clamped rows).
+template <class Cfg, int NS, int PIPE, bool BUF>
 __global__ __launch_bounds__(Cfg::kThreads) void fc_dma_kernel(FcArgs p) {
   __shared__ __attribute__((aligned(16))) v4i lds[NS * Cfg::STAGE_SLOTS];
   const int tiles_m = (p.M + Cfg::BM - 1) / Cfg::BM, tiles_n = (p.N + Cfg::BN - 1) / Cfg::BN;
   int tm, tn;
   tile_coords(blockIdx.x, tiles_m, tiles_n, tm, tn);
   const int m0 = tm * Cfg::BM, n0 = tn * Cfg::BN;
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
 
   v16i acc[Cfg::MI][Cfg::NI];
-  gemm_mainloop_dma<Cfg, NS, PIPE>(acc, p.data, m0, p.M, p.weight, n0, p.N, p.K, lds);
+  const int KT = (p.K + Cfg::BK - 1) / Cfg::BK;
+  if (BUF) {
+    RowIssuerBuffer<Cfg, Cfg::A_CHUNKS> ai;
+    RowIssuerBuffer<Cfg, Cfg::B_CHUNKS> bi;
+    ai.init(p.data, m0, p.M, p.K, wave, lane);
+    bi.init(p.weight, n0, p.N, p.K, wave, lane);
+    gemm_mainloop_dma<Cfg, NS, PIPE>(acc, ai, bi, KT, lds);
+  } else {
+    RowIssuerGlobal<Cfg, Cfg::A_CHUNKS> ai;
+    RowIssuerGlobal<Cfg, Cfg::B_CHUNKS> bi;
+    ai.init(p.data, m0, p.M, p.K, wave, lane);
+    bi.init(p.weight, n0, p.N, p.K, wave, lane);
+    gemm_mainloop_dma<Cfg, NS, PIPE>(acc, ai, bi, KT, lds);
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 
   static_assert(NS * Cfg::STAGE_SLOTS * 16 >=
                     Cfg::BN * 4 + (Cfg::kThreads / 64) * Cfg::TM * (Cfg::TN + 16),
                 "stage ring too small for the epilogue transpose");
-  gemm_epilogue_lds<Cfg>(acc, p.epi, m0, n0, p.M, p.N, static_cast<size_t>(p.N), lds);
+  gemm_epilogue_lds<Cfg>(acc, p.epi, m0, n0, p.M, p.N, static_cast<size_t>(p.ldo), lds);
   if (blockIdx.x == 0 && threadIdx.x == 0) epilogue_ranges(p.epi);
 }
 
-typedef GemmCfg<256, 256, 64, 2, 4> CfgL8;  // 8 waves, wave tile 128 x 64
-typedef GemmCfg<256, 256, 64, 2, 2> CfgL4;  // 4 waves, wave tile 128 x 128
-typedef GemmCfg<128, 128, 64, 2, 2> CfgM;   // 4 waves, wave tile 64 x 64
-typedef GemmCfg<64, 64, 64, 2, 2> CfgS;     // 4 waves, wave tile 32 x 32
+typedef GemmCfg<256, 256, 64, 2, 4> CfgL8;    // 8 waves, wave tile 128 x 64
+typedef GemmCfg<256, 256, 64, 2, 2> CfgL4;    // 4 waves, wave tile 128 x 128
+typedef GemmCfg<256, 128, 64, 4, 2> CfgW128;  // 8 waves, wave tile 64 x 64
+typedef GemmCfg<256, 64, 64, 4, 1> CfgW64;    // 4 waves, wave tile 64 x 64
+typedef GemmCfg<128, 128, 64, 2, 2> CfgM;     // 4 waves, wave tile 64 x 64
+typedef GemmCfg<64, 64, 64, 2, 2> CfgS;       // 4 waves, wave tile 32 x 32
 
-template <class Cfg, int NS, int PIPE>
+template <class Cfg, int NS, int PIPE, bool BUF>
 void launch_dma(hipStream_t s, const FcArgs& a) {
   const int tiles = ((a.M + Cfg::BM - 1) / Cfg::BM) * ((a.N + Cfg::BN - 1) / Cfg::BN);
-  hipLaunchKernelGGL((fc_dma_kernel<Cfg, NS, PIPE>), dim3(tiles), dim3(Cfg::kThreads), 0, s,
-                     a);
+  hipLaunchKernelGGL((fc_dma_kernel<Cfg, NS, PIPE, BUF>), dim3(tiles), dim3(Cfg::kThreads), 0,
+                     s, a);
   MXQ_LAUNCH_CHECK();
 }
 
@@ -105,55 +125,73 @@ int num_cus() {
 
 }  // namespace
 
+// Tile configurations:
+//   1..4    register-staged kernels (any shape): 256x256x8w, 256x256x4w, 128x128, 64x64
+//   11, 12  direct-to-LDS 256x256, 8 waves: compiler-scheduled / pinned pipeline
+//   14, 16  direct-to-LDS 256x256, 4 waves: compiler-scheduled / pinned pipeline
+//   21..24  direct-to-LDS buffer-load kernels 256x128, 256x64, 128x128, 64x64
+//   31, 32  as 12 / 16 with buffer loads (K % 16 == 0 instead of K % 64 == 0)
 void launch_fc(hipStream_t s, const int8_t* data, const int8_t* weight, int M, int N, int K,
-               const Epilogue& epi) {
+               int ldo, const Epilogue& epi) {
   FcArgs a;
   a.data = data;
   a.weight = weight;
   a.M = M;
   a.N = N;
   a.K = K;
+  a.ldo = ldo;
   a.epi = epi;
   const bool aligned = (K % 16 == 0) && aligned16(data) && aligned16(weight);
+  // direct-to-LDS kernels: operands below 2 GiB; K a multiple of the 64-byte stage for
+  // the global-load form, of 16 for the buffer-load form
+  const bool buf_ok = aligned && K >= 16 && static_cast<long long>(M) * K < (1LL << 31) &&
+                      static_cast<long long>(N) * K < (1LL << 31);
+  const bool glb_ok = buf_ok && (K % 64 == 0);
   int cfg = g_fc_config;
   if (cfg == 0) {
     const long cus = num_cus();
     auto tiles = [&](int bm, int bn) {
       return static_cast<long>((M + bm - 1) / bm) * ((N + bn - 1) / bn);
     };
-    if (tiles(256, 256) >= cus)
-      cfg = 1;
-    else if (tiles(128, 128) >= cus)
-      cfg = 3;
-    else
-      cfg = 4;
-    // large tiles that qualify go straight to LDS: 8 waves when only the int8
-    // output is written, 4 waves (128 x 128 per wave) when int32 is stored as well
-    const bool dma_shape = (K % 16 == 0) && aligned16(data) && aligned16(weight) && K >= 64 &&
-                           (K % 64 == 0) && static_cast<long long>(M) * K < (1LL << 31) &&
-                           static_cast<long long>(N) * K < (1LL << 31);
-    if (cfg == 1 && dma_shape) cfg = (epi.out32 != nullptr) ? 16 : 13;
+    if (buf_ok) {
+      // largest tile that still gives every CU work; 8 waves when only the int8 output
+      // is written, 4 waves (128 x 128 per wave) when int32 is stored as well
+      if (tiles(256, 256) >= cus)
+        cfg = glb_ok ? ((epi.out32 != nullptr) ? 16 : 12) : ((epi.out32 != nullptr) ? 32 : 31);
+      else if (N > 64 && tiles(256, 128) >= cus)
+        cfg = 21;
+      else if (N <= 64 && tiles(256, 64) >= cus)
+        cfg = 22;
+      else if (tiles(128, 128) >= cus)
+        cfg = 23;
+      else
+        cfg = 24;
+    } else {
+      if (tiles(256, 256) >= cus)
+        cfg = 1;
+      else if (tiles(128, 128) >= cus)
+        cfg = 3;
+      else
+        cfg = 4;
+    }
   }
-  // direct-to-LDS kernels: K a multiple of the 64-byte stage, operands below 2 GiB
-  const bool dma_ok = aligned && K >= 64 && (K % 64 == 0) &&
-                      static_cast<long long>(M) * K < (1LL << 31) &&
-                      static_cast<long long>(N) * K < (1LL << 31);
-  if (cfg >= 11 && cfg <= 18) MXQ_CHECK(dma_ok, "shape does not qualify for the DMA kernels");
-  if (cfg == 17 || cfg == 18)
-    MXQ_CHECK(K % 128 == 0, "the two-stages-per-barrier kernels need K % 128 == 0");
+  if (cfg >= 11 && cfg <= 16) MXQ_CHECK(glb_ok, "shape does not qualify for the DMA kernels");
+  if (cfg >= 21) MXQ_CHECK(buf_ok, "shape does not qualify for the buffer-load DMA kernels");
   switch (cfg) {
-    case 11: launch_dma<CfgL8, 3, 0>(s, a); break;
-    case 12: launch_dma<CfgL8, 4, 1>(s, a); break;
-    case 13: launch_dma<CfgL8, 4, 2>(s, a); break;
-    case 14: launch_dma<CfgL4, 3, 0>(s, a); break;
-    case 15: launch_dma<CfgL4, 4, 1>(s, a); break;
-    case 16: launch_dma<CfgL4, 4, 2>(s, a); break;
-    case 17: launch_dma<CfgL8, 5, 3>(s, a); break;
-    case 18: launch_dma<CfgL4, 5, 3>(s, a); break;
     case 1: launch_cfg<CfgL8>(s, a, aligned); break;
     case 2: launch_cfg<CfgL4>(s, a, aligned); break;
     case 3: launch_cfg<CfgM>(s, a, aligned); break;
     case 4: launch_cfg<CfgS>(s, a, aligned); break;
+    case 11: launch_dma<CfgL8, 4, 0, false>(s, a); break;
+    case 12: launch_dma<CfgL8, 4, 2, false>(s, a); break;
+    case 14: launch_dma<CfgL4, 4, 0, false>(s, a); break;
+    case 16: launch_dma<CfgL4, 4, 2, false>(s, a); break;
+    case 21: launch_dma<CfgW128, 4, 2, true>(s, a); break;
+    case 22: launch_dma<CfgW64, 4, 2, true>(s, a); break;
+    case 23: launch_dma<CfgM, 4, 2, true>(s, a); break;
+    case 24: launch_dma<CfgS, 4, 2, true>(s, a); break;
+    case 31: launch_dma<CfgL8, 4, 2, true>(s, a); break;
+    case 32: launch_dma<CfgL4, 4, 2, true>(s, a); break;
     default: MXQ_CHECK(false, "unknown fc tile configuration " << cfg);
   }
 }
@@ -195,6 +233,6 @@ extern "C" int mxq_quantized_fc(void* stream, const int8_t* data, const int8_t* 
   e.relu = relu;
   float a = fabsf(min_calib), b = fabsf(max_calib);
   e.real_range = (a < b) ? b : a;
-  launch_fc(static_cast<hipStream_t>(stream), data, weight, M, N, K, e);
+  launch_fc(static_cast<hipStream_t>(stream), data, weight, M, N, K, N, e);
   MXQ_API_END();
 }

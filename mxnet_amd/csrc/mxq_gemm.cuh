@@ -297,13 +297,11 @@ __device__ __forceinline__ void gemm_mainloop(v16i (&acc)[Cfg::MI][Cfg::NI], AF&
 }
 
 // ---- direct-to-LDS main loop ------------------------------------------------------
-// Fast path for operands whose K is a multiple of BK, 16-byte aligned and below
-// 2 GiB: tiles go from global memory straight into LDS (global_load_lds_dwordx4,
-// no staging registers, no ds_write) through an NS-stage ring.  Each wave
-// instruction fills 64 consecutive 16-byte slots; the bank swizzle is applied on
-// the global side (lane for slot (r, c') fetches chunk c' ^ swz(r) of row r).
-// Rows past the end of the operand are clamped to its last row: they only feed
-// accumulators that the epilogue never stores.
+// Fast path for 16-byte aligned operands below 2 GiB: tiles go from global memory
+// straight into LDS (global_load_lds_dwordx4 / buffer_load_dwordx4 ... lds: no
+// staging registers, no ds_write) through an NS-stage ring.  Each wave instruction
+// fills 64 consecutive 16-byte slots; the bank swizzle is applied on the global side
+// (lane for slot (r, c') fetches chunk c' ^ swz(r) of row r).
 //
 // The loads are issued through inline assembly, so the compiler's wait-count
 // pass does not see them; completion is enforced here by hand: vmcnt counts
@@ -311,8 +309,8 @@ __device__ __forceinline__ void gemm_mainloop(v16i (&acc)[Cfg::MI][Cfg::NI], AF&
 // are outstanding before it joins the work-group barrier that publishes a stage.
 #pragma clang diagnostic push
 #pragma clang diagnostic ignored "-Winline-asm"
-__device__ __forceinline__ void lds_dma16(uint32_t lds_byte_addr, uint32_t voffset,
-                                          const int8_t* sbase) {
+__device__ __forceinline__ void dma_global(uint32_t lds_byte_addr, uint32_t voffset,
+                                           const int8_t* sbase) {
 #ifndef MXQ_LAB_SKIP_DMA
   asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2"
                :
@@ -320,72 +318,154 @@ __device__ __forceinline__ void lds_dma16(uint32_t lds_byte_addr, uint32_t voffs
                : "memory", "m0");
 #endif
 }
+// Buffer form: lanes whose offset is outside [0, num_records) deliver zeros, which
+// is how image halos, rows past the end of an operand and the K tail are filled.
+__device__ __forceinline__ void dma_buffer(uint32_t lds_byte_addr, uint32_t voffset, v4i rsrc) {
+#ifndef MXQ_LAB_SKIP_DMA
+  asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
+               :
+               : "s"(lds_byte_addr), "v"(voffset), "s"(rsrc)
+               : "memory", "m0");
+#endif
+}
 #pragma clang diagnostic pop
+
+constexpr uint32_t kOutOfRange = 0x80000000u;  // operands are below 2 GiB
+
+// Raw buffer descriptor over [base, base + bytes): stride 0, 32-bit data format.
+__device__ __forceinline__ v4i make_rsrc(const void* base, uint32_t bytes) {
+  const uint64_t a = reinterpret_cast<uint64_t>(base);
+  v4i r;
+  r.x = __builtin_amdgcn_readfirstlane(static_cast<int>(static_cast<uint32_t>(a)));
+  r.y = __builtin_amdgcn_readfirstlane(static_cast<int>(static_cast<uint32_t>(a >> 32)));
+  r.z = __builtin_amdgcn_readfirstlane(static_cast<int>(bytes));
+  r.w = 0x00020000;
+  return r;
+}
 
 template <int N>
 __device__ __forceinline__ void wait_vmcnt() {
   static_assert(N >= 0 && N < 64, "vmcnt range");
   asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
 }
+// Wait until at most `ahead` (clamped to [0, MAXS]) stages of CPT loads are outstanding.
+template <int CPT, int MAXS>
+__device__ __forceinline__ void wait_ahead(int ahead) {
+  if constexpr (MAXS <= 0) {
+    wait_vmcnt<0>();
+  } else {
+    if (ahead >= MAXS)
+      wait_vmcnt<MAXS * CPT>();
+    else
+      wait_ahead<CPT, MAXS - 1>(ahead);
+  }
+}
 
-// Per-thread addressing of one operand for the DMA path.
-template <class Cfg, int INSTR, int ROWS_TILE>
-struct DmaOperand {
-  uint32_t voff[INSTR];  // byte offset of this lane's chunk from the operand base at k = 0
-  __device__ __forceinline__ void init(int row0, int rows, int K, int wave, int lane) {
-    constexpr int NW = Cfg::kThreads / 64;
-#pragma unroll
-    for (int i = 0; i < INSTR; ++i) {
-      const int slot = (i * NW + wave) * 64 + lane;
-      const int r = slot / Cfg::CH;
-      const int c = (slot % Cfg::CH) ^ swz<Cfg::CH>(r);
-      int row = row0 + r;
-      row = row < rows ? row : rows - 1;
-      voff[i] = static_cast<uint32_t>(row) * static_cast<uint32_t>(K) + c * 16;
-    }
+// Slot geometry of DMA instruction i of a wave: rows (i*NW + wave)*(64/CH) ..., the
+// chunk a lane fetches does not depend on i (swz() only looks at row bits the lane
+// index provides).
+template <class Cfg>
+struct DmaLane {
+  int row0;   // tile row of instruction 0 for this lane
+  int c16;    // byte offset (within a 64-byte stage row) of the chunk this lane fetches
+  static constexpr int kRowStep = (Cfg::kThreads / 64) * (64 / Cfg::CH);  // rows between instrs
+  __device__ __forceinline__ void init(int wave, int lane) {
+    const int slot = wave * 64 + lane;
+    row0 = slot / Cfg::CH;
+    c16 = ((slot % Cfg::CH) ^ swz<Cfg::CH>(row0)) * 16;
   }
 };
 
+// K-contiguous row-major operand (FC activation, every weight) through
+// global_load_lds.  Needs K % BK == 0; rows past the end are clamped to the last
+// row (they only feed accumulators that are never stored).
+template <class Cfg, int INSTR>
+struct RowIssuerGlobal {
+  uint32_t voff[INSTR];
+  const int8_t* base;
+  __device__ __forceinline__ void init(const int8_t* b, int row_begin, int rows, int K, int wave,
+                                       int lane) {
+    base = b;
+    DmaLane<Cfg> g;
+    g.init(wave, lane);
+#pragma unroll
+    for (int i = 0; i < INSTR; ++i) {
+      int row = row_begin + g.row0 + i * DmaLane<Cfg>::kRowStep;
+      row = row < rows ? row : rows - 1;
+      voff[i] = static_cast<uint32_t>(row) * static_cast<uint32_t>(K) + g.c16;
+    }
+  }
+  __device__ __forceinline__ void issue(int i, int stage, uint32_t lds_addr) {
+    dma_global(lds_addr, voff[i], base + static_cast<size_t>(stage) * Cfg::BK);
+  }
+  __device__ __forceinline__ void stage_done() {}
+};
+
+// The same operand through buffer loads: any K that is a multiple of 16; rows past
+// the end and chunks past K arrive as zeros.
+template <class Cfg, int INSTR>
+struct RowIssuerBuffer {
+  uint32_t roff[INSTR];
+  int c16, K;
+  v4i rsrc;
+  __device__ __forceinline__ void init(const int8_t* b, int row_begin, int rows, int K_, int wave,
+                                       int lane) {
+    K = K_;
+    rsrc = make_rsrc(b, static_cast<uint32_t>(rows) * static_cast<uint32_t>(K_));
+    DmaLane<Cfg> g;
+    g.init(wave, lane);
+    c16 = g.c16;
+#pragma unroll
+    for (int i = 0; i < INSTR; ++i) {
+      const int row = row_begin + g.row0 + i * DmaLane<Cfg>::kRowStep;
+      roff[i] = row < rows ? static_cast<uint32_t>(row) * static_cast<uint32_t>(K_) : kOutOfRange;
+    }
+  }
+  __device__ __forceinline__ void issue(int i, int stage, uint32_t lds_addr) {
+    const int k0 = stage * Cfg::BK + c16;
+    const uint32_t v = (k0 < K && roff[i] != kOutOfRange) ? roff[i] + k0 : kOutOfRange;
+    dma_buffer(lds_addr, v, rsrc);
+  }
+  __device__ __forceinline__ void stage_done() {}
+};
+
 // PIPE selects the software pipeline of the K loop:
-//   0  wait + barrier, issue next DMA, read fragments, MFMA   (compiler scheduled)
-//   1  as 0 plus fragment double-buffering across the barrier (compiler scheduled)
-//   2  as 1 with the instruction order pinned: after every MFMA exactly one
-//      fragment read for the next k-step (and, in the first k-step, one DMA issue)
-//      is placed, so the matrix pipe is fed back-to-back while LDS and DMA work
-//      trickles in between.
-template <class Cfg, int NS, int PIPE>
-__device__ __forceinline__ void gemm_mainloop_dma(v16i (&acc)[Cfg::MI][Cfg::NI],
-                                                  const int8_t* a_base, int a_row0, int a_rows,
-                                                  const int8_t* b_base, int b_row0, int b_rows,
-                                                  int K, v4i* lds) {
+//   0  wait + barrier, issue the next stage, read fragments, MFMA (compiler scheduled)
+//   2  fragments double-buffered in registers across the barrier and the instruction
+//      order pinned: after every MFMA exactly one fragment read for the next k-step
+//      (and, in the first k-step, one DMA issue) is placed, so the matrix pipe is fed
+//      back-to-back while LDS and DMA work trickles in between.
+// AIssuer / BIssuer provide issue(instr, stage, lds_byte_addr) and stage_done(); stages
+// are issued in increasing order, each exactly once, and only stages < KT.
+template <class Cfg, int NS, int PIPE, class AIssuer, class BIssuer>
+__device__ __forceinline__ void gemm_mainloop_dma(v16i (&acc)[Cfg::MI][Cfg::NI], AIssuer& ai,
+                                                  BIssuer& bi, int KT, v4i* lds) {
   constexpr int CH = Cfg::CH, NW = Cfg::kThreads / 64;
   constexpr int AI = Cfg::A_CHUNKS, BI = Cfg::B_CHUNKS, CPT = AI + BI;
   constexpr int MI = Cfg::MI, NI = Cfg::NI, KS = Cfg::KS;
   constexpr int STAGE_BYTES = Cfg::STAGE_SLOTS * 16;
   static_assert((Cfg::BM * CH) % (NW * 64) == 0 && (Cfg::BN * CH) % (NW * 64) == 0, "dma tiling");
+  static_assert(PIPE == 0 || PIPE == 2, "pipeline variant");
   static_assert(PIPE == 0 || NS >= 4, "cross-barrier fragment prefetch needs 4 stages");
   static_assert(CH == 4, "fragment addressing below assumes 64-byte stage rows");
+  static_assert((NS - 2) * CPT < 64, "vmcnt range");
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave / Cfg::WN, wn = wave % Cfg::WN;
-
-  DmaOperand<Cfg, AI, Cfg::BM> da;
-  DmaOperand<Cfg, BI, Cfg::BN> db;
-  da.init(a_row0, a_rows, K, wave, lane);
-  db.init(b_row0, b_rows, K, wave, lane);
   const uint32_t lds0 = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(lds));
 
-  const int KT = K / Cfg::BK;
-  // DMA instruction j (0 .. CPT-1) of a stage
+  // DMA instruction j (0 .. CPT-1) of a stage; nothing is issued past the last stage
   auto issue_one = [&](int stage, int j) {
-    const int kk = stage < KT ? stage : KT - 1;  // past the end: harmless reload
+    if (stage >= KT) return;
     const uint32_t sb = lds0 + static_cast<uint32_t>(stage % NS) * STAGE_BYTES;
     if (j < AI)
-      lds_dma16(sb + (j * NW + wave) * 1024, da.voff[j],
-                a_base + static_cast<size_t>(kk) * Cfg::BK);
+      ai.issue(j, stage, sb + (j * NW + wave) * 1024);
     else
-      lds_dma16(sb + Cfg::BM * CH * 16 + ((j - AI) * NW + wave) * 1024, db.voff[j - AI],
-                b_base + static_cast<size_t>(kk) * Cfg::BK);
+      bi.issue(j - AI, stage, sb + Cfg::BM * CH * 16 + ((j - AI) * NW + wave) * 1024);
+    if (j == CPT - 1) {
+      ai.stage_done();
+      bi.stage_done();
+    }
   };
   auto issue = [&](int stage) {
 #pragma unroll
@@ -417,13 +497,6 @@ __device__ __forceinline__ void gemm_mainloop_dma(v16i (&acc)[Cfg::MI][Cfg::NI],
 #pragma unroll
     for (int f = 0; f < MI + NI; ++f) read_one(stage, ks, f, fa, fb);
   };
-  auto mma = [&](v4i (&fa)[MI], v4i (&fb)[NI]) {
-#pragma unroll
-    for (int mi = 0; mi < MI; ++mi)
-#pragma unroll
-      for (int ni = 0; ni < NI; ++ni)
-        acc[mi][ni] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fb[ni], fa[mi], acc[mi][ni], 0, 0, 0);
-  };
 
 #pragma unroll
   for (int mi = 0; mi < MI; ++mi)
@@ -433,121 +506,69 @@ __device__ __forceinline__ void gemm_mainloop_dma(v16i (&acc)[Cfg::MI][Cfg::NI],
       for (int v = 0; v < 16; ++v) acc[mi][ni][v] = 0;
 
 #pragma unroll
-  for (int s = 0; s < (PIPE == 3 ? 3 : NS - 1); ++s) issue(s);
+  for (int s = 0; s < NS - 1; ++s) issue(s);  // stages 0 .. min(KT, NS-1)-1
+  auto last_issued = [&](int kt_now) {         // newest stage in flight during step kt_now
+    const int l = kt_now + NS - 2;
+    return l < KT - 1 ? l : KT - 1;
+  };
 
   if (PIPE == 0) {
     for (int kt = 0; kt < KT; ++kt) {
-      wait_vmcnt<(NS - 2) * CPT>();     // this wave's part of stage kt has landed
-      __builtin_amdgcn_s_barrier();     // ... and everybody else's; stage kt-1 is free
+      wait_ahead<CPT, NS - 2>(last_issued(kt) - kt);  // this wave's part of stage kt landed
+      __builtin_amdgcn_s_barrier();                    // ... everybody's; stage kt-1 is free
       issue(kt + NS - 1);
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) {
         v4i fa[MI], fb[NI];
         read_frags(kt, ks, fa, fb);
-        mma(fa, fb);
+#pragma unroll
+        for (int mi = 0; mi < MI; ++mi)
+#pragma unroll
+          for (int ni = 0; ni < NI; ++ni)
+            acc[mi][ni] =
+                __builtin_amdgcn_mfma_i32_32x32x32_i8(fb[ni], fa[mi], acc[mi][ni], 0, 0, 0);
       }
     }
-  } else if (PIPE == 1 || PIPE == 2) {
+  } else {
     static_assert(KS % 2 == 0, "fragment ping-pong assumes an even k-step count");
+    constexpr int NF = MI + NI, SLOTS = MI * NI;
     v4i fa[2][MI], fb[2][NI];
-    wait_vmcnt<(NS >= 4 ? NS - 3 : 0) * CPT>();  // stages 0 and 1 landed
+    // stages 0 and 1 landed: everything newer than stage 1 may stay in flight
+    wait_ahead<CPT, NS - 3>(last_issued(0) - 1);
     __builtin_amdgcn_s_barrier();
     read_frags(0, 0, fa[0], fb[0]);
     for (int kt = 0; kt < KT; ++kt) {
-      if (PIPE == 1) {
-        issue(kt + NS - 1);  // overwrites stage kt-1, consumed before the last barrier
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
-          if (ks + 1 < KS)
-            read_frags(kt, ks + 1, fa[(ks + 1) & 1], fb[(ks + 1) & 1]);
-          else
-            read_frags(kt + 1, 0, fa[(ks + 1) & 1], fb[(ks + 1) & 1]);  // published last barrier
-          mma(fa[ks & 1], fb[ks & 1]);
-        }
-      } else {
+      for (int ks = 0; ks < KS; ++ks) {
+        const int cur = ks & 1, nxt = cur ^ 1;
+        const int nstage = (ks + 1 < KS) ? kt : kt + 1;  // kt+1 was published one barrier ago
+        const int nks = (ks + 1 < KS) ? ks + 1 : 0;
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
-          constexpr int NF = MI + NI;
-          const int cur = ks & 1, nxt = cur ^ 1;
-          const int nstage = (ks + 1 < KS) ? kt : kt + 1;
-          const int nks = (ks + 1 < KS) ? ks + 1 : 0;
+        for (int mi = 0; mi < MI; ++mi) {
 #pragma unroll
-          for (int mi = 0; mi < MI; ++mi) {
+          for (int ni = 0; ni < NI; ++ni) {
+            const int step = mi * NI + ni;
+            acc[mi][ni] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fb[cur][ni], fa[cur][mi],
+                                                                acc[mi][ni], 0, 0, 0);
+            // spread NF fragment reads (and, in k-step 0, the CPT DMA issues of stage
+            // kt+NS-1, which overwrites stage kt-1) over the MFMA slots of this k-step
 #pragma unroll
-            for (int ni = 0; ni < NI; ++ni) {
-              const int step = mi * NI + ni;
-              acc[mi][ni] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fb[cur][ni], fa[cur][mi],
-                                                                  acc[mi][ni], 0, 0, 0);
-              // spread NF fragment reads (and, in k-step 0, CPT DMA issues) over the
-              // MI*NI MFMA slots of this k-step
-              constexpr int SLOTS = MI * NI;
+            for (int f = 0; f < NF; ++f)
+              if (f * SLOTS / NF == step) read_one(nstage, nks, f, fa[nxt], fb[nxt]);
+            if (ks == 0) {
 #pragma unroll
-              for (int f = 0; f < NF; ++f)
-                if (f * SLOTS / NF == step) read_one(nstage, nks, f, fa[nxt], fb[nxt]);
-              if (ks == 0) {
-#pragma unroll
-                for (int j = 0; j < CPT; ++j)
-                  if (j * SLOTS / CPT == step) issue_one(kt + NS - 1, j);
-              }
-              __builtin_amdgcn_sched_barrier(0);
+              for (int j = 0; j < CPT; ++j)
+                if (j * SLOTS / CPT == step) issue_one(kt + NS - 1, j);
             }
+            __builtin_amdgcn_sched_barrier(0);
           }
         }
       }
-      wait_vmcnt<(NS >= 4 ? NS - 3 : 0) * CPT>();  // stage kt+2 landed for this wave
+      // stage kt+2 landed for this wave; newest in flight is min(KT-1, kt+NS-1)
+      wait_ahead<CPT, NS - 3>(last_issued(kt + 1) - (kt + 2));
       __builtin_amdgcn_s_barrier();
     }
   }
-  if (PIPE == 3) {
-    // Two stages per barrier on a 5-stage ring: during super-step (kt, kt+1) the
-    // ring holds kt, kt+1 (being consumed), kt+2 (its first fragments are fetched
-    // before the closing barrier) and receives kt+3, kt+4 in the two buffers the
-    // previous super-step freed; everything issued in a super-step must have landed
-    // at its closing barrier, so the wait is vmcnt(0).  Needs an even stage count.
-    static_assert(PIPE != 3 || NS == 5, "two stages per barrier need a 5-stage ring");
-    static_assert(KS % 2 == 0, "fragment ping-pong assumes an even k-step count");
-    constexpr int SLOTS = MI * NI;
-    constexpr int NF = MI + NI;
-    v4i fa[2][MI], fb[2][NI];
-    wait_vmcnt<0>();  // the prologue issued stages 0, 1, 2
-    __builtin_amdgcn_s_barrier();
-    read_frags(0, 0, fa[0], fb[0]);
-    for (int kt = 0; kt < KT; kt += 2) {
-#pragma unroll
-      for (int st = 0; st < 2; ++st) {
-#pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
-          const int cur = ks & 1, nxt = cur ^ 1;
-          const int nstage = (ks + 1 < KS) ? kt + st : kt + st + 1;
-          const int nks = (ks + 1 < KS) ? ks + 1 : 0;
-#pragma unroll
-          for (int mi = 0; mi < MI; ++mi) {
-#pragma unroll
-            for (int ni = 0; ni < NI; ++ni) {
-              const int step = mi * NI + ni;
-              acc[mi][ni] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fb[cur][ni], fa[cur][mi],
-                                                                  acc[mi][ni], 0, 0, 0);
-#pragma unroll
-              for (int f = 0; f < NF; ++f)
-                if (f * SLOTS / NF == step) read_one(nstage, nks, f, fa[nxt], fb[nxt]);
-              // both new stages go out during the first stage of the super-step (into
-              // the two buffers freed by the previous one): kt+3 in k-step 0, kt+4 in
-              // k-step 1
-              if (st == 0) {
-#pragma unroll
-                for (int j = 0; j < CPT; ++j)
-                  if (j * SLOTS / CPT == step) issue_one(kt + 3 + ks, j);
-              }
-              __builtin_amdgcn_sched_barrier(0);
-            }
-          }
-        }
-      }
-      wait_vmcnt<0>();
-      __builtin_amdgcn_s_barrier();
-    }
-  }
-  wait_vmcnt<0>();  // drain the harmless tail loads before LDS is released
 }
 
 // Stores one wave's accumulators.  m_base/n_base: origin of the wave tile.

@@ -69,7 +69,7 @@ def test_conv_int32(capi, case, use_bias):
     assert (res["omin"].item(), res["omax"].item()) == (rmn, rmx)
 
 
-@pytest.mark.parametrize("cfg", [1, 2, 3, 4, 5])
+@pytest.mark.parametrize("cfg", [1, 2, 3, 4, 5, 11, 12, 13, 14, 15, 16])
 def test_conv_every_tile_config(capi, cfg):
     import mxnet_amd
     N, C, H, W, O, KH, KW, s, p, dl = (2, 32, 19, 19, 72, 3, 3, 1, 1, 1)
@@ -89,6 +89,32 @@ def test_conv_every_tile_config(capi, cfg):
     rq, qmn, qmx = oracle.requantize(ro, rmn, rmx, -0.02, 0.02)
     np.testing.assert_array_equal(res["out8_nchw"].cpu().numpy(), oracle.relu_i8(rq))
     assert (res["rmin"].item(), res["rmax"].item()) == (qmn, qmx)
+
+
+@pytest.mark.parametrize("cfg", [11, 12, 13, 14, 15, 16])
+@pytest.mark.parametrize("case", [(2, 16, 9, 11, 40, 3, 3, 1, 1, 1), (1, 48, 8, 8, 24, 5, 3, 2, 2, 1),
+                                  (2, 64, 14, 14, 96, 1, 1, 2, 0, 1), (1, 16, 12, 12, 20, 3, 3, 1, 2, 2),
+                                  (3, 128, 7, 7, 130, 3, 3, 1, 1, 1)])
+def test_conv_direct_to_lds_configs(capi, cfg, case):
+    """The buffer-load kernels on shapes that stress the tap bookkeeping: C = 16 (four
+    taps per 64-byte stage), C = 48 (taps straddle stages), stride 2, dilation, K tails."""
+    import mxnet_amd
+    N, C, H, W, O, KH, KW, s, p, dl = case
+    d = int8_uniform((N, C, H, W), seed=cfg + C)
+    w = int8_uniform((O, C, KH, KW), seed=cfg + O)
+    b = int8_uniform((O,), seed=cfg)
+    mxnet_amd._lib.set_tuning("conv_config", cfg)
+    try:
+        res = run_conv_nchw(capi, d, w, b, 1.0, 1.0, 1.0, (s, s), (p, p), (dl, dl),
+                            calib=(-0.05, 0.04), relu=False)
+        torch.cuda.synchronize()
+    finally:
+        mxnet_amd._lib.set_tuning("conv_config", 0)
+    ro, rmn, rmx = oracle.quantized_conv(d, w, b, -1.0, 1.0, -1.0, 1.0, -1.0, 1.0, (s, s),
+                                         (p, p), (dl, dl))
+    np.testing.assert_array_equal(res["out32_nchw"].cpu().numpy(), ro)
+    rq, qmn, qmx = oracle.requantize(ro, rmn, rmx, -0.05, 0.04)
+    np.testing.assert_array_equal(res["out8_nchw"].cpu().numpy(), rq)
 
 
 def test_layout_adapters(capi):

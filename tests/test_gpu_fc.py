@@ -57,14 +57,15 @@ def test_fc_int32(capi, M, K, N, use_bias):
     assert (res["omin"].item(), res["omax"].item()) == (rmn, rmx)
 
 
-@pytest.mark.parametrize("cfg", [1, 2, 3, 4, 11, 12, 13, 14, 15, 16, 17, 18])
+@pytest.mark.parametrize("cfg", [1, 2, 3, 4, 11, 12, 14, 16, 21, 22, 23, 24, 31, 32])
 @pytest.mark.parametrize("M,K,N", [(512, 512, 512), (300, 208, 270), (70, 444, 33),
-                                   (300, 192, 270), (1, 64, 1), (1024, 1024, 520)])
+                                   (300, 192, 270), (1, 64, 1), (1024, 1024, 520),
+                                   (130, 16, 70), (257, 80, 64)])
 def test_fc_every_tile_config(capi, cfg, M, K, N):
-    if cfg > 10 and K % 64 != 0:
-        pytest.skip("the direct-to-LDS kernels need K % 64 == 0")
-    if cfg in (17, 18) and K % 128 != 0:
-        pytest.skip("the two-stages-per-barrier kernels need K % 128 == 0")
+    if 10 < cfg < 20 and K % 64 != 0:
+        pytest.skip("the global-load direct-to-LDS kernels need K % 64 == 0")
+    if cfg > 20 and K % 16 != 0:
+        pytest.skip("the buffer-load direct-to-LDS kernels need K % 16 == 0")
     import mxnet_amd
     d = int8_uniform((M, K), seed=cfg + M)
     w = int8_uniform((N, K), seed=cfg + N + 7)
