@@ -131,6 +131,7 @@ int num_cus() {
 //   14, 16  direct-to-LDS 256x256, 4 waves: compiler-scheduled / pinned pipeline
 //   21..24  direct-to-LDS buffer-load kernels 256x128, 256x64, 128x128, 64x64
 //   31, 32  as 12 / 16 with buffer loads (K % 16 == 0 instead of K % 64 == 0)
+//   41..44  as 21..24 with a 2-stage ring (short K)
 void launch_fc(hipStream_t s, const int8_t* data, const int8_t* weight, int M, int N, int K,
                int ldo, const Epilogue& epi) {
   FcArgs a;
@@ -154,18 +155,21 @@ void launch_fc(hipStream_t s, const int8_t* data, const int8_t* weight, int M, i
       return static_cast<long>((M + bm - 1) / bm) * ((N + bn - 1) / bn);
     };
     if (buf_ok) {
-      // largest tile that still gives every CU work; 8 waves when only the int8 output
-      // is written, 4 waves (128 x 128 per wave) when int32 is stored as well
-      if (tiles(256, 256) >= cus)
+      // tile width follows N; the tallest tile that still gives every CU work.  8 waves
+      // when only the int8 output is written, 4 waves (128 x 128 per wave) when int32 is
+      // stored as well.  Short K (one or two stages) uses the 2-stage ring: less LDS,
+      // more resident work-groups to hide the load latency.
+      const bool short_k = K <= 128;
+      if (N > 128 && tiles(256, 256) >= cus)
         cfg = glb_ok ? ((epi.out32 != nullptr) ? 16 : 12) : ((epi.out32 != nullptr) ? 32 : 31);
       else if (N > 64 && tiles(256, 128) >= cus)
-        cfg = 21;
+        cfg = short_k ? 41 : 21;
       else if (N <= 64 && tiles(256, 64) >= cus)
-        cfg = 22;
+        cfg = short_k ? 42 : 22;
       else if (tiles(128, 128) >= cus)
-        cfg = 23;
+        cfg = short_k ? 43 : 23;
       else
-        cfg = 24;
+        cfg = short_k ? 44 : 24;
     } else {
       if (tiles(256, 256) >= cus)
         cfg = 1;
@@ -190,6 +194,10 @@ void launch_fc(hipStream_t s, const int8_t* data, const int8_t* weight, int M, i
     case 22: launch_dma<CfgW64, 4, 2, true>(s, a); break;
     case 23: launch_dma<CfgM, 4, 2, true>(s, a); break;
     case 24: launch_dma<CfgS, 4, 2, true>(s, a); break;
+    case 41: launch_dma<CfgW128, 2, 0, true>(s, a); break;
+    case 42: launch_dma<CfgW64, 2, 0, true>(s, a); break;
+    case 43: launch_dma<CfgM, 2, 0, true>(s, a); break;
+    case 44: launch_dma<CfgS, 2, 0, true>(s, a); break;
     case 31: launch_dma<CfgL8, 4, 2, true>(s, a); break;
     case 32: launch_dma<CfgL4, 4, 2, true>(s, a); break;
     default: MXQ_CHECK(false, "unknown fc tile configuration " << cfg);
