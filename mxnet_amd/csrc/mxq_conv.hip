@@ -209,6 +209,7 @@ __global__ __launch_bounds__(Cfg::kThreads) void conv_dma_kernel(ConvArgs p) {
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
 
+  const EpiPre pre = epi_prefetch<Cfg>(p.epi, n0, p.O);
   ConvIssuer<Cfg, Cfg::A_CHUNKS> ai;
   RowIssuerBuffer<Cfg, Cfg::B_CHUNKS> bi;
   ai.init(p, m0, wave, lane);
@@ -221,7 +222,7 @@ __global__ __launch_bounds__(Cfg::kThreads) void conv_dma_kernel(ConvArgs p) {
   static_assert(NS * Cfg::STAGE_SLOTS * 16 >=
                     Cfg::BN * 4 + (Cfg::kThreads / 64) * Cfg::TM * (Cfg::TN + 16),
                 "stage ring too small for the epilogue transpose");
-  gemm_epilogue_lds<Cfg>(acc, p.epi, m0, n0, p.M, p.O, static_cast<size_t>(p.O), lds);
+  gemm_epilogue_lds<Cfg>(acc, p.epi, pre, m0, n0, p.M, p.O, static_cast<size_t>(p.O), lds);
   if (blockIdx.x == 0 && threadIdx.x == 0) epilogue_ranges(p.epi);
 }
 

@@ -63,6 +63,7 @@ __global__ __launch_bounds__(Cfg::kThreads) void fc_dma_kernel(FcArgs p) {
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
 
+  const EpiPre pre = epi_prefetch<Cfg>(p.epi, n0, p.N);
   v16i acc[Cfg::MI][Cfg::NI];
   const int KT = (p.K + Cfg::BK - 1) / Cfg::BK;
   if (BUF) {
@@ -83,7 +84,7 @@ __global__ __launch_bounds__(Cfg::kThreads) void fc_dma_kernel(FcArgs p) {
   static_assert(NS * Cfg::STAGE_SLOTS * 16 >=
                     Cfg::BN * 4 + (Cfg::kThreads / 64) * Cfg::TM * (Cfg::TN + 16),
                 "stage ring too small for the epilogue transpose");
-  gemm_epilogue_lds<Cfg>(acc, p.epi, m0, n0, p.M, p.N, static_cast<size_t>(p.ldo), lds);
+  gemm_epilogue_lds<Cfg>(acc, p.epi, pre, m0, n0, p.M, p.N, static_cast<size_t>(p.ldo), lds);
   if (blockIdx.x == 0 && threadIdx.x == 0) epilogue_ranges(p.epi);
 }
 
@@ -160,16 +161,24 @@ void launch_fc(hipStream_t s, const int8_t* data, const int8_t* weight, int M, i
       // stored as well.  Short K (one or two stages) uses the 2-stage ring: less LDS,
       // more resident work-groups to hide the load latency.
       const bool short_k = K <= 128;
-      if (N > 128 && tiles(256, 256) >= cus)
+      if (short_k) {
+        // one or two stages: the kernel is all epilogue and stores, so go for many
+        // resident work-groups (2-stage ring, 64 x 64 wave tiles)
+        if (N > 64 && tiles(256, 128) >= cus) cfg = 41;
+        else if (N <= 64 && tiles(256, 64) >= cus) cfg = 42;
+        else if (tiles(128, 128) >= cus) cfg = 43;
+        else cfg = 44;
+      } else if (N > 128 && tiles(256, 256) >= cus) {
         cfg = glb_ok ? ((epi.out32 != nullptr) ? 16 : 12) : ((epi.out32 != nullptr) ? 32 : 31);
-      else if (N > 64 && tiles(256, 128) >= cus)
-        cfg = short_k ? 41 : 21;
-      else if (N <= 64 && tiles(256, 64) >= cus)
-        cfg = short_k ? 42 : 22;
-      else if (tiles(128, 128) >= cus)
-        cfg = short_k ? 43 : 23;
-      else
-        cfg = short_k ? 44 : 24;
+      } else if (N > 64 && tiles(256, 128) >= cus) {
+        cfg = 21;
+      } else if (N <= 64 && tiles(256, 64) >= cus) {
+        cfg = 22;
+      } else if (tiles(128, 128) >= cus) {
+        cfg = 23;
+      } else {
+        cfg = 24;
+      }
     } else {
       if (tiles(256, 256) >= cus)
         cfg = 1;

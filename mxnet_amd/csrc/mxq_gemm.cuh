@@ -311,22 +311,18 @@ __device__ __forceinline__ void gemm_mainloop(v16i (&acc)[Cfg::MI][Cfg::NI], AF&
 #pragma clang diagnostic ignored "-Winline-asm"
 __device__ __forceinline__ void dma_global(uint32_t lds_byte_addr, uint32_t voffset,
                                            const int8_t* sbase) {
-#ifndef MXQ_LAB_SKIP_DMA
   asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2"
                :
                : "s"(lds_byte_addr), "v"(voffset), "s"(sbase)
                : "memory", "m0");
-#endif
 }
 // Buffer form: lanes whose offset is outside [0, num_records) deliver zeros, which
 // is how image halos, rows past the end of an operand and the K tail are filled.
 __device__ __forceinline__ void dma_buffer(uint32_t lds_byte_addr, uint32_t voffset, v4i rsrc) {
-#ifndef MXQ_LAB_SKIP_DMA
   asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
                :
                : "s"(lds_byte_addr), "v"(voffset), "s"(rsrc)
                : "memory", "m0");
-#endif
 }
 #pragma clang diagnostic pop
 
@@ -485,13 +481,11 @@ __device__ __forceinline__ void gemm_mainloop_dma(v16i (&acc)[Cfg::MI][Cfg::NI],
   }
   // fragment f of a k-step: f < MI -> activation fragment f, else weight fragment f-MI
   auto read_one = [&](int stage, int ks, int f, v4i (&fa)[MI], v4i (&fb)[NI]) {
-#ifndef MXQ_LAB_SKIP_LDSREAD
     const v4i* st = lds + (stage % NS) * Cfg::STAGE_SLOTS;
     if (f < MI)
       fa[f] = st[fa0[ks] + f * 32 * CH];
     else
       fb[f - MI] = st[fb0[ks] + (f - MI) * 32 * CH];
-#endif
   };
   auto read_frags = [&](int stage, int ks, v4i (&fa)[MI], v4i (&fb)[NI]) {
 #pragma unroll
@@ -635,10 +629,28 @@ __device__ __forceinline__ void gemm_epilogue(v16i (&acc)[Cfg::MI][Cfg::NI], con
 // the MFMA, which would make every store instruction touch 32 cache lines with 8
 // bytes each; staged through LDS a store instruction writes whole 64..128-byte row
 // segments.  Falls back to gemm_epilogue when the output is not 16-byte friendly.
+// What the epilogue needs from global memory, fetched before the K loop so that the
+// scalar loads, the divisions and the bias load are hidden behind it: the range
+// scalars and the int32 bias of column n0 + threadIdx.x.
+struct EpiPre {
+  EpiScalars s;
+  int bias32;
+};
+template <class Cfg>
+__device__ __forceinline__ EpiPre epi_prefetch(const Epilogue& e, int n0, int N) {
+  static_assert(Cfg::kThreads >= Cfg::BN, "one thread per tile column");
+  EpiPre p;
+  p.s = epi_scalars(e);
+  const int t = threadIdx.x;
+  p.bias32 = (t < Cfg::BN && n0 + t < N) ? epi_bias32(e, p.s, n0 + t) : 0;
+  return p;
+}
+
 template <class Cfg>
 __device__ __forceinline__ void gemm_epilogue_lds(v16i (&acc)[Cfg::MI][Cfg::NI],
-                                                  const Epilogue& e, int m0, int n0, int M,
-                                                  int N, size_t ldo, v4i* lds_v) {
+                                                  const Epilogue& e, const EpiPre& pre, int m0,
+                                                  int n0, int M, int N, size_t ldo,
+                                                  v4i* lds_v) {
   constexpr int TM = Cfg::TM, TN = Cfg::TN, MI = Cfg::MI, NI = Cfg::NI;
   constexpr int LD = TN + 16;        // staged row pitch in bytes (keeps 16-byte alignment)
   constexpr int LPR = TN / 16;       // lanes per staged row on the way out
@@ -656,11 +668,10 @@ __device__ __forceinline__ void gemm_epilogue_lds(v16i (&acc)[Cfg::MI][Cfg::NI],
   char* lds = reinterpret_cast<char*>(lds_v);
   int* sbias = reinterpret_cast<int*>(lds);
   char* stage = lds + Cfg::BN * 4 + wave * (TM * LD);
-  const EpiScalars s = epi_scalars(e);
+  const EpiScalars s = pre.s;
 
   __syncthreads();  // every wave is done reading operand stages
-  for (int t = tid; t < Cfg::BN; t += Cfg::kThreads)
-    sbias[t] = (n0 + t < N) ? epi_bias32(e, s, n0 + t) : 0;
+  if (tid < Cfg::BN) sbias[tid] = pre.bias32;
   __syncthreads();
 
   const int lrow = lane & 31, lgrp = lane >> 5;
