@@ -17,6 +17,7 @@
 #include "../../include/mxq.h"
 #include "mxq_common.h"
 #include "mxq_gemm.cuh"
+#include "mxq_tiles.h"
 
 namespace mxq {
 
@@ -364,12 +365,26 @@ int mxq_quantized_conv_nhwc(void* stream, const int8_t* data, const int8_t* weig
     auto tiles = [&](int bm, int bn) {
       return static_cast<long>((a.M + bm - 1) / bm) * ((O + bn - 1) / bn);
     };
-    if (O > 128 && tiles(256, 256) >= cus) cfg = 1;
-    else if (O > 64 && tiles(256, 128) >= cus) cfg = 2;
-    else if (O <= 64 && tiles(256, 64) >= cus) cfg = 3;
-    else if (tiles(128, 128) >= cus) cfg = 4;
-    else cfg = 5;
-    if (dma_ok) cfg += 10;
+    if (dma_ok) {
+      switch (choose_tile(a.M, O, a.K, cus)) {
+        case Tile::kL8: cfg = 11; break;
+        case Tile::kW128x2: cfg = 22; break;
+        case Tile::kM128x2: cfg = 24; break;
+        case Tile::kM128x4: cfg = 14; break;
+        case Tile::kS64x2: cfg = 25; break;
+        case Tile::kS64x4: cfg = 15; break;
+      }
+    } else if (O > 128 && tiles(256, 256) >= cus) {
+      cfg = 1;
+    } else if (O > 64 && tiles(256, 128) >= cus) {
+      cfg = 2;
+    } else if (O <= 64 && tiles(256, 64) >= cus) {
+      cfg = 3;
+    } else if (tiles(128, 128) >= cus) {
+      cfg = 4;
+    } else {
+      cfg = 5;
+    }
   }
   if (cfg > 10) MXQ_CHECK(dma_ok, "shape does not qualify for the direct-to-LDS conv kernels");
   switch (cfg) {
@@ -384,6 +399,10 @@ int mxq_quantized_conv_nhwc(void* stream, const int8_t* data, const int8_t* weig
     case 14: launch_dma<CfgM, 4, 2>(s, a); break;
     case 15: launch_dma<CfgS, 4, 2>(s, a); break;
     case 16: launch_dma<CfgL4, 4, 2>(s, a); break;
+    case 22: launch_dma<CfgW128, 2, 0>(s, a); break;
+    case 23: launch_dma<CfgW64, 2, 0>(s, a); break;
+    case 24: launch_dma<CfgM, 2, 0>(s, a); break;
+    case 25: launch_dma<CfgS, 2, 0>(s, a); break;
     default: MXQ_CHECK(false, "unknown conv tile configuration " << cfg);
   }
   MXQ_API_END();

@@ -12,6 +12,7 @@
 #include "../../include/mxq.h"
 #include "mxq_common.h"
 #include "mxq_gemm.cuh"
+#include "mxq_tiles.h"
 
 namespace mxq {
 
@@ -156,28 +157,17 @@ void launch_fc(hipStream_t s, const int8_t* data, const int8_t* weight, int M, i
       return static_cast<long>((M + bm - 1) / bm) * ((N + bn - 1) / bn);
     };
     if (buf_ok) {
-      // tile width follows N; the tallest tile that still gives every CU work.  8 waves
-      // when only the int8 output is written, 4 waves (128 x 128 per wave) when int32 is
-      // stored as well.  Short K (one or two stages) uses the 2-stage ring: less LDS,
-      // more resident work-groups to hide the load latency.
-      const bool short_k = K <= 128;
-      if (short_k) {
-        // one or two stages: the kernel is all epilogue and stores, so go for many
-        // resident work-groups (2-stage ring, 64 x 64 wave tiles)
-        if (N > 64 && tiles(256, 128) >= cus) cfg = 41;
-        else if (N <= 64 && tiles(256, 64) >= cus) cfg = 42;
-        else if (tiles(128, 128) >= cus) cfg = 43;
-        else cfg = 44;
-      } else if (N > 128 && tiles(256, 256) >= cus) {
-        cfg = glb_ok ? ((epi.out32 != nullptr) ? 16 : 12) : ((epi.out32 != nullptr) ? 32 : 31);
-      } else if (N > 64 && tiles(256, 128) >= cus) {
-        cfg = 21;
-      } else if (N <= 64 && tiles(256, 64) >= cus) {
-        cfg = 22;
-      } else if (tiles(128, 128) >= cus) {
-        cfg = 23;
-      } else {
-        cfg = 24;
+      // the 256 x 256 tile runs 8 waves when only int8 is written and 4 waves (128 x 128
+      // wave tiles) when int32 is stored as well
+      switch (choose_tile(M, N, K, cus)) {
+        case Tile::kL8:
+          cfg = glb_ok ? ((epi.out32 != nullptr) ? 16 : 12) : ((epi.out32 != nullptr) ? 32 : 31);
+          break;
+        case Tile::kW128x2: cfg = 41; break;
+        case Tile::kM128x2: cfg = 43; break;
+        case Tile::kM128x4: cfg = 23; break;
+        case Tile::kS64x2: cfg = 44; break;
+        case Tile::kS64x4: cfg = 24; break;
       }
     } else {
       if (tiles(256, 256) >= cus)
