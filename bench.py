@@ -411,6 +411,60 @@ class BertChainWorkload(GraphWorkload):
         self.capture(torch, body)
 
 
+def mfma_context(torch, S):
+    """Context for the MFMA roofline fraction, measured in the same process: the
+    register-only MFMA probe (what the matrix pipes sustain with no data movement at
+    all, zero vs random operand bytes) and the vendor int8 GEMM (hipBLASLt through
+    torch._int_mm, int32 output, no bias, no requantize) on the same operand shapes."""
+    out = {}
+    path = os.path.join(ROOT, "mxnet_amd", "libmxq_probe.so")
+    if os.path.exists(path):
+        probe = ctypes.CDLL(path)
+        probe.mxq_probe_mfma_i8.restype = ctypes.c_double
+        probe.mxq_probe_mfma_i8.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_int,
+                                            ctypes.c_int, ctypes.c_void_p]
+        cus = torch.cuda.get_device_properties(0).multi_processor_count
+        blocks = 2 * cus  # 2 waves per SIMD, as the 256 x 256 FC tile runs
+        sink = torch.zeros(blocks * 256, dtype=torch.int32, device="cuda")
+        st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+        for zero, key in ((1, "zero_operands"), (0, "random_operands")):
+            best = None
+            for rep in range(4):
+                e0 = torch.cuda.Event(enable_timing=True)
+                e1 = torch.cuda.Event(enable_timing=True)
+                e0.record()
+                ops = probe.mxq_probe_mfma_i8(st, blocks, 2000, zero, sink.data_ptr())
+                e1.record()
+                torch.cuda.synchronize()
+                if ops < 0:
+                    raise RuntimeError("MFMA probe launch failed")
+                t = e0.elapsed_time(e1) / 1e3
+                if rep > 0 and (best is None or t < best):
+                    best = t
+            out["mfma_probe_%s_TOPS" % key] = round(ops / best / 1e12, 1)
+    try:
+        g = torch.Generator(device="cuda").manual_seed(1)
+        a = torch.randint(-127, 128, (S, S), device="cuda", dtype=torch.int8, generator=g)
+        b = (torch.randn((S, S), device="cuda", generator=g) * 24).clamp(-127, 127).round() \
+            .to(torch.int8)
+        bt = b.t()
+        for _ in range(5):
+            torch._int_mm(a, bt)
+        e0 = torch.cuda.Event(enable_timing=True)
+        e1 = torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        e0.record()
+        for _ in range(50):
+            torch._int_mm(a, bt)
+        e1.record()
+        torch.cuda.synchronize()
+        out["vendor_gemm_int32_out_TOPS"] = round(2.0 * S ** 3 * 50 / (e0.elapsed_time(e1) / 1e3)
+                                                  / 1e12, 1)
+    except Exception as e:  # informational only
+        out["vendor_gemm_int32_out_TOPS"] = "unavailable: %s" % e
+    return out
+
+
 def make_workload(name, torch, capi, lib):
     if name == "resnet50_convs":
         return ConvStackWorkload(torch, capi, lib)
@@ -491,6 +545,9 @@ def main():
         "device": torch.cuda.get_device_name(0),
         "roofline": roofline_of(wl, ev / args.steps, args.workload),
     }
+
+    if isinstance(wl, FcWorkload):
+        line["roofline"]["context"] = mfma_context(torch, wl.S)
 
     if not args.no_cast_ops:
         rows = []

@@ -54,6 +54,27 @@ def build(verbose=False):
     return LIB
 
 
+PROBE_LIB = os.path.join(HERE, "libmxq_probe.so")
+
+
+def build_probe(verbose=False):
+    """libmxq_probe.so: the register-only MFMA rate probe bench.py reports next to the
+    FC figures.  Kept out of libmxq_hip.so: it is not an operator."""
+    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+    cmd = [hipcc] + HIPCC_FLAGS + ["-shared", os.path.join(CSRC, "mxq_probe.hip"), "-o",
+                                   PROBE_LIB]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    out = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT)
+    text = "\n".join(l for l in out.stdout.decode().splitlines()
+                     if "packed-fp32-ops" not in l and l.strip())
+    if text:
+        print(text)
+    if out.returncode != 0:
+        raise RuntimeError("hipcc failed: mxq_probe.hip")
+    return PROBE_LIB
+
+
 OPS_LIB = os.path.join(HERE, "libmxq_ops.so")
 HOST_SOURCES = ["mxq_registry.cc", "mxq_quantization_ops.cc", "mxq_harness.cc"]
 
@@ -73,7 +94,6 @@ def build_ops(verbose=False):
 
 
 if __name__ == "__main__":
-    build(verbose="-v" in sys.argv)
-    print(build_ops(verbose="-v" in sys.argv))
-    sys.exit(0)
     print(build(verbose="-v" in sys.argv))
+    print(build_ops(verbose="-v" in sys.argv))
+    print(build_probe(verbose="-v" in sys.argv))
