@@ -47,7 +47,7 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="fc4096",
                     choices=["fc4096", "fc8192", "quantize", "quantize_uncal", "quantize_uint8",
-                             "requantize", "requantize_uncal", "dequantize", "copy",
+                             "requantize", "requantize_uncal", "dequantize", "copy", "maxpool", "avgpool",
                              "resnet50_convs", "bert_fc_chain"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-cast-ops", action="store_true")
@@ -248,6 +248,52 @@ class CastWorkload:
         return {"value": gbs, "unit": "GB/s", "cores": oracle.num_threads(), "kind": "port",
                 "sample": "oracle (OpenMP) on the first %d elements, %d repetitions, %.1f s"
                           % (n, reps, dt)}
+
+
+class PoolWorkload:
+    """_contrib_quantized_pooling on NCHW int8, buffers rotated past the Infinity Cache.
+    `maxpool`: the ResNet stem pool (3x3 / stride 2 / pad 1 on 112 x 112 x 64) at batch 256;
+    `avgpool`: the ResNet global average pool (7 x 7 x 2048) at batch 4096.  Algorithmic
+    bytes: input read once + output written once (1 B per element each)."""
+    NBUF = 3
+
+    def __init__(self, kind, torch, lib):
+        self.kind, self.torch, self.lib = kind, torch, lib
+        if kind == "maxpool":
+            self.shape, self.k, self.s, self.p, self.pool = (256, 64, 112, 112), 3, 2, 1, 0
+        else:
+            self.shape, self.k, self.s, self.p, self.pool = (4096, 2048, 7, 7), 7, 1, 0, 1
+        N, C, H, W = self.shape
+        self.OH = (H + 2 * self.p - self.k) // self.s + 1
+        g = torch.Generator(device="cuda").manual_seed(2)
+        self.src = [torch.randint(-127, 128, self.shape, device="cuda", generator=g,
+                                  dtype=torch.int8) for _ in range(self.NBUF)]
+        self.dst = [torch.empty((N, C, self.OH, self.OH), dtype=torch.int8, device="cuda")
+                    for _ in range(self.NBUF)]
+        self.sc = [torch.tensor([v], device="cuda") for v in (-1.0, 1.0, 0.0, 0.0)]
+        self.bytes = float(N * C * (H * W + self.OH * self.OH))
+        self.bound = "hbm"
+        self.kernel = "pool_lds_kernel"
+        self.name = "quantized_pooling %s %dx%d/%d on int8 NCHW %s" % (
+            "max" if self.pool == 0 else "avg", self.k, self.k, self.s, "x".join(map(str, self.shape)))
+        self.i = 0
+        self.P = lambda t: ctypes.c_void_p(t.data_ptr())
+
+    def step(self):
+        P = self.P
+        k = self.i % self.NBUF
+        self.i += 1
+        N, C, H, W = self.shape
+        st = ctypes.c_void_p(self.torch.cuda.current_stream().cuda_stream)
+        rc = self.lib.mxq_quantized_pooling_nchw(st, P(self.src[k]), 5, N, C, H, W, self.k, self.k,
+                                                 self.s, self.s, self.p, self.p, self.OH, self.OH,
+                                                 self.pool, 1, P(self.sc[0]), P(self.sc[1]),
+                                                 P(self.dst[k]), P(self.sc[2]), P(self.sc[3]))
+        if rc != 0:
+            raise RuntimeError(self.lib.mxq_last_error().decode())
+
+    def value(self, sec_per_step):
+        return self.bytes / sec_per_step / 1e9, "GB/s"
 
 
 class CopyWorkload:
@@ -472,6 +518,8 @@ def make_workload(name, torch, capi, lib):
         return BertChainWorkload(torch, capi, lib)
     if name == "copy":
         return CopyWorkload(torch)
+    if name in ("maxpool", "avgpool"):
+        return PoolWorkload(name, torch, lib)
     if name == "fc4096":
         return FcWorkload(4096, torch, capi, lib)
     if name == "fc8192":
@@ -552,8 +600,8 @@ def main():
     if not args.no_cast_ops:
         rows = []
         for kind in ["quantize", "quantize_uint8", "quantize_uncal", "requantize",
-                     "requantize_uncal", "dequantize", "fc8192", "resnet50_convs",
-                     "bert_fc_chain"]:
+                     "requantize_uncal", "dequantize", "maxpool", "avgpool", "fc8192",
+                     "resnet50_convs", "bert_fc_chain"]:
             if kind == args.workload:
                 continue
             w2 = make_workload(kind, torch, capi, lib)
@@ -566,7 +614,8 @@ def main():
             torch.cuda.empty_cache()
         line["other_kernels"] = rows
 
-    if not args.no_cpu_baseline and not isinstance(wl, (GraphWorkload, CopyWorkload)):
+    if not args.no_cpu_baseline and not isinstance(wl, (GraphWorkload, CopyWorkload,
+                                                       PoolWorkload)):
         import oracle
         line["cpu_baseline"] = wl.cpu_baseline(oracle)
         try:

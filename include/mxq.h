@@ -91,6 +91,34 @@ int mxq_dequantize(void* stream, const void* in, int in_type, const float* imin,
 int mxq_quantized_relu(void* stream, const int8_t* in, const float* imin, const float* imax,
                        int8_t* out, float* omin, float* omax, size_t n);
 
+/* ---- _contrib_quantized_pooling ---------------------------------------------
+ * Replaces QuantizedCuDNNPoolingOp::Forward
+ * (src/operator/quantization/quantized_pooling.cu:33-128): cudnnPoolingForward on
+ * the NCHW int8 tensor plus the two range copies.  OH / OW are the extents
+ * QuantizedPoolingShape computed (quantized_pooling.cc:82-121; global pooling is
+ * kernel = (H, W), stride 1, OH = OW = 1).  Windows and the divisor of avg follow
+ * the reference's own pooling loops (src/operator/nn/pool.h:476-522):
+ * count_include_pad != 0 is cuDNN's COUNT_INCLUDE_PADDING, the mode the reference
+ * selects.  max ignores padding; avg returns nearest-even(sum / divisor): that
+ * rounding lives inside cuDNN / oneDNN in the reference and is not pinned by its
+ * sources (its test accepts +-2).  in_type MXQ_INT8 or MXQ_UINT8 (the reference's
+ * GPU build takes int8 only). */
+#define MXQ_POOL_MAX 0
+#define MXQ_POOL_AVG 1
+int mxq_quantized_pooling_nchw(void* stream, const void* in, int in_type, int N, int C, int H,
+                               int W, int kernel_h, int kernel_w, int stride_h, int stride_w,
+                               int pad_h, int pad_w, int OH, int OW, int pool_type,
+                               int count_include_pad, const float* imin, const float* imax,
+                               void* out, float* omin, float* omax);
+
+/* ---- _contrib_quantized_flatten ----------------------------------------------
+ * Replaces QuantizedFlattenCompute (src/operator/quantization/quantized_flatten-inl.h:39-94;
+ * registered for cpu only in the reference, quantized_flatten.cc:35): copies n_bytes
+ * of int8/uint8 data and the two range scalars; in == out (the operator's in-place
+ * option, quantized_flatten.cc:52-56) copies nothing. */
+int mxq_quantized_flatten(void* stream, const void* in, const float* imin, const float* imax,
+                          void* out, float* omin, float* omax, size_t n_bytes);
+
 /* ---- _contrib_quantized_fully_connected ----------------------------------
  * Replaces QuantizedFullyConnectedForwardGPU
  * (src/operator/quantization/quantized_fully_connected.cu:58-138): cublasGemmEx

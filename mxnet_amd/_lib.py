@@ -38,6 +38,8 @@ SIGNATURES = {
     "mxq_requantize": (_i, [_p, _p, _p, _p, _p, _p, _p, _sz, _i, _f, _f, _p, _sz]),
     "mxq_dequantize": (_i, [_p, _p, _i, _p, _p, _p, _sz]),
     "mxq_quantized_relu": (_i, [_p, _p, _p, _p, _p, _p, _p, _sz]),
+    "mxq_quantized_pooling_nchw": (_i, [_p, _p, _i] + [_i] * 12 + [_i, _i, _p, _p, _p, _p, _p]),
+    "mxq_quantized_flatten": (_i, [_p, _p, _p, _p, _p, _p, _p, _sz]),
     "mxq_quantized_fc": (_i, [_p, _p, _p, _p, _i, _i, _i] + [_p] * 6 + [_p, _p, _p, _p, _p, _p,
                               _i, _f, _f]),
     "mxq_quantized_conv_nhwc": (_i, [_p, _p, _p, _p] + [_i] * 13 + [_p] * 6 +

@@ -50,3 +50,19 @@ def quantized_conv(data, weight, bias=None, min_data=None, max_data=None, min_we
 
 def quantized_act(data, min_data, max_data, act_type="relu"):
     return invoke("_contrib_quantized_act", data, min_data, max_data, act_type=act_type)
+
+
+def quantized_pooling(data, min_data, max_data, kernel=None, pool_type="max", global_pool=False,
+                      cudnn_off=False, pooling_convention="valid", stride=None, pad=None,
+                      count_include_pad=None, layout=None):
+    attrs = {"pool_type": pool_type, "global_pool": global_pool, "cudnn_off": cudnn_off,
+             "pooling_convention": pooling_convention}
+    for key, value in (("kernel", kernel), ("stride", stride), ("pad", pad),
+                       ("count_include_pad", count_include_pad), ("layout", layout)):
+        if value is not None:
+            attrs[key] = value
+    return invoke("_contrib_quantized_pooling", data, min_data, max_data, **attrs)
+
+
+def quantized_flatten(data, min_data, max_data):
+    return invoke("_contrib_quantized_flatten", data, min_data, max_data)

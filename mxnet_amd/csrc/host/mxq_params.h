@@ -8,6 +8,8 @@
 //   ConvolutionParam       src/operator/nn/convolution-inl.h:56-112 (+ the defaults
 //                          ConvolutionParamParser fills, src/operator/nn/convolution.cc:366-416)
 //   ActivationParam        src/operator/nn/activation-inl.h (act_type only)
+//   PoolingParam           src/operator/nn/pooling-inl.h:45-120 (+ PoolingParamParser,
+//                          src/operator/nn/pooling.cc:35-64)
 // Same field names, defaults, enum strings and error behaviour (unknown keys are
 // errors unless they look like __hidden__ keys).
 #ifndef MXQ_PARAMS_H_
@@ -359,6 +361,102 @@ struct ActivationParam {
   }
 };
 
+
+namespace pool_enum {
+enum PoolingOpType { kMaxPooling, kAvgPooling, kSumPooling, kLpPooling };
+enum PoolingOpPadConventionType { kValid, kFull, kSame };
+}  // namespace pool_enum
+
+struct PoolingParam {
+  TShape kernel, stride, pad;
+  int pool_type = pool_enum::kMaxPooling;
+  int pooling_convention = pool_enum::kValid;
+  bool global_pool = false;
+  bool cudnn_off = false;
+  dmlc::optional<int> p_value;
+  dmlc::optional<bool> count_include_pad;
+  dmlc::optional<int> layout;
+  bool has_output_size = false;  // adaptive pooling: recognised, not supported here
+  void Init(const param_detail::Dict& d) {
+    using namespace param_detail;
+    check_unknown(d, {"kernel", "pool_type", "global_pool", "cudnn_off", "pooling_convention",
+                      "stride", "pad", "p_value", "count_include_pad", "layout", "output_size"},
+                  "PoolingParam");
+    kernel = get_shape(d, "kernel", true);
+    stride = get_shape(d, "stride", true);
+    pad = get_shape(d, "pad", true);
+    for (int i = 0; i < kernel.ndim(); ++i)
+      if (kernel[i] == 0) bad_value("kernel", d.at("kernel"), "non-zero extents");
+    for (int i = 0; i < stride.ndim(); ++i)
+      if (stride[i] == 0) bad_value("stride", d.at("stride"), "non-zero extents");
+    pool_type = get_enum(d, "pool_type",
+                         {{"max", pool_enum::kMaxPooling},
+                          {"avg", pool_enum::kAvgPooling},
+                          {"sum", pool_enum::kSumPooling},
+                          {"lp", pool_enum::kLpPooling}},
+                         true, pool_enum::kMaxPooling);
+    pooling_convention = get_enum(d, "pooling_convention",
+                                  {{"full", pool_enum::kFull},
+                                   {"valid", pool_enum::kValid},
+                                   {"same", pool_enum::kSame}},
+                                  true, pool_enum::kValid);
+    global_pool = get_bool(d, "global_pool", false);
+    cudnn_off = get_bool(d, "cudnn_off", false);
+    auto it = d.find("p_value");
+    if (it != d.end() && trim(it->second) != "None")
+      p_value = dmlc::optional<int>(static_cast<int>(get_int(d, "p_value", false, 0, false, 0)));
+    it = d.find("count_include_pad");
+    if (it != d.end() && trim(it->second) != "None")
+      count_include_pad = dmlc::optional<bool>(get_bool(d, "count_include_pad", true));
+    it = d.find("layout");
+    if (it != d.end() && trim(it->second) != "None")
+      layout = dmlc::optional<int>(get_enum(d, "layout",
+                                            {{"NCW", mshadow::kNCW},
+                                             {"NCHW", mshadow::kNCHW},
+                                             {"NCDHW", mshadow::kNCDHW},
+                                             {"NWC", mshadow::kNWC},
+                                             {"NHWC", mshadow::kNHWC},
+                                             {"NDHWC", mshadow::kNDHWC}},
+                                            true, 0));
+    it = d.find("output_size");
+    has_output_size = it != d.end() && trim(it->second) != "None";
+  }
+  // pooling-inl.h:122-140
+  int GetLayout(int input_dim) const {
+    if (layout.has_value()) return layout.value();
+    switch (input_dim) {
+      case 3: return mshadow::kNCW;
+      case 4: return mshadow::kNCHW;
+      case 5: return mshadow::kNCDHW;
+      default: LOG_FATAL << "Unsupported input data dimension " << input_dim;
+    }
+    return mshadow::kNCHW;
+  }
+  static std::vector<nnvm::ParamFieldInfo> __FIELDS__() {
+    return {{"kernel", "Shape(tuple), optional, default=[]", "Pooling kernel size: (y, x) or (d, y, x)"},
+            {"pool_type", "{'avg', 'lp', 'max', 'sum'},optional, default='max'",
+             "Pooling type to be applied."},
+            {"global_pool", "boolean, optional, default=0",
+             "Ignore kernel size, do global pooling based on current input feature map. "},
+            {"cudnn_off", "boolean, optional, default=0",
+             "Turn off cudnn pooling and use MXNet pooling operator. "},
+            {"pooling_convention", "{'full', 'same', 'valid'},optional, default='valid'",
+             "Pooling convention to be applied."},
+            {"stride", "Shape(tuple), optional, default=[]",
+             "Stride: for pooling (y, x) or (d, y, x). Defaults to 1 for each dimension."},
+            {"pad", "Shape(tuple), optional, default=[]",
+             "Pad for pooling: (y, x) or (d, y, x). Defaults to no padding."},
+            {"p_value", "int or None, optional, default='None'", "Value of p for Lp pooling."},
+            {"count_include_pad", "boolean or None, optional, default=None",
+             "Only used for AvgPool, specify whether to count padding elements for average"
+             "calculation. Defaults to true."},
+            {"layout", "{None, 'NCDHW', 'NCHW', 'NCW', 'NDHWC', 'NHWC', 'NWC'},optional, "
+                       "default='None'",
+             "Set layout for input and output."},
+            {"output_size", "Shape(tuple) or None, optional", "Only used for Adaptive Pooling."}};
+  }
+};
+
 // src/operator/operator_common.h:478-495
 template <typename PType>
 inline void ParamParser(nnvm::NodeAttrs* attrs) {
@@ -398,6 +496,26 @@ inline void ConvolutionParamParser(nnvm::NodeAttrs* attrs) {
       << "Padding must have the same number of dimensions with kernel_size,"
       << "but kernel_size is set to " << param_.kernel << " while padding is " << param_.pad;
   attrs->parsed = std::move(param_);
+}
+
+// src/operator/nn/pooling.cc:35-64
+inline void PoolingParamParser(nnvm::NodeAttrs* attrs) {
+  ParamParser<PoolingParam>(attrs);
+  PoolingParam param = nnvm::get<PoolingParam>(attrs->parsed);
+  if (param.kernel.ndim() > 0) param.layout = param.GetLayout(param.kernel.ndim() + 2);
+  if (param.kernel.ndim() == 1) {
+    if (param.stride.ndim() == 0) param.stride = TShape(std::vector<index_t>{1});
+    if (param.pad.ndim() == 0) param.pad = TShape(std::vector<index_t>{0});
+  } else if (param.kernel.ndim() == 2) {
+    if (param.stride.ndim() == 0) param.stride = TShape(std::vector<index_t>{1, 1});
+    if (param.pad.ndim() == 0) param.pad = TShape(std::vector<index_t>{0, 0});
+  } else {
+    if (!param.global_pool && !param.has_output_size)
+      CHECK_EQ(param.kernel.ndim(), 3) << param.kernel.ndim() << "D pooling not supported";
+    if (param.stride.ndim() == 0) param.stride = TShape(std::vector<index_t>{1, 1, 1});
+    if (param.pad.ndim() == 0) param.pad = TShape(std::vector<index_t>{0, 0, 0});
+  }
+  attrs->parsed = std::move(param);
 }
 
 }  // namespace op

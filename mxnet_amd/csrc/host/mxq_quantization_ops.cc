@@ -13,6 +13,8 @@
 //   _contrib_quantized_fully_connected   quantized_fully_connected.cc:317-382, .cu:141-143
 //   _contrib_quantized_conv              quantized_conv.cc:176-237, .cu:293-294
 //   _contrib_quantized_act               quantized_activation.cc:84-120
+//   _contrib_quantized_pooling           quantized_pooling.cc:159-209, quantized_pooling.cu:126-127
+//   _contrib_quantized_flatten           quantized_flatten.cc:30-63
 // (all under src/operator/quantization/).  Inside MXNet only the "<gpu>" attributes
 // of this file would be compiled (the CPU .cc files already register the rest).
 #include <algorithm>
@@ -283,6 +285,100 @@ static bool QuantizedActivationType(const NodeAttrs& attrs, std::vector<int>* in
   return true;
 }
 
+// quantized_pooling.cc:32-133.  The reference's GPU build accepts 4-D NCHW with a 2-D
+// kernel only (:53-58); so does this one.
+static bool QuantizedPoolingShape(const NodeAttrs& attrs, ShapeVector* in, ShapeVector* out) {
+  const auto& param = nnvm::get<PoolingParam>(attrs.parsed);
+  CHECK_EQ(in->size(), 3U);
+  if (!shape_is_known((*in)[0])) return false;
+  const TShape& dshape = (*in)[0];
+  const int data_ndims = dshape.ndim();
+  const int kernel_ndims = param.kernel.ndim();
+  CHECK_EQ(data_ndims, 4) << "quantized_pooling: Input data should be 4D in "
+                          << "(batch, channel, y, x)";
+  const int layout = param.GetLayout(data_ndims);
+  CHECK_EQ(layout, static_cast<int>(mshadow::kNCHW))
+      << "QuantizedPoolingOp only supports NCHW layout for now, saw " << layout;
+  CHECK(param.global_pool || kernel_ndims == 2)
+      << "QuantizedPoolingOp only supports 2D pooling for now";
+  CHECK(!param.has_output_size) << "QuantizedPoolingOp does not support adaptive pooling";
+  const int N = 0, C = 1, H = 2, W = 3;
+  TShape oshape(data_ndims, -1);
+  oshape[N] = dshape[N];
+  oshape[C] = dshape[C];
+  if (param.global_pool) {
+    oshape[H] = 1;
+    oshape[W] = 1;
+  } else {
+    for (int idx = 0; idx < 2; ++idx) {
+      const int dim = H + idx;
+      CHECK(param.kernel[idx] <= dshape[dim] + 2 * param.pad[idx])
+          << "kernel size (" << param.kernel[idx] << ") exceeds input (" << dshape[dim]
+          << " padded to " << (dshape[dim] + 2 * param.pad[idx]) << ")";
+      const index_t span = dshape[dim] + 2 * param.pad[idx] - param.kernel[idx];
+      if (param.pooling_convention == pool_enum::kValid) {
+        oshape[dim] = 1 + span / param.stride[idx];
+      } else {
+        // the reference evaluates the ceiling in binary32 (:95-101); "same" takes this
+        // branch as well (:108-120)
+        oshape[dim] = 1 + static_cast<int>(std::ceil(static_cast<float>(span) /
+                                                     static_cast<float>(param.stride[idx])));
+      }
+    }
+  }
+  SHAPE_ASSIGN_CHECK(*in, 1, kScalarShape);
+  SHAPE_ASSIGN_CHECK(*in, 2, kScalarShape);
+  out->clear();
+  out->push_back(oshape);
+  out->push_back(kScalarShape);
+  out->push_back(kScalarShape);
+  return true;
+}
+
+// quantized_pooling.cc:135-157: the output takes the input's type (int8 or uint8).
+static bool QuantizedPoolingType(const NodeAttrs& attrs, std::vector<int>* in,
+                                 std::vector<int>* out) {
+  const auto& param = nnvm::get<PoolingParam>(attrs.parsed);
+  CHECK_EQ(in->size(), 3U);
+  CHECK_EQ(out->size(), 3U);
+  if (param.pool_type == pool_enum::kMaxPooling || param.pool_type == pool_enum::kAvgPooling) {
+    TYPE_ASSIGN_CHECK(*out, 0, (*in)[0]);
+  } else {
+    LOG_FATAL << "QuantizedPoolingOp only supports pool_type=max/avg for now";
+  }
+  TYPE_ASSIGN_CHECK(*in, 1, mshadow::kFloat32);
+  TYPE_ASSIGN_CHECK(*in, 2, mshadow::kFloat32);
+  TYPE_ASSIGN_CHECK(*out, 1, mshadow::kFloat32);
+  TYPE_ASSIGN_CHECK(*out, 2, mshadow::kFloat32);
+  return true;
+}
+
+// quantized_flatten-inl.h:96-131
+static bool QuantizedFlattenShape(const NodeAttrs&, ShapeVector* in, ShapeVector* out) {
+  CHECK_EQ(in->size(), 3U);
+  CHECK_EQ(out->size(), 3U);
+  const TShape& dshape = (*in)[0];
+  if (!shape_is_known(dshape)) return false;
+  index_t target_dim = 1;
+  for (int i = 1; i < dshape.ndim(); ++i) target_dim *= dshape[i];
+  SHAPE_ASSIGN_CHECK(*in, 1, kScalarShape);
+  SHAPE_ASSIGN_CHECK(*in, 2, kScalarShape);
+  SHAPE_ASSIGN_CHECK(*out, 0, TShape(std::vector<index_t>{dshape[0], target_dim}));
+  SHAPE_ASSIGN_CHECK(*out, 1, kScalarShape);
+  SHAPE_ASSIGN_CHECK(*out, 2, kScalarShape);
+  return true;
+}
+static bool QuantizedFlattenType(const NodeAttrs&, std::vector<int>* in, std::vector<int>* out) {
+  CHECK_EQ(in->size(), 3U);
+  CHECK_EQ(out->size(), 3U);
+  TYPE_ASSIGN_CHECK(*in, 1, mshadow::kFloat32);
+  TYPE_ASSIGN_CHECK(*in, 2, mshadow::kFloat32);
+  TYPE_ASSIGN_CHECK(*out, 0, (*in)[0]);
+  TYPE_ASSIGN_CHECK(*out, 1, mshadow::kFloat32);
+  TYPE_ASSIGN_CHECK(*out, 2, mshadow::kFloat32);
+  return (*in)[0] != -1;
+}
+
 static bool DefaultStorageType(const NodeAttrs&, const int, DispatchMode* dispatch_mode,
                                std::vector<int>* in, std::vector<int>* out) {
   *dispatch_mode = DispatchMode::kFCompute;
@@ -500,6 +596,60 @@ static void QuantizedActivationForwardGPU(const NodeAttrs& attrs, const OpContex
 }
 
 // Temp-space bytes the harness (or a framework without lazy resources) must provide.
+// _contrib_quantized_pooling (quantized_pooling.cu:101-124)
+static void QuantizedPoolingForwardGPU(const NodeAttrs& attrs, const OpContext& ctx,
+                                       const std::vector<TBlob>& inputs,
+                                       const std::vector<OpReqType>&,
+                                       const std::vector<TBlob>& outputs) {
+  const auto& param = nnvm::get<PoolingParam>(attrs.parsed);
+  CHECK_EQ(inputs.size(), 3U);
+  CHECK_EQ(outputs.size(), 3U);
+  CHECK(param.global_pool || param.kernel.ndim() == 2)
+      << "QuantizedPoolingForward<gpu> only supports 2D convolution for now";
+  CHECK(param.pool_type == pool_enum::kMaxPooling || param.pool_type == pool_enum::kAvgPooling)
+      << "QuantizedCuDNNPoolingOp only supports pool_type=max/avg";
+  const TShape& d = inputs[0].shape_;
+  const TShape& o = outputs[0].shape_;
+  CHECK_EQ(d.ndim(), 4);
+  CHECK_EQ(o.ndim(), 4);
+  CHECK(inputs[0].type_flag_ == mshadow::kInt8 || inputs[0].type_flag_ == mshadow::kUint8)
+      << "quantized_pooling takes int8 or uint8 data";
+  CHECK_EQ(outputs[0].type_flag_, inputs[0].type_flag_);
+  const bool g = param.global_pool;
+  const int kh = g ? static_cast<int>(d[2]) : static_cast<int>(param.kernel[0]);
+  const int kw = g ? static_cast<int>(d[3]) : static_cast<int>(param.kernel[1]);
+  const int sh = g ? 1 : static_cast<int>(param.stride[0]);
+  const int sw = g ? 1 : static_cast<int>(param.stride[1]);
+  const int ph = g ? 0 : static_cast<int>(param.pad[0]);
+  const int pw = g ? 0 : static_cast<int>(param.pad[1]);
+  const bool include_pad = !param.count_include_pad.has_value() || param.count_include_pad.value();
+  MXQ_CALL(mxq_quantized_pooling_nchw(
+      raw_stream(ctx), inputs[0].dptr_, inputs[0].type_flag_, static_cast<int>(d[0]),
+      static_cast<int>(d[1]), static_cast<int>(d[2]), static_cast<int>(d[3]), kh, kw, sh, sw, ph,
+      pw, static_cast<int>(o[2]), static_cast<int>(o[3]),
+      param.pool_type == pool_enum::kAvgPooling ? MXQ_POOL_AVG : MXQ_POOL_MAX, include_pad,
+      inputs[1].dptr<float>(), inputs[2].dptr<float>(), outputs[0].dptr_,
+      outputs[1].dptr<float>(), outputs[2].dptr<float>()));
+}
+
+// _contrib_quantized_flatten (quantized_flatten-inl.h:55-94): nothing to do when the
+// engine runs it in place.
+static void QuantizedFlattenComputeGPU(const NodeAttrs&, const OpContext& ctx,
+                                       const std::vector<TBlob>& inputs,
+                                       const std::vector<OpReqType>& req,
+                                       const std::vector<TBlob>& outputs) {
+  CHECK_EQ(inputs.size(), 3U);
+  CHECK_EQ(outputs.size(), 3U);
+  CHECK_EQ(req.size(), 3U);
+  if (req[0] == kWriteInplace && req[1] == kWriteInplace && req[2] == kWriteInplace) return;
+  CHECK(inputs[0].type_flag_ == mshadow::kInt8 || inputs[0].type_flag_ == mshadow::kUint8)
+      << "quantized_flatten op only supports int8 and uint8 as input and output type";
+  MXQ_CALL(mxq_quantized_flatten(raw_stream(ctx), inputs[0].dptr_, inputs[1].dptr<float>(),
+                                 inputs[2].dptr<float>(), outputs[0].dptr_,
+                                 outputs[1].dptr<float>(), outputs[2].dptr<float>(),
+                                 outputs[0].Size()));
+}
+
 size_t MXQTempSpaceBytes(const NodeAttrs& attrs, const ShapeVector& in, const ShapeVector& out) {
   const std::string& name = attrs.op->name;
   if (name == "_contrib_quantize_v2") return mxq_quantize_v2_workspace(in[0].Size());
@@ -731,6 +881,66 @@ NNVM_REGISTER_OP(_contrib_quantized_act)
     .add_argument("min_data", "NDArray-or-Symbol", "Minimum value of data.")
     .add_argument("max_data", "NDArray-or-Symbol", "Maximum value of data.")
     .add_arguments(ActivationParam::__FIELDS__());
+
+NNVM_REGISTER_OP(_contrib_quantized_pooling)
+    .add_alias("_npx_quantized_pooling")
+    .describe("Pooling operator for input and output data type of int8. Only `max` and `avg`.")
+    .set_num_inputs(3)
+    .set_num_outputs(3)
+    .set_attr_parser(PoolingParamParser)
+    .set_attr<nnvm::FListInputNames>("FListInputNames",
+                                     [](const NodeAttrs&) {
+                                       return std::vector<std::string>{"data", "min_data",
+                                                                       "max_data"};
+                                     })
+    .set_attr<nnvm::FListOutputNames>("FListOutputNames",
+                                      [](const NodeAttrs&) {
+                                        return std::vector<std::string>{"output", "min_output",
+                                                                        "max_output"};
+                                      })
+    .set_attr<mxnet::FInferShape>("FInferShape", QuantizedPoolingShape)
+    .set_attr<nnvm::FInferType>("FInferType", QuantizedPoolingType)
+    .set_attr<FInferStorageType>("FInferStorageType", DefaultStorageType)
+    .set_attr<FNeedRequantize>("FNeedRequantize",
+                               [](const NodeAttrs& attrs) {
+                                 const auto& param = nnvm::get<PoolingParam>(attrs.parsed);
+                                 CHECK(param.pool_type == pool_enum::kMaxPooling ||
+                                       param.pool_type == pool_enum::kAvgPooling)
+                                     << "QuantizedPoolingOp only supports pool_type=max/avg for now";
+                                 return false;
+                               })
+    .set_attr<FCompute>("FCompute<gpu>", QuantizedPoolingForwardGPU)
+    .add_argument("data", "NDArray-or-Symbol", "Input data.")
+    .add_argument("min_data", "NDArray-or-Symbol", "Minimum value of data.")
+    .add_argument("max_data", "NDArray-or-Symbol", "Maximum value of data.")
+    .add_arguments(PoolingParam::__FIELDS__());
+
+NNVM_REGISTER_OP(_contrib_quantized_flatten)
+    .add_alias("_npx_quantized_flatten")
+    .set_num_inputs(3)
+    .set_num_outputs(3)
+    .set_attr<mxnet::FInferShape>("FInferShape", QuantizedFlattenShape)
+    .set_attr<nnvm::FInferType>("FInferType", QuantizedFlattenType)
+    .set_attr<nnvm::FListInputNames>("FListInputNames",
+                                     [](const NodeAttrs&) {
+                                       return std::vector<std::string>{"data", "min_data",
+                                                                       "max_data"};
+                                     })
+    .set_attr<nnvm::FListOutputNames>("FListOutputNames",
+                                      [](const NodeAttrs&) {
+                                        return std::vector<std::string>{"output", "min_output",
+                                                                        "max_output"};
+                                      })
+    .set_attr<nnvm::FInplaceOption>("FInplaceOption",
+                                    [](const NodeAttrs&) {
+                                      return std::vector<std::pair<int, int>>{{0, 0}, {1, 1}, {2, 2}};
+                                    })
+    .set_attr<FCompute>("FCompute<gpu>", QuantizedFlattenComputeGPU)
+    .add_argument("data", "NDArray-or-Symbol", "A ndarray/symbol of type `float32`")
+    .add_argument("min_data", "NDArray-or-Symbol",
+                  "The minimum scalar value possibly produced for the data")
+    .add_argument("max_data", "NDArray-or-Symbol",
+                  "The maximum scalar value possibly produced for the data");
 
 }  // namespace op
 }  // namespace mxnet

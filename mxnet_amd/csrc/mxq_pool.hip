@@ -1,0 +1,481 @@
+// Quantized pooling and flatten for gfx950: the operators that sit between the
+// quantized convolutions and the quantized fully-connected layer of a CNN.
+//   _contrib_quantized_pooling  src/operator/quantization/quantized_pooling.cu:33-128
+//   _contrib_quantized_flatten  src/operator/quantization/quantized_flatten-inl.h:39-110
+//
+// Pooling is byte work bound by HBM: a work-group copies the contiguous run of input
+// rows its outputs need (one band of a large plane, or several whole small planes)
+// into LDS with 16-byte loads, then every thread folds its windows out of LDS.  The
+// input is read from memory once even where windows overlap (3x3 / stride 2).
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+
+#include "../../include/mxq.h"
+#include "mxq_common.h"
+#include "mxq_gemm.cuh"
+
+namespace mxq {
+namespace {
+
+constexpr int kPoolThreads = 256;
+constexpr int kPoolLdsBytes = 32768;  // input bytes staged per work-group (3+ groups per CU)
+
+struct PoolArgs {
+  const uint8_t* in;
+  uint8_t* out;
+  size_t total_in;  // bytes of the whole input tensor
+  int planes, H, W, OH, OW, KH, KW, sh, sw, ph, pw;
+  int is_avg, count_pad, is_unsigned;
+  int ppb;    // planes per work-group (> 1 only when band == OH)
+  int band;   // output rows per work-group
+  int bands;  // bands per plane
+  int vec_ok; // the tensor base is 16-byte aligned
+  // floor(n / d) = umulhi(n, magic) for n * d < 2^32 (magic = 2^32 / d + 1; 0 stands for d = 1)
+  uint32_t magic_ow4;        // d = ceil(OW / 4)
+  uint32_t magic_per_plane;  // d = OH * ceil(OW / 4), used when ppb > 1
+};
+
+__device__ __forceinline__ int fast_div(int n, uint32_t magic) {
+  return magic == 0 ? n : static_cast<int>(__umulhi(static_cast<uint32_t>(n), magic));
+}
+
+// One window out of a byte image (LDS or global): rows of `W` bytes starting at
+// `img`, whose first row is image row `row0`.
+template <bool UNSIGNED, typename Ptr>
+__device__ __forceinline__ int pool_window(Ptr img, int row0, const PoolArgs& a, int oh, int ow) {
+  int hstart = oh * a.sh - a.ph, wstart = ow * a.sw - a.pw;
+  int hend = min(hstart + a.KH, a.H + a.ph), wend = min(wstart + a.KW, a.W + a.pw);
+  int pool_size = (hend - hstart) * (wend - wstart);
+  hstart = max(hstart, 0);
+  wstart = max(wstart, 0);
+  hend = min(hend, a.H);
+  wend = min(wend, a.W);
+  if (!a.count_pad) pool_size = (hend - hstart) * (wend - wstart);
+  constexpr int lo = UNSIGNED ? 0 : -128, hi = UNSIGNED ? 255 : 127;
+  int acc = a.is_avg ? 0 : lo;
+  for (int h = hstart; h < hend; ++h) {
+    const int base = (h - row0) * a.W;
+    for (int w = wstart; w < wend; ++w) {
+      const uint8_t b = img[base + w];
+      const int v = UNSIGNED ? static_cast<int>(b) : static_cast<int>(static_cast<int8_t>(b));
+      acc = a.is_avg ? acc + v : max(acc, v);
+    }
+  }
+  if (!a.is_avg) return acc;
+  // nearest, ties to even, of sum / divisor (exact: the binary32 quotient is exact on
+  // ties and cannot round onto one)
+  const float avg = pool_size > 0 ? static_cast<float>(acc) / static_cast<float>(pool_size) : 0.f;
+  int q = static_cast<int>(rintf(avg));
+  return min(max(q, lo), hi);
+}
+
+// Four horizontally adjacent outputs of one row, for a compile-time window width and
+// stride.  The 3*SW + KW wide strip of every window row is read from LDS as three
+// aligned dwords (the LDS instruction rate and divergence are what bound this kernel,
+// not arithmetic), realigned with the byte funnel shift, and folded into the outputs
+// that cover each byte.  Columns outside the image are neutralised instead of branched
+// around (the staged image has 16 bytes of slack in front and 32 behind), so border
+// items take the same path as interior ones.
+template <bool UNSIGNED, int KW, int SW>
+__device__ __forceinline__ void pool_quad(const uint8_t* img, int row0, const PoolArgs& a, int oh,
+                                          int ow0, int (&q)[4]) {
+  constexpr int lo = UNSIGNED ? 0 : -128, hi = UNSIGNED ? 255 : 127;
+  constexpr int SPAN = 3 * SW + KW;
+  static_assert(SPAN + 3 <= 12, "three aligned dwords cover the strip at any byte offset");
+  int hstart = oh * a.sh - a.ph;
+  int hend = min(hstart + a.KH, a.H + a.ph);
+  const int padded_rows = hend - hstart;
+  hstart = max(hstart, 0);
+  hend = min(hend, a.H);
+  const int w0 = ow0 * SW - a.pw;
+  const int neutral = a.is_avg ? 0 : lo;
+  // byte masks of the columns inside the image, and what the others are replaced with
+  uint32_t keep[3] = {0u, 0u, 0u};
+#pragma unroll
+  for (int j = 0; j < SPAN; ++j)
+    if (static_cast<unsigned>(w0 + j) < static_cast<unsigned>(a.W))
+      keep[j / 4] |= 0xffu << (8 * (j % 4));
+  const uint32_t fill = (static_cast<uint32_t>(neutral) & 0xffu) * 0x01010101u;
+  int acc[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) acc[i] = neutral;
+  for (int h = hstart; h < hend; ++h) {
+    const uintptr_t addr = reinterpret_cast<uintptr_t>(img + (h - row0) * a.W + w0);
+    const uint32_t* wp = reinterpret_cast<const uint32_t*>(addr & ~static_cast<uintptr_t>(3));
+    const uint32_t sft = static_cast<uint32_t>(addr & 3u);
+    const uint32_t d0 = wp[0], d1 = wp[1], d2 = wp[2];
+    uint32_t x[3];
+    x[0] = __builtin_amdgcn_alignbyte(d1, d0, sft);
+    x[1] = __builtin_amdgcn_alignbyte(d2, d1, sft);
+    x[2] = __builtin_amdgcn_alignbyte(0u, d2, sft);
+#pragma unroll
+    for (int w = 0; w < 3; ++w) x[w] = (x[w] & keep[w]) | (fill & ~keep[w]);  // one v_bfi
+    int v[SPAN];
+#pragma unroll
+    for (int j = 0; j < SPAN; ++j) {
+      const uint32_t b = (x[j / 4] >> (8 * (j % 4))) & 0xffu;
+      v[j] = UNSIGNED ? static_cast<int>(b) : static_cast<int>(static_cast<int8_t>(b));
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int k = 0; k < KW; ++k)
+        acc[i] = a.is_avg ? acc[i] + v[i * SW + k] : max(acc[i], v[i * SW + k]);
+  }
+  if (!a.is_avg) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) q[i] = acc[i];
+    return;
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int wstart = w0 + i * SW;
+    const int wend = min(wstart + KW, a.W + a.pw);
+    const int pool_size = a.count_pad
+                              ? padded_rows * (wend - wstart)
+                              : (hend - hstart) * (min(wend, a.W) - max(wstart, 0));
+    const float avg =
+        pool_size > 0 ? static_cast<float>(acc[i]) / static_cast<float>(pool_size) : 0.f;
+    q[i] = min(max(static_cast<int>(rintf(avg)), lo), hi);
+  }
+}
+
+// Sum of the n bytes at LDS byte address `addr`: aligned dwords through the 4-way
+// byte dot product against 0x01010101, the partial first and last dwords masked.
+template <bool UNSIGNED>
+__device__ __forceinline__ int sum_bytes(const uint8_t* lds, int addr, int n) {
+  const uint32_t* words = reinterpret_cast<const uint32_t*>(lds);
+  const int lo = addr, hi = addr + n;
+  int sum = 0;
+  for (int w = lo >> 2; w < (hi + 3) >> 2; ++w) {
+    uint32_t x = words[w];
+    const int bs = max(lo - 4 * w, 0), be = min(hi - 4 * w, 4);
+    const uint32_t keep_hi = be >= 4 ? 0xffffffffu : ((1u << (8 * be)) - 1u);
+    const uint32_t drop_lo = (1u << (8 * bs)) - 1u;  // bs <= 3
+    x &= keep_hi & ~drop_lo;
+    if (UNSIGNED)
+      sum = static_cast<int>(__builtin_amdgcn_udot4(x, 0x01010101u, static_cast<uint32_t>(sum),
+                                                    false));
+    else
+      sum = __builtin_amdgcn_sdot4(static_cast<int>(x), 0x01010101, sum, false);
+  }
+  return sum;
+}
+
+// FAST: 0 generic windows; 1 quads with KW=3,SW=2; 2 quads KW=2,SW=2; 3 quads KW=3,SW=1;
+// 4 average over full-width windows (global pooling): contiguous byte sums.
+template <bool UNSIGNED, int FAST>
+__global__ __launch_bounds__(kPoolThreads) void pool_lds_kernel(PoolArgs a) {
+  // the staged bytes start 16 bytes into the array: strips that begin left of column 0
+  // read (and discard) what lies in front
+  __shared__ __attribute__((aligned(16))) uint8_t lds_raw[kPoolLdsBytes + 64];
+  uint8_t* lds = lds_raw + 16;
+  const int tid = threadIdx.x;
+  int p0, np, oh0, oh1;
+  if (a.ppb > 1) {
+    p0 = blockIdx.x * a.ppb;
+    np = min(a.ppb, a.planes - p0);
+    oh0 = 0;
+    oh1 = a.OH;
+  } else {
+    p0 = blockIdx.x / a.bands;
+    np = 1;
+    oh0 = (blockIdx.x % a.bands) * a.band;
+    oh1 = min(oh0 + a.band, a.OH);
+  }
+  const size_t plane_bytes = static_cast<size_t>(a.H) * a.W;
+  int hs = 0, he = a.H;
+  if (a.ppb <= 1) {
+    hs = min(max(oh0 * a.sh - a.ph, 0), a.H);
+    he = max(min((oh1 - 1) * a.sh - a.ph + a.KH, a.H), hs);
+  }
+  const size_t g0 = static_cast<size_t>(p0) * plane_bytes + static_cast<size_t>(hs) * a.W;
+  const size_t len = static_cast<size_t>(np - 1) * plane_bytes + static_cast<size_t>(he - hs) * a.W;
+  int shift = 0;
+  if (a.vec_ok) {
+    // 16-byte chunks from the aligned address below g0 straight into LDS (chunk c lands
+    // at byte 16*c), every chunk of the work-group in flight at once.  The descriptor ends
+    // at the last whole dword of the tensor: what lies past it arrives as zeros and the
+    // tensor's last 1..3 bytes are patched in below.
+    const size_t a0 = g0 & ~static_cast<size_t>(15);
+    shift = static_cast<int>(g0 - a0);
+    const int chunks = static_cast<int>((shift + len + 15) / 16);
+    const size_t whole = a.total_in & ~static_cast<size_t>(3);
+    const size_t avail = whole > a0 ? whole - a0 : 0;
+    const v4i rsrc = make_rsrc(a.in + a0, static_cast<uint32_t>(avail < 0xffffffffu ? avail
+                                                                                      : 0xffffffffu));
+    const uint32_t lds0 = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(lds));
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
+    for (int c0 = wave * 64; c0 < chunks; c0 += (kPoolThreads / 64) * 64) {
+      if (c0 + lane < chunks)
+        dma_buffer(lds0 + static_cast<uint32_t>(c0) * 16, static_cast<uint32_t>(c0 + lane) * 16,
+                   rsrc);
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    const size_t end = g0 + len;
+    if (tid < 3 && whole + tid < a.total_in && whole + tid >= g0 && whole + tid < end)
+      lds[whole + tid - a0] = a.in[whole + tid];
+  } else {
+    for (size_t i = tid; i < len; i += kPoolThreads) lds[i] = a.in[g0 + i];
+  }
+  __syncthreads();
+  const int rows = oh1 - oh0;
+  if (FAST == 4) {
+    // OW == 1 and every window spans the full width: rows [hstart, hend) of a plane are
+    // one contiguous run of bytes
+    constexpr int lo = UNSIGNED ? 0 : -128, hi = UNSIGNED ? 255 : 127;
+    const int outputs = np * rows;
+    for (int o = tid; o < outputs; o += kPoolThreads) {
+      const int p = o / rows, oh = oh0 + (o - p * rows);
+      int hstart = oh * a.sh - a.ph;
+      int hend = min(hstart + a.KH, a.H + a.ph);
+      const int padded = (hend - hstart) * a.W;  // pad_w == 0 and kernel_w == W here
+      hstart = max(hstart, 0);
+      hend = min(hend, a.H);
+      const int addr = shift + p * static_cast<int>(plane_bytes) + (hstart - hs) * a.W;
+      const int n = max(hend - hstart, 0) * a.W;
+      const int sum = sum_bytes<UNSIGNED>(lds, addr, n);
+      const int pool_size = a.count_pad ? padded : n;
+      const float avg =
+          pool_size > 0 ? static_cast<float>(sum) / static_cast<float>(pool_size) : 0.f;
+      const int q = min(max(static_cast<int>(rintf(avg)), lo), hi);
+      a.out[static_cast<size_t>(p0 + p) * a.OH + oh] = static_cast<uint8_t>(q);
+    }
+    return;
+  }
+  // items of four adjacent outputs of one row
+  const int OW4 = (a.OW + 3) >> 2;
+  const int per_plane = rows * OW4;
+  const int items = np * per_plane;
+  constexpr int KW = FAST == 1 ? 3 : FAST == 2 ? 2 : 3;
+  constexpr int SW = FAST == 3 ? 1 : 2;
+  for (int it = tid; it < items; it += kPoolThreads) {
+    const int p = a.ppb > 1 ? fast_div(it, a.magic_per_plane) : 0, r = it - p * per_plane;
+    const int orow = fast_div(r, a.magic_ow4), ow0 = (r - orow * OW4) * 4;
+    const int oh = oh0 + orow;
+    const int nout = min(4, a.OW - ow0);
+    const uint8_t* img = lds + shift + static_cast<size_t>(p) * plane_bytes;
+    int q[4] = {0, 0, 0, 0};
+    if (FAST != 0) {
+      pool_quad<UNSIGNED, KW, SW>(img, hs, a, oh, ow0, q);
+    } else {
+      // (fixed trip count: a runtime-indexed q[] would live in scratch memory)
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        if (i < nout) q[i] = pool_window<UNSIGNED>(img, hs, a, oh, ow0 + i);
+    }
+    const size_t off = (static_cast<size_t>(p0 + p) * a.OH + oh) * a.OW + ow0;
+    if (nout == 4 && ((reinterpret_cast<uintptr_t>(a.out) + off) & 3u) == 0) {
+      const uint32_t packed = (static_cast<uint32_t>(q[0]) & 0xffu) |
+                              ((static_cast<uint32_t>(q[1]) & 0xffu) << 8) |
+                              ((static_cast<uint32_t>(q[2]) & 0xffu) << 16) |
+                              (static_cast<uint32_t>(q[3]) << 24);
+      *reinterpret_cast<uint32_t*>(a.out + off) = packed;
+    } else {
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        if (i < nout) a.out[off + i] = static_cast<uint8_t>(q[i]);
+    }
+  }
+}
+
+// Fallback for images whose single window band does not fit the LDS budget.
+template <bool UNSIGNED>
+__global__ __launch_bounds__(kPoolThreads) void pool_direct_kernel(PoolArgs a) {
+  const size_t total = static_cast<size_t>(a.planes) * a.OH * a.OW;
+  for (size_t o = static_cast<size_t>(blockIdx.x) * kPoolThreads + threadIdx.x; o < total;
+       o += static_cast<size_t>(gridDim.x) * kPoolThreads) {
+    const size_t p = o / (static_cast<size_t>(a.OH) * a.OW);
+    const int r = static_cast<int>(o - p * a.OH * a.OW);
+    const int oh = r / a.OW, ow = r - oh * a.OW;
+    const uint8_t* img = a.in + p * static_cast<size_t>(a.H) * a.W;
+    a.out[o] = static_cast<uint8_t>(pool_window<UNSIGNED>(img, 0, a, oh, ow));
+  }
+}
+
+__global__ void copy_range_kernel(const float* imin, const float* imax, float* omin,
+                                  float* omax) {
+  *omin = *imin;
+  *omax = *imax;
+}
+
+// Flat byte copy, 16 bytes per lane where both pointers allow it.
+__global__ __launch_bounds__(256) void copy_bytes_kernel(const uint8_t* __restrict__ in,
+                                                         uint8_t* __restrict__ out, size_t n,
+                                                         int vec_ok) {
+  const size_t stride = static_cast<size_t>(gridDim.x) * 256;
+  const size_t t = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
+  if (vec_ok) {
+    const size_t nv = n / 16;
+    for (size_t i = t; i < nv; i += stride)
+      reinterpret_cast<uint4*>(out)[i] = reinterpret_cast<const uint4*>(in)[i];
+    for (size_t i = nv * 16 + t; i < n; i += stride) out[i] = in[i];
+  } else {
+    for (size_t i = t; i < n; i += stride) out[i] = in[i];
+  }
+}
+
+int device_cus() {
+  int dev = 0;
+  MXQ_HIP(hipGetDevice(&dev));
+  static thread_local int cached_dev = -1, cached_cus = 0;
+  if (cached_dev != dev) {
+    MXQ_HIP(hipDeviceGetAttribute(&cached_cus, hipDeviceAttributeMultiprocessorCount, dev));
+    cached_dev = dev;
+  }
+  return cached_cus;
+}
+
+}  // namespace
+}  // namespace mxq
+
+using namespace mxq;
+
+extern "C" {
+
+int mxq_quantized_pooling_nchw(void* stream, const void* in, int in_type, int N, int C, int H,
+                               int W, int kernel_h, int kernel_w, int stride_h, int stride_w,
+                               int pad_h, int pad_w, int OH, int OW, int pool_type,
+                               int count_include_pad, const float* imin, const float* imax,
+                               void* out, float* omin, float* omax) {
+  MXQ_API_BEGIN();
+  MXQ_CHECK(in_type == MXQ_INT8 || in_type == MXQ_UINT8, "pooling takes int8 or uint8 data");
+  MXQ_CHECK(pool_type == MXQ_POOL_MAX || pool_type == MXQ_POOL_AVG,
+            "QuantizedPoolingOp only supports pool_type=max/avg for now");
+  MXQ_CHECK(N >= 0 && C >= 0 && H > 0 && W > 0 && OH > 0 && OW > 0, "bad shape");
+  MXQ_CHECK(kernel_h > 0 && kernel_w > 0 && stride_h > 0 && stride_w > 0 && pad_h >= 0 &&
+                pad_w >= 0,
+            "bad kernel/stride/pad");
+  MXQ_CHECK(kernel_h <= H + 2 * pad_h && kernel_w <= W + 2 * pad_w,
+            "kernel size exceeds the padded input");
+  MXQ_CHECK(imin && imax && omin && omax, "null range pointer");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  hipLaunchKernelGGL(copy_range_kernel, dim3(1), dim3(1), 0, s, imin, imax, omin, omax);
+  MXQ_LAUNCH_CHECK();
+  const long long planes = static_cast<long long>(N) * C;
+  if (planes == 0) return 0;
+  MXQ_CHECK(in != nullptr && out != nullptr, "null data pointer");
+  MXQ_CHECK(planes < (1LL << 31) && static_cast<long long>(OH) * OW < (1LL << 31) &&
+                static_cast<long long>(H) * W < (1LL << 31),
+            "problem too large for 32-bit plane indices");
+  PoolArgs a;
+  a.in = static_cast<const uint8_t*>(in);
+  a.out = static_cast<uint8_t*>(out);
+  a.total_in = static_cast<size_t>(planes) * H * W;
+  a.planes = static_cast<int>(planes);
+  a.H = H; a.W = W; a.OH = OH; a.OW = OW; a.KH = kernel_h; a.KW = kernel_w;
+  a.sh = stride_h; a.sw = stride_w; a.ph = pad_h; a.pw = pad_w;
+  a.is_avg = pool_type == MXQ_POOL_AVG;
+  a.count_pad = count_include_pad != 0;
+  a.is_unsigned = in_type == MXQ_UINT8;
+  a.vec_ok = aligned16(in) ? 1 : 0;
+  const long long plane_bytes = static_cast<long long>(H) * W;
+  const int cus = device_cus();
+  long long blocks = 0;
+  bool direct = false;
+  if (2 * plane_bytes <= kPoolLdsBytes) {
+    // small planes: several per work-group, but keep at least ~4 groups per CU
+    long long ppb = kPoolLdsBytes / plane_bytes;
+    const long long spread = (planes + 4LL * cus - 1) / (4LL * cus);
+    if (ppb > spread) ppb = spread;
+    if (ppb < 1) ppb = 1;
+    a.ppb = static_cast<int>(ppb);
+    a.band = OH;
+    a.bands = 1;
+    blocks = (planes + ppb - 1) / ppb;
+  } else {
+    a.ppb = 1;
+    // rows_in(band) = (band - 1) * stride + kernel  <=  budget / W
+    const long long rows_fit = kPoolLdsBytes / W;
+    long long band = rows_fit >= kernel_h ? (rows_fit - kernel_h) / stride_h + 1 : 0;
+    if (band > OH) band = OH;
+    if (band < 1) {
+      direct = true;
+    } else {
+      a.band = static_cast<int>(band);
+      a.bands = static_cast<int>((OH + band - 1) / band);
+      blocks = planes * a.bands;
+    }
+  }
+  if (direct) {
+    a.band = OH;
+    a.bands = 1;
+    const long long total = planes * OH * OW;
+    long long g = (total + kPoolThreads - 1) / kPoolThreads;
+    if (g > 8LL * cus) g = 8LL * cus;
+    if (a.is_unsigned)
+      hipLaunchKernelGGL((pool_direct_kernel<true>), dim3(g), dim3(kPoolThreads), 0, s, a);
+    else
+      hipLaunchKernelGGL((pool_direct_kernel<false>), dim3(g), dim3(kPoolThreads), 0, s, a);
+  } else {
+    MXQ_CHECK(blocks < (1LL << 31), "pooling grid too large");
+    auto magic = [](long long d) {
+      return d <= 1 ? 0u : static_cast<uint32_t>((1ULL << 32) / static_cast<unsigned long long>(d) + 1ULL);
+    };
+    const long long ow4 = (OW + 3) / 4;
+    // items per work-group stay below 2^17 and the divisors below 2^15 (both bounded by
+    // the bytes staged in LDS), so n * d < 2^32 holds
+    MXQ_CHECK(ow4 * OH < (1LL << 15) || a.ppb <= 1, "pooling plane too large for the item index");
+    MXQ_CHECK(ow4 < (1LL << 15), "pooling row too long for the item index");
+    a.magic_ow4 = magic(ow4);
+    a.magic_per_plane = magic(ow4 * OH);
+    int fast = 0;
+    if (a.is_avg && OW == 1 && pad_w == 0 && kernel_w == W)
+      fast = 4;
+    else if (pad_w > 8)
+      fast = 0;  // the quad path reads at most 16 bytes in front of a row
+    else if (kernel_w == 3 && stride_w == 2)
+      fast = 1;
+    else if (kernel_w == 2 && stride_w == 2)
+      fast = 2;
+    else if (kernel_w == 3 && stride_w == 1)
+      fast = 3;
+#define MXQ_POOL(U, F) \
+  hipLaunchKernelGGL((pool_lds_kernel<U, F>), dim3(blocks), dim3(kPoolThreads), 0, s, a)
+#define MXQ_POOL_F(U)            \
+  switch (fast) {                \
+    case 1: MXQ_POOL(U, 1); break; \
+    case 2: MXQ_POOL(U, 2); break; \
+    case 3: MXQ_POOL(U, 3); break; \
+    case 4: MXQ_POOL(U, 4); break; \
+    default: MXQ_POOL(U, 0); break; \
+  }
+    if (a.is_unsigned) {
+      MXQ_POOL_F(true)
+    } else {
+      MXQ_POOL_F(false)
+    }
+#undef MXQ_POOL_F
+#undef MXQ_POOL
+  }
+  MXQ_LAUNCH_CHECK();
+  MXQ_API_END();
+}
+
+int mxq_quantized_flatten(void* stream, const void* in, const float* imin, const float* imax,
+                          void* out, float* omin, float* omax, size_t n_bytes) {
+  MXQ_API_BEGIN();
+  MXQ_CHECK(imin && imax && omin && omax, "null range pointer");
+  MXQ_CHECK(n_bytes == 0 || (in != nullptr && out != nullptr), "null data pointer");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (omin != imin || omax != imax) {
+    hipLaunchKernelGGL(copy_range_kernel, dim3(1), dim3(1), 0, s, imin, imax, omin, omax);
+    MXQ_LAUNCH_CHECK();
+  }
+  if (n_bytes != 0 && in != out) {
+    const int vec_ok = aligned16(in) && aligned16(out);
+    size_t g = (n_bytes / (vec_ok ? 16 : 1) + 255) / 256;
+    const size_t cap = static_cast<size_t>(device_cus()) * 8;
+    if (g > cap) g = cap;
+    if (g < 1) g = 1;
+    hipLaunchKernelGGL(copy_bytes_kernel, dim3(static_cast<unsigned>(g)), dim3(256), 0, s,
+                       static_cast<const uint8_t*>(in), static_cast<uint8_t*>(out), n_bytes,
+                       vec_ok);
+    MXQ_LAUNCH_CHECK();
+  }
+  MXQ_API_END();
+}
+
+}  // extern "C"

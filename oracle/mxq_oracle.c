@@ -25,6 +25,14 @@
  *   - qref_fc / qref_conv_nchw: numpy int64 matmul, torch int conv on the
  *     same operands, the reference test's integer-valued fp32 Dense/Conv
  *     construction, identity / single-tap special cases.
+ *   - qref_pool_nchw: max pooling is exact integer work, pinned against torch
+ *     max_pool2d on integer-valued floats and brute force.  For avg pooling the
+ *     window and divisor follow the reference's own fp32 pooling loop, but the
+ *     ROUNDING of the quotient to int8 lives in cuDNN / oneDNN (third-party,
+ *     absent): PARITY UNPINNED for that one step.  Here: nearest, ties to even,
+ *     of the exact quotient; checked against an exact rational evaluation and
+ *     against the reference test's own bound (|int8 - fp32 pooling| <= 2,
+ *     tests/python/quantization/test_quantization.py:634-639).
  */
 #include <math.h>
 #include <stddef.h>
@@ -275,4 +283,66 @@ void qref_conv_nchw(const int8_t* data, const int8_t* weight, const int32_t* bia
 void qref_relu_i8(const int8_t* in, size_t n, int8_t* out) {
 #pragma omp parallel for schedule(static)
   for (ptrdiff_t i = 0; i < (ptrdiff_t)n; ++i) out[i] = in[i] > 0 ? in[i] : 0;
+}
+
+/* ---- _contrib_quantized_pooling ------------------------------------------
+ * 2-D pooling of an NCHW int8 (is_unsigned = 0) or uint8 tensor; min/max pass
+ * through (quantized_pooling.cu:76-98).  Output extents are the caller's
+ * (QuantizedPoolingShape, quantized_pooling.cc:32-133).  The window of output
+ * (oh, ow) and the divisor follow pool_sum_2d_nchw_cpu / pool_max_2d_nchw_cpu
+ * (src/operator/nn/pool.h:476-522): hstart = oh*sh - ph, hend = min(hstart+kh,
+ * H+ph), divisor = (hend-hstart)*(wend-wstart) before clipping to the image when
+ * padding counts (cuDNN's COUNT_INCLUDE_PADDING, quantized_pooling.cu:46-50),
+ * after clipping otherwise.  max: padding never wins (cudnn NOT_PROPAGATE_NAN
+ * max over valid taps); an empty window yields the type's minimum.
+ * avg: q = nearest-even(sum / divisor), saturated - see the header. */
+void qref_pool_nchw(const void* in_, int is_unsigned, int N, int C, int H, int W, int KH,
+                    int KW, int sh, int sw, int ph, int pw, int OH, int OW, int is_avg,
+                    int count_include_pad, void* out_) {
+  const int8_t* in_s = (const int8_t*)in_;
+  const uint8_t* in_u = (const uint8_t*)in_;
+  int8_t* out_s = (int8_t*)out_;
+  uint8_t* out_u = (uint8_t*)out_;
+  const int lo = is_unsigned ? 0 : -128, hi = is_unsigned ? 255 : 127;
+#pragma omp parallel for schedule(static)
+  for (ptrdiff_t nc = 0; nc < (ptrdiff_t)N * C; ++nc) {
+    const size_t ibase = (size_t)nc * H * W, obase = (size_t)nc * OH * OW;
+    for (int oh = 0; oh < OH; ++oh) {
+      for (int ow = 0; ow < OW; ++ow) {
+        int hstart = oh * sh - ph, wstart = ow * sw - pw;
+        int hend = hstart + KH < H + ph ? hstart + KH : H + ph;
+        int wend = wstart + KW < W + pw ? wstart + KW : W + pw;
+        int pool_size = (hend - hstart) * (wend - wstart);
+        if (hstart < 0) hstart = 0;
+        if (wstart < 0) wstart = 0;
+        if (hend > H) hend = H;
+        if (wend > W) wend = W;
+        if (!count_include_pad) pool_size = (hend - hstart) * (wend - wstart);
+        int32_t acc = is_avg ? 0 : lo;
+        for (int h = hstart; h < hend; ++h)
+          for (int w = wstart; w < wend; ++w) {
+            const size_t i = ibase + (size_t)h * W + w;
+            const int v = is_unsigned ? (int)in_u[i] : (int)in_s[i];
+            if (is_avg)
+              acc += v;
+            else if (v > acc)
+              acc = v;
+          }
+        int q = acc;
+        if (is_avg) {
+          /* float(sum)/float(divisor) is exact whenever the quotient is a tie (k + 0.5
+           * is representable) and cannot be rounded onto one otherwise, so rintf of
+           * it is nearest-even of the exact quotient */
+          const float avg = pool_size > 0 ? (float)acc / (float)pool_size : 0.0f;
+          q = (int)rintf(avg);
+          if (q < lo) q = lo;
+          if (q > hi) q = hi;
+        }
+        if (is_unsigned)
+          out_u[obase + (size_t)oh * OW + ow] = (uint8_t)q;
+        else
+          out_s[obase + (size_t)oh * OW + ow] = (int8_t)q;
+      }
+    }
+  }
 }

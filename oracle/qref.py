@@ -48,6 +48,7 @@ _lib.qref_bias_i8_to_i32.argtypes = [_p, _sz, _f, _f, _f, _f, _p]
 _lib.qref_fc.argtypes = [_p, _p, _p, _i, _i, _i, _p]
 _lib.qref_conv_nchw.argtypes = [_p, _p, _p] + [_i] * 13 + [_p]
 _lib.qref_relu_i8.argtypes = [_p, _sz, _p]
+_lib.qref_pool_nchw.argtypes = [_p, _i] + [_i] * 12 + [_i, _i, _p]
 
 
 def _c(a, dtype):
@@ -219,3 +220,49 @@ def relu_i8(q):
     out = np.empty_like(q)
     _lib.qref_relu_i8(_ptr(q), q.size, _ptr(out))
     return out
+
+
+def pooling_output_hw(H, W, kernel, stride, pad, global_pool=False, convention="valid"):
+    """Output extents of QuantizedPoolingShape (quantized_pooling.cc:82-121)."""
+    if global_pool:
+        return 1, 1
+    out = []
+    for size, k, s, p in ((H, kernel[0], stride[0], pad[0]), (W, kernel[1], stride[1], pad[1])):
+        if k > size + 2 * p:
+            raise ValueError("kernel size (%d) exceeds input (%d padded to %d)"
+                             % (k, size, size + 2 * p))
+        if convention == "valid":
+            out.append(1 + (size + 2 * p - k) // s)
+        elif convention == "full":
+            # 1 + int(ceil(float(x) / s)) evaluated in binary32 as the reference does
+            out.append(1 + int(np.ceil(np.float32(size + 2 * p - k) / np.float32(s))))
+        else:
+            raise ValueError("pooling_convention %r is not supported" % convention)
+    return out[0], out[1]
+
+
+def quantized_pooling(data, min_data, max_data, kernel=(1, 1), pool_type="max", stride=(1, 1),
+                      pad=(0, 0), global_pool=False, convention="valid",
+                      count_include_pad=True):
+    """_contrib_quantized_pooling on NCHW int8/uint8 -> (out, min, max)."""
+    if data.dtype not in (np.int8, np.uint8):
+        raise TypeError("quantized_pooling takes int8 or uint8")
+    if pool_type not in ("max", "avg"):
+        raise ValueError("QuantizedPoolingOp only supports pool_type=max/avg for now")
+    d = _c(data, data.dtype)
+    N, C, H, W = d.shape
+    if global_pool:
+        kernel, stride, pad = (H, W), (1, 1), pad
+    OH, OW = pooling_output_hw(H, W, kernel, stride, pad, global_pool, convention)
+    out = np.empty((N, C, OH, OW), dtype=d.dtype)
+    _lib.qref_pool_nchw(_ptr(d), int(d.dtype == np.uint8), N, C, H, W, kernel[0], kernel[1],
+                        stride[0], stride[1], pad[0], pad[1], OH, OW, int(pool_type == "avg"),
+                        int(bool(count_include_pad)), _ptr(out))
+    return out, np.float32(min_data), np.float32(max_data)
+
+
+def quantized_flatten(data, min_data, max_data):
+    """_contrib_quantized_flatten (quantized_flatten-inl.h:39-110): a reshape to
+    (d0, prod(rest)); the ranges pass through."""
+    d = np.ascontiguousarray(data)
+    return d.reshape(d.shape[0], -1).copy(), np.float32(min_data), np.float32(max_data)

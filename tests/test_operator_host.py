@@ -154,3 +154,46 @@ def test_type_inference():
     with pytest.raises(MXNetError, match="relu"):
         Node("_contrib_quantized_act", act_type="tanh").infer_type([I8, None, None])
     assert Node("_contrib_quantize_v2").infer_type([I8])[1][0] == I8   # pass-through input
+
+
+def test_pooling_and_flatten_inference():
+    """quantized_pooling.cc:32-157, quantized_flatten-inl.h:96-131; the shapes are those
+    of the reference's test (test_quantization.py:641-658)."""
+    for n in ["_contrib_quantized_pooling", "_contrib_quantized_flatten"]:
+        assert op.has_attr(n, "FCompute<gpu>") and op.has_attr(n, "FInferShape")
+    assert op.has_attr("_npx_quantized_pooling", "FInferType")
+    assert op.has_attr("_contrib_quantized_pooling", "FNeedRequantize")
+    assert op.has_attr("_contrib_quantized_flatten", "FInplaceOption")
+    n = Node("_contrib_quantized_pooling", kernel=(3, 3), pool_type="max", stride=(2, 2))
+    assert n.list_inputs() == ["data", "min_data", "max_data"]
+    assert n.list_outputs() == ["output", "min_output", "max_output"]
+    ins, outs = n.infer_shape([(3, 4, 56, 56), None, None])
+    assert ins == [(3, 4, 56, 56), (1,), (1,)] and outs == [(3, 4, 27, 27), (1,), (1,)]
+    n = Node("_contrib_quantized_pooling", kernel=(3, 3), pool_type="max", stride=(2, 2),
+             pooling_convention="full")
+    assert n.infer_shape([(3, 4, 56, 56), None, None])[1][0] == (3, 4, 28, 28)
+    n = Node("_contrib_quantized_pooling", kernel=(3, 3), pool_type="max", stride=(2, 2),
+             global_pool=True)
+    assert n.infer_shape([(3, 4, 56, 56), None, None])[1][0] == (3, 4, 1, 1)
+    n = Node("_contrib_quantized_pooling", kernel=(7, 7), pool_type="avg")
+    assert n.infer_shape([(3, 512, 7, 7), None, None])[1][0] == (3, 512, 1, 1)
+    n = Node("_contrib_quantized_pooling", kernel=(3, 3), pool_type="max", stride=(2, 2),
+             pad=(1, 1))
+    assert n.infer_shape([(64, 64, 112, 112), None, None])[1][0] == (64, 64, 56, 56)
+    # output type follows the data type
+    assert n.infer_type([I8, None, None]) == ([I8, F32, F32], [I8, F32, F32])
+    assert n.infer_type([U8, None, None])[1][0] == U8
+    with pytest.raises(MXNetError, match="exceeds input"):
+        Node("_contrib_quantized_pooling", kernel=(9, 9)).infer_shape([(1, 1, 7, 7), None, None])
+    with pytest.raises(MXNetError, match="4D"):
+        Node("_contrib_quantized_pooling", kernel=(3, 3)).infer_shape(
+            [(1, 1, 3, 7, 7), None, None])
+    with pytest.raises(MXNetError, match="max/avg"):
+        Node("_contrib_quantized_pooling", kernel=(3, 3), pool_type="sum").infer_type(
+            [I8, None, None])
+    with pytest.raises(MXNetError, match="pool_type"):
+        Node("_contrib_quantized_pooling", kernel=(3, 3), pool_type="median")
+    n = Node("_contrib_quantized_flatten")
+    assert n.infer_shape([(2, 3, 4, 5), None, None]) == ([(2, 3, 4, 5), (1,), (1,)],
+                                                         [(2, 60), (1,), (1,)])
+    assert n.infer_type([U8, None, None]) == ([U8, F32, F32], [U8, F32, F32])
