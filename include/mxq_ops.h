@@ -61,6 +61,31 @@ int mxq_node_temp_bytes(void* node, int num_in, const mxq_blob* in, int num_out,
 int mxq_node_forward(void* node, void* stream, int dev_id, int num_in, const mxq_blob* in,
                      int num_out, const mxq_blob* out, void* temp_space, size_t temp_bytes);
 
+/* ---- graph passes over symbol JSON ------------------------------------------------
+ * Counterparts of MXQuantizeSymbol and MXSetCalibTableToQuantizedSymbol
+ * (src/c_api/c_api_symbolic.cc:916-972, 1031-1050) with the symbol passed as the text
+ * of its `-symbol.json`.  dev_type is Context::DeviceType (1 cpu, 2 gpu): a float
+ * operator is replaced only if its quantized counterpart has a compute function for
+ * that device.  Returned strings belong to the calling thread and stay valid until its
+ * next call into this library. */
+int mxq_quantize_symbol(const char* symbol_json, int dev_type, int num_excluded_nodes,
+                        const char** excluded_nodes, int num_excluded_ops,
+                        const char** excluded_ops, int num_offline, const char** offline_params,
+                        const char* quantized_dtype, const char* quantize_mode,
+                        const char* quantize_granularity, const char** out_symbol_json,
+                        int* out_num_calib_names, const char*** out_calib_names);
+int mxq_set_calib_table(const char* qsymbol_json, int num_layers, const char** layer_names,
+                        const float* min_ranges, const float* max_ranges,
+                        const char** out_symbol_json);
+/* Loads and re-saves a symbol: nodes reachable from the heads, renumbered in
+ * depth-first post-order, as the reference writes them. */
+int mxq_symbol_normalize(const char* symbol_json, const char** out_symbol_json);
+
+/* _contrib_calibrate_entropy (src/operator/quantization/calibrate.cc:89-186); host
+ * arrays: hist[num_bins] (num_bins odd), hist_edges[num_bins + 1]. */
+int mxq_calibrate_entropy(const float* hist, const float* hist_edges, size_t num_bins,
+                          int num_quantized_bins, float* out_threshold, float* out_divergence);
+
 #ifdef __cplusplus
 }
 #endif

@@ -76,7 +76,8 @@ def build_probe(verbose=False):
 
 
 OPS_LIB = os.path.join(HERE, "libmxq_ops.so")
-HOST_SOURCES = ["mxq_registry.cc", "mxq_quantization_ops.cc", "mxq_harness.cc"]
+HOST_SOURCES = ["mxq_registry.cc", "mxq_quantization_ops.cc", "mxq_float_ops.cc", "mxq_graph.cc",
+                "mxq_quantize_graph_pass.cc", "mxq_calibrate.cc", "mxq_harness.cc"]
 
 
 def build_ops(verbose=False):
@@ -84,7 +85,7 @@ def build_ops(verbose=False):
     C++17, no HIP headers: it reaches the GPU only through libmxq_hip.so's C ABI."""
     cxx = os.environ.get("CXX", "g++")
     srcs = [os.path.join(CSRC, "host", s) for s in HOST_SOURCES]
-    cmd = [cxx, "-O2", "-std=c++17", "-fPIC", "-shared", "-Wall", "-Wextra",
+    cmd = [cxx, "-O2", "-std=c++17", "-fPIC", "-shared", "-ffp-contract=off", "-Wall", "-Wextra",
            "-Wno-unused-parameter", "-o", OPS_LIB] + srcs + \
           ["-L" + HERE, "-lmxq_hip", "-Wl,-rpath,$ORIGIN"]
     if verbose:

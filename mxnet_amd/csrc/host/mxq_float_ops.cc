@@ -1,0 +1,185 @@
+// Graph-level registrations of the float operators the quantization pass looks at: no
+// compute functions, only what the pass asks the registry (argument and output names,
+// output counts, FQuantizable, FQuantizedOp).  Each block cites the registration it
+// restates in the reference.
+#include <string>
+#include <vector>
+
+#include "mxq_params.h"
+#include "mxq_shim.h"
+
+namespace mxnet {
+namespace op {
+
+namespace {
+
+std::vector<std::string> OneOutput(const NodeAttrs&) { return {"output"}; }
+std::vector<std::string> DataOnly(const NodeAttrs&) { return {"data"}; }
+
+// The common body of the FQuantizedOp functions: same attribute dict under the
+// quantized operator, named "quantized_<name>" (e.g. quantized_conv.cc:242-251).
+nnvm::ObjectPtr QuantizedTwin(const NodeAttrs& attrs, const char* quantized_op) {
+  nnvm::ObjectPtr node = nnvm::Node::Create();
+  node->attrs.op = nnvm::Op::Get(quantized_op);
+  node->attrs.name = "quantized_" + attrs.name;
+  node->attrs.dict = attrs.dict;
+  if (node->op()->attr_parser) node->op()->attr_parser(&(node->attrs));
+  return node;
+}
+
+// A float node that stays as it is: no operator on the returned node tells the pass so
+// (quantized_activation.cc:128-133).
+nnvm::ObjectPtr NotQuantized(const NodeAttrs& attrs) {
+  nnvm::ObjectPtr node = nnvm::Node::Create();
+  node->attrs.op = nullptr;
+  node->attrs.name = attrs.name;
+  node->attrs.dict = attrs.dict;
+  return node;
+}
+
+}  // namespace
+
+// src/operator/nn/convolution.cc:435-548, quantized_conv.cc:239-251
+NNVM_REGISTER_OP(Convolution)
+    .set_num_inputs([](const NodeAttrs& attrs) {
+      return nnvm::get<ConvolutionParam>(attrs.parsed).no_bias ? 2U : 3U;
+    })
+    .set_num_outputs(1)
+    .set_attr_parser(ConvolutionParamParser)
+    .set_attr<nnvm::FListInputNames>("FListInputNames",
+                                     [](const NodeAttrs& attrs) {
+                                       if (nnvm::get<ConvolutionParam>(attrs.parsed).no_bias)
+                                         return std::vector<std::string>{"data", "weight"};
+                                       return std::vector<std::string>{"data", "weight", "bias"};
+                                     })
+    .set_attr<nnvm::FListOutputNames>("FListOutputNames", OneOutput)
+    .set_attr<FQuantizable>("FQuantizable",
+                            [](const NodeAttrs&) { return QuantizeType::kMust; })
+    .set_attr<FQuantizedOp>("FQuantizedOp", [](const NodeAttrs& attrs) {
+      return QuantizedTwin(attrs, "_contrib_quantized_conv");
+    });
+
+// src/operator/nn/fully_connected.cc:255-326, quantized_fully_connected.cc:384-396
+NNVM_REGISTER_OP(FullyConnected)
+    .set_num_inputs([](const NodeAttrs& attrs) {
+      return nnvm::get<FullyConnectedParam>(attrs.parsed).no_bias ? 2U : 3U;
+    })
+    .set_num_outputs(1)
+    .set_attr_parser(ParamParser<FullyConnectedParam>)
+    .set_attr<nnvm::FListInputNames>("FListInputNames",
+                                     [](const NodeAttrs& attrs) {
+                                       if (nnvm::get<FullyConnectedParam>(attrs.parsed).no_bias)
+                                         return std::vector<std::string>{"data", "weight"};
+                                       return std::vector<std::string>{"data", "weight", "bias"};
+                                     })
+    .set_attr<nnvm::FListOutputNames>("FListOutputNames", OneOutput)
+    .set_attr<FQuantizable>("FQuantizable",
+                            [](const NodeAttrs&) { return QuantizeType::kMust; })
+    .set_attr<FQuantizedOp>("FQuantizedOp", [](const NodeAttrs& attrs) {
+      return QuantizedTwin(attrs, "_contrib_quantized_fully_connected");
+    });
+
+// src/operator/nn/activation.cc:157-193, quantized_activation.cc:122-140: relu only
+NNVM_REGISTER_OP(Activation)
+    .set_num_inputs(1)
+    .set_num_outputs(1)
+    .set_attr_parser(ParamParser<ActivationParam>)
+    .set_attr<nnvm::FListInputNames>("FListInputNames", DataOnly)
+    .set_attr<nnvm::FListOutputNames>("FListOutputNames", OneOutput)
+    .set_attr<FQuantizedOp>("FQuantizedOp", [](const NodeAttrs& attrs) {
+      const ActivationParam& param = nnvm::get<ActivationParam>(attrs.parsed);
+      if (param.act_type == activation::kReLU) return QuantizedTwin(attrs, "_contrib_quantized_act");
+      return NotQuantized(attrs);
+    });
+
+// src/operator/nn/pooling.cc:358-446, quantized_pooling.cc:218-236: max and avg only.
+// (For sum / lp pooling the reference hands back a node that still carries the float
+// Pooling operator; here such a node is simply left alone.)
+NNVM_REGISTER_OP(Pooling)
+    .set_num_inputs(1)
+    .set_num_outputs(1)
+    .set_attr_parser(PoolingParamParser)
+    .set_attr<nnvm::FListInputNames>("FListInputNames", DataOnly)
+    .set_attr<nnvm::FListOutputNames>("FListOutputNames", OneOutput)
+    .set_attr<FQuantizedOp>("FQuantizedOp", [](const NodeAttrs& attrs) {
+      PoolingParam param;
+      param.Init(attrs.dict);
+      if (param.pool_type == pool_enum::kMaxPooling || param.pool_type == pool_enum::kAvgPooling)
+        return QuantizedTwin(attrs, "_contrib_quantized_pooling");
+      return NotQuantized(attrs);
+    });
+
+// src/operator/tensor/matrix_op.cc:256-290 (no argument or output names registered),
+// quantized_flatten.cc:65-74
+NNVM_REGISTER_OP(Flatten)
+    .add_alias("flatten")
+    .set_num_inputs(1)
+    .set_num_outputs(1)
+    .set_attr<FQuantizedOp>("FQuantizedOp", [](const NodeAttrs& attrs) {
+      return QuantizedTwin(attrs, "_contrib_quantized_flatten");
+    });
+
+// Float operators that are never quantized here but whose output names the pass spells
+// into node and calibration names.
+// src/operator/nn/batch_norm.cc:571-640
+NNVM_REGISTER_OP(BatchNorm)
+    .set_num_inputs(5)
+    .set_num_outputs(3)
+    .set_attr<nnvm::FListInputNames>("FListInputNames",
+                                     [](const NodeAttrs&) {
+                                       return std::vector<std::string>{"data", "gamma", "beta",
+                                                                       "moving_mean",
+                                                                       "moving_var"};
+                                     })
+    .set_attr<nnvm::FListOutputNames>("FListOutputNames",
+                                      [](const NodeAttrs&) {
+                                        return std::vector<std::string>{"output", "mean", "var"};
+                                      })
+    .set_attr<nnvm::FNumVisibleOutputs>("FNumVisibleOutputs",
+                                        [](const NodeAttrs&) { return 1U; });
+
+// src/operator/nn/softmax.cc:108-160
+NNVM_REGISTER_OP(softmax)
+    .set_num_inputs(1)
+    .set_num_outputs(1)
+    .set_attr<nnvm::FListInputNames>("FListInputNames", DataOnly)
+    .set_attr<nnvm::FListOutputNames>("FListOutputNames", OneOutput);
+
+// src/operator/softmax_output.cc:166-272
+NNVM_REGISTER_OP(SoftmaxOutput)
+    .add_alias("Softmax")
+    .set_num_inputs(2)
+    .set_num_outputs(1)
+    .set_attr<nnvm::FListInputNames>("FListInputNames",
+                                     [](const NodeAttrs&) {
+                                       return std::vector<std::string>{"data", "label"};
+                                     })
+    .set_attr<nnvm::FListOutputNames>("FListOutputNames", OneOutput);
+
+// src/operator/nn/dropout.cc:64-110
+NNVM_REGISTER_OP(Dropout)
+    .set_num_inputs(1)
+    .set_num_outputs(2)
+    .set_attr<nnvm::FListInputNames>("FListInputNames", DataOnly)
+    .set_attr<nnvm::FListOutputNames>("FListOutputNames",
+                                      [](const NodeAttrs&) {
+                                        return std::vector<std::string>{"output", "mask"};
+                                      })
+    .set_attr<nnvm::FNumVisibleOutputs>("FNumVisibleOutputs",
+                                        [](const NodeAttrs&) { return 1U; });
+
+// src/operator/tensor/elemwise_binary_op_basic.cc:85-110 (quantized only by oneDNN in
+// the reference, quantized_elemwise_add.cc:130)
+NNVM_REGISTER_OP(elemwise_add)
+    .add_alias("_add")
+    .add_alias("_plus")
+    .set_num_inputs(2)
+    .set_num_outputs(1)
+    .set_attr<nnvm::FListInputNames>("FListInputNames",
+                                     [](const NodeAttrs&) {
+                                       return std::vector<std::string>{"lhs", "rhs"};
+                                     })
+    .set_attr<nnvm::FListOutputNames>("FListOutputNames", OneOutput);
+
+}  // namespace op
+}  // namespace mxnet

@@ -7,6 +7,7 @@
 #include <vector>
 
 #include "../../../include/mxq_ops.h"
+#include "mxq_graph_pass.h"
 #include "mxq_shim.h"
 
 namespace mxnet {
@@ -108,7 +109,8 @@ int mxq_node_num_inputs(void* node, int* out) {
 
 int mxq_node_num_outputs(void* node, int* out) {
   OPS_API_BEGIN();
-  *out = static_cast<int>(static_cast<Node*>(node)->attrs.op->num_outputs);
+  Node* n = static_cast<Node*>(node);
+  *out = static_cast<int>(n->attrs.op->NumOutputs(n->attrs));
   OPS_API_END();
 }
 
@@ -223,6 +225,72 @@ int mxq_node_forward(void* node, void* stream, int dev_id, int num_in, const mxq
     return 0;
   }
   throw dmlc::Error("Operator " + op->name + " is not implemented for GPU.");
+  OPS_API_END();
+}
+
+
+namespace {
+thread_local std::string tl_json;
+thread_local std::vector<std::string> tl_names;
+thread_local std::vector<const char*> tl_name_ptrs;
+}  // namespace
+
+int mxq_quantize_symbol(const char* symbol_json, int dev_type, int num_excluded_nodes,
+                        const char** excluded_nodes, int num_excluded_ops,
+                        const char** excluded_ops, int num_offline, const char** offline_params,
+                        const char* quantized_dtype, const char* quantize_mode,
+                        const char* quantize_granularity, const char** out_symbol_json,
+                        int* out_num_calib_names, const char*** out_calib_names) {
+  OPS_API_BEGIN();
+  CHECK(symbol_json && quantized_dtype && quantize_mode && quantize_granularity &&
+        out_symbol_json && out_num_calib_names && out_calib_names)
+      << "null argument";
+  mxq_graph::QuantizeOptions opt;
+  for (int i = 0; i < num_excluded_nodes; ++i) opt.excluded_nodes.insert(excluded_nodes[i]);
+  for (int i = 0; i < num_excluded_ops; ++i) opt.excluded_ops.insert(excluded_ops[i]);
+  for (int i = 0; i < num_offline; ++i) opt.offline_params.insert(offline_params[i]);
+  opt.quantized_dtype = quantized_dtype;
+  opt.quantize_mode = quantize_mode;
+  opt.quantize_granularity = quantize_granularity;
+  opt.dev_type = dev_type;
+  mxq_graph::QuantizeResult r = mxq_graph::QuantizeGraph(mxq_graph::LoadJSON(symbol_json), opt);
+  tl_json = mxq_graph::SaveJSON(r.graph);
+  tl_names = r.calib_nodes;
+  tl_name_ptrs.clear();
+  for (const std::string& n : tl_names) tl_name_ptrs.push_back(n.c_str());
+  *out_symbol_json = tl_json.c_str();
+  *out_num_calib_names = static_cast<int>(tl_names.size());
+  *out_calib_names = tl_name_ptrs.data();
+  OPS_API_END();
+}
+
+int mxq_set_calib_table(const char* qsymbol_json, int num_layers, const char** layer_names,
+                        const float* min_ranges, const float* max_ranges,
+                        const char** out_symbol_json) {
+  OPS_API_BEGIN();
+  CHECK(qsymbol_json && out_symbol_json) << "null argument";
+  std::map<std::string, std::pair<float, float>> table;
+  for (int i = 0; i < num_layers; ++i)
+    table.emplace(layer_names[i], std::make_pair(min_ranges[i], max_ranges[i]));
+  tl_json = mxq_graph::SaveJSON(mxq_graph::SetCalibTable(mxq_graph::LoadJSON(qsymbol_json), table));
+  *out_symbol_json = tl_json.c_str();
+  OPS_API_END();
+}
+
+int mxq_symbol_normalize(const char* symbol_json, const char** out_symbol_json) {
+  OPS_API_BEGIN();
+  CHECK(symbol_json && out_symbol_json) << "null argument";
+  tl_json = mxq_graph::SaveJSON(mxq_graph::LoadJSON(symbol_json));
+  *out_symbol_json = tl_json.c_str();
+  OPS_API_END();
+}
+
+int mxq_calibrate_entropy(const float* hist, const float* hist_edges, size_t num_bins,
+                          int num_quantized_bins, float* out_threshold, float* out_divergence) {
+  OPS_API_BEGIN();
+  CHECK(hist && hist_edges && out_threshold && out_divergence) << "null argument";
+  mxq_graph::CalibrateEntropy(hist, hist_edges, num_bins, num_quantized_bins, out_threshold,
+                              out_divergence);
   OPS_API_END();
 }
 

@@ -51,6 +51,13 @@ const Op* Op::Get(const std::string& name) {
   return it->second;
 }
 
+const Op* Op::Find(const std::string& name) {
+  Registry& r = Registry::Get();
+  std::lock_guard<std::mutex> lk(r.mu);
+  auto it = r.by_name.find(name);
+  return it == r.by_name.end() ? nullptr : it->second;
+}
+
 std::vector<std::string> Op::ListAllNames() {
   Registry& r = Registry::Get();
   std::lock_guard<std::mutex> lk(r.mu);

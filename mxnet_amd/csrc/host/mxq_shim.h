@@ -363,11 +363,20 @@ class Op {
     AttrTable()[key][this] = std::any(value);
     return *this;
   }
+  Op& set_num_outputs(std::function<uint32_t(const NodeAttrs&)> fn) {
+    get_num_outputs = fn;
+    return *this;
+  }
   uint32_t NumInputs(const NodeAttrs& attrs) const {
     return get_num_inputs ? get_num_inputs(attrs) : num_inputs;
   }
+  uint32_t NumOutputs(const NodeAttrs& attrs) const {
+    return get_num_outputs ? get_num_outputs(attrs) : num_outputs;
+  }
+  std::function<uint32_t(const NodeAttrs&)> get_num_outputs;
 
-  static const Op* Get(const std::string& name);
+  static const Op* Get(const std::string& name);   // throws when the name is unknown
+  static const Op* Find(const std::string& name);  // nullptr when the name is unknown
   static Op& RegisterOrGet(const std::string& name);
   static std::vector<std::string> ListAllNames();
   template <typename ValueType>
@@ -387,6 +396,16 @@ typedef std::function<std::vector<std::string>(const NodeAttrs&)> FListOutputNam
 typedef std::function<bool(const NodeAttrs&, std::vector<int>*, std::vector<int>*)> FInferType;
 typedef std::function<std::vector<std::pair<int, int>>(const NodeAttrs&)> FInplaceOption;
 typedef std::function<std::vector<bool>(const NodeAttrs&)> FInplaceIdentity;
+typedef std::function<uint32_t(const NodeAttrs&)> FNumVisibleOutputs;
+
+// What FQuantizedOp hands back in the reference is a graph node; only its attributes
+// (operator, name, dict, parsed struct) are ever looked at.
+struct Node {
+  NodeAttrs attrs;
+  const Op* op() const { return attrs.op; }
+  static std::shared_ptr<Node> Create() { return std::make_shared<Node>(); }
+};
+typedef std::shared_ptr<Node> ObjectPtr;
 
 }  // namespace nnvm
 
@@ -417,6 +436,12 @@ typedef std::function<std::vector<ResourceRequest>(const NodeAttrs&)> FResourceR
 typedef std::function<bool(const NodeAttrs&)> FNeedRequantize;
 typedef std::function<std::vector<int>(const NodeAttrs&)> FNeedCalibrateInput;
 typedef std::function<std::vector<int>(const NodeAttrs&)> FNeedCalibrateOutput;
+// include/mxnet/op_attr_types.h:134-142, 318-357
+enum class QuantizeType { kNone = 0, kMust, kSupport };
+typedef std::function<QuantizeType(const NodeAttrs&)> FQuantizable;
+typedef std::function<nnvm::ObjectPtr(const NodeAttrs&)> FQuantizedOp;
+typedef std::function<bool(const NodeAttrs&, const size_t, const std::string)> FAvoidQuantizeInput;
+typedef std::function<bool(const NodeAttrs&, const size_t)> FAvoidDequantizeOutput;
 
 namespace op {
 

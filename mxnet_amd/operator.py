@@ -46,6 +46,15 @@ OPS_SIGNATURES = {
     "mxq_node_infer_type": (_i, [_p, _i, _pi, _i, _pi]),
     "mxq_node_temp_bytes": (_i, [_p, _i, _pb, _i, _pb, ctypes.POINTER(_sz)]),
     "mxq_node_forward": (_i, [_p, _p, _i, _i, _pb, _i, _pb, _p, _sz]),
+    "mxq_quantize_symbol": (_i, [ctypes.c_char_p, _i, _i, _pps, _i, _pps, _i, _pps,
+                                 ctypes.c_char_p, ctypes.c_char_p, ctypes.c_char_p, _pps, _pi,
+                                 ctypes.POINTER(_pps)]),
+    "mxq_set_calib_table": (_i, [ctypes.c_char_p, _i, _pps, ctypes.POINTER(ctypes.c_float),
+                                 ctypes.POINTER(ctypes.c_float), _pps]),
+    "mxq_symbol_normalize": (_i, [ctypes.c_char_p, _pps]),
+    "mxq_calibrate_entropy": (_i, [ctypes.POINTER(ctypes.c_float), ctypes.POINTER(ctypes.c_float),
+                                   _sz, _i, ctypes.POINTER(ctypes.c_float),
+                                   ctypes.POINTER(ctypes.c_float)]),
 }
 for _name, (_res, _args) in OPS_SIGNATURES.items():
     _fn = getattr(ops, _name)

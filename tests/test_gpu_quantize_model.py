@@ -1,0 +1,126 @@
+"""quantize_model end to end on the GPU: float symbol + parameters -> calibrated int8
+symbol + offline-quantized parameters -> executed through the registered operators.
+Follows the reference's test_quantize_model (tests/python/quantization/test_quantization.py
+:1172-1312: parameter names and types of the quantized model, calibration attributes on the
+requantize nodes) and adds what the reference cannot check without a model zoo: the int8
+network's output against the float network's, and the quantized prefix of the graph against
+the CPU oracle, bit for bit."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+
+pytestmark = pytest.mark.gpu
+
+
+def build():
+    from mxnet_amd import symbol as S
+    data = S.Variable("data")
+    conv = S.Convolution(data, kernel=(3, 3), pad=(1, 1), num_filter=16, name="conv")
+    bn = S.BatchNorm(data=conv, eps=2e-05, fix_gamma=False, momentum=0.9,
+                     use_global_stats=False, name="bn")
+    act = S.Activation(data=bn, act_type="relu", name="relu")
+    pool = S.Pooling(act, kernel=(4, 4), stride=(4, 4), pool_type="avg", name="pool")
+    flat = S.Flatten(pool, name="flat")
+    fc = S.FullyConnected(flat, num_hidden=10, flatten=True, name="fc")
+    return S.softmax(fc, name="softmax")
+
+
+def params(rng):
+    arg = {"conv_weight": rng.normal(0, 0.2, (16, 4, 3, 3)), "conv_bias": rng.normal(0, 0.1, 16),
+           "bn_gamma": rng.uniform(0.5, 1.5, 16), "bn_beta": rng.normal(0, 0.1, 16),
+           "fc_weight": rng.normal(0, 0.1, (10, 16 * 2 * 2)), "fc_bias": rng.normal(0, 0.1, 10)}
+    aux = {"bn_moving_mean": rng.normal(0, 0.1, 16), "bn_moving_var": rng.uniform(0.5, 1.5, 16)}
+    f = lambda d: {k: torch.tensor(v, dtype=torch.float32) for k, v in d.items()}
+    return f(arg), f(aux)
+
+
+@pytest.mark.parametrize("calib_mode", ["naive", "entropy"])
+@pytest.mark.parametrize("quantize_mode", ["full", "smart"])
+def test_quantize_model_runs_and_tracks_the_float_network(calib_mode, quantize_mode):
+    from mxnet_amd import quantization as Q
+    from mxnet_amd.executor import Executor
+    rng = np.random.default_rng(0)
+    sym = build()
+    arg, aux = params(rng)
+    calib = [torch.tensor(rng.normal(0, 1, (16, 4, 8, 8)), dtype=torch.float32) for _ in range(3)]
+    qsym, qarg, qaux = Q.quantize_model(sym, arg, aux, calib_mode=calib_mode, calib_data=calib,
+                                        num_calib_batches=3, quantize_mode=quantize_mode)
+    # parameters: int8 weights and biases with fp32 (1,) ranges; float ones untouched
+    for name in ["conv_weight_quantize", "conv_bias_quantize", "fc_weight_quantize",
+                 "fc_bias_quantize"]:
+        assert qarg[name].dtype == torch.int8
+        assert qarg[name + "_min"].shape == (1,) and qarg[name + "_min"].dtype == torch.float32
+        assert qarg[name + "_min"].item() == -qarg[name + "_max"].item()
+    assert qarg["conv_weight_quantize"].shape == (16, 4, 3, 3)
+    assert torch.equal(qarg["bn_gamma"], arg["bn_gamma"]) and "conv_weight" not in qarg
+    assert set(qsym.list_arguments()) - {"data"} == set(qarg.keys())
+    # every requantize / quantize node got its calibrated range
+    attrs = qsym.attr_dict()
+    calibrated = [n for n in attrs if n.startswith("requantize_") or n.endswith("_quantize")]
+    assert "requantize_conv" in calibrated and "requantize_fc" in calibrated
+    for n in calibrated:
+        assert "min_calib_range" in attrs[n] and "max_calib_range" in attrs[n]
+        assert float(attrs[n]["min_calib_range"]) < float(attrs[n]["max_calib_range"])
+    # the offline weights are exactly the oracle's v1 quantize of the float weights
+    w = arg["conv_weight"].numpy()
+    ref, rmin, rmax = oracle.quantize(w, w.min(), w.max(), "int8")
+    np.testing.assert_array_equal(qarg["conv_weight_quantize"].cpu().numpy(), ref)
+    assert qarg["conv_weight_quantize_max"].item() == rmax
+    # run both networks on fresh data
+    x = torch.tensor(rng.normal(0, 1, (32, 4, 8, 8)), dtype=torch.float32)
+    fp = Executor(sym, {**arg, **aux}).forward(data=x)[0]
+    q = Executor(qsym, {**qarg, **qaux}).forward(data=x)[0]
+    assert q.shape == fp.shape == (32, 10) and q.dtype == torch.float32
+    err = (q - fp).abs().max().item()
+    assert err < 0.06, err
+    assert (q.argmax(1) == fp.argmax(1)).float().mean().item() >= 0.85
+
+
+def test_quantized_prefix_matches_the_oracle_bit_for_bit():
+    """data -> quantize_v2 -> quantized_conv -> requantize -> dequantize against the
+    oracle's functions with the same calibrated attributes."""
+    from mxnet_amd import quantization as Q
+    from mxnet_amd.executor import Executor
+    rng = np.random.default_rng(1)
+    sym = build()
+    arg, aux = params(rng)
+    calib = [torch.tensor(rng.normal(0, 1, (8, 4, 8, 8)), dtype=torch.float32)]
+    qsym, qarg, qaux = Q.quantize_model(sym, arg, aux, calib_mode="naive", calib_data=calib,
+                                        quantize_mode="full")
+    internals = qsym.get_internals()
+    head = internals["conv_dequantize_output"]
+    x = rng.normal(0, 1, (5, 4, 8, 8)).astype(np.float32)
+    got = Executor(head, {**qarg, **qaux}).forward(data=torch.from_numpy(x))[0].cpu().numpy()
+    attrs = qsym.attr_dict()
+    a = attrs["conv_data_quantize"]
+    qd, dmin, dmax = oracle.quantize_v2(x, "int8", float(a["min_calib_range"]),
+                                        float(a["max_calib_range"]))
+    wq = qarg["conv_weight_quantize"].cpu().numpy()
+    bq = qarg["conv_bias_quantize"].cpu().numpy()
+    acc, omin, omax = oracle.quantized_conv(
+        qd, wq, bq, dmin, dmax, qarg["conv_weight_quantize_min"].item(),
+        qarg["conv_weight_quantize_max"].item(), qarg["conv_bias_quantize_min"].item(),
+        qarg["conv_bias_quantize_max"].item(), stride=(1, 1), pad=(1, 1))
+    r = attrs["requantize_conv"]
+    q8, rmin, rmax = oracle.requantize(acc, omin, omax, float(r["min_calib_range"]),
+                                       float(r["max_calib_range"]))
+    want = oracle.dequantize(q8, rmin, rmax)
+    np.testing.assert_array_equal(got, want)
+
+
+def test_calibration_sees_every_requested_tensor():
+    from mxnet_amd import quantization as Q
+    from mxnet_amd.executor import Executor
+    rng = np.random.default_rng(2)
+    sym = build()
+    arg, aux = params(rng)
+    qsym, calib_layers = Q._quantize_symbol(sym, "gpu", offline_params=list(arg.keys()),
+                                            quantize_mode="full")
+    seen = []
+    ex = Executor(sym, {**arg, **aux})
+    ex.register_op_hook(lambda name, op, arr: seen.append(name), monitor_all=True)
+    ex.forward(data=torch.tensor(rng.normal(0, 1, (2, 4, 8, 8)), dtype=torch.float32))
+    assert set(calib_layers) <= set(seen)
+    assert "conv_data" in seen and "conv_output" in seen and "bn_output" in seen

@@ -1,0 +1,339 @@
+"""The QuantizeGraph / SetCalibTable passes, the symbol JSON reader/writer and entropy
+calibration on the CPU (no kernel runs).  Expectations come from the reference's pass
+(src/operator/quantization/quantize_graph_pass.cc) worked by hand on small graphs and from
+its own tests (tests/python/quantization/test_quantization.py:1092-1115 test_quantize_params,
+:1365-1399 test_quantize_sym_with_calib, :1451-1493 the optimal-threshold tests)."""
+import json
+
+import numpy as np
+import pytest
+
+from mxnet_amd import quantization as Q
+from mxnet_amd import symbol as S
+from mxnet_amd.operator import MXNetError
+
+
+def fp32_sym():
+    # get_fp32_sym of test_quantize_sym_with_calib
+    data = S.Variable("data")
+    conv = S.Convolution(data, kernel=(1, 1), num_filter=16, name="conv")
+    bn = S.BatchNorm(data=conv, eps=2e-05, fix_gamma=False, momentum=0.9,
+                     use_global_stats=False, name="bn")
+    act = S.Activation(data=bn, act_type="relu", name="relu")
+    pool = S.Pooling(act, kernel=(4, 4), pool_type="avg", name="pool")
+    fc = S.FullyConnected(pool, num_hidden=10, flatten=True, name="fc")
+    return S.softmax(fc, name="softmax")
+
+
+def offline_of(sym):
+    return [n for n in sym.list_arguments() if not n.startswith("data") and not n.endswith("label")]
+
+
+def ops_of(sym):
+    return [(op, name) for op, name, _, _ in sym.nodes() if op != "null"]
+
+
+def node(sym, name):
+    nodes = sym.nodes()
+    for op, n, attrs, inputs in nodes:
+        if n == name:
+            return op, attrs, [(nodes[j][1], k) for j, k in inputs]
+    raise KeyError(name)
+
+
+def test_symbol_composition_and_json_round_trip():
+    sym = fp32_sym()
+    assert sym.list_arguments() == ["data", "conv_weight", "conv_bias", "bn_gamma", "bn_beta",
+                                    "fc_weight", "fc_bias"]
+    assert sym.list_auxiliary_states() == ["bn_moving_mean", "bn_moving_var"]
+    assert sym.list_outputs() == ["softmax_output"]
+    text = sym.tojson()
+    g = json.loads(text)
+    assert [n["name"] for n in g["nodes"]][:4] == ["data", "conv_weight", "conv_bias", "conv"]
+    assert g["nodes"][3]["attrs"] == {"kernel": "(1, 1)", "num_filter": "16"}
+    assert g["nodes"][3]["inputs"] == [[0, 0, 0], [1, 0, 0], [2, 0, 0]]
+    assert g["arg_nodes"] == [i for i, n in enumerate(g["nodes"]) if n["op"] == "null"]
+    # BatchNorm has three outputs: node_row_ptr advances by 3 over it
+    bn = [n["name"] for n in g["nodes"]].index("bn")
+    assert g["node_row_ptr"][bn + 1] - g["node_row_ptr"][bn] == 3
+    assert g["heads"] == [[len(g["nodes"]) - 1, 0, 0]]
+    assert S.Symbol.fromjson(text).tojson() == text
+    # files written by old versions keep attributes under "param" / "attr"
+    old = json.loads(text)
+    for n in old["nodes"]:
+        if "attrs" in n:
+            n["param"] = n.pop("attrs")
+    assert S.Symbol.fromjson(json.dumps(old)).tojson() == text
+    with pytest.raises(MXNetError, match="symbol JSON"):
+        S.Symbol.fromjson('{"nodes": [], "heads": [[3, 0, 0]]}').tojson()
+
+
+def test_quantize_full_mode_graph():
+    sym = fp32_sym()
+    qsym, calib = Q._quantize_symbol(sym, "gpu", offline_params=offline_of(sym),
+                                     quantize_mode="full")
+    assert ops_of(qsym) == [
+        ("_contrib_quantize_v2", "conv_data_quantize"),
+        ("_contrib_quantized_conv", "quantized_conv"),
+        ("_contrib_requantize", "requantize_conv"),
+        ("_contrib_dequantize", "conv_dequantize"),
+        ("BatchNorm", "bn"),
+        ("_contrib_quantize_v2", "bn_output_quantize"),
+        ("_contrib_quantized_act", "quantized_relu"),
+        ("_contrib_quantized_pooling", "quantized_pool"),
+        ("_contrib_quantized_fully_connected", "quantized_fc"),
+        ("_contrib_requantize", "requantize_fc"),
+        ("_contrib_dequantize", "fc_dequantize"),
+        ("softmax", "softmax")]
+    # data inputs first, then (min, max) per input in input order
+    op, attrs, inputs = node(qsym, "quantized_conv")
+    assert attrs == {"kernel": "(1, 1)", "num_filter": "16"}
+    assert inputs == [("conv_data_quantize", 0), ("conv_weight_quantize", 0),
+                      ("conv_bias_quantize", 0), ("conv_data_quantize", 1),
+                      ("conv_data_quantize", 2), ("conv_weight_quantize_min", 0),
+                      ("conv_weight_quantize_max", 0), ("conv_bias_quantize_min", 0),
+                      ("conv_bias_quantize_max", 0)]
+    assert node(qsym, "requantize_conv")[1:] == ({"out_type": "int8"},
+                                                 [("quantized_conv", 0), ("quantized_conv", 1),
+                                                  ("quantized_conv", 2)])
+    assert node(qsym, "conv_dequantize")[2] == [("requantize_conv", 0), ("requantize_conv", 1),
+                                                ("requantize_conv", 2)]
+    assert node(qsym, "bn")[2][0] == ("conv_dequantize", 0)
+    # int8 flows from relu through pooling into the FC without leaving int8
+    assert node(qsym, "quantized_relu")[2] == [("bn_output_quantize", 0),
+                                               ("bn_output_quantize", 1),
+                                               ("bn_output_quantize", 2)]
+    assert node(qsym, "quantized_pool")[2] == [("quantized_relu", 0), ("quantized_relu", 1),
+                                               ("quantized_relu", 2)]
+    assert node(qsym, "quantized_fc")[2][:5] == [("quantized_pool", 0), ("fc_weight_quantize", 0),
+                                                 ("fc_bias_quantize", 0), ("quantized_pool", 1),
+                                                 ("quantized_pool", 2)]
+    assert node(qsym, "softmax")[2] == [("fc_dequantize", 0)]
+    assert calib == ["conv_data", "conv_output", "bn_output", "fc_output"]
+    assert qsym.list_outputs() == ["softmax_output"]
+
+
+def test_quantize_smart_mode_keeps_isolated_supporting_ops_float():
+    sym = fp32_sym()
+    qsym, calib = Q._quantize_symbol(sym, "gpu", offline_params=offline_of(sym),
+                                     quantize_mode="smart")
+    names = [n for _, n in ops_of(qsym)]
+    # relu and pool sit between a float BatchNorm and the FC: int8 does not reach them
+    # from a must-quantize producer, so they stay float
+    assert names == ["conv_data_quantize", "quantized_conv", "requantize_conv",
+                     "conv_dequantize", "bn", "relu", "pool", "pool_output_quantize",
+                     "quantized_fc", "requantize_fc", "fc_dequantize", "softmax"]
+    assert calib == ["conv_data", "conv_output", "pool_output", "fc_output"]
+    # conv -> relu -> conv: the relu is between two must-quantize nodes and goes int8
+    d = S.Variable("data")
+    c1 = S.Convolution(d, kernel=(3, 3), num_filter=8, name="c1")
+    r = S.Activation(c1, act_type="relu", name="r")
+    c2 = S.Convolution(r, kernel=(3, 3), num_filter=8, name="c2")
+    q2, calib2 = Q._quantize_symbol(c2, "gpu", offline_params=offline_of(c2),
+                                    quantize_mode="smart")
+    assert [n for _, n in ops_of(q2)] == ["c1_data_quantize", "quantized_c1", "requantize_c1",
+                                          "quantized_r", "quantized_c2", "requantize_c2",
+                                          "c2_dequantize"]
+    assert node(q2, "quantized_c2")[2][0] == ("quantized_r", 0)
+    assert node(q2, "quantized_c2")[2][3:5] == [("quantized_r", 1), ("quantized_r", 2)]
+    assert calib2 == ["c1_data", "c1_output", "c2_output"]
+    assert q2.list_outputs() == ["c2_dequantize_output"]
+    with pytest.raises(MXNetError, match="unrecognized quantize mode"):
+        Q._quantize_symbol(c2, "gpu", quantize_mode="clever")
+
+
+def test_exclusions_and_device():
+    sym = fp32_sym()
+    off = offline_of(sym)
+    # the reference's GPU build has no quantized relu / flatten kernels; excluding the
+    # float operators reproduces its graph
+    qsym, calib = Q._quantize_symbol(sym, "gpu", offline_params=off, quantize_mode="full",
+                                     excluded_operators=["Activation", "Flatten"])
+    assert [n for _, n in ops_of(qsym)] == [
+        "conv_data_quantize", "quantized_conv", "requantize_conv", "conv_dequantize", "bn",
+        "relu", "relu_output_quantize", "quantized_pool", "quantized_fc", "requantize_fc",
+        "fc_dequantize", "softmax"]
+    assert calib == ["conv_data", "conv_output", "relu_output", "fc_output"]
+    qsym, _ = Q._quantize_symbol(sym, "gpu", offline_params=off, quantize_mode="full",
+                                 excluded_symbols=["conv"])
+    assert ("Convolution", "conv") in ops_of(qsym)
+    assert "conv_weight" in qsym.list_arguments()
+    # no quantized operator has a cpu kernel in this build: nothing is replaced
+    qsym, calib = Q._quantize_symbol(sym, "cpu", offline_params=off, quantize_mode="full")
+    assert ops_of(qsym) == ops_of(sym) and calib == []
+    # non-relu activations and sum pooling have no quantized counterpart
+    d = S.Variable("data")
+    t = S.Activation(S.Convolution(d, kernel=(1, 1), num_filter=4, name="c"), act_type="tanh",
+                     name="t")
+    qsym, _ = Q._quantize_symbol(t, "gpu", quantize_mode="full")
+    assert ops_of(qsym)[-2:] == [("_contrib_dequantize", "c_dequantize"), ("Activation", "t")]
+    with pytest.raises(MXNetError, match="channel-wise"):
+        Q._quantize_symbol(sym, "gpu", quantize_granularity="channel-wise")
+
+
+def test_weights_quantized_online_when_not_offline():
+    d = S.Variable("data")
+    fc = S.FullyConnected(d, num_hidden=4, no_bias=True, name="fc")
+    qsym, calib = Q._quantize_symbol(fc, "gpu", quantize_mode="full")
+    assert [n for _, n in ops_of(qsym)] == ["fc_data_quantize", "fc_weight_quantize",
+                                            "quantized_fc", "requantize_fc", "fc_dequantize"]
+    assert node(qsym, "fc_weight_quantize")[2] == [("fc_weight", 0)]
+    assert node(qsym, "quantized_fc")[2] == [("fc_data_quantize", 0), ("fc_weight_quantize", 0),
+                                             ("fc_data_quantize", 1), ("fc_data_quantize", 2),
+                                             ("fc_weight_quantize", 1), ("fc_weight_quantize", 2)]
+    assert calib == ["fc_data", "fc_weight", "fc_output"]
+
+
+def test_shared_float_producer_gets_one_quantize_node():
+    d = S.Variable("data")
+    bn = S.BatchNorm(d, name="bn")
+    a = S.FullyConnected(bn, num_hidden=4, no_bias=True, name="a")
+    b = S.FullyConnected(bn, num_hidden=4, no_bias=True, name="b")
+    out = S.elemwise_add(a, b, name="sum")
+    qsym, calib = Q._quantize_symbol(out, "gpu", offline_params=["a_weight", "b_weight"],
+                                     quantize_mode="full")
+    names = [n for _, n in ops_of(qsym)]
+    assert names.count("bn_output_quantize") == 1
+    assert node(qsym, "quantized_a")[2][0] == ("bn_output_quantize", 0)
+    assert node(qsym, "quantized_b")[2][0] == ("bn_output_quantize", 0)
+    assert node(qsym, "sum")[2] == [("a_dequantize", 0), ("b_dequantize", 0)]
+    assert calib == ["bn_output", "a_output", "b_output"]
+
+
+def test_quantize_params_names():
+    # test_quantize_params: conv + bn, every non-data argument offline
+    data = S.Variable("data")
+    conv = S.Convolution(data, kernel=(1, 1), num_filter=2048, name="conv")
+    sym = S.BatchNorm(data=conv, eps=2e-05, fix_gamma=False, momentum=0.9,
+                      use_global_stats=False, name="bn")
+    qsym, _ = Q._quantize_symbol(sym, "gpu", offline_params=offline_of(sym), quantize_mode="full")
+    args = qsym.list_arguments()
+    assert [a for a in args if a.startswith("conv")] == [
+        "conv_weight_quantize", "conv_bias_quantize", "conv_weight_quantize_min",
+        "conv_weight_quantize_max", "conv_bias_quantize_min", "conv_bias_quantize_max"]
+    assert [a for a in args if a.startswith("bn")] == ["bn_gamma", "bn_beta"]
+
+
+def test_set_calib_table():
+    # test_quantize_sym_with_calib
+    sym = fp32_sym()
+    qsym, _ = Q._quantize_symbol(sym, "gpu", offline_params=offline_of(sym), quantize_mode="full")
+    rng = np.random.default_rng(0)
+    table = {"conv_output": (rng.uniform(100.0, 200.0), rng.uniform(100.0, 200.0)),
+             "fc_output": (rng.uniform(100.0, 200.0), rng.uniform(100.0, 200.0)),
+             "conv_data": (-1.5, 2.5), "bn_output": (-0.25, 7.0), "unused_output": (0.0, 1.0)}
+    cqsym = Q._calibrate_quantized_sym(qsym, table)
+    attrs = cqsym.attr_dict()
+    for name, key in [("requantize_conv", "conv_output"), ("requantize_fc", "fc_output"),
+                      ("conv_data_quantize", "conv_data"), ("bn_output_quantize", "bn_output")]:
+        np.testing.assert_allclose(float(attrs[name]["min_calib_range"]), table[key][0],
+                                   rtol=1e-6, atol=1e-6)
+        np.testing.assert_allclose(float(attrs[name]["max_calib_range"]), table[key][1],
+                                   rtol=1e-3, atol=1e-4)
+    # std::to_string(float) spelling, as the operators' parsers receive it
+    assert attrs["conv_data_quantize"]["min_calib_range"] == "-1.500000"
+    assert ops_of(cqsym) == ops_of(qsym)
+    assert Q._calibrate_quantized_sym(qsym, {}) is qsym
+
+
+def test_optimal_threshold_adversarial_case():
+    # all mass in the last bin: the threshold must be the maximum
+    hist = [0] * 998 + [1000]
+    min_val, max_val = -2, 2
+    edges = [(max_val - min_val) / 999 * i + min_val for i in range(999)] + [max_val]
+    hist_data = (hist, edges, min_val, max_val, max_val)
+    for dtype in ["uint8", "int8", "auto"]:
+        res = Q._LayerHistogramCollector.get_optimal_threshold(hist_data, dtype,
+                                                               num_quantized_bins=5)
+        assert abs(res[2] - 2) < 1e-5
+
+
+def test_get_optimal_thresholds_uniform():
+    # uniform data: the best threshold is (close to) the largest magnitude
+    rng = np.random.default_rng(3)
+    for dtype in ["uint8", "int8", "auto"]:
+        arr = rng.uniform(-10.532, 11.3432, size=(8, 3, 23, 23))
+        lo, hi = arr.min(), arr.max()
+        th = max(abs(lo), abs(hi))
+        hist, edges = np.histogram(arr, bins=8001, range=(-th, th))
+        out = Q._LayerHistogramCollector.get_optimal_thresholds(
+            {"layer1": (hist, edges, lo, hi, th)}, dtype)
+        assert out["layer1"][0] == -out["layer1"][1]
+        np.testing.assert_allclose(out["layer1"][1], th, rtol=1e-2, atol=1e-4)
+
+
+def kl_threshold_numpy(hist, edges, nq):
+    """Independent float64 evaluation of the same search with scipy's entropy."""
+    from scipy.stats import entropy
+    hist = np.asarray(hist, dtype=np.float64)
+    nb = hist.size
+    zero = nb // 2
+    best = (np.inf, None)
+
+    def smooth(p, eps=0.0001):
+        z = p == 0
+        nz = p.size - z.sum()
+        if nz == 0:
+            return None
+        eps1 = eps * z.sum() / nz
+        if eps1 >= 1:
+            return None
+        return p + eps * z - eps1 * (~z)
+
+    for i in range(nq // 2, zero + 1):
+        start, stop = zero - i, zero + i + 1
+        sliced = hist[start:stop].copy()
+        p = sliced.copy()
+        p[0] = hist[:start + 1].sum()
+        p[-1] = hist[stop - 1:].sum()
+        sliced[0] = 0  # the reference leaves the first kept bin out of the merged levels
+        merged = sliced.size // nq
+        q = np.zeros_like(sliced)
+        for j in range(nq):
+            lo = j * merged
+            hi = sliced.size if j == nq - 1 else (j + 1) * merged
+            level = sliced[lo:hi].sum()
+            nonempty = (sliced[lo:hi] != 0).sum()
+            if nonempty:
+                q[lo:hi] = np.where(p[lo:hi] != 0, level / nonempty, 0)
+        ps, qs = smooth(p), smooth(q)
+        d = np.inf if qs is None else entropy(ps, qs)
+        if d < best[0]:
+            best = (d, edges[stop])
+    return best[1], best[0]
+
+
+def test_entropy_against_float64_search():
+    rng = np.random.default_rng(7)
+    arr = np.concatenate([rng.standard_normal(200000), rng.uniform(-9, 9, 300)])
+    th = np.abs(arr).max()
+    for bins, nq in [(2001, 255), (801, 127)]:
+        hist, edges = np.histogram(arr, bins=bins, range=(-th, th))
+        got_th, got_div = Q.calibrate_entropy(hist, edges, nq)
+        want_th, want_div = kl_threshold_numpy(hist, edges, nq)
+        # binary32 vs binary64 accumulation: the divergence agrees to a few digits and the
+        # chosen threshold is the same candidate or a neighbour with an equal divergence
+        np.testing.assert_allclose(got_div, want_div, rtol=2e-3)
+        step = edges[1] - edges[0]
+        assert abs(got_th - want_th) <= 2 * step + 1e-6
+
+
+def test_histogram_collector_merges_batches():
+    c = Q._LayerHistogramCollector("int8", num_bins=11, include_layers=["x"])
+    import torch
+    c.collect("x", "op", torch.tensor([-1.0, 0.0, 0.5, 1.0]))
+    c.collect("ignored", "op", torch.tensor([100.0]))
+    hist, edges, lo, hi, th = c.hist_dict["x"]
+    assert hist.sum() == 4 and th == 1.0 and len(hist) == 11
+    c.collect("x", "op", torch.tensor([0.25, -0.25]))        # inside the old range
+    assert c.hist_dict["x"][0].sum() == 6 and c.hist_dict["x"][4] == 1.0
+    c.collect("x", "op", torch.tensor([2.0, -0.1]))          # widens by whole old bins
+    hist, edges, lo, hi, th = c.hist_dict["x"]
+    assert hist.sum() == 8 and len(hist) % 2 == 1 and th >= 2.0 and (lo, hi) == (-1.0, 2.0)
+    old_step = 2.0 / 11
+    np.testing.assert_allclose(edges[1] - edges[0], old_step, rtol=1e-5)
+    assert "ignored" not in c.hist_dict
+    m = Q._LayerOutputMinMaxCollector("int8", include_layers=["x"])
+    m.collect("x", "op", torch.tensor([-1.0, 3.0]))
+    m.collect("x", "op", torch.tensor([-2.0, 1.0]))
+    assert m.post_collect() == {"x": (-2.0, 3.0)}
