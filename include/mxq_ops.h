@@ -86,6 +86,19 @@ int mxq_symbol_normalize(const char* symbol_json, const char** out_symbol_json);
 int mxq_calibrate_entropy(const float* hist, const float* hist_edges, size_t num_bins,
                           int num_quantized_bins, float* out_threshold, float* out_divergence);
 
+/* ---- NDArray list files (`.params`, mx.nd.save / mx.nd.load) ------------------------
+ * src/ndarray/ndarray.cc:1856-2146: dense arrays of the V2 / V3 record layouts plus the
+ * two legacy layouts on load; V2 (np_shape = 0) or V3 records on save.  Arrays live in
+ * host memory (mxq_blob.data is a host pointer here); what mxq_ndlist_get returns stays
+ * valid until mxq_ndlist_free. */
+int mxq_ndlist_load(const char* path, void** out_handle, int* out_count, int* out_has_names);
+int mxq_ndlist_get(void* handle, int index, const char** out_name, int* out_is_none,
+                   int* out_dtype, int* out_ndim, const int64_t** out_shape,
+                   const void** out_data, size_t* out_bytes);
+int mxq_ndlist_free(void* handle);
+int mxq_ndlist_save(const char* path, int count, const char** names, const mxq_blob* arrays,
+                    int np_shape);
+
 #ifdef __cplusplus
 }
 #endif

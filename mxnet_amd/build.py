@@ -77,7 +77,8 @@ def build_probe(verbose=False):
 
 OPS_LIB = os.path.join(HERE, "libmxq_ops.so")
 HOST_SOURCES = ["mxq_registry.cc", "mxq_quantization_ops.cc", "mxq_float_ops.cc", "mxq_graph.cc",
-                "mxq_quantize_graph_pass.cc", "mxq_calibrate.cc", "mxq_harness.cc"]
+                "mxq_quantize_graph_pass.cc", "mxq_calibrate.cc", "mxq_ndarray_io.cc",
+                "mxq_harness.cc"]
 
 
 def build_ops(verbose=False):

@@ -57,6 +57,9 @@ extern "C" {
 
 const char* mxq_ops_last_error(void) { return tl_error.c_str(); }
 
+// lets the other translation units of the library report through the same channel
+void mxq_ops_set_error(const char* text) { tl_error = text ? text : ""; }
+
 int mxq_op_count(void) { return static_cast<int>(nnvm::Op::ListAllNames().size()); }
 
 const char* mxq_op_name(int index) {

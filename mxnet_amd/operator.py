@@ -52,6 +52,11 @@ OPS_SIGNATURES = {
     "mxq_set_calib_table": (_i, [ctypes.c_char_p, _i, _pps, ctypes.POINTER(ctypes.c_float),
                                  ctypes.POINTER(ctypes.c_float), _pps]),
     "mxq_symbol_normalize": (_i, [ctypes.c_char_p, _pps]),
+    "mxq_ndlist_load": (_i, [ctypes.c_char_p, ctypes.POINTER(_p), _pi, _pi]),
+    "mxq_ndlist_get": (_i, [_p, _i, _pps, _pi, _pi, _pi, ctypes.POINTER(_pl),
+                            ctypes.POINTER(_p), ctypes.POINTER(_sz)]),
+    "mxq_ndlist_free": (_i, [_p]),
+    "mxq_ndlist_save": (_i, [ctypes.c_char_p, _i, _pps, _pb, _i]),
     "mxq_calibrate_entropy": (_i, [ctypes.POINTER(ctypes.c_float), ctypes.POINTER(ctypes.c_float),
                                    _sz, _i, ctypes.POINTER(ctypes.c_float),
                                    ctypes.POINTER(ctypes.c_float)]),

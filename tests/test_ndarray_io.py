@@ -1,0 +1,104 @@
+"""NDArray list files: the reference's own legacy fixture
+(tests/python/unittest/legacy_ndarray.v0, checked by test_ndarray_legacy_load,
+tests/python/unittest/test_ndarray.py:439-447: six arrays equal to arange(128)), a byte-level
+check of what is written against the layout in src/ndarray/ndarray.cc:1865-1936 and
+:2126-2135, and round trips of a quantized model's parameters."""
+import os
+import struct
+
+import numpy as np
+import pytest
+import torch
+
+from mxnet_amd import ndarray as nd
+from mxnet_amd.operator import MXNetError
+
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+
+
+def test_legacy_fixture_of_the_reference():
+    data = nd.load(os.path.join(GOLDEN, "legacy_ndarray.v0"))
+    assert isinstance(data, list) and len(data) == 6
+    for t in data:
+        assert t.dtype == torch.float32 and tuple(t.shape) == (128,)
+        np.testing.assert_array_equal(t.numpy(), np.arange(128, dtype=np.float32))
+
+
+def test_written_bytes_follow_the_v2_layout(tmp_path):
+    path = str(tmp_path / "one.params")
+    w = torch.tensor([[1, -2, 3], [4, 5, -6]], dtype=torch.int8)
+    nd.save(path, {"arg:fc_weight_quantize": w})
+    raw = open(path, "rb").read()
+    name = b"arg:fc_weight_quantize"
+    want = struct.pack("<QQQ", 0x112, 0, 1)                       # list magic, reserved, count
+    want += struct.pack("<Ii", 0xF993FAC9, 0)                     # V2 magic, default storage
+    want += struct.pack("<iqq", 2, 2, 3)                          # shape: ndim, extents
+    want += struct.pack("<ii", 1, 0)                              # context cpu(0)
+    want += struct.pack("<i", 5)                                  # mshadow::kInt8
+    want += bytes(w.numpy().tobytes())
+    want += struct.pack("<Q", 1) + struct.pack("<Q", len(name)) + name
+    assert raw == want
+    nd.save(path, [torch.zeros(())], np_shape=True)               # V3: zero-dim allowed
+    raw = open(path, "rb").read()
+    assert struct.unpack_from("<I", raw, 24)[0] == 0xF993FACA
+    assert raw[-8:] == struct.pack("<Q", 0)                       # no names for a list
+    with pytest.raises(MXNetError, match="numpy shape semantics"):
+        nd.save(path, [torch.zeros(())])
+
+
+def test_round_trips(tmp_path):
+    rng = np.random.default_rng(0)
+    path = str(tmp_path / "model-0000.params")
+    params = {
+        "conv_weight_quantize": torch.from_numpy(rng.integers(-127, 128, (16, 4, 3, 3)).astype(np.int8)),
+        "conv_weight_quantize_min": torch.tensor([-0.75]),
+        "conv_weight_quantize_max": torch.tensor([0.75]),
+        "bn_gamma": torch.from_numpy(rng.normal(size=16).astype(np.float32)),
+        "acc": torch.from_numpy(rng.integers(-2 ** 31, 2 ** 31, (5, 7)).astype(np.int32)),
+        "u8": torch.from_numpy(rng.integers(0, 256, 33).astype(np.uint8)),
+        "f64": torch.from_numpy(rng.normal(size=(2, 2))),
+        "f16": torch.from_numpy(rng.normal(size=9).astype(np.float16)),
+        "bf16": torch.tensor([1.5, -2.25, 3.0], dtype=torch.bfloat16),
+        "i64": torch.tensor([2 ** 40, -1]),
+        "flag": torch.tensor([True, False]),
+        "empty": torch.zeros((0, 4)),
+    }
+    for np_shape in (False, True):
+        nd.save(path, params, np_shape=np_shape)
+        back = nd.load(path)
+        assert list(back.keys()) == list(params.keys())
+        for k, v in params.items():
+            assert back[k].dtype == v.dtype and back[k].shape == v.shape, k
+            assert torch.equal(back[k], v), k
+    nd.save(path, list(params.values())[:3])
+    back = nd.load(path)
+    assert isinstance(back, list) and len(back) == 3 and torch.equal(back[0], params["conv_weight_quantize"])
+
+
+def test_checkpoint_helpers(tmp_path):
+    from mxnet_amd import symbol as S
+    fc = S.FullyConnected(S.Variable("data"), num_hidden=4, name="fc")
+    prefix = str(tmp_path / "net")
+    arg = {"fc_weight": torch.ones(4, 3), "fc_bias": torch.zeros(4)}
+    aux = {"bn_moving_mean": torch.arange(4.0)}
+    nd.save_checkpoint(prefix, 7, fc, arg, aux)
+    assert os.path.exists(prefix + "-symbol.json") and os.path.exists(prefix + "-0007.params")
+    sym, a, x = nd.load_checkpoint(prefix, 7)
+    assert sym.tojson() == fc.tojson()
+    assert set(a) == set(arg) and set(x) == set(aux) and torch.equal(x["bn_moving_mean"], aux["bn_moving_mean"])
+
+
+def test_malformed_files(tmp_path):
+    path = str(tmp_path / "bad.params")
+    open(path, "wb").write(b"not an ndarray file at all")
+    with pytest.raises(MXNetError, match="Invalid NDArray file format"):
+        nd.load(path)
+    open(path, "wb").write(struct.pack("<QQQ", 0x112, 0, 1) + struct.pack("<Ii", 0xF993FAC9, 1))
+    with pytest.raises(MXNetError, match="dense"):
+        nd.load(path)
+    open(path, "wb").write(struct.pack("<QQQ", 0x112, 0, 1) + struct.pack("<Ii", 0xF993FAC9, 0) +
+                           struct.pack("<iq", 1, 100))            # truncated after the shape
+    with pytest.raises(MXNetError, match="Invalid NDArray file format"):
+        nd.load(path)
+    with pytest.raises(MXNetError, match="cannot open"):
+        nd.load(str(tmp_path / "missing.params"))
