@@ -92,15 +92,17 @@ __device__ __forceinline__ int epi_bias32(const Epilogue& e, const EpiScalars& s
   return static_cast<int>(p / s.foq);
 }
 
-// FloatToQuantized<int8>(float(acc) * in_scale): trunc(sign(f) * min(|f|*s + 0.5, 127)).
-// The magnitude v is >= 0.5, so copysign(v, f) followed by the truncating convert
-// equals sign(f) * v truncated, including f == +-0 (trunc(+-0.5) = 0).
-__device__ __forceinline__ int epi_requant(int acc, const EpiScalars& s) {
+// FloatToQuantized<int8>(float(acc) * in_scale): trunc(sign(f) * min(|f|*s + 0.5, 127)),
+// optionally followed by the int8 relu.  The magnitude |f|*s + 0.5 is >= 0.5, so giving
+// it f's sign and clamping the signed value to [lo, 127] (lo = -127, or 0 with relu)
+// before the truncating convert yields the same integer: copysign and clamp commute,
+// trunc(+-0.5) = 0 covers f = +-0, and a negative value clamped to 0 is what relu makes
+// of the negative int8.  One v_med3_f32 replaces the min and the integer max.
+__device__ __forceinline__ int epi_requant(int acc, const EpiScalars& s, float lo) {
   float f = static_cast<float>(acc) * s.in_scale;
   float t = fabsf(f) * s.qscale;
-  float u = t + 0.5f;
-  float v = fminf(u, 127.0f);
-  return static_cast<int>(copysignf(v, f));
+  float u = copysignf(t + 0.5f, f);
+  return static_cast<int>(__builtin_amdgcn_fmed3f(u, lo, 127.0f));
 }
 
 // {a,b,c,d} low bytes -> one dword (a in byte 0).
@@ -607,8 +609,7 @@ __device__ __forceinline__ void gemm_epilogue(v16i (&acc)[Cfg::MI][Cfg::NI], con
           int q[4];
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
-            q[i] = epi_requant(v[i], s);
-            if (e.relu) q[i] = q[i] > 0 ? q[i] : 0;
+            q[i] = epi_requant(v[i], s, e.relu ? 0.0f : -127.0f);
           }
           if (full) {
             *reinterpret_cast<uint32_t*>(e.out8 + off) = pack_bytes(q[0], q[1], q[2], q[3]);
@@ -700,8 +701,7 @@ __device__ __forceinline__ void gemm_epilogue_lds(v16i (&acc)[Cfg::MI][Cfg::NI],
           int q[4];
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
-            q[i] = epi_requant(v[i], s);
-            if (e.relu) q[i] = q[i] > 0 ? q[i] : 0;
+            q[i] = epi_requant(v[i], s, e.relu ? 0.0f : -127.0f);
           }
           *reinterpret_cast<uint32_t*>(stage + ml * LD + nl) = pack_bytes(q[0], q[1], q[2], q[3]);
         }

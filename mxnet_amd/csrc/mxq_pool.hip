@@ -32,8 +32,8 @@ struct PoolArgs {
   int bands;  // bands per plane
   int vec_ok; // the tensor base is 16-byte aligned
   // floor(n / d) = umulhi(n, magic) for n * d < 2^32 (magic = 2^32 / d + 1; 0 stands for d = 1)
-  uint32_t magic_ow4;        // d = ceil(OW / 4)
-  uint32_t magic_per_plane;  // d = OH * ceil(OW / 4), used when ppb > 1
+  uint32_t magic_per_row;    // d = items per output row
+  uint32_t magic_per_plane;  // d = items per plane, used when ppb > 1
 };
 
 __device__ __forceinline__ int fast_div(int n, uint32_t magic) {
@@ -70,71 +70,82 @@ __device__ __forceinline__ int pool_window(Ptr img, int row0, const PoolArgs& a,
   return min(max(q, lo), hi);
 }
 
-// Four horizontally adjacent outputs of one row, for a compile-time window width and
-// stride.  The 3*SW + KW wide strip of every window row is read from LDS as three
-// aligned dwords (the LDS instruction rate and divergence are what bound this kernel,
-// not arithmetic), realigned with the byte funnel shift, and folded into the outputs
-// that cover each byte.  Columns outside the image are neutralised instead of branched
-// around (the staged image has 16 bytes of slack in front and 32 behind), so border
-// items take the same path as interior ones.
-template <bool UNSIGNED, int KW, int SW>
-__device__ __forceinline__ void pool_quad(const uint8_t* img, int row0, const PoolArgs& a, int oh,
-                                          int ow0, int (&q)[4]) {
+constexpr int kPoolItem = 8;  // horizontally adjacent outputs one thread computes at a time
+
+// kPoolItem adjacent outputs of one row for a compile-time K x K window and horizontal
+// stride.  Per window row the (kPoolItem-1)*SW + K wide strip is read from LDS as aligned
+// dwords (indexing the shared array directly, so the reads stay LDS reads), realigned with
+// the byte funnel shift and folded into the outputs that cover each byte.  Nothing branches
+// on position: columns outside the image are replaced through a byte mask, rows outside it
+// read a clamped row and are masked as a whole (the staged bytes have 16 bytes of slack in
+// front and 64 behind), so border items cost what interior items cost.
+// `base` is the byte offset, inside the shared array, of row `row0` of the item's plane.
+template <bool UNSIGNED, bool AVG, int K, int SW>
+__device__ __forceinline__ void pool_strip(const uint8_t* lds, int base, int row0, int row1,
+                                           const PoolArgs& a, int oh, int ow0,
+                                           int (&q)[kPoolItem]) {
   constexpr int lo = UNSIGNED ? 0 : -128, hi = UNSIGNED ? 255 : 127;
-  constexpr int SPAN = 3 * SW + KW;
-  static_assert(SPAN + 3 <= 12, "three aligned dwords cover the strip at any byte offset");
-  int hstart = oh * a.sh - a.ph;
-  int hend = min(hstart + a.KH, a.H + a.ph);
-  const int padded_rows = hend - hstart;
-  hstart = max(hstart, 0);
-  hend = min(hend, a.H);
+  constexpr int SPAN = (kPoolItem - 1) * SW + K;
+  constexpr int NW = (SPAN + 3 + 3) / 4;  // aligned dwords covering the strip at any offset
+  constexpr int neutral = AVG ? 0 : lo;
+  constexpr uint32_t fill = (static_cast<uint32_t>(neutral) & 0xffu) * 0x01010101u;
+  const uint32_t* words = reinterpret_cast<const uint32_t*>(lds);
+  const int h0 = oh * a.sh - a.ph;
   const int w0 = ow0 * SW - a.pw;
-  const int neutral = a.is_avg ? 0 : lo;
-  // byte masks of the columns inside the image, and what the others are replaced with
-  uint32_t keep[3] = {0u, 0u, 0u};
+  uint32_t keep[NW];
+#pragma unroll
+  for (int w = 0; w < NW; ++w) keep[w] = 0u;
 #pragma unroll
   for (int j = 0; j < SPAN; ++j)
     if (static_cast<unsigned>(w0 + j) < static_cast<unsigned>(a.W))
       keep[j / 4] |= 0xffu << (8 * (j % 4));
-  const uint32_t fill = (static_cast<uint32_t>(neutral) & 0xffu) * 0x01010101u;
-  int acc[4];
+  int acc[kPoolItem];
 #pragma unroll
-  for (int i = 0; i < 4; ++i) acc[i] = neutral;
-  for (int h = hstart; h < hend; ++h) {
-    const uintptr_t addr = reinterpret_cast<uintptr_t>(img + (h - row0) * a.W + w0);
-    const uint32_t* wp = reinterpret_cast<const uint32_t*>(addr & ~static_cast<uintptr_t>(3));
-    const uint32_t sft = static_cast<uint32_t>(addr & 3u);
-    const uint32_t d0 = wp[0], d1 = wp[1], d2 = wp[2];
-    uint32_t x[3];
-    x[0] = __builtin_amdgcn_alignbyte(d1, d0, sft);
-    x[1] = __builtin_amdgcn_alignbyte(d2, d1, sft);
-    x[2] = __builtin_amdgcn_alignbyte(0u, d2, sft);
+  for (int i = 0; i < kPoolItem; ++i) acc[i] = neutral;
+  int rows_inside = 0;
 #pragma unroll
-    for (int w = 0; w < 3; ++w) x[w] = (x[w] & keep[w]) | (fill & ~keep[w]);  // one v_bfi
+  for (int r = 0; r < K; ++r) {
+    const int h = h0 + r;
+    const bool inside = static_cast<unsigned>(h) < static_cast<unsigned>(a.H);
+    rows_inside += inside;
+    const int hh = min(max(h, row0), row1 - 1);  // a staged row, whatever h is
+    const int off = base + (hh - row0) * a.W + w0;
+    const int wi = off >> 2;
+    const uint32_t sft = static_cast<uint32_t>(off & 3);
+    uint32_t d[NW + 1];
+#pragma unroll
+    for (int w = 0; w < NW; ++w) d[w] = words[wi + w];
+    d[NW] = 0u;
+    uint32_t x[NW];
+#pragma unroll
+    for (int w = 0; w < NW; ++w) {
+      const uint32_t k = inside ? keep[w] : 0u;
+      x[w] = (__builtin_amdgcn_alignbyte(d[w + 1], d[w], sft) & k) | (fill & ~k);
+    }
     int v[SPAN];
 #pragma unroll
     for (int j = 0; j < SPAN; ++j) {
-      const uint32_t b = (x[j / 4] >> (8 * (j % 4))) & 0xffu;
-      v[j] = UNSIGNED ? static_cast<int>(b) : static_cast<int>(static_cast<int8_t>(b));
+      const uint32_t byte = (x[j / 4] >> (8 * (j % 4))) & 0xffu;
+      v[j] = UNSIGNED ? static_cast<int>(byte) : static_cast<int>(static_cast<int8_t>(byte));
     }
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < kPoolItem; ++i)
 #pragma unroll
-      for (int k = 0; k < KW; ++k)
-        acc[i] = a.is_avg ? acc[i] + v[i * SW + k] : max(acc[i], v[i * SW + k]);
+      for (int k = 0; k < K; ++k)
+        acc[i] = AVG ? acc[i] + v[i * SW + k] : max(acc[i], v[i * SW + k]);
   }
-  if (!a.is_avg) {
+  if (!AVG) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) q[i] = acc[i];
+    for (int i = 0; i < kPoolItem; ++i) q[i] = acc[i];
     return;
   }
+  const int padded_rows = min(h0 + K, a.H + a.ph) - h0;
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
+  for (int i = 0; i < kPoolItem; ++i) {
     const int wstart = w0 + i * SW;
-    const int wend = min(wstart + KW, a.W + a.pw);
-    const int pool_size = a.count_pad
-                              ? padded_rows * (wend - wstart)
-                              : (hend - hstart) * (min(wend, a.W) - max(wstart, 0));
+    const int wend = min(wstart + K, a.W + a.pw);
+    const int pool_size = a.count_pad ? padded_rows * (wend - wstart)
+                                      : rows_inside * (min(wend, a.W) - max(wstart, 0));
     const float avg =
         pool_size > 0 ? static_cast<float>(acc[i]) / static_cast<float>(pool_size) : 0.f;
     q[i] = min(max(static_cast<int>(rintf(avg)), lo), hi);
@@ -163,13 +174,13 @@ __device__ __forceinline__ int sum_bytes(const uint8_t* lds, int addr, int n) {
   return sum;
 }
 
-// FAST: 0 generic windows; 1 quads with KW=3,SW=2; 2 quads KW=2,SW=2; 3 quads KW=3,SW=1;
-// 4 average over full-width windows (global pooling): contiguous byte sums.
-template <bool UNSIGNED, int FAST>
+// FAST: 0 generic windows; 1 quads with a 3x3 window, horizontal stride 2; 2 quads 2x2 /
+// 2; 3 quads 3x3 / 1; 4 average over full-width windows (global pooling): contiguous sums.
+template <bool UNSIGNED, bool AVG, int FAST>
 __global__ __launch_bounds__(kPoolThreads) void pool_lds_kernel(PoolArgs a) {
   // the staged bytes start 16 bytes into the array: strips that begin left of column 0
   // read (and discard) what lies in front
-  __shared__ __attribute__((aligned(16))) uint8_t lds_raw[kPoolLdsBytes + 64];
+  __shared__ __attribute__((aligned(16))) uint8_t lds_raw[kPoolLdsBytes + 96];
   uint8_t* lds = lds_raw + 16;
   const int tid = threadIdx.x;
   int p0, np, oh0, oh1;
@@ -245,37 +256,45 @@ __global__ __launch_bounds__(kPoolThreads) void pool_lds_kernel(PoolArgs a) {
     }
     return;
   }
-  // items of four adjacent outputs of one row
-  const int OW4 = (a.OW + 3) >> 2;
-  const int per_plane = rows * OW4;
+  // items of kPoolItem adjacent outputs of one row
+  const int per_row = (a.OW + kPoolItem - 1) / kPoolItem;
+  const int per_plane = rows * per_row;
   const int items = np * per_plane;
-  constexpr int KW = FAST == 1 ? 3 : FAST == 2 ? 2 : 3;
+  constexpr int K = FAST == 2 ? 2 : 3;
   constexpr int SW = FAST == 3 ? 1 : 2;
   for (int it = tid; it < items; it += kPoolThreads) {
     const int p = a.ppb > 1 ? fast_div(it, a.magic_per_plane) : 0, r = it - p * per_plane;
-    const int orow = fast_div(r, a.magic_ow4), ow0 = (r - orow * OW4) * 4;
+    const int orow = fast_div(r, a.magic_per_row), ow0 = (r - orow * per_row) * kPoolItem;
     const int oh = oh0 + orow;
-    const int nout = min(4, a.OW - ow0);
-    const uint8_t* img = lds + shift + static_cast<size_t>(p) * plane_bytes;
-    int q[4] = {0, 0, 0, 0};
+    const int nout = min(kPoolItem, a.OW - ow0);
+    int q[kPoolItem];
+#pragma unroll
+    for (int i = 0; i < kPoolItem; ++i) q[i] = 0;
     if (FAST != 0) {
-      pool_quad<UNSIGNED, KW, SW>(img, hs, a, oh, ow0, q);
+      const int base = 16 + shift + p * static_cast<int>(plane_bytes);
+      pool_strip<UNSIGNED, AVG, K, SW>(lds_raw, base, hs, he, a, oh, ow0, q);
     } else {
+      const uint8_t* img = lds + shift + static_cast<size_t>(p) * plane_bytes;
       // (fixed trip count: a runtime-indexed q[] would live in scratch memory)
 #pragma unroll
-      for (int i = 0; i < 4; ++i)
+      for (int i = 0; i < kPoolItem; ++i)
         if (i < nout) q[i] = pool_window<UNSIGNED>(img, hs, a, oh, ow0 + i);
     }
     const size_t off = (static_cast<size_t>(p0 + p) * a.OH + oh) * a.OW + ow0;
-    if (nout == 4 && ((reinterpret_cast<uintptr_t>(a.out) + off) & 3u) == 0) {
-      const uint32_t packed = (static_cast<uint32_t>(q[0]) & 0xffu) |
-                              ((static_cast<uint32_t>(q[1]) & 0xffu) << 8) |
-                              ((static_cast<uint32_t>(q[2]) & 0xffu) << 16) |
-                              (static_cast<uint32_t>(q[3]) << 24);
-      *reinterpret_cast<uint32_t*>(a.out + off) = packed;
+    uint32_t packed[kPoolItem / 4];
+#pragma unroll
+    for (int w = 0; w < kPoolItem / 4; ++w)
+      packed[w] = (static_cast<uint32_t>(q[4 * w]) & 0xffu) |
+                  ((static_cast<uint32_t>(q[4 * w + 1]) & 0xffu) << 8) |
+                  ((static_cast<uint32_t>(q[4 * w + 2]) & 0xffu) << 16) |
+                  (static_cast<uint32_t>(q[4 * w + 3]) << 24);
+    if (nout == kPoolItem && ((reinterpret_cast<uintptr_t>(a.out) + off) & 3u) == 0) {
+#pragma unroll
+      for (int w = 0; w < kPoolItem / 4; ++w)
+        reinterpret_cast<uint32_t*>(a.out + off)[w] = packed[w];
     } else {
 #pragma unroll
-      for (int i = 0; i < 4; ++i)
+      for (int i = 0; i < kPoolItem; ++i)
         if (i < nout) a.out[off + i] = static_cast<uint8_t>(q[i]);
     }
   }
@@ -414,38 +433,51 @@ int mxq_quantized_pooling_nchw(void* stream, const void* in, int in_type, int N,
     auto magic = [](long long d) {
       return d <= 1 ? 0u : static_cast<uint32_t>((1ULL << 32) / static_cast<unsigned long long>(d) + 1ULL);
     };
-    const long long ow4 = (OW + 3) / 4;
+    const long long ow4 = (OW + kPoolItem - 1) / kPoolItem;  // items per output row
     // items per work-group stay below 2^17 and the divisors below 2^15 (both bounded by
     // the bytes staged in LDS), so n * d < 2^32 holds
     MXQ_CHECK(ow4 * OH < (1LL << 15) || a.ppb <= 1, "pooling plane too large for the item index");
     MXQ_CHECK(ow4 < (1LL << 15), "pooling row too long for the item index");
-    a.magic_ow4 = magic(ow4);
+    a.magic_per_row = magic(ow4);
     a.magic_per_plane = magic(ow4 * OH);
     int fast = 0;
     if (a.is_avg && OW == 1 && pad_w == 0 && kernel_w == W)
       fast = 4;
     else if (pad_w > 8)
       fast = 0;  // the quad path reads at most 16 bytes in front of a row
-    else if (kernel_w == 3 && stride_w == 2)
+    else if (kernel_h == 3 && kernel_w == 3 && stride_w == 2)
       fast = 1;
-    else if (kernel_w == 2 && stride_w == 2)
+    else if (kernel_h == 2 && kernel_w == 2 && stride_w == 2)
       fast = 2;
-    else if (kernel_w == 3 && stride_w == 1)
+    else if (kernel_h == 3 && kernel_w == 3 && stride_w == 1)
       fast = 3;
-#define MXQ_POOL(U, F) \
-  hipLaunchKernelGGL((pool_lds_kernel<U, F>), dim3(blocks), dim3(kPoolThreads), 0, s, a)
-#define MXQ_POOL_F(U)            \
-  switch (fast) {                \
-    case 1: MXQ_POOL(U, 1); break; \
-    case 2: MXQ_POOL(U, 2); break; \
-    case 3: MXQ_POOL(U, 3); break; \
-    case 4: MXQ_POOL(U, 4); break; \
-    default: MXQ_POOL(U, 0); break; \
+#define MXQ_POOL(U, A, F) \
+  hipLaunchKernelGGL((pool_lds_kernel<U, A, F>), dim3(blocks), dim3(kPoolThreads), 0, s, a)
+#define MXQ_POOL_F(U, A)               \
+  switch (fast) {                      \
+    case 1: MXQ_POOL(U, A, 1); break;  \
+    case 2: MXQ_POOL(U, A, 2); break;  \
+    case 3: MXQ_POOL(U, A, 3); break;  \
+    default: MXQ_POOL(U, A, 0); break; \
   }
-    if (a.is_unsigned) {
-      MXQ_POOL_F(true)
+    if (fast == 4) {
+      if (a.is_unsigned) {
+        MXQ_POOL(true, true, 4);
+      } else {
+        MXQ_POOL(false, true, 4);
+      }
+    } else if (a.is_unsigned) {
+      if (a.is_avg) {
+        MXQ_POOL_F(true, true)
+      } else {
+        MXQ_POOL_F(true, false)
+      }
     } else {
-      MXQ_POOL_F(false)
+      if (a.is_avg) {
+        MXQ_POOL_F(false, true)
+      } else {
+        MXQ_POOL_F(false, false)
+      }
     }
 #undef MXQ_POOL_F
 #undef MXQ_POOL
