@@ -48,7 +48,7 @@ def parse_args():
     ap.add_argument("--workload", default="fc4096",
                     choices=["fc4096", "fc8192", "quantize", "quantize_uncal", "quantize_uint8",
                              "requantize", "requantize_uncal", "dequantize", "copy", "maxpool", "avgpool",
-                             "resnet50_convs", "bert_fc_chain"])
+                             "resnet50_convs", "bert_fc_chain", "bert_fc_chain_fused"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-cast-ops", action="store_true")
     return ap.parse_args()
@@ -411,11 +411,15 @@ class BertChainWorkload(GraphWorkload):
     quantize_v2 -> quantized_fully_connected (+ int8 bias) -> requantize -> dequantize, as
     the unfused graph runs it.  Activations N(0,1) with 0.1% outliers at +-20."""
 
-    def __init__(self, torch, capi, lib):
+    def __init__(self, torch, capi, lib, fused=False):
         self.kernel = "quantize + fc_dma + requantize + dequantize kernels"
         self.bound = "mfma"
         self.name = "BERT-base FC chain M=4096: 768->2304, 768->768, 768->3072, 3072->768, " \
                     "quantize_v2 -> quantized_fc -> requantize -> dequantize per layer"
+        if fused:
+            self.kernel = "quantize + fc_dma (requantize in the epilogue) + dequantize kernels"
+            self.name = self.name.replace("quantized_fc -> requantize",
+                                          "quantized_fc with the requantize fused")
         P = lambda t: ctypes.c_void_p(t.data_ptr())
         g = torch.Generator(device="cuda").manual_seed(5)
         M = 4096
@@ -443,6 +447,19 @@ class BertChainWorkload(GraphWorkload):
             st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
             for (K, N, wq, bq, wmin, wmax, bmin, bmax, r, B) in self.layers:
                 sc = B["sc"]
+                if fused:
+                    rcs = [
+                        lib.mxq_quantize_v2(st, P(B["x"]), P(B["q"]), P(sc[0]), P(sc[1]), M * K,
+                                            5, 1, -20.0, 20.0, None, 0),
+                        lib.mxq_quantized_fc(st, P(B["q"]), P(wq), P(bq), M, N, K, P(sc[0]),
+                                             P(sc[1]), P(wmin), P(wmax), P(bmin), P(bmax), None,
+                                             P(sc[2]), P(sc[3]), P(B["q8"]), P(sc[4]), P(sc[5]),
+                                             0, -r, r),
+                        lib.mxq_dequantize(st, P(B["q8"]), 5, P(sc[4]), P(sc[5]), P(B["y"]),
+                                           M * N)]
+                    if any(rcs):
+                        raise RuntimeError(lib.mxq_last_error().decode())
+                    continue
                 rcs = [
                     lib.mxq_quantize_v2(st, P(B["x"]), P(B["q"]), P(sc[0]), P(sc[1]), M * K, 5, 1,
                                         -20.0, 20.0, None, 0),
@@ -516,6 +533,8 @@ def make_workload(name, torch, capi, lib):
         return ConvStackWorkload(torch, capi, lib)
     if name == "bert_fc_chain":
         return BertChainWorkload(torch, capi, lib)
+    if name == "bert_fc_chain_fused":
+        return BertChainWorkload(torch, capi, lib, fused=True)
     if name == "copy":
         return CopyWorkload(torch)
     if name in ("maxpool", "avgpool"):
@@ -601,11 +620,12 @@ def main():
         rows = []
         for kind in ["quantize", "quantize_uint8", "quantize_uncal", "requantize",
                      "requantize_uncal", "dequantize", "maxpool", "avgpool", "fc8192",
-                     "resnet50_convs", "bert_fc_chain"]:
+                     "resnet50_convs", "bert_fc_chain", "bert_fc_chain_fused"]:
             if kind == args.workload:
                 continue
             w2 = make_workload(kind, torch, capi, lib)
-            steps2 = 20 if kind in ("fc8192", "resnet50_convs", "bert_fc_chain") else 60
+            steps2 = 20 if kind in ("fc8192", "resnet50_convs", "bert_fc_chain",
+                                    "bert_fc_chain_fused") else 60
             wall2, ev2 = timed_run(torch, w2, steps2, 5)
             r = roofline_of(w2, ev2 / steps2, kind)
             r["workload"] = w2.name

@@ -210,14 +210,16 @@ __global__ __launch_bounds__(Cfg::kThreads) void conv_dma_kernel(ConvArgs p) {
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
 
-  const EpiPre pre = epi_prefetch<Cfg>(p.epi, n0, p.O);
+  // what the epilogue needs is fetched while the first operand stages are in flight
+  EpiPre pre;
+  auto prefetch = [&]() { pre = epi_prefetch<Cfg>(p.epi, n0, p.O); };
   ConvIssuer<Cfg, Cfg::A_CHUNKS> ai;
   RowIssuerBuffer<Cfg, Cfg::B_CHUNKS> bi;
   ai.init(p, m0, wave, lane);
   bi.init(p.weight, n0, p.O, p.K, wave, lane);
 
   v16i acc[Cfg::MI][Cfg::NI];
-  gemm_mainloop_dma<Cfg, NS, PIPE>(acc, ai, bi, (p.K + Cfg::BK - 1) / Cfg::BK, lds);
+  gemm_mainloop_dma<Cfg, NS, PIPE>(acc, ai, bi, (p.K + Cfg::BK - 1) / Cfg::BK, lds, prefetch);
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 
   static_assert(NS * Cfg::STAGE_SLOTS * 16 >=

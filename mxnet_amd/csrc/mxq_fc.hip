@@ -64,7 +64,9 @@ __global__ __launch_bounds__(Cfg::kThreads) void fc_dma_kernel(FcArgs p) {
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
 
-  const EpiPre pre = epi_prefetch<Cfg>(p.epi, n0, p.N);
+  // what the epilogue needs is fetched while the first operand stages are in flight
+  EpiPre pre;
+  auto prefetch = [&]() { pre = epi_prefetch<Cfg>(p.epi, n0, p.N); };
   v16i acc[Cfg::MI][Cfg::NI];
   const int KT = (p.K + Cfg::BK - 1) / Cfg::BK;
   if (BUF) {
@@ -72,13 +74,13 @@ __global__ __launch_bounds__(Cfg::kThreads) void fc_dma_kernel(FcArgs p) {
     RowIssuerBuffer<Cfg, Cfg::B_CHUNKS> bi;
     ai.init(p.data, m0, p.M, p.K, wave, lane);
     bi.init(p.weight, n0, p.N, p.K, wave, lane);
-    gemm_mainloop_dma<Cfg, NS, PIPE>(acc, ai, bi, KT, lds);
+    gemm_mainloop_dma<Cfg, NS, PIPE>(acc, ai, bi, KT, lds, prefetch);
   } else {
     RowIssuerGlobal<Cfg, Cfg::A_CHUNKS> ai;
     RowIssuerGlobal<Cfg, Cfg::B_CHUNKS> bi;
     ai.init(p.data, m0, p.M, p.K, wave, lane);
     bi.init(p.weight, n0, p.N, p.K, wave, lane);
-    gemm_mainloop_dma<Cfg, NS, PIPE>(acc, ai, bi, KT, lds);
+    gemm_mainloop_dma<Cfg, NS, PIPE>(acc, ai, bi, KT, lds, prefetch);
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 

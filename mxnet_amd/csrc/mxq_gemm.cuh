@@ -435,9 +435,13 @@ struct RowIssuerBuffer {
 //      back-to-back while LDS and DMA work trickles in between.
 // AIssuer / BIssuer provide issue(instr, stage, lds_byte_addr) and stage_done(); stages
 // are issued in increasing order, each exactly once, and only stages < KT.
-template <class Cfg, int NS, int PIPE, class AIssuer, class BIssuer>
+// `after_prologue` runs once the first NS-1 stages are on their way: the place for work
+// that only the epilogue needs (range scalars, bias) and whose loads and divisions should
+// hide behind the first operand fetch rather than in front of it.
+template <class Cfg, int NS, int PIPE, class AIssuer, class BIssuer, class AfterPrologue>
 __device__ __forceinline__ void gemm_mainloop_dma(v16i (&acc)[Cfg::MI][Cfg::NI], AIssuer& ai,
-                                                  BIssuer& bi, int KT, v4i* lds) {
+                                                  BIssuer& bi, int KT, v4i* lds,
+                                                  AfterPrologue&& after_prologue) {
   constexpr int CH = Cfg::CH, NW = Cfg::kThreads / 64;
   constexpr int AI = Cfg::A_CHUNKS, BI = Cfg::B_CHUNKS, CPT = AI + BI;
   constexpr int MI = Cfg::MI, NI = Cfg::NI, KS = Cfg::KS;
@@ -503,6 +507,7 @@ __device__ __forceinline__ void gemm_mainloop_dma(v16i (&acc)[Cfg::MI][Cfg::NI],
 
 #pragma unroll
   for (int s = 0; s < NS - 1; ++s) issue(s);  // stages 0 .. min(KT, NS-1)-1
+  after_prologue();
   auto last_issued = [&](int kt_now) {         // newest stage in flight during step kt_now
     const int l = kt_now + NS - 2;
     return l < KT - 1 ? l : KT - 1;
