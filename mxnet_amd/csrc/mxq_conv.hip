@@ -222,10 +222,8 @@ __global__ __launch_bounds__(Cfg::kThreads) void conv_dma_kernel(ConvArgs p) {
   gemm_mainloop_dma<Cfg, NS, PIPE>(acc, ai, bi, (p.K + Cfg::BK - 1) / Cfg::BK, lds, prefetch);
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 
-  static_assert(NS * Cfg::STAGE_SLOTS * 16 >=
-                    Cfg::BN * 4 + (Cfg::kThreads / 64) * Cfg::TM * (Cfg::TN + 16),
-                "stage ring too small for the epilogue transpose");
-  gemm_epilogue_lds<Cfg>(acc, p.epi, pre, m0, n0, p.M, p.O, static_cast<size_t>(p.O), lds);
+  gemm_epilogue_lds<Cfg, NS * Cfg::STAGE_SLOTS * 16>(acc, p.epi, pre, m0, n0, p.M, p.O,
+                                                     static_cast<size_t>(p.O), lds);
   if (blockIdx.x == 0 && threadIdx.x == 0) epilogue_ranges(p.epi);
 }
 

@@ -84,10 +84,8 @@ __global__ __launch_bounds__(Cfg::kThreads) void fc_dma_kernel(FcArgs p) {
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 
-  static_assert(NS * Cfg::STAGE_SLOTS * 16 >=
-                    Cfg::BN * 4 + (Cfg::kThreads / 64) * Cfg::TM * (Cfg::TN + 16),
-                "stage ring too small for the epilogue transpose");
-  gemm_epilogue_lds<Cfg>(acc, p.epi, pre, m0, n0, p.M, p.N, static_cast<size_t>(p.ldo), lds);
+  gemm_epilogue_lds<Cfg, NS * Cfg::STAGE_SLOTS * 16>(acc, p.epi, pre, m0, n0, p.M, p.N,
+                                                     static_cast<size_t>(p.ldo), lds);
   if (blockIdx.x == 0 && threadIdx.x == 0) epilogue_ranges(p.epi);
 }
 
@@ -159,12 +157,8 @@ void launch_fc(hipStream_t s, const int8_t* data, const int8_t* weight, int M, i
       return static_cast<long>((M + bm - 1) / bm) * ((N + bn - 1) / bn);
     };
     if (buf_ok) {
-      // the 256 x 256 tile runs 8 waves when only int8 is written and 4 waves (128 x 128
-      // wave tiles) when int32 is stored as well
       switch (choose_tile(M, N, K, cus)) {
-        case Tile::kL8:
-          cfg = glb_ok ? ((epi.out32 != nullptr) ? 16 : 12) : ((epi.out32 != nullptr) ? 32 : 31);
-          break;
+        case Tile::kL8: cfg = glb_ok ? 12 : 31; break;
         case Tile::kW128x2: cfg = 41; break;
         case Tile::kM128x2: cfg = 43; break;
         case Tile::kM128x4: cfg = 23; break;

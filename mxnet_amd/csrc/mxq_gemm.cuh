@@ -652,11 +652,30 @@ __device__ __forceinline__ EpiPre epi_prefetch(const Epilogue& e, int n0, int N)
   return p;
 }
 
+// Bytes of the stage ring one wave uses as scratch in gemm_epilogue_lds: its int8 tile
+// (row pitch TN + 16) and, when the ring is large enough, one 32 x 32 int32 MFMA tile
+// (row pitch 36 dwords: 16-byte aligned rows whose 16-lane write groups cover all banks).
 template <class Cfg>
+struct EpiScratch {
+  static constexpr int kTile8 = Cfg::TM * (Cfg::TN + 16);
+  static constexpr int kPitch32 = 36;
+  static constexpr int kTile32 = 32 * kPitch32 * 4;
+  static constexpr int kPerWave = kTile8 > kTile32 ? kTile8 : kTile32;
+  static constexpr int kWaves = Cfg::kThreads / 64;
+  // the int8 tile always has to fit; the int32 tile is optional
+  static constexpr int kNeed8 = Cfg::BN * 4 + kWaves * kTile8;
+  static constexpr int kNeed32 = Cfg::BN * 4 + kWaves * kPerWave;
+};
+
+template <class Cfg, int RING_BYTES>
 __device__ __forceinline__ void gemm_epilogue_lds(v16i (&acc)[Cfg::MI][Cfg::NI],
                                                   const Epilogue& e, const EpiPre& pre, int m0,
                                                   int n0, int M, int N, size_t ldo,
                                                   v4i* lds_v) {
+  typedef EpiScratch<Cfg> Scratch;
+  static_assert(RING_BYTES >= Scratch::kNeed8, "stage ring too small for the epilogue transpose");
+  constexpr bool kStage32 = RING_BYTES >= Scratch::kNeed32;
+  constexpr int kPerWave = kStage32 ? Scratch::kPerWave : Scratch::kTile8;
   constexpr int TM = Cfg::TM, TN = Cfg::TN, MI = Cfg::MI, NI = Cfg::NI;
   constexpr int LD = TN + 16;        // staged row pitch in bytes (keeps 16-byte alignment)
   constexpr int LPR = TN / 16;       // lanes per staged row on the way out
@@ -665,15 +684,19 @@ __device__ __forceinline__ void gemm_epilogue_lds(v16i (&acc)[Cfg::MI][Cfg::NI],
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave / Cfg::WN, wn = wave % Cfg::WN;
   const int m_base = m0 + wm * TM, n_base = n0 + wn * TN;
-  const bool fast = (N % 16 == 0) && (ldo % 16 == 0) &&
-                    ((reinterpret_cast<uintptr_t>(e.out8) & 15u) == 0);
-  if (!fast) {
+  const bool fast8 = e.out8 == nullptr ||
+                     ((N % 16 == 0) && (ldo % 16 == 0) &&
+                      ((reinterpret_cast<uintptr_t>(e.out8) & 15u) == 0));
+  const bool fast32 = e.out32 == nullptr ||
+                      ((N % 4 == 0) && (ldo % 4 == 0) &&
+                       ((reinterpret_cast<uintptr_t>(e.out32) & 15u) == 0));
+  if (!(fast8 && fast32)) {
     gemm_epilogue<Cfg>(acc, e, m_base, n_base, M, N, ldo);
     return;
   }
   char* lds = reinterpret_cast<char*>(lds_v);
   int* sbias = reinterpret_cast<int*>(lds);
-  char* stage = lds + Cfg::BN * 4 + wave * (TM * LD);
+  char* stage = lds + Cfg::BN * 4 + wave * kPerWave;
   const EpiScalars s = pre.s;
 
   __syncthreads();  // every wave is done reading operand stages
@@ -681,6 +704,7 @@ __device__ __forceinline__ void gemm_epilogue_lds(v16i (&acc)[Cfg::MI][Cfg::NI],
   __syncthreads();
 
   const int lrow = lane & 31, lgrp = lane >> 5;
+  // accumulator + bias in place: both outputs below start from it
 #pragma unroll
   for (int ni = 0; ni < NI; ++ni) {
 #pragma unroll
@@ -688,32 +712,81 @@ __device__ __forceinline__ void gemm_epilogue_lds(v16i (&acc)[Cfg::MI][Cfg::NI],
       const int nl = ni * 32 + 8 * vq + 4 * lgrp;  // column inside the wave tile
       const v4i b = *reinterpret_cast<const v4i*>(sbias + wn * TN + nl);
 #pragma unroll
-      for (int mi = 0; mi < MI; ++mi) {
-        int v[4];
+      for (int mi = 0; mi < MI; ++mi)
 #pragma unroll
         for (int i = 0; i < 4; ++i)
-          v[i] = static_cast<int>(static_cast<uint32_t>(acc[mi][ni][4 * vq + i]) +
-                                  static_cast<uint32_t>(b[i]));
-        const int ml = mi * 32 + lrow;
-        if (e.out32 != nullptr) {
-          const int m = m_base + ml, n = n_base + nl;
-          if (m < M && n < N) {
-            v4i w = {v[0], v[1], v[2], v[3]};
-            *reinterpret_cast<v4i*>(e.out32 + static_cast<size_t>(m) * ldo + n) = w;
-          }
-        }
-        if (e.out8 != nullptr) {
-          int q[4];
-#pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            q[i] = epi_requant(v[i], s, e.relu ? 0.0f : -127.0f);
-          }
-          *reinterpret_cast<uint32_t*>(stage + ml * LD + nl) = pack_bytes(q[0], q[1], q[2], q[3]);
-        }
-      }
+          acc[mi][ni][4 * vq + i] = static_cast<int>(
+              static_cast<uint32_t>(acc[mi][ni][4 * vq + i]) + static_cast<uint32_t>(b[i]));
     }
   }
+
+  if (e.out32 != nullptr) {
+    if (kStage32) {
+      // One 32 x 32 MFMA tile at a time through the wave's scratch: a lane holds 4
+      // adjacent columns of one row per register quad, which stored directly touches 32
+      // rows with 32 bytes each; read back, 8 lanes cover one 128-byte row and a store
+      // instruction writes 8 whole cache lines.
+      int* t32 = reinterpret_cast<int*>(stage);
+#pragma unroll
+      for (int mi = 0; mi < MI; ++mi) {
+#pragma unroll
+        for (int ni = 0; ni < NI; ++ni) {
+#pragma unroll
+          for (int vq = 0; vq < 4; ++vq) {
+            const v4i w = {acc[mi][ni][4 * vq], acc[mi][ni][4 * vq + 1], acc[mi][ni][4 * vq + 2],
+                           acc[mi][ni][4 * vq + 3]};
+            *reinterpret_cast<v4i*>(t32 + lrow * Scratch::kPitch32 + 8 * vq + 4 * lgrp) = w;
+          }
+          asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+          __builtin_amdgcn_wave_barrier();
+          v4i back[4];
+#pragma unroll
+          for (int it = 0; it < 4; ++it)
+            back[it] = *reinterpret_cast<const v4i*>(t32 + (it * 8 + (lane >> 3)) *
+                                                               Scratch::kPitch32 +
+                                                     (lane & 7) * 4);
+          asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+          __builtin_amdgcn_wave_barrier();
+#pragma unroll
+          for (int it = 0; it < 4; ++it) {
+            const int m = m_base + mi * 32 + it * 8 + (lane >> 3);
+            const int n = n_base + ni * 32 + (lane & 7) * 4;
+            if (m < M && n < N)
+              *reinterpret_cast<v4i*>(e.out32 + static_cast<size_t>(m) * ldo + n) = back[it];
+          }
+        }
+      }
+    } else {
+#pragma unroll
+      for (int ni = 0; ni < NI; ++ni)
+#pragma unroll
+        for (int vq = 0; vq < 4; ++vq)
+#pragma unroll
+          for (int mi = 0; mi < MI; ++mi) {
+            const int m = m_base + mi * 32 + lrow, n = n_base + ni * 32 + 8 * vq + 4 * lgrp;
+            if (m < M && n < N) {
+              const v4i w = {acc[mi][ni][4 * vq], acc[mi][ni][4 * vq + 1],
+                             acc[mi][ni][4 * vq + 2], acc[mi][ni][4 * vq + 3]};
+              *reinterpret_cast<v4i*>(e.out32 + static_cast<size_t>(m) * ldo + n) = w;
+            }
+          }
+    }
+  }
+
   if (e.out8 != nullptr) {
+    const float lo = e.relu ? 0.0f : -127.0f;
+#pragma unroll
+    for (int ni = 0; ni < NI; ++ni)
+#pragma unroll
+      for (int vq = 0; vq < 4; ++vq)
+#pragma unroll
+        for (int mi = 0; mi < MI; ++mi) {
+          const int nl = ni * 32 + 8 * vq + 4 * lgrp, ml = mi * 32 + lrow;
+          int q[4];
+#pragma unroll
+          for (int i = 0; i < 4; ++i) q[i] = epi_requant(acc[mi][ni][4 * vq + i], s, lo);
+          *reinterpret_cast<uint32_t*>(stage + ml * LD + nl) = pack_bytes(q[0], q[1], q[2], q[3]);
+        }
     // the wave reads back what its own lanes wrote: LDS executes a wave's
     // instructions in order, the wait makes the writes complete first
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
