@@ -346,6 +346,32 @@ class GraphWorkload:
     def value(self, sec_per_step):
         return self.ops / sec_per_step / 1e12, "TOPS"
 
+    def time_alone(self, torch, body, reps=10, replays=30):
+        """Average time of one pass of `body` when it is the only thing running: captured
+        `reps` times into its own graph.  Its operands stay cache-warm between passes, so
+        this is an upper bound on what the same launches reach inside the whole step."""
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            body()
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            for _ in range(reps):
+                body()
+        for _ in range(5):
+            g.replay()
+        e0 = torch.cuda.Event(enable_timing=True)
+        e1 = torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        e0.record()
+        for _ in range(replays):
+            g.replay()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / 1e3 / (reps * replays)
+
     def cpu_baseline(self, oracle, budget_s=0):
         return None
 
@@ -393,16 +419,31 @@ class ConvStackWorkload(GraphWorkload):
             self.ops += 2.0 * N * OH * OH * O * k * k * C
             del x, w, ref
 
-        def body():
+        def body(only=None):
             st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
-            for (d, wq, bq, dmin, dmax, wmin, wmax, bmin, bmax, out8, sc, geo, r) in self.layers:
+            for i, (d, wq, bq, dmin, dmax, wmin, wmax, bmin, bmax, out8, sc, geo,
+                    r) in enumerate(self.layers):
+                if only is not None and i != only:
+                    continue
                 rc = lib.mxq_quantized_conv_nhwc(st, P(d), P(wq), P(bq), *geo, 1, 1, P(dmin),
                                                  P(dmax), P(wmin), P(wmax), P(bmin), P(bmax),
                                                  None, P(sc[0]), P(sc[1]), P(out8), P(sc[2]),
                                                  P(sc[3]), 1, -r, r)
                 if rc != 0:
                     raise RuntimeError(lib.mxq_last_error().decode())
+        self.body = body
         self.capture(torch, body)
+
+    def per_layer(self, torch):
+        rows = []
+        for i, (H, C, O, k, s) in enumerate(RESNET50_CONVS):
+            pad = 1 if k == 3 else 0
+            OH = (H + 2 * pad - k) // s + 1
+            ops = 2.0 * 64 * OH * OH * O * k * k * C
+            t = self.time_alone(torch, lambda: self.body(i))
+            rows.append({"layer": "%dx%d %d->%d k%d s%d" % (H, H, C, O, k, s),
+                         "us": round(t * 1e6, 2), "TOPS": round(ops / t / 1e12, 1)})
+        return rows
 
 
 BERT_FCS = [(768, 2304), (768, 768), (768, 3072), (3072, 768)]
@@ -445,9 +486,11 @@ class BertChainWorkload(GraphWorkload):
             self.ops += 2.0 * M * N * K
             del w
 
-        def body():
+        def body(only=None):
             st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
-            for (K, N, wq, bq, wmin, wmax, bmin, bmax, r, B) in self.layers:
+            for i, (K, N, wq, bq, wmin, wmax, bmin, bmax, r, B) in enumerate(self.layers):
+                if only is not None and i != only:
+                    continue
                 sc = B["sc"]
                 if fused:
                     rcs = [
@@ -473,7 +516,17 @@ class BertChainWorkload(GraphWorkload):
                     lib.mxq_dequantize(st, P(B["q8"]), 5, P(sc[4]), P(sc[5]), P(B["y"]), M * N)]
                 if any(rcs):
                     raise RuntimeError(lib.mxq_last_error().decode())
+        self.body = body
         self.capture(torch, body)
+
+    def per_layer(self, torch):
+        """One layer's launches (cast operators included) alone."""
+        rows = []
+        for i, (K, N) in enumerate(BERT_FCS):
+            t = self.time_alone(torch, lambda: self.body(i))
+            rows.append({"layer": "M=4096 K=%d N=%d" % (K, N), "us": round(t * 1e6, 2),
+                         "TOPS": round(2.0 * 4096 * N * K / t / 1e12, 1)})
+        return rows
 
 
 def mfma_context(torch, S):
@@ -618,6 +671,8 @@ def main():
 
     if isinstance(wl, FcWorkload):
         line["roofline"]["context"] = mfma_context(torch, wl.S)
+    if isinstance(wl, GraphWorkload):
+        line["roofline"]["layers_alone"] = wl.per_layer(torch)
 
     if not args.no_cast_ops:
         rows = []
@@ -631,6 +686,8 @@ def main():
             wall2, ev2 = timed_run(torch, w2, steps2, 300)
             r = roofline_of(w2, ev2 / steps2, kind)
             r["workload"] = w2.name
+            if isinstance(w2, GraphWorkload):
+                r["layers_alone"] = w2.per_layer(torch)
             rows.append(r)
             del w2
             torch.cuda.empty_cache()

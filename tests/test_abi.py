@@ -78,3 +78,13 @@ def test_no_fallback_without_library(tmp_path, monkeypatch):
         sys.modules.pop("mxnet_amd_copy", None)
         for k in [k for k in sys.modules if k.startswith("mxnet_amd_copy.")]:
             sys.modules.pop(k)
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """bench.py measures one GPU: any other --gpus value exits with a message."""
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"],
+                       capture_output=True, text=True, timeout=120)
+    assert r.returncode == 2 and "one GPU" in r.stderr
