@@ -112,18 +112,26 @@ __device__ __forceinline__ float to_float(int32_t x) { return static_cast<float>
 template <typename SrcT, typename Rule, bool PRE>
 __device__ __forceinline__ void narrow_stream(const SrcT* __restrict__ in,
                                               uint8_t* __restrict__ out, size_t n, Rule rule,
-                                              float pre) {
+                                              float pre, bool rev = false) {
   typedef SrcT Vec4 __attribute__((ext_vector_type(4)));
   const size_t nquad = n >> 2;  // groups of 4 elements
   const Vec4* in4 = reinterpret_cast<const Vec4*>(in);
   uint32_t* out4 = reinterpret_cast<uint32_t*>(out);
+  if (rev) {
+    // back to front: the tail of the tensor, which the range reduction read last, is what
+    // the memory-side cache still holds (measured: 3 % off the two-launch time at 256 MB)
+    in4 += nquad - 1;
+    out4 += nquad - 1;
+  }
+  const ptrdiff_t dir = rev ? -1 : 1;
   const size_t stride = size_t(gridDim.x) * kThreads;
   size_t q = size_t(blockIdx.x) * kThreads + threadIdx.x;
   // main loop: kUnroll segments, each `stride` quads apart
   for (; q + size_t(kUnroll - 1) * stride < nquad; q += size_t(kUnroll) * stride) {
     Vec4 x[kUnroll];
 #pragma unroll
-    for (int j = 0; j < kUnroll; ++j) x[j] = nt_load(in4 + q + size_t(j) * stride);
+    for (int j = 0; j < kUnroll; ++j)
+      x[j] = nt_load(in4 + dir * static_cast<ptrdiff_t>(q + size_t(j) * stride));
 #pragma unroll
     for (int j = 0; j < kUnroll; ++j) {
       float f0 = to_float(x[j].x), f1 = to_float(x[j].y), f2 = to_float(x[j].z),
@@ -134,11 +142,12 @@ __device__ __forceinline__ void narrow_stream(const SrcT* __restrict__ in,
         f2 = f2 * pre;
         f3 = f3 * pre;
       }
-      stream_store(pack4(rule(f0), rule(f1), rule(f2), rule(f3)), out4 + q + size_t(j) * stride);
+      stream_store(pack4(rule(f0), rule(f1), rule(f2), rule(f3)),
+                   out4 + dir * static_cast<ptrdiff_t>(q + size_t(j) * stride));
     }
   }
   for (; q < nquad; q += stride) {
-    Vec4 x = nt_load(in4 + q);
+    Vec4 x = nt_load(in4 + dir * static_cast<ptrdiff_t>(q));
     float f0 = to_float(x.x), f1 = to_float(x.y), f2 = to_float(x.z), f3 = to_float(x.w);
     if (PRE) {
       f0 = f0 * pre;
@@ -146,7 +155,8 @@ __device__ __forceinline__ void narrow_stream(const SrcT* __restrict__ in,
       f2 = f2 * pre;
       f3 = f3 * pre;
     }
-    stream_store(pack4(rule(f0), rule(f1), rule(f2), rule(f3)), out4 + q);
+    stream_store(pack4(rule(f0), rule(f1), rule(f2), rule(f3)),
+                 out4 + dir * static_cast<ptrdiff_t>(q));
   }
   // ragged tail (< 4 elements)
   if (blockIdx.x == 0) {
@@ -265,7 +275,7 @@ __global__ __launch_bounds__(kThreads) void quantize_kernel(const float* __restr
                                                             const float* __restrict__ dlo,
                                                             const float* __restrict__ dhi,
                                                             const uint32_t* __restrict__ parts,
-                                                            int nparts) {
+                                                            int nparts, int rev) {
   if (dlo != nullptr) {
     lo = *dlo;
     hi = *dhi;
@@ -277,7 +287,7 @@ __global__ __launch_bounds__(kThreads) void quantize_kernel(const float* __restr
     rule.lo = lo;
     rule.s = static_cast<float>((255.0 - 0.0) / static_cast<double>(hi - lo));
     if (VEC)
-      narrow_stream<float, QuantU8, false>(in, out, n, rule, 0.f);
+      narrow_stream<float, QuantU8, false>(in, out, n, rule, 0.f, rev != 0);
     else
       narrow_scalar<float, QuantU8, false>(in, out, n, rule, 0.f);
     if (blockIdx.x == 0 && threadIdx.x == 0) {
@@ -289,7 +299,7 @@ __global__ __launch_bounds__(kThreads) void quantize_kernel(const float* __restr
     QuantI8 rule;
     rule.s = 127.0f / r;
     if (VEC)
-      narrow_stream<float, QuantI8, false>(in, out, n, rule, 0.f);
+      narrow_stream<float, QuantI8, false>(in, out, n, rule, 0.f, rev != 0);
     else
       narrow_scalar<float, QuantI8, false>(in, out, n, rule, 0.f);
     if (blockIdx.x == 0 && threadIdx.x == 0) {
@@ -307,7 +317,7 @@ __global__ __launch_bounds__(kThreads) void requantize_kernel(
     const int32_t* __restrict__ in, uint8_t* __restrict__ out, float* __restrict__ omin,
     float* __restrict__ omax, size_t n, const float* __restrict__ imin,
     const float* __restrict__ imax, float real_range, const uint32_t* __restrict__ parts,
-    int nparts) {
+    int nparts, int rev) {
   const float in_scale = maxabs(*imin, *imax) / 2147483648.0f;
   if (parts != nullptr) {
     float lo, hi;
@@ -317,7 +327,7 @@ __global__ __launch_bounds__(kThreads) void requantize_kernel(
   QuantI8 rule;
   rule.s = 127.0f / maxabs(-real_range, real_range);
   if (VEC)
-    narrow_stream<int32_t, QuantI8, true>(in, out, n, rule, in_scale);
+    narrow_stream<int32_t, QuantI8, true>(in, out, n, rule, in_scale, rev != 0);
   else
     narrow_scalar<int32_t, QuantI8, true>(in, out, n, rule, in_scale);
   if (blockIdx.x == 0 && threadIdx.x == 0) {
@@ -616,7 +626,8 @@ void launch_quantize(hipStream_t s, const float* in, void* out, float* omin, flo
   uint8_t* o = static_cast<uint8_t*>(out);
 #define MXQ_Q(U, V) \
   hipLaunchKernelGGL((quantize_kernel<U, V>), dim3(grid), dim3(kThreads), 0, s, in, o, omin, \
-                     omax, n, lo, hi, dlo, dhi, parts, nparts)
+                     omax, n, lo, hi, dlo, dhi, parts, nparts,                           \
+                     parts != nullptr ? 1 : 0)
   if (out_type == MXQ_UINT8) {
     if (vec) MXQ_Q(true, true); else MXQ_Q(true, false);
   } else {
@@ -740,10 +751,12 @@ int mxq_requantize(void* stream, const int32_t* in, const float* imin, const flo
   }
   if (vec)
     hipLaunchKernelGGL((requantize_kernel<true>), dim3(grid), dim3(kThreads), 0, s, in, o, omin,
-                       omax, n, imin, imax, real_range, parts, nparts);
+                       omax, n, imin, imax, real_range, parts, nparts,
+                       parts != nullptr ? 1 : 0);
   else
     hipLaunchKernelGGL((requantize_kernel<false>), dim3(grid), dim3(kThreads), 0, s, in, o,
-                       omin, omax, n, imin, imax, real_range, parts, nparts);
+                       omin, omax, n, imin, imax, real_range, parts, nparts,
+                       parts != nullptr ? 1 : 0);
   MXQ_LAUNCH_CHECK();
   MXQ_API_END();
 }
