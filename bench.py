@@ -50,7 +50,7 @@ def parse_args():
     ap.add_argument("--workload", default="fc4096",
                     choices=["fc4096", "fc8192", "quantize", "quantize_uncal", "quantize_uint8",
                              "requantize", "requantize_uncal", "dequantize", "copy", "maxpool", "avgpool",
-                             "resnet50_convs", "bert_fc_chain", "bert_fc_chain_fused"])
+                             "elemwise_add", "elemwise_add_int8", "concat", "resnet50_convs", "bert_fc_chain", "bert_fc_chain_fused"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-cast-ops", action="store_true")
     return ap.parse_args()
@@ -186,6 +186,37 @@ class CastWorkload:
             self.bytes = 5.0 * n
             self.kernel = "dequantize_kernel"
             self.name = "dequantize int8->fp32"
+        elif kind in ("elemwise_add", "elemwise_add_int8"):
+            self.src = [torch.randint(-127, 128, (n,), device="cuda", generator=g,
+                                      dtype=torch.int8) for _ in range(self.NBUF)]
+            self.rhs = [torch.randint(-127, 128, (n,), device="cuda", generator=g,
+                                      dtype=torch.int8) for _ in range(self.NBUF)]
+            out_dtype = torch.int32 if kind == "elemwise_add" else torch.int8
+            self.dst = [torch.empty(n, dtype=out_dtype, device="cuda") for _ in range(self.NBUF)]
+            self.imin = torch.tensor([-3.0], device="cuda")
+            self.imax = torch.tensor([3.0], device="cuda")
+            self.bytes = (6.0 if kind == "elemwise_add" else 3.0) * n
+            self.kernel = "add_kernel"
+            self.name = ("quantized_elemwise_add int8+int8->" +
+                         ("int32" if kind == "elemwise_add" else "int8 calibrated (-5,5)"))
+        elif kind == "concat":
+            half = n // 2
+            self.src = [torch.randint(-127, 128, (half,), device="cuda", generator=g,
+                                      dtype=torch.int8) for _ in range(self.NBUF)]
+            self.rhs = [torch.randint(-127, 128, (half,), device="cuda", generator=g,
+                                      dtype=torch.int8) for _ in range(self.NBUF)]
+            self.dst = [torch.empty(n, dtype=torch.int8, device="cuda") for _ in range(self.NBUF)]
+            self.ranges = [torch.tensor([v], device="cuda") for v in (-1.0, 1.0, -2.0, 2.0)]
+            self.c_types = (ctypes.c_int * 2)(5, 5)
+            self.c_mins = (ctypes.c_void_p * 2)(self.ranges[0].data_ptr(),
+                                                self.ranges[2].data_ptr())
+            self.c_maxs = (ctypes.c_void_p * 2)(self.ranges[1].data_ptr(),
+                                                self.ranges[3].data_ptr())
+            self.c_ext = (ctypes.c_int64 * 2)(half, half)
+            self.bytes = 2.0 * n
+            self.kernel = "concat_kernel"
+            self.name = "quantized_concat of two int8 halves, ranges (-1,1) and (-2,2): " \
+                        "one half rescaled, one copied"
         else:
             raise ValueError(kind)
         self.name += ", %d elements" % n
@@ -214,6 +245,21 @@ class CastWorkload:
             rc = lib.mxq_requantize(st, P(self.src[k]), P(self.imin), P(self.imax),
                                     P(self.dst[k]), P(self.omin), P(self.omax), n, 0, 0.0, 0.0,
                                     P(self.ws), self.ws.numel())
+        elif kind == "concat":
+            ptrs = (ctypes.c_void_p * 2)(self.src[k].data_ptr(), self.rhs[k].data_ptr())
+            rc = lib.mxq_quantized_concat(st, 2, ptrs, self.c_types, self.c_mins, self.c_maxs,
+                                          self.c_ext, 1, 1, P(self.dst[k]), 5, P(self.omin),
+                                          P(self.omax))
+        elif kind == "elemwise_add":
+            rc = lib.mxq_quantized_elemwise_add(st, P(self.src[k]), 5, P(self.rhs[k]), 5,
+                                                P(self.imin), P(self.imax), P(self.imin),
+                                                P(self.imax), P(self.dst[k]), 4, P(self.omin),
+                                                P(self.omax), n, 0, 0.0, 0.0)
+        elif kind == "elemwise_add_int8":
+            rc = lib.mxq_quantized_elemwise_add(st, P(self.src[k]), 5, P(self.rhs[k]), 5,
+                                                P(self.imin), P(self.imax), P(self.imin),
+                                                P(self.imax), P(self.dst[k]), 5, P(self.omin),
+                                                P(self.omax), n, 1, -5.0, 5.0)
         else:
             rc = lib.mxq_dequantize(st, P(self.src[k]), 5, P(self.imin), P(self.imax),
                                     P(self.dst[k]), n)
@@ -240,11 +286,17 @@ class CastWorkload:
                 oracle.requantize(x, -1.0, 1.0, -0.1, 0.1)
             elif kind == "requantize_uncal":
                 oracle.requantize(x, -1.0, 1.0)
+            elif kind == "concat":
+                oracle.quantized_concat([x[:n // 2], x[n // 2:]], [-1.0, -2.0], [1.0, 2.0], dim=0)
+            elif kind == "elemwise_add":
+                oracle.quantized_elemwise_add(x, x, -3.0, 3.0, -3.0, 3.0)
+            elif kind == "elemwise_add_int8":
+                oracle.quantized_elemwise_add(x, x, -3.0, 3.0, -3.0, 3.0, -5.0, 5.0)
             else:
                 oracle.dequantize(x, -3.0, 3.0)
             reps += 1
             dt = time.perf_counter() - t0
-            if dt > budget_s / 2 or reps >= 50:
+            if dt > budget_s / 2 or reps >= 2000:
                 break
         gbs = self.bytes / self.N * n * reps / dt / 1e9
         return {"value": gbs, "unit": "GB/s", "cores": oracle.num_threads(), "kind": "port",
@@ -677,7 +729,8 @@ def main():
     if not args.no_cast_ops:
         rows = []
         for kind in ["quantize", "quantize_uint8", "quantize_uncal", "requantize",
-                     "requantize_uncal", "dequantize", "maxpool", "avgpool", "fc8192",
+                     "requantize_uncal", "dequantize", "elemwise_add", "elemwise_add_int8",
+                     "concat", "maxpool", "avgpool", "fc8192",
                      "resnet50_convs", "bert_fc_chain", "bert_fc_chain_fused"]:
             if kind == args.workload:
                 continue

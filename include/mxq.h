@@ -119,6 +119,38 @@ int mxq_quantized_pooling_nchw(void* stream, const void* in, int in_type, int N,
 int mxq_quantized_flatten(void* stream, const void* in, const float* imin, const float* imax,
                           void* out, float* omin, float* omax, size_t n_bytes);
 
+/* ---- _contrib_quantized_elemwise_add ---------------------------------------------
+ * Replaces DNNLQuantizedElemwiseAddForward
+ * (src/operator/quantization/dnnl/dnnl_quantized_elemwise_add.cc:134-257; the operator is
+ * cpu-only in the reference, quantized_elemwise_add.cc:80-87) for operands of one shape:
+ * out = saturate(nearest-even(lhs * s0 + rhs * s1)) in binary32, s = output scale / input
+ * scale with the reference's ranges (127.5 int8, 255.5 uint8, 2^31 - 1 int32).
+ * Uncalibrated: out is int32 over (-(|A|+|B|), |A|+|B|).  Calibrated: out has the inputs'
+ * type (int8 when they differ) over (min_calib, max_calib).  A uint8 operand beside an
+ * int8 one is first halved to int8, as the reference does.  The rounding itself lives
+ * inside oneDNN in the reference and is not pinned by its sources (its test accepts a
+ * dequantized error of 2). */
+int mxq_quantized_elemwise_add(void* stream, const void* lhs, int lhs_type, const void* rhs,
+                               int rhs_type, const float* lhs_min, const float* lhs_max,
+                               const float* rhs_min, const float* rhs_max, void* out, int out_type,
+                               float* omin, float* omax, size_t n, int calibrated,
+                               float min_calib, float max_calib);
+
+/* ---- _contrib_quantized_concat -----------------------------------------------------
+ * Replaces DNNLQuantizedConcatForward
+ * (src/operator/quantization/dnnl/dnnl_quantized_concat.cc:41-115; cpu-only in the
+ * reference).  Input i is [outer, in_axis[i], inner] contiguous, the output
+ * [outer, sum in_axis, inner].  Output range = hull of the input ranges and 0; out_type is
+ * int8 as soon as one input is (quantized_concat.cc:83-103).  An input whose scale equals
+ * the output's is copied, any other is rescaled: saturate(nearest-even(x * out_scale /
+ * in_scale)) in binary32 (oneDNN's reorder; same caveat as above).  in, in_type, in_min,
+ * in_max, in_axis are host arrays of num_args entries; the data and range pointers in
+ * them are device pointers. */
+int mxq_quantized_concat(void* stream, int num_args, const void* const* in, const int* in_type,
+                         const float* const* in_min, const float* const* in_max,
+                         const int64_t* in_axis, int64_t outer, int64_t inner, void* out,
+                         int out_type, float* omin, float* omax);
+
 /* ---- _contrib_quantized_fully_connected ----------------------------------
  * Replaces QuantizedFullyConnectedForwardGPU
  * (src/operator/quantization/quantized_fully_connected.cu:58-138): cublasGemmEx

@@ -40,6 +40,10 @@ SIGNATURES = {
     "mxq_quantized_relu": (_i, [_p, _p, _p, _p, _p, _p, _p, _sz]),
     "mxq_quantized_pooling_nchw": (_i, [_p, _p, _i] + [_i] * 12 + [_i, _i, _p, _p, _p, _p, _p]),
     "mxq_quantized_flatten": (_i, [_p, _p, _p, _p, _p, _p, _p, _sz]),
+    "mxq_quantized_elemwise_add": (_i, [_p, _p, _i, _p, _i, _p, _p, _p, _p, _p, _i, _p, _p, _sz,
+                                        _i, _f, _f]),
+    "mxq_quantized_concat": (_i, [_p, _i, _p, _p, _p, _p, _p, ctypes.c_int64, ctypes.c_int64, _p,
+                                  _i, _p, _p]),
     "mxq_quantized_fc": (_i, [_p, _p, _p, _p, _i, _i, _i] + [_p] * 6 + [_p, _p, _p, _p, _p, _p,
                               _i, _f, _f]),
     "mxq_quantized_conv_nhwc": (_i, [_p, _p, _p, _p] + [_i] * 13 + [_p] * 6 +

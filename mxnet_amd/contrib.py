@@ -66,3 +66,16 @@ def quantized_pooling(data, min_data, max_data, kernel=None, pool_type="max", gl
 
 def quantized_flatten(data, min_data, max_data):
     return invoke("_contrib_quantized_flatten", data, min_data, max_data)
+
+
+def quantized_elemwise_add(lhs, rhs, lhs_min, lhs_max, rhs_min, rhs_max, min_calib_range=None,
+                           max_calib_range=None):
+    return invoke("_contrib_quantized_elemwise_add", lhs, rhs, lhs_min, lhs_max, rhs_min,
+                  rhs_max, min_calib_range=min_calib_range, max_calib_range=max_calib_range)
+
+
+def quantized_concat(*data, num_args=None, dim=1):
+    """`data` is arg0..argN-1 followed by (arg0_min, arg0_max, ..., argN-1_min, argN-1_max)."""
+    if num_args is None:
+        num_args = len(data) // 3
+    return invoke("_contrib_quantized_concat", *data, num_args=num_args, dim=dim)

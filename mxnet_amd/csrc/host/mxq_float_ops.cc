@@ -168,18 +168,44 @@ NNVM_REGISTER_OP(Dropout)
     .set_attr<nnvm::FNumVisibleOutputs>("FNumVisibleOutputs",
                                         [](const NodeAttrs&) { return 1U; });
 
-// src/operator/tensor/elemwise_binary_op_basic.cc:85-110 (quantized only by oneDNN in
-// the reference, quantized_elemwise_add.cc:130)
+// src/operator/tensor/elemwise_binary_op_basic.cc:82-110, quantized_elemwise_add.cc:124-133
 NNVM_REGISTER_OP(elemwise_add)
     .add_alias("_add")
     .add_alias("_plus")
+    .add_alias("_Plus")
     .set_num_inputs(2)
     .set_num_outputs(1)
     .set_attr<nnvm::FListInputNames>("FListInputNames",
                                      [](const NodeAttrs&) {
                                        return std::vector<std::string>{"lhs", "rhs"};
                                      })
-    .set_attr<nnvm::FListOutputNames>("FListOutputNames", OneOutput);
+    .set_attr<nnvm::FListOutputNames>("FListOutputNames", OneOutput)
+    .set_attr<FQuantizedOp>("FQuantizedOp", [](const NodeAttrs& attrs) {
+      return QuantizedTwin(attrs, "_contrib_quantized_elemwise_add");
+    });
+
+// src/operator/nn/concat.cc:325-411, quantized_concat.cc:143-152
+NNVM_REGISTER_OP(Concat)
+    .add_alias("concat")
+    .set_num_inputs([](const NodeAttrs& attrs) {
+      return static_cast<uint32_t>(nnvm::get<ConcatParam>(attrs.parsed).num_args);
+    })
+    .set_num_outputs(1)
+    .set_attr_parser(ParamParser<ConcatParam>)
+    .set_attr<nnvm::FListInputNames>("FListInputNames",
+                                     [](const NodeAttrs& attrs) {
+                                       const ConcatParam& params =
+                                           nnvm::get<ConcatParam>(attrs.parsed);
+                                       std::vector<std::string> ret;
+                                       for (int i = 0; i < params.num_args; ++i)
+                                         ret.push_back("arg" + std::to_string(i));
+                                       return ret;
+                                     })
+    .set_attr<nnvm::FListOutputNames>("FListOutputNames", OneOutput)
+    .set_attr<std::string>("key_var_num_args", "num_args")
+    .set_attr<FQuantizedOp>("FQuantizedOp", [](const NodeAttrs& attrs) {
+      return QuantizedTwin(attrs, "_contrib_quantized_concat");
+    });
 
 }  // namespace op
 }  // namespace mxnet

@@ -10,6 +10,8 @@
 //   ActivationParam        src/operator/nn/activation-inl.h (act_type only)
 //   PoolingParam           src/operator/nn/pooling-inl.h:45-120 (+ PoolingParamParser,
 //                          src/operator/nn/pooling.cc:35-64)
+//   QuantizeElemwiseAddParam  src/operator/quantization/quantized_elemwise_add-inl.h:34-51
+//   ConcatParam            src/operator/nn/concat-inl.h:48-64
 // Same field names, defaults, enum strings and error behaviour (unknown keys are
 // errors unless they look like __hidden__ keys).
 #ifndef MXQ_PARAMS_H_
@@ -496,6 +498,57 @@ inline void ConvolutionParamParser(nnvm::NodeAttrs* attrs) {
       << "Padding must have the same number of dimensions with kernel_size,"
       << "but kernel_size is set to " << param_.kernel << " while padding is " << param_.pad;
   attrs->parsed = std::move(param_);
+}
+
+struct QuantizeElemwiseAddParam {
+  dmlc::optional<float> min_calib_range;
+  dmlc::optional<float> max_calib_range;
+  void Init(const param_detail::Dict& d) {
+    using namespace param_detail;
+    check_unknown(d, {"min_calib_range", "max_calib_range"}, "QuantizeElemwiseAddParam");
+    min_calib_range = get_optional_float(d, "min_calib_range");
+    max_calib_range = get_optional_float(d, "max_calib_range");
+  }
+  static std::vector<nnvm::ParamFieldInfo> __FIELDS__() {
+    return {{"min_calib_range", "float or None, optional, default=None",
+             "The minimum scalar value in the form of float32 obtained through calibration. If "
+             "present, it will be used to requantize the int8 output data."},
+            {"max_calib_range", "float or None, optional, default=None",
+             "The maximum scalar value in the form of float32 obtained through calibration. If "
+             "present, it will be used to requantize the int8 output data."}};
+  }
+};
+
+struct ConcatParam {
+  int num_args = 0;
+  dmlc::optional<int> dim = dmlc::optional<int>(1);
+  void Init(const param_detail::Dict& d) {
+    using namespace param_detail;
+    check_unknown(d, {"num_args", "dim"}, "ConcatParam");
+    num_args = static_cast<int>(get_int(d, "num_args", false, 0, true, 1));
+    auto it = d.find("dim");
+    if (it != d.end()) {
+      if (trim(it->second) == "None")
+        dim = dmlc::optional<int>();
+      else
+        dim = dmlc::optional<int>(static_cast<int>(get_int(d, "dim", true, 1, false, 0)));
+    }
+  }
+  static std::vector<nnvm::ParamFieldInfo> __FIELDS__() {
+    return {{"num_args", "int, required", "Number of inputs to be concated."},
+            {"dim", "int or None, optional, default='1'", "the dimension to be concated."}};
+  }
+};
+
+// src/operator/tensor/broadcast_reduce_op.h:240-249: a negative axis counts from the end
+inline int CheckAxis(const int axis, const int ndim) {
+  if (ndim == 0) {
+    CHECK(axis == 0 || axis == -1) << "axis " << axis << " is out of bounds for 0-dimension tensor";
+    return 0;
+  }
+  CHECK(axis < ndim && axis >= -ndim)
+      << "axis " << axis << " exceeds the input dimension of " << ndim;
+  return (axis + ndim) % ndim;
 }
 
 // src/operator/nn/pooling.cc:35-64

@@ -379,6 +379,99 @@ static bool QuantizedFlattenType(const NodeAttrs&, std::vector<int>* in, std::ve
   return (*in)[0] != -1;
 }
 
+// quantized_elemwise_add.cc:30-78
+static bool ElemwiseAddShape(const NodeAttrs&, ShapeVector* in_shape, ShapeVector* out_shape) {
+  // A, B, A_min, A_max, B_min, B_max -> C, C_min, C_max
+  CHECK_EQ(in_shape->size(), 6U);
+  CHECK_EQ(out_shape->size(), 3U);
+  CHECK_EQ((*in_shape)[0], (*in_shape)[1]);
+  for (int i = 2; i < 6; ++i) SHAPE_ASSIGN_CHECK(*in_shape, i, kScalarShape);
+  SHAPE_ASSIGN_CHECK(*out_shape, 0, (*in_shape)[0]);
+  SHAPE_ASSIGN_CHECK(*out_shape, 1, kScalarShape);
+  SHAPE_ASSIGN_CHECK(*out_shape, 2, kScalarShape);
+  return true;
+}
+static bool ElemwiseAddType(const NodeAttrs& attrs, std::vector<int>* in_type,
+                            std::vector<int>* out_type) {
+  CHECK_EQ(in_type->size(), 6U);
+  CHECK_EQ(out_type->size(), 3U);
+  for (int i = 0; i < 2; ++i) {
+    if (in_type->at(i) == mshadow::kInt8) {
+      TYPE_ASSIGN_CHECK(*in_type, i, mshadow::kInt8);
+    } else {
+      TYPE_ASSIGN_CHECK(*in_type, i, mshadow::kUint8);
+    }
+  }
+  int dtype = mshadow::kInt32;
+  const auto& params = nnvm::get<QuantizeElemwiseAddParam>(attrs.parsed);
+  if (params.max_calib_range.has_value() && params.min_calib_range.has_value())
+    dtype = (in_type->at(0) == in_type->at(1)) ? in_type->at(0) : mshadow::kInt8;
+  TYPE_ASSIGN_CHECK(*out_type, 0, dtype);
+  TYPE_ASSIGN_CHECK(*out_type, 1, mshadow::kFloat32);
+  TYPE_ASSIGN_CHECK(*out_type, 2, mshadow::kFloat32);
+  return true;
+}
+
+// quantized_concat.cc:31-103
+static bool QuantizedConcatShape(const NodeAttrs& attrs, ShapeVector* in_shape,
+                                 ShapeVector* out_shape) {
+  const ConcatParam& param_ = nnvm::get<ConcatParam>(attrs.parsed);
+  CHECK_EQ(in_shape->size(), static_cast<size_t>(param_.num_args * 3));
+  CHECK_EQ(out_shape->size(), 3U);
+  TShape dshape;
+  index_t size = 0;
+  bool has_unknown_dim_size = false;
+  int axis = -1;
+  const int param_dim = param_.dim.has_value() ? param_.dim.value() : 0;
+  for (int i = 0; i < param_.num_args; ++i) {
+    TShape tmp = (*in_shape)[i];
+    if (tmp.ndim() > 0) {
+      axis = CheckAxis(param_dim, tmp.ndim());
+      has_unknown_dim_size = !dim_size_is_known(tmp, axis) || has_unknown_dim_size;
+      size += tmp[axis];
+      tmp[axis] = -1;
+      shape_assign(&dshape, tmp);
+    }
+  }
+  TShape tmp = (*out_shape)[0];
+  if (tmp.ndim() > 0) {
+    axis = CheckAxis(param_dim, tmp.ndim());
+    tmp[axis] = -1;
+    shape_assign(&dshape, tmp);
+  }
+  if (!ndim_is_known(dshape)) return false;
+  for (int i = 0; i < param_.num_args; ++i) {
+    CHECK(shape_assign(&(*in_shape)[i], dshape))
+        << "Incompatible input shape: expected " << dshape << ", got " << (*in_shape)[i];
+  }
+  if (!has_unknown_dim_size) dshape[axis] = size;
+  CHECK(shape_assign(&(*out_shape)[0], dshape))
+      << "Incompatible output shape: expected " << dshape << ", got " << (*out_shape)[0];
+  for (int i = param_.num_args; i < param_.num_args * 3; ++i)
+    SHAPE_ASSIGN_CHECK(*in_shape, i, kScalarShape);
+  SHAPE_ASSIGN_CHECK(*out_shape, 1, kScalarShape);
+  SHAPE_ASSIGN_CHECK(*out_shape, 2, kScalarShape);
+  return shape_is_known(dshape);
+}
+static bool QuantizedConcatType(const NodeAttrs& attrs, std::vector<int>* in_type,
+                                std::vector<int>* out_type) {
+  const ConcatParam& param_ = nnvm::get<ConcatParam>(attrs.parsed);
+  CHECK_EQ(in_type->size(), static_cast<size_t>(param_.num_args * 3));
+  CHECK_EQ(out_type->size(), 3U);
+  int dtype = mshadow::kUint8;
+  for (int i = 0; i < param_.num_args; ++i) {
+    if (in_type->at(i) == mshadow::kInt8) {
+      dtype = mshadow::kInt8;
+    } else {
+      TYPE_ASSIGN_CHECK(*in_type, i, mshadow::kUint8);
+    }
+  }
+  TYPE_ASSIGN_CHECK(*out_type, 0, dtype);
+  TYPE_ASSIGN_CHECK(*out_type, 1, mshadow::kFloat32);
+  TYPE_ASSIGN_CHECK(*out_type, 2, mshadow::kFloat32);
+  return true;
+}
+
 static bool DefaultStorageType(const NodeAttrs&, const int, DispatchMode* dispatch_mode,
                                std::vector<int>* in, std::vector<int>* out) {
   *dispatch_mode = DispatchMode::kFCompute;
@@ -648,6 +741,61 @@ static void QuantizedFlattenComputeGPU(const NodeAttrs&, const OpContext& ctx,
                                  inputs[2].dptr<float>(), outputs[0].dptr_,
                                  outputs[1].dptr<float>(), outputs[2].dptr<float>(),
                                  outputs[0].Size()));
+}
+
+// _contrib_quantized_elemwise_add (dnnl_quantized_elemwise_add.cc:134-257; operands of
+// one shape, the only form the operator's shape function admits)
+static void QuantizedElemwiseAddForwardGPU(const NodeAttrs& attrs, const OpContext& ctx,
+                                           const std::vector<TBlob>& inputs,
+                                           const std::vector<OpReqType>&,
+                                           const std::vector<TBlob>& outputs) {
+  const auto& params = nnvm::get<QuantizeElemwiseAddParam>(attrs.parsed);
+  CHECK_EQ(inputs.size(), 6U) << "should be A, B, A_min, A_max, B_min, B_max";
+  CHECK_EQ(outputs.size(), 3U) << "should be C, C_min, C_max";
+  CHECK_EQ(inputs[0].Size(), inputs[1].Size());
+  const bool calibrated = params.max_calib_range.has_value() && params.min_calib_range.has_value();
+  MXQ_CALL(mxq_quantized_elemwise_add(
+      raw_stream(ctx), inputs[0].dptr_, inputs[0].type_flag_, inputs[1].dptr_,
+      inputs[1].type_flag_, inputs[2].dptr<float>(), inputs[3].dptr<float>(),
+      inputs[4].dptr<float>(), inputs[5].dptr<float>(), outputs[0].dptr_, outputs[0].type_flag_,
+      outputs[1].dptr<float>(), outputs[2].dptr<float>(), outputs[0].Size(), calibrated ? 1 : 0,
+      calibrated ? params.min_calib_range.value() : 0.f,
+      calibrated ? params.max_calib_range.value() : 0.f));
+}
+
+// _contrib_quantized_concat (dnnl_quantized_concat.cc:41-115)
+static void QuantizedConcatForwardGPU(const NodeAttrs& attrs, const OpContext& ctx,
+                                      const std::vector<TBlob>& inputs,
+                                      const std::vector<OpReqType>&,
+                                      const std::vector<TBlob>& outputs) {
+  const ConcatParam& param_ = nnvm::get<ConcatParam>(attrs.parsed);
+  const int n = param_.num_args;
+  CHECK_EQ(inputs.size(), static_cast<size_t>(n * 3));
+  CHECK_EQ(outputs.size(), 3U);
+  const TShape& oshape = outputs[0].shape_;
+  const int axis = CheckAxis(param_.dim.has_value() ? param_.dim.value() : 0, oshape.ndim());
+  int64_t outer = 1, inner = 1;
+  for (int i = 0; i < axis; ++i) outer *= oshape[i];
+  for (int i = axis + 1; i < oshape.ndim(); ++i) inner *= oshape[i];
+  std::vector<const void*> data(n);
+  std::vector<int> types(n);
+  std::vector<const float*> mins(n), maxs(n);
+  std::vector<int64_t> extents(n);
+  int64_t total = 0;
+  for (int i = 0; i < n; ++i) {
+    CHECK_EQ(inputs[i].shape_.ndim(), oshape.ndim());
+    data[i] = inputs[i].dptr_;
+    types[i] = inputs[i].type_flag_;
+    mins[i] = inputs[n + 2 * i].dptr<float>();
+    maxs[i] = inputs[n + 2 * i + 1].dptr<float>();
+    extents[i] = inputs[i].shape_[axis];
+    total += extents[i];
+  }
+  CHECK_EQ(total, oshape[axis]);
+  MXQ_CALL(mxq_quantized_concat(raw_stream(ctx), n, data.data(), types.data(), mins.data(),
+                                maxs.data(), extents.data(), outer, inner, outputs[0].dptr_,
+                                outputs[0].type_flag_, outputs[1].dptr<float>(),
+                                outputs[2].dptr<float>()));
 }
 
 size_t MXQTempSpaceBytes(const NodeAttrs& attrs, const ShapeVector& in, const ShapeVector& out) {
@@ -941,6 +1089,74 @@ NNVM_REGISTER_OP(_contrib_quantized_flatten)
                   "The minimum scalar value possibly produced for the data")
     .add_argument("max_data", "NDArray-or-Symbol",
                   "The maximum scalar value possibly produced for the data");
+
+// quantized_elemwise_add.cc:89-122 (+ the parser and argument fields the oneDNN file
+// attaches, dnnl_quantized_elemwise_add.cc:270-275)
+NNVM_REGISTER_OP(_contrib_quantized_elemwise_add)
+    .add_alias("_npx_quantized_elemwise_add")
+    .describe("elemwise_add operator for input dataA and input dataB data type of int8, and "
+              "accumulates in type int32 for the output.")
+    .set_num_inputs(6)
+    .set_num_outputs(3)
+    .set_attr_parser(ParamParser<QuantizeElemwiseAddParam>)
+    .set_attr<nnvm::FListInputNames>("FListInputNames",
+                                     [](const NodeAttrs&) {
+                                       return std::vector<std::string>{"lhs",     "rhs",
+                                                                       "lhs_min", "lhs_max",
+                                                                       "rhs_min", "rhs_max"};
+                                     })
+    .set_attr<nnvm::FListOutputNames>("FListOutputNames",
+                                      [](const NodeAttrs&) {
+                                        return std::vector<std::string>{"output", "min_output",
+                                                                        "max_output"};
+                                      })
+    .set_attr<nnvm::FInferType>("FInferType", ElemwiseAddType)
+    .set_attr<mxnet::FInferShape>("FInferShape", ElemwiseAddShape)
+    .set_attr<FInferStorageType>("FInferStorageType", DefaultStorageType)
+    .set_attr<FNeedRequantize>("FNeedRequantize", [](const NodeAttrs&) { return true; })
+    .set_attr<FCompute>("FCompute<gpu>", QuantizedElemwiseAddForwardGPU)
+    .add_argument("lhs", "NDArray-or-Symbol", "first input")
+    .add_argument("rhs", "NDArray-or-Symbol", "second input")
+    .add_argument("lhs_min", "NDArray-or-Symbol", "3rd input")
+    .add_argument("lhs_max", "NDArray-or-Symbol", "4th input")
+    .add_argument("rhs_min", "NDArray-or-Symbol", "5th input")
+    .add_argument("rhs_max", "NDArray-or-Symbol", "6th input")
+    .add_arguments(QuantizeElemwiseAddParam::__FIELDS__());
+
+// quantized_concat.cc:105-141
+NNVM_REGISTER_OP(_contrib_quantized_concat)
+    .describe("Joins input arrays along a given axis.  All inputs with different min/max will "
+              "be rescaled by using largest [min, max] pairs.  If any input holds int8, then "
+              "the output will be int8. Otherwise output will be uint8.")
+    .set_num_inputs([](const NodeAttrs& attrs) {
+      return static_cast<uint32_t>(nnvm::get<ConcatParam>(attrs.parsed).num_args * 3);
+    })
+    .set_num_outputs(3)
+    .set_attr_parser(ParamParser<ConcatParam>)
+    .set_attr<nnvm::FListInputNames>(
+        "FListInputNames",
+        [](const NodeAttrs& attrs) {
+          const ConcatParam& params = nnvm::get<ConcatParam>(attrs.parsed);
+          std::vector<std::string> ret;
+          for (int i = 0; i < params.num_args; ++i) ret.push_back("arg" + std::to_string(i));
+          for (int i = 0; i < params.num_args; ++i) {
+            ret.push_back("arg" + std::to_string(i) + "_min");
+            ret.push_back("arg" + std::to_string(i) + "_max");
+          }
+          return ret;
+        })
+    .set_attr<nnvm::FListOutputNames>("FListOutputNames",
+                                      [](const NodeAttrs&) {
+                                        return std::vector<std::string>{"output", "min_output",
+                                                                        "max_output"};
+                                      })
+    .set_attr<nnvm::FInferType>("FInferType", QuantizedConcatType)
+    .set_attr<mxnet::FInferShape>("FInferShape", QuantizedConcatShape)
+    .set_attr<FInferStorageType>("FInferStorageType", DefaultStorageType)
+    .set_attr<std::string>("key_var_num_args", "num_args")
+    .set_attr<FCompute>("FCompute<gpu>", QuantizedConcatForwardGPU)
+    .add_argument("data", "NDArray-or-Symbol[]", "List of arrays to concatenate")
+    .add_arguments(ConcatParam::__FIELDS__());
 
 }  // namespace op
 }  // namespace mxnet

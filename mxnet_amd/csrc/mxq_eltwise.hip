@@ -1,0 +1,572 @@
+// Quantized element-wise add and concat for gfx950: the two operators that join
+// branches of a quantized CNN (residual sums, inception-style concatenations).
+//   _contrib_quantized_elemwise_add  src/operator/quantization/quantized_elemwise_add.cc:30-134
+//                                    dnnl/dnnl_quantized_elemwise_add.cc:134-257
+//   _contrib_quantized_concat        src/operator/quantization/quantized_concat.cc:31-141
+//                                    dnnl/dnnl_quantized_concat.cc:41-115
+// Both exist for cpu only in the reference and hand their arithmetic to oneDNN
+// (dnnl::sum / dnnl::reorder with scales).  What is restated here is the scale
+// derivation of the reference's own files plus the primitives' documented rule
+// dst = saturate(round_nearest_even(sum_i scale_i * src_i)), evaluated in binary32 with
+// every operation rounded on its own.
+//
+// Both are byte streams bound by HBM: 16 elements per lane per segment where the
+// output is a byte type, 4 where it is int32 (so that every lane stores 16 bytes).
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+
+#include "../../include/mxq.h"
+#include "mxq_common.h"
+
+namespace mxq {
+
+extern int g_cast_blocks_per_cu;  // mxq_cast.hip: work-groups per CU of the streaming kernels
+
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kMaxConcatPerLaunch = 16;
+
+typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+typedef int i4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ float maxabs(float a, float b) {
+  float x = fabsf(a), y = fabsf(b);
+  return (x < y) ? y : x;
+}
+
+// quantization_utils.h:37-39
+__device__ __forceinline__ float type_range(int type) {
+  return type == MXQ_INT8 ? 127.5f : 255.5f;
+}
+__device__ __forceinline__ double type_range_wide(int type) {
+  return type == MXQ_INT32 ? 2147483647.0 : (type == MXQ_INT8 ? 127.5 : 255.5);
+}
+
+// saturate, then round to nearest even, into the output type; NaN converts to 0
+template <int OUT>
+__device__ __forceinline__ int narrow(float f) {
+  constexpr float lo = OUT == MXQ_INT32 ? -2147483648.f : (OUT == MXQ_INT8 ? -128.f : 0.f);
+  constexpr float hi = OUT == MXQ_INT32 ? 2147483520.f : (OUT == MXQ_INT8 ? 127.f : 255.f);
+  if (f != f) return 0;
+  f = f < lo ? lo : f;
+  f = f > hi ? hi : f;
+  return static_cast<int>(rintf(f));
+}
+
+// The same for a value known not to be NaN, as the low byte of the returned word: one
+// clamp, then an add of 1.5 * 2^23, which leaves nearest-even(f) in the low mantissa bits
+// (|f| <= 255, the sum's unit in the last place is 1 and 1.5 * 2^23 is even).
+template <int OUT>
+__device__ __forceinline__ uint32_t narrow_byte(float f) {
+  constexpr float lo = OUT == MXQ_INT8 ? -128.f : 0.f;
+  constexpr float hi = OUT == MXQ_INT8 ? 127.f : 255.f;
+  return __float_as_uint(__builtin_amdgcn_fmed3f(f, lo, hi) + 12582912.f);
+}
+// 16 bytes written through the XCD's L2 (device-scope store) instead of lingering there as
+// a dirty line: keeps the HBM write stream of a narrowing kernel sequential.  A store of
+// more than 8 bytes reads its data registers over the two wait states after it issues and
+// no VALU instruction may overwrite them before; the compiler pads its own stores but
+// cannot see into this one, hence the s_nop.
+__device__ __forceinline__ void stream_store16(u4 v, u4* p) {
+  asm volatile("global_store_dwordx4 %0, %1, off sc1\n\ts_nop 1" ::"v"(p), "v"(v) : "memory");
+}
+// the low bytes of four words in one word
+__device__ __forceinline__ uint32_t pack_low_bytes(uint32_t b0, uint32_t b1, uint32_t b2,
+                                                   uint32_t b3) {
+  const uint32_t lo = __builtin_amdgcn_perm(b1, b0, 0x0c0c0400u);  // {b0.0, b1.0, 0, 0}
+  const uint32_t hi = __builtin_amdgcn_perm(b3, b2, 0x04000c0cu);  // {0, 0, b2.0, b3.0}
+  return lo | hi;
+}
+
+template <bool UNSIGNED>
+__device__ __forceinline__ int byte_of(uint32_t w, int k) {
+  const uint32_t b = (w >> (8 * k)) & 0xffu;
+  return UNSIGNED ? static_cast<int>(b) : static_cast<int>(static_cast<int8_t>(b));
+}
+__device__ __forceinline__ int byte_at(uint32_t w, int k, bool is_unsigned) {
+  return is_unsigned ? byte_of<true>(w, k) : byte_of<false>(w, k);
+}
+
+// uint8 -> int8 at half scale, as the reference's reorder with scale 0.5 does before a
+// mixed-type sum (dnnl_quantized_elemwise_add.cc:189-210)
+__device__ __forceinline__ int halve_u8(int v) {
+  return narrow<MXQ_INT8>(static_cast<float>(v) * 0.5f);
+}
+
+struct AddArgs {
+  const uint8_t* lhs;
+  const uint8_t* rhs;
+  void* out;
+  size_t n;
+  const float* lhs_min;
+  const float* lhs_max;
+  const float* rhs_min;
+  const float* rhs_max;
+  float* omin;
+  float* omax;
+  float min_calib, max_calib;
+  int calibrated, vec_ok;
+};
+
+// LU / RU: the operand is uint8.  FAST: both scales are small enough that neither
+// product overflows, so no NaN can arise and the one-instruction clamp applies.
+template <int OUT, bool LU, bool RU>
+struct AddRule {
+  float s0, s1, omin, omax;
+  static constexpr bool kHalveL = LU && !RU, kHalveR = RU && !LU;
+  __device__ __forceinline__ float sum(int a, int b) const {
+    if (kHalveL) a = halve_u8(a);
+    if (kHalveR) b = halve_u8(b);
+    const float x = static_cast<float>(a) * s0;
+    const float y = static_cast<float>(b) * s1;
+    return x + y;
+  }
+  __device__ __forceinline__ int apply(int a, int b) const { return narrow<OUT>(sum(a, b)); }
+  template <bool FAST>
+  __device__ __forceinline__ uint32_t apply4(uint32_t x, uint32_t y) const {
+    uint32_t q[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const float f = sum(byte_of<LU>(x, k), byte_of<RU>(y, k));
+      q[k] = FAST ? narrow_byte<OUT>(f) : static_cast<uint32_t>(narrow<OUT>(f));
+    }
+    return pack_low_bytes(q[0], q[1], q[2], q[3]);
+  }
+  __device__ __forceinline__ bool fast() const {
+    return fabsf(s0) < 1e30f && fabsf(s1) < 1e30f;  // false for NaN as well
+  }
+};
+
+// dnnl_quantized_elemwise_add.cc:143-210
+template <int OUT, bool LU, bool RU>
+__device__ __forceinline__ AddRule<OUT, LU, RU> add_rule(const AddArgs& a) {
+  AddRule<OUT, LU, RU> r;
+  const float a_absmax = maxabs(*a.lhs_min, *a.lhs_max);
+  const float b_absmax = maxabs(*a.rhs_min, *a.rhs_max);
+  const float a_scale = type_range(LU ? MXQ_UINT8 : MXQ_INT8) / a_absmax;
+  const float b_scale = type_range(RU ? MXQ_UINT8 : MXQ_INT8) / b_absmax;
+  const double out_range = type_range_wide(OUT);
+  float out_scale;
+  if (a.calibrated) {
+    r.omin = a.min_calib;
+    r.omax = a.max_calib;
+    out_scale = static_cast<float>(out_range / static_cast<double>(maxabs(r.omin, r.omax)));
+  } else {
+    r.omax = a_absmax + b_absmax;
+    r.omin = -r.omax;
+    out_scale = static_cast<float>(out_range / static_cast<double>(r.omax));
+  }
+  r.s0 = out_scale / a_scale;
+  r.s1 = out_scale / b_scale;
+  if (r.kHalveL) r.s0 = static_cast<float>(static_cast<double>(r.s0) * (1.0 / 0.5));
+  if (r.kHalveR) r.s1 = static_cast<float>(static_cast<double>(r.s1) * (1.0 / 0.5));
+  return r;
+}
+
+// 16 elements per lane and segment: 16 bytes of each operand in, 16 bytes out
+template <int OUT, bool LU, bool RU, bool FAST>
+__device__ __forceinline__ void add_bytes(const AddArgs& a, const AddRule<OUT, LU, RU>& r,
+                                          size_t t0, size_t stride) {
+  const size_t nv = a.n >> 4;
+  const u4* l16 = reinterpret_cast<const u4*>(a.lhs);
+  const u4* r16 = reinterpret_cast<const u4*>(a.rhs);
+  u4* o16 = reinterpret_cast<u4*>(a.out);
+  size_t q = t0;
+  for (; q + stride < nv; q += 2 * stride) {
+    u4 x[2], y[2];
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      x[j] = __builtin_nontemporal_load(l16 + q + j * stride);
+      y[j] = __builtin_nontemporal_load(r16 + q + j * stride);
+    }
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      u4 v;
+#pragma unroll
+      for (int w = 0; w < 4; ++w) v[w] = r.template apply4<FAST>(x[j][w], y[j][w]);
+      stream_store16(v, o16 + q + j * stride);
+    }
+  }
+  for (; q < nv; q += stride) {
+    const u4 x = l16[q], y = r16[q];
+    u4 v;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) v[w] = r.template apply4<FAST>(x[w], y[w]);
+    stream_store16(v, o16 + q);
+  }
+}
+
+template <int OUT, bool LU, bool RU>
+__global__ __launch_bounds__(kThreads) void add_kernel(AddArgs a) {
+  const AddRule<OUT, LU, RU> r = add_rule<OUT, LU, RU>(a);
+  const size_t stride = size_t(gridDim.x) * kThreads;
+  const size_t t0 = size_t(blockIdx.x) * kThreads + threadIdx.x;
+  size_t done = 0;
+  if (a.vec_ok) {
+    if (OUT == MXQ_INT32) {
+      // 4 elements per lane: a dword of each operand in, 16 bytes out
+      const size_t nq = a.n >> 2;
+      const uint32_t* l4 = reinterpret_cast<const uint32_t*>(a.lhs);
+      const uint32_t* r4 = reinterpret_cast<const uint32_t*>(a.rhs);
+      i4* o4 = reinterpret_cast<i4*>(a.out);
+      size_t q = t0;
+      for (; q + 3 * stride < nq; q += 4 * stride) {
+        uint32_t x[4], y[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          x[j] = __builtin_nontemporal_load(l4 + q + j * stride);
+          y[j] = __builtin_nontemporal_load(r4 + q + j * stride);
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          i4 v;
+#pragma unroll
+          for (int k = 0; k < 4; ++k) v[k] = r.apply(byte_of<LU>(x[j], k), byte_of<RU>(y[j], k));
+          __builtin_nontemporal_store(v, o4 + q + j * stride);
+        }
+      }
+      for (; q < nq; q += stride) {
+        const uint32_t x = l4[q], y = r4[q];
+        i4 v;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) v[k] = r.apply(byte_of<LU>(x, k), byte_of<RU>(y, k));
+        __builtin_nontemporal_store(v, o4 + q);
+      }
+      done = nq << 2;
+    } else {
+      if (r.fast())
+        add_bytes<OUT, LU, RU, true>(a, r, t0, stride);
+      else
+        add_bytes<OUT, LU, RU, false>(a, r, t0, stride);
+      done = (a.n >> 4) << 4;
+    }
+  }
+  for (size_t i = done + t0; i < a.n; i += stride) {
+    const int x = LU ? static_cast<int>(a.lhs[i]) : static_cast<int>(static_cast<int8_t>(a.lhs[i]));
+    const int y = RU ? static_cast<int>(a.rhs[i]) : static_cast<int>(static_cast<int8_t>(a.rhs[i]));
+    const int s = r.apply(x, y);
+    if (OUT == MXQ_INT32)
+      static_cast<int32_t*>(a.out)[i] = s;
+    else
+      static_cast<uint8_t*>(a.out)[i] = static_cast<uint8_t>(s);
+  }
+  if (blockIdx.x == 0 && threadIdx.x == 0) {
+    *a.omin = r.omin;
+    *a.omax = r.omax;
+  }
+}
+
+// ---- concat -----------------------------------------------------------------------
+
+struct ConcatRanges {
+  const float* mn[kMaxConcatPerLaunch];
+  const float* mx[kMaxConcatPerLaunch];
+  int count, first;
+};
+
+// dnnl_quantized_concat.cc:53-67: the output range is the hull of the input ranges and 0
+__device__ __forceinline__ void range_hull(const float* const* mn, const float* const* mx,
+                                           int count, float& lo, float& hi) {
+  for (int i = 0; i < count; ++i) {
+    const float a = *mn[i], b = *mx[i];
+    if (a < lo) lo = a;
+    if (b > hi) hi = b;
+  }
+}
+
+// Only for more inputs than one launch carries: folds their ranges into omin / omax.
+__global__ void concat_range_kernel(ConcatRanges r, float* omin, float* omax) {
+  float lo = r.first ? 0.f : *omin;
+  float hi = r.first ? 0.f : *omax;
+  range_hull(r.mn, r.mx, r.count, lo, hi);
+  *omin = lo;
+  *omax = hi;
+}
+
+// Up to kMaxConcatPerLaunch inputs in one launch; input i owns the work-groups
+// [block_end[i-1], block_end[i]).
+struct ConcatArgs {
+  const uint8_t* in[kMaxConcatPerLaunch];
+  const float* mn[kMaxConcatPerLaunch];
+  const float* mx[kMaxConcatPerLaunch];
+  size_t row_bytes[kMaxConcatPerLaunch];  // extent along the axis x the trailing dimensions
+  size_t out_off[kMaxConcatPerLaunch];    // first output byte of the input's slab
+  int block_end[kMaxConcatPerLaunch];
+  int in_type[kMaxConcatPerLaunch];
+  int vec_ok[kMaxConcatPerLaunch];
+  uint8_t* out;
+  size_t rows;       // product of the dimensions before the axis
+  size_t out_pitch;  // the output's extent along the axis x the trailing dimensions
+  float* omin;
+  float* omax;
+  int count, out_type;
+  int given_range;   // omin / omax already hold the hull of all inputs (more than one launch)
+};
+
+// MODE 0: byte copy, 1: rescale of finite scale (one-instruction clamp), 2: rescale, general
+template <int MODE, bool IN_U, bool OUT_U>
+__device__ __forceinline__ uint32_t concat_word(uint32_t w, float scale) {
+  if (MODE == 0) return w;
+  uint32_t q[4];
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    const float f = static_cast<float>(byte_of<IN_U>(w, k)) * scale;
+    constexpr int OUT = OUT_U ? MXQ_UINT8 : MXQ_INT8;
+    q[k] = MODE == 1 ? narrow_byte<OUT>(f) : static_cast<uint32_t>(narrow<OUT>(f));
+  }
+  return pack_low_bytes(q[0], q[1], q[2], q[3]);
+}
+
+template <int MODE, bool IN_U, bool OUT_U>
+__device__ __forceinline__ void concat_slab(const uint8_t* __restrict__ in,
+                                            uint8_t* __restrict__ out, size_t rows,
+                                            size_t row_bytes, size_t out_pitch, float scale,
+                                            bool vec_ok, size_t t0, size_t stride) {
+  if (vec_ok) {
+    const size_t per_row = row_bytes >> 4;
+    const size_t total = rows * per_row;
+    const bool one_row = rows == 1;
+    const bool narrow_index = total < (1ull << 32);
+    for (size_t q = t0; q < total; q += stride) {
+      size_t row = 0, col = q;
+      if (!one_row) {
+        if (narrow_index) {
+          const uint32_t r32 = static_cast<uint32_t>(q) / static_cast<uint32_t>(per_row);
+          row = r32;
+          col = static_cast<uint32_t>(q) - r32 * static_cast<uint32_t>(per_row);
+        } else {
+          row = q / per_row;
+          col = q - row * per_row;
+        }
+      }
+      u4 v = __builtin_nontemporal_load(reinterpret_cast<const u4*>(in + row * row_bytes) + col);
+#pragma unroll
+      for (int w = 0; w < 4; ++w) v[w] = concat_word<MODE, IN_U, OUT_U>(v[w], scale);
+      stream_store16(v, reinterpret_cast<u4*>(out + row * out_pitch) + col);
+    }
+  } else {
+    const size_t total = rows * row_bytes;
+    for (size_t i = t0; i < total; i += stride) {
+      const size_t row = i / row_bytes, col = i - row * row_bytes;
+      uint8_t o = in[i];
+      if (MODE != 0) {
+        const int v = IN_U ? static_cast<int>(o) : static_cast<int>(static_cast<int8_t>(o));
+        constexpr int OUT = OUT_U ? MXQ_UINT8 : MXQ_INT8;
+        o = static_cast<uint8_t>(narrow<OUT>(static_cast<float>(v) * scale));
+      }
+      out[row * out_pitch + col] = o;
+    }
+  }
+}
+
+// dnnl_quantized_concat.cc:68-98: an input whose scale equals the output's is copied,
+// any other goes through a reorder with scale out_scale / in_scale.
+__global__ __launch_bounds__(kThreads) void concat_kernel(ConcatArgs a) {
+  float lo = 0.f, hi = 0.f;
+  if (a.given_range) {
+    lo = *a.omin;
+    hi = *a.omax;
+  } else {
+    range_hull(a.mn, a.mx, a.count, lo, hi);
+  }
+  int part = 0;
+  while (part + 1 < a.count && static_cast<int>(blockIdx.x) >= a.block_end[part]) ++part;
+  const int first_block = part == 0 ? 0 : a.block_end[part - 1];
+  const size_t stride = size_t(a.block_end[part] - first_block) * kThreads;
+  const size_t t0 = size_t(blockIdx.x - first_block) * kThreads + threadIdx.x;
+  const int in_type = a.in_type[part];
+  const float out_scale = type_range(a.out_type) / maxabs(lo, hi);
+  const float in_scale = type_range(in_type) / maxabs(*a.mn[part], *a.mx[part]);
+  const float scale = out_scale / in_scale;
+  const bool copy = (in_scale == out_scale) && in_type == a.out_type;
+  const bool finite = fabsf(scale) < 1e30f;  // false for NaN as well
+  const uint8_t* in = a.in[part];
+  uint8_t* out = a.out + a.out_off[part];
+  const size_t rb = a.row_bytes[part];
+  const bool v = a.vec_ok[part] != 0;
+#define MXQ_SLAB(M, I, O) \
+  concat_slab<M, I, O>(in, out, a.rows, rb, a.out_pitch, scale, v, t0, stride)
+  const bool in_u = in_type == MXQ_UINT8, out_u = a.out_type == MXQ_UINT8;
+  if (copy) {
+    MXQ_SLAB(0, false, false);
+  } else if (finite) {
+    if (out_u) MXQ_SLAB(1, true, true);  // a uint8 output has uint8 inputs only
+    else if (in_u) MXQ_SLAB(1, true, false);
+    else MXQ_SLAB(1, false, false);
+  } else {
+    if (out_u) MXQ_SLAB(2, true, true);
+    else if (in_u) MXQ_SLAB(2, true, false);
+    else MXQ_SLAB(2, false, false);
+  }
+#undef MXQ_SLAB
+  if (!a.given_range && blockIdx.x == 0 && threadIdx.x == 0) {
+    *a.omin = lo;
+    *a.omax = hi;
+  }
+}
+
+int grid_for(size_t work_items) {
+  int dev = 0;
+  MXQ_HIP(hipGetDevice(&dev));
+  static thread_local int cached_dev = -1, cached_cus = 0;
+  if (cached_dev != dev) {
+    MXQ_HIP(hipDeviceGetAttribute(&cached_cus, hipDeviceAttributeMultiprocessorCount, dev));
+    cached_dev = dev;
+  }
+  size_t want = (work_items + kThreads - 1) / kThreads;
+  const size_t cap = size_t(cached_cus) * size_t(g_cast_blocks_per_cu);
+  if (want < 1) want = 1;
+  return static_cast<int>(want < cap ? want : cap);
+}
+
+bool byte_type(int t) { return t == MXQ_INT8 || t == MXQ_UINT8; }
+
+}  // namespace
+}  // namespace mxq
+
+using namespace mxq;
+
+extern "C" {
+
+int mxq_quantized_elemwise_add(void* stream, const void* lhs, int lhs_type, const void* rhs,
+                               int rhs_type, const float* lhs_min, const float* lhs_max,
+                               const float* rhs_min, const float* rhs_max, void* out, int out_type,
+                               float* omin, float* omax, size_t n, int calibrated,
+                               float min_calib, float max_calib) {
+  MXQ_API_BEGIN();
+  MXQ_CHECK(byte_type(lhs_type) && byte_type(rhs_type),
+            "quantized_elemwise_add takes int8 or uint8 inputs, got " << lhs_type << " and "
+                                                                      << rhs_type);
+  // ElemwiseAddType (quantized_elemwise_add.cc:50-78)
+  const int want = !calibrated ? MXQ_INT32 : (lhs_type == rhs_type ? lhs_type : MXQ_INT8);
+  MXQ_CHECK(out_type == want, "output type must be " << want << " for these inputs"
+                                                     << (calibrated ? " (calibrated)" : "")
+                                                     << ", got " << out_type);
+  MXQ_CHECK(lhs_min != nullptr && lhs_max != nullptr && rhs_min != nullptr && rhs_max != nullptr &&
+                omin != nullptr && omax != nullptr,
+            "null range pointer");
+  MXQ_CHECK(n == 0 || (lhs != nullptr && rhs != nullptr && out != nullptr), "null data pointer");
+  AddArgs a;
+  a.lhs = static_cast<const uint8_t*>(lhs);
+  a.rhs = static_cast<const uint8_t*>(rhs);
+  a.out = out;
+  a.n = n;
+  a.lhs_min = lhs_min; a.lhs_max = lhs_max; a.rhs_min = rhs_min; a.rhs_max = rhs_max;
+  a.omin = omin; a.omax = omax;
+  a.min_calib = min_calib; a.max_calib = max_calib;
+  a.calibrated = calibrated != 0;
+  const bool in_ok = out_type == MXQ_INT32
+                         ? ((reinterpret_cast<uintptr_t>(lhs) | reinterpret_cast<uintptr_t>(rhs)) & 3u) == 0
+                         : (aligned16(lhs) && aligned16(rhs));
+  a.vec_ok = (in_ok && aligned16(out)) ? 1 : 0;
+  const size_t per_lane = out_type == MXQ_INT32 ? 4 : 16;
+  const int grid = grid_for(a.vec_ok ? (n + per_lane - 1) / per_lane : n);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const bool lu = lhs_type == MXQ_UINT8, ru = rhs_type == MXQ_UINT8;
+#define MXQ_ADD(O, L, R) \
+  hipLaunchKernelGGL((add_kernel<O, L, R>), dim3(grid), dim3(kThreads), 0, s, a)
+  if (out_type == MXQ_INT32) {
+    if (lu) { if (ru) MXQ_ADD(MXQ_INT32, true, true); else MXQ_ADD(MXQ_INT32, true, false); }
+    else    { if (ru) MXQ_ADD(MXQ_INT32, false, true); else MXQ_ADD(MXQ_INT32, false, false); }
+  } else if (out_type == MXQ_UINT8) {
+    MXQ_ADD(MXQ_UINT8, true, true);
+  } else {
+    if (lu) MXQ_ADD(MXQ_INT8, true, false);
+    else if (ru) MXQ_ADD(MXQ_INT8, false, true);
+    else MXQ_ADD(MXQ_INT8, false, false);
+  }
+#undef MXQ_ADD
+  MXQ_LAUNCH_CHECK();
+  MXQ_API_END();
+}
+
+int mxq_quantized_concat(void* stream, int num_args, const void* const* in, const int* in_type,
+                         const float* const* in_min, const float* const* in_max,
+                         const int64_t* in_axis, int64_t outer, int64_t inner, void* out,
+                         int out_type, float* omin, float* omax) {
+  MXQ_API_BEGIN();
+  MXQ_CHECK(num_args >= 1, "concat needs at least one input");
+  MXQ_CHECK(in != nullptr && in_type != nullptr && in_min != nullptr && in_max != nullptr &&
+                in_axis != nullptr,
+            "null argument table");
+  MXQ_CHECK(omin != nullptr && omax != nullptr, "null range pointer");
+  MXQ_CHECK(outer >= 0 && inner >= 0, "negative extent");
+  // QuantizedConcatType (quantized_concat.cc:83-103): int8 as soon as one input is
+  int want = MXQ_UINT8;
+  int64_t axis_total = 0;
+  for (int i = 0; i < num_args; ++i) {
+    MXQ_CHECK(byte_type(in_type[i]), "quantized_concat takes int8 or uint8 inputs, input "
+                                         << i << " has type " << in_type[i]);
+    if (in_type[i] == MXQ_INT8) want = MXQ_INT8;
+    MXQ_CHECK(in_axis[i] >= 0, "negative extent of input " << i);
+    MXQ_CHECK(in_min[i] != nullptr && in_max[i] != nullptr, "null range pointer of input " << i);
+    axis_total += in_axis[i];
+  }
+  MXQ_CHECK(out_type == want, "output type must be " << want << ", got " << out_type);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const bool several = num_args > kMaxConcatPerLaunch;
+  if (several) {
+    for (int first = 0; first < num_args; first += kMaxConcatPerLaunch) {
+      ConcatRanges r;
+      r.count = num_args - first < kMaxConcatPerLaunch ? num_args - first : kMaxConcatPerLaunch;
+      r.first = first == 0;
+      for (int i = 0; i < kMaxConcatPerLaunch; ++i) {
+        r.mn[i] = i < r.count ? in_min[first + i] : nullptr;
+        r.mx[i] = i < r.count ? in_max[first + i] : nullptr;
+      }
+      hipLaunchKernelGGL(concat_range_kernel, dim3(1), dim3(1), 0, s, r, omin, omax);
+      MXQ_LAUNCH_CHECK();
+    }
+  }
+  const size_t pitch = static_cast<size_t>(axis_total) * static_cast<size_t>(inner);
+  size_t offset = 0;
+  for (int first = 0; first < num_args; first += kMaxConcatPerLaunch) {
+    ConcatArgs a;
+    a.count = num_args - first < kMaxConcatPerLaunch ? num_args - first : kMaxConcatPerLaunch;
+    a.out = static_cast<uint8_t*>(out);
+    a.rows = static_cast<size_t>(outer);
+    a.out_pitch = pitch;
+    a.omin = omin;
+    a.omax = omax;
+    a.out_type = out_type;
+    a.given_range = several ? 1 : 0;
+    int blocks = 0;
+    size_t launch_bytes = 0;
+    for (int i = 0; i < a.count; ++i)
+      launch_bytes += a.rows * static_cast<size_t>(in_axis[first + i]) * static_cast<size_t>(inner);
+    // twice the work-groups per CU of the narrowing kernels: a 1:1 byte stream holds less
+    // per lane and measured fastest there
+    const int budget = 2 * grid_for(launch_bytes);
+    for (int i = 0; i < kMaxConcatPerLaunch; ++i) {
+      const int k = first + (i < a.count ? i : 0);  // unused slots repeat a valid entry
+      a.in[i] = static_cast<const uint8_t*>(in[k]);
+      a.mn[i] = in_min[k];
+      a.mx[i] = in_max[k];
+      a.in_type[i] = in_type[k];
+      a.row_bytes[i] = static_cast<size_t>(in_axis[k]) * static_cast<size_t>(inner);
+      a.out_off[i] = offset;
+      a.vec_ok[i] = 0;
+      if (i < a.count) {
+        const size_t bytes = a.rows * a.row_bytes[i];
+        MXQ_CHECK(bytes == 0 || (in[k] != nullptr && out != nullptr), "null data pointer");
+        const uint8_t* dst = a.out + offset;
+        a.vec_ok[i] = (aligned16(a.in[i]) && aligned16(dst) && a.row_bytes[i] % 16 == 0 &&
+                       (a.rows == 1 || pitch % 16 == 0)) ? 1 : 0;
+        // work-groups in proportion to the bytes (at least one each, so that the block
+        // table stays monotonic): the inputs of one launch finish together
+        const size_t share = launch_bytes == 0 ? 1 : (size_t(budget) * bytes) / launch_bytes;
+        const int fit = grid_for(a.vec_ok[i] ? bytes / 16 : bytes);
+        blocks += share < 1 ? 1 : (share < size_t(fit) ? static_cast<int>(share) : fit);
+        offset += a.row_bytes[i];
+      }
+      a.block_end[i] = blocks;
+    }
+    hipLaunchKernelGGL(concat_kernel, dim3(blocks), dim3(kThreads), 0, s, a);
+    MXQ_LAUNCH_CHECK();
+  }
+  MXQ_API_END();
+}
+
+}  // extern "C"

@@ -90,6 +90,8 @@ _FLOAT_OPS = {
     "Dropout": lambda a, x: x,
     "elemwise_add": lambda a, x, y: x + y,
     "_plus": lambda a, x, y: x + y,
+    "Concat": lambda a, *xs: torch.cat(xs, dim=int(a.get("dim", "1"))),
+    "concat": lambda a, *xs: torch.cat(xs, dim=int(a.get("dim", "1"))),
 }
 
 

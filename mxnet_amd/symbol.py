@@ -240,3 +240,12 @@ softmax = _make("softmax")
 SoftmaxOutput = _make("SoftmaxOutput")
 Dropout = _make("Dropout")
 elemwise_add = _make("elemwise_add")
+
+
+def Concat(*args, name=None, dim=1, **kwargs):
+    """`mx.sym.Concat(a, b, ..., dim=1)`: num_args is the number of symbols given
+    (the operator's key_var_num_args)."""
+    return create("Concat", *args, name=name, num_args=len(args), dim=dim, **kwargs)
+
+
+concat = Concat

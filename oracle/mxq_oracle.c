@@ -33,6 +33,16 @@
  *     of the exact quotient; checked against an exact rational evaluation and
  *     against the reference test's own bound (|int8 - fp32 pooling| <= 2,
  *     tests/python/quantization/test_quantization.py:634-639).
+ *   - qref_elemwise_add / qref_concat_rescale: the scale derivation follows the
+ *     reference's own files, but the arithmetic that applies the scales runs inside
+ *     oneDNN (dnnl::sum, dnnl::reorder; third-party, absent): PARITY UNPINNED for
+ *     the rounding of each element.  Here: saturate(nearest-even(sum of the scaled
+ *     operands)) with every binary32 operation rounded on its own; checked against
+ *     an exact rational evaluation of that rule, against the reference test's own
+ *     bound (|dequantized - fp32 sum| <= 2,
+ *     tests/python/quantization/test_quantization.py:375-433) and through the
+ *     special cases the scales make exact (equal ranges, concat of equal scales is a
+ *     byte copy).
  */
 #include <math.h>
 #include <stddef.h>
@@ -344,5 +354,94 @@ void qref_pool_nchw(const void* in_, int is_unsigned, int N, int C, int H, int W
           out_s[obase + (size_t)oh * OW + ow] = (int8_t)q;
       }
     }
+  }
+}
+
+/* ---- _contrib_quantized_elemwise_add / _contrib_quantized_concat ---------------
+ * The DNNL operators' ranges: 127.5 for int8, 255.5 for uint8, 2^31 - 1 for int32
+ * (quantization_utils.h:37-39). */
+static inline float q_type_range(int is_unsigned) { return is_unsigned ? 255.5f : 127.5f; }
+
+/* saturate to [lo, hi], then nearest-even; NaN converts to 0 */
+static inline int32_t q_round_sat(float f, float lo, float hi) {
+  if (f != f) return 0;
+  if (f < lo) f = lo;
+  if (f > hi) f = hi;
+  return (int32_t)rintf(f);
+}
+
+/* dnnl_quantized_elemwise_add.cc:134-257 for operands of one shape.
+ * out_kind: 0 int32 (uncalibrated), 1 int8, 2 uint8 (calibrated).  Scales:
+ * A_scale = range(A) / MaxAbs(A_min, A_max) (:152-157); output scale =
+ * double(range(out)) / MaxAbs(calib) or / (|A| + |B|), rounded to float (:169-178);
+ * scales[i] = output_scale / scale_i (:180-182).  A uint8 operand next to an int8 one
+ * is first reordered to int8 with scale 0.5 and its scale doubled (:189-210).
+ * The sum itself is dnnl::sum: dst = saturate(round(s0 * a + s1 * b)). */
+void qref_elemwise_add(const void* lhs_, int lhs_unsigned, const void* rhs_, int rhs_unsigned,
+                       size_t n, float lhs_min, float lhs_max, float rhs_min, float rhs_max,
+                       int out_kind, int calibrated, float min_calib, float max_calib,
+                       void* out_, float* omin, float* omax) {
+  const float a_absmax = q_maxabs(lhs_min, lhs_max), b_absmax = q_maxabs(rhs_min, rhs_max);
+  const float a_scale = q_type_range(lhs_unsigned) / a_absmax;
+  const float b_scale = q_type_range(rhs_unsigned) / b_absmax;
+  const double out_range = out_kind == 0 ? 2147483647.0 : (out_kind == 1 ? 127.5 : 255.5);
+  float output_min, output_max, output_scale;
+  if (calibrated) {
+    output_min = min_calib;
+    output_max = max_calib;
+    output_scale = (float)(out_range / (double)q_maxabs(output_min, output_max));
+  } else {
+    output_max = a_absmax + b_absmax;
+    output_min = -output_max;
+    output_scale = (float)(out_range / (double)output_max);
+  }
+  float s0 = output_scale / a_scale, s1 = output_scale / b_scale;
+  const int halve_a = lhs_unsigned && !rhs_unsigned, halve_b = rhs_unsigned && !lhs_unsigned;
+  if (halve_a) s0 = (float)((double)s0 * (1.0 / 0.5));
+  if (halve_b) s1 = (float)((double)s1 * (1.0 / 0.5));
+  const float lo = out_kind == 0 ? -2147483648.0f : (out_kind == 1 ? -128.0f : 0.0f);
+  /* the largest binary32 below 2^31: what oneDNN saturates int32 to */
+  const float hi = out_kind == 0 ? 2147483520.0f : (out_kind == 1 ? 127.0f : 255.0f);
+#pragma omp parallel for schedule(static)
+  for (ptrdiff_t i = 0; i < (ptrdiff_t)n; ++i) {
+    int a = lhs_unsigned ? (int)((const uint8_t*)lhs_)[i] : (int)((const int8_t*)lhs_)[i];
+    int b = rhs_unsigned ? (int)((const uint8_t*)rhs_)[i] : (int)((const int8_t*)rhs_)[i];
+    if (halve_a) a = q_round_sat((float)a * 0.5f, -128.0f, 127.0f);
+    if (halve_b) b = q_round_sat((float)b * 0.5f, -128.0f, 127.0f);
+    const float x = (float)a * s0;
+    const float y = (float)b * s1;
+    const int32_t q = q_round_sat(x + y, lo, hi);
+    if (out_kind == 0)
+      ((int32_t*)out_)[i] = q;
+    else if (out_kind == 1)
+      ((int8_t*)out_)[i] = (int8_t)q;
+    else
+      ((uint8_t*)out_)[i] = (uint8_t)q;
+  }
+  *omin = output_min;
+  *omax = output_max;
+}
+
+/* One input of dnnl_quantized_concat.cc:68-98 brought to the output's scale:
+ * scale_x = range(type x) / MaxAbs(min_x, max_x) (GetScale, :35-38); equal scales (and
+ * types) copy, otherwise a reorder with scale out_scale / in_scale. */
+void qref_concat_rescale(const void* in_, int in_unsigned, size_t n, float imin, float imax,
+                         float omin, float omax, int out_unsigned, void* out_) {
+  const float out_scale = q_type_range(out_unsigned) / q_maxabs(omin, omax);
+  const float in_scale = q_type_range(in_unsigned) / q_maxabs(imin, imax);
+  if (in_scale == out_scale && in_unsigned == out_unsigned) {
+    memcpy(out_, in_, n);
+    return;
+  }
+  const float scale = out_scale / in_scale;
+  const float lo = out_unsigned ? 0.0f : -128.0f, hi = out_unsigned ? 255.0f : 127.0f;
+#pragma omp parallel for schedule(static)
+  for (ptrdiff_t i = 0; i < (ptrdiff_t)n; ++i) {
+    const int v = in_unsigned ? (int)((const uint8_t*)in_)[i] : (int)((const int8_t*)in_)[i];
+    const int32_t q = q_round_sat((float)v * scale, lo, hi);
+    if (out_unsigned)
+      ((uint8_t*)out_)[i] = (uint8_t)q;
+    else
+      ((int8_t*)out_)[i] = (int8_t)q;
   }
 }

@@ -49,6 +49,9 @@ _lib.qref_fc.argtypes = [_p, _p, _p, _i, _i, _i, _p]
 _lib.qref_conv_nchw.argtypes = [_p, _p, _p] + [_i] * 13 + [_p]
 _lib.qref_relu_i8.argtypes = [_p, _sz, _p]
 _lib.qref_pool_nchw.argtypes = [_p, _i] + [_i] * 12 + [_i, _i, _p]
+_lib.qref_elemwise_add.argtypes = [_p, _i, _p, _i, _sz, _f, _f, _f, _f, _i, _i, _f, _f, _p, _pf,
+                                   _pf]
+_lib.qref_concat_rescale.argtypes = [_p, _i, _sz, _f, _f, _f, _f, _i, _p]
 
 
 def _c(a, dtype):
@@ -266,3 +269,57 @@ def quantized_flatten(data, min_data, max_data):
     (d0, prod(rest)); the ranges pass through."""
     d = np.ascontiguousarray(data)
     return d.reshape(d.shape[0], -1).copy(), np.float32(min_data), np.float32(max_data)
+
+
+def quantized_elemwise_add(lhs, rhs, lhs_min, lhs_max, rhs_min, rhs_max, min_calib_range=None,
+                           max_calib_range=None):
+    """_contrib_quantized_elemwise_add on operands of one shape -> (out, min, max); int32
+    without calibration, else the inputs' type (int8 when they differ)
+    (quantized_elemwise_add.cc:50-78)."""
+    for x in (lhs, rhs):
+        if x.dtype not in (np.int8, np.uint8):
+            raise TypeError("quantized_elemwise_add takes int8 or uint8")
+    if lhs.shape != rhs.shape:
+        raise ValueError("operands must have one shape")
+    a, b = _c(lhs, lhs.dtype), _c(rhs, rhs.dtype)
+    calibrated = min_calib_range is not None and max_calib_range is not None
+    if not calibrated:
+        out_dtype, kind = np.int32, 0
+    elif a.dtype == b.dtype:
+        out_dtype, kind = a.dtype, (1 if a.dtype == np.int8 else 2)
+    else:
+        out_dtype, kind = np.int8, 1
+    out = np.empty(a.shape, dtype=out_dtype)
+    omin, omax = ctypes.c_float(), ctypes.c_float()
+    _lib.qref_elemwise_add(_ptr(a), int(a.dtype == np.uint8), _ptr(b), int(b.dtype == np.uint8),
+                           a.size, lhs_min, lhs_max, rhs_min, rhs_max, kind, int(calibrated),
+                           min_calib_range if calibrated else 0.0,
+                           max_calib_range if calibrated else 0.0, _ptr(out),
+                           ctypes.byref(omin), ctypes.byref(omax))
+    return out, np.float32(omin.value), np.float32(omax.value)
+
+
+def quantized_concat(arrays, mins, maxs, dim=1):
+    """_contrib_quantized_concat -> (out, min, max): the output range is the hull of the
+    input ranges and 0 (dnnl_quantized_concat.cc:53-67), the type int8 as soon as one
+    input is int8 (quantized_concat.cc:83-103)."""
+    if not arrays or len(arrays) != len(mins) or len(arrays) != len(maxs):
+        raise ValueError("one range per input")
+    for x in arrays:
+        if x.dtype not in (np.int8, np.uint8):
+            raise TypeError("quantized_concat takes int8 or uint8")
+    out_dtype = np.int8 if any(x.dtype == np.int8 for x in arrays) else np.uint8
+    omin, omax = np.float32(0.0), np.float32(0.0)
+    for lo, hi in zip(mins, maxs):
+        if np.float32(lo) < omin:
+            omin = np.float32(lo)
+        if np.float32(hi) > omax:
+            omax = np.float32(hi)
+    parts = []
+    for x, lo, hi in zip(arrays, mins, maxs):
+        x = _c(x, x.dtype)
+        y = np.empty(x.shape, dtype=out_dtype)
+        _lib.qref_concat_rescale(_ptr(x), int(x.dtype == np.uint8), x.size, lo, hi, omin, omax,
+                                 int(out_dtype == np.uint8), _ptr(y))
+        parts.append(y)
+    return np.concatenate(parts, axis=dim), omin, omax

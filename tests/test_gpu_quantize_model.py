@@ -124,3 +124,62 @@ def test_calibration_sees_every_requested_tensor():
     ex.forward(data=torch.tensor(rng.normal(0, 1, (2, 4, 8, 8)), dtype=torch.float32))
     assert set(calib_layers) <= set(seen)
     assert "conv_data" in seen and "conv_output" in seen and "bn_output" in seen
+
+
+def build_residual():
+    from mxnet_amd import symbol as S
+    data = S.Variable("data")
+    c1 = S.Convolution(data, kernel=(3, 3), pad=(1, 1), num_filter=16, name="conv1")
+    r1 = S.Activation(c1, act_type="relu", name="relu1")
+    c2 = S.Convolution(r1, kernel=(3, 3), pad=(1, 1), num_filter=16, name="conv2")
+    add = S.elemwise_add(c2, r1, name="add")
+    r2 = S.Activation(add, act_type="relu", name="relu2")
+    c3 = S.Convolution(r2, kernel=(1, 1), num_filter=8, name="conv3")
+    cat = S.Concat(c3, r1, name="cat")
+    pool = S.Pooling(cat, kernel=(8, 8), global_pool=True, pool_type="avg", name="pool")
+    flat = S.Flatten(pool, name="flat")
+    return S.FullyConnected(flat, num_hidden=10, name="fc")
+
+
+def test_residual_block_with_concat_stays_int8_end_to_end():
+    """A residual sum and a concatenation between quantized convolutions: the int8 graph
+    runs through _contrib_quantized_elemwise_add / _contrib_quantized_concat, tracks the
+    float network, and the sum's output equals the oracle's on the tensors that reach it."""
+    from mxnet_amd import quantization as Q
+    from mxnet_amd.executor import Executor
+    rng = np.random.default_rng(7)
+    sym = build_residual()
+    f = lambda v: torch.tensor(v, dtype=torch.float32)
+    arg = {"conv1_weight": f(rng.normal(0, 0.2, (16, 4, 3, 3))), "conv1_bias": f(rng.normal(0, 0.1, 16)),
+           "conv2_weight": f(rng.normal(0, 0.1, (16, 16, 3, 3))), "conv2_bias": f(rng.normal(0, 0.1, 16)),
+           "conv3_weight": f(rng.normal(0, 0.2, (8, 16, 1, 1))), "conv3_bias": f(rng.normal(0, 0.1, 8)),
+           "fc_weight": f(rng.normal(0, 0.2, (10, 24))), "fc_bias": f(rng.normal(0, 0.1, 10))}
+    calib = [f(rng.normal(0, 1, (16, 4, 8, 8))) for _ in range(3)]
+    qsym, qarg, qaux = Q.quantize_model(sym, arg, {}, calib_mode="naive", calib_data=calib,
+                                        num_calib_batches=3, quantize_mode="full")
+    ops = [op for op, _, _, _ in qsym.nodes() if op != "null"]
+    assert ops.count("_contrib_quantized_elemwise_add") == 1
+    assert ops.count("_contrib_quantized_concat") == 1
+    # int8 from the first quantize to the last dequantize
+    assert ops.count("_contrib_quantize_v2") == 1 and ops.count("_contrib_dequantize") == 1
+    attrs = qsym.attr_dict()
+    assert "min_calib_range" in attrs["requantize_add"]
+    x = f(rng.normal(0, 1, (32, 4, 8, 8)))
+    fp = Executor(sym, arg).forward(data=x)[0]
+    q = Executor(qsym, {**qarg, **qaux}).forward(data=x)[0]
+    assert q.shape == fp.shape == (32, 10)
+    scale = fp.abs().max().item()
+    assert (q - fp).abs().max().item() < 0.08 * scale
+    # the sum itself against the oracle, on the operands the graph feeds it
+    internals = qsym.get_internals()
+    from mxnet_amd import symbol as S
+    probe = S.Group([internals["requantize_conv2_output0"], internals["requantize_conv2_output1"],
+                     internals["requantize_conv2_output2"], internals["quantized_relu1_output"],
+                     internals["quantized_relu1_min_output"], internals["quantized_relu1_max_output"],
+                     internals["quantized_add_output"], internals["quantized_add_min_output"],
+                     internals["quantized_add_max_output"]])
+    a, amin, amax, b, bmin, bmax, s, smin, smax = [
+        t.cpu().numpy() for t in Executor(probe, {**qarg, **qaux}).forward(data=x)]
+    ref, rmin, rmax = oracle.quantized_elemwise_add(a, b, amin[0], amax[0], bmin[0], bmax[0])
+    np.testing.assert_array_equal(s, ref)
+    assert smin[0] == rmin and smax[0] == rmax

@@ -197,3 +197,51 @@ def test_pooling_and_flatten_inference():
     assert n.infer_shape([(2, 3, 4, 5), None, None]) == ([(2, 3, 4, 5), (1,), (1,)],
                                                          [(2, 60), (1,), (1,)])
     assert n.infer_type([U8, None, None]) == ([U8, F32, F32], [U8, F32, F32])
+
+
+def test_elemwise_add_and_concat_inference():
+    """quantized_elemwise_add.cc:30-122, quantized_concat.cc:31-141."""
+    for n in ["_contrib_quantized_elemwise_add", "_contrib_quantized_concat"]:
+        assert op.has_attr(n, "FCompute<gpu>") and op.has_attr(n, "FInferShape")
+    assert op.has_attr("_npx_quantized_elemwise_add", "FInferType")
+    assert op.has_attr("_contrib_quantized_elemwise_add", "FNeedRequantize")
+    assert not op.has_attr("_contrib_quantized_concat", "FNeedRequantize")
+    assert op.has_attr("elemwise_add", "FQuantizedOp") and op.has_attr("Concat", "FQuantizedOp")
+    n = Node("_contrib_quantized_elemwise_add")
+    assert n.list_inputs() == ["lhs", "rhs", "lhs_min", "lhs_max", "rhs_min", "rhs_max"]
+    assert n.list_outputs() == ["output", "min_output", "max_output"]
+    ins, outs = n.infer_shape([(3, 4, 5), (3, 4, 5), None, None, None, None])
+    assert ins == [(3, 4, 5), (3, 4, 5)] + [(1,)] * 4 and outs == [(3, 4, 5), (1,), (1,)]
+    with pytest.raises(MXNetError):
+        n.infer_shape([(3, 4, 5), (3, 4, 6), None, None, None, None])
+    # int32 unless calibrated; then the operands' type, int8 when they differ
+    assert n.infer_type([I8, U8, None, None, None, None])[1] == [I32, F32, F32]
+    c = Node("_contrib_quantized_elemwise_add", min_calib_range=-1.0, max_calib_range=2.0)
+    assert c.infer_type([I8, I8, None, None, None, None])[1][0] == I8
+    assert c.infer_type([U8, U8, None, None, None, None])[1][0] == U8
+    assert c.infer_type([I8, U8, None, None, None, None])[1][0] == I8
+    half = Node("_contrib_quantized_elemwise_add", min_calib_range=-1.0)
+    assert half.infer_type([I8, I8, None, None, None, None])[1][0] == I32
+    with pytest.raises(MXNetError):
+        Node("_contrib_quantized_elemwise_add", out_type="int8")
+
+    n = Node("_contrib_quantized_concat", num_args=3, dim=1)
+    assert n.num_inputs == 9
+    assert n.list_inputs() == ["arg0", "arg1", "arg2", "arg0_min", "arg0_max", "arg1_min",
+                               "arg1_max", "arg2_min", "arg2_max"]
+    ins, outs = n.infer_shape([(2, 3, 4), (2, 5, 4), (2, 1, 4)] + [None] * 6)
+    assert ins[:3] == [(2, 3, 4), (2, 5, 4), (2, 1, 4)] and ins[3:] == [(1,)] * 6
+    assert outs == [(2, 9, 4), (1,), (1,)]
+    assert Node("_contrib_quantized_concat", num_args=2, dim=-1).infer_shape(
+        [(2, 3), (2, 4)] + [None] * 4)[1][0] == (2, 7)
+    assert Node("_contrib_quantized_concat", num_args=2, dim=0).infer_shape(
+        [(2, 3), (5, 3)] + [None] * 4)[1][0] == (7, 3)
+    with pytest.raises(MXNetError, match="Incompatible input shape"):
+        n.infer_shape([(2, 3, 4), (2, 5, 5), (2, 1, 4)] + [None] * 6)
+    with pytest.raises(MXNetError, match="exceeds the input dimension"):
+        Node("_contrib_quantized_concat", num_args=2, dim=2).infer_shape(
+            [(2, 3), (2, 4)] + [None] * 4)
+    assert n.infer_type([U8, U8, U8] + [None] * 6)[1] == [U8, F32, F32]
+    assert n.infer_type([U8, I8, U8] + [None] * 6)[1] == [I8, F32, F32]
+    with pytest.raises(MXNetError, match="num_args"):
+        Node("_contrib_quantized_concat", dim=1)

@@ -191,13 +191,20 @@ def test_shared_float_producer_gets_one_quantize_node():
     b = S.FullyConnected(bn, num_hidden=4, no_bias=True, name="b")
     out = S.elemwise_add(a, b, name="sum")
     qsym, calib = Q._quantize_symbol(out, "gpu", offline_params=["a_weight", "b_weight"],
-                                     quantize_mode="full")
+                                     quantize_mode="full", excluded_operators=["elemwise_add"])
     names = [n for _, n in ops_of(qsym)]
     assert names.count("bn_output_quantize") == 1
     assert node(qsym, "quantized_a")[2][0] == ("bn_output_quantize", 0)
     assert node(qsym, "quantized_b")[2][0] == ("bn_output_quantize", 0)
     assert node(qsym, "sum")[2] == [("a_dequantize", 0), ("b_dequantize", 0)]
     assert calib == ["bn_output", "a_output", "b_output"]
+    # with the sum quantized as well the graph leaves int8 only at its head
+    qsym, calib = Q._quantize_symbol(out, "gpu", offline_params=["a_weight", "b_weight"],
+                                     quantize_mode="full")
+    assert [n for _, n in ops_of(qsym)][-3:] == ["quantized_sum", "requantize_sum",
+                                                 "sum_dequantize"]
+    assert node(qsym, "quantized_sum")[2][:2] == [("requantize_a", 0), ("requantize_b", 0)]
+    assert calib == ["bn_output", "a_output", "b_output", "sum_output"]
 
 
 def test_quantize_params_names():
@@ -337,3 +344,54 @@ def test_histogram_collector_merges_batches():
     m.collect("x", "op", torch.tensor([-1.0, 3.0]))
     m.collect("x", "op", torch.tensor([-2.0, 1.0]))
     assert m.post_collect() == {"x": (-2.0, 3.0)}
+
+
+def test_residual_add_and_concat_stay_int8():
+    """elemwise_add (quantized_elemwise_add.cc:124-133, FNeedRequantize) and Concat
+    (quantized_concat.cc:143-152): data inputs first, then one (min, max) pair per input in
+    input order, as quantize_graph_pass.cc wires every quantized operator."""
+    d = S.Variable("data")
+    c1 = S.Convolution(d, kernel=(3, 3), pad=(1, 1), num_filter=16, name="conv1")
+    r1 = S.Activation(c1, act_type="relu", name="relu1")
+    c2 = S.Convolution(r1, kernel=(3, 3), pad=(1, 1), num_filter=16, name="conv2")
+    add = S.elemwise_add(c2, r1, name="add")
+    c3 = S.Convolution(add, kernel=(1, 1), num_filter=8, name="conv3")
+    cat = S.Concat(c3, r1, name="cat")
+    fc = S.FullyConnected(cat, num_hidden=10, name="fc")
+    assert node(fc, "cat")[1] == {"dim": "1", "num_args": "2"}
+    qsym, calib = Q._quantize_symbol(fc, "gpu", offline_params=offline_of(fc),
+                                     quantize_mode="full")
+    assert [o for o in ops_of(qsym) if o[0] != "_contrib_quantized_conv"] == [
+        ("_contrib_quantize_v2", "conv1_data_quantize"),
+        ("_contrib_requantize", "requantize_conv1"),
+        ("_contrib_quantized_act", "quantized_relu1"),
+        ("_contrib_requantize", "requantize_conv2"),
+        ("_contrib_quantized_elemwise_add", "quantized_add"),
+        ("_contrib_requantize", "requantize_add"),
+        ("_contrib_requantize", "requantize_conv3"),
+        ("_contrib_quantized_concat", "quantized_cat"),
+        ("_contrib_quantized_fully_connected", "quantized_fc"),
+        ("_contrib_requantize", "requantize_fc"),
+        ("_contrib_dequantize", "fc_dequantize")]
+    assert node(qsym, "quantized_add")[2] == [
+        ("requantize_conv2", 0), ("quantized_relu1", 0), ("requantize_conv2", 1),
+        ("requantize_conv2", 2), ("quantized_relu1", 1), ("quantized_relu1", 2)]
+    assert node(qsym, "requantize_add")[2] == [("quantized_add", 0), ("quantized_add", 1),
+                                               ("quantized_add", 2)]
+    assert node(qsym, "quantized_cat")[1:] == (
+        {"dim": "1", "num_args": "2"},
+        [("requantize_conv3", 0), ("quantized_relu1", 0), ("requantize_conv3", 1),
+         ("requantize_conv3", 2), ("quantized_relu1", 1), ("quantized_relu1", 2)])
+    assert node(qsym, "quantized_fc")[2][0] == ("quantized_cat", 0)
+    assert calib == ["conv1_data", "conv1_output", "conv2_output", "add_output", "conv3_output",
+                     "fc_output"]
+    # the calibrated range of the sum lands on its requantize node
+    cq = Q._calibrate_quantized_sym(qsym, {"add_output": (-3.0, 5.0)})
+    assert node(cq, "requantize_add")[1] == {"out_type": "int8", "min_calib_range": "-3",
+                                             "max_calib_range": "5"} or \
+        float(node(cq, "requantize_add")[1]["max_calib_range"]) == 5.0
+    # the reference's GPU registry has neither operator: excluding them reproduces its graph
+    gsym, _ = Q._quantize_symbol(fc, "gpu", offline_params=offline_of(fc), quantize_mode="full",
+                                 excluded_operators=["elemwise_add", "Concat"])
+    names = [n for _, n in ops_of(gsym)]
+    assert "add" in names and "cat" in names and "quantized_add" not in names
