@@ -1,0 +1,169 @@
+"""The benchmark configurations at their full sizes: 2^26-element cast tensors compared with
+the oracle element for element; the 8192^3 fully-connected layer and the BERT-base layers
+through sampled rows and columns the oracle recomputes, linearity, and the identity
+fused-int8 == requantize(int32); every distinct ResNet-50 bottleneck convolution at batch 64
+against the oracle on the first and last image of the batch."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+
+pytestmark = pytest.mark.gpu
+
+N_CAST = 1 << 26
+
+
+@pytest.fixture(scope="module")
+def capi():
+    import mxnet_amd
+    return mxnet_amd.capi
+
+
+@pytest.fixture(scope="module")
+def contrib():
+    import mxnet_amd
+    return mxnet_amd.contrib
+
+
+def f32(v):
+    return torch.tensor([v], dtype=torch.float32, device="cuda")
+
+
+def cast_input(seed):
+    """N(0,1) with 0.01 % of the positions at +-50, as the benchmark draws it."""
+    g = torch.Generator(device="cuda").manual_seed(seed)
+    x = torch.randn(N_CAST, device="cuda", generator=g)
+    idx = torch.randint(0, N_CAST, (N_CAST // 10000,), device="cuda", generator=g)
+    sign = torch.randint(0, 2, (N_CAST // 10000,), device="cuda", generator=g) * 2 - 1
+    x[idx] = 50.0 * sign.to(torch.float32)
+    return x
+
+
+@pytest.mark.parametrize("calib", [None, (-50.0, 50.0), (-4.0, 4.0)])
+def test_quantize_v2_64m(capi, calib):
+    x = cast_input(1)
+    kw = {} if calib is None else {"min_calib_range": calib[0], "max_calib_range": calib[1]}
+    q, mn, mx = capi.quantize_v2(x, "int8", **kw)
+    ref, rmn, rmx = oracle.quantize_v2(x.cpu().numpy(), "int8", *(calib or ()))
+    assert (mn.item(), mx.item()) == (rmn, rmx)
+    assert np.array_equal(q.cpu().numpy(), ref)
+
+
+def test_quantize_v2_uint8_64m(capi):
+    x = cast_input(2)
+    lo, hi = float(x.min()), float(x.max())
+    q, mn, mx = capi.quantize_v2(x, "uint8", min_calib_range=lo, max_calib_range=hi)
+    ref, rmn, rmx = oracle.quantize_v2(x.cpu().numpy(), "uint8", lo, hi)
+    assert (mn.item(), mx.item()) == (rmn, rmx)
+    assert np.array_equal(q.cpu().numpy(), ref)
+
+
+@pytest.mark.parametrize("calibrated", [False, True])
+def test_requantize_64m(capi, calibrated):
+    g = torch.Generator(device="cuda").manual_seed(3)
+    x = torch.randint(-2 ** 28, 2 ** 28, (N_CAST,), device="cuda", generator=g, dtype=torch.int32)
+    kw = {"min_calib_range": -0.1, "max_calib_range": 0.1} if calibrated else {}
+    q, mn, mx = capi.requantize(x, f32(-1.0), f32(1.0), **kw)
+    ref, rmn, rmx = oracle.requantize(x.cpu().numpy(), -1.0, 1.0, *kw.values())
+    assert (mn.item(), mx.item()) == (rmn, rmx)
+    assert np.array_equal(q.cpu().numpy(), ref)
+
+
+def test_dequantize_64m(capi):
+    g = torch.Generator(device="cuda").manual_seed(4)
+    q = torch.randint(-127, 128, (N_CAST,), device="cuda", generator=g, dtype=torch.int8)
+    y = capi.dequantize(q, f32(-3.0), f32(3.0))
+    ref = oracle.dequantize(q.cpu().numpy(), -3.0, 3.0)
+    got = y.cpu().numpy()
+    assert np.array_equal(got.view(np.uint32), ref.view(np.uint32))
+
+
+def test_elemwise_add_64m(contrib):
+    g = torch.Generator(device="cuda").manual_seed(5)
+    a = torch.randint(-127, 128, (N_CAST,), device="cuda", generator=g, dtype=torch.int8)
+    b = torch.randint(-127, 128, (N_CAST,), device="cuda", generator=g, dtype=torch.int8)
+    for kw in ({}, {"min_calib_range": -5.0, "max_calib_range": 5.0}):
+        out, mn, mx = contrib.quantized_elemwise_add(a, b, f32(-3.0), f32(3.0), f32(-3.0),
+                                                     f32(3.0), **kw)
+        ref, rmn, rmx = oracle.quantized_elemwise_add(a.cpu().numpy(), b.cpu().numpy(), -3.0, 3.0,
+                                                      -3.0, 3.0, **kw)
+        assert (mn.item(), mx.item()) == (rmn, rmx)
+        assert np.array_equal(out.cpu().numpy(), ref)
+
+
+def check_fc(capi, M, K, N, seed):
+    g = torch.Generator(device="cuda").manual_seed(seed)
+    d1 = torch.randint(-60, 61, (M, K), device="cuda", generator=g, dtype=torch.int8)
+    d2 = torch.randint(-60, 61, (M, K), device="cuda", generator=g, dtype=torch.int8)
+    w = torch.randint(-127, 128, (N, K), device="cuda", generator=g, dtype=torch.int8)
+    b = torch.randint(-127, 128, (N,), device="cuda", generator=g, dtype=torch.int8)
+    one = f32(1.0)
+    args = (-one, one, -one, one)
+    r1 = capi.quantized_fc(d1, w, None, *args)["out32"]
+    r2 = capi.quantized_fc(d2, w, None, *args)["out32"]
+    r12 = capi.quantized_fc(d1 + d2, w, None, *args)["out32"]
+    assert torch.equal(r1 + r2, r12)                      # linear in the data operand
+    rows = sorted({0, 1, 255, 256, M // 2 - 1, M // 2, M - 257, M - 1})
+    want = oracle.fc_int32(d1[rows].cpu().numpy(), w.cpu().numpy())
+    assert np.array_equal(r1[rows].cpu().numpy(), want)
+    cols = sorted({0, 31, 32, 255, 256, N // 2, N - 1})
+    want_c = oracle.fc_int32(d1.cpu().numpy(), w[cols].cpu().numpy())
+    assert np.array_equal(r1[:, cols].cpu().numpy(), want_c)
+    del r2, r12
+    # the fused epilogue (bias + relu + requantize) is the int32 result requantized
+    # calibrated to two standard deviations of the accumulator (in its float units)
+    c = 2.0 * 35.0 * 73.0 * K ** 0.5 / 127.0 ** 2
+    res = capi.quantized_fc(d1, w, b, *args, -one, one, calib=(-c, c), relu=True)
+    q, mn, mx = capi.requantize(res["out32"], res["omin"], res["omax"], min_calib_range=-c,
+                                max_calib_range=c)
+    assert torch.equal(res["out8"], torch.clamp(q, min=0))
+    assert (res["rmin"].item(), res["rmax"].item()) == (mn.item(), mx.item())
+    assert int(res["out8"].max()) == 127 and 0.2 < float((res["out8"] > 0).float().mean()) < 0.8
+
+
+def test_fc_8192(capi):
+    check_fc(capi, 8192, 8192, 8192, seed=8)
+
+
+@pytest.mark.parametrize("K,N", [(768, 2304), (768, 768), (768, 3072), (3072, 768)])
+def test_fc_bert_base_layers(capi, K, N):
+    check_fc(capi, 4096, K, N, seed=K + N)
+
+
+RESNET50_CONVS = [(56, 64, 64, 1, 1), (56, 64, 64, 3, 1), (56, 64, 256, 1, 1), (56, 256, 64, 1, 1),
+                  (56, 256, 128, 1, 2), (28, 128, 128, 3, 1), (28, 128, 512, 1, 1),
+                  (28, 512, 128, 1, 1), (56, 256, 512, 1, 2), (28, 512, 256, 1, 2),
+                  (14, 256, 256, 3, 1), (14, 256, 1024, 1, 1), (14, 1024, 256, 1, 1),
+                  (28, 512, 1024, 1, 2), (14, 1024, 512, 1, 2), (7, 512, 512, 3, 1),
+                  (7, 512, 2048, 1, 1), (7, 2048, 512, 1, 1), (14, 1024, 2048, 1, 2)]
+
+
+@pytest.mark.parametrize("H,C,O,k,s", RESNET50_CONVS)
+def test_resnet50_conv_batch64(capi, H, C, O, k, s):
+    batch, pad = 64, (1 if k == 3 else 0)
+    g = torch.Generator(device="cuda").manual_seed(H + C + O + k)
+    d = torch.randint(-127, 128, (batch, H, H, C), device="cuda", generator=g, dtype=torch.int8)
+    w = torch.randint(-127, 128, (O, k, k, C), device="cuda", generator=g, dtype=torch.int8)
+    b = torch.randint(-127, 128, (O,), device="cuda", generator=g, dtype=torch.int8)
+    one = f32(1.0)
+    r = 2.0 * 73.0 * 73.0 * (k * k * C) ** 0.5 / 127.0 ** 2   # two standard deviations
+    res = capi.quantized_conv_nhwc(d, w, b, -one, one, -one, one, -one, one, stride=(s, s),
+                                   pad=(pad, pad), calib=(-r, r), relu=True)
+    images = [0, batch - 1]
+    dn = d[images].permute(0, 3, 1, 2).contiguous().cpu().numpy()
+    wn = w.permute(0, 3, 1, 2).contiguous().cpu().numpy()
+    acc, omin, omax = oracle.quantized_conv(dn, wn, b.cpu().numpy(), -1.0, 1.0, -1.0, 1.0, -1.0,
+                                            1.0, stride=(s, s), pad=(pad, pad))
+    got32 = res["out32"][images].permute(0, 3, 1, 2).contiguous().cpu().numpy()
+    assert np.array_equal(got32, acc)
+    assert (res["omin"].item(), res["omax"].item()) == (omin, omax)
+    q, rmin, rmax = oracle.requantize(acc, omin, omax, -r, r)
+    got8 = res["out8"][images].permute(0, 3, 1, 2).contiguous().cpu().numpy()
+    assert np.array_equal(got8, np.maximum(q, 0))
+    # the images between them through the identity fused == requantize(int32)
+    q_all, _, _ = capi.requantize(res["out32"], res["omin"], res["omax"], min_calib_range=-r,
+                                  max_calib_range=r)
+    assert torch.equal(res["out8"], torch.clamp(q_all, min=0))
+    frac = float((res["out8"] > 0).float().mean())
+    assert 0.2 < frac < 0.8 and int(res["out8"].max()) == 127
