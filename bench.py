@@ -32,13 +32,21 @@ METRIC = "int8 FC TOPS (% MFMA peak) + quant/requant GB/s (% HBM peak), 1 GPU"
 HBM_PEAK_GBS = 8000.0    # MI355X HBM3E
 INT8_PEAK_TOPS = 5000.0  # MI355X dense int8 MFMA
 
-# HBM bytes per launch of the workload's kernel from `rocprofv3 --pmc FETCH_SIZE` and
-# `--pmc WRITE_SIZE` runs (FETCH_SIZE x 2.00 per the copy-kernel calibration); the
-# summaries are profiles/fc_dma_kernel_4096.md, profiles/quantize_kernel_64M.md and
-# profiles/copy_calibration_64M.md.  None = not measured.
+# HBM bytes per step of the workload's kernels from `rocprofv3 --pmc FETCH_SIZE` and
+# `--pmc WRITE_SIZE` runs (KiB per dispatch; FETCH_SIZE x 2.00 per the copy-kernel
+# calibration, profiles/copy_calibration_64M.md); each entry names its summary under
+# profiles/.  None = not measured.
+_KIB = 1024.0
 MEASURED_TRAFFIC_BYTES = {
-    "fc4096": 2.0 * 49309.8 * 1024 + 16384.1 * 1024,
-    "quantize": 2.0 * 131102.5 * 1024 + 65536.1 * 1024,
+    "fc4096": (2.0 * 49309.8 + 16384.1) * _KIB,                 # fc_dma_kernel_4096.md
+    "quantize": (2.0 * 131102.5 + 65536.1) * _KIB,              # quantize_kernel_64M.md
+    "quantize_uncal": (2.0 * (131093.7 + 131139.1) + 65536.1) * _KIB,   # quantize_uncalibrated_64M.md
+    "requantize": (2.0 * 131104.8 + 65536.1) * _KIB,            # requantize_kernel_64M.md
+    "requantize_uncal": (2.0 * (131089.2 + 131139.2) + 65536.1) * _KIB,  # requantize_uncalibrated_64M.md
+    "dequantize": (2.0 * 32784.6 + 262224.7) * _KIB,            # dequantize_kernel_64M.md
+    "elemwise_add": (2.0 * 65570.1 + 262176.7) * _KIB,          # add_kernel_int32_64M.md
+    "elemwise_add_int8": (2.0 * 65583.7 + 65536.1) * _KIB,      # add_kernel_int8_64M.md
+    "concat": (2.0 * 32840.8 + 65536.1) * _KIB,                 # concat_kernel_64M.md
 }
 
 
