@@ -85,9 +85,6 @@ __device__ __forceinline__ int byte_of(uint32_t w, int k) {
   const uint32_t b = (w >> (8 * k)) & 0xffu;
   return UNSIGNED ? static_cast<int>(b) : static_cast<int>(static_cast<int8_t>(b));
 }
-__device__ __forceinline__ int byte_at(uint32_t w, int k, bool is_unsigned) {
-  return is_unsigned ? byte_of<true>(w, k) : byte_of<false>(w, k);
-}
 
 // uint8 -> int8 at half scale, as the reference's reorder with scale 0.5 does before a
 // mixed-type sum (dnnl_quantized_elemwise_add.cc:189-210)

@@ -152,6 +152,78 @@ __device__ __forceinline__ void pool_strip(const uint8_t* lds, int base, int row
   }
 }
 
+// Max over K x K windows at horizontal stride 2 without touching single bytes: the strip's
+// dwords are split into their even and odd bytes as two 16-bit lanes each (two ANDs), and
+// rows, then neighbouring columns, are folded with the packed 16-bit max.  Signed bytes are
+// first biased by 0x80 so that unsigned order is their order (0 is then the lowest value,
+// which is also what masked-out positions become).  Per eight outputs: 4 instructions per
+// strip dword and window row, 4 per dword to fold the rows, 4 per output pair to fold the
+// columns, 2 to pack; the byte-at-a-time form above needs about twice as many.
+typedef unsigned short us2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t pk_max_u16(uint32_t x, uint32_t y) {
+  return __builtin_bit_cast(uint32_t, __builtin_elementwise_max(__builtin_bit_cast(us2, x),
+                                                                __builtin_bit_cast(us2, y)));
+}
+
+template <bool UNSIGNED, int K>
+__device__ __forceinline__ void pool_strip_max2(const uint8_t* lds, int base, int row0, int row1,
+                                                const PoolArgs& a, int oh, int ow0,
+                                                uint32_t (&packed)[kPoolItem / 4]) {
+  static_assert(K == 2 || K == 3, "window");
+  constexpr int SPAN = (kPoolItem - 1) * 2 + K;
+  constexpr int NW = (SPAN + 3 + 3) / 4;
+  constexpr uint32_t bias = UNSIGNED ? 0u : 0x80808080u;
+  const uint32_t* words = reinterpret_cast<const uint32_t*>(lds);
+  const int h0 = oh * a.sh - a.ph;
+  const int w0 = ow0 * 2 - a.pw;
+  // Columns outside the image are masked to 0, the lowest biased value: one bit per strip
+  // byte, then each dword's four bits spread to byte masks (bit k of the nibble times
+  // 0x00204081 lands on bit 8k without carries).
+  const int first = max(-w0, 0), last = max(min(a.W - w0, SPAN), first);
+  const uint32_t valid = __builtin_amdgcn_ubfe(0xffffffffu, 0, last - first) << first;
+  uint32_t keep[NW];
+#pragma unroll
+  for (int w = 0; w < NW; ++w)
+    keep[w] = ((((valid >> (4 * w)) & 0xfu) * 0x00204081u) & 0x01010101u) * 0xffu;
+  uint32_t even[NW], odd[NW];  // bytes 0,2 in the low byte / bytes 1,3 in the high byte of a lane
+#pragma unroll
+  for (int w = 0; w < NW; ++w) even[w] = odd[w] = 0u;
+  // Rows outside the image are replaced by the nearest staged row: that row belongs to the
+  // same window whenever the window meets the image at all, and a repeated row leaves a
+  // maximum unchanged.  A window that lies outside altogether is dealt with at the end.
+#pragma unroll
+  for (int r = 0; r < K; ++r) {
+    const int hh = min(max(h0 + r, row0), row1 - 1);
+    const int off = base + (hh - row0) * a.W + w0;
+    const int wi = off >> 2;
+    const uint32_t sft = static_cast<uint32_t>(off & 3);
+    uint32_t d[NW + 1];
+#pragma unroll
+    for (int w = 0; w < NW; ++w) d[w] = words[wi + w];
+    d[NW] = 0u;
+#pragma unroll
+    for (int w = 0; w < NW; ++w) {
+      const uint32_t x = (__builtin_amdgcn_alignbyte(d[w + 1], d[w], sft) ^ bias) & keep[w];
+      even[w] = pk_max_u16(even[w], x & 0x00ff00ffu);
+      odd[w] = pk_max_u16(odd[w], x & 0xff00ff00u);
+    }
+  }
+  // lanes of `even`: bytes 4w, 4w+2; of `odd` (after the shift): bytes 4w+1, 4w+3.
+  // outputs 2w, 2w+1 = max(b[4w], b[4w+1], b[4w+2]), max(b[4w+2], b[4w+3], b[4w+4])
+  uint32_t res[kPoolItem / 2];
+#pragma unroll
+  for (int w = 0; w < kPoolItem / 2; ++w) {
+    res[w] = pk_max_u16(even[w], odd[w] >> 8);
+    if (K == 3)
+      res[w] = pk_max_u16(res[w], __builtin_amdgcn_alignbit(even[w + 1], even[w], 16));
+  }
+  const bool meets_image = h0 < a.H && h0 + K > 0;
+#pragma unroll
+  for (int w = 0; w < kPoolItem / 4; ++w)
+    packed[w] = meets_image ? (__builtin_amdgcn_perm(res[2 * w + 1], res[2 * w], 0x06040200u) ^ bias)
+                            : bias;
+}
+
 // Sum of the n bytes at LDS byte address `addr`: aligned dwords through the 4-way
 // byte dot product against 0x01010101, the partial first and last dwords masked.
 template <bool UNSIGNED>
@@ -267,27 +339,32 @@ __global__ __launch_bounds__(kPoolThreads) void pool_lds_kernel(PoolArgs a) {
     const int orow = fast_div(r, a.magic_per_row), ow0 = (r - orow * per_row) * kPoolItem;
     const int oh = oh0 + orow;
     const int nout = min(kPoolItem, a.OW - ow0);
-    int q[kPoolItem];
-#pragma unroll
-    for (int i = 0; i < kPoolItem; ++i) q[i] = 0;
-    if (FAST != 0) {
+    uint32_t packed[kPoolItem / 4];
+    if (!AVG && (FAST == 1 || FAST == 2)) {
       const int base = 16 + shift + p * static_cast<int>(plane_bytes);
-      pool_strip<UNSIGNED, AVG, K, SW>(lds_raw, base, hs, he, a, oh, ow0, q);
+      pool_strip_max2<UNSIGNED, K>(lds_raw, base, hs, he, a, oh, ow0, packed);
     } else {
-      const uint8_t* img = lds + shift + static_cast<size_t>(p) * plane_bytes;
-      // (fixed trip count: a runtime-indexed q[] would live in scratch memory)
+      int q[kPoolItem];
 #pragma unroll
-      for (int i = 0; i < kPoolItem; ++i)
-        if (i < nout) q[i] = pool_window<UNSIGNED>(img, hs, a, oh, ow0 + i);
+      for (int i = 0; i < kPoolItem; ++i) q[i] = 0;
+      if (FAST != 0) {
+        const int base = 16 + shift + p * static_cast<int>(plane_bytes);
+        pool_strip<UNSIGNED, AVG, K, SW>(lds_raw, base, hs, he, a, oh, ow0, q);
+      } else {
+        const uint8_t* img = lds + shift + static_cast<size_t>(p) * plane_bytes;
+        // (fixed trip count: a runtime-indexed q[] would live in scratch memory)
+#pragma unroll
+        for (int i = 0; i < kPoolItem; ++i)
+          if (i < nout) q[i] = pool_window<UNSIGNED>(img, hs, a, oh, ow0 + i);
+      }
+#pragma unroll
+      for (int w = 0; w < kPoolItem / 4; ++w)
+        packed[w] = (static_cast<uint32_t>(q[4 * w]) & 0xffu) |
+                    ((static_cast<uint32_t>(q[4 * w + 1]) & 0xffu) << 8) |
+                    ((static_cast<uint32_t>(q[4 * w + 2]) & 0xffu) << 16) |
+                    (static_cast<uint32_t>(q[4 * w + 3]) << 24);
     }
     const size_t off = (static_cast<size_t>(p0 + p) * a.OH + oh) * a.OW + ow0;
-    uint32_t packed[kPoolItem / 4];
-#pragma unroll
-    for (int w = 0; w < kPoolItem / 4; ++w)
-      packed[w] = (static_cast<uint32_t>(q[4 * w]) & 0xffu) |
-                  ((static_cast<uint32_t>(q[4 * w + 1]) & 0xffu) << 8) |
-                  ((static_cast<uint32_t>(q[4 * w + 2]) & 0xffu) << 16) |
-                  (static_cast<uint32_t>(q[4 * w + 3]) << 24);
     if (nout == kPoolItem && ((reinterpret_cast<uintptr_t>(a.out) + off) & 3u) == 0) {
 #pragma unroll
       for (int w = 0; w < kPoolItem / 4; ++w)
@@ -295,7 +372,7 @@ __global__ __launch_bounds__(kPoolThreads) void pool_lds_kernel(PoolArgs a) {
     } else {
 #pragma unroll
       for (int i = 0; i < kPoolItem; ++i)
-        if (i < nout) a.out[off + i] = static_cast<uint8_t>(q[i]);
+        if (i < nout) a.out[off + i] = static_cast<uint8_t>(packed[i / 4] >> (8 * (i % 4)));
     }
   }
 }
@@ -400,6 +477,21 @@ int mxq_quantized_pooling_nchw(void* stream, const void* in, int in_type, int N,
     const long long spread = (planes + 4LL * cus - 1) / (4LL * cus);
     if (ppb > spread) ppb = spread;
     if (ppb < 1) ppb = 1;
+    // a group's work items (one per output row for full-width average windows, else one
+    // per kPoolItem outputs) should fill whole passes of its threads: 668 planes of one
+    // item each would leave the third pass of 256 threads 39 % full
+    const bool full_width = a.is_avg && OW == 1 && pad_w == 0 && kernel_w == W;
+    const long long units =
+        full_width ? OH : static_cast<long long>((OW + kPoolItem - 1) / kPoolItem) * OH;
+    auto fill = [&](long long planes_per_group) {
+      const long long items = planes_per_group * units;
+      return static_cast<double>(items) /
+             static_cast<double>((items + kPoolThreads - 1) / kPoolThreads * kPoolThreads);
+    };
+    long long best = ppb;
+    for (long long c = ppb - 1; c >= 1 && 2 * c >= ppb; --c)
+      if (fill(c) > fill(best) + 0.03) best = c;
+    ppb = best;
     a.ppb = static_cast<int>(ppb);
     a.band = OH;
     a.bands = 1;
