@@ -181,10 +181,14 @@ __device__ __forceinline__ void pool_strip_max2(const uint8_t* lds, int base, in
   // 0x00204081 lands on bit 8k without carries).
   const int first = max(-w0, 0), last = max(min(a.W - w0, SPAN), first);
   const uint32_t valid = __builtin_amdgcn_ubfe(0xffffffffu, 0, last - first) << first;
-  uint32_t keep[NW];
+  uint32_t keep_even[NW], keep_odd[NW];
 #pragma unroll
-  for (int w = 0; w < NW; ++w)
-    keep[w] = ((((valid >> (4 * w)) & 0xfu) * 0x00204081u) & 0x01010101u) * 0xffu;
+  for (int w = 0; w < NW; ++w) {
+    // (24-bit multiplies run at full rate: every operand here stays below 2^24)
+    const uint32_t bits = __umul24((valid >> (4 * w)) & 0xfu, 0x00204081u);
+    keep_even[w] = __umul24(bits & 0x00010001u, 0xffu);
+    keep_odd[w] = __umul24((bits >> 8) & 0x00010001u, 0xff00u);
+  }
   uint32_t even[NW], odd[NW];  // bytes 0,2 in the low byte / bytes 1,3 in the high byte of a lane
 #pragma unroll
   for (int w = 0; w < NW; ++w) even[w] = odd[w] = 0u;
@@ -194,7 +198,7 @@ __device__ __forceinline__ void pool_strip_max2(const uint8_t* lds, int base, in
 #pragma unroll
   for (int r = 0; r < K; ++r) {
     const int hh = min(max(h0 + r, row0), row1 - 1);
-    const int off = base + (hh - row0) * a.W + w0;
+    const int off = base + __mul24(hh - row0, a.W) + w0;  // staged: < 2^24
     const int wi = off >> 2;
     const uint32_t sft = static_cast<uint32_t>(off & 3);
     uint32_t d[NW + 1];
@@ -203,9 +207,9 @@ __device__ __forceinline__ void pool_strip_max2(const uint8_t* lds, int base, in
     d[NW] = 0u;
 #pragma unroll
     for (int w = 0; w < NW; ++w) {
-      const uint32_t x = (__builtin_amdgcn_alignbyte(d[w + 1], d[w], sft) ^ bias) & keep[w];
-      even[w] = pk_max_u16(even[w], x & 0x00ff00ffu);
-      odd[w] = pk_max_u16(odd[w], x & 0xff00ff00u);
+      const uint32_t x = __builtin_amdgcn_alignbyte(d[w + 1], d[w], sft) ^ bias;
+      even[w] = pk_max_u16(even[w], x & keep_even[w]);
+      odd[w] = pk_max_u16(odd[w], x & keep_odd[w]);
     }
   }
   // lanes of `even`: bytes 4w, 4w+2; of `odd` (after the shift): bytes 4w+1, 4w+3.
