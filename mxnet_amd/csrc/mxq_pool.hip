@@ -32,6 +32,10 @@ struct PoolArgs {
   int bands;  // bands per plane
   int vec_ok; // the tensor base is 16-byte aligned
   // floor(n / d) = umulhi(n, magic) for n * d < 2^32 (magic = 2^32 / d + 1; 0 stands for d = 1)
+  const float* imin;  // the range passes through: written by the first thread of the grid
+  const float* imax;
+  float* omin;
+  float* omax;
   uint32_t magic_per_row;    // d = items per output row
   uint32_t magic_per_plane;  // d = items per plane, used when ppb > 1
 };
@@ -259,6 +263,10 @@ __global__ __launch_bounds__(kPoolThreads) void pool_lds_kernel(PoolArgs a) {
   __shared__ __attribute__((aligned(16))) uint8_t lds_raw[kPoolLdsBytes + 96];
   uint8_t* lds = lds_raw + 16;
   const int tid = threadIdx.x;
+  if (blockIdx.x == 0 && tid == 0) {
+    *a.omin = *a.imin;
+    *a.omax = *a.imax;
+  }
   int p0, np, oh0, oh1;
   if (a.ppb > 1) {
     p0 = blockIdx.x * a.ppb;
@@ -384,6 +392,10 @@ __global__ __launch_bounds__(kPoolThreads) void pool_lds_kernel(PoolArgs a) {
 // Fallback for images whose single window band does not fit the LDS budget.
 template <bool UNSIGNED>
 __global__ __launch_bounds__(kPoolThreads) void pool_direct_kernel(PoolArgs a) {
+  if (blockIdx.x == 0 && threadIdx.x == 0) {
+    *a.omin = *a.imin;
+    *a.omax = *a.imax;
+  }
   const size_t total = static_cast<size_t>(a.planes) * a.OH * a.OW;
   for (size_t o = static_cast<size_t>(blockIdx.x) * kPoolThreads + threadIdx.x; o < total;
        o += static_cast<size_t>(gridDim.x) * kPoolThreads) {
@@ -452,10 +464,12 @@ int mxq_quantized_pooling_nchw(void* stream, const void* in, int in_type, int N,
             "kernel size exceeds the padded input");
   MXQ_CHECK(imin && imax && omin && omax, "null range pointer");
   hipStream_t s = static_cast<hipStream_t>(stream);
-  hipLaunchKernelGGL(copy_range_kernel, dim3(1), dim3(1), 0, s, imin, imax, omin, omax);
-  MXQ_LAUNCH_CHECK();
   const long long planes = static_cast<long long>(N) * C;
-  if (planes == 0) return 0;
+  if (planes == 0 || static_cast<long long>(OH) * OW == 0) {
+    hipLaunchKernelGGL(copy_range_kernel, dim3(1), dim3(1), 0, s, imin, imax, omin, omax);
+    MXQ_LAUNCH_CHECK();
+    return 0;
+  }
   MXQ_CHECK(in != nullptr && out != nullptr, "null data pointer");
   MXQ_CHECK(planes < (1LL << 31) && static_cast<long long>(OH) * OW < (1LL << 31) &&
                 static_cast<long long>(H) * W < (1LL << 31),
@@ -463,6 +477,7 @@ int mxq_quantized_pooling_nchw(void* stream, const void* in, int in_type, int N,
   PoolArgs a;
   a.in = static_cast<const uint8_t*>(in);
   a.out = static_cast<uint8_t*>(out);
+  a.imin = imin; a.imax = imax; a.omin = omin; a.omax = omax;
   a.total_in = static_cast<size_t>(planes) * H * W;
   a.planes = static_cast<int>(planes);
   a.H = H; a.W = W; a.OH = OH; a.OW = OW; a.KH = kernel_h; a.KW = kernel_w;
