@@ -416,9 +416,15 @@ __global__ void copy_range_kernel(const float* imin, const float* imax, float* o
 // Flat byte copy, 16 bytes per lane where both pointers allow it.
 __global__ __launch_bounds__(256) void copy_bytes_kernel(const uint8_t* __restrict__ in,
                                                          uint8_t* __restrict__ out, size_t n,
-                                                         int vec_ok) {
+                                                         int vec_ok, const float* imin,
+                                                         const float* imax, float* omin,
+                                                         float* omax) {
   const size_t stride = static_cast<size_t>(gridDim.x) * 256;
   const size_t t = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
+  if (t == 0 && omin != nullptr) {  // the range goes with the data (null: it is in place)
+    *omin = *imin;
+    *omax = *imax;
+  }
   if (vec_ok) {
     const size_t nv = n / 16;
     for (size_t i = t; i < nv; i += stride)
@@ -603,10 +609,7 @@ int mxq_quantized_flatten(void* stream, const void* in, const float* imin, const
   MXQ_CHECK(imin && imax && omin && omax, "null range pointer");
   MXQ_CHECK(n_bytes == 0 || (in != nullptr && out != nullptr), "null data pointer");
   hipStream_t s = static_cast<hipStream_t>(stream);
-  if (omin != imin || omax != imax) {
-    hipLaunchKernelGGL(copy_range_kernel, dim3(1), dim3(1), 0, s, imin, imax, omin, omax);
-    MXQ_LAUNCH_CHECK();
-  }
+  const bool range_moves = omin != imin || omax != imax;
   if (n_bytes != 0 && in != out) {
     const int vec_ok = aligned16(in) && aligned16(out);
     size_t g = (n_bytes / (vec_ok ? 16 : 1) + 255) / 256;
@@ -615,7 +618,10 @@ int mxq_quantized_flatten(void* stream, const void* in, const float* imin, const
     if (g < 1) g = 1;
     hipLaunchKernelGGL(copy_bytes_kernel, dim3(static_cast<unsigned>(g)), dim3(256), 0, s,
                        static_cast<const uint8_t*>(in), static_cast<uint8_t*>(out), n_bytes,
-                       vec_ok);
+                       vec_ok, imin, imax, range_moves ? omin : nullptr, omax);
+    MXQ_LAUNCH_CHECK();
+  } else if (range_moves) {
+    hipLaunchKernelGGL(copy_range_kernel, dim3(1), dim3(1), 0, s, imin, imax, omin, omax);
     MXQ_LAUNCH_CHECK();
   }
   MXQ_API_END();
