@@ -65,7 +65,7 @@ def parse_args():
 
 
 class FcWorkload:
-    """BASELINE config 3: data quantized from U(-1,1) with calib (-1,1), weight from
+    """Benchmark configuration 3: data quantized from U(-1,1) with calib (-1,1), weight from
     N(0,0.02) with its own min/max, int8 bias, fused requantize with a calibrated range."""
 
     def __init__(self, S, torch, capi, lib):
@@ -136,7 +136,7 @@ class FcWorkload:
 
 
 class CastWorkload:
-    """BASELINE config 2: 64M-element flat tensors, buffers rotated so that the
+    """Benchmark configuration 2: 64M-element flat tensors, buffers rotated so that the
     256 MB Infinity Cache cannot serve the reads."""
     N = 1 << 26
     NBUF = 3
@@ -446,7 +446,7 @@ RESNET50_CONVS = [(56, 64, 64, 1, 1), (56, 64, 64, 3, 1), (56, 64, 256, 1, 1), (
 
 
 class ConvStackWorkload(GraphWorkload):
-    """BASELINE config 4: the distinct 1x1 / 3x3 bottleneck convolutions of ResNet-50 v1 at
+    """Benchmark configuration 4: the distinct 1x1 / 3x3 bottleneck convolutions of ResNet-50 v1 at
     batch 64 on NHWC int8, weights N(0, sqrt(2/fan_in)) quantized with their own min/max, each
     with the quantized ReLU and a calibrated requantize fused in the epilogue."""
 
@@ -510,7 +510,7 @@ BERT_FCS = [(768, 2304), (768, 768), (768, 3072), (3072, 768)]
 
 
 class BertChainWorkload(GraphWorkload):
-    """BASELINE config 5: BERT-base FC shapes at M = 32 x 128 = 4096; per layer calibrated
+    """Benchmark configuration 5: BERT-base FC shapes at M = 32 x 128 = 4096; per layer calibrated
     quantize_v2 -> quantized_fully_connected (+ int8 bias) -> requantize -> dequantize, as
     the unfused graph runs it.  Activations N(0,1) with 0.1% outliers at +-20."""
 
@@ -696,7 +696,7 @@ def main():
     args = parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (the operators "
-              "shard trivially, see DESIGN.md); run with --gpus 1", file=sys.stderr)
+              "shard without any exchange but one 8-byte min/max all-reduce); run with --gpus 1", file=sys.stderr)
         sys.exit(2)
     import torch
     if not torch.cuda.is_available():
