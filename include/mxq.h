@@ -194,6 +194,11 @@ int mxq_quantized_conv_nhwc(void* stream, const int8_t* data, const int8_t* weig
 
 /* [N,C,H,W] int8 -> [N,H,W,C] int8 (also OIHW -> OHWI for the weight). */
 int mxq_nchw_to_nhwc_i8(void* stream, const int8_t* in, int8_t* out, int N, int C, int H, int W);
+/* The same with the channel extent of the output padded to C_padded >= C with zeros
+ * ([N,H,W,C_padded]): zero channels add nothing to a convolution, and a channel count
+ * that is a multiple of 16 takes mxq_quantized_conv_nhwc's fast path. */
+int mxq_nchw_to_nhwc_pad_i8(void* stream, const int8_t* in, int8_t* out, int N, int C, int H,
+                            int W, int C_padded);
 /* [N,H,W,C] -> [N,C,H,W]; elem_bytes 1 (int8) or 4 (int32). */
 int mxq_nhwc_to_nchw(void* stream, const void* in, void* out, int N, int C, int H, int W,
                      int elem_bytes);

@@ -263,35 +263,38 @@ int num_cus() {
 }
 
 // ---- layout adapters ------------------------------------------------------------
-// Batched transpose [B][R][S] -> [B][S][R] through a padded LDS tile; reads are
-// contiguous along S, writes contiguous along R.
+// Batched transpose [B][R][S] -> [B][S][RP] through a padded LDS tile; reads are
+// contiguous along S, writes contiguous along R.  RP >= R: positions R..RP-1 of every
+// output row are written as zeros (channel padding).
 template <typename T>
 __global__ __launch_bounds__(256) void transpose_kernel(const T* __restrict__ in,
-                                                        T* __restrict__ out, int R, int S) {
+                                                        T* __restrict__ out, int R, int S,
+                                                        int RP) {
   __shared__ T tile[64][65];
   const size_t b = blockIdx.z;
   const int r0 = blockIdx.y * 64, s0 = blockIdx.x * 64;
   const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
   const T* src = in + b * static_cast<size_t>(R) * S;
-  T* dst = out + b * static_cast<size_t>(R) * S;
+  T* dst = out + b * static_cast<size_t>(RP) * S;
   for (int i = ty; i < 64; i += 4) {
     const int r = r0 + i, s = s0 + tx;
-    if (r < R && s < S) tile[i][tx] = src[static_cast<size_t>(r) * S + s];
+    tile[i][tx] = (r < R && s < S) ? src[static_cast<size_t>(r) * S + s] : T(0);
   }
   __syncthreads();
   for (int i = ty; i < 64; i += 4) {
     const int s = s0 + i, r = r0 + tx;
-    if (r < R && s < S) dst[static_cast<size_t>(s) * R + r] = tile[tx][i];
+    if (r < RP && s < S) dst[static_cast<size_t>(s) * RP + r] = tile[tx][i];
   }
 }
 
 template <typename T>
-void launch_transpose(hipStream_t s, const void* in, void* out, int B, int R, int S) {
-  if (B == 0 || R == 0 || S == 0) return;
-  MXQ_CHECK(B <= 65535 && (R + 63) / 64 <= 65535, "transpose grid too large");
-  dim3 grid((S + 63) / 64, (R + 63) / 64, B);
+void launch_transpose(hipStream_t s, const void* in, void* out, int B, int R, int S, int RP) {
+  if (B == 0 || RP == 0 || S == 0) return;
+  MXQ_CHECK(RP >= R, "padded extent below the extent");
+  MXQ_CHECK(B <= 65535 && (RP + 63) / 64 <= 65535, "transpose grid too large");
+  dim3 grid((S + 63) / 64, (RP + 63) / 64, B);
   hipLaunchKernelGGL((transpose_kernel<T>), grid, dim3(256), 0, s, static_cast<const T*>(in),
-                     static_cast<T*>(out), R, S);
+                     static_cast<T*>(out), R, S, RP);
   MXQ_LAUNCH_CHECK();
 }
 
@@ -415,7 +418,19 @@ int mxq_nchw_to_nhwc_i8(void* stream, const int8_t* in, int8_t* out, int N, int 
   MXQ_CHECK((static_cast<long long>(H) * W) < (1LL << 31), "image too large");
   if (static_cast<long long>(N) * C * H * W == 0) return 0;
   MXQ_CHECK(in != nullptr && out != nullptr, "null pointer");
-  launch_transpose<int8_t>(static_cast<hipStream_t>(stream), in, out, N, C, H * W);
+  launch_transpose<int8_t>(static_cast<hipStream_t>(stream), in, out, N, C, H * W, C);
+  MXQ_API_END();
+}
+
+int mxq_nchw_to_nhwc_pad_i8(void* stream, const int8_t* in, int8_t* out, int N, int C, int H,
+                            int W, int C_padded) {
+  MXQ_API_BEGIN();
+  MXQ_CHECK(N >= 0 && C >= 0 && H >= 0 && W >= 0, "negative dimension");
+  MXQ_CHECK(C_padded >= C, "C_padded must be at least C");
+  MXQ_CHECK((static_cast<long long>(H) * W) < (1LL << 31), "image too large");
+  if (static_cast<long long>(N) * C_padded * H * W == 0) return 0;
+  MXQ_CHECK(in != nullptr && out != nullptr, "null pointer");
+  launch_transpose<int8_t>(static_cast<hipStream_t>(stream), in, out, N, C, H * W, C_padded);
   MXQ_API_END();
 }
 
@@ -429,9 +444,9 @@ int mxq_nhwc_to_nchw(void* stream, const void* in, void* out, int N, int C, int 
   MXQ_CHECK(in != nullptr && out != nullptr, "null pointer");
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (elem_bytes == 1)
-    launch_transpose<int8_t>(s, in, out, N, H * W, C);
+    launch_transpose<int8_t>(s, in, out, N, H * W, C, H * W);
   else
-    launch_transpose<int32_t>(s, in, out, N, H * W, C);
+    launch_transpose<int32_t>(s, in, out, N, H * W, C, H * W);
   MXQ_API_END();
 }
 

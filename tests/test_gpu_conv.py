@@ -127,6 +127,24 @@ def test_layout_adapters(capi):
                                           dtype=np.int32)
     z = capi.nhwc_to_nchw(dev(v))
     np.testing.assert_array_equal(z.cpu().numpy(), v.transpose(0, 3, 1, 2))
+    # channel padding: zeros behind the C real channels of every pixel
+    import ctypes
+    import mxnet_amd
+    for shape, cp in (((3, 5, 7, 9), 16), ((2, 3, 70, 33), 16), ((1, 70, 5, 5), 80),
+                      ((2, 16, 4, 4), 16)):
+        x = int8_uniform(shape, seed=3)
+        n, c, h, w = shape
+        out = torch.full((n, h, w, cp), 77, dtype=torch.int8, device="cuda")
+        st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+        rc = mxnet_amd._lib.lib.mxq_nchw_to_nhwc_pad_i8(st, ctypes.c_void_p(dev(x).data_ptr()),
+                                                        ctypes.c_void_p(out.data_ptr()), n, c, h,
+                                                        w, cp)
+        assert rc == 0
+        want = np.zeros((n, h, w, cp), np.int8)
+        want[..., :c] = x.transpose(0, 2, 3, 1)
+        np.testing.assert_array_equal(out.cpu().numpy(), want)
+    rc = mxnet_amd._lib.lib.mxq_nchw_to_nhwc_pad_i8(st, None, None, 1, 8, 2, 2, 4)
+    assert rc == -1 and b"C_padded" in mxnet_amd._lib.lib.mxq_last_error()
 
 
 def test_conv_1x1_equals_fc(capi):

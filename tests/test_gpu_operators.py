@@ -210,6 +210,28 @@ def test_quantized_conv(contrib, use_bias):
     assert (mn.item(), mx.item()) == (rmn, rmx)
 
 
+@pytest.mark.parametrize("shape,filters,kernel,stride,pad", [
+    ((2, 3, 64, 64), 64, (7, 7), (2, 2), (3, 3)),     # a 3-channel stem: channels padded to 16
+    ((2, 20, 9, 11), 36, (5, 3), (1, 1), (2, 1)),     # 20 channels padded to 32
+    ((1, 17, 8, 8), 8, (1, 1), (1, 1), (0, 0)),
+])
+def test_quantized_conv_channel_counts_off_16(contrib, shape, filters, kernel, stride, pad):
+    """The operator pads the channels with zeros while it brings NCHW to NHWC; the result
+    is that of the unpadded convolution."""
+    rng = np.random.default_rng(71)
+    data = rng.integers(-127, 128, shape).astype(np.int8)
+    weight = rng.integers(-127, 128, (filters, shape[1]) + kernel).astype(np.int8)
+    bias = rng.integers(-127, 128, (filters,)).astype(np.int8)
+    out, mn, mx = contrib.quantized_conv(dev(data), dev(weight), dev(bias), scalar(-1.0),
+                                         scalar(1.0), scalar(-0.5), scalar(0.5), scalar(-2.0),
+                                         scalar(2.0), kernel=kernel, stride=stride, pad=pad,
+                                         num_filter=filters, no_bias=False)
+    ro, rmn, rmx = oracle.quantized_conv(data, weight, bias, -1.0, 1.0, -0.5, 0.5, -2.0, 2.0,
+                                         stride, pad, (1, 1))
+    np.testing.assert_array_equal(out.cpu().numpy(), ro)
+    assert (mn.item(), mx.item()) == (rmn, rmx)
+
+
 def test_quantized_act(contrib):
     q = np.random.default_rng(8).integers(-128, 128, size=(5, 1000), dtype=np.int8)
     out, mn, mx = contrib.quantized_act(dev(q), scalar(-2.5), scalar(2.5), act_type="relu")
