@@ -191,6 +191,17 @@ int mxq_quantized_conv_nhwc(void* stream, const int8_t* data, const int8_t* weig
                             const float* max_bias, int32_t* out32, float* omin, float* omax,
                             int8_t* out8, float* rmin, float* rmax, int relu, float min_calib,
                             float max_calib);
+/* The same convolution with the int32 output written as the operator's own layout,
+ * [N,O,OH,OW]: the kernel's epilogue stores channel planes directly, which replaces the
+ * third TransposeImpl (quantized_conv.cu:183) and the NHWC int32 buffer it reads. */
+int mxq_quantized_conv_nhwc_out_nchw(void* stream, const int8_t* data, const int8_t* weight,
+                                     const int8_t* bias, int N, int H, int W, int C, int O,
+                                     int KH, int KW, int stride_h, int stride_w, int pad_h,
+                                     int pad_w, int dilate_h, int dilate_w,
+                                     const float* min_data, const float* max_data,
+                                     const float* min_weight, const float* max_weight,
+                                     const float* min_bias, const float* max_bias,
+                                     int32_t* out32_nchw, float* omin, float* omax);
 
 /* [N,C,H,W] int8 -> [N,H,W,C] int8 (also OIHW -> OHWI for the weight). */
 int mxq_nchw_to_nhwc_i8(void* stream, const int8_t* in, int8_t* out, int N, int C, int H, int W);

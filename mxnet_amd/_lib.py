@@ -48,6 +48,8 @@ SIGNATURES = {
                               _i, _f, _f]),
     "mxq_quantized_conv_nhwc": (_i, [_p, _p, _p, _p] + [_i] * 13 + [_p] * 6 +
                                 [_p, _p, _p, _p, _p, _p, _i, _f, _f]),
+    "mxq_quantized_conv_nhwc_out_nchw": (_i, [_p, _p, _p, _p] + [_i] * 13 + [_p] * 6 +
+                                         [_p, _p, _p]),
     "mxq_nchw_to_nhwc_i8": (_i, [_p, _p, _p, _i, _i, _i, _i]),
     "mxq_nchw_to_nhwc_pad_i8": (_i, [_p, _p, _p, _i, _i, _i, _i, _i]),
     "mxq_nhwc_to_nchw": (_i, [_p, _p, _p, _i, _i, _i, _i, _i]),

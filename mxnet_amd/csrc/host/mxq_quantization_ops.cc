@@ -644,7 +644,8 @@ static size_t QuantizedConvTempBytes(const TShape& d, const TShape& w, const TSh
   const size_t scale_num = static_cast<size_t>(ConvPaddedChannels(static_cast<int>(C)));
   const size_t d_bytes = C == 0 ? 0 : d.Size() / C * scale_num;
   const size_t w_bytes = C == 0 ? 0 : w.Size() / C * scale_num;
-  return up(d_bytes) + up(w_bytes) + up(o.Size() * sizeof(int32_t));
+  (void)o;  // the output is written in its own layout: no third buffer
+  return up(d_bytes) + up(w_bytes);
 }
 
 // QuantizedConvForwardGPU, quantized_conv.cu:268-291
@@ -665,26 +666,21 @@ static void QuantizedConvForwardGPU(const NodeAttrs& attrs, const OpContext& ctx
   const int N = d[0], C = d[1], H = d[2], W = d[3], O = w[0], KH = w[2], KW = w[3];
   const int CP = ConvPaddedChannels(C);
   const size_t d_bytes = static_cast<size_t>(N) * H * W * CP;
-  const size_t w_bytes = static_cast<size_t>(O) * KH * KW * CP;
   int8_t* d_nhwc = reinterpret_cast<int8_t*>(ws);
   int8_t* w_ohwi = reinterpret_cast<int8_t*>(ws + up(d_bytes));
-  int32_t* o_nhwc = reinterpret_cast<int32_t*>(ws + up(d_bytes) + up(w_bytes));
   void* stream = raw_stream(ctx);
   MXQ_CALL(mxq_nchw_to_nhwc_pad_i8(stream, inputs[0].dptr<int8_t>(), d_nhwc, N, C, H, W, CP));
   MXQ_CALL(mxq_nchw_to_nhwc_pad_i8(stream, inputs[1].dptr<int8_t>(), w_ohwi, O, C, KH, KW, CP));
   const size_t ni = param.no_bias ? 2 : 3;
-  MXQ_CALL(mxq_quantized_conv_nhwc(
+  MXQ_CALL(mxq_quantized_conv_nhwc_out_nchw(
       stream, d_nhwc, w_ohwi, param.no_bias ? nullptr : inputs[2].dptr<int8_t>(), N, H, W, CP, O,
       KH, KW, static_cast<int>(param.stride[0]), static_cast<int>(param.stride[1]),
       static_cast<int>(param.pad[0]), static_cast<int>(param.pad[1]),
       static_cast<int>(param.dilate[0]), static_cast<int>(param.dilate[1]),
       inputs[ni].dptr<float>(), inputs[ni + 1].dptr<float>(), inputs[ni + 2].dptr<float>(),
       inputs[ni + 3].dptr<float>(), param.no_bias ? nullptr : inputs[7].dptr<float>(),
-      param.no_bias ? nullptr : inputs[8].dptr<float>(), o_nhwc, outputs[1].dptr<float>(),
-      outputs[2].dptr<float>(), nullptr, nullptr, nullptr, 0, 0.f, 0.f));
-  MXQ_CALL(mxq_nhwc_to_nchw(stream, o_nhwc, outputs[0].dptr<int32_t>(), static_cast<int>(o[0]),
-                            static_cast<int>(o[1]), static_cast<int>(o[2]),
-                            static_cast<int>(o[3]), 4));
+      param.no_bias ? nullptr : inputs[8].dptr<float>(), outputs[0].dptr<int32_t>(),
+      outputs[1].dptr<float>(), outputs[2].dptr<float>()));
 }
 
 // _contrib_quantized_act: int8 relu, ranges pass through (dnnl_quantized_act.cc:33-45)

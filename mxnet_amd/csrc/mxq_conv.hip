@@ -287,34 +287,87 @@ __global__ __launch_bounds__(256) void transpose_kernel(const T* __restrict__ in
   }
 }
 
+// The byte form of the same transpose for friendly shapes (S % 4 == 0, RP % 16 == 0,
+// aligned pointers): a work-group takes 64 rows x 128 columns, every thread loads dwords
+// along S (a wave reads whole 128-byte runs), transposes 4 x 4 bytes in registers with
+// v_perm and parks the result in LDS, from where 16-byte pieces of the output rows leave
+// (a wave writes 1 KiB contiguous when the group covers all RP positions of its rows).
+__global__ __launch_bounds__(256) void transpose_i8_kernel(const uint8_t* __restrict__ in,
+                                                           uint8_t* __restrict__ out, int R,
+                                                           int S, int RP) {
+  constexpr int kPitch = 17;  // dwords per transposed row: 64 bytes + 4 of padding
+  __shared__ uint32_t tile[128 * kPitch];
+  const size_t b = blockIdx.z;
+  const int r0 = blockIdx.y * 64, s0 = blockIdx.x * 128;
+  const int t = threadIdx.x;
+  const uint8_t* src = in + b * static_cast<size_t>(R) * S;
+  uint8_t* dst = out + b * static_cast<size_t>(RP) * S;
+  const int sq = t & 31;
+#pragma unroll
+  for (int pass = 0; pass < 2; ++pass) {
+    const int rq = (t >> 5) + 8 * pass;
+    const int s = s0 + 4 * sq;
+    uint32_t w[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int r = r0 + 4 * rq + j;
+      w[j] = (r < R && s < S)
+                 ? *reinterpret_cast<const uint32_t*>(src + static_cast<size_t>(r) * S + s)
+                 : 0u;
+    }
+    // x[i] = byte i of w[0..3]
+    const uint32_t t0 = __builtin_amdgcn_perm(w[1], w[0], 0x05010400u);
+    const uint32_t t1 = __builtin_amdgcn_perm(w[1], w[0], 0x07030602u);
+    const uint32_t t2 = __builtin_amdgcn_perm(w[3], w[2], 0x05010400u);
+    const uint32_t t3 = __builtin_amdgcn_perm(w[3], w[2], 0x07030602u);
+    tile[(4 * sq + 0) * kPitch + rq] = __builtin_amdgcn_perm(t2, t0, 0x05040100u);
+    tile[(4 * sq + 1) * kPitch + rq] = __builtin_amdgcn_perm(t2, t0, 0x07060302u);
+    tile[(4 * sq + 2) * kPitch + rq] = __builtin_amdgcn_perm(t3, t1, 0x05040100u);
+    tile[(4 * sq + 3) * kPitch + rq] = __builtin_amdgcn_perm(t3, t1, 0x07060302u);
+  }
+  __syncthreads();
+  const int nb = min(64, RP - r0);  // bytes of every output row this group owns (16 | nb)
+  const int per_row = nb >> 4;      // 16-byte pieces per row: 1..4
+  const int pieces = 128 * per_row;
+  for (int c = t; c < pieces; c += 256) {
+    const int sl = per_row == 4 ? (c >> 2) : (per_row == 2 ? (c >> 1) : (per_row == 1 ? c : c / 3));
+    const int k = c - sl * per_row;
+    if (s0 + sl >= S) continue;
+    typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+    u4 v;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) v[i] = tile[sl * kPitch + 4 * k + i];
+    *reinterpret_cast<u4*>(dst + static_cast<size_t>(s0 + sl) * RP + r0 + 16 * k) = v;
+  }
+}
+
 template <typename T>
 void launch_transpose(hipStream_t s, const void* in, void* out, int B, int R, int S, int RP) {
   if (B == 0 || RP == 0 || S == 0) return;
   MXQ_CHECK(RP >= R, "padded extent below the extent");
   MXQ_CHECK(B <= 65535 && (RP + 63) / 64 <= 65535, "transpose grid too large");
+  if (sizeof(T) == 1 && S % 4 == 0 && RP % 16 == 0 &&
+      (reinterpret_cast<uintptr_t>(in) & 3u) == 0 && aligned16(out)) {
+    dim3 grid128((S + 127) / 128, (RP + 63) / 64, B);
+    hipLaunchKernelGGL(transpose_i8_kernel, grid128, dim3(256), 0, s,
+                       static_cast<const uint8_t*>(in), static_cast<uint8_t*>(out), R, S, RP);
+    MXQ_LAUNCH_CHECK();
+    return;
+  }
   dim3 grid((S + 63) / 64, (RP + 63) / 64, B);
   hipLaunchKernelGGL((transpose_kernel<T>), grid, dim3(256), 0, s, static_cast<const T*>(in),
                      static_cast<T*>(out), R, S, RP);
   MXQ_LAUNCH_CHECK();
 }
 
-}  // namespace
-}  // namespace mxq
-
-using namespace mxq;
-
-extern "C" {
-
-int mxq_quantized_conv_nhwc(void* stream, const int8_t* data, const int8_t* weight,
-                            const int8_t* bias, int N, int H, int W, int C, int O, int KH,
-                            int KW, int stride_h, int stride_w, int pad_h, int pad_w,
-                            int dilate_h, int dilate_w, const float* min_data,
-                            const float* max_data, const float* min_weight,
-                            const float* max_weight, const float* min_bias,
-                            const float* max_bias, int32_t* out32, float* omin, float* omax,
-                            int8_t* out8, float* rmin, float* rmax, int relu, float min_calib,
-                            float max_calib) {
-  MXQ_API_BEGIN();
+// Both C entry points: `planar` writes out32 as [N][O][OH][OW] instead of [N][OH][OW][O].
+void conv_nhwc(void* stream, const int8_t* data, const int8_t* weight, const int8_t* bias, int N,
+               int H, int W, int C, int O, int KH, int KW, int stride_h, int stride_w, int pad_h,
+               int pad_w, int dilate_h, int dilate_w, const float* min_data,
+               const float* max_data, const float* min_weight, const float* max_weight,
+               const float* min_bias, const float* max_bias, int32_t* out32, float* omin,
+               float* omax, int8_t* out8, float* rmin, float* rmax, int relu, float min_calib,
+               float max_calib, bool planar) {
   MXQ_CHECK(N >= 0 && H > 0 && W > 0 && C > 0 && O > 0 && KH > 0 && KW > 0, "bad shape");
   MXQ_CHECK(stride_h > 0 && stride_w > 0 && dilate_h > 0 && dilate_w > 0 && pad_h >= 0 &&
                 pad_w >= 0,
@@ -338,7 +391,7 @@ int mxq_quantized_conv_nhwc(void* stream, const int8_t* data, const int8_t* weig
   MXQ_CHECK(M < (1LL << 31) && K < (1LL << 31), "problem too large for 32-bit tile indices");
   a.M = static_cast<int>(M);
   a.K = static_cast<int>(K);
-  if (a.M == 0) return 0;
+  if (a.M == 0) return;
   MXQ_CHECK(data != nullptr && weight != nullptr, "null operand pointer");
   Epilogue& e = a.epi;
   e.bias = bias;
@@ -350,6 +403,7 @@ int mxq_quantized_conv_nhwc(void* stream, const int8_t* data, const int8_t* weig
   e.relu = relu;
   float x = fabsf(min_calib), y = fabsf(max_calib);
   e.real_range = (x < y) ? y : x;
+  e.plane = planar ? a.OH * a.OW : 0;
 
   hipStream_t s = static_cast<hipStream_t>(stream);
   const bool aligned = (C % 16 == 0) && aligned16(data) && aligned16(weight);
@@ -361,7 +415,7 @@ int mxq_quantized_conv_nhwc(void* stream, const int8_t* data, const int8_t* weig
   if (cfg == 0 && KH == 1 && KW == 1 && stride_h == 1 && stride_w == 1 && pad_h == 0 &&
       pad_w == 0) {
     launch_fc(s, data, weight, a.M, O, C, O, e);
-    return 0;
+    return;
   }
   if (cfg == 0) {
     const long cus = num_cus();
@@ -408,8 +462,47 @@ int mxq_quantized_conv_nhwc(void* stream, const int8_t* data, const int8_t* weig
     case 25: launch_dma<CfgS, 2, 0>(s, a); break;
     default: MXQ_CHECK(false, "unknown conv tile configuration " << cfg);
   }
+}
+
+}  // namespace
+}  // namespace mxq
+
+using namespace mxq;
+
+extern "C" {
+
+int mxq_quantized_conv_nhwc(void* stream, const int8_t* data, const int8_t* weight,
+                            const int8_t* bias, int N, int H, int W, int C, int O, int KH,
+                            int KW, int stride_h, int stride_w, int pad_h, int pad_w,
+                            int dilate_h, int dilate_w, const float* min_data,
+                            const float* max_data, const float* min_weight,
+                            const float* max_weight, const float* min_bias,
+                            const float* max_bias, int32_t* out32, float* omin, float* omax,
+                            int8_t* out8, float* rmin, float* rmax, int relu, float min_calib,
+                            float max_calib) {
+  MXQ_API_BEGIN();
+  conv_nhwc(stream, data, weight, bias, N, H, W, C, O, KH, KW, stride_h, stride_w, pad_h, pad_w,
+            dilate_h, dilate_w, min_data, max_data, min_weight, max_weight, min_bias, max_bias,
+            out32, omin, omax, out8, rmin, rmax, relu, min_calib, max_calib, false);
   MXQ_API_END();
 }
+
+int mxq_quantized_conv_nhwc_out_nchw(void* stream, const int8_t* data, const int8_t* weight,
+                                     const int8_t* bias, int N, int H, int W, int C, int O,
+                                     int KH, int KW, int stride_h, int stride_w, int pad_h,
+                                     int pad_w, int dilate_h, int dilate_w,
+                                     const float* min_data, const float* max_data,
+                                     const float* min_weight, const float* max_weight,
+                                     const float* min_bias, const float* max_bias,
+                                     int32_t* out32_nchw, float* omin, float* omax) {
+  MXQ_API_BEGIN();
+  MXQ_CHECK(out32_nchw != nullptr, "no output buffer");
+  conv_nhwc(stream, data, weight, bias, N, H, W, C, O, KH, KW, stride_h, stride_w, pad_h, pad_w,
+            dilate_h, dilate_w, min_data, max_data, min_weight, max_weight, min_bias, max_bias,
+            out32_nchw, omin, omax, nullptr, nullptr, nullptr, 0, 0.f, 0.f, true);
+  MXQ_API_END();
+}
+
 
 int mxq_nchw_to_nhwc_i8(void* stream, const int8_t* in, int8_t* out, int N, int C, int H,
                         int W) {

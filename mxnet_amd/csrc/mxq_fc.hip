@@ -236,6 +236,7 @@ extern "C" int mxq_quantized_fc(void* stream, const int8_t* data, const int8_t* 
   e.relu = relu;
   float a = fabsf(min_calib), b = fabsf(max_calib);
   e.real_range = (a < b) ? b : a;
+  e.plane = 0;
   launch_fc(static_cast<hipStream_t>(stream), data, weight, M, N, K, N, e);
   MXQ_API_END();
 }

@@ -55,6 +55,10 @@ struct Epilogue {
   float* rmax;
   int relu;
   float real_range;        // MaxAbs(min_calib, max_calib), host-computed
+  // 0: out32 is row-major [M][ldo].  > 0: the rows are pixels of images of `plane` pixels
+  // and out32 is written planar, [M / plane][N][plane] (NCHW for an NHWC convolution);
+  // only out32 has this form.
+  int plane;
 };
 
 __device__ __forceinline__ float dev_maxabs(float a, float b) {
@@ -600,7 +604,13 @@ __device__ __forceinline__ void gemm_epilogue(v16i (&acc)[Cfg::MI][Cfg::NI], con
                                   static_cast<uint32_t>(b32[i]));
         const size_t off = static_cast<size_t>(m) * ldo + n;
         const bool full = n_vec_ok && (n + 3 < N);
-        if (e.out32 != nullptr) {
+        if (e.out32 != nullptr && e.plane > 0) {
+          const int img = m / e.plane, pix = m - img * e.plane;
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            if (n + i < N)
+              e.out32[(static_cast<size_t>(img) * N + (n + i)) * e.plane + pix] = v[i];
+        } else if (e.out32 != nullptr) {
           if (full) {
             v4i w = {v[0], v[1], v[2], v[3]};
             *reinterpret_cast<v4i*>(e.out32 + off) = w;
@@ -731,6 +741,52 @@ __device__ __forceinline__ void gemm_epilogue_lds(v16i (&acc)[Cfg::MI][Cfg::NI],
       for (int mi = 0; mi < MI; ++mi) {
 #pragma unroll
         for (int ni = 0; ni < NI; ++ni) {
+          if (e.plane > 0) {
+            // planar: the tile goes into the scratch channel-major (a lane's 16 values are
+            // one pixel of 16 channels; 32 lanes write 32 adjacent dwords), so that read
+            // back a lane holds 4 adjacent pixels of one channel and 8 lanes cover the
+            // tile's 32 pixels = one 128-byte run of that channel's plane (two runs where
+            // the tile straddles two images)
+#pragma unroll
+            for (int vq = 0; vq < 4; ++vq)
+#pragma unroll
+              for (int i = 0; i < 4; ++i)
+                t32[(8 * vq + 4 * lgrp + i) * Scratch::kPitch32 + lrow] = acc[mi][ni][4 * vq + i];
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            __builtin_amdgcn_wave_barrier();
+            const int c = lane >> 3, p4 = (lane & 7) * 4;
+            v4i col[4];
+#pragma unroll
+            for (int it = 0; it < 4; ++it)
+              col[it] = *reinterpret_cast<const v4i*>(t32 + (it * 8 + c) * Scratch::kPitch32 + p4);
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            __builtin_amdgcn_wave_barrier();
+            const int m0 = m_base + mi * 32 + p4;
+            const int img = m0 / e.plane, pix = m0 - img * e.plane;
+            const bool quad = (e.plane & 3) == 0;  // then 4 | pix and the quad is in one image
+#pragma unroll
+            for (int it = 0; it < 4; ++it) {
+              const int n = n_base + ni * 32 + it * 8 + c;
+              if (n >= N) continue;
+              if (quad) {
+                if (m0 < M)
+                  *reinterpret_cast<v4i*>(e.out32 + (static_cast<size_t>(img) * N + n) * e.plane +
+                                          pix) = col[it];
+              } else {
+                int im = img, px = pix;
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                  if (m0 + j < M)
+                    e.out32[(static_cast<size_t>(im) * N + n) * e.plane + px] = col[it][j];
+                  if (++px == e.plane) {
+                    px = 0;
+                    ++im;
+                  }
+                }
+              }
+            }
+            continue;
+          }
 #pragma unroll
           for (int vq = 0; vq < 4; ++vq) {
             const v4i w = {acc[mi][ni][4 * vq], acc[mi][ni][4 * vq + 1], acc[mi][ni][4 * vq + 2],
@@ -767,7 +823,14 @@ __device__ __forceinline__ void gemm_epilogue_lds(v16i (&acc)[Cfg::MI][Cfg::NI],
             if (m < M && n < N) {
               const v4i w = {acc[mi][ni][4 * vq], acc[mi][ni][4 * vq + 1],
                              acc[mi][ni][4 * vq + 2], acc[mi][ni][4 * vq + 3]};
-              *reinterpret_cast<v4i*>(e.out32 + static_cast<size_t>(m) * ldo + n) = w;
+              if (e.plane > 0) {
+                const int img = m / e.plane, pix = m - img * e.plane;
+#pragma unroll
+                for (int i = 0; i < 4; ++i)  // N % 4 == 0 on this path
+                  e.out32[(static_cast<size_t>(img) * N + (n + i)) * e.plane + pix] = w[i];
+              } else {
+                *reinterpret_cast<v4i*>(e.out32 + static_cast<size_t>(m) * ldo + n) = w;
+              }
             }
           }
     }

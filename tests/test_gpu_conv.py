@@ -123,6 +123,10 @@ def test_layout_adapters(capi):
     np.testing.assert_array_equal(y.cpu().numpy(), x.transpose(0, 2, 3, 1))
     z = capi.nhwc_to_nchw(y)
     np.testing.assert_array_equal(z.cpu().numpy(), x)
+    for shape in ((2, 8, 8, 64), (3, 4, 12, 20), (1, 16, 16, 132)):   # int8 NHWC -> NCHW, dword kernel
+        v8 = int8_uniform(shape, seed=4)
+        z8 = capi.nhwc_to_nchw(dev(v8))
+        np.testing.assert_array_equal(z8.cpu().numpy(), v8.transpose(0, 3, 1, 2))
     v = np.random.default_rng(2).integers(-2**31, 2**31 - 1, size=(2, 70, 66, 130),
                                           dtype=np.int32)
     z = capi.nhwc_to_nchw(dev(v))
@@ -130,8 +134,12 @@ def test_layout_adapters(capi):
     # channel padding: zeros behind the C real channels of every pixel
     import ctypes
     import mxnet_amd
+    # (the last six take the dword kernel: H*W % 4 == 0; 1, 2, 3 and 4 sixteen-byte pieces
+    # per output row, more than 64 channels, a ragged last 128-column tile)
     for shape, cp in (((3, 5, 7, 9), 16), ((2, 3, 70, 33), 16), ((1, 70, 5, 5), 80),
-                      ((2, 16, 4, 4), 16)):
+                      ((2, 16, 4, 4), 16), ((2, 3, 8, 8), 16), ((2, 64, 12, 12), 64),
+                      ((3, 70, 4, 8), 80), ((2, 130, 16, 4), 144), ((1, 40, 4, 4), 48),
+                      ((2, 20, 10, 30), 32)):
         x = int8_uniform(shape, seed=3)
         n, c, h, w = shape
         out = torch.full((n, h, w, cp), 77, dtype=torch.int8, device="cuda")
@@ -157,3 +165,43 @@ def test_conv_1x1_equals_fc(capi):
     rf = capi.quantized_fc(dev(d.reshape(-1, C)), dev(w.reshape(O, C)), None, -one, one, -one,
                            one)
     assert torch.equal(rc["out32"].reshape(-1, O), rf["out32"])
+
+
+@pytest.mark.parametrize("case", [
+    (2, 64, 56, 56, 64, 3, 3, 1, 1, 1),     # planes of 3136 pixels: whole 128-byte runs
+    (3, 32, 28, 28, 96, 1, 1, 1, 0, 1),     # 1x1: the fully-connected route; 784-pixel planes straddle tiles
+    (5, 16, 7, 7, 40, 3, 3, 1, 1, 1),       # 49-pixel planes (not a multiple of 4), O % 16 != 0
+    (2, 16, 13, 9, 33, 3, 3, 2, 1, 1),      # ragged everything, odd O
+    (1, 48, 14, 14, 256, 1, 1, 2, 0, 1),    # strided 1x1
+    (2, 20, 9, 11, 36, 5, 3, 1, 2, 1),      # C % 16 != 0: the register-staged kernel
+])
+@pytest.mark.parametrize("use_bias", [False, True])
+def test_conv_int32_written_as_nchw(capi, case, use_bias):
+    """mxq_quantized_conv_nhwc_out_nchw == the NHWC convolution followed by the layout
+    adapter, and both equal the oracle."""
+    import ctypes
+    import mxnet_amd
+    lib = mxnet_amd._lib.lib
+    N, C, H, W, O, KH, KW, stride, pad, dilate = case
+    d = int8_uniform((N, C, H, W), seed=sum(case))
+    w = int8_uniform((O, C, KH, KW), seed=sum(case) + 1)
+    b = int8_uniform((O,), seed=3) if use_bias else None
+    dn, wn = capi.nchw_to_nhwc_i8(dev(d)), capi.nchw_to_nhwc_i8(dev(w))
+    eh, ew = dilate * (KH - 1) + 1, dilate * (KW - 1) + 1
+    OH, OW = (H + 2 * pad - eh) // stride + 1, (W + 2 * pad - ew) // stride + 1
+    out = torch.full((N, O, OH, OW), 12345, dtype=torch.int32, device="cuda")
+    sc = [f32(v) for v in (-1.0, 1.0, -0.5, 0.5, -2.0, 2.0)]
+    omin, omax = f32(0.0), f32(0.0)
+    P = lambda t: ctypes.c_void_p(t.data_ptr()) if t is not None else None
+    bd = dev(b) if use_bias else None
+    st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    rc = lib.mxq_quantized_conv_nhwc_out_nchw(
+        st, P(dn), P(wn), P(bd), N, H, W, C, O, KH, KW, stride, stride, pad, pad, dilate, dilate,
+        P(sc[0]), P(sc[1]), P(sc[2]), P(sc[3]), P(sc[4]) if use_bias else None,
+        P(sc[5]) if use_bias else None, P(out), P(omin), P(omax))
+    assert rc == 0, lib.mxq_last_error()
+    ro, rmn, rmx = oracle.quantized_conv(d, w, b, -1.0, 1.0, -0.5, 0.5, -2.0 if use_bias else None,
+                                         2.0 if use_bias else None, (stride, stride), (pad, pad),
+                                         (dilate, dilate))
+    np.testing.assert_array_equal(out.cpu().numpy(), ro)
+    assert (omin.item(), omax.item()) == (rmn, rmx)
