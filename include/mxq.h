@@ -210,6 +210,15 @@ int mxq_nchw_to_nhwc_i8(void* stream, const int8_t* in, int8_t* out, int N, int 
  * that is a multiple of 16 takes mxq_quantized_conv_nhwc's fast path. */
 int mxq_nchw_to_nhwc_pad_i8(void* stream, const int8_t* in, int8_t* out, int N, int C, int H,
                             int W, int C_padded);
+/* Space-to-depth by 2 on the way: [N,C,H,W] -> [N,H2,W2,C_padded] with
+ * out[n][h2][w2][(dh*2+dw)*C + c] = in[n][c][2*h2 - off_h + dh][2*w2 - off_w + dw] (zero
+ * outside the image; channels 4*C..C_padded-1 zero), H2 = (H + off_h + 1) / 2, likewise W2,
+ * off in {0,1}.  A KxK stride-2 convolution with padding p over C channels equals the
+ * ceil(K/2) x ceil(K/2) unit-stride convolution with padding (p - off) / 2 over this tensor
+ * (off = p mod 2) and the weight transformed the same way with off = 0, whenever both
+ * give the same output extent; few-channel stride-2 stems run that way. */
+int mxq_nchw_to_s2d_nhwc_i8(void* stream, const int8_t* in, int8_t* out, int N, int C, int H,
+                            int W, int off_h, int off_w, int C_padded);
 /* [N,H,W,C] -> [N,C,H,W]; elem_bytes 1 (int8) or 4 (int32). */
 int mxq_nhwc_to_nchw(void* stream, const void* in, void* out, int N, int C, int H, int W,
                      int elem_bytes);

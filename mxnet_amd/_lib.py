@@ -52,6 +52,7 @@ SIGNATURES = {
                                          [_p, _p, _p]),
     "mxq_nchw_to_nhwc_i8": (_i, [_p, _p, _p, _i, _i, _i, _i]),
     "mxq_nchw_to_nhwc_pad_i8": (_i, [_p, _p, _p, _i, _i, _i, _i, _i]),
+    "mxq_nchw_to_s2d_nhwc_i8": (_i, [_p, _p, _p, _i, _i, _i, _i, _i, _i, _i]),
     "mxq_nhwc_to_nchw": (_i, [_p, _p, _p, _i, _i, _i, _i, _i]),
 }
 

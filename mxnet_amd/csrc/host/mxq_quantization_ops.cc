@@ -638,13 +638,52 @@ static void QuantizedFullyConnectedForwardGPU(const NodeAttrs& attrs, const OpCo
 // byte-granular fallback.
 static int ConvPaddedChannels(int C) { return (C + 15) / 16 * 16; }
 
-static size_t QuantizedConvTempBytes(const TShape& d, const TShape& w, const TShape& o) {
+// A stride-2 convolution over at most 4 channels (an image stem) is run as the unit-stride
+// convolution over the space-to-depth form of its operands (see mxq_nchw_to_s2d_nhwc_i8):
+// 4 * C real channels out of 16 instead of C out of 16.
+struct ConvS2D {
+  bool use;
+  int off_h, off_w;  // pad mod 2
+  int H2, W2;        // extents of the transformed image
+  int K2h, K2w;      // transformed window
+  int pad_h, pad_w;  // transformed padding
+};
+static ConvS2D ConvSpaceToDepth(const ConvolutionParam& param, const TShape& d, const TShape& w,
+                                const TShape& o) {
+  ConvS2D r = {};
+  const int C = d[1], H = d[2], W = d[3], KH = w[2], KW = w[3];
+  if (C > 4 || param.stride[0] != 2 || param.stride[1] != 2 || param.dilate[0] != 1 ||
+      param.dilate[1] != 1 || KH < 2 || KW < 2)
+    return r;
+  const int ph = param.pad[0], pw = param.pad[1];
+  r.off_h = ph & 1;
+  r.off_w = pw & 1;
+  r.H2 = (H + r.off_h + 1) / 2;
+  r.W2 = (W + r.off_w + 1) / 2;
+  r.K2h = (KH + 1) / 2;
+  r.K2w = (KW + 1) / 2;
+  r.pad_h = (ph - r.off_h) / 2;
+  r.pad_w = (pw - r.off_w) / 2;
+  // the transformed problem must produce exactly the operator's output extent
+  r.use = r.H2 + 2 * r.pad_h - r.K2h + 1 == static_cast<int>(o[2]) &&
+          r.W2 + 2 * r.pad_w - r.K2w + 1 == static_cast<int>(o[3]);
+  return r;
+}
+
+static size_t QuantizedConvTempBytes(const ConvolutionParam& param, const TShape& d,
+                                     const TShape& w, const TShape& o) {
   auto up = [](size_t x) { return (x + 255) / 256 * 256; };
+  const ConvS2D s2d = ConvSpaceToDepth(param, d, w, o);
+  if (s2d.use) {
+    const size_t CP = static_cast<size_t>(ConvPaddedChannels(4 * static_cast<int>(d[1])));
+    return up(static_cast<size_t>(d[0]) * s2d.H2 * s2d.W2 * CP) +
+           up(static_cast<size_t>(w[0]) * s2d.K2h * s2d.K2w * CP);
+  }
   const size_t C = static_cast<size_t>(d[1]);
   const size_t scale_num = static_cast<size_t>(ConvPaddedChannels(static_cast<int>(C)));
   const size_t d_bytes = C == 0 ? 0 : d.Size() / C * scale_num;
   const size_t w_bytes = C == 0 ? 0 : w.Size() / C * scale_num;
-  (void)o;  // the output is written in its own layout: no third buffer
+  // the output is written in its own layout: no third buffer
   return up(d_bytes) + up(w_bytes);
 }
 
@@ -662,21 +701,36 @@ static void QuantizedConvForwardGPU(const NodeAttrs& attrs, const OpContext& ctx
   const TShape& o = outputs[0].shape_;
   CHECK(!ctx.requested.empty()) << "quantized_conv needs its temp space resource";
   auto up = [](size_t x) { return (x + 255) / 256 * 256; };
-  char* ws = ctx.requested[0].get_space(QuantizedConvTempBytes(d, w, o));
+  char* ws = ctx.requested[0].get_space(QuantizedConvTempBytes(param, d, w, o));
   const int N = d[0], C = d[1], H = d[2], W = d[3], O = w[0], KH = w[2], KW = w[3];
-  const int CP = ConvPaddedChannels(C);
-  const size_t d_bytes = static_cast<size_t>(N) * H * W * CP;
-  int8_t* d_nhwc = reinterpret_cast<int8_t*>(ws);
-  int8_t* w_ohwi = reinterpret_cast<int8_t*>(ws + up(d_bytes));
   void* stream = raw_stream(ctx);
-  MXQ_CALL(mxq_nchw_to_nhwc_pad_i8(stream, inputs[0].dptr<int8_t>(), d_nhwc, N, C, H, W, CP));
-  MXQ_CALL(mxq_nchw_to_nhwc_pad_i8(stream, inputs[1].dptr<int8_t>(), w_ohwi, O, C, KH, KW, CP));
+  int8_t* d_nhwc = reinterpret_cast<int8_t*>(ws);
+  // the convolution as the kernel sees it
+  int cH = H, cW = W, cC = ConvPaddedChannels(C), cKH = KH, cKW = KW;
+  int sh = static_cast<int>(param.stride[0]), sw = static_cast<int>(param.stride[1]);
+  int ph = static_cast<int>(param.pad[0]), pw = static_cast<int>(param.pad[1]);
+  const ConvS2D s2d = ConvSpaceToDepth(param, d, w, o);
+  int8_t* w_ohwi;
+  if (s2d.use) {
+    cC = ConvPaddedChannels(4 * C);
+    cH = s2d.H2; cW = s2d.W2; cKH = s2d.K2h; cKW = s2d.K2w;
+    sh = sw = 1;
+    ph = s2d.pad_h; pw = s2d.pad_w;
+    w_ohwi = reinterpret_cast<int8_t*>(ws + up(static_cast<size_t>(N) * cH * cW * cC));
+    MXQ_CALL(mxq_nchw_to_s2d_nhwc_i8(stream, inputs[0].dptr<int8_t>(), d_nhwc, N, C, H, W,
+                                     s2d.off_h, s2d.off_w, cC));
+    MXQ_CALL(mxq_nchw_to_s2d_nhwc_i8(stream, inputs[1].dptr<int8_t>(), w_ohwi, O, C, KH, KW, 0, 0,
+                                     cC));
+  } else {
+    w_ohwi = reinterpret_cast<int8_t*>(ws + up(static_cast<size_t>(N) * H * W * cC));
+    MXQ_CALL(mxq_nchw_to_nhwc_pad_i8(stream, inputs[0].dptr<int8_t>(), d_nhwc, N, C, H, W, cC));
+    MXQ_CALL(mxq_nchw_to_nhwc_pad_i8(stream, inputs[1].dptr<int8_t>(), w_ohwi, O, C, KH, KW, cC));
+  }
   const size_t ni = param.no_bias ? 2 : 3;
   MXQ_CALL(mxq_quantized_conv_nhwc_out_nchw(
-      stream, d_nhwc, w_ohwi, param.no_bias ? nullptr : inputs[2].dptr<int8_t>(), N, H, W, CP, O,
-      KH, KW, static_cast<int>(param.stride[0]), static_cast<int>(param.stride[1]),
-      static_cast<int>(param.pad[0]), static_cast<int>(param.pad[1]),
-      static_cast<int>(param.dilate[0]), static_cast<int>(param.dilate[1]),
+      stream, d_nhwc, w_ohwi, param.no_bias ? nullptr : inputs[2].dptr<int8_t>(), N, cH, cW, cC,
+      O, cKH, cKW, sh, sw, ph, pw, static_cast<int>(param.dilate[0]),
+      static_cast<int>(param.dilate[1]),
       inputs[ni].dptr<float>(), inputs[ni + 1].dptr<float>(), inputs[ni + 2].dptr<float>(),
       inputs[ni + 3].dptr<float>(), param.no_bias ? nullptr : inputs[7].dptr<float>(),
       param.no_bias ? nullptr : inputs[8].dptr<float>(), outputs[0].dptr<int32_t>(),
@@ -811,7 +865,8 @@ size_t MXQTempSpaceBytes(const NodeAttrs& attrs, const ShapeVector& in, const Sh
   const std::string& name = attrs.op->name;
   if (name == "_contrib_quantize_v2") return mxq_quantize_v2_workspace(in[0].Size());
   if (name == "_contrib_requantize") return mxq_requantize_workspace(in[0].Size());
-  if (name == "_contrib_quantized_conv") return QuantizedConvTempBytes(in[0], in[1], out[0]);
+  if (name == "_contrib_quantized_conv")
+    return QuantizedConvTempBytes(nnvm::get<ConvolutionParam>(attrs.parsed), in[0], in[1], out[0]);
   return 0;
 }
 

@@ -341,6 +341,34 @@ __global__ __launch_bounds__(256) void transpose_i8_kernel(const uint8_t* __rest
   }
 }
 
+// Space-to-depth by 2 while going from planes to pixels: out[b][h2][w2][(dh*2+dw)*C + c] =
+// in[b][c][2*h2 - off_h + dh][2*w2 - off_w + dw] (zero outside the plane), the channel run
+// of every output pixel zero-padded to CP bytes.  A stride-2 convolution over few channels
+// becomes a unit-stride one over 4*C channels and half the window, which suits the
+// direct-to-LDS kernels (16-byte channel runs) far better than 3 or 4 channels do.
+__global__ __launch_bounds__(256) void s2d_nhwc_kernel(const int8_t* __restrict__ in,
+                                                       int8_t* __restrict__ out, int C, int H,
+                                                       int W, int H2, int W2, int off_h,
+                                                       int off_w, int CP, size_t pixels) {
+  for (size_t p = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x; p < pixels;
+       p += static_cast<size_t>(gridDim.x) * 256) {
+    const int w2 = static_cast<int>(p % W2);
+    const size_t t = p / W2;
+    const int h2 = static_cast<int>(t % H2);
+    const size_t b = t / H2;
+    const int8_t* img = in + b * static_cast<size_t>(C) * H * W;
+    int8_t* dst = out + p * CP;
+    for (int d = 0; d < 4; ++d) {
+      const int h = 2 * h2 - off_h + (d >> 1), w = 2 * w2 - off_w + (d & 1);
+      const bool inside = static_cast<unsigned>(h) < static_cast<unsigned>(H) &&
+                          static_cast<unsigned>(w) < static_cast<unsigned>(W);
+      for (int c = 0; c < C; ++c)
+        dst[d * C + c] = inside ? img[(static_cast<size_t>(c) * H + h) * W + w] : int8_t(0);
+    }
+    for (int c = 4 * C; c < CP; ++c) dst[c] = 0;
+  }
+}
+
 template <typename T>
 void launch_transpose(hipStream_t s, const void* in, void* out, int B, int R, int S, int RP) {
   if (B == 0 || RP == 0 || S == 0) return;
@@ -524,6 +552,25 @@ int mxq_nchw_to_nhwc_pad_i8(void* stream, const int8_t* in, int8_t* out, int N, 
   if (static_cast<long long>(N) * C_padded * H * W == 0) return 0;
   MXQ_CHECK(in != nullptr && out != nullptr, "null pointer");
   launch_transpose<int8_t>(static_cast<hipStream_t>(stream), in, out, N, C, H * W, C_padded);
+  MXQ_API_END();
+}
+
+int mxq_nchw_to_s2d_nhwc_i8(void* stream, const int8_t* in, int8_t* out, int N, int C, int H,
+                            int W, int off_h, int off_w, int C_padded) {
+  MXQ_API_BEGIN();
+  MXQ_CHECK(N >= 0 && C >= 0 && H >= 0 && W >= 0, "negative dimension");
+  MXQ_CHECK((off_h == 0 || off_h == 1) && (off_w == 0 || off_w == 1), "offsets are 0 or 1");
+  MXQ_CHECK(C_padded >= 4 * C, "C_padded must be at least 4 * C");
+  const int H2 = (H + off_h + 1) / 2, W2 = (W + off_w + 1) / 2;
+  const size_t pixels = static_cast<size_t>(N) * H2 * W2;
+  if (pixels == 0 || C_padded == 0) return 0;
+  MXQ_CHECK(in != nullptr && out != nullptr, "null pointer");
+  size_t g = (pixels + 255) / 256;
+  if (g > 65535u * 16u) g = 65535u * 16u;
+  hipLaunchKernelGGL(s2d_nhwc_kernel, dim3(static_cast<unsigned>(g)), dim3(256), 0,
+                     static_cast<hipStream_t>(stream), in, out, C, H, W, H2, W2, off_h, off_w,
+                     C_padded, pixels);
+  MXQ_LAUNCH_CHECK();
   MXQ_API_END();
 }
 

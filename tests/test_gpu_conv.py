@@ -153,6 +153,28 @@ def test_layout_adapters(capi):
         np.testing.assert_array_equal(out.cpu().numpy(), want)
     rc = mxnet_amd._lib.lib.mxq_nchw_to_nhwc_pad_i8(st, None, None, 1, 8, 2, 2, 4)
     assert rc == -1 and b"C_padded" in mxnet_amd._lib.lib.mxq_last_error()
+    # space-to-depth by 2 with an offset of 0 or 1 in each direction
+    for shape, off_h, off_w, cp in (((2, 3, 8, 10), 1, 1, 16), ((1, 3, 7, 9), 0, 1, 16),
+                                    ((2, 4, 5, 5), 1, 0, 16), ((3, 1, 6, 6), 0, 0, 4),
+                                    ((1, 2, 224, 224), 1, 1, 32)):
+        x = int8_uniform(shape, seed=5)
+        n, c, h, w = shape
+        h2, w2 = (h + off_h + 1) // 2, (w + off_w + 1) // 2
+        out = torch.full((n, h2, w2, cp), 77, dtype=torch.int8, device="cuda")
+        rc = mxnet_amd._lib.lib.mxq_nchw_to_s2d_nhwc_i8(st, ctypes.c_void_p(dev(x).data_ptr()),
+                                                        ctypes.c_void_p(out.data_ptr()), n, c, h,
+                                                        w, off_h, off_w, cp)
+        assert rc == 0
+        padded = np.zeros((n, c, 2 * h2 + 2, 2 * w2 + 2), np.int8)
+        padded[:, :, off_h:off_h + h, off_w:off_w + w] = x
+        want = np.zeros((n, h2, w2, cp), np.int8)
+        for dh in range(2):
+            for dw in range(2):
+                blk = padded[:, :, dh:dh + 2 * h2:2, dw:dw + 2 * w2:2]     # [n, c, h2, w2]
+                want[..., (dh * 2 + dw) * c:(dh * 2 + dw + 1) * c] = blk.transpose(0, 2, 3, 1)
+        np.testing.assert_array_equal(out.cpu().numpy(), want)
+    rc = mxnet_amd._lib.lib.mxq_nchw_to_s2d_nhwc_i8(st, None, None, 1, 8, 2, 2, 0, 0, 16)
+    assert rc == -1 and b"4 * C" in mxnet_amd._lib.lib.mxq_last_error()
 
 
 def test_conv_1x1_equals_fc(capi):

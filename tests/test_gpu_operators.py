@@ -211,7 +211,14 @@ def test_quantized_conv(contrib, use_bias):
 
 
 @pytest.mark.parametrize("shape,filters,kernel,stride,pad", [
-    ((2, 3, 64, 64), 64, (7, 7), (2, 2), (3, 3)),     # a 3-channel stem: channels padded to 16
+    ((2, 3, 64, 64), 64, (7, 7), (2, 2), (3, 3)),     # a 3-channel stem: space-to-depth route
+    ((1, 3, 32, 30), 16, (3, 3), (2, 2), (1, 1)),     # the same route, odd padding
+    ((2, 4, 17, 19), 24, (5, 5), (2, 2), (2, 2)),     # even padding, odd extents
+    ((2, 1, 16, 16), 8, (2, 2), (2, 2), (0, 0)),      # one channel, window = stride
+    ((1, 3, 15, 15), 32, (7, 7), (2, 2), (3, 3)),
+    ((1, 2, 12, 14), 8, (4, 3), (2, 2), (1, 1)),      # rectangular window
+    ((1, 3, 9, 9), 8, (2, 2), (2, 2), (0, 0)),        # extents disagree: plain route, 16 channels
+    ((2, 3, 20, 20), 8, (3, 3), (2, 1), (1, 1)),      # stride 2 in one direction only: plain route
     ((2, 20, 9, 11), 36, (5, 3), (1, 1), (2, 1)),     # 20 channels padded to 32
     ((1, 17, 8, 8), 8, (1, 1), (1, 1), (0, 0)),
 ])
