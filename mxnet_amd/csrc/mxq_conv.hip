@@ -233,6 +233,11 @@ typedef GemmCfg<256, 64, 64, 4, 1> CfgW64;   // 4 waves, wave tile 64 x 64
 typedef GemmCfg<128, 128, 64, 2, 2> CfgM;    // 4 waves, wave tile 64 x 64
 typedef GemmCfg<64, 64, 64, 2, 2> CfgS;      // 4 waves, wave tile 32 x 32
 typedef GemmCfg<256, 256, 64, 2, 2> CfgL4;   // 4 waves, wave tile 128 x 128
+// 128-byte stages: half as many K steps
+typedef GemmCfg<256, 256, 128, 2, 4> CfgL8K;
+typedef GemmCfg<256, 128, 128, 4, 2> CfgW128K;
+typedef GemmCfg<128, 128, 128, 2, 2> CfgMK;
+typedef GemmCfg<64, 64, 128, 2, 2> CfgSK;
 
 template <class Cfg, int NS, int PIPE>
 void launch_dma(hipStream_t s, const ConvArgs& a) {
@@ -454,10 +459,12 @@ void conv_nhwc(void* stream, const int8_t* data, const int8_t* weight, const int
       switch (choose_tile(a.M, O, a.K, cus)) {
         case Tile::kL8: cfg = 11; break;
         case Tile::kW128x2: cfg = 22; break;
+        case Tile::kW128K2: cfg = 36; break;
         case Tile::kM128x2: cfg = 24; break;
-        case Tile::kM128x4: cfg = 14; break;
+        case Tile::kM128K2: cfg = 33; break;
         case Tile::kS64x2: cfg = 25; break;
         case Tile::kS64x4: cfg = 15; break;
+        case Tile::kS64K2: cfg = 31; break;
       }
     } else if (O > 128 && tiles(256, 256) >= cus) {
       cfg = 1;
@@ -484,6 +491,12 @@ void conv_nhwc(void* stream, const int8_t* data, const int8_t* weight, const int
     case 14: launch_dma<CfgM, 4, 2>(s, a); break;
     case 15: launch_dma<CfgS, 4, 2>(s, a); break;
     case 16: launch_dma<CfgL4, 4, 2>(s, a); break;
+    case 31: launch_dma<CfgSK, 2, 0>(s, a); break;
+    case 32: launch_dma<CfgSK, 3, 0>(s, a); break;
+    case 33: launch_dma<CfgMK, 2, 0>(s, a); break;
+    case 34: launch_dma<CfgMK, 3, 0>(s, a); break;
+    case 35: launch_dma<CfgL8K, 2, 0>(s, a); break;
+    case 36: launch_dma<CfgW128K, 2, 0>(s, a); break;
     case 22: launch_dma<CfgW128, 2, 0>(s, a); break;
     case 23: launch_dma<CfgW64, 2, 0>(s, a); break;
     case 24: launch_dma<CfgM, 2, 0>(s, a); break;

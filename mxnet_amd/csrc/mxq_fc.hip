@@ -95,6 +95,11 @@ typedef GemmCfg<256, 128, 64, 4, 2> CfgW128;  // 8 waves, wave tile 64 x 64
 typedef GemmCfg<256, 64, 64, 4, 1> CfgW64;    // 4 waves, wave tile 64 x 64
 typedef GemmCfg<128, 128, 64, 2, 2> CfgM;     // 4 waves, wave tile 64 x 64
 typedef GemmCfg<64, 64, 64, 2, 2> CfgS;       // 4 waves, wave tile 32 x 32
+// 128-byte stages: half as many K steps (each costs a barrier and a round of DMA latency)
+typedef GemmCfg<256, 256, 128, 2, 4> CfgL8K;   // 8 waves, wave tile 128 x 64
+typedef GemmCfg<256, 128, 128, 4, 2> CfgW128K; // 8 waves, wave tile 64 x 64
+typedef GemmCfg<128, 128, 128, 2, 2> CfgMK;    // 4 waves, wave tile 64 x 64
+typedef GemmCfg<64, 64, 128, 2, 2> CfgSK;      // 4 waves, wave tile 32 x 32
 
 template <class Cfg, int NS, int PIPE, bool BUF>
 void launch_dma(hipStream_t s, const FcArgs& a) {
@@ -134,6 +139,7 @@ int num_cus() {
 //   21..24  direct-to-LDS buffer-load kernels 256x128, 256x64, 128x128, 64x64
 //   31, 32  as 12 / 16 with buffer loads (K % 16 == 0 instead of K % 64 == 0)
 //   41..44  as 21..24 with a 2-stage ring (short K)
+//   51..56  128-byte stages: 64x64 (2, 3 stages), 128x128 (2, 3), 256x256 (2), 256x128 (2)
 void launch_fc(hipStream_t s, const int8_t* data, const int8_t* weight, int M, int N, int K,
                int ldo, const Epilogue& epi) {
   FcArgs a;
@@ -160,10 +166,12 @@ void launch_fc(hipStream_t s, const int8_t* data, const int8_t* weight, int M, i
       switch (choose_tile(M, N, K, cus)) {
         case Tile::kL8: cfg = glb_ok ? 12 : 31; break;
         case Tile::kW128x2: cfg = 41; break;
+        case Tile::kW128K2: cfg = 56; break;
         case Tile::kM128x2: cfg = 43; break;
-        case Tile::kM128x4: cfg = 23; break;
+        case Tile::kM128K2: cfg = 53; break;
         case Tile::kS64x2: cfg = 44; break;
         case Tile::kS64x4: cfg = 24; break;
+        case Tile::kS64K2: cfg = 51; break;
       }
     } else {
       if (tiles(256, 256) >= cus)
@@ -193,6 +201,12 @@ void launch_fc(hipStream_t s, const int8_t* data, const int8_t* weight, int M, i
     case 42: launch_dma<CfgW64, 2, 0, true>(s, a); break;
     case 43: launch_dma<CfgM, 2, 0, true>(s, a); break;
     case 44: launch_dma<CfgS, 2, 0, true>(s, a); break;
+    case 51: launch_dma<CfgSK, 2, 0, true>(s, a); break;
+    case 52: launch_dma<CfgSK, 3, 0, true>(s, a); break;
+    case 53: launch_dma<CfgMK, 2, 0, true>(s, a); break;
+    case 54: launch_dma<CfgMK, 3, 0, true>(s, a); break;
+    case 55: launch_dma<CfgL8K, 2, 0, true>(s, a); break;
+    case 56: launch_dma<CfgW128K, 2, 0, true>(s, a); break;
     case 31: launch_dma<CfgL8, 4, 2, true>(s, a); break;
     case 32: launch_dma<CfgL4, 4, 2, true>(s, a); break;
     default: MXQ_CHECK(false, "unknown fc tile configuration " << cfg);

@@ -57,7 +57,8 @@ def test_fc_int32(capi, M, K, N, use_bias):
     assert (res["omin"].item(), res["omax"].item()) == (rmn, rmx)
 
 
-@pytest.mark.parametrize("cfg", [1, 2, 3, 4, 11, 12, 14, 16, 21, 22, 23, 24, 31, 32, 41, 42, 43, 44])
+@pytest.mark.parametrize("cfg", [1, 2, 3, 4, 11, 12, 14, 16, 21, 22, 23, 24, 31, 32, 41, 42, 43, 44,
+                                 51, 52, 53, 54, 55, 56])
 @pytest.mark.parametrize("M,K,N", [(512, 512, 512), (300, 208, 270), (70, 444, 33),
                                    (300, 192, 270), (1, 64, 1), (1024, 1024, 520),
                                    (130, 16, 70), (257, 80, 64)])
