@@ -238,6 +238,9 @@ typedef GemmCfg<256, 256, 128, 2, 4> CfgL8K;
 typedef GemmCfg<256, 128, 128, 4, 2> CfgW128K;
 typedef GemmCfg<128, 128, 128, 2, 2> CfgMK;
 typedef GemmCfg<64, 64, 128, 2, 2> CfgSK;
+typedef GemmCfg<128, 64, 128, 2, 2> CfgRK;
+typedef GemmCfg<64, 128, 128, 2, 2> CfgQK;
+typedef GemmCfg<64, 64, 256, 2, 2> CfgSK2;
 
 template <class Cfg, int NS, int PIPE>
 void launch_dma(hipStream_t s, const ConvArgs& a) {
@@ -456,7 +459,7 @@ void conv_nhwc(void* stream, const int8_t* data, const int8_t* weight, const int
       return static_cast<long>((a.M + bm - 1) / bm) * ((O + bn - 1) / bn);
     };
     if (dma_ok) {
-      switch (choose_tile(a.M, O, a.K, cus)) {
+      switch (choose_tile(a.M, O, a.K, cus, true)) {
         case Tile::kL8: cfg = 11; break;
         case Tile::kW128x2: cfg = 22; break;
         case Tile::kW128K2: cfg = 36; break;
@@ -465,6 +468,9 @@ void conv_nhwc(void* stream, const int8_t* data, const int8_t* weight, const int
         case Tile::kS64x2: cfg = 25; break;
         case Tile::kS64x4: cfg = 15; break;
         case Tile::kS64K2: cfg = 31; break;
+        case Tile::kR128K2: cfg = 37; break;
+        case Tile::kQ128K2: cfg = 38; break;
+        case Tile::kS64K4: cfg = 39; break;
       }
     } else if (O > 128 && tiles(256, 256) >= cus) {
       cfg = 1;
@@ -497,6 +503,9 @@ void conv_nhwc(void* stream, const int8_t* data, const int8_t* weight, const int
     case 34: launch_dma<CfgMK, 3, 0>(s, a); break;
     case 35: launch_dma<CfgL8K, 2, 0>(s, a); break;
     case 36: launch_dma<CfgW128K, 2, 0>(s, a); break;
+    case 37: launch_dma<CfgRK, 2, 0>(s, a); break;
+    case 38: launch_dma<CfgQK, 2, 0>(s, a); break;
+    case 39: launch_dma<CfgSK2, 2, 0>(s, a); break;
     case 22: launch_dma<CfgW128, 2, 0>(s, a); break;
     case 23: launch_dma<CfgW64, 2, 0>(s, a); break;
     case 24: launch_dma<CfgM, 2, 0>(s, a); break;

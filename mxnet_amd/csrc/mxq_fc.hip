@@ -100,6 +100,9 @@ typedef GemmCfg<256, 256, 128, 2, 4> CfgL8K;   // 8 waves, wave tile 128 x 64
 typedef GemmCfg<256, 128, 128, 4, 2> CfgW128K; // 8 waves, wave tile 64 x 64
 typedef GemmCfg<128, 128, 128, 2, 2> CfgMK;    // 4 waves, wave tile 64 x 64
 typedef GemmCfg<64, 64, 128, 2, 2> CfgSK;      // 4 waves, wave tile 32 x 32
+typedef GemmCfg<128, 64, 128, 2, 2> CfgRK;     // 4 waves, wave tile 64 x 32
+typedef GemmCfg<64, 128, 128, 2, 2> CfgQK;     // 4 waves, wave tile 32 x 64
+typedef GemmCfg<64, 64, 256, 2, 2> CfgSK2;     // 256-byte stages for very long K
 
 template <class Cfg, int NS, int PIPE, bool BUF>
 void launch_dma(hipStream_t s, const FcArgs& a) {
@@ -140,6 +143,7 @@ int num_cus() {
 //   31, 32  as 12 / 16 with buffer loads (K % 16 == 0 instead of K % 64 == 0)
 //   41..44  as 21..24 with a 2-stage ring (short K)
 //   51..56  128-byte stages: 64x64 (2, 3 stages), 128x128 (2, 3), 256x256 (2), 256x128 (2)
+//   57..59  128x64 and 64x128 with 128-byte stages, 64x64 with 256-byte stages
 void launch_fc(hipStream_t s, const int8_t* data, const int8_t* weight, int M, int N, int K,
                int ldo, const Epilogue& epi) {
   FcArgs a;
@@ -172,6 +176,9 @@ void launch_fc(hipStream_t s, const int8_t* data, const int8_t* weight, int M, i
         case Tile::kS64x2: cfg = 44; break;
         case Tile::kS64x4: cfg = 24; break;
         case Tile::kS64K2: cfg = 51; break;
+        case Tile::kR128K2: cfg = 57; break;
+        case Tile::kQ128K2: cfg = 58; break;
+        case Tile::kS64K4: cfg = 59; break;
       }
     } else {
       if (tiles(256, 256) >= cus)
@@ -207,6 +214,9 @@ void launch_fc(hipStream_t s, const int8_t* data, const int8_t* weight, int M, i
     case 54: launch_dma<CfgMK, 3, 0, true>(s, a); break;
     case 55: launch_dma<CfgL8K, 2, 0, true>(s, a); break;
     case 56: launch_dma<CfgW128K, 2, 0, true>(s, a); break;
+    case 57: launch_dma<CfgRK, 2, 0, true>(s, a); break;
+    case 58: launch_dma<CfgQK, 2, 0, true>(s, a); break;
+    case 59: launch_dma<CfgSK2, 2, 0, true>(s, a); break;
     case 31: launch_dma<CfgL8, 4, 2, true>(s, a); break;
     case 32: launch_dma<CfgL4, 4, 2, true>(s, a); break;
     default: MXQ_CHECK(false, "unknown fc tile configuration " << cfg);

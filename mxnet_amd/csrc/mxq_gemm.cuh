@@ -128,6 +128,7 @@ template <int CH>
 __device__ __forceinline__ int swz(int r) {
   if (CH == 4) return (((r >> 1) ^ (r >> 3)) & 1) | (((r >> 2) & 1) << 1);
   if (CH == 8) return (r ^ (r >> 2)) & 7;
+  if (CH == 16) return r & 15;
   return 0;
 }
 
@@ -453,7 +454,8 @@ __device__ __forceinline__ void gemm_mainloop_dma(v16i (&acc)[Cfg::MI][Cfg::NI],
   static_assert((Cfg::BM * CH) % (NW * 64) == 0 && (Cfg::BN * CH) % (NW * 64) == 0, "dma tiling");
   static_assert(PIPE == 0 || PIPE == 2, "pipeline variant");
   static_assert(PIPE == 0 || NS >= 4, "cross-barrier fragment prefetch needs 4 stages");
-  static_assert(CH == 4 || CH == 8, "fragment addressing below needs swz() to ignore row bit 5");
+  static_assert(CH == 4 || CH == 8 || CH == 16,
+                "fragment addressing below needs swz() to ignore row bit 5");
   static_assert((NS - 2) * CPT < 64, "vmcnt range");
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);

@@ -12,7 +12,10 @@ enum class Tile {
   kM128K2,  // 128 x 128, 128-byte stages, 2-stage ring
   kS64x2,   // 64 x 64, 64-byte stages, 2-stage ring
   kS64x4,   // 64 x 64, 64-byte stages, 4-stage ring, pinned pipeline
-  kS64K2    // 64 x 64, 128-byte stages, 2-stage ring
+  kS64K2,   // 64 x 64, 128-byte stages, 2-stage ring
+  kS64K4,   // 64 x 64, 256-byte stages, 2-stage ring
+  kR128K2,  // 128 x 64, 128-byte stages, 2-stage ring
+  kQ128K2   // 64 x 128, 128-byte stages, 2-stage ring
 };
 
 // M x N outputs, reduction length K, `cus` compute units.  Distilled from sweeps over
@@ -27,14 +30,31 @@ enum class Tile {
 //    deep (half as many steps: 10-20 % on every mid-size shape measured); below that the
 //    deeper stage would mostly be padding or leave too few steps to overlap;
 //  * 256 x 128 from 0.75 tiles per CU (fewer, larger stores per loaded byte), 128 x 128
-//    once it fills the chip, else 64 x 64 keeps every CU busy.
-inline Tile choose_tile(long M, long N, long K, long cus) {
+//    once it fills the chip, then 128 x 64 / 64 x 128, else 64 x 64 keeps every CU busy.
+// `gather` says that the left operand is gathered pixel by pixel (convolution): the 64-row
+// tile then issues half as many gathers per wave and measures a few per cent ahead of the
+// 128-row one, which in turn is ahead for plain row-major operands.
+inline Tile choose_tile(long M, long N, long K, long cus, bool gather = false) {
   auto tiles = [&](long bm, long bn) { return ((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
   if (K > 256 && N > 128 && 16 * tiles(256, 256) >= 9 * cus) return Tile::kL8;
   if (N <= 64) return (K >= 4096) ? Tile::kS64x4 : Tile::kS64x2;
   if (4 * tiles(256, 128) >= 3 * cus) return (K >= 512) ? Tile::kW128K2 : Tile::kW128x2;
   if (tiles(128, 128) >= cus) return (K >= 256) ? Tile::kM128K2 : Tile::kM128x2;
-  return (K >= 512) ? Tile::kS64K2 : Tile::kS64x2;
+  if (K < 512) return Tile::kS64x2;
+  // half-size tiles while they still give every CU one: 12544 x 2304 -> 256 takes 14.1 us on
+  // 392 tiles of 64 x 128 against 17.6 us on 784 tiles of 64 x 64.  From K = 4096 on the
+  // 64 x 64 tile with 256-byte stages is the better of the two unless the half-size tiles
+  // still come two to a CU (512 x 4096 -> 4096: 18.3 us against 19.8 us on 256 tiles).
+  const long tq = tiles(64, 128), tr = tiles(128, 64);
+  const long need = (K >= 4096) ? 2 * cus : cus;
+  if (tq >= need || tr >= need) {
+    const bool q_fits = tq >= need && N % 128 == 0, r_fits = tr >= need;
+    if (q_fits && (gather || !r_fits)) return Tile::kQ128K2;
+    return r_fits ? Tile::kR128K2 : Tile::kQ128K2;
+  }
+  // 256-byte stages once K is long enough to leave them several steps (3136 x 4608 -> 512:
+  // 15.8 us against 19.8 us)
+  return (K >= 4096) ? Tile::kS64K4 : Tile::kS64K2;
 }
 
 }  // namespace mxq

@@ -70,7 +70,7 @@ def test_conv_int32(capi, case, use_bias):
 
 
 @pytest.mark.parametrize("cfg", [1, 2, 3, 4, 5, 11, 12, 13, 14, 15, 16, 22, 23, 24, 25, 31, 32, 33, 34,
-                                 35, 36])
+                                 35, 36, 37, 38, 39])
 def test_conv_every_tile_config(capi, cfg):
     import mxnet_amd
     N, C, H, W, O, KH, KW, s, p, dl = (2, 32, 19, 19, 72, 3, 3, 1, 1, 1)
@@ -92,7 +92,8 @@ def test_conv_every_tile_config(capi, cfg):
     assert (res["rmin"].item(), res["rmax"].item()) == (qmn, qmx)
 
 
-@pytest.mark.parametrize("cfg", [11, 12, 13, 14, 15, 16, 22, 23, 24, 25, 31, 32, 33, 34, 35, 36])
+@pytest.mark.parametrize("cfg", [11, 12, 13, 14, 15, 16, 22, 23, 24, 25, 31, 32, 33, 34, 35, 36, 37,
+                                 38, 39])
 @pytest.mark.parametrize("case", [(2, 16, 9, 11, 40, 3, 3, 1, 1, 1), (1, 48, 8, 8, 24, 5, 3, 2, 2, 1),
                                   (2, 64, 14, 14, 96, 1, 1, 2, 0, 1), (1, 16, 12, 12, 20, 3, 3, 1, 2, 2),
                                   (3, 128, 7, 7, 130, 3, 3, 1, 1, 1)])

@@ -58,7 +58,7 @@ def test_fc_int32(capi, M, K, N, use_bias):
 
 
 @pytest.mark.parametrize("cfg", [1, 2, 3, 4, 11, 12, 14, 16, 21, 22, 23, 24, 31, 32, 41, 42, 43, 44,
-                                 51, 52, 53, 54, 55, 56])
+                                 51, 52, 53, 54, 55, 56, 57, 58, 59])
 @pytest.mark.parametrize("M,K,N", [(512, 512, 512), (300, 208, 270), (70, 444, 33),
                                    (300, 192, 270), (1, 64, 1), (1024, 1024, 520),
                                    (130, 16, 70), (257, 80, 64)])
