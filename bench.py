@@ -47,6 +47,10 @@ MEASURED_TRAFFIC_BYTES = {
     "elemwise_add": (2.0 * 65570.1 + 262176.7) * _KIB,          # add_kernel_int32_64M.md
     "elemwise_add_int8": (2.0 * 65583.7 + 65536.1) * _KIB,      # add_kernel_int8_64M.md
     "concat": (2.0 * 32840.8 + 65536.1) * _KIB,                 # concat_kernel_64M.md
+    "elemwise_mul_int8": (2.0 * 65565.8 + 65536.1) * _KIB,      # mul_kernel_int8_64M.md
+    "quantize_asym": (2.0 * 131099.2 + 65536.1) * _KIB,         # quantize_asym_kernel_64M.md
+    "embedding": (2.0 * 31709.6 + 65535.8) * _KIB,              # embedding_kernel_bert_vocab.md
+    "transpose": (2.0 * 32796.4 + 65536.1) * _KIB,              # permute_elem_kernel_attention_64M.md
 }
 
 
@@ -58,7 +62,9 @@ def parse_args():
     ap.add_argument("--workload", default="fc4096",
                     choices=["fc4096", "fc8192", "quantize", "quantize_uncal", "quantize_uint8",
                              "requantize", "requantize_uncal", "dequantize", "copy", "maxpool", "avgpool",
-                             "elemwise_add", "elemwise_add_int8", "concat", "resnet50_convs", "bert_fc_chain", "bert_fc_chain_fused"])
+                             "elemwise_add", "elemwise_add_int8", "concat", "elemwise_mul_int8", "quantize_asym",
+                             "embedding", "transpose", "resnet50_convs", "bert_fc_chain",
+                             "bert_fc_chain_fused"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-cast-ops", action="store_true")
     return ap.parse_args()
@@ -154,7 +160,7 @@ class CastWorkload:
         self.omin = torch.empty(1, device="cuda")
         self.omax = torch.empty(1, device="cuda")
         self.ws = torch.empty(lib.mxq_quantize_v2_workspace(n), dtype=torch.uint8, device="cuda")
-        if kind.startswith("quantize"):
+        if kind in ("quantize", "quantize_uncal", "quantize_uint8"):
             self.src = []
             for _ in range(self.NBUF):
                 x = torch.randn(n, device="cuda", generator=g)
@@ -225,6 +231,53 @@ class CastWorkload:
             self.kernel = "concat_kernel"
             self.name = "quantized_concat of two int8 halves, ranges (-1,1) and (-2,2): " \
                         "one half rescaled, one copied"
+        elif kind == "elemwise_mul_int8":
+            self.src = [torch.randint(-127, 128, (n,), device="cuda", generator=g,
+                                      dtype=torch.int8) for _ in range(self.NBUF)]
+            self.rhs = [torch.randint(-127, 128, (n,), device="cuda", generator=g,
+                                      dtype=torch.int8) for _ in range(self.NBUF)]
+            self.dst = [torch.empty(n, dtype=torch.int8, device="cuda") for _ in range(self.NBUF)]
+            self.imin = torch.tensor([-3.0], device="cuda")
+            self.imax = torch.tensor([3.0], device="cuda")
+            self.bytes = 3.0 * n
+            self.kernel = "mul_kernel"
+            self.name = "quantized_elemwise_mul int8*int8->int8 calibrated (-9,9)"
+        elif kind == "quantize_asym":
+            self.src = [torch.randn(n, device="cuda", generator=g) for _ in range(self.NBUF)]
+            self.dst = [torch.empty(n, dtype=torch.uint8, device="cuda")
+                        for _ in range(self.NBUF)]
+            self.bytes = 5.0 * n
+            self.kernel = "quantize_asym_kernel"
+            self.name = "quantize_asym fp32->uint8 calibrated (-6,6)"
+        elif kind == "embedding":
+            # BERT-base vocabulary: 30522 rows of 768 int8; n / 768 token ids per launch
+            self.rows = n // 768
+            self.table = torch.randint(-127, 128, (30522, 768), device="cuda", generator=g,
+                                       dtype=torch.int8)
+            self.src = [torch.randint(0, 30522, (self.rows,), device="cuda", generator=g,
+                                      dtype=torch.int32) for _ in range(self.NBUF)]
+            self.dst = [torch.empty((self.rows, 768), dtype=torch.int8, device="cuda")
+                        for _ in range(self.NBUF)]
+            self.imin = torch.tensor([-1.0], device="cuda")
+            self.imax = torch.tensor([1.0], device="cuda")
+            # the gathered rows are read once each (the 23 MB table stays in cache) and
+            # written once, plus 4 bytes of index per row
+            self.bytes = (2.0 * 768 + 4.0) * self.rows
+            self.kernel = "embedding_kernel"
+            self.name = "quantized_embedding, 30522 x 768 int8 table, %d int32 ids" % self.rows
+        elif kind == "transpose":
+            # attention layout change (batch, seq, heads, 64) -> (batch, heads, seq, 64)
+            self.shape = (n // (512 * 16 * 64), 512, 16, 64)
+            self.src = [torch.randint(-127, 128, self.shape, device="cuda", generator=g,
+                                      dtype=torch.int8) for _ in range(self.NBUF)]
+            self.dst = [torch.empty(n, dtype=torch.int8, device="cuda") for _ in range(self.NBUF)]
+            self.imin = torch.tensor([-1.0], device="cuda")
+            self.imax = torch.tensor([1.0], device="cuda")
+            self.c_shape = (ctypes.c_int64 * 4)(*self.shape)
+            self.c_axes = (ctypes.c_int * 4)(0, 2, 1, 3)
+            self.bytes = 2.0 * n
+            self.kernel = "permute_elem_kernel"
+            self.name = "quantized_transpose int8 %s axes (0,2,1,3)" % (self.shape,)
         else:
             raise ValueError(kind)
         self.name += ", %d elements" % n
@@ -268,6 +321,22 @@ class CastWorkload:
                                                 P(self.imin), P(self.imax), P(self.imin),
                                                 P(self.imax), P(self.dst[k]), 5, P(self.omin),
                                                 P(self.omax), n, 1, -5.0, 5.0)
+        elif kind == "elemwise_mul_int8":
+            rc = lib.mxq_quantized_elemwise_mul(st, P(self.src[k]), P(self.rhs[k]), P(self.imin),
+                                                P(self.imax), P(self.imin), P(self.imax),
+                                                P(self.dst[k]), 5, P(self.omin), P(self.omax), n,
+                                                1, -9.0, 9.0)
+        elif kind == "quantize_asym":
+            rc = lib.mxq_quantize_asym(st, P(self.src[k]), 0, P(self.dst[k]), P(self.omin),
+                                       P(self.omax), n, 1, -6.0, 6.0, None, 0)
+        elif kind == "embedding":
+            rc = lib.mxq_quantized_embedding(st, P(self.src[k]), 4, P(self.table), P(self.imin),
+                                             P(self.imax), P(self.dst[k]), P(self.omin),
+                                             P(self.omax), self.rows, 30522, 768)
+        elif kind == "transpose":
+            rc = lib.mxq_quantized_transpose(st, P(self.src[k]), P(self.imin), P(self.imax),
+                                             P(self.dst[k]), P(self.omin), P(self.omax), 4,
+                                             self.c_shape, self.c_axes)
         else:
             rc = lib.mxq_dequantize(st, P(self.src[k]), 5, P(self.imin), P(self.imax),
                                     P(self.dst[k]), n)
@@ -281,7 +350,14 @@ class CastWorkload:
         import numpy as np
         n = 1 << 24
         kind = self.kind
-        x = self.src[0][:n].cpu().numpy()
+        if kind == "embedding":
+            n = (n // 768) * 768
+            x = self.src[0][:n // 768].cpu().numpy()
+            table = self.table.cpu().numpy()
+        elif kind == "transpose":
+            x = self.src[0][:n // (512 * 16 * 64)].cpu().numpy()
+        else:
+            x = self.src[0][:n].cpu().numpy()
         reps, t0 = 0, time.perf_counter()
         while True:
             if kind == "quantize":
@@ -300,6 +376,14 @@ class CastWorkload:
                 oracle.quantized_elemwise_add(x, x, -3.0, 3.0, -3.0, 3.0)
             elif kind == "elemwise_add_int8":
                 oracle.quantized_elemwise_add(x, x, -3.0, 3.0, -3.0, 3.0, -5.0, 5.0)
+            elif kind == "elemwise_mul_int8":
+                oracle.quantized_elemwise_mul(x, x, -3.0, 3.0, -3.0, 3.0, -9.0, 9.0)
+            elif kind == "quantize_asym":
+                oracle.quantize_asym(x, -6.0, 6.0)
+            elif kind == "embedding":
+                oracle.quantized_embedding(x, table, -1.0, 1.0)
+            elif kind == "transpose":
+                oracle.quantized_transpose(x, -1.0, 1.0, (0, 2, 1, 3))
             else:
                 oracle.dequantize(x, -3.0, 3.0)
             reps += 1
@@ -738,7 +822,8 @@ def main():
         rows = []
         for kind in ["quantize", "quantize_uint8", "quantize_uncal", "requantize",
                      "requantize_uncal", "dequantize", "elemwise_add", "elemwise_add_int8",
-                     "concat", "maxpool", "avgpool", "fc8192",
+                     "concat", "elemwise_mul_int8", "quantize_asym", "embedding", "transpose",
+                     "maxpool", "avgpool", "fc8192",
                      "resnet50_convs", "bert_fc_chain", "bert_fc_chain_fused"]:
             if kind == args.workload:
                 continue

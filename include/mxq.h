@@ -31,9 +31,11 @@ extern "C" {
 
 /* element type codes = mshadow::TypeFlag (3rdparty/mshadow/mshadow/base.h:351-364) */
 #define MXQ_FLOAT32 0
+#define MXQ_FLOAT64 1
 #define MXQ_UINT8 3
 #define MXQ_INT32 4
 #define MXQ_INT8 5
+#define MXQ_INT64 6
 
 /* Last error message of the calling thread ("" if none). */
 const char* mxq_last_error(void);
@@ -135,6 +137,63 @@ int mxq_quantized_elemwise_add(void* stream, const void* lhs, int lhs_type, cons
                                const float* rhs_min, const float* rhs_max, void* out, int out_type,
                                float* omin, float* omax, size_t n, int calibrated,
                                float min_calib, float max_calib);
+
+/* ---- _contrib_quantized_elemwise_mul ---------------------------------------------
+ * Replaces QuantizedElemwiseMulOpForward
+ * (src/operator/quantization/quantized_elemwise_mul.cc:114-206; registered for cpu only,
+ * :232) for int8 operands of one shape: out[i] = (out_type)(lhs[i] * rhs[i] * out_scale),
+ * the int product converted to binary32, multiplied, truncated.
+ *   out_type MXQ_INT32 (uncalibrated): out_scale = 1, range from
+ *     QuantizationRangeForMultiplication<int8,int8,int32> (quantization_utils.h:141-170);
+ *   out_type MXQ_INT8 (calibrated): out_scale = (127.5 / MaxAbs(calib)) / lhs_scale /
+ *     rhs_scale with scale = 127.5 / MaxAbs(range), range (min_calib, max_calib);
+ *   out_type MXQ_FLOAT32 (enable_float_output): out_scale = 1 / lhs_scale / rhs_scale in
+ *     binary64, rounded once; omin / omax are not written and may be NULL.
+ * A calibrated product whose truncated value does not fit int8 is undefined in the
+ * reference; the low byte of the truncated int32 is stored (what its x86 build does). */
+int mxq_quantized_elemwise_mul(void* stream, const int8_t* lhs, const int8_t* rhs,
+                               const float* lhs_min, const float* lhs_max, const float* rhs_min,
+                               const float* rhs_max, void* out, int out_type, float* omin,
+                               float* omax, size_t n, int calibrated, float min_calib,
+                               float max_calib);
+
+/* ---- _contrib_quantized_embedding --------------------------------------------------
+ * Replaces QuantizedEmbeddingOpForward
+ * (src/operator/quantization/quantized_indexing_op.cc:103-122; cpu only, :146) and the
+ * TakeZeroAxisCPU<clip> kernel it launches (src/operator/tensor/indexing_op.cc:30-61):
+ * out[i, :] = weight[clip(int64(indices[i]), 0, input_dim - 1), :], int8 rows of output_dim
+ * bytes; the weight's range is passed through.  index_type is the mshadow type flag of
+ * `indices` (float32, float64, uint8, int32, int8 or int64). */
+int mxq_quantized_embedding(void* stream, const void* indices, int index_type,
+                            const int8_t* weight, const float* min_weight,
+                            const float* max_weight, int8_t* out, float* omin, float* omax,
+                            size_t n_indices, int64_t input_dim, int64_t output_dim);
+
+/* ---- _contrib_quantized_transpose --------------------------------------------------
+ * Replaces DNNLQuantizedTransposeForward
+ * (src/operator/quantization/dnnl/dnnl_quantized_transpose.cc; shapes and types
+ * quantized_transpose.cc:31-66; cpu only in the reference): out = in permuted so that out
+ * axis d is in axis axes[d] (axes == NULL reverses the axes, TransposeParam's default),
+ * one byte per element (int8 or uint8), ndim <= 8; the range is passed through.
+ * _contrib_quantized_reshape (quantized_reshape.cc:31-46) needs no entry point of its own:
+ * it is mxq_quantized_flatten's copy. */
+int mxq_quantized_transpose(void* stream, const void* in, const float* imin, const float* imax,
+                            void* out, float* omin, float* omax, int ndim,
+                            const int64_t* in_shape, const int* axes);
+
+/* ---- _contrib_quantize_asym ----------------------------------------------------------
+ * Replaces QuantizeAsymOp<gpu>::Forward
+ * (src/operator/quantization/quantize_asym-inl.h:78-160): float32 -> uint8 with
+ * scale = 255 / (max - min), shift = 255 - max * scale,
+ * out = (uint8)(in * scale + shift + 0.5) (the 0.5 in binary64), over (min_calib,
+ * max_calib) or, uncalibrated, the data's own min and max (workspace of
+ * mxq_quantize_asym_workspace(n) bytes, 16-byte aligned).  int8 input: out = in + 128,
+ * scale 1, shift 128; uint8 input: copied, scale 1, shift 0.  A value outside [0, 256) is
+ * undefined in the reference; the low byte of the truncated int32 is stored. */
+size_t mxq_quantize_asym_workspace(size_t n);
+int mxq_quantize_asym(void* stream, const void* in, int in_type, uint8_t* out, float* oscale,
+                      float* oshift, size_t n, int calibrated, float min_calib, float max_calib,
+                      void* workspace, size_t workspace_bytes);
 
 /* ---- _contrib_quantized_concat -----------------------------------------------------
  * Replaces DNNLQuantizedConcatForward

@@ -8,7 +8,7 @@ CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libmxq_hip.so")
 
 HIP_SOURCES = ["mxq_capi.hip", "mxq_cast.hip", "mxq_fc.hip", "mxq_conv.hip", "mxq_pool.hip",
-               "mxq_eltwise.hip"]
+               "mxq_eltwise.hip", "mxq_layout.hip"]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950",
@@ -77,7 +77,8 @@ def build_probe(verbose=False):
 
 
 OPS_LIB = os.path.join(HERE, "libmxq_ops.so")
-HOST_SOURCES = ["mxq_registry.cc", "mxq_quantization_ops.cc", "mxq_float_ops.cc", "mxq_graph.cc",
+HOST_SOURCES = ["mxq_registry.cc", "mxq_quantization_ops.cc", "mxq_quantized_tensor_ops.cc",
+                "mxq_float_ops.cc", "mxq_graph.cc",
                 "mxq_quantize_graph_pass.cc", "mxq_calibrate.cc", "mxq_ndarray_io.cc",
                 "mxq_harness.cc"]
 

@@ -79,3 +79,31 @@ def quantized_concat(*data, num_args=None, dim=1):
     if num_args is None:
         num_args = len(data) // 3
     return invoke("_contrib_quantized_concat", *data, num_args=num_args, dim=dim)
+
+
+def quantized_elemwise_mul(lhs, rhs, lhs_min, lhs_max, rhs_min, rhs_max, min_calib_range=None,
+                           max_calib_range=None, enable_float_output=False):
+    return invoke("_contrib_quantized_elemwise_mul", lhs, rhs, lhs_min, lhs_max, rhs_min,
+                  rhs_max, min_calib_range=min_calib_range, max_calib_range=max_calib_range,
+                  enable_float_output=enable_float_output)
+
+
+def quantized_embedding(data, weight, min_weight, max_weight, input_dim=None, output_dim=None,
+                        dtype="float32", sparse_grad=False):
+    return invoke("_contrib_quantized_embedding", data, weight, min_weight, max_weight,
+                  input_dim=input_dim, output_dim=output_dim, dtype=dtype,
+                  sparse_grad=sparse_grad)
+
+
+def quantized_reshape(data, min_data, max_data, shape=(), reverse=False):
+    return invoke("_contrib_quantized_reshape", data, min_data, max_data, shape=shape,
+                  reverse=reverse)
+
+
+def quantized_transpose(data, min_data, max_data, axes=()):
+    return invoke("_contrib_quantized_transpose", data, min_data, max_data, axes=axes)
+
+
+def quantize_asym(data, min_calib_range=None, max_calib_range=None):
+    return invoke("_contrib_quantize_asym", data, min_calib_range=min_calib_range,
+                  max_calib_range=max_calib_range)

@@ -207,5 +207,71 @@ NNVM_REGISTER_OP(Concat)
       return QuantizedTwin(attrs, "_contrib_quantized_concat");
     });
 
+// src/operator/tensor/elemwise_binary_op_basic.cc:236-263, quantized_elemwise_mul.cc:247-256.
+// Like the three operators after it, it registers no output names: its output is spelled
+// "<name>_0" in calibration keys (common::GetOutputName, src/common/utils.h), and so is the
+// quantized twin's, which is how the two meet in the calibration table.
+NNVM_REGISTER_OP(elemwise_mul)
+    .add_alias("_mul")
+    .add_alias("_Mul")
+    .set_num_inputs(2)
+    .set_num_outputs(1)
+    .set_attr<nnvm::FListInputNames>("FListInputNames",
+                                     [](const NodeAttrs&) {
+                                       return std::vector<std::string>{"lhs", "rhs"};
+                                     })
+    .set_attr<FQuantizedOp>("FQuantizedOp", [](const NodeAttrs& attrs) {
+      return QuantizedTwin(attrs, "_contrib_quantized_elemwise_mul");
+    });
+
+// src/operator/tensor/indexing_op.cc:565-650, quantized_indexing_op.cc:162-190: float32
+// tables only; the indices (input 0) are never quantized
+NNVM_REGISTER_OP(Embedding)
+    .set_num_inputs(2)
+    .set_num_outputs(1)
+    .set_attr_parser(ParamParser<EmbeddingParam>)
+    .set_attr<nnvm::FListInputNames>("FListInputNames",
+                                     [](const NodeAttrs&) {
+                                       return std::vector<std::string>{"data", "weight"};
+                                     })
+    .set_attr<FQuantizable>("FQuantizable",
+                            [](const NodeAttrs&) { return QuantizeType::kSupport; })
+    .set_attr<FQuantizedOp>("FQuantizedOp",
+                            [](const NodeAttrs& attrs) {
+                              EmbeddingParam param;
+                              param.Init(attrs.dict);
+                              if (param.dtype == mshadow::kFloat32)
+                                return QuantizedTwin(attrs, "_contrib_quantized_embedding");
+                              nnvm::ObjectPtr node = nnvm::Node::Create();
+                              node->attrs.op = nnvm::Op::Get("Embedding");
+                              node->attrs.name = attrs.name;
+                              node->attrs.dict = attrs.dict;
+                              if (node->op()->attr_parser) node->op()->attr_parser(&(node->attrs));
+                              return node;
+                            })
+    .set_attr<FAvoidQuantizeInput>("FAvoidQuantizeInput",
+                                   [](const NodeAttrs&, const size_t index, const std::string) {
+                                     return index == 0;
+                                   });
+
+// src/operator/tensor/matrix_op.cc:110-190, quantized_reshape.cc:119-127
+NNVM_REGISTER_OP(Reshape)
+    .add_alias("reshape")
+    .set_num_inputs(1)
+    .set_num_outputs(1)
+    .set_attr_parser(ParamParser<ReshapeParam>)
+    .set_attr<FQuantizedOp>("FQuantizedOp", [](const NodeAttrs& attrs) {
+      return QuantizedTwin(attrs, "_contrib_quantized_reshape");
+    });
+
+// src/operator/tensor/matrix_op.cc:292-350, quantized_transpose.cc:106-115
+NNVM_REGISTER_OP(transpose)
+    .set_num_inputs(1)
+    .set_num_outputs(1)
+    .set_attr_parser(ParamParser<TransposeParam>)
+    .set_attr<FQuantizedOp>("FQuantizedOp", [](const NodeAttrs& attrs) {
+      return QuantizedTwin(attrs, "_contrib_quantized_transpose");
+    });
+
 }  // namespace op
 }  // namespace mxnet

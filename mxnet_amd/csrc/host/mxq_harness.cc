@@ -181,7 +181,7 @@ int mxq_node_forward(void* node, void* stream, int dev_id, int num_in, const mxq
   const nnvm::Op* op = n->attrs.op;
   if (num_in != static_cast<int>(op->NumInputs(n->attrs)))
     throw dmlc::Error("wrong number of inputs for " + op->name);
-  if (num_out != static_cast<int>(op->num_outputs))
+  if (num_out != static_cast<int>(op->NumOutputs(n->attrs)))
     throw dmlc::Error("wrong number of outputs for " + op->name);
   std::vector<mxnet::TBlob> ins, outs;
   mxnet::ShapeVector in_shapes;

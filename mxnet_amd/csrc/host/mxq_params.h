@@ -12,6 +12,11 @@
 //                          src/operator/nn/pooling.cc:35-64)
 //   QuantizeElemwiseAddParam  src/operator/quantization/quantized_elemwise_add-inl.h:34-51
 //   ConcatParam            src/operator/nn/concat-inl.h:48-64
+//   QuantizeElemwiseMulParam  src/operator/quantization/quantized_elemwise_mul-inl.h:33-55
+//   EmbeddingParam         src/operator/tensor/indexing_op.h:66-96
+//   ReshapeParam           src/operator/tensor/matrix_op-inl.h:53-80
+//   TransposeParam         src/operator/tensor/matrix_op-inl.h:269-280
+//   QuantizeAsymParam      src/operator/quantization/quantize_asym-inl.h:41-59
 // Same field names, defaults, enum strings and error behaviour (unknown keys are
 // errors unless they look like __hidden__ keys).
 #ifndef MXQ_PARAMS_H_
@@ -537,6 +542,122 @@ struct ConcatParam {
   static std::vector<nnvm::ParamFieldInfo> __FIELDS__() {
     return {{"num_args", "int, required", "Number of inputs to be concated."},
             {"dim", "int or None, optional, default='1'", "the dimension to be concated."}};
+  }
+};
+
+struct QuantizeElemwiseMulParam {
+  dmlc::optional<float> min_calib_range;
+  dmlc::optional<float> max_calib_range;
+  bool enable_float_output = false;
+  void Init(const param_detail::Dict& d) {
+    using namespace param_detail;
+    check_unknown(d, {"min_calib_range", "max_calib_range", "enable_float_output"},
+                  "QuantizeElemwiseMulParam");
+    min_calib_range = get_optional_float(d, "min_calib_range");
+    max_calib_range = get_optional_float(d, "max_calib_range");
+    enable_float_output = get_bool(d, "enable_float_output", false);
+  }
+  static std::vector<nnvm::ParamFieldInfo> __FIELDS__() {
+    return {{"min_calib_range", "float or None, optional, default=None",
+             "The minimum scalar value in the form of float32 obtained through calibration. If "
+             "present, it will be used to requantize the int8 output data."},
+            {"max_calib_range", "float or None, optional, default=None",
+             "The maximum scalar value in the form of float32 obtained through calibration. If "
+             "present, it will be used to requantize the int8 output data."},
+            {"enable_float_output", "boolean, optional, default=0",
+             "Whether to enable float32 output"}};
+  }
+};
+
+struct QuantizeAsymParam {
+  dmlc::optional<float> min_calib_range;
+  dmlc::optional<float> max_calib_range;
+  void Init(const param_detail::Dict& d) {
+    using namespace param_detail;
+    check_unknown(d, {"min_calib_range", "max_calib_range"}, "QuantizeAsymParam");
+    min_calib_range = get_optional_float(d, "min_calib_range");
+    max_calib_range = get_optional_float(d, "max_calib_range");
+  }
+  static std::vector<nnvm::ParamFieldInfo> __FIELDS__() {
+    return {{"min_calib_range", "float or None, optional, default=None",
+             "The minimum scalar value in the form of float32. If present, it will be used to "
+             "quantize the fp32 data."},
+            {"max_calib_range", "float or None, optional, default=None",
+             "The maximum scalar value in the form of float32. If present, it will be used to "
+             "quantize the fp32 data."}};
+  }
+};
+
+static const std::vector<std::pair<std::string, int>> kAllTypeNames = {
+    {"bfloat16", 12}, {"float16", mshadow::kFloat16}, {"float32", mshadow::kFloat32},
+    {"float64", mshadow::kFloat64}, {"int32", mshadow::kInt32}, {"int64", mshadow::kInt64},
+    {"int8", mshadow::kInt8}, {"uint8", mshadow::kUint8}};
+
+struct EmbeddingParam {
+  index_t input_dim = 0;
+  index_t output_dim = 0;
+  int dtype = mshadow::kFloat32;
+  bool sparse_grad = false;
+  void Init(const param_detail::Dict& d) {
+    using namespace param_detail;
+    check_unknown(d, {"input_dim", "output_dim", "dtype", "sparse_grad"}, "EmbeddingParam");
+    input_dim = get_int(d, "input_dim", false, 0, true, 1);
+    output_dim = get_int(d, "output_dim", false, 0, true, 1);
+    dtype = get_enum(d, "dtype", kAllTypeNames, true, mshadow::kFloat32);
+    sparse_grad = get_bool(d, "sparse_grad", false);
+  }
+  static std::vector<nnvm::ParamFieldInfo> __FIELDS__() {
+    return {{"input_dim", "long, required", "Vocabulary size of the input indices."},
+            {"output_dim", "long, required", "Dimension of the embedding vectors."},
+            {"dtype",
+             "{'bfloat16', 'float16', 'float32', 'float64', 'int32', 'int64', 'int8', "
+             "'uint8'},optional, default='float32'",
+             "Data type of weight."},
+            {"sparse_grad", "boolean, optional, default=0",
+             "Compute row sparse gradient in the backward calculation. If set to True, the "
+             "grad's storage type is row_sparse."}};
+  }
+};
+
+struct ReshapeParam {
+  TShape target_shape = TShape(0, -1);  // deprecated form; ndim 0 = not given
+  bool keep_highest = false;
+  TShape shape = TShape(0, -1);         // with the special values 0, -1, -2, -3, -4
+  bool reverse = false;
+  void Init(const param_detail::Dict& d) {
+    using namespace param_detail;
+    check_unknown(d, {"shape", "reverse", "target_shape", "keep_highest"}, "ReshapeParam");
+    shape = get_shape(d, "shape", true);
+    if (shape.ndim() < 0) shape = TShape(0, -1);
+    reverse = get_bool(d, "reverse", false);
+    target_shape = get_shape(d, "target_shape", true);
+    if (target_shape.ndim() < 0) target_shape = TShape(0, -1);
+    keep_highest = get_bool(d, "keep_highest", false);
+  }
+  static std::vector<nnvm::ParamFieldInfo> __FIELDS__() {
+    return {{"shape", "Shape(tuple), optional, default=[]", "The target shape"},
+            {"reverse", "boolean, optional, default=0",
+             "If true then the special values are inferred from right to left"},
+            {"target_shape", "Shape(tuple), optional, default=[]",
+             "(Deprecated! Use ``shape`` instead.) Target new shape. One and only one dim can "
+             "be 0, in which case it will be inferred from the rest of dims"},
+            {"keep_highest", "boolean, optional, default=0",
+             "(Deprecated! Use ``shape`` instead.) Whether keep the highest dim unchanged.If set "
+             "to true, then the first dim in target_shape is ignored,and always fixed as input"}};
+  }
+};
+
+struct TransposeParam {
+  TShape axes = TShape(0, -1);
+  void Init(const param_detail::Dict& d) {
+    using namespace param_detail;
+    check_unknown(d, {"axes"}, "TransposeParam");
+    axes = get_shape(d, "axes", true);
+    if (axes.ndim() < 0) axes = TShape(0, -1);
+  }
+  static std::vector<nnvm::ParamFieldInfo> __FIELDS__() {
+    return {{"axes", "Shape(tuple), optional, default=[]",
+             "Target axis order. By default the axes will be inverted."}};
   }
 };
 

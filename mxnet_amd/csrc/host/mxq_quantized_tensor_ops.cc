@@ -1,0 +1,643 @@
+// Host side of the quantized operators that surround FC / conv in BERT-like and
+// embedding graphs, for the gpu device: attribute parsing, shape / type inference and
+// FCompute<gpu> functions under the reference's operator names.  As in
+// mxq_quantization_ops.cc every compute function only unpacks TBlobs and calls the C ABI
+// of libmxq_hip.so.
+//
+// Reference registrations this file mirrors (all under src/operator/quantization/):
+//   _contrib_quantized_elemwise_mul   quantized_elemwise_mul.cc:33-89,208-245
+//   _contrib_quantized_embedding      quantized_indexing_op.cc:30-73,124-160
+//   _contrib_quantized_reshape        quantized_reshape.cc:48-100, quantized_reshape-inl.h:38-68
+//   _contrib_quantized_transpose      quantized_transpose.cc:31-104
+//   _contrib_quantize_asym            quantize_asym.cc:36-157
+// The reference computes all five on the cpu only (quantize_asym also has a gpu class
+// but registers no gpu attribute); here they are attached as "<gpu>" attributes.
+#include <algorithm>
+#include <iostream>
+#include <string>
+#include <vector>
+
+#include "../../../include/mxq.h"
+#include "mxq_params.h"
+#include "mxq_shim.h"
+
+namespace mxnet {
+namespace op {
+
+using mshadow::gpu;
+
+namespace {
+
+inline void MXQ_CALL(int rc) {
+  if (rc != 0) throw dmlc::Error(std::string("libmxq_hip: ") + mxq_last_error());
+}
+
+inline void* raw_stream(const OpContext& ctx) {
+  mshadow::Stream<gpu>* s = ctx.get_stream<gpu>();
+  return s ? s->stream_ : nullptr;
+}
+
+const TShape kScalarShape{1};
+
+bool AllDefaultStorage(const NodeAttrs&, const int, DispatchMode* dispatch_mode,
+                       std::vector<int>* in_attrs, std::vector<int>* out_attrs) {
+  *dispatch_mode = DispatchMode::kFCompute;
+  for (auto& v : *in_attrs) v = kDefaultStorage;
+  for (auto& v : *out_attrs) v = kDefaultStorage;
+  return true;
+}
+
+std::vector<std::string> DataMinMax(const NodeAttrs&) { return {"data", "min_data", "max_data"}; }
+std::vector<std::string> OutputMinMax(const NodeAttrs&) {
+  return {"output", "min_output", "max_output"};
+}
+
+}  // namespace
+
+// ---- _contrib_quantized_elemwise_mul ------------------------------------------------------
+
+// quantized_elemwise_mul.cc:33-60
+static bool ElemwiseMulShape(const NodeAttrs& attrs, ShapeVector* in_attrs,
+                             ShapeVector* out_attrs) {
+  const auto& params = nnvm::get<QuantizeElemwiseMulParam>(attrs.parsed);
+  const TShape& lshape = (*in_attrs)[0];
+  const TShape& rshape = (*in_attrs)[1];
+  if (!ndim_is_known(lshape) || !ndim_is_known(rshape)) return false;
+  CHECK_EQ(lshape.ndim(), rshape.ndim())
+      << "Currently, quantized elemwise multiply doesn't support broadcast.";
+  for (int i = 0; i < lshape.ndim(); ++i) CHECK_EQ(lshape[i], rshape[i]);
+  for (int i = 2; i < 6; ++i) SHAPE_ASSIGN_CHECK(*in_attrs, i, kScalarShape);
+  SHAPE_ASSIGN_CHECK(*out_attrs, 0, lshape);
+  if (!params.enable_float_output) {
+    SHAPE_ASSIGN_CHECK(*out_attrs, 1, kScalarShape);
+    SHAPE_ASSIGN_CHECK(*out_attrs, 2, kScalarShape);
+  }
+  return true;
+}
+
+// quantized_elemwise_mul.cc:62-89
+static bool ElemwiseMulType(const NodeAttrs& attrs, std::vector<int>* in_type,
+                            std::vector<int>* out_type) {
+  const auto& params = nnvm::get<QuantizeElemwiseMulParam>(attrs.parsed);
+  for (int i = 0; i < 2; ++i) {
+    if (in_type->at(i) == mshadow::kInt8) {
+      TYPE_ASSIGN_CHECK(*in_type, i, mshadow::kInt8);
+    } else {
+      std::cerr << "currently, quantized elemwise mul only support int8 inputs." << std::endl;
+    }
+  }
+  for (int i = 2; i < 6; ++i) TYPE_ASSIGN_CHECK(*in_type, i, mshadow::kFloat32);
+  int dtype = mshadow::kInt32;
+  if (params.max_calib_range.has_value() && params.min_calib_range.has_value())
+    dtype = mshadow::kInt8;
+  if (!params.enable_float_output) {
+    TYPE_ASSIGN_CHECK(*out_type, 0, dtype);
+    TYPE_ASSIGN_CHECK(*out_type, 1, mshadow::kFloat32);
+    TYPE_ASSIGN_CHECK(*out_type, 2, mshadow::kFloat32);
+  } else {
+    TYPE_ASSIGN_CHECK(*out_type, 0, mshadow::kFloat32);
+  }
+  return true;
+}
+
+// quantized_elemwise_mul.cc:114-206
+static void QuantizedElemwiseMulForwardGPU(const NodeAttrs& attrs, const OpContext& ctx,
+                                           const std::vector<TBlob>& inputs,
+                                           const std::vector<OpReqType>&,
+                                           const std::vector<TBlob>& outputs) {
+  const auto& params = nnvm::get<QuantizeElemwiseMulParam>(attrs.parsed);
+  CHECK_EQ(inputs.size(), 6U);
+  CHECK_EQ(outputs.size(), params.enable_float_output ? 1U : 3U);
+  CHECK(inputs[0].type_flag_ == mshadow::kInt8 && inputs[1].type_flag_ == mshadow::kInt8)
+      << "lhs and rhs only support iny8 dtype.";
+  CHECK_EQ(inputs[0].Size(), inputs[1].Size());
+  const bool calibrated = params.max_calib_range.has_value() && params.min_calib_range.has_value();
+  MXQ_CALL(mxq_quantized_elemwise_mul(
+      raw_stream(ctx), inputs[0].dptr<int8_t>(), inputs[1].dptr<int8_t>(),
+      inputs[2].dptr<float>(), inputs[3].dptr<float>(), inputs[4].dptr<float>(),
+      inputs[5].dptr<float>(), outputs[0].dptr_, outputs[0].type_flag_,
+      params.enable_float_output ? nullptr : outputs[1].dptr<float>(),
+      params.enable_float_output ? nullptr : outputs[2].dptr<float>(), outputs[0].Size(),
+      calibrated ? 1 : 0, calibrated ? params.min_calib_range.value() : 0.f,
+      calibrated ? params.max_calib_range.value() : 0.f));
+}
+
+// ---- _contrib_quantized_embedding -----------------------------------------------------------
+
+// quantized_indexing_op.cc:30-52
+static bool QuantizedEmbeddingShape(const NodeAttrs& attrs, ShapeVector* in_attrs,
+                                    ShapeVector* out_attrs) {
+  const TShape& dshape = (*in_attrs)[0];
+  if (!ndim_is_known(dshape)) return false;
+  const EmbeddingParam& param = nnvm::get<EmbeddingParam>(attrs.parsed);
+  SHAPE_ASSIGN_CHECK(*in_attrs, 1, Shape2(param.input_dim, param.output_dim));
+  SHAPE_ASSIGN_CHECK(*in_attrs, 2, kScalarShape);
+  SHAPE_ASSIGN_CHECK(*in_attrs, 3, kScalarShape);
+  out_attrs->clear();
+  TShape oshape(dshape.ndim() + 1, -1);
+  for (int i = 0; i < dshape.ndim(); ++i) oshape[i] = dshape[i];
+  oshape[dshape.ndim()] = param.output_dim;
+  out_attrs->push_back(oshape);
+  out_attrs->push_back(kScalarShape);
+  out_attrs->push_back(kScalarShape);
+  return shape_is_known(oshape);
+}
+
+// quantized_indexing_op.cc:54-71 (the two range outputs are float32 = type flag 0)
+static bool QuantizedEmbeddingType(const NodeAttrs&, std::vector<int>* in_type,
+                                   std::vector<int>* out_type) {
+  CHECK_EQ(in_type->size(), 4U);
+  CHECK_GE(out_type->size(), 3U);
+  const int itype = (*in_type)[0];
+  CHECK_NE(itype, -1) << "First input must have specified type";
+  TYPE_ASSIGN_CHECK(*in_type, 1, mshadow::kInt8);
+  TYPE_ASSIGN_CHECK(*in_type, 2, mshadow::kFloat32);
+  TYPE_ASSIGN_CHECK(*in_type, 3, mshadow::kFloat32);
+  out_type->clear();
+  out_type->push_back(mshadow::kInt8);
+  out_type->push_back(mshadow::kFloat32);
+  out_type->push_back(mshadow::kFloat32);
+  return true;
+}
+
+// quantized_indexing_op.cc:103-122
+static void QuantizedEmbeddingForwardGPU(const NodeAttrs&, const OpContext& ctx,
+                                         const std::vector<TBlob>& inputs,
+                                         const std::vector<OpReqType>& req,
+                                         const std::vector<TBlob>& outputs) {
+  CHECK_EQ(req[0], kWriteTo);
+  CHECK_EQ(inputs.size(), 4U);
+  CHECK_EQ(outputs.size(), 3U);
+  CHECK_EQ(inputs[1].shape_.ndim(), 2)
+      << "Embedding layer expects its weight to be two-dimensional. " << inputs[1].shape_.ndim()
+      << " dimensional input is given instead";
+  CHECK_EQ(inputs[1].type_flag_, mshadow::kInt8);
+  const TShape& w = inputs[1].shape_;
+  MXQ_CALL(mxq_quantized_embedding(raw_stream(ctx), inputs[0].dptr_, inputs[0].type_flag_,
+                                   inputs[1].dptr<int8_t>(), inputs[2].dptr<float>(),
+                                   inputs[3].dptr<float>(), outputs[0].dptr<int8_t>(),
+                                   outputs[1].dptr<float>(), outputs[2].dptr<float>(),
+                                   inputs[0].Size(), w[0], w[1]));
+}
+
+// ---- _contrib_quantized_reshape -------------------------------------------------------------
+
+namespace {
+
+// matrix_op-inl.h:95-182: the special values of `shape`
+TShape InferReshapeShape(const TShape& shape, const TShape& dshape, bool reverse) {
+  std::vector<index_t> dshape_vec, param_shape_vec;
+  for (int i = 0; i < dshape.ndim(); ++i) dshape_vec.push_back(dshape[i]);
+  for (int i = 0; i < shape.ndim(); ++i) param_shape_vec.push_back(shape[i]);
+  std::vector<index_t> tmp;
+  size_t src_idx = 0;
+  int inf_idx = -1;
+  if (reverse) {
+    std::reverse(dshape_vec.begin(), dshape_vec.end());
+    std::reverse(param_shape_vec.begin(), param_shape_vec.end());
+  }
+  const size_t dshape_len = dshape_vec.size(), params_len = param_shape_vec.size();
+  for (size_t i = 0; i < params_len; ++i) {
+    const index_t proposed_dim = param_shape_vec[i];
+    if (proposed_dim == 0) {
+      CHECK_LT(src_idx, dshape_len);
+      tmp.push_back(dshape_vec[src_idx++]);
+    } else if (proposed_dim == -1) {
+      CHECK_LT(inf_idx, 0) << "One and only one dim can be inferred";
+      inf_idx = static_cast<int>(i);
+      tmp.push_back(1);
+      src_idx++;
+    } else if (proposed_dim == -2) {
+      while (src_idx < dshape_len) tmp.push_back(dshape_vec[src_idx++]);
+    } else if (proposed_dim == -3) {
+      CHECK_LT(src_idx, dshape_len - 1);
+      const index_t d1 = dshape_vec[src_idx++];
+      const index_t d2 = dshape_vec[src_idx++];
+      tmp.push_back((d1 < 0 || d2 < 0) ? -1 : d1 * d2);
+    } else if (proposed_dim == -4) {
+      CHECK_LT(i + 2, params_len);
+      CHECK_LT(src_idx, dshape_len);
+      const index_t d0 = dshape_vec[src_idx++];
+      index_t d1 = param_shape_vec[++i];
+      index_t d2 = param_shape_vec[++i];
+      CHECK(d1 != -1 || d2 != -1) << "Split dims cannot both be -1.";
+      if (d1 == -1 && d0 >= 0) d1 = d0 / d2;
+      if (d2 == -1 && d0 >= 0) d2 = d0 / d1;
+      CHECK(d1 * d2 == d0 || d0 == -1)
+          << "Split dims " << d1 << ", " << d2 << " do not divide original dim " << d0;
+      tmp.push_back(d1);
+      tmp.push_back(d2);
+    } else {
+      tmp.push_back(proposed_dim);
+      src_idx++;
+    }
+  }
+  if (inf_idx >= 0) {
+    if (shape_is_known(dshape)) {
+      index_t new_size = 1;
+      for (index_t x : tmp) new_size *= x;
+      tmp[inf_idx] = static_cast<index_t>(dshape.Size()) / new_size;
+    } else {
+      tmp[inf_idx] = -1;
+    }
+  }
+  if (reverse) std::reverse(tmp.begin(), tmp.end());
+  return TShape(tmp);
+}
+
+// matrix_op-inl.h:184-205
+bool ReverseReshapeInferShape(TShape* in, const TShape& out) {
+  if (shape_is_known(*in) && shape_is_known(out)) return true;
+  if (!shape_is_known(out)) return false;
+  int zero_axis = -1;
+  index_t known_dim_size_prod = 1;
+  for (int i = 0; i < in->ndim(); i++) {
+    if (!dim_size_is_known(*in, i)) {
+      if (zero_axis != -1) return false;
+      zero_axis = i;
+    } else {
+      known_dim_size_prod *= (*in)[i];
+    }
+  }
+  (*in)[zero_axis] = static_cast<index_t>(out.Size()) / known_dim_size_prod;
+  return true;
+}
+
+// matrix_op-inl.h:206-250
+bool ReshapeShape(const NodeAttrs& attrs, ShapeVector* in_attrs, ShapeVector* out_attrs) {
+  const ReshapeParam& param_ = nnvm::get<ReshapeParam>(attrs.parsed);
+  CHECK_EQ(in_attrs->size(), 1U) << "Input: [data]";
+  CHECK_EQ(out_attrs->size(), 1U);
+  TShape& dshape = (*in_attrs)[0];
+  if (!ndim_is_known(dshape)) return false;
+  TShape oshape;
+  if (param_.shape.ndim() != 0) {
+    oshape = InferReshapeShape(param_.shape, dshape, param_.reverse);
+  } else if (param_.target_shape.ndim() != 0) {
+    oshape = param_.target_shape;
+    int neg_count = 0;
+    int inf_idx = 0;
+    const int start_idx = param_.keep_highest ? 1 : 0;
+    if (param_.keep_highest) oshape[0] = dshape[0];
+    for (int i = start_idx; i < oshape.ndim(); ++i) {
+      if (oshape[i] == 0) {
+        neg_count++;
+        inf_idx = i;
+      }
+    }
+    if (neg_count == 1) {
+      oshape[inf_idx] = 1;
+      oshape[inf_idx] = static_cast<index_t>(dshape.Size() / oshape.Size());
+    }
+  } else {
+    return shape_is_known((*out_attrs)[0]) &&
+           ReverseReshapeInferShape(&(*in_attrs)[0], (*out_attrs)[0]);
+  }
+  ReverseReshapeInferShape(&dshape, oshape);
+  SHAPE_ASSIGN_CHECK(*out_attrs, 0, oshape);
+  return ReverseReshapeInferShape(&(*in_attrs)[0], (*out_attrs)[0]);
+}
+
+}  // namespace
+
+// quantized_reshape-inl.h:38-56
+static bool QuantizedReshapeShape(const NodeAttrs& attrs, ShapeVector* in_attrs,
+                                  ShapeVector* out_attrs) {
+  CHECK_EQ(in_attrs->size(), 3U);
+  CHECK_EQ(out_attrs->size(), 3U);
+  ShapeVector input = {in_attrs->at(0)};
+  ShapeVector output = {out_attrs->at(0)};
+  const bool ret = ReshapeShape(attrs, &input, &output);
+  SHAPE_ASSIGN_CHECK(*in_attrs, 1, kScalarShape);
+  SHAPE_ASSIGN_CHECK(*in_attrs, 2, kScalarShape);
+  SHAPE_ASSIGN_CHECK(*out_attrs, 0, output[0]);
+  SHAPE_ASSIGN_CHECK(*out_attrs, 1, kScalarShape);
+  SHAPE_ASSIGN_CHECK(*out_attrs, 2, kScalarShape);
+  return ret;
+}
+
+// quantized_reshape-inl.h:58-68 and quantized_transpose.cc:31-42: the data keeps its type
+static bool PassThroughType(const NodeAttrs&, std::vector<int>* in_attrs,
+                            std::vector<int>* out_attrs) {
+  CHECK_EQ(in_attrs->size(), 3U);
+  CHECK_EQ(out_attrs->size(), 3U);
+  TYPE_ASSIGN_CHECK(*in_attrs, 1, mshadow::kFloat32);
+  TYPE_ASSIGN_CHECK(*in_attrs, 2, mshadow::kFloat32);
+  TYPE_ASSIGN_CHECK(*out_attrs, 0, (*in_attrs)[0]);
+  TYPE_ASSIGN_CHECK(*out_attrs, 1, mshadow::kFloat32);
+  TYPE_ASSIGN_CHECK(*out_attrs, 2, mshadow::kFloat32);
+  return (*in_attrs)[0] != -1;
+}
+
+// quantized_reshape.cc:31-46: an identity copy unless the engine runs it in place
+static void QuantizedReshapeComputeGPU(const NodeAttrs&, const OpContext& ctx,
+                                       const std::vector<TBlob>& inputs,
+                                       const std::vector<OpReqType>& req,
+                                       const std::vector<TBlob>& outputs) {
+  CHECK_EQ(inputs.size(), 3U);
+  CHECK_EQ(outputs.size(), 3U);
+  CHECK_EQ(req.size(), 3U);
+  CHECK(inputs[0].type_flag_ == mshadow::kInt8 || inputs[0].type_flag_ == mshadow::kUint8)
+      << "quantized_reshape takes int8 or uint8 data";
+  CHECK_EQ(inputs[0].Size(), outputs[0].Size());
+  // in place: mxq_quantized_flatten copies nothing where in == out
+  MXQ_CALL(mxq_quantized_flatten(raw_stream(ctx), inputs[0].dptr_, inputs[1].dptr<float>(),
+                                 inputs[2].dptr<float>(),
+                                 req[0] == kWriteInplace ? inputs[0].dptr_ : outputs[0].dptr_,
+                                 outputs[1].dptr<float>(), outputs[2].dptr<float>(),
+                                 outputs[0].Size()));
+}
+
+// ---- _contrib_quantized_transpose -----------------------------------------------------------
+
+namespace {
+
+// matrix_op-inl.h:579-613
+bool TransposeShape(const NodeAttrs& attrs, ShapeVector* in_attrs, ShapeVector* out_attrs) {
+  const TransposeParam& param = nnvm::get<TransposeParam>(attrs.parsed);
+  CHECK_EQ(in_attrs->size(), 1U);
+  CHECK_EQ(out_attrs->size(), 1U);
+  TShape& shp = (*in_attrs)[0];
+  TShape& out_shp = (*out_attrs)[0];
+  if (!ndim_is_known(shp) && !ndim_is_known(out_shp)) return false;
+  if (out_shp.ndim() >= 0 && shp.ndim() >= 0) CHECK_EQ(out_shp.ndim(), shp.ndim());
+  const int nd = std::max(shp.ndim(), out_shp.ndim());
+  TShape get(nd, -1), ret(nd, -1);
+  if (param.axes.ndim() == 0) {
+    for (int i = 0; i < shp.ndim(); ++i) ret[i] = shp[shp.ndim() - 1 - i];
+    for (int i = 0; i < out_shp.ndim(); ++i) get[nd - 1 - i] = out_shp[i];
+  } else {
+    CHECK_EQ(nd, param.axes.ndim());
+    for (int i = 0; i < shp.ndim(); ++i) {
+      CHECK(param.axes[i] < static_cast<index_t>(shp.ndim()));
+      ret[i] = shp[static_cast<int>(param.axes[i])];
+    }
+    for (int i = 0; i < out_shp.ndim(); ++i) get[static_cast<int>(param.axes[i])] = out_shp[i];
+  }
+  SHAPE_ASSIGN_CHECK(*in_attrs, 0, get);
+  SHAPE_ASSIGN_CHECK(*out_attrs, 0, ret);
+  return shape_is_known(ret);
+}
+
+}  // namespace
+
+// quantized_transpose.cc:49-66
+static bool QuantizedTransposeShape(const NodeAttrs& attrs, ShapeVector* in_attrs,
+                                    ShapeVector* out_attrs) {
+  CHECK_EQ(in_attrs->size(), 3U);
+  CHECK_EQ(out_attrs->size(), 3U);
+  ShapeVector qin_attrs(1), qout_attrs(1);
+  SHAPE_ASSIGN_CHECK(qin_attrs, 0, (*in_attrs)[0]);
+  SHAPE_ASSIGN_CHECK(qout_attrs, 0, (*out_attrs)[0]);
+  const bool ret = TransposeShape(attrs, &qin_attrs, &qout_attrs);
+  SHAPE_ASSIGN_CHECK(*in_attrs, 0, qin_attrs[0]);
+  SHAPE_ASSIGN_CHECK(*out_attrs, 0, qout_attrs[0]);
+  SHAPE_ASSIGN_CHECK(*in_attrs, 1, kScalarShape);
+  SHAPE_ASSIGN_CHECK(*in_attrs, 2, kScalarShape);
+  SHAPE_ASSIGN_CHECK(*out_attrs, 1, kScalarShape);
+  SHAPE_ASSIGN_CHECK(*out_attrs, 2, kScalarShape);
+  return ret;
+}
+
+// dnnl_quantized_transpose.cc: the float transpose on one-byte elements, ranges copied
+static void QuantizedTransposeForwardGPU(const NodeAttrs& attrs, const OpContext& ctx,
+                                         const std::vector<TBlob>& inputs,
+                                         const std::vector<OpReqType>& req,
+                                         const std::vector<TBlob>& outputs) {
+  const TransposeParam& param = nnvm::get<TransposeParam>(attrs.parsed);
+  CHECK_EQ(inputs.size(), 3U);
+  CHECK_EQ(outputs.size(), 3U);
+  CHECK(req[0] == kWriteTo) << "Transpose does not support inplace";
+  CHECK(inputs[0].type_flag_ == mshadow::kInt8 || inputs[0].type_flag_ == mshadow::kUint8)
+      << "quantized_transpose takes int8 or uint8 data";
+  const TShape& shp = inputs[0].shape_;
+  std::vector<int64_t> dims(shp.ndim());
+  for (int i = 0; i < shp.ndim(); ++i) dims[i] = shp[i];
+  std::vector<int> axes(param.axes.ndim());
+  for (int i = 0; i < param.axes.ndim(); ++i) axes[i] = static_cast<int>(param.axes[i]);
+  if (!axes.empty()) CHECK_EQ(axes.size(), dims.size());
+  MXQ_CALL(mxq_quantized_transpose(raw_stream(ctx), inputs[0].dptr_, inputs[1].dptr<float>(),
+                                   inputs[2].dptr<float>(), outputs[0].dptr_,
+                                   outputs[1].dptr<float>(), outputs[2].dptr<float>(),
+                                   shp.ndim(), dims.data(), axes.empty() ? nullptr : axes.data()));
+}
+
+// ---- _contrib_quantize_asym -----------------------------------------------------------------
+
+// quantize_asym.cc:36-54
+static bool QuantizeAsymShape(const NodeAttrs&, ShapeVector* in_attrs, ShapeVector* out_attrs) {
+  CHECK_EQ(in_attrs->size(), 1U);
+  CHECK_EQ(out_attrs->size(), 3U);
+  TShape dshape = in_attrs->at(0);
+  SHAPE_ASSIGN_CHECK(*out_attrs, 0, dshape);
+  SHAPE_ASSIGN_CHECK(*out_attrs, 1, kScalarShape);
+  SHAPE_ASSIGN_CHECK(*out_attrs, 2, kScalarShape);
+  if (out_attrs->at(0).ndim() > 0) {
+    dshape[0] = out_attrs->at(0)[0];
+    SHAPE_ASSIGN_CHECK(*in_attrs, 0, dshape);
+  }
+  return !shape_is_none(out_attrs->at(0));
+}
+
+// quantize_asym.cc:56-69
+static bool QuantizeAsymType(const NodeAttrs&, std::vector<int>* in_attrs,
+                             std::vector<int>* out_attrs) {
+  CHECK_EQ(in_attrs->size(), 1U);
+  CHECK_EQ(out_attrs->size(), 3U);
+  CHECK_EQ(in_attrs->at(0), mshadow::kFloat32);
+  TYPE_ASSIGN_CHECK(*out_attrs, 0, mshadow::kUint8);
+  TYPE_ASSIGN_CHECK(*out_attrs, 1, mshadow::kFloat32);
+  TYPE_ASSIGN_CHECK(*out_attrs, 2, mshadow::kFloat32);
+  return out_attrs->at(0) != -1;
+}
+
+// quantize_asym-inl.h:78-160.  The operator state only carries the attributes.
+class QuantizeAsymOperatorGPU {
+ public:
+  explicit QuantizeAsymOperatorGPU(const NodeAttrs& attrs) : attrs_(attrs) {}
+  void Forward(const OpContext& ctx, const std::vector<TBlob>& inputs,
+               const std::vector<OpReqType>&, const std::vector<TBlob>& outputs) {
+    CHECK_EQ(outputs[0].type_flag_, mshadow::kUint8)
+        << "Asymmetric quantization only supports uint8 outputs.";
+    const auto& param = nnvm::get<QuantizeAsymParam>(attrs_.parsed);
+    const bool calibrated = param.min_calib_range.has_value() && param.max_calib_range.has_value();
+    void* ws = nullptr;
+    size_t ws_bytes = 0;
+    if (inputs[0].type_flag_ == mshadow::kFloat32 && !calibrated) {
+      CHECK(!ctx.requested.empty()) << "uncalibrated quantize_asym needs its temp space resource";
+      ws_bytes = mxq_quantize_asym_workspace(inputs[0].Size());
+      ws = ctx.requested[0].get_space(ws_bytes);
+    }
+    MXQ_CALL(mxq_quantize_asym(raw_stream(ctx), inputs[0].dptr_, inputs[0].type_flag_,
+                               outputs[0].dptr<uint8_t>(), outputs[1].dptr<float>(),
+                               outputs[2].dptr<float>(), inputs[0].Size(), calibrated ? 1 : 0,
+                               calibrated ? param.min_calib_range.value() : 0.f,
+                               calibrated ? param.max_calib_range.value() : 0.f, ws, ws_bytes));
+  }
+
+ private:
+  NodeAttrs attrs_;
+};
+
+static OpStatePtr CreateQuantizeAsymState(const NodeAttrs& attrs, Context ctx, const ShapeVector&,
+                                          const std::vector<int>&) {
+  CHECK(ctx.dev_type == Context::kGPU) << "this build only provides the gpu operator";
+  return OpStatePtr::Create<QuantizeAsymOperatorGPU>(attrs);
+}
+
+static void QuantizeAsymForwardGPU(const OpStatePtr& state, const OpContext& ctx,
+                                   const std::vector<TBlob>& inputs,
+                                   const std::vector<OpReqType>& req,
+                                   const std::vector<TBlob>& outputs) {
+  state.get_state<QuantizeAsymOperatorGPU>().Forward(ctx, inputs, req, outputs);
+}
+
+// Temp space of the operators of this file, in bytes (0 for all but the uncalibrated
+// asymmetric quantize).
+size_t MXQTensorOpsTempSpaceBytes(const NodeAttrs& attrs, const ShapeVector& in) {
+  if (attrs.op->name == "_contrib_quantize_asym") {
+    const auto& param = nnvm::get<QuantizeAsymParam>(attrs.parsed);
+    if (param.min_calib_range.has_value() && param.max_calib_range.has_value()) return 0;
+    return mxq_quantize_asym_workspace(in[0].Size());
+  }
+  return 0;
+}
+
+// ---- registration ---------------------------------------------------------------------------
+
+// quantized_elemwise_mul.cc:208-245
+NNVM_REGISTER_OP(_contrib_quantized_elemwise_mul)
+    .add_alias("_npx_quantized_elemwise_mul")
+    .describe("Multiplies arguments int8 element-wise.")
+    .set_num_inputs(6)
+    .set_num_outputs([](const NodeAttrs& attrs) {
+      return nnvm::get<QuantizeElemwiseMulParam>(attrs.parsed).enable_float_output ? 1U : 3U;
+    })
+    .set_attr_parser(ParamParser<QuantizeElemwiseMulParam>)
+    .set_attr<nnvm::FListInputNames>("FListInputNames",
+                                     [](const NodeAttrs&) {
+                                       return std::vector<std::string>{"lhs",     "rhs",
+                                                                       "lhs_min", "lhs_max",
+                                                                       "rhs_min", "rhs_max"};
+                                     })
+    .set_attr<mxnet::FInferShape>("FInferShape", ElemwiseMulShape)
+    .set_attr<nnvm::FInferType>("FInferType", ElemwiseMulType)
+    .set_attr<FInferStorageType>("FInferStorageType", AllDefaultStorage)
+    .set_attr<FCompute>("FCompute<gpu>", QuantizedElemwiseMulForwardGPU)
+    .set_attr<FNeedRequantize>("FNeedRequantize", [](const NodeAttrs&) { return true; })
+    .add_argument("lhs", "NDArray-or-Symbol", "first input")
+    .add_argument("rhs", "NDArray-or-Symbol", "second input")
+    .add_argument("lhs_min", "NDArray-or-Symbol", "Minimum value of first input.")
+    .add_argument("lhs_max", "NDArray-or-Symbol", "Maximum value of first input.")
+    .add_argument("rhs_min", "NDArray-or-Symbol", "Minimum value of second input.")
+    .add_argument("rhs_max", "NDArray-or-Symbol", "Maximum value of second input.")
+    .add_arguments(QuantizeElemwiseMulParam::__FIELDS__());
+
+// quantized_indexing_op.cc:124-160
+NNVM_REGISTER_OP(_contrib_quantized_embedding)
+    .add_alias("_npx_quantized_embedding")
+    .describe("Maps integer indices to int8 vector representations (embeddings).")
+    .set_num_inputs(4)
+    .set_num_outputs(3)
+    .set_attr_parser(ParamParser<EmbeddingParam>)
+    .set_attr<nnvm::FListInputNames>("FListInputNames",
+                                     [](const NodeAttrs&) {
+                                       return std::vector<std::string>{"data", "weight",
+                                                                       "min_weight",
+                                                                       "max_weight"};
+                                     })
+    .set_attr<nnvm::FListOutputNames>("FListOutputNames", OutputMinMax)
+    .set_attr<mxnet::FInferShape>("FInferShape", QuantizedEmbeddingShape)
+    .set_attr<nnvm::FInferType>("FInferType", QuantizedEmbeddingType)
+    .set_attr<FInferStorageType>("FInferStorageType", AllDefaultStorage)
+    .set_attr<FCompute>("FCompute<gpu>", QuantizedEmbeddingForwardGPU)
+    .add_argument("data", "NDArray-or-Symbol", "The input array to the embedding operator.")
+    .add_argument("weight", "NDArray-or-Symbol", "The embedding weight matrix.")
+    .add_argument("min_weight", "NDArray-or-Symbol", "Minimum value of data.")
+    .add_argument("max_weight", "NDArray-or-Symbol", "Maximum value of data.")
+    .add_arguments(EmbeddingParam::__FIELDS__());
+
+// quantized_reshape.cc:48-100
+NNVM_REGISTER_OP(_contrib_quantized_reshape)
+    .add_alias("quantized_reshape")
+    .set_num_inputs(3)
+    .set_num_outputs(3)
+    .set_attr_parser(ParamParser<ReshapeParam>)
+    .set_attr<nnvm::FListInputNames>("FListInputNames", DataMinMax)
+    .set_attr<nnvm::FListOutputNames>("FListOutputNames", OutputMinMax)
+    .set_attr<nnvm::FInplaceOption>("FInplaceOption",
+                                    [](const NodeAttrs&) {
+                                      return std::vector<std::pair<int, int>>{{0, 0}, {1, 1}, {2, 2}};
+                                    })
+    .set_attr<mxnet::FInferShape>("FInferShape", QuantizedReshapeShape)
+    .set_attr<nnvm::FInferType>("FInferType", PassThroughType)
+    .set_attr<FCompute>("FCompute<gpu>", QuantizedReshapeComputeGPU)
+    .set_attr<FQuantizable>("FQuantizable",
+                            [](const NodeAttrs&) { return QuantizeType::kSupport; })
+    .add_argument("data", "NDArray-or-Symbol", "Array to be reshaped.")
+    .add_argument("min_data", "NDArray-or-Symbol",
+                  "The minimum scalar value possibly produced for the data")
+    .add_argument("max_data", "NDArray-or-Symbol",
+                  "The maximum scalar value possibly produced for the data")
+    .add_arguments(ReshapeParam::__FIELDS__());
+
+// quantized_transpose.cc:68-104
+NNVM_REGISTER_OP(_contrib_quantized_transpose)
+    .add_alias("quantized_transpose")
+    .set_num_inputs(3)
+    .set_num_outputs(3)
+    .set_attr_parser(ParamParser<TransposeParam>)
+    .set_attr<nnvm::FListInputNames>("FListInputNames", DataMinMax)
+    .set_attr<nnvm::FListOutputNames>("FListOutputNames", OutputMinMax)
+    .set_attr<mxnet::FInferShape>("FInferShape", QuantizedTransposeShape)
+    .set_attr<nnvm::FInferType>("FInferType", PassThroughType)
+    .set_attr<FCompute>("FCompute<gpu>", QuantizedTransposeForwardGPU)
+    .set_attr<FQuantizable>("FQuantizable",
+                            [](const NodeAttrs&) { return QuantizeType::kSupport; })
+    .add_argument("data", "NDArray-or-Symbol", "Array to be transposed.")
+    .add_argument("min_data", "NDArray-or-Symbol",
+                  "The minimum scalar value possibly produced for the data")
+    .add_argument("max_data", "NDArray-or-Symbol",
+                  "The maximum scalar value possibly produced for the data")
+    .add_arguments(TransposeParam::__FIELDS__());
+
+// quantize_asym.cc:100-157
+NNVM_REGISTER_OP(_contrib_quantize_asym)
+    .describe("Quantize a input tensor from float to uint8_t.  Output `scale` and `shift` are "
+              "scalar floats that specify the quantization parameters for the input data: "
+              "`out[i] = in[i] * scale + shift + 0.5` with `scale = uint8_range / (max_range - "
+              "min_range)` and `shift = numeric_limits<T>::max - max_range * scale`.")
+    .set_attr_parser(ParamParser<QuantizeAsymParam>)
+    .set_num_inputs(1)
+    .set_num_outputs(3)
+    .set_attr<nnvm::FListInputNames>("FListInputNames",
+                                     [](const NodeAttrs&) {
+                                       return std::vector<std::string>{"data"};
+                                     })
+    .set_attr<nnvm::FListOutputNames>("FListOutputNames",
+                                      [](const NodeAttrs&) {
+                                        return std::vector<std::string>{"output", "scale",
+                                                                        "shift"};
+                                      })
+    .set_attr<mxnet::FInferShape>("FInferShape", QuantizeAsymShape)
+    .set_attr<nnvm::FInferType>("FInferType", QuantizeAsymType)
+    .set_attr<FInferStorageType>("FInferStorageType", AllDefaultStorage)
+    .set_attr<FCreateOpState>("FCreateOpState", CreateQuantizeAsymState)
+    .set_attr<FStatefulCompute>("FStatefulCompute<gpu>", QuantizeAsymForwardGPU)
+    .set_attr<FNeedCalibrateInput>("FNeedCalibrateInput",
+                                   [](const NodeAttrs&) { return std::vector<int>{0}; })
+    .set_attr<FResourceRequest>("FResourceRequest",
+                                [](const NodeAttrs& attrs) {
+                                  const auto& param =
+                                      nnvm::get<QuantizeAsymParam>(attrs.parsed);
+                                  if (param.max_calib_range.has_value() &&
+                                      param.min_calib_range.has_value())
+                                    return std::vector<ResourceRequest>();
+                                  return std::vector<ResourceRequest>(
+                                      1, ResourceRequest::kTempSpace);
+                                })
+    .add_argument("data", "NDArray-or-Symbol", "A ndarray/symbol of type `float32`")
+    .add_arguments(QuantizeAsymParam::__FIELDS__());
+
+}  // namespace op
+}  // namespace mxnet

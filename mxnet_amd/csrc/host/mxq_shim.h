@@ -66,6 +66,9 @@ class optional {
 #define CHECK(cond) \
   if (!(cond)) ::mxq_shim::FatalStream(__FILE__, __LINE__).stream() << "Check failed: " #cond " "
 #define CHECK_EQ(a, b) CHECK((a) == (b)) << "(" << (a) << " vs. " << (b) << ") "
+#define CHECK_NE(a, b) CHECK((a) != (b)) << "(" << (a) << " vs. " << (b) << ") "
+#define CHECK_LT(a, b) CHECK((a) < (b)) << "(" << (a) << " vs. " << (b) << ") "
+#define CHECK_GE(a, b) CHECK((a) >= (b)) << "(" << (a) << " vs. " << (b) << ") "
 #define LOG_FATAL ::mxq_shim::FatalStream(__FILE__, __LINE__).stream()
 
 namespace mxq_shim {

@@ -102,6 +102,17 @@ struct QuantU8 {
   __device__ __forceinline__ int operator()(float x) const { return quant_u8(x, lo, s); }
 };
 
+// static_cast<uint8_t>(x * scale + shift + 0.5) with the 0.5 a double
+// (quantize_asym-inl.h:62-76).  Outside [0, 256) that conversion is undefined in the
+// reference; here the low byte of the truncated int32 is kept, as its x86 build does.
+struct QuantAsym {
+  float scale, shift;
+  __device__ __forceinline__ int operator()(float x) const {
+    const float t = x * scale + shift;
+    return static_cast<int>(static_cast<double>(t) + 0.5);
+  }
+};
+
 __device__ __forceinline__ float to_float(float x) { return x; }
 __device__ __forceinline__ float to_float(int32_t x) { return static_cast<float>(x); }
 
@@ -306,6 +317,58 @@ __global__ __launch_bounds__(kThreads) void quantize_kernel(const float* __restr
       *omin = -r;
       *omax = r;
     }
+  }
+}
+
+// ---- asymmetric quantize (float -> uint8 over [min, max]) ---------------------------
+// scale = 255 / (max - min), shift = 255 - max * scale (quantize_asym-inl.h:103-152); the
+// range is (lo, hi) by value or the reduction partials.
+template <bool VEC>
+__global__ __launch_bounds__(kThreads) void quantize_asym_kernel(
+    const float* __restrict__ in, uint8_t* __restrict__ out, float* __restrict__ oscale,
+    float* __restrict__ oshift, size_t n, float lo, float hi, const uint32_t* __restrict__ parts,
+    int nparts, int rev) {
+  if (parts != nullptr) load_range_f32(parts, nparts, lo, hi);
+  QuantAsym rule;
+  rule.scale = 255.0f / (hi - lo);
+  rule.shift = 255.0f - hi * rule.scale;
+  if (VEC)
+    narrow_stream<float, QuantAsym, false>(in, out, n, rule, 0.f, rev != 0);
+  else
+    narrow_scalar<float, QuantAsym, false>(in, out, n, rule, 0.f);
+  if (blockIdx.x == 0 && threadIdx.x == 0) {
+    *oscale = rule.scale;
+    *oshift = rule.shift;
+  }
+}
+
+// int8 -> uint8 with scale 1 and shift 128 (the sign bit flipped), or the uint8 identity
+// with scale 1 and shift 0 (quantize_asym-inl.h:85-101)
+template <bool FLIP>
+__global__ __launch_bounds__(kThreads) void asym_bytes_kernel(const uint8_t* __restrict__ in,
+                                                              uint8_t* __restrict__ out,
+                                                              float* __restrict__ oscale,
+                                                              float* __restrict__ oshift,
+                                                              size_t n, int vec) {
+  const size_t stride = size_t(gridDim.x) * kThreads;
+  const size_t t0 = size_t(blockIdx.x) * kThreads + threadIdx.x;
+  size_t done = 0;
+  if (vec) {
+    typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+    const size_t nv = n >> 4;
+    const u4* i16 = reinterpret_cast<const u4*>(in);
+    u4* o16 = reinterpret_cast<u4*>(out);
+    for (size_t q = t0; q < nv; q += stride) {
+      u4 v = nt_load(i16 + q);
+      if (FLIP) v ^= 0x80808080u;
+      nt_store(v, o16 + q);
+    }
+    done = nv << 4;
+  }
+  for (size_t i = done + t0; i < n; i += stride) out[i] = FLIP ? (in[i] ^ 0x80u) : in[i];
+  if (blockIdx.x == 0 && threadIdx.x == 0) {
+    *oscale = 1.0f;
+    *oshift = FLIP ? 128.0f : 0.0f;
   }
 }
 
@@ -691,6 +754,59 @@ int mxq_quantize(void* stream, const float* in, const float* imin, const float* 
   if (n == 0) return 0;
   launch_quantize(static_cast<hipStream_t>(stream), in, out, omin, omax, n, out_type, 0.f, 0.f,
                   imin, imax, nullptr, 0);
+  MXQ_API_END();
+}
+
+size_t mxq_quantize_asym_workspace(size_t) { return kWsBytes; }
+
+int mxq_quantize_asym(void* stream, const void* in, int in_type, uint8_t* out, float* oscale,
+                      float* oshift, size_t n, int calibrated, float min_calib, float max_calib,
+                      void* workspace, size_t workspace_bytes) {
+  MXQ_API_BEGIN();
+  MXQ_CHECK(in_type == MXQ_FLOAT32 || in_type == MXQ_INT8 || in_type == MXQ_UINT8,
+            "Asymmetric quantizaiton only supports int8, uint8 and float inputs, got "
+                << in_type);
+  MXQ_CHECK(oscale != nullptr && oshift != nullptr, "null scale / shift output");
+  MXQ_CHECK(n == 0 || (in != nullptr && out != nullptr), "null data pointer");
+  if (n == 0) return 0;  // Kernel<gpu>::Launch is a no-op for N == 0
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (in_type != MXQ_FLOAT32) {
+    const int vec = (aligned16(in) && aligned16(out)) ? 1 : 0;
+    const int grid = stream_grid(vec ? (n + 15) / 16 : n);
+    const uint8_t* i8 = static_cast<const uint8_t*>(in);
+    if (in_type == MXQ_INT8)
+      hipLaunchKernelGGL((asym_bytes_kernel<true>), dim3(grid), dim3(kThreads), 0, s, i8, out,
+                         oscale, oshift, n, vec);
+    else
+      hipLaunchKernelGGL((asym_bytes_kernel<false>), dim3(grid), dim3(kThreads), 0, s, i8, out,
+                         oscale, oshift, n, vec);
+    MXQ_LAUNCH_CHECK();
+    return 0;
+  }
+  const float* f = static_cast<const float*>(in);
+  const uint32_t* parts = nullptr;
+  int nparts = 0;
+  if (!calibrated) {
+    uint32_t* ws = carve(workspace, workspace_bytes);
+    nparts = reduce_grid(n);
+    if (aligned16(in))
+      hipLaunchKernelGGL((minmax_f32_kernel<true>), dim3(nparts), dim3(kThreads), 0, s, f, n, ws);
+    else
+      hipLaunchKernelGGL((minmax_f32_kernel<false>), dim3(nparts), dim3(kThreads), 0, s, f, n, ws);
+    MXQ_LAUNCH_CHECK();
+    parts = ws;
+  }
+  const bool vec = aligned16(in) && ((reinterpret_cast<uintptr_t>(out) & 3u) == 0);
+  const int grid = stream_grid(vec ? (n + 3) / 4 : n);
+  if (vec)
+    hipLaunchKernelGGL((quantize_asym_kernel<true>), dim3(grid), dim3(kThreads), 0, s, f, out,
+                       oscale, oshift, n, min_calib, max_calib, parts, nparts,
+                       parts != nullptr ? 1 : 0);
+  else
+    hipLaunchKernelGGL((quantize_asym_kernel<false>), dim3(grid), dim3(kThreads), 0, s, f, out,
+                       oscale, oshift, n, min_calib, max_calib, parts, nparts,
+                       parts != nullptr ? 1 : 0);
+  MXQ_LAUNCH_CHECK();
   MXQ_API_END();
 }
 

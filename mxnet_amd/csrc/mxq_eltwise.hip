@@ -30,6 +30,7 @@ constexpr int kMaxConcatPerLaunch = 16;
 
 typedef uint32_t u4 __attribute__((ext_vector_type(4)));
 typedef int i4 __attribute__((ext_vector_type(4)));
+typedef float f4 __attribute__((ext_vector_type(4)));
 
 __device__ __forceinline__ float maxabs(float a, float b) {
   float x = fabsf(a), y = fabsf(b);
@@ -404,6 +405,153 @@ __global__ __launch_bounds__(kThreads) void concat_kernel(ConcatArgs a) {
   }
 }
 
+// ---- elemwise_mul ---------------------------------------------------------------------
+
+struct MulArgs {
+  const uint8_t* lhs;
+  const uint8_t* rhs;
+  void* out;
+  size_t n;
+  const float* lhs_min;
+  const float* lhs_max;
+  const float* rhs_min;
+  const float* rhs_max;
+  float* omin;
+  float* omax;
+  float min_calib, max_calib;
+  int vec_ok;
+};
+
+// quantized_elemwise_mul.cc:114-155: the factor applied to the integer product and the
+// output range, for the three forms of the output
+template <int OUT>
+__device__ __forceinline__ float mul_scale(const MulArgs& a, float& omin, float& omax) {
+  const float la = maxabs(*a.lhs_min, *a.lhs_max), lb = maxabs(*a.rhs_min, *a.rhs_max);
+  if (OUT == MXQ_INT32) {
+    // QuantizationRangeForMultiplication<int8, int8, int32>, all_sign
+    omax = (la / 127.0f) * (lb / 127.0f) * 2147483648.0f;
+    omin = -omax;
+    return 1.0f;
+  }
+  const float lhs_scale = 127.5f / la, rhs_scale = 127.5f / lb;
+  if (OUT == MXQ_FLOAT32)
+    return static_cast<float>(1.0 / static_cast<double>(lhs_scale) / static_cast<double>(rhs_scale));
+  omin = a.min_calib;
+  omax = a.max_calib;
+  const float out_data_scale =
+      static_cast<float>(127.5 / static_cast<double>(maxabs(a.min_calib, a.max_calib)));
+  return out_data_scale / lhs_scale / rhs_scale;
+}
+
+__device__ __forceinline__ int sbyte(uint32_t w, int k) {
+  return static_cast<int>(static_cast<int8_t>((w >> (8 * k)) & 0xffu));
+}
+
+// static_cast<out_type>(a * b * out_scale) (quantized_elemwise_mul.cc:163-199): the int
+// product as a float, times the factor, truncated.  Where the truncated value does not
+// fit int8 the reference's conversion is undefined; this takes the low byte of the
+// truncated int32, which is what the x86 build of the reference's loop produces.
+template <int OUT>
+__global__ __launch_bounds__(kThreads) void mul_kernel(MulArgs a) {
+  float omin = 0.f, omax = 0.f;
+  const float scale = mul_scale<OUT>(a, omin, omax);
+  const size_t stride = size_t(gridDim.x) * kThreads;
+  const size_t t0 = size_t(blockIdx.x) * kThreads + threadIdx.x;
+  size_t done = 0;
+  if (a.vec_ok) {
+    if (OUT == MXQ_INT8) {
+      const size_t nv = a.n >> 4;
+      const u4* l16 = reinterpret_cast<const u4*>(a.lhs);
+      const u4* r16 = reinterpret_cast<const u4*>(a.rhs);
+      u4* o16 = reinterpret_cast<u4*>(a.out);
+      auto product16 = [&](const u4& x, const u4& y) {
+        u4 v;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+          uint32_t b[4];
+#pragma unroll
+          for (int k = 0; k < 4; ++k)
+            b[k] = static_cast<uint32_t>(
+                static_cast<int>(static_cast<float>(sbyte(x[w], k) * sbyte(y[w], k)) * scale));
+          v[w] = pack_low_bytes(b[0], b[1], b[2], b[3]);
+        }
+        return v;
+      };
+      size_t q = t0;
+      for (; q + stride < nv; q += 2 * stride) {
+        u4 x[2], y[2];
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+          x[j] = __builtin_nontemporal_load(l16 + q + j * stride);
+          y[j] = __builtin_nontemporal_load(r16 + q + j * stride);
+        }
+#pragma unroll
+        for (int j = 0; j < 2; ++j) stream_store16(product16(x[j], y[j]), o16 + q + j * stride);
+      }
+      for (; q < nv; q += stride) stream_store16(product16(l16[q], r16[q]), o16 + q);
+      done = nv << 4;
+    } else {
+      const size_t nq = a.n >> 2;
+      const uint32_t* l4 = reinterpret_cast<const uint32_t*>(a.lhs);
+      const uint32_t* r4 = reinterpret_cast<const uint32_t*>(a.rhs);
+      size_t q = t0;
+      for (; q + stride < nq; q += 2 * stride) {
+        uint32_t x[2], y[2];
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+          x[j] = __builtin_nontemporal_load(l4 + q + j * stride);
+          y[j] = __builtin_nontemporal_load(r4 + q + j * stride);
+        }
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+          if (OUT == MXQ_INT32) {
+            i4 v;
+#pragma unroll
+            for (int k = 0; k < 4; ++k) v[k] = sbyte(x[j], k) * sbyte(y[j], k);
+            __builtin_nontemporal_store(v, reinterpret_cast<i4*>(a.out) + q + j * stride);
+          } else {
+            f4 v;
+#pragma unroll
+            for (int k = 0; k < 4; ++k)
+              v[k] = static_cast<float>(sbyte(x[j], k) * sbyte(y[j], k)) * scale;
+            __builtin_nontemporal_store(v, reinterpret_cast<f4*>(a.out) + q + j * stride);
+          }
+        }
+      }
+      for (; q < nq; q += stride) {
+        const uint32_t x = l4[q], y = r4[q];
+        if (OUT == MXQ_INT32) {
+          i4 v;
+#pragma unroll
+          for (int k = 0; k < 4; ++k) v[k] = sbyte(x, k) * sbyte(y, k);
+          reinterpret_cast<i4*>(a.out)[q] = v;
+        } else {
+          f4 v;
+#pragma unroll
+          for (int k = 0; k < 4; ++k) v[k] = static_cast<float>(sbyte(x, k) * sbyte(y, k)) * scale;
+          reinterpret_cast<f4*>(a.out)[q] = v;
+        }
+      }
+      done = nq << 2;
+    }
+  }
+  for (size_t i = done + t0; i < a.n; i += stride) {
+    const int p = static_cast<int>(static_cast<int8_t>(a.lhs[i])) *
+                  static_cast<int>(static_cast<int8_t>(a.rhs[i]));
+    const float f = static_cast<float>(p) * scale;
+    if (OUT == MXQ_INT32)
+      static_cast<int32_t*>(a.out)[i] = p;
+    else if (OUT == MXQ_FLOAT32)
+      static_cast<float*>(a.out)[i] = f;
+    else
+      static_cast<uint8_t*>(a.out)[i] = static_cast<uint8_t>(static_cast<int>(f));
+  }
+  if (OUT != MXQ_FLOAT32 && blockIdx.x == 0 && threadIdx.x == 0) {
+    *a.omin = omin;
+    *a.omax = omax;
+  }
+}
+
 int grid_for(size_t work_items) {
   int dev = 0;
   MXQ_HIP(hipGetDevice(&dev));
@@ -475,6 +623,46 @@ int mxq_quantized_elemwise_add(void* stream, const void* lhs, int lhs_type, cons
     else MXQ_ADD(MXQ_INT8, false, false);
   }
 #undef MXQ_ADD
+  MXQ_LAUNCH_CHECK();
+  MXQ_API_END();
+}
+
+int mxq_quantized_elemwise_mul(void* stream, const int8_t* lhs, const int8_t* rhs,
+                               const float* lhs_min, const float* lhs_max, const float* rhs_min,
+                               const float* rhs_max, void* out, int out_type, float* omin,
+                               float* omax, size_t n, int calibrated, float min_calib,
+                               float max_calib) {
+  MXQ_API_BEGIN();
+  // QuantizedElemwiseMulOpType (quantized_elemwise_mul.cc:62-89)
+  MXQ_CHECK(out_type == MXQ_FLOAT32 || out_type == (calibrated ? MXQ_INT8 : MXQ_INT32),
+            "output type must be float32, or " << (calibrated ? "int8 (calibrated)" : "int32")
+                                               << ", got " << out_type);
+  MXQ_CHECK(lhs_min != nullptr && lhs_max != nullptr && rhs_min != nullptr && rhs_max != nullptr,
+            "null range pointer");
+  MXQ_CHECK(out_type == MXQ_FLOAT32 || (omin != nullptr && omax != nullptr),
+            "null output range pointer");
+  MXQ_CHECK(n == 0 || (lhs != nullptr && rhs != nullptr && out != nullptr), "null data pointer");
+  MulArgs a;
+  a.lhs = reinterpret_cast<const uint8_t*>(lhs);
+  a.rhs = reinterpret_cast<const uint8_t*>(rhs);
+  a.out = out;
+  a.n = n;
+  a.lhs_min = lhs_min; a.lhs_max = lhs_max; a.rhs_min = rhs_min; a.rhs_max = rhs_max;
+  a.omin = omin; a.omax = omax;
+  a.min_calib = min_calib; a.max_calib = max_calib;
+  const bool in_ok = out_type == MXQ_INT8
+                         ? (aligned16(lhs) && aligned16(rhs))
+                         : ((reinterpret_cast<uintptr_t>(lhs) | reinterpret_cast<uintptr_t>(rhs)) & 3u) == 0;
+  a.vec_ok = (in_ok && aligned16(out)) ? 1 : 0;
+  const size_t per_lane = out_type == MXQ_INT8 ? 16 : 4;
+  const int grid = grid_for(a.vec_ok ? (n + per_lane - 1) / per_lane : n);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (out_type == MXQ_INT8)
+    hipLaunchKernelGGL((mul_kernel<MXQ_INT8>), dim3(grid), dim3(kThreads), 0, s, a);
+  else if (out_type == MXQ_INT32)
+    hipLaunchKernelGGL((mul_kernel<MXQ_INT32>), dim3(grid), dim3(kThreads), 0, s, a);
+  else
+    hipLaunchKernelGGL((mul_kernel<MXQ_FLOAT32>), dim3(grid), dim3(kThreads), 0, s, a);
   MXQ_LAUNCH_CHECK();
   MXQ_API_END();
 }

@@ -77,6 +77,33 @@ def _batch_norm(a, data, gamma, beta, mean, var):
         gamma.reshape(shape) + beta.reshape(shape)
 
 
+def _shape_attr(value):
+    text = str(value).strip()
+    if text in ("", "None", "()", "[]"):
+        return ()
+    return tuple(int(v) for v in text.strip("()[] ").split(",") if v.strip())
+
+
+def _reshape(a, x):
+    """`Reshape` for the plain target shapes (positive extents, 0 = keep, one -1); the
+    other special values are resolved by the operator host for the quantized twin only."""
+    shape = list(_shape_attr(a.get("shape", "()")))
+    if any(v < -1 for v in shape) or _bool(a.get("reverse"), False):
+        raise NotImplementedError("Reshape special values -2/-3/-4 in the float executor")
+    shape = [x.shape[i] if v == 0 else v for i, v in enumerate(shape)]
+    return x.reshape(shape)
+
+
+def _transpose(a, x):
+    axes = _shape_attr(a.get("axes", "()"))
+    return x.permute(*(axes if axes else reversed(range(x.dim())))).contiguous()
+
+
+def _embedding(a, idx, weight):
+    j = idx.to(torch.int64).clamp(0, weight.shape[0] - 1)
+    return weight[j]
+
+
 _FLOAT_OPS = {
     "Convolution": _convolution,
     "FullyConnected": _fully_connected,
@@ -90,6 +117,11 @@ _FLOAT_OPS = {
     "Dropout": lambda a, x: x,
     "elemwise_add": lambda a, x, y: x + y,
     "_plus": lambda a, x, y: x + y,
+    "elemwise_mul": lambda a, x, y: x * y,
+    "Embedding": _embedding,
+    "Reshape": _reshape,
+    "reshape": _reshape,
+    "transpose": _transpose,
     "Concat": lambda a, *xs: torch.cat(xs, dim=int(a.get("dim", "1"))),
     "concat": lambda a, *xs: torch.cat(xs, dim=int(a.get("dim", "1"))),
 }

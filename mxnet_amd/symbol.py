@@ -240,6 +240,11 @@ softmax = _make("softmax")
 SoftmaxOutput = _make("SoftmaxOutput")
 Dropout = _make("Dropout")
 elemwise_add = _make("elemwise_add")
+elemwise_mul = _make("elemwise_mul")
+Embedding = _make("Embedding")
+Reshape = _make("Reshape")
+reshape = Reshape
+transpose = _make("transpose")
 
 
 def Concat(*args, name=None, dim=1, **kwargs):

@@ -43,6 +43,13 @@
  *     tests/python/quantization/test_quantization.py:375-433) and through the
  *     special cases the scales make exact (equal ranges, concat of equal scales is a
  *     byte copy).
+ *   - qref_elemwise_mul / qref_quantize_asym: native CPU loops of the reference, every
+ *     step a written C++ operation: exact rational evaluation of each rounding step,
+ *     hand-derived known answers, the reference test's own bound for the product
+ *     (tests/python/quantization/test_quantization.py:436-497), closed forms (the
+ *     int32 product is exact; asymmetric quantization maps min -> 0 and max -> 255).
+ *     Results outside the output type are undefined in the reference: the low byte of
+ *     the truncated int32 is kept, as gcc's x86 code for that conversion does.
  */
 #include <math.h>
 #include <stddef.h>
@@ -444,4 +451,58 @@ void qref_concat_rescale(const void* in_, int in_unsigned, size_t n, float imin,
     else
       ((int8_t*)out_)[i] = (int8_t)q;
   }
+}
+
+/* QuantizedElemwiseMulOpForward, quantized_elemwise_mul.cc:114-206.  out_kind: 0 int32
+ * (uncalibrated, out_scale = 1, range from QuantizationRangeForMultiplication), 1 int8
+ * (calibrated), 2 float32 (enable_float_output; omin / omax untouched).
+ * kInt8Range is the float 127.5 (quantization_utils.h:38); output_data_range is a double. */
+void qref_elemwise_mul(const int8_t* lhs, const int8_t* rhs, size_t n, float lhs_min,
+                       float lhs_max, float rhs_min, float rhs_max, int out_kind,
+                       float min_calib, float max_calib, void* out_, float* omin, float* omax) {
+  const float k_int8_range = 127.5f;
+  float out_scale = 1.0f;
+  if (out_kind == 1) {
+    const double output_data_range = (double)k_int8_range;
+    const float out_data_scale =
+        (float)(output_data_range / (double)q_maxabs(min_calib, max_calib));
+    const float lhs_scale = k_int8_range / q_maxabs(lhs_min, lhs_max);
+    const float rhs_scale = k_int8_range / q_maxabs(rhs_min, rhs_max);
+    out_scale = out_data_scale / lhs_scale / rhs_scale;
+    *omin = min_calib;
+    *omax = max_calib;
+  } else if (out_kind == 0) {
+    qref_range_for_multiplication(lhs_min, lhs_max, rhs_min, rhs_max, omin, omax);
+  } else {
+    const float lhs_scale = k_int8_range / q_maxabs(lhs_min, lhs_max);
+    const float rhs_scale = k_int8_range / q_maxabs(rhs_min, rhs_max);
+    out_scale = (float)(1.0 / (double)lhs_scale / (double)rhs_scale);
+  }
+#pragma omp parallel for schedule(static)
+  for (ptrdiff_t i = 0; i < (ptrdiff_t)n; ++i) {
+    const int8_t a = lhs[i], b = rhs[i];
+    const float f = (float)(a * b) * out_scale;
+    if (out_kind == 0)
+      ((int32_t*)out_)[i] = (int32_t)f;
+    else if (out_kind == 1)
+      ((int8_t*)out_)[i] = (int8_t)(int32_t)f;
+    else
+      ((float*)out_)[i] = f;
+  }
+}
+
+/* quantize_asymmetric::Map and QuantizeAsymOp::Forward for float input,
+ * quantize_asym-inl.h:62-76,103-152: scale = 255 / (max - min), shift = 255 - max * scale,
+ * out = (uint8)(x * scale + shift + 0.5), the last addition in double. */
+void qref_quantize_asym(const float* in, size_t n, float min_range, float max_range,
+                        uint8_t* out, float* oscale, float* oshift) {
+  const float scale = 255.0f / (max_range - min_range);
+  const float shift = 255.0f - max_range * scale;
+#pragma omp parallel for schedule(static)
+  for (ptrdiff_t i = 0; i < (ptrdiff_t)n; ++i) {
+    const float t = in[i] * scale + shift;
+    out[i] = (uint8_t)(int32_t)((double)t + 0.5);
+  }
+  *oscale = scale;
+  *oshift = shift;
 }

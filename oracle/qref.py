@@ -52,6 +52,8 @@ _lib.qref_pool_nchw.argtypes = [_p, _i] + [_i] * 12 + [_i, _i, _p]
 _lib.qref_elemwise_add.argtypes = [_p, _i, _p, _i, _sz, _f, _f, _f, _f, _i, _i, _f, _f, _p, _pf,
                                    _pf]
 _lib.qref_concat_rescale.argtypes = [_p, _i, _sz, _f, _f, _f, _f, _i, _p]
+_lib.qref_elemwise_mul.argtypes = [_p, _p, _sz, _f, _f, _f, _f, _i, _f, _f, _p, _pf, _pf]
+_lib.qref_quantize_asym.argtypes = [_p, _sz, _f, _f, _p, _pf, _pf]
 
 
 def _c(a, dtype):
@@ -323,3 +325,77 @@ def quantized_concat(arrays, mins, maxs, dim=1):
                                  int(out_dtype == np.uint8), _ptr(y))
         parts.append(y)
     return np.concatenate(parts, axis=dim), omin, omax
+
+
+def quantized_elemwise_mul(lhs, rhs, lhs_min, lhs_max, rhs_min, rhs_max, min_calib_range=None,
+                           max_calib_range=None, enable_float_output=False):
+    """_contrib_quantized_elemwise_mul on int8 operands of one shape
+    (quantized_elemwise_mul.cc:62-206): float32 output alone with enable_float_output, else
+    (out, min, max) with out int8 when both calibration bounds are given and int32 when not."""
+    if lhs.dtype != np.int8 or rhs.dtype != np.int8:
+        raise TypeError("quantized_elemwise_mul takes int8")
+    if lhs.shape != rhs.shape:
+        raise ValueError("operands must have one shape")
+    a, b = _c(lhs, np.int8), _c(rhs, np.int8)
+    calibrated = min_calib_range is not None and max_calib_range is not None
+    if enable_float_output:
+        out_dtype, kind = np.float32, 2
+    elif calibrated:
+        out_dtype, kind = np.int8, 1
+    else:
+        out_dtype, kind = np.int32, 0
+    out = np.empty(a.shape, dtype=out_dtype)
+    omin, omax = ctypes.c_float(), ctypes.c_float()
+    _lib.qref_elemwise_mul(_ptr(a), _ptr(b), a.size, lhs_min, lhs_max, rhs_min, rhs_max, kind,
+                           min_calib_range if calibrated else 0.0,
+                           max_calib_range if calibrated else 0.0, _ptr(out), ctypes.byref(omin),
+                           ctypes.byref(omax))
+    if enable_float_output:
+        return out
+    return out, np.float32(omin.value), np.float32(omax.value)
+
+
+def quantized_embedding(data, weight, min_weight, max_weight):
+    """_contrib_quantized_embedding -> (out, min, max): rows of the int8 table taken at
+    int64(data) clipped to [0, input_dim - 1] (indexing_op.cc:44-58), the table's range
+    passed through (quantized_indexing_op.cc:118-121)."""
+    if weight.dtype != np.int8 or weight.ndim != 2:
+        raise TypeError("the table is a 2-D int8 array")
+    idx = np.asarray(data)
+    with np.errstate(invalid="ignore"):
+        j = np.trunc(idx).astype(np.int64) if idx.dtype.kind == "f" else idx.astype(np.int64)
+    j = np.clip(j, 0, weight.shape[0] - 1)
+    return weight[j.reshape(-1)].reshape(idx.shape + (weight.shape[1],)).copy(), \
+        np.float32(min_weight), np.float32(max_weight)
+
+
+def quantized_reshape(data, min_data, max_data, shape):
+    """_contrib_quantized_reshape (quantized_reshape.cc:31-46): the data under another
+    shape, the range passed through.  `shape` is the inferred output shape."""
+    return np.ascontiguousarray(data).reshape(shape).copy(), np.float32(min_data), \
+        np.float32(max_data)
+
+
+def quantized_transpose(data, min_data, max_data, axes=None):
+    """_contrib_quantized_transpose (quantized_transpose.cc:49-104): numpy's transpose, the
+    range passed through."""
+    return np.array(np.transpose(data, axes), order="C", copy=True), np.float32(min_data), \
+        np.float32(max_data)
+
+
+def quantize_asym(data, min_calib_range=None, max_calib_range=None):
+    """_contrib_quantize_asym -> (out uint8, scale, shift) (quantize_asym-inl.h:78-160)."""
+    d = np.ascontiguousarray(data)
+    if d.dtype == np.uint8:
+        return d.copy(), np.float32(1.0), np.float32(0.0)
+    if d.dtype == np.int8:
+        return (d.astype(np.int16) + 128).astype(np.uint8), np.float32(1.0), np.float32(128.0)
+    if d.dtype != np.float32:
+        raise TypeError("quantize_asym takes float32, int8 or uint8")
+    if min_calib_range is None or max_calib_range is None:
+        min_calib_range, max_calib_range = minmax_f32(d)
+    out = np.empty(d.shape, dtype=np.uint8)
+    scale, shift = ctypes.c_float(), ctypes.c_float()
+    _lib.qref_quantize_asym(_ptr(d), d.size, min_calib_range, max_calib_range, _ptr(out),
+                            ctypes.byref(scale), ctypes.byref(shift))
+    return out, np.float32(scale.value), np.float32(shift.value)

@@ -183,3 +183,62 @@ def test_residual_block_with_concat_stays_int8_end_to_end():
     ref, rmin, rmax = oracle.quantized_elemwise_add(a, b, amin[0], amax[0], bmin[0], bmax[0])
     np.testing.assert_array_equal(s, ref)
     assert smin[0] == rmin and smax[0] == rmax
+
+
+def build_attention_like():
+    from mxnet_amd import symbol as S
+    d = S.Variable("data")
+    emb = S.Embedding(d, input_dim=200, output_dim=32, name="emb")
+    fc1 = S.FullyConnected(emb, num_hidden=32, flatten=False, name="fc1")
+    rs = S.Reshape(fc1, shape=(0, 0, 4, 8), name="rs")
+    tr = S.transpose(rs, axes=(0, 2, 1, 3), name="tr")
+    mul = S.elemwise_mul(tr, tr, name="mul")
+    return S.FullyConnected(mul, num_hidden=10, name="fc2")
+
+
+def test_embedding_transpose_mul_network_stays_int8_end_to_end():
+    """Token ids -> int8 embedding rows -> FC -> reshape -> transpose -> element-wise product
+    -> FC, all through the quantized operators; tracks the float network, and the byte movers'
+    outputs equal the oracle's on the tensors that reach them."""
+    from mxnet_amd import quantization as Q
+    from mxnet_amd import symbol as S
+    from mxnet_amd.executor import Executor
+    rng = np.random.default_rng(17)
+    sym = build_attention_like()
+    f = lambda v: torch.tensor(v, dtype=torch.float32)
+    arg = {"emb_weight": f(rng.normal(0, 1.0, (200, 32))),
+           "fc1_weight": f(rng.normal(0, 0.2, (32, 32))), "fc1_bias": f(rng.normal(0, 0.1, 32)),
+           "fc2_weight": f(rng.normal(0, 0.05, (10, 4 * 12 * 8))), "fc2_bias": f(rng.normal(0, 0.1, 10))}
+    calib = [f(rng.integers(0, 200, (16, 12))) for _ in range(3)]
+    qsym, qarg, qaux = Q.quantize_model(sym, arg, {}, calib_mode="naive", calib_data=calib,
+                                        num_calib_batches=3, quantize_mode="full")
+    ops = [op for op, _, _, _ in qsym.nodes() if op != "null"]
+    for name in ["_contrib_quantized_embedding", "_contrib_quantized_reshape",
+                 "_contrib_quantized_transpose", "_contrib_quantized_elemwise_mul"]:
+        assert ops.count(name) == 1
+    assert "_contrib_quantize_v2" not in ops and ops.count("_contrib_dequantize") == 1
+    assert qarg["emb_weight_quantize"].dtype == torch.int8
+    attrs = qsym.attr_dict()
+    assert "min_calib_range" in attrs["requantize_mul"]
+    x = f(rng.integers(0, 200, (32, 12)))
+    fp = Executor(sym, arg).forward(data=x)[0]
+    q = Executor(qsym, {**qarg, **qaux}).forward(data=x)[0]
+    assert q.shape == fp.shape == (32, 10)
+    assert (q - fp).abs().max().item() < 0.1 * fp.abs().max().item()
+    internals = qsym.get_internals()
+    names = ["quantized_emb_output", "requantize_fc1_output0", "requantize_fc1_output1",
+             "requantize_fc1_output2", "quantized_rs_output", "quantized_tr_output",
+             "quantized_tr_min_output", "quantized_tr_max_output", "quantized_mul_output0",
+             "quantized_mul_output1", "quantized_mul_output2"]
+    emb, h, hmin, hmax, rs, tr, trmin, trmax, mul, mulmin, mulmax = [
+        t.cpu().numpy() for t in Executor(S.Group([internals[n] for n in names]),
+                                          {**qarg, **qaux}).forward(data=x)]
+    w8 = qarg["emb_weight_quantize"].cpu().numpy()
+    np.testing.assert_array_equal(emb, w8[x.cpu().numpy().astype(np.int64)])
+    np.testing.assert_array_equal(rs, h.reshape(32, 12, 4, 8))
+    ref, rmin, rmax = oracle.quantized_transpose(rs, hmin[0], hmax[0], (0, 2, 1, 3))
+    np.testing.assert_array_equal(tr, ref)
+    assert (trmin[0], trmax[0]) == (rmin, rmax)
+    ref, rmin, rmax = oracle.quantized_elemwise_mul(tr, tr, trmin[0], trmax[0], trmin[0], trmax[0])
+    np.testing.assert_array_equal(mul, ref)
+    assert (mulmin[0], mulmax[0]) == (rmin, rmax)

@@ -245,3 +245,109 @@ def test_elemwise_add_and_concat_inference():
     assert n.infer_type([U8, I8, U8] + [None] * 6)[1] == [I8, F32, F32]
     with pytest.raises(MXNetError, match="num_args"):
         Node("_contrib_quantized_concat", dim=1)
+
+
+# src/operator/tensor/matrix_op.cc:154-196: the examples of the Reshape documentation, and
+# the quantized_reshape cases of tests/python/quantization/test_quantization.py:1057-1073
+# that use the legacy special values only
+RESHAPE_EXAMPLES = [
+    ((2, 3, 4), (4, 0, 2), False, (4, 3, 2)), ((2, 3, 4), (2, 0, 0), False, (2, 3, 4)),
+    ((2, 3, 4), (6, 1, -1), False, (6, 1, 4)), ((2, 3, 4), (3, -1, 8), False, (3, 1, 8)),
+    ((2, 3, 4), (-1,), False, (24,)), ((2, 3, 4), (-2,), False, (2, 3, 4)),
+    ((2, 3, 4), (2, -2), False, (2, 3, 4)), ((2, 3, 4), (-2, 1, 1), False, (2, 3, 4, 1, 1)),
+    ((2, 3, 4), (-3, 4), False, (6, 4)), ((2, 3, 4, 5), (-3, -3), False, (6, 20)),
+    ((2, 3, 4), (0, -3), False, (2, 12)), ((2, 3, 4), (-3, -2), False, (6, 4)),
+    ((2, 3, 4), (-4, 1, 2, -2), False, (1, 2, 3, 4)),
+    ((2, 3, 4), (2, -4, -1, 3, -2), False, (2, 1, 3, 4)),
+    ((10, 5, 4), (-1, 0), False, (40, 5)), ((10, 5, 4), (-1, 0), True, (50, 4)),
+]
+
+
+def test_tensor_op_registrations_and_inference():
+    """quantized_elemwise_mul.cc:33-89,208-256, quantized_indexing_op.cc:30-190,
+    quantized_reshape.cc:48-127, quantized_transpose.cc:31-115, quantize_asym.cc:36-157."""
+    for n in ["_contrib_quantized_elemwise_mul", "_contrib_quantized_embedding",
+              "_contrib_quantized_reshape", "_contrib_quantized_transpose"]:
+        assert op.has_attr(n, "FCompute<gpu>") and op.has_attr(n, "FInferShape")
+        assert op.has_attr(n, "FInferType")
+    assert op.has_attr("_contrib_quantize_asym", "FStatefulCompute<gpu>")
+    assert op.has_attr("_contrib_quantize_asym", "FNeedCalibrateInput")
+    for alias in ["_npx_quantized_elemwise_mul", "_npx_quantized_embedding", "quantized_reshape",
+                  "quantized_transpose"]:
+        assert op.has_attr(alias, "FInferShape")
+    assert op.has_attr("_contrib_quantized_elemwise_mul", "FNeedRequantize")
+    for n in ["_contrib_quantized_embedding", "_contrib_quantized_reshape",
+              "_contrib_quantized_transpose"]:
+        assert not op.has_attr(n, "FNeedRequantize")
+    for n in ["elemwise_mul", "Embedding", "Reshape", "transpose"]:
+        assert op.has_attr(n, "FQuantizedOp")
+    assert op.has_attr("Embedding", "FAvoidQuantizeInput")
+
+    # elemwise_mul: three outputs, or the float product alone
+    n = Node("_contrib_quantized_elemwise_mul")
+    assert n.list_inputs() == ["lhs", "rhs", "lhs_min", "lhs_max", "rhs_min", "rhs_max"]
+    assert n.num_outputs == 3
+    ins, outs = n.infer_shape([(3, 4), (3, 4), None, None, None, None])
+    assert ins == [(3, 4), (3, 4)] + [(1,)] * 4 and outs == [(3, 4), (1,), (1,)]
+    with pytest.raises(MXNetError):
+        n.infer_shape([(3, 4), (3, 5), None, None, None, None])
+    with pytest.raises(MXNetError, match="broadcast"):
+        n.infer_shape([(3, 4), (4,), None, None, None, None])
+    assert n.infer_type([I8, I8, None, None, None, None])[1] == [I32, F32, F32]
+    c = Node("_contrib_quantized_elemwise_mul", min_calib_range=-1.0, max_calib_range=2.0)
+    assert c.infer_type([I8, I8, None, None, None, None])[1] == [I8, F32, F32]
+    fo = Node("_contrib_quantized_elemwise_mul", enable_float_output=True)
+    assert fo.num_outputs == 1
+    assert fo.infer_shape([(3, 4), (3, 4), None, None, None, None])[1] == [(3, 4)]
+    assert fo.infer_type([I8, I8, None, None, None, None])[1] == [F32]
+    with pytest.raises(MXNetError):
+        Node("_contrib_quantized_elemwise_mul", out_type="int8")
+
+    # embedding
+    e = Node("_contrib_quantized_embedding", input_dim=1000, output_dim=256)
+    assert e.list_inputs() == ["data", "weight", "min_weight", "max_weight"]
+    assert e.list_outputs() == ["output", "min_output", "max_output"]
+    ins, outs = e.infer_shape([(32, 128), None, None, None])
+    assert ins == [(32, 128), (1000, 256), (1,), (1,)]
+    assert outs == [(32, 128, 256), (1,), (1,)]
+    with pytest.raises(MXNetError):
+        e.infer_shape([(32,), (999, 256), None, None])
+    assert e.infer_type([F32, None, None, None]) == ([F32, I8, F32, F32], [I8, F32, F32])
+    assert e.infer_type([I32, None, None, None])[1] == [I8, F32, F32]
+    with pytest.raises(MXNetError, match="input_dim"):
+        Node("_contrib_quantized_embedding", output_dim=4)
+    with pytest.raises(MXNetError):
+        Node("_contrib_quantized_embedding", input_dim=0, output_dim=4)
+
+    # reshape: the special values
+    for shape, newshape, reverse, expected in RESHAPE_EXAMPLES:
+        r = Node("_contrib_quantized_reshape", shape=newshape, reverse=reverse)
+        ins, outs = r.infer_shape([shape, None, None])
+        assert outs == [expected, (1,), (1,)] and ins == [shape, (1,), (1,)]
+    r = Node("_contrib_quantized_reshape", shape=(-1, 4))
+    assert r.infer_type([U8, None, None]) == ([U8, F32, F32], [U8, F32, F32])
+    with pytest.raises(MXNetError, match="Split dims"):
+        Node("_contrib_quantized_reshape", shape=(-4, 5, -1, -2)).infer_shape(
+            [(12, 3), None, None])
+
+    # transpose
+    t = Node("_contrib_quantized_transpose", axes=(2, 3, 0, 1))
+    assert t.list_inputs() == ["data", "min_data", "max_data"]
+    ins, outs = t.infer_shape([(5, 3, 6, 8), None, None])
+    assert outs == [(6, 8, 5, 3), (1,), (1,)] and ins == [(5, 3, 6, 8), (1,), (1,)]
+    assert Node("_contrib_quantized_transpose").infer_shape([(5, 3, 6), None, None])[1][0] == \
+        (6, 3, 5)
+    # the input's shape from the output's
+    ins, _ = t.infer_shape([None, None, None], [(6, 8, 5, 3), None, None])
+    assert ins[0] == (5, 3, 6, 8)
+    assert t.infer_type([I8, None, None]) == ([I8, F32, F32], [I8, F32, F32])
+    with pytest.raises(MXNetError):
+        t.infer_shape([(5, 3, 6), None, None])
+
+    # quantize_asym
+    q = Node("_contrib_quantize_asym")
+    assert q.list_inputs() == ["data"] and q.list_outputs() == ["output", "scale", "shift"]
+    assert q.infer_shape([(4, 5, 6)])[1] == [(4, 5, 6), (1,), (1,)]
+    assert q.infer_type([F32])[1] == [U8, F32, F32]
+    with pytest.raises(MXNetError):
+        q.infer_type([I8])

@@ -395,3 +395,66 @@ def test_residual_add_and_concat_stay_int8():
                                  excluded_operators=["elemwise_add", "Concat"])
     names = [n for _, n in ops_of(gsym)]
     assert "add" in names and "cat" in names and "quantized_add" not in names
+
+
+def attention_like():
+    d = S.Variable("data")
+    emb = S.Embedding(d, input_dim=100, output_dim=16, name="emb")
+    fc1 = S.FullyConnected(emb, num_hidden=16, flatten=False, name="fc1")
+    rs = S.Reshape(fc1, shape=(0, 0, 4, 4), name="rs")
+    tr = S.transpose(rs, axes=(0, 2, 1, 3), name="tr")
+    mul = S.elemwise_mul(tr, tr, name="mul")
+    return S.FullyConnected(mul, num_hidden=8, name="fc2")
+
+
+def test_embedding_reshape_transpose_and_mul_stay_int8():
+    """Embedding (quantized_indexing_op.cc:162-190: its indices are never quantized, its table
+    is quantized offline), Reshape (quantized_reshape.cc:119-127), transpose
+    (quantized_transpose.cc:106-115) and elemwise_mul (quantized_elemwise_mul.cc:247-256,
+    FNeedRequantize) between two fully-connected layers."""
+    sym = attention_like()
+    offline = [n for n in sym.list_arguments() if n != "data"]
+    assert offline == ["emb_weight", "fc1_weight", "fc1_bias", "fc2_weight", "fc2_bias"]
+    qsym, calib = Q._quantize_symbol(sym, "gpu", offline_params=offline, quantize_mode="full")
+    assert ops_of(qsym) == [
+        ("_contrib_quantized_embedding", "quantized_emb"),
+        ("_contrib_quantized_fully_connected", "quantized_fc1"),
+        ("_contrib_requantize", "requantize_fc1"),
+        ("_contrib_quantized_reshape", "quantized_rs"),
+        ("_contrib_quantized_transpose", "quantized_tr"),
+        ("_contrib_quantized_elemwise_mul", "quantized_mul"),
+        ("_contrib_requantize", "requantize_mul"),
+        ("_contrib_quantized_fully_connected", "quantized_fc2"),
+        ("_contrib_requantize", "requantize_fc2"),
+        ("_contrib_dequantize", "fc2_dequantize")]
+    # token ids go in as they are; the table and its range are the offline-quantized variables
+    assert node(qsym, "quantized_emb")[1:] == (
+        {"input_dim": "100", "output_dim": "16"},
+        [("data", 0), ("emb_weight_quantize", 0), ("emb_weight_quantize_min", 0),
+         ("emb_weight_quantize_max", 0)])
+    assert node(qsym, "quantized_fc1")[2][0] == ("quantized_emb", 0)
+    assert node(qsym, "quantized_fc1")[2][3:5] == [("quantized_emb", 1), ("quantized_emb", 2)]
+    assert node(qsym, "quantized_rs")[1:] == (
+        {"shape": "(0, 0, 4, 4)"},
+        [("requantize_fc1", 0), ("requantize_fc1", 1), ("requantize_fc1", 2)])
+    assert node(qsym, "quantized_tr")[1:] == (
+        {"axes": "(0, 2, 1, 3)"},
+        [("quantized_rs", 0), ("quantized_rs", 1), ("quantized_rs", 2)])
+    assert node(qsym, "quantized_mul")[2] == [
+        ("quantized_tr", 0), ("quantized_tr", 0), ("quantized_tr", 1), ("quantized_tr", 2),
+        ("quantized_tr", 1), ("quantized_tr", 2)]
+    # elemwise_mul registers no output names, float or quantized: its tensor is "<name>_0"
+    # (common::GetOutputName, src/common/utils.h) on both sides of the calibration table
+    assert calib == ["fc1_output", "mul_0", "fc2_output"]
+    cq = Q._calibrate_quantized_sym(qsym, {"mul_0": (-3.0, 5.0), "mul_output": (-9.0, 9.0)})
+    assert float(node(cq, "requantize_mul")[1]["max_calib_range"]) == 5.0
+    assert "emb_weight_quantize" in qsym.list_arguments() and "emb_weight" not in \
+        qsym.list_arguments()
+    # an int32 Embedding table is not a float32 one: the node stays as it is
+    d = S.Variable("data")
+    e32 = S.Embedding(d, input_dim=10, output_dim=4, dtype="int32", name="emb")
+    fc = S.FullyConnected(e32, num_hidden=3, name="fc")
+    names = [n for _, n in ops_of(Q._quantize_symbol(fc, "gpu", offline_params=["fc_weight",
+                                                                               "fc_bias"],
+                                                     quantize_mode="full")[0])]
+    assert "emb" in names and "quantized_emb" not in names
