@@ -32,6 +32,8 @@
 
 #include <hip/hip_runtime.h>
 
+#include <type_traits>
+
 #include <cstdint>
 
 namespace mxq {
@@ -107,6 +109,15 @@ __device__ __forceinline__ int epi_requant(int acc, const EpiScalars& s, float l
   float t = fabsf(f) * s.qscale;
   float u = copysignf(t + 0.5f, f);
   return static_cast<int>(__builtin_amdgcn_fmed3f(u, lo, 127.0f));
+}
+// The same with the relu, without the sign handling: for f > 0 these are the operations
+// above (|f| = f); for f <= 0 the product is the exact negative of |f|*s, so the sum is at
+// most 0.5 and the clamp to [0, 127] followed by the truncation gives the 0 that relu makes
+// of a non-positive int8.
+__device__ __forceinline__ int epi_requant_relu(int acc, const EpiScalars& s) {
+  float f = static_cast<float>(acc) * s.in_scale;
+  float u = f * s.qscale + 0.5f;
+  return static_cast<int>(__builtin_amdgcn_fmed3f(u, 0.0f, 127.0f));
 }
 
 // {a,b,c,d} low bytes -> one dword (a in byte 0).
@@ -839,19 +850,27 @@ __device__ __forceinline__ void gemm_epilogue_lds(v16i (&acc)[Cfg::MI][Cfg::NI],
   }
 
   if (e.out8 != nullptr) {
-    const float lo = e.relu ? 0.0f : -127.0f;
+    auto requantize_tile = [&](auto relu) {
 #pragma unroll
-    for (int ni = 0; ni < NI; ++ni)
+      for (int ni = 0; ni < NI; ++ni)
 #pragma unroll
-      for (int vq = 0; vq < 4; ++vq)
+        for (int vq = 0; vq < 4; ++vq)
 #pragma unroll
-        for (int mi = 0; mi < MI; ++mi) {
-          const int nl = ni * 32 + 8 * vq + 4 * lgrp, ml = mi * 32 + lrow;
-          int q[4];
+          for (int mi = 0; mi < MI; ++mi) {
+            const int nl = ni * 32 + 8 * vq + 4 * lgrp, ml = mi * 32 + lrow;
+            int q[4];
 #pragma unroll
-          for (int i = 0; i < 4; ++i) q[i] = epi_requant(acc[mi][ni][4 * vq + i], s, lo);
-          *reinterpret_cast<uint32_t*>(stage + ml * LD + nl) = pack_bytes(q[0], q[1], q[2], q[3]);
-        }
+            for (int i = 0; i < 4; ++i)
+              q[i] = decltype(relu)::value ? epi_requant_relu(acc[mi][ni][4 * vq + i], s)
+                                           : epi_requant(acc[mi][ni][4 * vq + i], s, -127.0f);
+            *reinterpret_cast<uint32_t*>(stage + ml * LD + nl) =
+                pack_bytes(q[0], q[1], q[2], q[3]);
+          }
+    };
+    if (e.relu)
+      requantize_tile(std::true_type());
+    else
+      requantize_tile(std::false_type());
     // the wave reads back what its own lanes wrote: LDS executes a wave's
     // instructions in order, the wait makes the writes complete first
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
