@@ -9,6 +9,7 @@ namespace mxq {
 
 extern int g_cast_blocks_per_cu;
 extern int g_fc_config;
+extern int g_fc_stream_groups;
 extern int g_conv_config;
 
 static thread_local std::string tl_last_error;
@@ -32,6 +33,11 @@ int mxq_set_tuning(const char* key, int value) {
   }
   if (std::strcmp(key, "fc_config") == 0) {
     mxq::g_fc_config = value;
+    return 0;
+  }
+  if (std::strcmp(key, "fc_stream_groups") == 0) {
+    if (value < 1 || value > 16) return -1;
+    mxq::g_fc_stream_groups = value;
     return 0;
   }
   if (std::strcmp(key, "conv_config") == 0) {

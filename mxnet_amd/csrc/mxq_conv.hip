@@ -114,7 +114,7 @@ struct ConvFetch {
 };
 
 template <class Cfg, bool ALIGNED>
-__global__ __launch_bounds__(Cfg::kThreads) void conv_kernel(ConvArgs p) {
+__global__ __launch_bounds__(Cfg::kThreads, Cfg::kMinWaves) void conv_kernel(ConvArgs p) {
   __shared__ __attribute__((aligned(16))) v4i lds[2][Cfg::STAGE_SLOTS];
   const int wave = threadIdx.x >> 6;
   const int wm = wave / Cfg::WN, wn = wave % Cfg::WN;
@@ -201,7 +201,7 @@ struct ConvIssuer {
 };
 
 template <class Cfg, int NS, int PIPE>
-__global__ __launch_bounds__(Cfg::kThreads) void conv_dma_kernel(ConvArgs p) {
+__global__ __launch_bounds__(Cfg::kThreads, NS <= 2 ? Cfg::kMinWaves : 1) void conv_dma_kernel(ConvArgs p) {
   __shared__ __attribute__((aligned(16))) v4i lds[NS * Cfg::STAGE_SLOTS];
   const int tiles_m = (p.M + Cfg::BM - 1) / Cfg::BM, tiles_n = (p.O + Cfg::BN - 1) / Cfg::BN;
   int tm, tn;

@@ -17,6 +17,7 @@
 namespace mxq {
 
 int g_fc_config = 0;  // 0 = choose by shape; 1.. force a tile configuration (tuning/tests)
+int g_fc_stream_groups = 2;  // work-groups per CU of the short-K streaming kernel when forced
 
 namespace {
 
@@ -29,7 +30,7 @@ struct FcArgs {
 };
 
 template <class Cfg, bool ALIGNED>
-__global__ __launch_bounds__(Cfg::kThreads) void fc_kernel(FcArgs p) {
+__global__ __launch_bounds__(Cfg::kThreads, Cfg::kMinWaves) void fc_kernel(FcArgs p) {
   __shared__ __attribute__((aligned(16))) v4i lds[2][Cfg::STAGE_SLOTS];
   const int wave = threadIdx.x >> 6;
   const int wm = wave / Cfg::WN, wn = wave % Cfg::WN;
@@ -55,7 +56,7 @@ __global__ __launch_bounds__(Cfg::kThreads) void fc_kernel(FcArgs p) {
 // operands qualify.  BUF selects buffer loads (any K % 16 == 0, zero-filled tails)
 // over global loads (K % 64 == 0, clamped rows).
 template <class Cfg, int NS, int PIPE, bool BUF>
-__global__ __launch_bounds__(Cfg::kThreads) void fc_dma_kernel(FcArgs p) {
+__global__ __launch_bounds__(Cfg::kThreads, NS <= 2 ? Cfg::kMinWaves : 1) void fc_dma_kernel(FcArgs p) {
   __shared__ __attribute__((aligned(16))) v4i lds[NS * Cfg::STAGE_SLOTS];
   const int tiles_m = (p.M + Cfg::BM - 1) / Cfg::BM, tiles_n = (p.N + Cfg::BN - 1) / Cfg::BN;
   int tm, tn;
@@ -103,6 +104,134 @@ typedef GemmCfg<64, 64, 128, 2, 2> CfgSK;      // 4 waves, wave tile 32 x 32
 typedef GemmCfg<128, 64, 128, 2, 2> CfgRK;     // 4 waves, wave tile 64 x 32
 typedef GemmCfg<64, 128, 128, 2, 2> CfgQK;     // 4 waves, wave tile 32 x 64
 typedef GemmCfg<64, 64, 256, 2, 2> CfgSK2;     // 256-byte stages for very long K
+
+// Short-K form (K = 32, 64 or 128; int8 output only).  With one or two K steps a tile of
+// the kernels above is all prologue and epilogue: a round of DMA latency, two barriers, and
+// an epilogue that keeps the CU's VALUs busy half the time.  Here the weight strip of a
+// work-group (up to 256 rows of K bytes) is parked in LDS once, and every wave on its own
+// streams work items "32 data rows x 32*NI columns": the data fragment straight from global
+// memory into the MFMA layout (a row of K bytes is consumed whole by the wave's K/16 loads),
+// the next item's fragment requested before the current one is multiplied, weights read from
+// LDS, then the fused epilogue and a transpose of the int8 tile through the wave's own LDS
+// scratch.  No barrier after the weights are staged; waves only meet the memory system.
+template <int KS, int NI>
+__global__ __launch_bounds__(256, 2) void fc_stream_kernel(FcArgs p, int bn, int strips) {
+  constexpr int K = 32 * KS, CH = 2 * KS;  // bytes and 16-byte chunks per row
+  constexpr int TN = 32 * NI, LD = TN + 16;
+  constexpr int LPR = TN / 16, RPI = 64 / LPR;
+  __shared__ __attribute__((aligned(16))) v4i ldsB[256 * CH];
+  __shared__ __attribute__((aligned(16))) int sbias[256];
+  __shared__ __attribute__((aligned(16))) char stage_all[4 * 32 * LD];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int n_begin = blockIdx.y * bn;
+  const int cols = (p.N - n_begin) < bn ? (p.N - n_begin) : bn;  // a multiple of TN
+  for (int i = tid; i < cols * CH; i += 256) {
+    const int r = i / CH, c = i - r * CH;
+    ldsB[r * CH + (c ^ swz<CH>(r))] = *reinterpret_cast<const v4i*>(
+        p.weight + static_cast<size_t>(n_begin + r) * K + c * 16);
+  }
+  const EpiScalars s = epi_scalars(p.epi);
+  if (tid < cols) sbias[tid] = epi_bias32(p.epi, s, n_begin + tid);
+  __syncthreads();
+
+  const int lrow = lane & 31, lgrp = lane >> 5;
+  char* stage = stage_all + wave * 32 * LD;
+  const int tiles_m = (p.M + 31) / 32;
+  const int items = tiles_m * strips;
+  const int step = gridDim.x * 4;
+  auto load_a = [&](int item, v4i (&f)[KS]) {
+    const int m = (item / strips) * 32 + lrow;
+    const bool ok = m < p.M;
+    const int8_t* row = p.data + static_cast<size_t>(ok ? m : 0) * K + lgrp * 16;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      f[ks] = *reinterpret_cast<const v4i*>(row + ks * 32);
+      if (!ok) f[ks] = v4i{0, 0, 0, 0};
+    }
+  };
+  int item = blockIdx.x * 4 + wave;
+  v4i fa[KS];
+  if (item < items) load_a(item, fa);
+  const bool relu = p.epi.relu != 0;
+  for (; item < items; item += step) {
+    v4i fa_next[KS];
+    const bool more = item + step < items;
+    if (more) load_a(item + step, fa_next);
+    const int tile = item / strips;
+    const int s0 = (item - tile * strips) * TN;  // first column of the strip inside the group's
+    const int m_base = tile * 32;
+    v16i acc[NI];
+#pragma unroll
+    for (int ni = 0; ni < NI; ++ni)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[ni][v] = 0;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+      for (int ni = 0; ni < NI; ++ni) {
+        const int r = s0 + ni * 32 + lrow;
+        const v4i fb = ldsB[r * CH + ((ks * 2 + lgrp) ^ swz<CH>(r))];
+        acc[ni] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fb, fa[ks], acc[ni], 0, 0, 0);
+      }
+    auto requantize_tile = [&](auto with_relu) {
+#pragma unroll
+      for (int ni = 0; ni < NI; ++ni)
+#pragma unroll
+        for (int vq = 0; vq < 4; ++vq) {
+          const int nl = ni * 32 + 8 * vq + 4 * lgrp;
+          const v4i b = *reinterpret_cast<const v4i*>(sbias + s0 + nl);
+          int q[4];
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const int v = static_cast<int>(static_cast<uint32_t>(acc[ni][4 * vq + i]) +
+                                           static_cast<uint32_t>(b[i]));
+            q[i] = decltype(with_relu)::value ? epi_requant_relu(v, s) : epi_requant(v, s, -127.0f);
+          }
+          *reinterpret_cast<uint32_t*>(stage + lrow * LD + nl) = pack_bytes(q[0], q[1], q[2], q[3]);
+        }
+    };
+    if (relu)
+      requantize_tile(std::true_type());
+    else
+      requantize_tile(std::false_type());
+    // the wave reads back what its own lanes wrote: LDS executes a wave's instructions in
+    // order, the wait makes the writes complete first
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int it = 0; it < 32 / RPI; ++it) {
+      const int rr = it * RPI + lane / LPR, c16 = lane % LPR;
+      const v4i val = *reinterpret_cast<const v4i*>(stage + rr * LD + c16 * 16);
+      const int m = m_base + rr;
+      if (m < p.M)
+        *reinterpret_cast<v4i*>(p.epi.out8 + static_cast<size_t>(m) * p.ldo + n_begin + s0 +
+                                c16 * 16) = val;
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_wave_barrier();
+    if (more) {
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) fa[ks] = fa_next[ks];
+    }
+  }
+  if (blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0) epilogue_ranges(p.epi);
+}
+
+template <int KS, int NI>
+void launch_stream(hipStream_t s, const FcArgs& a, long cus, int groups_per_cu) {
+  constexpr int TN = 32 * NI;
+  const int bn = a.N < 256 ? a.N : 256;
+  const int ny = (a.N + bn - 1) / bn;
+  const int strips = bn / TN;
+  const long items = static_cast<long>((a.M + 31) / 32) * strips;
+  long gx = cus * groups_per_cu / ny;
+  if (gx < 1) gx = 1;
+  if (gx * 4 > items) gx = (items + 3) / 4;
+  hipLaunchKernelGGL((fc_stream_kernel<KS, NI>), dim3(static_cast<unsigned>(gx), ny), dim3(256), 0,
+                     s, a, bn, strips);
+  MXQ_LAUNCH_CHECK();
+}
 
 template <class Cfg, int NS, int PIPE, bool BUF>
 void launch_dma(hipStream_t s, const FcArgs& a) {
@@ -190,6 +319,32 @@ void launch_fc(hipStream_t s, const int8_t* data, const int8_t* weight, int M, i
     }
   }
   if (cfg >= 11 && cfg <= 16) MXQ_CHECK(glb_ok, "shape does not qualify for the DMA kernels");
+  // 61 / 62: the short-K streaming kernel with 64- / 128-column strips
+  const bool stream_ok = aligned && (K == 32 || K == 64 || K == 128) && epi.out32 == nullptr &&
+                         epi.out8 != nullptr && N % 64 == 0 && (N <= 256 || N % 256 == 0) &&
+                         ldo % 16 == 0 && aligned16(epi.out8);
+  // chosen for tall outputs of at most 256 columns (200704 x 64 -> 64: 8.5 us against 10.2;
+  // -> 256: 18.5 against 21.9; 200704 x 128 -> 128: 15.3 against 17.1); from 512 columns on
+  // the tiled kernels are level or ahead
+  int stream_groups = g_fc_stream_groups;
+  if (g_fc_config == 0 && stream_ok && N <= 256 && M >= 32768) {
+    cfg = (N % 128 == 0) ? 62 : 61;
+    stream_groups = K <= 64 ? 4 : 3;
+  }
+  if (cfg == 61 || cfg == 62) {
+    MXQ_CHECK(stream_ok && (cfg == 61 || N % 128 == 0),
+              "shape does not qualify for the short-K streaming kernel");
+    const long cus = num_cus();
+#define MXQ_STREAM(NI)                                                          \
+  do {                                                                          \
+    if (K == 32) launch_stream<1, NI>(s, a, cus, stream_groups);           \
+    else if (K == 64) launch_stream<2, NI>(s, a, cus, stream_groups);      \
+    else launch_stream<4, NI>(s, a, cus, stream_groups);                   \
+  } while (0)
+    if (cfg == 61) MXQ_STREAM(2); else MXQ_STREAM(4);
+#undef MXQ_STREAM
+    return;
+  }
   if (cfg >= 21) MXQ_CHECK(buf_ok, "shape does not qualify for the buffer-load DMA kernels");
   switch (cfg) {
     case 1: launch_cfg<CfgL8>(s, a, aligned); break;

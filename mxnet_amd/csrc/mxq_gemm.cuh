@@ -157,6 +157,13 @@ struct GemmCfg {
   static constexpr int B_CHUNKS = BN * CH / kThreads;
   static constexpr int ROWS_PER_PASS = kThreads / CH;
   static constexpr int STAGE_SLOTS = (BM + BN) * CH;
+  // Second __launch_bounds__ argument (minimum waves per SIMD).  A 4-wave work-group alone
+  // asks for 1, which lets the compiler budget 512 registers per lane and put the MFMA
+  // results in the accumulation half of the file, from where every value costs the epilogue
+  // a v_accvgpr_read (and a v_accvgpr_write to zero it).  Asking for 2 caps the budget at
+  // 256 architected registers and selects the MFMA form that writes them directly; only
+  // done where the accumulators leave room (not for 256 x 256 on 4 waves).
+  static constexpr int kMinWaves = (kThreads <= 256 && MI * NI * 16 <= 128) ? 2 : 1;
   static_assert(BM % (32 * WM) == 0 && BN % (32 * WN) == 0, "wave tile");
   static_assert((BM * CH) % kThreads == 0 && (BN * CH) % kThreads == 0, "loader");
   static_assert(kThreads % CH == 0, "loader rows");

@@ -156,3 +156,48 @@ def test_fc_errors(capi):
     b = torch.zeros(4, dtype=torch.int8, device="cuda")
     with pytest.raises(mxnet_amd._lib.MXQError, match="bias given without its range"):
         capi.quantized_fc(d, d, b, -one, one, -one, one)
+
+
+@pytest.mark.parametrize("cfg", [61, 62])
+@pytest.mark.parametrize("M,K,N", [(32, 64, 64), (1, 32, 128), (33, 64, 256), (1000, 128, 128),
+                                   (4099, 64, 512), (257, 128, 768), (70, 32, 1024),
+                                   (6272, 64, 256)])
+@pytest.mark.parametrize("relu,use_bias", [(False, True), (True, True), (True, False)])
+def test_fc_short_k_streaming_kernel(capi, cfg, M, K, N, relu, use_bias):
+    """The short-K kernel (weights parked in LDS, data streamed by independent waves): fused
+    int8 output against requantize(oracle int32), ragged M, one to several column groups."""
+    if cfg == 62 and N % 128 != 0:
+        pytest.skip("128-column strips need N % 128 == 0")
+    import mxnet_amd
+    d = int8_uniform((M, K), seed=cfg + M)
+    w = int8_uniform((N, K), seed=K + N, lo=-40, hi=40)
+    b = int8_uniform((N,), seed=N) if use_bias else None
+    rd, rw, rb = 1.0, 0.08, 0.5
+    ro, rmn, rmx = oracle_fc(d, w, b, rd, rw, rb)
+    fl = ro.astype(np.float64) * (float(rmx) / 2147483648.0)
+    R = float(np.percentile(np.abs(fl), 98.0))
+    mxnet_amd._lib.set_tuning("fc_config", cfg)
+    try:
+        res = run_fc(capi, d, w, b, rd, rw, rb, calib=(-R, 0.9 * R), relu=relu, want_int32=False)
+        torch.cuda.synchronize()
+    finally:
+        mxnet_amd._lib.set_tuning("fc_config", 0)
+    rq, qmn, qmx = oracle.requantize(ro, rmn, rmx, -R, 0.9 * R)
+    if relu:
+        rq = oracle.relu_i8(rq)
+    np.testing.assert_array_equal(res["out8"].cpu().numpy(), rq)
+    assert (res["omin"].item(), res["omax"].item()) == (rmn, rmx)
+    assert (res["rmin"].item(), res["rmax"].item()) == (qmn, qmx)
+
+
+def test_fc_short_k_streaming_kernel_refuses_other_shapes(capi):
+    import mxnet_amd
+    d, w = int8_uniform((64, 96), seed=1), int8_uniform((64, 96), seed=2)
+    mxnet_amd._lib.set_tuning("fc_config", 61)
+    try:
+        with pytest.raises(mxnet_amd._lib.MXQError, match="short-K"):
+            run_fc(capi, d, w, None, 1.0, 1.0, 1.0, calib=(-1.0, 1.0), want_int32=False)
+        with pytest.raises(mxnet_amd._lib.MXQError, match="short-K"):   # int32 output wanted
+            run_fc(capi, d[:, :64].copy(), w[:, :64].copy(), None, 1.0, 1.0, 1.0)
+    finally:
+        mxnet_amd._lib.set_tuning("fc_config", 0)
