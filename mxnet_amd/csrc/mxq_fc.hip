@@ -105,10 +105,10 @@ typedef GemmCfg<128, 64, 128, 2, 2> CfgRK;     // 4 waves, wave tile 64 x 32
 typedef GemmCfg<64, 128, 128, 2, 2> CfgQK;     // 4 waves, wave tile 32 x 64
 typedef GemmCfg<64, 64, 256, 2, 2> CfgSK2;     // 256-byte stages for very long K
 
-// Short-K form (K = 32, 64 or 128; int8 output only).  With one or two K steps a tile of
+// Short-K form (K = 32, 64, 128 or 256; int8 output only).  With one or two K steps a tile of
 // the kernels above is all prologue and epilogue: a round of DMA latency, two barriers, and
 // an epilogue that keeps the CU's VALUs busy half the time.  Here the weight strip of a
-// work-group (up to 256 rows of K bytes) is parked in LDS once, and every wave on its own
+// work-group (up to 256 rows of K bytes, 128 for K = 256) is parked in LDS once, and every wave on its own
 // streams work items "32 data rows x 32*NI columns": the data fragment straight from global
 // memory into the MFMA layout (a row of K bytes is consumed whole by the wave's K/16 loads),
 // the next item's fragment requested before the current one is multiplied, weights read from
@@ -119,7 +119,8 @@ __global__ __launch_bounds__(256, 2) void fc_stream_kernel(FcArgs p, int bn, int
   constexpr int K = 32 * KS, CH = 2 * KS;  // bytes and 16-byte chunks per row
   constexpr int TN = 32 * NI, LD = TN + 16;
   constexpr int LPR = TN / 16, RPI = 64 / LPR;
-  __shared__ __attribute__((aligned(16))) v4i ldsB[256 * CH];
+  constexpr int kMaxRows = KS <= 4 ? 256 : 128;  // weight rows per work-group: at most 32 KB
+  __shared__ __attribute__((aligned(16))) v4i ldsB[kMaxRows * CH];
   __shared__ __attribute__((aligned(16))) int sbias[256];
   __shared__ __attribute__((aligned(16))) char stage_all[4 * 32 * LD];
   const int tid = threadIdx.x, lane = tid & 63;
@@ -221,7 +222,8 @@ __global__ __launch_bounds__(256, 2) void fc_stream_kernel(FcArgs p, int bn, int
 template <int KS, int NI>
 void launch_stream(hipStream_t s, const FcArgs& a, long cus, int groups_per_cu) {
   constexpr int TN = 32 * NI;
-  const int bn = a.N < 256 ? a.N : 256;
+  const int max_rows = KS <= 4 ? 256 : 128;
+  const int bn = a.N < max_rows ? a.N : max_rows;
   const int ny = (a.N + bn - 1) / bn;
   const int strips = bn / TN;
   const long items = static_cast<long>((a.M + 31) / 32) * strips;
@@ -320,14 +322,16 @@ void launch_fc(hipStream_t s, const int8_t* data, const int8_t* weight, int M, i
   }
   if (cfg >= 11 && cfg <= 16) MXQ_CHECK(glb_ok, "shape does not qualify for the DMA kernels");
   // 61 / 62: the short-K streaming kernel with 64- / 128-column strips
-  const bool stream_ok = aligned && (K == 32 || K == 64 || K == 128) && epi.out32 == nullptr &&
-                         epi.out8 != nullptr && N % 64 == 0 && (N <= 256 || N % 256 == 0) &&
-                         ldo % 16 == 0 && aligned16(epi.out8);
+  const int stream_rows = K == 256 ? 128 : 256;  // weight rows one work-group parks in LDS
+  const bool stream_ok = aligned && (K == 32 || K == 64 || K == 128 || K == 256) &&
+                         epi.out32 == nullptr && epi.out8 != nullptr && N % 64 == 0 &&
+                         (N <= stream_rows || N % stream_rows == 0) && ldo % 16 == 0 &&
+                         aligned16(epi.out8);
   // chosen for tall outputs of at most 256 columns (200704 x 64 -> 64: 8.5 us against 10.2;
   // -> 256: 18.5 against 21.9; 200704 x 128 -> 128: 15.3 against 17.1); from 512 columns on
   // the tiled kernels are level or ahead
   int stream_groups = g_fc_stream_groups;
-  if (g_fc_config == 0 && stream_ok && N <= 256 && M >= 32768) {
+  if (g_fc_config == 0 && stream_ok && N <= 256 && K <= 128 && M >= 32768) {
     cfg = (N % 128 == 0) ? 62 : 61;
     stream_groups = K <= 64 ? 4 : 3;
   }
@@ -339,7 +343,8 @@ void launch_fc(hipStream_t s, const int8_t* data, const int8_t* weight, int M, i
   do {                                                                          \
     if (K == 32) launch_stream<1, NI>(s, a, cus, stream_groups);           \
     else if (K == 64) launch_stream<2, NI>(s, a, cus, stream_groups);      \
-    else launch_stream<4, NI>(s, a, cus, stream_groups);                   \
+    else if (K == 128) launch_stream<4, NI>(s, a, cus, stream_groups);     \
+    else launch_stream<8, NI>(s, a, cus, stream_groups);                   \
   } while (0)
     if (cfg == 61) MXQ_STREAM(2); else MXQ_STREAM(4);
 #undef MXQ_STREAM

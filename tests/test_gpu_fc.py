@@ -161,7 +161,7 @@ def test_fc_errors(capi):
 @pytest.mark.parametrize("cfg", [61, 62])
 @pytest.mark.parametrize("M,K,N", [(32, 64, 64), (1, 32, 128), (33, 64, 256), (1000, 128, 128),
                                    (4099, 64, 512), (257, 128, 768), (70, 32, 1024),
-                                   (6272, 64, 256)])
+                                   (6272, 64, 256), (300, 256, 64), (1111, 256, 384)])
 @pytest.mark.parametrize("relu,use_bias", [(False, True), (True, True), (True, False)])
 def test_fc_short_k_streaming_kernel(capi, cfg, M, K, N, relu, use_bias):
     """The short-K kernel (weights parked in LDS, data streamed by independent waves): fused
