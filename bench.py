@@ -51,6 +51,7 @@ MEASURED_TRAFFIC_BYTES = {
     "quantize_asym": (2.0 * 131099.2 + 65536.1) * _KIB,         # quantize_asym_kernel_64M.md
     "embedding": (2.0 * 31709.6 + 65535.8) * _KIB,              # embedding_kernel_bert_vocab.md
     "transpose": (2.0 * 32796.4 + 65536.1) * _KIB,              # permute_elem_kernel_attention_64M.md
+    "resnet50_convs": 512.1e6,                                  # conv_stack_resnet50.md (19 launches)
 }
 
 
