@@ -286,3 +286,70 @@ def quantize_model(sym, arg_params, aux_params, data_names=("data",), device="gp
         qsym = _calibrate_quantized_sym(qsym, min_max_dict)
     qarg_params = _quantize_params(qsym, arg_params, min_max_dict)
     return qsym, qarg_params, aux_params
+
+
+def quantize_graph(sym, arg_params, aux_params, device="gpu", excluded_sym_names=None,
+                   excluded_op_names=None, calib_mode="entropy", quantized_dtype="int8",
+                   quantize_mode="full", quantize_granularity="tensor-wise",
+                   LayerOutputCollector=None, logger=None):
+    """The two-step form of quantize_model (python/mxnet/contrib/quantization.py:613-738):
+    returns (qsym, qarg_params, aux_params, collector, calib_layers).  The caller feeds the
+    collector (e.g. `Executor.register_op_hook(collector.collect)` over calibration batches)
+    and then calls `calib_graph`."""
+    excluded_sym_names = excluded_sym_names or []
+    if not isinstance(excluded_sym_names, list):
+        raise ValueError("excluded_sym_names must be a list of strings representing the names of "
+                         "the symbols that will not be quantized, while received type %s"
+                         % type(excluded_sym_names))
+    if quantized_dtype not in ("int8", "uint8", "auto"):
+        raise ValueError("unknown quantized_dtype %s received, expected `int8`, `uint8` or `auto`"
+                         % quantized_dtype)
+    if quantize_granularity not in ("tensor-wise", "channel-wise"):
+        raise ValueError("unkonwn quantize_granularity %s received, expected `tensor-wise` or "
+                         "`channel-wise`." % quantize_granularity)
+    qsym, calib_layers = _quantize_symbol(sym, device, excluded_symbols=excluded_sym_names,
+                                          excluded_operators=excluded_op_names,
+                                          offline_params=list(arg_params.keys()),
+                                          quantized_dtype=quantized_dtype,
+                                          quantize_mode=quantize_mode,
+                                          quantize_granularity=quantize_granularity)
+    collector = None
+    if calib_mode is not None and calib_mode != "none":
+        if calib_mode == "entropy":
+            collector = _LayerHistogramCollector(quantized_dtype=quantized_dtype,
+                                                 include_layers=calib_layers, logger=logger)
+        elif calib_mode == "naive":
+            collector = _LayerOutputMinMaxCollector(quantized_dtype=quantized_dtype,
+                                                    include_layers=calib_layers, logger=logger)
+        elif calib_mode == "custom" and LayerOutputCollector is not None:
+            if not isinstance(LayerOutputCollector, CalibrationCollector):
+                raise ValueError("LayerOutputCollecotr must be a subclass of a "
+                                 "CalibrationCollector class, but it is %s"
+                                 % LayerOutputCollector.__class__)
+            collector = LayerOutputCollector
+            # the names of the tensors that need calibration, unless the collector brings its own
+            if getattr(collector, "include_layers", None) is None:
+                collector.include_layers = calib_layers
+        else:
+            raise ValueError("unknown calibration mode %s received, expected `none`, `naive`, "
+                             "`entropy` or `custom`" % calib_mode)
+    qarg_params = _quantize_params(qsym, arg_params, min_max_dict={})
+    return qsym, qarg_params, aux_params, collector, calib_layers
+
+
+def calib_graph(qsym, arg_params, aux_params, collector, calib_mode="entropy", logger=None):
+    """Second step (python/mxnet/contrib/quantization.py:740-796): the collector's thresholds
+    onto the quantized symbol, the parameters quantized against it.  `arg_params` are the
+    FP32 parameters."""
+    if calib_mode is not None and calib_mode != "none":
+        if calib_mode in ("entropy", "naive", "custom"):
+            min_max_dict = collector.post_collect()
+        else:
+            raise ValueError("unknown calibration mode %s received, expected `none`, `naive`, "
+                             "`entropy` or `custom`" % calib_mode)
+        qsym = _calibrate_quantized_sym(qsym, min_max_dict)
+    else:
+        raise ValueError("Please set calibration mode to naive, entropy or custom (with custom "
+                         "CalibrationCollector)")
+    qarg_params = _quantize_params(qsym, arg_params, min_max_dict)
+    return qsym, qarg_params, aux_params

@@ -458,3 +458,4 @@ def test_embedding_reshape_transpose_and_mul_stay_int8():
                                                                                "fc_bias"],
                                                      quantize_mode="full")[0])]
     assert "emb" in names and "quantized_emb" not in names
+
