@@ -49,6 +49,7 @@ MEASURED_TRAFFIC_BYTES = {
     "concat": (2.0 * 32840.8 + 65536.1) * _KIB,                 # concat_kernel_64M.md
     "elemwise_mul_int8": (2.0 * 65565.8 + 65536.1) * _KIB,      # mul_kernel_int8_64M.md
     "quantize_asym": (2.0 * 131099.2 + 65536.1) * _KIB,         # quantize_asym_kernel_64M.md
+    "batch_norm": (2.0 * 32819.7 + 65536.0) * _KIB,             # bn_rows_kernel_nchw_64M.md
     "embedding": (2.0 * 31709.6 + 65535.8) * _KIB,              # embedding_kernel_bert_vocab.md
     "transpose": (2.0 * 32796.4 + 65536.1) * _KIB,              # permute_elem_kernel_attention_64M.md
     "resnet50_convs": 512.1e6,                                  # conv_stack_resnet50.md (19 launches)
@@ -64,7 +65,7 @@ def parse_args():
                     choices=["fc4096", "fc8192", "quantize", "quantize_uncal", "quantize_uint8",
                              "requantize", "requantize_uncal", "dequantize", "copy", "maxpool", "avgpool",
                              "elemwise_add", "elemwise_add_int8", "concat", "elemwise_mul_int8", "quantize_asym",
-                             "embedding", "transpose", "resnet50_convs", "bert_fc_chain",
+                             "batch_norm", "embedding", "transpose", "resnet50_convs", "bert_fc_chain",
                              "bert_fc_chain_fused"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-cast-ops", action="store_true")
@@ -250,6 +251,25 @@ class CastWorkload:
             self.bytes = 5.0 * n
             self.kernel = "quantize_asym_kernel"
             self.name = "quantize_asym fp32->uint8 calibrated (-6,6)"
+        elif kind == "batch_norm":
+            # NCHW (64, 256, 64, 64) int8 -> int8, relu fused: one byte in, one out per element
+            self.channels, self.inner = 256, 64 * 64
+            self.outer = n // (self.channels * self.inner)
+            self.src = [torch.randint(-127, 128, (n,), device="cuda", generator=g,
+                                      dtype=torch.int8) for _ in range(self.NBUF)]
+            self.dst = [torch.empty(n, dtype=torch.int8, device="cuda") for _ in range(self.NBUF)]
+            self.gamma = torch.rand(self.channels, device="cuda", generator=g) + 0.5
+            self.beta = torch.randn(self.channels, device="cuda", generator=g)
+            self.mean = torch.randn(self.channels, device="cuda", generator=g)
+            self.var = torch.rand(self.channels, device="cuda", generator=g) + 0.5
+            self.imin = torch.tensor([-3.0], device="cuda")
+            self.imax = torch.tensor([3.0], device="cuda")
+            self.ws = torch.empty(lib.mxq_quantized_batch_norm_workspace(self.channels),
+                                  dtype=torch.uint8, device="cuda")
+            self.bytes = 2.0 * n
+            self.kernel = "bn_rows_kernel"
+            self.name = "quantized_batch_norm_relu int8->int8, NCHW (%d,256,64,64), calibrated " \
+                        "(-6,6)" % self.outer
         elif kind == "embedding":
             # BERT-base vocabulary: 30522 rows of 768 int8; n / 768 token ids per launch
             self.rows = n // 768
@@ -330,6 +350,12 @@ class CastWorkload:
         elif kind == "quantize_asym":
             rc = lib.mxq_quantize_asym(st, P(self.src[k]), 0, P(self.dst[k]), P(self.omin),
                                        P(self.omax), n, 1, -6.0, 6.0, None, 0)
+        elif kind == "batch_norm":
+            rc = lib.mxq_quantized_batch_norm(st, P(self.src[k]), 5, P(self.gamma), P(self.beta),
+                                              P(self.mean), P(self.var), P(self.imin),
+                                              P(self.imax), P(self.dst[k]), P(self.omin),
+                                              P(self.omax), self.outer, self.channels, self.inner,
+                                              1e-3, -6.0, 6.0, 1, P(self.ws), self.ws.numel())
         elif kind == "embedding":
             rc = lib.mxq_quantized_embedding(st, P(self.src[k]), 4, P(self.table), P(self.imin),
                                              P(self.imax), P(self.dst[k]), P(self.omin),
@@ -357,6 +383,9 @@ class CastWorkload:
             table = self.table.cpu().numpy()
         elif kind == "transpose":
             x = self.src[0][:n // (512 * 16 * 64)].cpu().numpy()
+        elif kind == "batch_norm":
+            x = self.src[0][:n].cpu().numpy().reshape(-1, self.channels, self.inner)
+            bn = [t.cpu().numpy() for t in (self.gamma, self.beta, self.mean, self.var)]
         else:
             x = self.src[0][:n].cpu().numpy()
         reps, t0 = 0, time.perf_counter()
@@ -381,6 +410,8 @@ class CastWorkload:
                 oracle.quantized_elemwise_mul(x, x, -3.0, 3.0, -3.0, 3.0, -9.0, 9.0)
             elif kind == "quantize_asym":
                 oracle.quantize_asym(x, -6.0, 6.0)
+            elif kind == "batch_norm":
+                oracle.quantized_batch_norm(x, *bn, -3.0, 3.0, -6.0, 6.0, relu=True)
             elif kind == "embedding":
                 oracle.quantized_embedding(x, table, -1.0, 1.0)
             elif kind == "transpose":
@@ -823,8 +854,8 @@ def main():
         rows = []
         for kind in ["quantize", "quantize_uint8", "quantize_uncal", "requantize",
                      "requantize_uncal", "dequantize", "elemwise_add", "elemwise_add_int8",
-                     "concat", "elemwise_mul_int8", "quantize_asym", "embedding", "transpose",
-                     "maxpool", "avgpool", "fc8192",
+                     "concat", "elemwise_mul_int8", "quantize_asym", "batch_norm", "embedding",
+                     "transpose", "maxpool", "avgpool", "fc8192",
                      "resnet50_convs", "bert_fc_chain", "bert_fc_chain_fused"]:
             if kind == args.workload:
                 continue

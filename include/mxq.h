@@ -195,6 +195,30 @@ int mxq_quantize_asym(void* stream, const void* in, int in_type, uint8_t* out, f
                       float* oshift, size_t n, int calibrated, float min_calib, float max_calib,
                       void* workspace, size_t workspace_bytes);
 
+/* ---- _contrib_quantized_batch_norm, _contrib_quantized_batch_norm_relu ----------------
+ * Replaces DNNLQuantizedBatchNormForward
+ * (src/operator/quantization/dnnl/dnnl_quantized_batch_norm.cc:34-130; cpu-only in the
+ * reference): data [outer][channels][inner] int8 (uint8 is first scaled to int8 by
+ * 127.5 / 255.5), inference statistics.  Per channel
+ *   invstd = float(1.0 / sqrt(double(var) + eps)),
+ *   w = gamma * invstd * MaxAbs(data range) / MaxAbs(calib range),
+ *   b = (beta - mean * gamma * invstd) * 127.5 / MaxAbs(calib range),
+ * out = saturate(nearest-even((w / sqrt(1 + eps)) * x + b)), with max(0, .) before the
+ * rounding for the relu form; the output range is (min_calib, max_calib), which the
+ * operator requires.  The factor and offset follow the reference's own file; the
+ * normalisation itself (the second division by sqrt(1 + eps), the order of multiply and
+ * add, the rounding) runs inside oneDNN there and is not pinned by its sources (its test
+ * accepts rtol 0.1, atol 8).  workspace: mxq_quantized_batch_norm_workspace(channels)
+ * bytes, 4-byte aligned. */
+size_t mxq_quantized_batch_norm_workspace(int64_t channels);
+int mxq_quantized_batch_norm(void* stream, const void* data, int data_type, const float* gamma,
+                             const float* beta, const float* moving_mean,
+                             const float* moving_var, const float* min_data,
+                             const float* max_data, int8_t* out, float* omin, float* omax,
+                             int64_t outer, int64_t channels, int64_t inner, double eps,
+                             float min_calib, float max_calib, int relu, void* workspace,
+                             size_t workspace_bytes);
+
 /* ---- _contrib_quantized_concat -----------------------------------------------------
  * Replaces DNNLQuantizedConcatForward
  * (src/operator/quantization/dnnl/dnnl_quantized_concat.cc:41-115; cpu-only in the

@@ -49,6 +49,9 @@ SIGNATURES = {
     "mxq_quantized_transpose": (_i, [_p, _p, _p, _p, _p, _p, _p, _i, _p, _p]),
     "mxq_quantize_asym_workspace": (_sz, [_sz]),
     "mxq_quantize_asym": (_i, [_p, _p, _i, _p, _p, _p, _sz, _i, _f, _f, _p, _sz]),
+    "mxq_quantized_batch_norm_workspace": (_sz, [ctypes.c_int64]),
+    "mxq_quantized_batch_norm": (_i, [_p, _p, _i] + [_p] * 6 + [_p, _p, _p] +
+                                 [ctypes.c_int64] * 3 + [ctypes.c_double, _f, _f, _i, _p, _sz]),
     "mxq_quantized_concat": (_i, [_p, _i, _p, _p, _p, _p, _p, ctypes.c_int64, ctypes.c_int64, _p,
                                   _i, _p, _p]),
     "mxq_quantized_fc": (_i, [_p, _p, _p, _p, _i, _i, _i] + [_p] * 6 + [_p, _p, _p, _p, _p, _p,

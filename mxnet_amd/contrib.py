@@ -107,3 +107,14 @@ def quantized_transpose(data, min_data, max_data, axes=()):
 def quantize_asym(data, min_calib_range=None, max_calib_range=None):
     return invoke("_contrib_quantize_asym", data, min_calib_range=min_calib_range,
                   max_calib_range=max_calib_range)
+
+
+def quantized_batch_norm(data, gamma, beta, moving_mean, moving_var, min_data, max_data,
+                         eps=1e-3, momentum=0.9, fix_gamma=True, use_global_stats=False,
+                         axis=1, min_calib_range=None, max_calib_range=None, relu=False):
+    """_contrib_quantized_batch_norm, or _contrib_quantized_batch_norm_relu with relu=True."""
+    return invoke("_contrib_quantized_batch_norm_relu" if relu else
+                  "_contrib_quantized_batch_norm", data, gamma, beta, moving_mean, moving_var,
+                  min_data, max_data, eps=eps, momentum=momentum, fix_gamma=fix_gamma,
+                  use_global_stats=use_global_stats, axis=axis, min_calib_range=min_calib_range,
+                  max_calib_range=max_calib_range)

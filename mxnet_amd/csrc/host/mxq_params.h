@@ -17,6 +17,7 @@
 //   ReshapeParam           src/operator/tensor/matrix_op-inl.h:53-80
 //   TransposeParam         src/operator/tensor/matrix_op-inl.h:269-280
 //   QuantizeAsymParam      src/operator/quantization/quantize_asym-inl.h:41-59
+//   BatchNormParam         src/operator/nn/batch_norm-inl.h:87-133
 // Same field names, defaults, enum strings and error behaviour (unknown keys are
 // errors unless they look like __hidden__ keys).
 #ifndef MXQ_PARAMS_H_
@@ -644,6 +645,69 @@ struct ReshapeParam {
             {"keep_highest", "boolean, optional, default=0",
              "(Deprecated! Use ``shape`` instead.) Whether keep the highest dim unchanged.If set "
              "to true, then the first dim in target_shape is ignored,and always fixed as input"}};
+  }
+};
+
+inline double get_double(const param_detail::Dict& d, const std::string& key, double def) {
+  auto it = d.find(key);
+  if (it == d.end()) return def;
+  const std::string s = param_detail::trim(it->second);
+  char* end = nullptr;
+  const double v = std::strtod(s.c_str(), &end);
+  if (end == s.c_str() || *end) param_detail::bad_value(key, it->second, "double");
+  return v;
+}
+
+struct BatchNormParam {
+  double eps = 1e-3f;  // the reference's default is the float literal
+  float momentum = 0.9f;
+  bool fix_gamma = true;
+  bool use_global_stats = false;
+  bool output_mean_var = false;
+  int axis = 1;
+  bool cudnn_off = false;
+  dmlc::optional<float> min_calib_range;
+  dmlc::optional<float> max_calib_range;
+  void Init(const param_detail::Dict& d) {
+    using namespace param_detail;
+    check_unknown(d, {"eps", "momentum", "fix_gamma", "use_global_stats", "output_mean_var",
+                      "axis", "cudnn_off", "min_calib_range", "max_calib_range"},
+                  "BatchNormParam");
+    eps = get_double(d, "eps", 1e-3f);
+    float m = 0.9f;
+    auto it = d.find("momentum");
+    if (it != d.end() && !parse_float(it->second, &m)) bad_value("momentum", it->second, "float");
+    momentum = m;
+    fix_gamma = get_bool(d, "fix_gamma", true);
+    use_global_stats = get_bool(d, "use_global_stats", false);
+    output_mean_var = get_bool(d, "output_mean_var", false);
+    axis = static_cast<int>(get_int(d, "axis", true, 1, false, 0));
+    cudnn_off = get_bool(d, "cudnn_off", false);
+    min_calib_range = get_optional_float(d, "min_calib_range");
+    max_calib_range = get_optional_float(d, "max_calib_range");
+  }
+  static std::vector<nnvm::ParamFieldInfo> __FIELDS__() {
+    return {{"eps", "double, optional, default=0.0010000000474974513",
+             "Epsilon to prevent div 0. Must be no less than CUDNN_BN_MIN_EPSILON defined in "
+             "cudnn.h when using cudnn (usually 1e-5)"},
+            {"momentum", "float, optional, default=0.899999976", "Momentum for moving average"},
+            {"fix_gamma", "boolean, optional, default=1", "Fix gamma while training"},
+            {"use_global_stats", "boolean, optional, default=0",
+             "Whether use global moving statistics instead of local batch-norm. This will force "
+             "change batch-norm into a scale shift operator."},
+            {"output_mean_var", "boolean, optional, default=0", "Output the mean and inverse std "},
+            {"axis", "int, optional, default='1'",
+             "Specify which shape axis the channel is specified"},
+            {"cudnn_off", "boolean, optional, default=0",
+             "Do not select CUDNN operator, if available"},
+            {"min_calib_range", "float or None, optional, default=None",
+             "The minimum scalar value in the form of float32 obtained through calibration. If "
+             "present, it will be used to by quantized batch norm op to calculate primitive "
+             "scale.Note: this calib_range is to calib bn output."},
+            {"max_calib_range", "float or None, optional, default=None",
+             "The maximum scalar value in the form of float32 obtained through calibration. If "
+             "present, it will be used to by quantized batch norm op to calculate primitive "
+             "scale.Note: this calib_range is to calib bn output."}};
   }
 };
 

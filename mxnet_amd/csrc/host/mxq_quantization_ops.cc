@@ -865,7 +865,9 @@ size_t MXQTensorOpsTempSpaceBytes(const NodeAttrs& attrs, const ShapeVector& in)
 
 size_t MXQTempSpaceBytes(const NodeAttrs& attrs, const ShapeVector& in, const ShapeVector& out) {
   const std::string& name = attrs.op->name;
-  if (name == "_contrib_quantize_asym") return MXQTensorOpsTempSpaceBytes(attrs, in);
+  if (name == "_contrib_quantize_asym" || name == "_contrib_quantized_batch_norm" ||
+      name == "_contrib_quantized_batch_norm_relu")
+    return MXQTensorOpsTempSpaceBytes(attrs, in);
   if (name == "_contrib_quantize_v2") return mxq_quantize_v2_workspace(in[0].Size());
   if (name == "_contrib_requantize") return mxq_requantize_workspace(in[0].Size());
   if (name == "_contrib_quantized_conv")

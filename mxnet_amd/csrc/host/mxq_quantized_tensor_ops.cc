@@ -10,6 +10,8 @@
 //   _contrib_quantized_reshape        quantized_reshape.cc:48-100, quantized_reshape-inl.h:38-68
 //   _contrib_quantized_transpose      quantized_transpose.cc:31-104
 //   _contrib_quantize_asym            quantize_asym.cc:36-157
+//   _contrib_quantized_batch_norm     quantized_batch_norm.cc:34-122
+//   _contrib_quantized_batch_norm_relu  quantized_batch_norm_relu.cc:33-121
 // The reference computes all five on the cpu only (quantize_asym also has a gpu class
 // but registers no gpu attribute); here they are attached as "<gpu>" attributes.
 #include <algorithm>
@@ -492,9 +494,83 @@ static void QuantizeAsymForwardGPU(const OpStatePtr& state, const OpContext& ctx
   state.get_state<QuantizeAsymOperatorGPU>().Forward(ctx, inputs, req, outputs);
 }
 
-// Temp space of the operators of this file, in bytes (0 for all but the uncalibrated
-// asymmetric quantize).
+// ---- _contrib_quantized_batch_norm(_relu) -----------------------------------------------------
+
+// quantized_batch_norm.cc:34-61
+static bool QuantizedBatchNormShape(const NodeAttrs& attrs, ShapeVector* in_shape,
+                                    ShapeVector* out_shape) {
+  const BatchNormParam& param = nnvm::get<BatchNormParam>(attrs.parsed);
+  CHECK_EQ(in_shape->size(), 7U)
+      << "Input:[data, gamma, beta, moving_mean, moving_var, min_data, max_data]";
+  CHECK_EQ(out_shape->size(), 3U);
+  const TShape& dshape = in_shape->at(0);
+  if (!ndim_is_known(dshape)) return false;
+  const int channelAxis = param.axis < 0 ? dshape.ndim() + param.axis : param.axis;
+  CHECK(channelAxis >= 0 && channelAxis < dshape.ndim())
+      << "Channel axis out of range: " << param.axis;
+  const index_t channelCount = dshape[channelAxis];
+  for (int i = 1; i < 5; ++i) SHAPE_ASSIGN_CHECK(*in_shape, i, Shape1(channelCount));
+  SHAPE_ASSIGN_CHECK(*in_shape, 5, kScalarShape);
+  SHAPE_ASSIGN_CHECK(*in_shape, 6, kScalarShape);
+  SHAPE_ASSIGN_CHECK(*out_shape, 0, dshape);
+  SHAPE_ASSIGN_CHECK(*out_shape, 1, kScalarShape);
+  SHAPE_ASSIGN_CHECK(*out_shape, 2, kScalarShape);
+  return true;
+}
+
+// quantized_batch_norm.cc:63-87 (the oneDNN branch: int8 or uint8 data)
+static bool QuantizedBatchNormType(const NodeAttrs&, std::vector<int>* in_type,
+                                   std::vector<int>* out_type) {
+  CHECK_EQ(in_type->size(), 7U);
+  CHECK_EQ(out_type->size(), 3U);
+  CHECK(in_type->at(0) == mshadow::kInt8 || in_type->at(0) == mshadow::kUint8)
+      << "QuantizedBatchNorm only supports int8/uint8 input, while " << in_type->at(0)
+      << " is given.";
+  for (size_t i = 1; i < 7; ++i) TYPE_ASSIGN_CHECK(*in_type, i, mshadow::kFloat32);
+  TYPE_ASSIGN_CHECK(*out_type, 0, mshadow::kInt8);
+  TYPE_ASSIGN_CHECK(*out_type, 1, mshadow::kFloat32);
+  TYPE_ASSIGN_CHECK(*out_type, 2, mshadow::kFloat32);
+  return true;
+}
+
+// dnnl_quantized_batch_norm.cc:34-130
+template <bool fuse_relu>
+static void QuantizedBatchNormForwardGPU(const NodeAttrs& attrs, const OpContext& ctx,
+                                         const std::vector<TBlob>& inputs,
+                                         const std::vector<OpReqType>&,
+                                         const std::vector<TBlob>& outputs) {
+  CHECK_EQ(inputs.size(), 7U);
+  CHECK_EQ(outputs.size(), 3U);
+  const BatchNormParam& param = nnvm::get<BatchNormParam>(attrs.parsed);
+  CHECK(param.min_calib_range.has_value() && param.max_calib_range.has_value())
+      << "min_calib_range or max_calib_range is not available. Quantized BN currently "
+         "don't support calib_mode=None";
+  const TShape& shp = inputs[0].shape_;
+  const int axis = param.axis < 0 ? shp.ndim() + param.axis : param.axis;
+  CHECK(axis >= 0 && axis < shp.ndim()) << "Channel axis out of range: " << param.axis;
+  int64_t outer = 1, inner = 1;
+  for (int i = 0; i < axis; ++i) outer *= shp[i];
+  for (int i = axis + 1; i < shp.ndim(); ++i) inner *= shp[i];
+  CHECK(!ctx.requested.empty()) << "quantized batch norm needs its temp space resource";
+  const size_t ws_bytes = mxq_quantized_batch_norm_workspace(shp[axis]);
+  void* ws = ctx.requested[0].get_space(ws_bytes);
+  MXQ_CALL(mxq_quantized_batch_norm(
+      raw_stream(ctx), inputs[0].dptr_, inputs[0].type_flag_, inputs[1].dptr<float>(),
+      inputs[2].dptr<float>(), inputs[3].dptr<float>(), inputs[4].dptr<float>(),
+      inputs[5].dptr<float>(), inputs[6].dptr<float>(), outputs[0].dptr<int8_t>(),
+      outputs[1].dptr<float>(), outputs[2].dptr<float>(), outer, shp[axis], inner, param.eps,
+      param.min_calib_range.value(), param.max_calib_range.value(), fuse_relu ? 1 : 0, ws,
+      ws_bytes));
+}
+
+// Temp space of the operators of this file, in bytes.
 size_t MXQTensorOpsTempSpaceBytes(const NodeAttrs& attrs, const ShapeVector& in) {
+  if (attrs.op->name == "_contrib_quantized_batch_norm" ||
+      attrs.op->name == "_contrib_quantized_batch_norm_relu") {
+    const BatchNormParam& param = nnvm::get<BatchNormParam>(attrs.parsed);
+    const int axis = param.axis < 0 ? in[0].ndim() + param.axis : param.axis;
+    return mxq_quantized_batch_norm_workspace(in[0][axis]);
+  }
   if (attrs.op->name == "_contrib_quantize_asym") {
     const auto& param = nnvm::get<QuantizeAsymParam>(attrs.parsed);
     if (param.min_calib_range.has_value() && param.max_calib_range.has_value()) return 0;
@@ -638,6 +714,54 @@ NNVM_REGISTER_OP(_contrib_quantize_asym)
                                 })
     .add_argument("data", "NDArray-or-Symbol", "A ndarray/symbol of type `float32`")
     .add_arguments(QuantizeAsymParam::__FIELDS__());
+
+// quantized_batch_norm.cc:89-122 and quantized_batch_norm_relu.cc:88-121, with the resource
+// request the oneDNN files attach (dnnl_quantized_batch_norm.cc:150-167).  The reference
+// stores its FNeedCalibrateOutput function under that key with the input variant's type.
+#define MXQ_REGISTER_QUANTIZED_BATCH_NORM(name, relu, text)                                       \
+  NNVM_REGISTER_OP(name)                                                                          \
+      .describe(text)                                                                             \
+      .set_num_inputs(7)                                                                          \
+      .set_num_outputs(3)                                                                         \
+      .set_attr_parser(ParamParser<BatchNormParam>)                                               \
+      .set_attr<nnvm::FListInputNames>(                                                           \
+          "FListInputNames",                                                                      \
+          [](const NodeAttrs&) {                                                                  \
+            return std::vector<std::string>{"data",       "gamma",    "beta",    "moving_mean",   \
+                                            "moving_var", "min_data", "max_data"};                \
+          })                                                                                      \
+      .set_attr<nnvm::FListOutputNames>("FListOutputNames", OutputMinMax)                         \
+      .set_attr<nnvm::FMutateInputs>("FMutateInputs",                                             \
+                                     [](const NodeAttrs&) { return std::vector<uint32_t>{3, 4}; }) \
+      .set_attr<mxnet::FInferShape>("FInferShape", QuantizedBatchNormShape)                       \
+      .set_attr<nnvm::FInferType>("FInferType", QuantizedBatchNormType)                           \
+      .set_attr<FInferStorageType>("FInferStorageType", AllDefaultStorage)                        \
+      .set_attr<FNeedRequantize>("FNeedRequantize", [](const NodeAttrs&) { return false; })       \
+      .set_attr<FNeedCalibrateOutput>("FNeedCalibrateOutput",                                     \
+                                      [](const NodeAttrs&) { return std::vector<int>{0}; })       \
+      .set_attr<FResourceRequest>("FResourceRequest",                                             \
+                                  [](const NodeAttrs&) {                                          \
+                                    return std::vector<ResourceRequest>{                          \
+                                        ResourceRequest::kTempSpace};                             \
+                                  })                                                              \
+      .set_attr<FCompute>("FCompute<gpu>", QuantizedBatchNormForwardGPU<relu>)                    \
+      .add_argument("data", "NDArray-or-Symbol", "Input data.")                                   \
+      .add_argument("gamma", "NDArray-or-Symbol", "gamma.")                                       \
+      .add_argument("beta", "NDArray-or-Symbol", "beta.")                                         \
+      .add_argument("moving_mean", "NDArray-or-Symbol", "moving_mean.")                           \
+      .add_argument("moving_var", "NDArray-or-Symbol", "moving_var.")                             \
+      .add_argument("min_data", "NDArray-or-Symbol", "Minimum value of data.")                    \
+      .add_argument("max_data", "NDArray-or-Symbol", "Maximum value of data.")                    \
+      .add_arguments(BatchNormParam::__FIELDS__())
+
+MXQ_REGISTER_QUANTIZED_BATCH_NORM(
+    _contrib_quantized_batch_norm, false,
+    "BatchNorm operator for input and output data type of int8.  The input and output data "
+    "comes with min and max thresholds for quantizing the float32 data into int8.");
+MXQ_REGISTER_QUANTIZED_BATCH_NORM(
+    _contrib_quantized_batch_norm_relu, true,
+    "BatchNorm with ReLU operator for input and output data type of int8.  The input and "
+    "output data comes with min and max thresholds for quantizing the float32 data into int8.");
 
 }  // namespace op
 }  // namespace mxnet

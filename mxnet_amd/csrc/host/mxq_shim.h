@@ -400,6 +400,8 @@ typedef std::function<bool(const NodeAttrs&, std::vector<int>*, std::vector<int>
 typedef std::function<std::vector<std::pair<int, int>>(const NodeAttrs&)> FInplaceOption;
 typedef std::function<std::vector<bool>(const NodeAttrs&)> FInplaceIdentity;
 typedef std::function<uint32_t(const NodeAttrs&)> FNumVisibleOutputs;
+// include/nnvm/op_attr_types.h: indices of the inputs an operator writes (moving statistics)
+typedef std::function<std::vector<uint32_t>(const NodeAttrs&)> FMutateInputs;
 
 // What FQuantizedOp hands back in the reference is a graph node; only its attributes
 // (operator, name, dict, parsed struct) are ever looked at.

@@ -552,6 +552,175 @@ __global__ __launch_bounds__(kThreads) void mul_kernel(MulArgs a) {
   }
 }
 
+// ---- batch norm ---------------------------------------------------------------------------
+
+struct BnArgs {
+  const uint8_t* in;
+  uint8_t* out;
+  const float* gamma;
+  const float* beta;
+  const float* mean;
+  const float* var;
+  const float* min_data;
+  const float* max_data;
+  float* omin;
+  float* omax;
+  float* table;  // [2][C]: per-channel factor and offset in int8 units
+  size_t n;
+  uint32_t channels, inner;
+  double eps;
+  float min_calib, max_calib;
+  int relu, vec_ok;
+};
+
+// dnnl_quantized_batch_norm.cc:66-112: gamma, beta and the moving statistics folded into
+// one factor and one offset per channel in the units of the int8 input and output; then the
+// library's own normalisation over mean 0 and variance 1, which divides the factor by
+// sqrt(1 + eps) once more.
+__global__ __launch_bounds__(kThreads) void bn_table_kernel(BnArgs a) {
+  const float max_abs_data = maxabs(*a.min_data, *a.max_data);
+  const float max_abs_output = maxabs(a.min_calib, a.max_calib);
+  const float unit_std = sqrtf(1.0f + static_cast<float>(a.eps));
+  for (uint32_t c = blockIdx.x * kThreads + threadIdx.x; c < a.channels;
+       c += gridDim.x * kThreads) {
+    const float invstd =
+        static_cast<float>(1.0 / sqrt(static_cast<double>(a.var[c]) + a.eps));
+    const float w = a.gamma[c] * invstd * max_abs_data / max_abs_output;
+    const float b = (a.beta[c] - a.mean[c] * a.gamma[c] * invstd) * 127.5f / max_abs_output;
+    a.table[c] = w / unit_std;
+    a.table[a.channels + c] = b;
+  }
+  if (blockIdx.x == 0 && threadIdx.x == 0) {
+    *a.omin = a.min_calib;
+    *a.omax = a.max_calib;
+  }
+}
+
+// uint8 data is first brought to int8 at 127.5 / 255.5 of its value
+// (dnnl_quantized_batch_norm.cc:47-65); at most 127.25, so no clamp is needed
+template <bool IN_U>
+__device__ __forceinline__ float bn_input(uint32_t word, int k) {
+  if (!IN_U) return static_cast<float>(byte_of<false>(word, k));
+  return rintf(static_cast<float>(byte_of<true>(word, k)) * (127.5f / 255.5f));
+}
+
+// relu before the rounding is a lower clamp at 0 instead of -128
+template <bool IN_U, bool FAST>
+__device__ __forceinline__ uint32_t bn_word(uint32_t x, float w, float b, float lo) {
+  uint32_t r[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const float f = bn_input<IN_U>(x, j) * w + b;
+    if (FAST) {
+      r[j] = __float_as_uint(__builtin_amdgcn_fmed3f(f, lo, 127.f) + 12582912.f);
+    } else {
+      r[j] = static_cast<uint32_t>(narrow<MXQ_INT8>(f < lo ? lo : f));
+    }
+  }
+  return pack_low_bytes(r[0], r[1], r[2], r[3]);
+}
+
+template <bool IN_U>
+__device__ __forceinline__ u4 bn_sixteen(u4 x, float w, float b, float lo) {
+  u4 v;
+  // a finite factor and offset of this size keep every x * w + b finite: one-instruction
+  // clamp; anything else (NaN, infinities from a zero range) takes the guarded conversion
+  if (fabsf(w) < 1e30f && fabsf(b) < 1e30f) {
+#pragma unroll
+    for (int k = 0; k < 4; ++k) v[k] = bn_word<IN_U, true>(x[k], w, b, lo);
+  } else {
+#pragma unroll
+    for (int k = 0; k < 4; ++k) v[k] = bn_word<IN_U, false>(x[k], w, b, lo);
+  }
+  return v;
+}
+
+template <bool IN_U>
+__global__ __launch_bounds__(kThreads) void bn_kernel(BnArgs a) {
+  const size_t stride = size_t(gridDim.x) * kThreads;
+  const size_t t0 = size_t(blockIdx.x) * kThreads + threadIdx.x;
+  const float* tw = a.table;
+  const float* tb = a.table + a.channels;
+  const float lo = a.relu != 0 ? 0.f : -128.f;
+  if (a.vec_ok) {
+    // 16 bytes of one channel per lane (inner % 16 == 0, fewer than 2^32 elements), two
+    // loads in flight
+    const uint32_t nv = static_cast<uint32_t>(a.n >> 4), inner16 = a.inner >> 4;
+    const uint32_t step = static_cast<uint32_t>(stride);
+    const u4* i16 = reinterpret_cast<const u4*>(a.in);
+    u4* o16 = reinterpret_cast<u4*>(a.out);
+    uint32_t q = static_cast<uint32_t>(t0);
+    if (t0 >= nv) return;
+    for (; nv - q > step; q += 2 * step) {
+      const uint32_t q1 = q + step;
+      const u4 x0 = __builtin_nontemporal_load(i16 + q);
+      const u4 x1 = __builtin_nontemporal_load(i16 + q1);
+      const uint32_t c0 = (q / inner16) % a.channels, c1 = (q1 / inner16) % a.channels;
+      const float w0 = tw[c0], b0 = tb[c0], w1 = tw[c1], b1 = tb[c1];
+      // both results before the first store: the stores are opaque to the compiler's count
+      // of outstanding memory operations, a wait placed behind one would wait for it too
+      const u4 v0 = bn_sixteen<IN_U>(x0, w0, b0, lo);
+      const u4 v1 = bn_sixteen<IN_U>(x1, w1, b1, lo);
+      stream_store16(v0, o16 + q);
+      stream_store16(v1, o16 + q1);
+      if (nv - q1 <= step) return;
+    }
+    const uint32_t c = (q / inner16) % a.channels;
+    stream_store16(bn_sixteen<IN_U>(__builtin_nontemporal_load(i16 + q), tw[c], tb[c], lo),
+                   o16 + q);
+    return;
+  }
+  for (size_t i = t0; i < a.n; i += stride) {
+    const uint32_t c = static_cast<uint32_t>((i / a.inner) % a.channels);
+    const float f = bn_input<IN_U>(a.in[i], 0) * tw[c] + tb[c];
+    a.out[i] = static_cast<uint8_t>(narrow<MXQ_INT8>(f < lo ? lo : f));
+  }
+}
+
+// Rows of at least 1 KiB (inner % 16 == 0): one wave per 4 KiB piece of a row, so the channel,
+// its factor and offset are wave-uniform (scalar loads, no per-lane division) and a lane keeps
+// four 16-byte loads in flight.
+template <bool IN_U>
+__global__ __launch_bounds__(kThreads) void bn_rows_kernel(BnArgs a) {
+  const uint32_t inner16 = a.inner >> 4;
+  const uint32_t chunks = (inner16 + 255u) >> 8;
+  const uint32_t rows = static_cast<uint32_t>(a.n / a.inner);
+  const uint32_t items = rows * chunks;  // n < 2^32
+  const uint32_t lane = threadIdx.x & 63u;
+  const uint32_t wave =
+      __builtin_amdgcn_readfirstlane(blockIdx.x * (kThreads / 64) + (threadIdx.x >> 6));
+  const uint32_t nwaves = gridDim.x * (kThreads / 64);
+  const float lo = a.relu != 0 ? 0.f : -128.f;
+  const u4* i16 = reinterpret_cast<const u4*>(a.in);
+  u4* o16 = reinterpret_cast<u4*>(a.out);
+  for (uint32_t item = wave; item < items; item += nwaves) {
+    const uint32_t row = item / chunks, k = item - row * chunks;
+    const uint32_t c = row % a.channels;
+    const float w = a.table[c], b = a.table[a.channels + c];
+    const uint32_t left = inner16 - (k << 8);
+    const size_t base = size_t(row) * inner16 + (k << 8) + lane;
+    u4 x[4] = {};
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      if (lane + 64u * j < left) x[j] = __builtin_nontemporal_load(i16 + base + 64 * j);
+    u4 v[4];
+    if (fabsf(w) < 1e30f && fabsf(b) < 1e30f) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) v[j][q] = bn_word<IN_U, true>(x[j][q], w, b, lo);
+    } else {
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) v[j][q] = bn_word<IN_U, false>(x[j][q], w, b, lo);
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      if (lane + 64u * j < left) stream_store16(v[j], o16 + base + 64 * j);
+  }
+}
+
 int grid_for(size_t work_items) {
   int dev = 0;
   MXQ_HIP(hipGetDevice(&dev));
@@ -663,6 +832,71 @@ int mxq_quantized_elemwise_mul(void* stream, const int8_t* lhs, const int8_t* rh
     hipLaunchKernelGGL((mul_kernel<MXQ_INT32>), dim3(grid), dim3(kThreads), 0, s, a);
   else
     hipLaunchKernelGGL((mul_kernel<MXQ_FLOAT32>), dim3(grid), dim3(kThreads), 0, s, a);
+  MXQ_LAUNCH_CHECK();
+  MXQ_API_END();
+}
+
+size_t mxq_quantized_batch_norm_workspace(int64_t channels) {
+  return channels > 0 ? static_cast<size_t>(channels) * 2 * sizeof(float) : 0;
+}
+
+int mxq_quantized_batch_norm(void* stream, const void* data, int data_type, const float* gamma,
+                             const float* beta, const float* moving_mean,
+                             const float* moving_var, const float* min_data,
+                             const float* max_data, int8_t* out, float* omin, float* omax,
+                             int64_t outer, int64_t channels, int64_t inner, double eps,
+                             float min_calib, float max_calib, int relu, void* workspace,
+                             size_t workspace_bytes) {
+  MXQ_API_BEGIN();
+  MXQ_CHECK(byte_type(data_type),
+            "QuantizedBatchNorm only supports int8/uint8 input, while " << data_type
+                                                                          << " is given.");
+  MXQ_CHECK(outer >= 0 && channels > 0 && inner >= 0, "bad shape");
+  MXQ_CHECK(channels < (int64_t(1) << 31) && inner < (int64_t(1) << 31), "extent too large");
+  MXQ_CHECK(gamma != nullptr && beta != nullptr && moving_mean != nullptr && moving_var != nullptr,
+            "null parameter pointer");
+  MXQ_CHECK(min_data != nullptr && max_data != nullptr && omin != nullptr && omax != nullptr,
+            "null range pointer");
+  MXQ_CHECK(workspace != nullptr && workspace_bytes >= mxq_quantized_batch_norm_workspace(channels),
+            "workspace too small: " << workspace_bytes << " < "
+                                    << mxq_quantized_batch_norm_workspace(channels));
+  MXQ_CHECK((reinterpret_cast<uintptr_t>(workspace) & 3u) == 0, "workspace must be 4-byte aligned");
+  BnArgs a;
+  a.in = static_cast<const uint8_t*>(data);
+  a.out = reinterpret_cast<uint8_t*>(out);
+  a.gamma = gamma; a.beta = beta; a.mean = moving_mean; a.var = moving_var;
+  a.min_data = min_data; a.max_data = max_data; a.omin = omin; a.omax = omax;
+  a.table = static_cast<float*>(workspace);
+  a.n = static_cast<size_t>(outer) * static_cast<size_t>(channels) * static_cast<size_t>(inner);
+  a.channels = static_cast<uint32_t>(channels);
+  a.inner = static_cast<uint32_t>(inner);
+  a.eps = eps;
+  a.min_calib = min_calib; a.max_calib = max_calib;
+  a.relu = relu;
+  MXQ_CHECK(a.n == 0 || (data != nullptr && out != nullptr), "null data pointer");
+  a.vec_ok = (inner % 16 == 0 && a.n < (size_t(1) << 32) && aligned16(data) && aligned16(out)) ? 1 : 0;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  hipLaunchKernelGGL(bn_table_kernel, dim3((a.channels + kThreads - 1) / kThreads < 64
+                                               ? (a.channels + kThreads - 1) / kThreads
+                                               : 64),
+                     dim3(kThreads), 0, s, a);
+  MXQ_LAUNCH_CHECK();
+  if (a.n == 0) return 0;
+  if (a.vec_ok && inner >= 1024) {
+    const size_t waves = (a.n / a.inner) * ((a.inner / 16 + 255) / 256);
+    // twice the work-groups per CU of the narrowing kernels, as for concat: measured fastest
+    const int grid = 2 * grid_for(waves * 64);
+    if (data_type == MXQ_UINT8)
+      hipLaunchKernelGGL((bn_rows_kernel<true>), dim3(grid), dim3(kThreads), 0, s, a);
+    else
+      hipLaunchKernelGGL((bn_rows_kernel<false>), dim3(grid), dim3(kThreads), 0, s, a);
+  } else {
+    const int grid = 2 * grid_for(a.vec_ok ? (a.n + 15) / 16 : a.n);
+    if (data_type == MXQ_UINT8)
+      hipLaunchKernelGGL((bn_kernel<true>), dim3(grid), dim3(kThreads), 0, s, a);
+    else
+      hipLaunchKernelGGL((bn_kernel<false>), dim3(grid), dim3(kThreads), 0, s, a);
+  }
   MXQ_LAUNCH_CHECK();
   MXQ_API_END();
 }

@@ -50,6 +50,14 @@
  *     int32 product is exact; asymmetric quantization maps min -> 0 and max -> 255).
  *     Results outside the output type are undefined in the reference: the low byte of
  *     the truncated int32 is kept, as gcc's x86 code for that conversion does.
+ *   - qref_batch_norm: the per-channel factor and offset follow the reference's own file
+ *     (dnnl_quantized_batch_norm.cc:66-112) and are pinned by exact rational evaluation;
+ *     the normalisation that applies them runs inside oneDNN (third-party, absent):
+ *     PARITY UNPINNED for the second division by sqrt(1 + eps), the order of multiply and
+ *     add and the rounding of each element.  Here: saturate(nearest-even(w' * x + b)),
+ *     every binary32 operation rounded on its own; checked against an exact rational
+ *     evaluation of that rule and the reference test's own bound against the float batch
+ *     norm (tests/python/quantization/test_quantization.py:990-1054).
  */
 #include <math.h>
 #include <stddef.h>
@@ -505,4 +513,37 @@ void qref_quantize_asym(const float* in, size_t n, float min_range, float max_ra
   }
   *oscale = scale;
   *oshift = shift;
+}
+
+/* DNNLQuantizedBatchNormForward, dnnl_quantized_batch_norm.cc:34-130, on data laid out
+ * [outer][channels][inner]; the reference's dnnl::batch_normalization_forward over mean 0
+ * and variance 1 is restated as dst = saturate(round((w / sqrtf(1 + eps)) * src + b)). */
+void qref_batch_norm(const void* data_, int data_unsigned, size_t outer, size_t channels,
+                     size_t inner, const float* gamma, const float* beta, const float* mean,
+                     const float* var, float min_data, float max_data, double eps,
+                     float min_calib, float max_calib, int relu, int8_t* out, float* omin,
+                     float* omax) {
+  const float max_abs_data = q_maxabs(min_data, max_data);
+  const float max_abs_output = q_maxabs(min_calib, max_calib);
+  const float unit_std = sqrtf(1.0f + (float)eps);
+  *omin = min_calib;
+  *omax = max_calib;
+#pragma omp parallel for schedule(static) collapse(2)
+  for (ptrdiff_t o = 0; o < (ptrdiff_t)outer; ++o) {
+    for (ptrdiff_t c = 0; c < (ptrdiff_t)channels; ++c) {
+      const float invstd = (float)(1.0 / sqrt((double)var[c] + eps));
+      const float w = gamma[c] * invstd * max_abs_data / max_abs_output;
+      const float b = (beta[c] - mean[c] * gamma[c] * invstd) * 127.5f / max_abs_output;
+      const float wn = w / unit_std;
+      const size_t base = ((size_t)o * channels + (size_t)c) * inner;
+      for (size_t i = 0; i < inner; ++i) {
+        int x = data_unsigned ? (int)((const uint8_t*)data_)[base + i]
+                              : (int)((const int8_t*)data_)[base + i];
+        if (data_unsigned) x = q_round_sat((float)x * (127.5f / 255.5f), -128.0f, 127.0f);
+        float f = (float)x * wn + b;
+        if (relu && f < 0.0f) f = 0.0f;
+        out[base + i] = (int8_t)q_round_sat(f, -128.0f, 127.0f);
+      }
+    }
+  }
 }

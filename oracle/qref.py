@@ -54,6 +54,8 @@ _lib.qref_elemwise_add.argtypes = [_p, _i, _p, _i, _sz, _f, _f, _f, _f, _i, _i, 
 _lib.qref_concat_rescale.argtypes = [_p, _i, _sz, _f, _f, _f, _f, _i, _p]
 _lib.qref_elemwise_mul.argtypes = [_p, _p, _sz, _f, _f, _f, _f, _i, _f, _f, _p, _pf, _pf]
 _lib.qref_quantize_asym.argtypes = [_p, _sz, _f, _f, _p, _pf, _pf]
+_lib.qref_batch_norm.argtypes = [_p, _i, _sz, _sz, _sz, _p, _p, _p, _p, _f, _f, ctypes.c_double,
+                                 _f, _f, _i, _p, _pf, _pf]
 
 
 def _c(a, dtype):
@@ -399,3 +401,29 @@ def quantize_asym(data, min_calib_range=None, max_calib_range=None):
     _lib.qref_quantize_asym(_ptr(d), d.size, min_calib_range, max_calib_range, _ptr(out),
                             ctypes.byref(scale), ctypes.byref(shift))
     return out, np.float32(scale.value), np.float32(shift.value)
+
+
+def quantized_batch_norm(data, gamma, beta, moving_mean, moving_var, min_data, max_data,
+                         min_calib_range, max_calib_range, eps=1e-3, axis=1, relu=False):
+    """_contrib_quantized_batch_norm / _relu -> (out int8, min, max); the output range is the
+    calibrated one, which the operator requires (dnnl_quantized_batch_norm.cc:76-85)."""
+    if data.dtype not in (np.int8, np.uint8):
+        raise TypeError("quantized_batch_norm takes int8 or uint8 data")
+    if min_calib_range is None or max_calib_range is None:
+        raise ValueError("min_calib_range or max_calib_range is not available")
+    d = np.ascontiguousarray(data)
+    axis = axis + d.ndim if axis < 0 else axis
+    channels = d.shape[axis]
+    outer = int(np.prod(d.shape[:axis], dtype=np.int64))
+    inner = int(np.prod(d.shape[axis + 1:], dtype=np.int64))
+    vec = [_c(v, np.float32) for v in (gamma, beta, moving_mean, moving_var)]
+    for v in vec:
+        if v.shape != (channels,):
+            raise ValueError("per-channel parameters must have shape (%d,)" % channels)
+    out = np.empty(d.shape, dtype=np.int8)
+    omin, omax = ctypes.c_float(), ctypes.c_float()
+    _lib.qref_batch_norm(_ptr(d), int(d.dtype == np.uint8), outer, channels, inner, _ptr(vec[0]),
+                         _ptr(vec[1]), _ptr(vec[2]), _ptr(vec[3]), min_data, max_data,
+                         float(eps), min_calib_range, max_calib_range, int(relu), _ptr(out),
+                         ctypes.byref(omin), ctypes.byref(omax))
+    return out, np.float32(omin.value), np.float32(omax.value)

@@ -362,3 +362,71 @@ def test_quantize_asym_errors(lib):
     assert rc != 0 and "workspace" in lib.last_error()
     rc = lib.lib.mxq_quantize_asym(stream(), P(x), 4, P(out), P(s), P(s), 8, 1, 0.0, 1.0, None, 0)
     assert rc != 0 and "only supports int8, uint8 and float" in lib.last_error()
+
+
+# ---- batch norm -----------------------------------------------------------------------------
+
+def bn_params(rng, C):
+    return (rng.uniform(0.5, 2.0, C).astype(np.float32), rng.normal(0, 0.5, C).astype(np.float32),
+            rng.normal(0, 0.3, C).astype(np.float32), rng.uniform(0.3, 2.0, C).astype(np.float32))
+
+
+@pytest.mark.parametrize("shape,axis", [((32, 512, 4, 4), 1), ((4, 3, 224, 224), 1),
+                                        ((8, 7, 5, 3), 1), ((6, 5, 4, 16), -1), ((10, 33), 1),
+                                        ((2, 16, 1), 1), ((0, 4, 3), 1),
+                                        ((3, 5, 4112), 1), ((2, 4, 1040), 1), ((2, 3, 1024), 1)])
+@pytest.mark.parametrize("dtype", [np.int8, np.uint8])
+@pytest.mark.parametrize("relu", [False, True])
+def test_quantized_batch_norm_matches_oracle(contrib, shape, axis, dtype, relu):
+    rng = np.random.default_rng(len(shape) + shape[-1])
+    C = shape[axis]
+    lo, hi = (0, 256) if dtype == np.uint8 else (-128, 128)
+    d = rng.integers(lo, hi, shape).astype(dtype)
+    gamma, beta, mean, var = bn_params(rng, C)
+    rd = (0.0, 3.1) if dtype == np.uint8 else (-2.7, 3.1)
+    out, mn, mx = contrib.quantized_batch_norm(
+        dev(d), dev(gamma), dev(beta), dev(mean), dev(var), scalar(rd[0]), scalar(rd[1]),
+        eps=2e-5, axis=axis, min_calib_range=-6.5, max_calib_range=7.25, relu=relu)
+    ref, rmn, rmx = oracle.quantized_batch_norm(d, gamma, beta, mean, var, rd[0], rd[1], -6.5,
+                                                7.25, eps=2e-5, axis=axis, relu=relu)
+    assert out.dtype == torch.int8 and tuple(out.shape) == shape
+    np.testing.assert_array_equal(host(out), ref)
+    assert (host(mn)[0], host(mx)[0]) == (rmn, rmx)
+
+
+def test_reference_quantized_bn(contrib):
+    """check_quantized_bn (test_quantization.py:1005-1050): against the float batch norm with
+    the statistics of the data itself, rtol 0.1 / atol 8 as there."""
+    rng = np.random.default_rng(71)
+    shape = (32, 512, 4, 4)
+    data = rng.uniform(-127.0, 127.0, size=shape).astype(np.float32)
+    gamma = rng.uniform(-127.0, 127.0, 512).astype(np.float32)
+    beta = rng.uniform(-127.0, 127.0, 512).astype(np.float32)
+    mean = data.mean(axis=(0, 2, 3))
+    var = data.var(axis=(0, 2, 3))
+    want = (data - mean.reshape(1, -1, 1, 1)) / np.sqrt(var.reshape(1, -1, 1, 1) + 1e-5) * \
+        gamma.reshape(1, -1, 1, 1) + beta.reshape(1, -1, 1, 1)
+    r_in = float(np.abs(data).max())
+    q, _, _ = oracle.quantize_v2(data, "int8", -r_in, r_in)
+    R = float(np.abs(want).max())
+    out, mn, mx = contrib.quantized_batch_norm(
+        dev(q), dev(gamma), dev(beta), dev(mean), dev(var), scalar(-r_in), scalar(r_in),
+        eps=1e-5, min_calib_range=-R, max_calib_range=R)
+    back = host(out).astype(np.float32) * np.float32(R / 127.0)
+    np.testing.assert_allclose(back, want, rtol=1e-1, atol=8)
+
+
+def test_quantized_batch_norm_errors(lib, contrib):
+    import mxnet_amd
+    x = torch.zeros((2, 4, 3), dtype=torch.int8, device="cuda")
+    v = torch.ones(4, device="cuda")
+    s = scalar(1.0)
+    with pytest.raises(mxnet_amd.operator.MXNetError, match="calib"):
+        contrib.quantized_batch_norm(x, v, v, v, v, s, s)
+    out = torch.zeros_like(x)
+    rc = lib.lib.mxq_quantized_batch_norm(stream(), P(x), 5, P(v), P(v), P(v), P(v), P(s), P(s),
+                                          P(out), P(s), P(s), 2, 4, 3, 1e-3, -1.0, 1.0, 0, None, 0)
+    assert rc != 0 and "workspace" in lib.last_error()
+    rc = lib.lib.mxq_quantized_batch_norm(stream(), P(x), 0, P(v), P(v), P(v), P(v), P(s), P(s),
+                                          P(out), P(s), P(s), 2, 4, 3, 1e-3, -1.0, 1.0, 0, P(v), 64)
+    assert rc != 0 and "int8/uint8" in lib.last_error()

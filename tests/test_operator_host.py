@@ -351,3 +351,30 @@ def test_tensor_op_registrations_and_inference():
     assert q.infer_type([F32])[1] == [U8, F32, F32]
     with pytest.raises(MXNetError):
         q.infer_type([I8])
+
+
+def test_quantized_batch_norm_registration_and_inference():
+    """quantized_batch_norm.cc:34-122, quantized_batch_norm_relu.cc:33-121."""
+    for n in ["_contrib_quantized_batch_norm", "_contrib_quantized_batch_norm_relu"]:
+        assert op.has_attr(n, "FCompute<gpu>") and op.has_attr(n, "FNeedCalibrateOutput")
+        assert op.has_attr(n, "FResourceRequest") and op.has_attr(n, "FMutateInputs")
+        node = Node(n, min_calib_range=-1.0, max_calib_range=2.0)
+        assert node.list_inputs() == ["data", "gamma", "beta", "moving_mean", "moving_var",
+                                      "min_data", "max_data"]
+        assert node.list_outputs() == ["output", "min_output", "max_output"]
+        ins, outs = node.infer_shape([(8, 16, 5, 5)] + [None] * 6)
+        assert ins == [(8, 16, 5, 5)] + [(16,)] * 4 + [(1,), (1,)]
+        assert outs == [(8, 16, 5, 5), (1,), (1,)]
+        assert node.infer_type([U8] + [None] * 6) == ([U8] + [F32] * 6, [I8, F32, F32])
+        assert node.infer_type([I8] + [None] * 6)[1] == [I8, F32, F32]
+        with pytest.raises(MXNetError, match="int8/uint8"):
+            node.infer_type([F32] + [None] * 6)
+    last = Node("_contrib_quantized_batch_norm", axis=-1)
+    assert last.infer_shape([(8, 5, 5, 16)] + [None] * 6)[0][1] == (16,)
+    with pytest.raises(MXNetError, match="Channel axis out of range"):
+        Node("_contrib_quantized_batch_norm", axis=4).infer_shape([(8, 5, 5, 16)] + [None] * 6)
+    with pytest.raises(MXNetError):
+        Node("_contrib_quantized_batch_norm", epsilon=1.0)
+    # the float BatchNorm keeps no FQuantizedOp here: the pass leaves it float, as the
+    # reference does for the gpu context
+    assert not op.has_attr("BatchNorm", "FQuantizedOp")

@@ -231,3 +231,85 @@ def test_reshape_is_a_copy_with_ranges():
     out, mn, mx = qref.quantized_reshape(d, -1023.343, 2343.324275, (6, 20))
     assert out.shape == (6, 20) and np.array_equal(out.ravel(), d.ravel())
     assert (mn, mx) == (F(-1023.343), F(2343.324275))
+
+
+# ---- batch norm -----------------------------------------------------------------------------
+
+def round_half_even(q):
+    fl = q.numerator // q.denominator
+    rem = q - fl
+    return fl + (1 if rem > Fraction(1, 2) or (rem == Fraction(1, 2) and fl % 2 == 1) else 0)
+
+
+def exact_bn(x, unsigned, gamma, beta, mean, var, min_data, max_data, eps, calib, relu):
+    """dnnl_quantized_batch_norm.cc:66-112 for one element, one rounding per written operation;
+    then the stated rule saturate(nearest-even((w / sqrtf(1 + eps)) * x + b))."""
+    from math import isqrt
+    max_abs_data, max_abs_out = maxabs(min_data, max_data), maxabs(*calib)
+    # float(1.0 / sqrt(double(var) + eps)): the double sqrt and division through Python floats
+    # (IEEE binary64, correctly rounded), then one rounding to binary32
+    invstd = f(F(1.0 / np.sqrt(np.float64(F(var)) + np.float64(eps))))
+    g, b_, m = f(F(gamma)), f(F(beta)), f(F(mean))
+    w = fl32(fl32(fl32(g * invstd) * max_abs_data) / max_abs_out)
+    b = fl32(fl32(fl32(b_ - fl32(fl32(m * g) * invstd)) * Fraction(255, 2)) / max_abs_out)
+    unit = f(np.sqrt(F(1.0) + F(eps), dtype=np.float32))
+    wn = fl32(w / unit)
+    if unsigned:
+        x = max(-128, min(127, round_half_even(fl32(Fraction(int(x)) * f(F(127.5) / F(255.5))))))
+    v = fl32(fl32(Fraction(int(x)) * wn) + b)
+    if relu and v < 0:
+        v = Fraction(0)
+    return max(-128, min(127, round_half_even(v)))
+
+
+@pytest.mark.parametrize("dtype", [np.int8, np.uint8])
+@pytest.mark.parametrize("relu", [False, True])
+@pytest.mark.parametrize("eps", [1e-3, 2e-5])
+def test_batch_norm_rule_exactly(dtype, relu, eps):
+    rng = np.random.default_rng(13)
+    C = 5
+    lo, hi = (0, 256) if dtype == np.uint8 else (-128, 128)
+    d = rng.integers(lo, hi, (3, C, 7)).astype(dtype)
+    gamma = rng.uniform(0.5, 2.0, C).astype(np.float32)
+    beta = rng.normal(0, 0.5, C).astype(np.float32)
+    mean = rng.normal(0, 0.3, C).astype(np.float32)
+    var = rng.uniform(0.3, 2.0, C).astype(np.float32)
+    rd = (0.0, 3.1) if dtype == np.uint8 else (-2.7, 3.1)
+    calib = (-6.5, 7.25)
+    out, mn, mx = qref.quantized_batch_norm(d, gamma, beta, mean, var, rd[0], rd[1], calib[0],
+                                            calib[1], eps=eps, relu=relu)
+    assert out.dtype == np.int8 and (mn, mx) == (F(calib[0]), F(calib[1]))
+    for idx in np.ndindex(*d.shape):
+        c = idx[1]
+        assert int(out[idx]) == exact_bn(d[idx], dtype == np.uint8, gamma[c], beta[c], mean[c],
+                                         var[c], rd[0], rd[1], eps, calib, relu), idx
+
+
+@pytest.mark.parametrize("shape,axis", [((8, 16, 4, 4), 1), ((4, 6, 5, 3), -1), ((10, 7), 1)])
+def test_batch_norm_tracks_the_float_operator(shape, axis):
+    """check_quantized_bn (test_quantization.py:1005-1050): the dequantized int8 result is the
+    float batch norm within rtol 0.1 / atol 8 there; within 1.5 output levels + the 0.05 %
+    that the library's second division by sqrt(1 + eps) costs here."""
+    rng = np.random.default_rng(17)
+    C = shape[axis]
+    d = rng.integers(-127, 128, shape).astype(np.int8)
+    gamma = rng.uniform(0.5, 2.0, C).astype(np.float32)
+    beta = rng.normal(0, 0.5, C).astype(np.float32)
+    mean = rng.normal(0, 0.3, C).astype(np.float32)
+    var = rng.uniform(0.5, 2.0, C).astype(np.float32)
+    rd = 3.0
+    bshape = [1] * len(shape)
+    bshape[axis] = C
+    real = d.astype(np.float64) * rd / 127.5
+    want = (real - mean.reshape(bshape)) / np.sqrt(var.reshape(bshape) + 1e-3) * \
+        gamma.reshape(bshape) + beta.reshape(bshape)
+    R = float(np.abs(want).max())
+    out, mn, mx = qref.quantized_batch_norm(d, gamma, beta, mean, var, -rd, rd, -R, R, eps=1e-3,
+                                            axis=axis)
+    back = out.astype(np.float64) * R / 127.5
+    assert np.abs(back - want).max() <= 1.5 * R / 127.5 + 1e-3 * R
+    relu, _, _ = qref.quantized_batch_norm(d, gamma, beta, mean, var, -rd, rd, -R, R, eps=1e-3,
+                                           axis=axis, relu=True)
+    assert np.array_equal(relu, np.maximum(out, 0))
+    with pytest.raises(ValueError):
+        qref.quantized_batch_norm(d, gamma, beta, mean, var, -rd, rd, None, None)
