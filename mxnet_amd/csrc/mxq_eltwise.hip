@@ -179,13 +179,15 @@ __device__ __forceinline__ void add_bytes(const AddArgs& a, const AddRule<OUT, L
       x[j] = __builtin_nontemporal_load(l16 + q + j * stride);
       y[j] = __builtin_nontemporal_load(r16 + q + j * stride);
     }
+    // both results before the first store: the stores are opaque to the compiler's count of
+    // outstanding memory operations, a wait placed behind one would wait for it too
+    u4 v[2];
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      u4 v;
+    for (int j = 0; j < 2; ++j)
 #pragma unroll
-      for (int w = 0; w < 4; ++w) v[w] = r.template apply4<FAST>(x[j][w], y[j][w]);
-      stream_store16(v, o16 + q + j * stride);
-    }
+      for (int w = 0; w < 4; ++w) v[j][w] = r.template apply4<FAST>(x[j][w], y[j][w]);
+#pragma unroll
+    for (int j = 0; j < 2; ++j) stream_store16(v[j], o16 + q + j * stride);
   }
   for (; q < nv; q += stride) {
     const u4 x = l16[q], y = r16[q];
