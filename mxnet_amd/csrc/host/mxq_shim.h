@@ -100,10 +100,10 @@ enum TypeFlag {
 enum LayoutFlag { kNCHW = 0, kNHWC, kCHWN, kNCW = 1 << 3, kNWC, kCWN, kNCDHW = 1 << 5, kNDHWC, kCDHWN };
 
 struct cpu {
-  static const int kDevMask = 1;
+  static constexpr int kDevMask = 1;
 };
 struct gpu {
-  static const int kDevMask = 2;
+  static constexpr int kDevMask = 2;
 };
 
 // The reference's Stream<gpu> owns a cudaStream_t plus cuBLAS/cuDNN handles
