@@ -104,6 +104,17 @@ def quantized_transpose(data, min_data, max_data, axes=()):
     return invoke("_contrib_quantized_transpose", data, min_data, max_data, axes=axes)
 
 
+def npx_quantized_reshape(data, min_data, max_data, newshape, reverse=False, order="C"):
+    """_npx_quantized_reshape: numpy-namespace reshape, newshape with -1 ... -6."""
+    return invoke("_npx_quantized_reshape", data, min_data, max_data, newshape=newshape,
+                  reverse=reverse, order=order)
+
+
+def npx_quantized_transpose(data, min_data, max_data, axes=None):
+    """_npx_quantized_transpose: axes None reverses; negative axes count from the end."""
+    return invoke("_npx_quantized_transpose", data, min_data, max_data, axes=axes)
+
+
 def quantize_asym(data, min_calib_range=None, max_calib_range=None):
     return invoke("_contrib_quantize_asym", data, min_calib_range=min_calib_range,
                   max_calib_range=max_calib_range)

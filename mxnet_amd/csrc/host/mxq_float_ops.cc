@@ -273,5 +273,24 @@ NNVM_REGISTER_OP(transpose)
       return QuantizedTwin(attrs, "_contrib_quantized_transpose");
     });
 
+// src/operator/numpy/np_matrix_op.cc:353-375, quantized_reshape.cc:125-126
+NNVM_REGISTER_OP(_npx_reshape)
+    .add_alias("_npi_reshape")
+    .set_num_inputs(1)
+    .set_num_outputs(1)
+    .set_attr_parser(ParamParser<NumpyXReshapeParam>)
+    .set_attr<FQuantizedOp>("FQuantizedOp", [](const NodeAttrs& attrs) {
+      return QuantizedTwin(attrs, "_npx_quantized_reshape");
+    });
+
+// src/operator/numpy/np_matrix_op.cc:80-110, quantized_transpose.cc:118-127
+NNVM_REGISTER_OP(_npi_transpose)
+    .set_num_inputs(1)
+    .set_num_outputs(1)
+    .set_attr_parser(ParamParser<NumpyTransposeParam>)
+    .set_attr<FQuantizedOp>("FQuantizedOp", [](const NodeAttrs& attrs) {
+      return QuantizedTwin(attrs, "_npx_quantized_transpose");
+    });
+
 }  // namespace op
 }  // namespace mxnet

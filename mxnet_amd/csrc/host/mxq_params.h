@@ -725,6 +725,48 @@ struct TransposeParam {
   }
 };
 
+// src/operator/numpy/np_matrix_op-inl.h:44-62: unknown axes (the default) reverse the
+// dimensions; negative axes count from the end
+struct NumpyTransposeParam {
+  TShape axes;  // ndim -1: not given
+  void Init(const param_detail::Dict& d) {
+    using namespace param_detail;
+    check_unknown(d, {"axes"}, "NumpyTransposeParam");
+    axes = d.count("axes") ? get_shape(d, "axes", true) : TShape();
+  }
+  static std::vector<nnvm::ParamFieldInfo> __FIELDS__() {
+    return {{"axes", "Shape(tuple), optional, default=None",
+             "By default, reverse the dimensions, otherwise permute the axes according to the "
+             "values given."}};
+  }
+};
+
+// src/operator/numpy/np_matrix_op-inl.h:109-146
+struct NumpyXReshapeParam {
+  TShape newshape;  // with the special values -1 ... -6
+  bool reverse = false;
+  std::string order = "C";
+  void Init(const param_detail::Dict& d) {
+    using namespace param_detail;
+    check_unknown(d, {"newshape", "reverse", "order"}, "NumpyXReshapeParam");
+    newshape = get_shape(d, "newshape", false);
+    reverse = get_bool(d, "reverse", false);
+    auto it = d.find("order");
+    if (it != d.end()) order = trim(it->second);
+  }
+  static std::vector<nnvm::ParamFieldInfo> __FIELDS__() {
+    return {{"newshape", "Shape(tuple), required",
+             "The new shape should be compatible with the original shape. One shape dimension "
+             "can be -1 (inferred); -2 copies a dimension, -3 skips a dimension of size one, -4 "
+             "copies all remaining dimensions, -5 merges two dimensions, -6 splits one dimension "
+             "into the two that follow."},
+            {"reverse", "boolean, optional, default=0",
+             "If true then the special values are inferred from right to left"},
+            {"order", "string, optional, default='C'",
+             "Only C-like index order is supported"}};
+  }
+};
+
 // src/operator/tensor/broadcast_reduce_op.h:240-249: a negative axis counts from the end
 inline int CheckAxis(const int axis, const int ndim) {
   if (ndim == 0) {

@@ -300,16 +300,140 @@ bool ReshapeShape(const NodeAttrs& attrs, ShapeVector* in_attrs, ShapeVector* ou
   return ReverseReshapeInferShape(&(*in_attrs)[0], (*out_attrs)[0]);
 }
 
+// np_matrix_op.cc:180-289
+bool NumpyXReshapeInferShape(const TShape& src, const TShape& target, TShape* output,
+                             const std::string& default_error_msg) {
+  bool target_shape_is_known = true;
+  index_t target_size = 1;
+  for (int i = 0; i < target.ndim(); ++i) {
+    if (target[i] < 0) {
+      target_shape_is_known = false;
+      target_size = -1;
+      break;
+    }
+    target_size *= target[i];
+  }
+  if (shape_is_known(src) && target_shape_is_known) {
+    CHECK_EQ(static_cast<index_t>(src.Size()), target_size) << default_error_msg;
+    *output = target;
+    return true;
+  }
+  if (!shape_is_known(src) || target.ndim() == -1) return false;
+  int unknown_axis = -1;
+  index_t known_dim_size_prod = 1;
+  std::vector<index_t> out;
+  int src_inx = 0;
+  for (int i = 0; i < target.ndim(); ++i) {
+    const index_t proposed_dim = target[i];
+    CHECK(proposed_dim >= -6) << "Dimension size must be greater than -6, received "
+                              << proposed_dim;
+    if (proposed_dim == -1) {
+      CHECK_LT(unknown_axis, 0) << "One and only one dim can be inferred";
+      unknown_axis = static_cast<int>(out.size());
+      out.push_back(-1);
+      src_inx++;
+    } else if (proposed_dim == -2) {
+      CHECK_LT(src_inx, src.ndim()) << "Unmatching dimension of proposed new shape";
+      known_dim_size_prod *= src[src_inx];
+      out.push_back(src[src_inx++]);
+    } else if (proposed_dim == -3) {
+      CHECK_LT(src_inx, src.ndim()) << "Unmatching dimension of proposed new shape";
+      CHECK_EQ(src[src_inx], 1) << "-3 index should only be used to skip dimension size 1";
+      src_inx++;
+    } else if (proposed_dim == -4) {
+      while (src_inx < src.ndim()) {
+        known_dim_size_prod *= src[src_inx];
+        out.push_back(src[src_inx++]);
+      }
+    } else if (proposed_dim == -5) {
+      CHECK_LT(src_inx, src.ndim() - 1) << "Not enough dimensions left for the product";
+      const index_t d1 = src[src_inx++];
+      const index_t d2 = src[src_inx++];
+      known_dim_size_prod *= d1 * d2;
+      out.push_back(d1 * d2);
+    } else if (proposed_dim == -6) {
+      CHECK_LT(i + 2, target.ndim());
+      CHECK_LT(src_inx, src.ndim());
+      const index_t d0 = src[src_inx++];
+      index_t d1 = target[++i];
+      index_t d2 = target[++i];
+      CHECK(d1 != -1 || d2 != -1) << "Split dims cannot both be -1.";
+      CHECK(d1 != 0 && d2 != 0) << "Split dims " << d1 << ", " << d2
+                                << " do not divide original dim " << d0;
+      if (d1 == -1) d1 = d0 / d2;
+      if (d2 == -1) d2 = d0 / d1;
+      CHECK(d1 * d2 == d0) << "Split dims " << d1 << ", " << d2
+                           << " do not divide original dim " << d0;
+      known_dim_size_prod *= d0;
+      out.push_back(d1);
+      out.push_back(d2);
+    } else {
+      known_dim_size_prod *= proposed_dim;
+      out.push_back(proposed_dim);
+      src_inx++;
+    }
+  }
+  if (unknown_axis > -1) {
+    CHECK_NE(known_dim_size_prod, 0) << default_error_msg;
+    CHECK(static_cast<index_t>(src.Size()) % known_dim_size_prod == 0) << default_error_msg;
+    out[unknown_axis] = static_cast<index_t>(src.Size()) / known_dim_size_prod;
+  }
+  *output = TShape(out);
+  CHECK_EQ(output->Size(), src.Size()) << default_error_msg;
+  return true;
+}
+
+// np_matrix_op.cc:291-327
+bool NumpyXReshapeShape(const NodeAttrs& attrs, ShapeVector* in_attrs, ShapeVector* out_attrs) {
+  CHECK_EQ(in_attrs->size(), 1U) << "Input: [data]";
+  CHECK_EQ(out_attrs->size(), 1U);
+  const NumpyXReshapeParam& param = nnvm::get<NumpyXReshapeParam>(attrs.parsed);
+  CHECK(param.order == "C") << "only C-like index order is supported, got " << param.order;
+  bool has_unknown_dim_size = false;
+  for (int i = 0; i < param.newshape.ndim(); ++i) {
+    if (param.newshape[i] < 0) {
+      CHECK_GE(param.newshape[i], -6) << "Dimension size must be greater than or equal to -6";
+      if (param.newshape[i] == -1) {
+        CHECK(!has_unknown_dim_size) << "Can only specify one unknown dimension";
+        has_unknown_dim_size = true;
+      }
+    }
+  }
+  TShape output_shape;
+  bool success;
+  std::ostringstream ss;
+  ss << "Cannot reshape array of shape " << in_attrs->at(0) << " into shape " << param.newshape
+     << " , reverse = " << param.reverse;
+  if (!param.reverse) {
+    success = NumpyXReshapeInferShape(in_attrs->at(0), param.newshape, &output_shape, ss.str());
+  } else {
+    std::vector<index_t> rin, rnew;
+    for (int i = in_attrs->at(0).ndim() - 1; i >= 0; --i) rin.push_back(in_attrs->at(0)[i]);
+    for (int i = param.newshape.ndim() - 1; i >= 0; --i) rnew.push_back(param.newshape[i]);
+    if (!ndim_is_known(in_attrs->at(0))) return false;
+    success = NumpyXReshapeInferShape(TShape(rin), TShape(rnew), &output_shape, ss.str());
+    if (success) {
+      std::vector<index_t> rev;
+      for (int i = output_shape.ndim() - 1; i >= 0; --i) rev.push_back(output_shape[i]);
+      output_shape = TShape(rev);
+    }
+  }
+  if (!success) return false;
+  SHAPE_ASSIGN_CHECK(*out_attrs, 0, output_shape);
+  return true;
+}
+
 }  // namespace
 
 // quantized_reshape-inl.h:38-56
+template <bool (*Inner)(const NodeAttrs&, ShapeVector*, ShapeVector*)>
 static bool QuantizedReshapeShape(const NodeAttrs& attrs, ShapeVector* in_attrs,
                                   ShapeVector* out_attrs) {
   CHECK_EQ(in_attrs->size(), 3U);
   CHECK_EQ(out_attrs->size(), 3U);
   ShapeVector input = {in_attrs->at(0)};
   ShapeVector output = {out_attrs->at(0)};
-  const bool ret = ReshapeShape(attrs, &input, &output);
+  const bool ret = Inner(attrs, &input, &output);
   SHAPE_ASSIGN_CHECK(*in_attrs, 1, kScalarShape);
   SHAPE_ASSIGN_CHECK(*in_attrs, 2, kScalarShape);
   SHAPE_ASSIGN_CHECK(*out_attrs, 0, output[0]);
@@ -381,9 +505,80 @@ bool TransposeShape(const NodeAttrs& attrs, ShapeVector* in_attrs, ShapeVector* 
   return shape_is_known(ret);
 }
 
+// src/common/utils.h:917-929
+TShape CanonicalizeAxes(const TShape& src) {
+  const int ndim = src.ndim();
+  TShape axes = src;
+  for (int i = 0; i < ndim; ++i) {
+    if (axes[i] < 0) axes[i] += ndim;
+    CHECK(axes[i] >= 0 && axes[i] < ndim)
+        << "axes[" << i << "]=" << axes[i] << " exceeds the range [" << 0 << ", " << ndim << ")";
+  }
+  return axes;
+}
+
+// np_matrix_op-inl.h:179-234
+bool NumpyTransposeShape(const NodeAttrs& attrs, ShapeVector* in_attrs, ShapeVector* out_attrs) {
+  const NumpyTransposeParam& param = nnvm::get<NumpyTransposeParam>(attrs.parsed);
+  CHECK_EQ(in_attrs->size(), 1U);
+  CHECK_EQ(out_attrs->size(), 1U);
+  TShape& shp = (*in_attrs)[0];
+  TShape& out_shp = (*out_attrs)[0];
+  int ndim = -1;
+  if (ndim_is_known(shp)) {
+    ndim = shp.ndim();
+  } else if (ndim_is_known(out_shp)) {
+    ndim = out_shp.ndim();
+  }
+  if (ndim < 0) return false;
+  if (out_shp.ndim() >= 0 && shp.ndim() >= 0) CHECK_EQ(out_shp.ndim(), shp.ndim());
+  TShape get(ndim, -1), ret(ndim, -1);
+  if (ndim_is_known(param.axes)) {
+    CHECK_EQ(ndim, param.axes.ndim())
+        << "The number of axes does not match the dimension of the tensor. axes = " << param.axes
+        << ", input tensor shape = " << shp;
+    const TShape axes = CanonicalizeAxes(param.axes);
+    std::vector<bool> seen(ndim, false);
+    for (int i = 0; i < ndim; ++i) {
+      CHECK(!seen[axes[i]]) << "ValueError: Repeated axis in transpose. param.axes = "
+                            << param.axes;
+      seen[axes[i]] = true;
+    }
+    if (ndim_is_known(shp))
+      for (int i = 0; i < ndim; ++i) ret[i] = shp[static_cast<int>(axes[i])];
+    if (ndim_is_known(out_shp))
+      for (int i = 0; i < ndim; ++i) get[static_cast<int>(axes[i])] = out_shp[i];
+  } else {
+    if (ndim_is_known(shp))
+      for (int i = 0; i < ndim; ++i) ret[i] = shp[ndim - 1 - i];
+    if (ndim_is_known(out_shp))
+      for (int i = 0; i < ndim; ++i) get[ndim - 1 - i] = out_shp[i];
+  }
+  SHAPE_ASSIGN_CHECK(*in_attrs, 0, get);
+  SHAPE_ASSIGN_CHECK(*out_attrs, 0, ret);
+  return shape_is_known((*in_attrs)[0]) && shape_is_known((*out_attrs)[0]);
+}
+
+// the permutation an operator instance applies to data of `ndim` axes; empty = reverse
+std::vector<int> transpose_axes(const TransposeParam& param, int) {
+  std::vector<int> axes(param.axes.ndim());
+  for (int i = 0; i < param.axes.ndim(); ++i) axes[i] = static_cast<int>(param.axes[i]);
+  return axes;
+}
+std::vector<int> transpose_axes(const NumpyTransposeParam& param, int ndim) {
+  std::vector<int> axes;
+  if (!ndim_is_known(param.axes)) return axes;
+  CHECK_EQ(param.axes.ndim(), ndim);
+  const TShape canon = CanonicalizeAxes(param.axes);
+  for (int i = 0; i < ndim; ++i) axes.push_back(static_cast<int>(canon[i]));
+  if (axes.empty()) axes.push_back(0);  // never reached with data: 0-d has nothing to permute
+  return axes;
+}
+
 }  // namespace
 
 // quantized_transpose.cc:49-66
+template <bool (*Inner)(const NodeAttrs&, ShapeVector*, ShapeVector*)>
 static bool QuantizedTransposeShape(const NodeAttrs& attrs, ShapeVector* in_attrs,
                                     ShapeVector* out_attrs) {
   CHECK_EQ(in_attrs->size(), 3U);
@@ -391,7 +586,7 @@ static bool QuantizedTransposeShape(const NodeAttrs& attrs, ShapeVector* in_attr
   ShapeVector qin_attrs(1), qout_attrs(1);
   SHAPE_ASSIGN_CHECK(qin_attrs, 0, (*in_attrs)[0]);
   SHAPE_ASSIGN_CHECK(qout_attrs, 0, (*out_attrs)[0]);
-  const bool ret = TransposeShape(attrs, &qin_attrs, &qout_attrs);
+  const bool ret = Inner(attrs, &qin_attrs, &qout_attrs);
   SHAPE_ASSIGN_CHECK(*in_attrs, 0, qin_attrs[0]);
   SHAPE_ASSIGN_CHECK(*out_attrs, 0, qout_attrs[0]);
   SHAPE_ASSIGN_CHECK(*in_attrs, 1, kScalarShape);
@@ -402,11 +597,12 @@ static bool QuantizedTransposeShape(const NodeAttrs& attrs, ShapeVector* in_attr
 }
 
 // dnnl_quantized_transpose.cc: the float transpose on one-byte elements, ranges copied
+template <typename Param>
 static void QuantizedTransposeForwardGPU(const NodeAttrs& attrs, const OpContext& ctx,
                                          const std::vector<TBlob>& inputs,
                                          const std::vector<OpReqType>& req,
                                          const std::vector<TBlob>& outputs) {
-  const TransposeParam& param = nnvm::get<TransposeParam>(attrs.parsed);
+  const Param& param = nnvm::get<Param>(attrs.parsed);
   CHECK_EQ(inputs.size(), 3U);
   CHECK_EQ(outputs.size(), 3U);
   CHECK(req[0] == kWriteTo) << "Transpose does not support inplace";
@@ -415,8 +611,8 @@ static void QuantizedTransposeForwardGPU(const NodeAttrs& attrs, const OpContext
   const TShape& shp = inputs[0].shape_;
   std::vector<int64_t> dims(shp.ndim());
   for (int i = 0; i < shp.ndim(); ++i) dims[i] = shp[i];
-  std::vector<int> axes(param.axes.ndim());
-  for (int i = 0; i < param.axes.ndim(); ++i) axes[i] = static_cast<int>(param.axes[i]);
+  std::vector<int> axes = transpose_axes(param, shp.ndim());
+  if (shp.ndim() == 0) axes.clear();
   if (!axes.empty()) CHECK_EQ(axes.size(), dims.size());
   MXQ_CALL(mxq_quantized_transpose(raw_stream(ctx), inputs[0].dptr_, inputs[1].dptr<float>(),
                                    inputs[2].dptr<float>(), outputs[0].dptr_,
@@ -645,7 +841,7 @@ NNVM_REGISTER_OP(_contrib_quantized_reshape)
                                     [](const NodeAttrs&) {
                                       return std::vector<std::pair<int, int>>{{0, 0}, {1, 1}, {2, 2}};
                                     })
-    .set_attr<mxnet::FInferShape>("FInferShape", QuantizedReshapeShape)
+    .set_attr<mxnet::FInferShape>("FInferShape", QuantizedReshapeShape<ReshapeShape>)
     .set_attr<nnvm::FInferType>("FInferType", PassThroughType)
     .set_attr<FCompute>("FCompute<gpu>", QuantizedReshapeComputeGPU)
     .set_attr<FQuantizable>("FQuantizable",
@@ -665,9 +861,9 @@ NNVM_REGISTER_OP(_contrib_quantized_transpose)
     .set_attr_parser(ParamParser<TransposeParam>)
     .set_attr<nnvm::FListInputNames>("FListInputNames", DataMinMax)
     .set_attr<nnvm::FListOutputNames>("FListOutputNames", OutputMinMax)
-    .set_attr<mxnet::FInferShape>("FInferShape", QuantizedTransposeShape)
+    .set_attr<mxnet::FInferShape>("FInferShape", QuantizedTransposeShape<TransposeShape>)
     .set_attr<nnvm::FInferType>("FInferType", PassThroughType)
-    .set_attr<FCompute>("FCompute<gpu>", QuantizedTransposeForwardGPU)
+    .set_attr<FCompute>("FCompute<gpu>", QuantizedTransposeForwardGPU<TransposeParam>)
     .set_attr<FQuantizable>("FQuantizable",
                             [](const NodeAttrs&) { return QuantizeType::kSupport; })
     .add_argument("data", "NDArray-or-Symbol", "Array to be transposed.")
@@ -676,6 +872,48 @@ NNVM_REGISTER_OP(_contrib_quantized_transpose)
     .add_argument("max_data", "NDArray-or-Symbol",
                   "The maximum scalar value possibly produced for the data")
     .add_arguments(TransposeParam::__FIELDS__());
+
+// quantized_reshape.cc:91-100: the numpy-namespace form, newshape with -1 ... -6
+NNVM_REGISTER_OP(_npx_quantized_reshape)
+    .set_num_inputs(3)
+    .set_num_outputs(3)
+    .set_attr_parser(ParamParser<NumpyXReshapeParam>)
+    .set_attr<nnvm::FListInputNames>("FListInputNames", DataMinMax)
+    .set_attr<nnvm::FListOutputNames>("FListOutputNames", OutputMinMax)
+    .set_attr<nnvm::FInplaceOption>("FInplaceOption",
+                                    [](const NodeAttrs&) {
+                                      return std::vector<std::pair<int, int>>{{0, 0}, {1, 1}, {2, 2}};
+                                    })
+    .set_attr<mxnet::FInferShape>("FInferShape", QuantizedReshapeShape<NumpyXReshapeShape>)
+    .set_attr<nnvm::FInferType>("FInferType", PassThroughType)
+    .set_attr<FCompute>("FCompute<gpu>", QuantizedReshapeComputeGPU)
+    .set_attr<FQuantizable>("FQuantizable",
+                            [](const NodeAttrs&) { return QuantizeType::kSupport; })
+    .add_argument("data", "NDArray-or-Symbol", "Array to be reshaped.")
+    .add_argument("min_data", "NDArray-or-Symbol",
+                  "The minimum scalar value possibly produced for the data")
+    .add_argument("max_data", "NDArray-or-Symbol",
+                  "The maximum scalar value possibly produced for the data")
+    .add_arguments(NumpyXReshapeParam::__FIELDS__());
+
+// quantized_transpose.cc:96-99: the numpy-namespace form, negative axes allowed
+NNVM_REGISTER_OP(_npx_quantized_transpose)
+    .set_num_inputs(3)
+    .set_num_outputs(3)
+    .set_attr_parser(ParamParser<NumpyTransposeParam>)
+    .set_attr<nnvm::FListInputNames>("FListInputNames", DataMinMax)
+    .set_attr<nnvm::FListOutputNames>("FListOutputNames", OutputMinMax)
+    .set_attr<mxnet::FInferShape>("FInferShape", QuantizedTransposeShape<NumpyTransposeShape>)
+    .set_attr<nnvm::FInferType>("FInferType", PassThroughType)
+    .set_attr<FCompute>("FCompute<gpu>", QuantizedTransposeForwardGPU<NumpyTransposeParam>)
+    .set_attr<FQuantizable>("FQuantizable",
+                            [](const NodeAttrs&) { return QuantizeType::kSupport; })
+    .add_argument("data", "NDArray-or-Symbol", "Array to be transposed.")
+    .add_argument("min_data", "NDArray-or-Symbol",
+                  "The minimum scalar value possibly produced for the data")
+    .add_argument("max_data", "NDArray-or-Symbol",
+                  "The maximum scalar value possibly produced for the data")
+    .add_arguments(NumpyTransposeParam::__FIELDS__());
 
 // quantize_asym.cc:100-157
 NNVM_REGISTER_OP(_contrib_quantize_asym)

@@ -134,6 +134,9 @@ def cases():
     out.append(("_contrib_quantized_batch_norm_relu", dict(eps=1e-3, min_calib_range=-6.5,
                                                            max_calib_range=7.25),
                 [bd.view(np.uint8)] + bn + [s(0.0), s(3.1)]))
+    out.append(("_npx_quantized_transpose", dict(axes=(-1, 0, -2, 1)), [t, s(-1.0), s(1.0)]))
+    out.append(("_npx_quantized_reshape", dict(newshape=(-2, -5, -6, 4, -1)),
+                [t, s(-1.0), s(1.0)]))
     return out
 
 
@@ -190,6 +193,12 @@ def run_oracle(op, attrs, ins):
         # (0, -3, -1) on (3, 5, 4, 16): keep, merge two, infer the rest
         assert tuple(attrs["shape"]) == (0, -3, -1) and ins[0].shape == (3, 5, 4, 16)
         res = oracle.quantized_reshape(ins[0], f(ins[1]), f(ins[2]), (3, 20, 16))
+    elif op == "_npx_quantized_transpose":
+        res = oracle.quantized_transpose(ins[0], f(ins[1]), f(ins[2]), tuple(attrs["axes"]))
+    elif op == "_npx_quantized_reshape":
+        # (-2, -5, -6, 4, -1) on (3, 5, 4, 16): copy, merge two, split the last into 4 x 4
+        assert tuple(attrs["newshape"]) == (-2, -5, -6, 4, -1) and ins[0].shape == (3, 5, 4, 16)
+        res = oracle.quantized_reshape(ins[0], f(ins[1]), f(ins[2]), (3, 20, 4, 4))
     elif op == "_contrib_quantize_asym":
         res = oracle.quantize_asym(ins[0], *cal)
     elif op in ("_contrib_quantized_batch_norm", "_contrib_quantized_batch_norm_relu"):

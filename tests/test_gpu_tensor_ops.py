@@ -430,3 +430,32 @@ def test_quantized_batch_norm_errors(lib, contrib):
     rc = lib.lib.mxq_quantized_batch_norm(stream(), P(x), 0, P(v), P(v), P(v), P(v), P(s), P(s),
                                           P(out), P(s), P(s), 2, 4, 3, 1e-3, -1.0, 1.0, 0, P(v), 64)
     assert rc != 0 and "int8/uint8" in lib.last_error()
+
+
+# ---- numpy-namespace reshape / transpose ----------------------------------------------------
+
+@pytest.mark.parametrize("shape,axes", [((3, 5, 7), None), ((3, 5, 7), (-1, 0, 1)),
+                                        ((2, 16, 8, 64), (0, -2, 1, 3)), ((4, 6), (1, 0)),
+                                        ((5,), None), ((2, 3, 4, 5, 6), (-1, -3, 0, 1, 3))])
+@pytest.mark.parametrize("dtype", [np.int8, np.uint8])
+def test_npx_quantized_transpose(contrib, shape, axes, dtype):
+    rng = np.random.default_rng(len(shape))
+    d = rng.integers(0, 128, shape).astype(dtype)
+    out, mn, mx = contrib.npx_quantized_transpose(dev(d), scalar(-1.5), scalar(2.0), axes=axes)
+    np.testing.assert_array_equal(host(out), np.transpose(d, axes))
+    assert (host(mn)[0], host(mx)[0]) == (np.float32(-1.5), np.float32(2.0))
+
+
+@pytest.mark.parametrize("shape,newshape,reverse,want", [
+    ((2, 3, 8), (-2, -2, 2, -1), False, (2, 3, 2, 4)),
+    ((8, 3, 2, 4, 8), (-4, -1, 2, -6), True, (8, 3, 2, 4, 4, 2)),
+    ((64, 1, 2, 3), (-6, 16, -1, -4), False, (16, 4, 1, 2, 3)),
+    ((1, 1, 1, 1), (-3, -3, -3, -3), False, ()),
+    ((2, 3, 5, 6), (-5, -1), False, (6, 30))])
+def test_npx_quantized_reshape(contrib, shape, newshape, reverse, want):
+    d = np.random.default_rng(3).integers(-128, 128, shape).astype(np.int8)
+    out, mn, mx = contrib.npx_quantized_reshape(dev(d), scalar(-1.5), scalar(2.0), newshape,
+                                                reverse=reverse)
+    assert tuple(out.shape) == want
+    np.testing.assert_array_equal(host(out), d.reshape(want))
+    assert (host(mn)[0], host(mx)[0]) == (np.float32(-1.5), np.float32(2.0))

@@ -1,6 +1,7 @@
 """The C++ operator host on the CPU: registry contents, attribute parsing, shape and
 type inference (no kernel is launched).  Expected values are read off the reference's
 registrations and inference functions (src/operator/quantization/*.cc, *-inl.h)."""
+import numpy as np
 import pytest
 import torch
 
@@ -378,3 +379,78 @@ def test_quantized_batch_norm_registration_and_inference():
     # the float BatchNorm keeps no FQuantizedOp here: the pass leaves it float, as the
     # reference does for the gpu context
     assert not op.has_attr("BatchNorm", "FQuantizedOp")
+
+
+# (input shape, newshape, reverse, output shape): the examples of the reference's npx.reshape
+# documentation (python/mxnet/_numpy_op_doc.py:607-624), the cases of its own test
+# (tests/python/unittest/test_numpy_op.py:9316-9334), then inputs it must refuse
+NPX_RESHAPE_EXAMPLES = [
+    ((2, 3, 8), (-2, -2, 2, -1), False, (2, 3, 2, 4)),
+    ((8, 3, 3, 3, 4, 4), (-6, 2, -1, -4), False, (2, 4, 3, 3, 3, 4, 4)),
+    ((8, 3, 3, 3, 4, 4), (-5, -4), False, (24, 3, 3, 4, 4)),
+    ((8, 1, 1, 1, 3), (-2, -3, -3, -3, -2), False, (8, 3)),
+    ((8, 3, 3, 3, 3, 8), (-4, -5), True, (8, 3, 3, 3, 24)),
+    ((8, 3, 2, 4, 8), (-4, -1, 2, -6), True, (8, 3, 2, 4, 4, 2)),
+    ((2, 3, 5, 5), (-2, -1), False, (2, 75)),
+    ((2, 3, 5, 5), (-2, -2, -1), False, (2, 3, 25)),
+    ((5, 3, 4, 5), (-2, -1, -2), False, (5, 15, 4)),
+    ((2, 3, 5, 4), (-1, -2, -2), False, (8, 3, 5)),
+    ((2, 3, 5, 5), (-2, -2, -2, -2), False, (2, 3, 5, 5)),
+    ((2, 1, 4, 5), (-2, -3, -2, -2), False, (2, 4, 5)),
+    ((1, 1, 4, 1), (-3, -3, -2, -2), False, (4, 1)),
+    ((1, 1, 1, 1), (-3, -3, -3, -3), False, ()),
+    ((2, 4, 5, 3), (-1, 2, 2, 1), False, (30, 2, 2, 1)),
+    ((2, 3, 5, 6), (-4,), False, (2, 3, 5, 6)),
+    ((2, 3, 5, 6), (6, 1, -4), False, (6, 1, 5, 6)),
+    ((2, 3, 5, 6), (-5, -5), False, (6, 30)),
+    ((2, 3, 5, 6), (-5, -1), False, (6, 30)),
+    ((64,), (-6, 16, 4), False, (16, 4)),
+    ((64,), (-6, 16, -1), False, (16, 4)),
+    ((64, 1, 2, 3), (-6, 16, -1, -4), False, (16, 4, 1, 2, 3)),
+    ((8, 5, 4, 6), (-4, -1, 3, -6), True, (8, 5, 4, 2, 3)),
+    ((2, 3, 8), (6, 8), False, (6, 8)),
+    ((0, 3), (-1,), False, (0,)),
+    ((0, 3), (-1, 0), False, None),
+    ((2, 3, 8), (5, -1), False, None),
+    ((2, 3, 8), (-2, -3, -4), False, None),
+    ((2, 3, 8), (-6, 3, 2, -4), False, None),
+    ((2, 3, 8), (-1, -1), False, None),
+    ((2, 3, 8), (-7,), False, None),
+]
+
+
+def test_numpy_namespace_reshape_and_transpose_inference():
+    """quantized_reshape.cc:91-100, quantized_transpose.cc:96-99."""
+    for n in ["_npx_quantized_reshape", "_npx_quantized_transpose"]:
+        assert op.has_attr(n, "FCompute<gpu>") and op.has_attr(n, "FQuantizable")
+    assert op.has_attr("_npx_reshape", "FQuantizedOp") and op.has_attr("_npi_reshape", "FQuantizedOp")
+    assert op.has_attr("_npi_transpose", "FQuantizedOp")
+    for shape, newshape, reverse, want in NPX_RESHAPE_EXAMPLES:
+        node = Node("_npx_quantized_reshape", newshape=newshape, reverse=reverse)
+        if want is None:
+            with pytest.raises(MXNetError):
+                node.infer_shape([shape, None, None])
+            continue
+        ins, outs = node.infer_shape([shape, None, None])
+        assert outs == [want, (1,), (1,)], (shape, newshape, reverse)
+        assert ins == [shape, (1,), (1,)]
+        # numpy agrees wherever the special values reduce to a plain reshape
+        assert np.zeros(shape, np.int8).reshape(want).shape == want
+    with pytest.raises(MXNetError):
+        Node("_npx_quantized_reshape")
+    with pytest.raises(MXNetError, match="order"):
+        Node("_npx_quantized_reshape", newshape=(-1,), order="F").infer_shape([(2, 3), None, None])
+    assert Node("_npx_quantized_reshape", newshape=(-1,)).infer_type([I8, None, None]) == \
+        ([I8, F32, F32], [I8, F32, F32])
+
+    t = Node("_npx_quantized_transpose")
+    assert t.infer_shape([(2, 3, 4), None, None])[1] == [(4, 3, 2), (1,), (1,)]
+    t = Node("_npx_quantized_transpose", axes=(-1, 0, -2))
+    assert t.infer_shape([(2, 3, 4), None, None])[1] == [(4, 2, 3), (1,), (1,)]
+    assert t.infer_type([U8, None, None])[1] == [U8, F32, F32]
+    with pytest.raises(MXNetError, match="Repeated axis"):
+        Node("_npx_quantized_transpose", axes=(0, -3, 1)).infer_shape([(2, 3, 4), None, None])
+    with pytest.raises(MXNetError, match="exceeds the range"):
+        Node("_npx_quantized_transpose", axes=(0, 1, 3)).infer_shape([(2, 3, 4), None, None])
+    with pytest.raises(MXNetError, match="number of axes"):
+        Node("_npx_quantized_transpose", axes=(0, 1)).infer_shape([(2, 3, 4), None, None])

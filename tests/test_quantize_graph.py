@@ -459,3 +459,32 @@ def test_embedding_reshape_transpose_and_mul_stay_int8():
                                                      quantize_mode="full")[0])]
     assert "emb" in names and "quantized_emb" not in names
 
+
+
+def test_numpy_namespace_reshape_and_transpose_take_their_quantized_twins():
+    """quantized_reshape.cc:125-126 (_npx_reshape -> _npx_quantized_reshape) and
+    quantized_transpose.cc:118-127 (_npi_transpose -> _npx_quantized_transpose); both keep
+    the float node's attribute dictionary."""
+    d = S.Variable("data")
+    fc1 = S.FullyConnected(d, num_hidden=16, flatten=False, name="fc1")
+    rs = S.create("_npx_reshape", fc1, name="rs", newshape=(-2, -2, -6, 4, -1))
+    tr = S.create("_npi_transpose", rs, name="tr", axes=(0, -2, 1, -1))
+    fc2 = S.FullyConnected(tr, num_hidden=8, flatten=False, name="fc2")
+    offline = [n for n in fc2.list_arguments() if n != "data"]
+    qsym, calib = Q._quantize_symbol(fc2, "gpu", offline_params=offline, quantize_mode="full")
+    assert ops_of(qsym) == [
+        ("_contrib_quantize_v2", "fc1_data_quantize"),
+        ("_contrib_quantized_fully_connected", "quantized_fc1"),
+        ("_contrib_requantize", "requantize_fc1"),
+        ("_npx_quantized_reshape", "quantized_rs"),
+        ("_npx_quantized_transpose", "quantized_tr"),
+        ("_contrib_quantized_fully_connected", "quantized_fc2"),
+        ("_contrib_requantize", "requantize_fc2"),
+        ("_contrib_dequantize", "fc2_dequantize")]
+    assert node(qsym, "quantized_rs")[1:] == (
+        {"newshape": "(-2, -2, -6, 4, -1)"},
+        [("requantize_fc1", 0), ("requantize_fc1", 1), ("requantize_fc1", 2)])
+    assert node(qsym, "quantized_tr")[1:] == (
+        {"axes": "(0, -2, 1, -1)"},
+        [("quantized_rs", 0), ("quantized_rs", 1), ("quantized_rs", 2)])
+    assert calib == ["fc1_data", "fc1_output", "fc2_output"]
