@@ -138,6 +138,20 @@ int mxq_quantized_elemwise_add(void* stream, const void* lhs, int lhs_type, cons
                                float* omin, float* omax, size_t n, int calibrated,
                                float min_calib, float max_calib);
 
+/* _contrib_quantized_npi_add (src/operator/quantization/quantized_elemwise_add.cc:141-178,
+ * dnnl/dnnl_quantized_elemwise_add.cc:134-257; cpu only in the reference): the quantized sum
+ * of two contiguous operands under numpy broadcasting (shapes aligned at the last axis, an
+ * extent of 1 stretches).  Equal shapes are forwarded to mxq_quantized_elemwise_add; for
+ * different shapes a uint8 operand next to an int8 one is taken at its own scale, as the
+ * reference's binary primitive does.  out_type as for mxq_quantized_elemwise_add; the output
+ * has fewer than 2^32 elements. */
+int mxq_quantized_broadcast_add(void* stream, const void* lhs, int lhs_type, int lhs_ndim,
+                                const int64_t* lhs_shape, const void* rhs, int rhs_type,
+                                int rhs_ndim, const int64_t* rhs_shape, const float* lhs_min,
+                                const float* lhs_max, const float* rhs_min, const float* rhs_max,
+                                void* out, int out_type, float* omin, float* omax,
+                                int calibrated, float min_calib, float max_calib);
+
 /* ---- _contrib_quantized_elemwise_mul ---------------------------------------------
  * Replaces QuantizedElemwiseMulOpForward
  * (src/operator/quantization/quantized_elemwise_mul.cc:114-206; registered for cpu only,

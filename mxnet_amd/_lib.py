@@ -42,6 +42,8 @@ SIGNATURES = {
     "mxq_quantized_flatten": (_i, [_p, _p, _p, _p, _p, _p, _p, _sz]),
     "mxq_quantized_elemwise_add": (_i, [_p, _p, _i, _p, _i, _p, _p, _p, _p, _p, _i, _p, _p, _sz,
                                         _i, _f, _f]),
+    "mxq_quantized_broadcast_add": (_i, [_p, _p, _i, _i, _p, _p, _i, _i, _p, _p, _p, _p, _p, _p,
+                                         _i, _p, _p, _i, _f, _f]),
     "mxq_quantized_elemwise_mul": (_i, [_p, _p, _p, _p, _p, _p, _p, _p, _i, _p, _p, _sz, _i, _f,
                                         _f]),
     "mxq_quantized_embedding": (_i, [_p, _p, _i, _p, _p, _p, _p, _p, _p, _sz, ctypes.c_int64,

@@ -74,6 +74,13 @@ def quantized_elemwise_add(lhs, rhs, lhs_min, lhs_max, rhs_min, rhs_max, min_cal
                   rhs_max, min_calib_range=min_calib_range, max_calib_range=max_calib_range)
 
 
+def quantized_npi_add(lhs, rhs, lhs_min, lhs_max, rhs_min, rhs_max, min_calib_range=None,
+                      max_calib_range=None):
+    """_contrib_quantized_npi_add: the quantized sum under numpy broadcasting."""
+    return invoke("_contrib_quantized_npi_add", lhs, rhs, lhs_min, lhs_max, rhs_min, rhs_max,
+                  min_calib_range=min_calib_range, max_calib_range=max_calib_range)
+
+
 def quantized_concat(*data, num_args=None, dim=1):
     """`data` is arg0..argN-1 followed by (arg0_min, arg0_max, ..., argN-1_min, argN-1_max)."""
     if num_args is None:

@@ -273,6 +273,14 @@ NNVM_REGISTER_OP(transpose)
       return QuantizedTwin(attrs, "_contrib_quantized_transpose");
     });
 
+// src/operator/numpy/np_elemwise_broadcast_op_add.cc, quantized_elemwise_add.cc:180-189
+NNVM_REGISTER_OP(_npi_add)
+    .set_num_inputs(2)
+    .set_num_outputs(1)
+    .set_attr<FQuantizedOp>("FQuantizedOp", [](const NodeAttrs& attrs) {
+      return QuantizedTwin(attrs, "_contrib_quantized_npi_add");
+    });
+
 // src/operator/numpy/np_matrix_op.cc:353-375, quantized_reshape.cc:125-126
 NNVM_REGISTER_OP(_npx_reshape)
     .add_alias("_npi_reshape")

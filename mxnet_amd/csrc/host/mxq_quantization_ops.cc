@@ -826,6 +826,64 @@ static void QuantizedElemwiseAddForwardGPU(const NodeAttrs& attrs, const OpConte
       calibrated ? params.max_calib_range.value() : 0.f));
 }
 
+// quantized_elemwise_add-inl.h:58-70 over elemwise_binary_broadcast_op.h:41-78
+static bool QuantizedBinaryBroadcastShape(const NodeAttrs&, ShapeVector* in_attrs,
+                                          ShapeVector* out_attrs) {
+  CHECK_EQ(in_attrs->size(), 6U);
+  CHECK_EQ(out_attrs->size(), 3U);
+  for (int i = 2; i < 6; ++i) SHAPE_ASSIGN_CHECK(*in_attrs, i, TShape{1});
+  SHAPE_ASSIGN_CHECK(*out_attrs, 1, TShape{1});
+  SHAPE_ASSIGN_CHECK(*out_attrs, 2, TShape{1});
+  const TShape& lhs = (*in_attrs)[0];
+  const TShape& rhs = (*in_attrs)[1];
+  if (!ndim_is_known(lhs) || !ndim_is_known(rhs)) return false;
+  if (lhs == rhs) {
+    SHAPE_ASSIGN_CHECK(*out_attrs, 0, lhs);
+    return shape_is_known(lhs);
+  }
+  TShape out(std::max(lhs.ndim(), rhs.ndim()), -1);
+  const int bl = out.ndim() - lhs.ndim();
+  const int br = out.ndim() - rhs.ndim();
+  for (int i = 0; i < out.ndim(); ++i) {
+    index_t l = 1, r = 1;
+    if (i >= bl) l = lhs[i - bl];
+    if (i >= br) r = rhs[i - br];
+    if (l < 0 || r < 0) continue;
+    if (l != r) {
+      CHECK(l == 1 || r == 1) << "operands could not be broadcast together with shapes " << lhs
+                              << " " << rhs;
+      out[i] = (l == 1 ? r : l);
+    } else {
+      out[i] = l;
+    }
+  }
+  SHAPE_ASSIGN_CHECK(*out_attrs, 0, out);
+  return shape_is_known(lhs) && shape_is_known(rhs) && shape_is_known(out);
+}
+
+// _contrib_quantized_npi_add (dnnl_quantized_elemwise_add.cc:134-257): operands of one shape
+// take the sum above, others the broadcasting form
+static void QuantizedNpiAddForwardGPU(const NodeAttrs& attrs, const OpContext& ctx,
+                                      const std::vector<TBlob>& inputs,
+                                      const std::vector<OpReqType>&,
+                                      const std::vector<TBlob>& outputs) {
+  const auto& params = nnvm::get<QuantizeElemwiseAddParam>(attrs.parsed);
+  CHECK_EQ(inputs.size(), 6U) << "should be A, B, A_min, A_max, B_min, B_max";
+  CHECK_EQ(outputs.size(), 3U) << "should be C, C_min, C_max";
+  const bool calibrated = params.max_calib_range.has_value() && params.min_calib_range.has_value();
+  std::vector<int64_t> ls, rs;
+  for (int i = 0; i < inputs[0].shape_.ndim(); ++i) ls.push_back(inputs[0].shape_[i]);
+  for (int i = 0; i < inputs[1].shape_.ndim(); ++i) rs.push_back(inputs[1].shape_[i]);
+  MXQ_CALL(mxq_quantized_broadcast_add(
+      raw_stream(ctx), inputs[0].dptr_, inputs[0].type_flag_, static_cast<int>(ls.size()),
+      ls.data(), inputs[1].dptr_, inputs[1].type_flag_, static_cast<int>(rs.size()), rs.data(),
+      inputs[2].dptr<float>(), inputs[3].dptr<float>(), inputs[4].dptr<float>(),
+      inputs[5].dptr<float>(), outputs[0].dptr_, outputs[0].type_flag_, outputs[1].dptr<float>(),
+      outputs[2].dptr<float>(), calibrated ? 1 : 0,
+      calibrated ? params.min_calib_range.value() : 0.f,
+      calibrated ? params.max_calib_range.value() : 0.f));
+}
+
 // _contrib_quantized_concat (dnnl_quantized_concat.cc:41-115)
 static void QuantizedConcatForwardGPU(const NodeAttrs& attrs, const OpContext& ctx,
                                       const std::vector<TBlob>& inputs,
@@ -1184,6 +1242,38 @@ NNVM_REGISTER_OP(_contrib_quantized_elemwise_add)
     .set_attr<FInferStorageType>("FInferStorageType", DefaultStorageType)
     .set_attr<FNeedRequantize>("FNeedRequantize", [](const NodeAttrs&) { return true; })
     .set_attr<FCompute>("FCompute<gpu>", QuantizedElemwiseAddForwardGPU)
+    .add_argument("lhs", "NDArray-or-Symbol", "first input")
+    .add_argument("rhs", "NDArray-or-Symbol", "second input")
+    .add_argument("lhs_min", "NDArray-or-Symbol", "3rd input")
+    .add_argument("lhs_max", "NDArray-or-Symbol", "4th input")
+    .add_argument("rhs_min", "NDArray-or-Symbol", "5th input")
+    .add_argument("rhs_max", "NDArray-or-Symbol", "6th input")
+    .add_arguments(QuantizeElemwiseAddParam::__FIELDS__());
+
+// quantized_elemwise_add.cc:141-178 (+ dnnl_quantized_elemwise_add.cc:276-281)
+NNVM_REGISTER_OP(_contrib_quantized_npi_add)
+    .add_alias("_npx_quantized_npi_add")
+    .describe("elemwise_add operator with numpy broadcasting for input dataA and input dataB "
+              "data type of int8, and accumulates in type int32 for the output.")
+    .set_num_inputs(6)
+    .set_num_outputs(3)
+    .set_attr_parser(ParamParser<QuantizeElemwiseAddParam>)
+    .set_attr<nnvm::FListInputNames>("FListInputNames",
+                                     [](const NodeAttrs&) {
+                                       return std::vector<std::string>{"lhs",     "rhs",
+                                                                       "lhs_min", "lhs_max",
+                                                                       "rhs_min", "rhs_max"};
+                                     })
+    .set_attr<nnvm::FListOutputNames>("FListOutputNames",
+                                      [](const NodeAttrs&) {
+                                        return std::vector<std::string>{"output", "min_output",
+                                                                        "max_output"};
+                                      })
+    .set_attr<nnvm::FInferType>("FInferType", ElemwiseAddType)
+    .set_attr<mxnet::FInferShape>("FInferShape", QuantizedBinaryBroadcastShape)
+    .set_attr<FInferStorageType>("FInferStorageType", DefaultStorageType)
+    .set_attr<FNeedRequantize>("FNeedRequantize", [](const NodeAttrs&) { return true; })
+    .set_attr<FCompute>("FCompute<gpu>", QuantizedNpiAddForwardGPU)
     .add_argument("lhs", "NDArray-or-Symbol", "first input")
     .add_argument("rhs", "NDArray-or-Symbol", "second input")
     .add_argument("lhs_min", "NDArray-or-Symbol", "3rd input")

@@ -14,6 +14,8 @@
 // output is a byte type, 4 where it is int32 (so that every lane stores 16 bytes).
 #include <hip/hip_runtime.h>
 
+#include <vector>
+
 #include <cstdint>
 
 #include "../../include/mxq.h"
@@ -255,6 +257,120 @@ __global__ __launch_bounds__(kThreads) void add_kernel(AddArgs a) {
   if (blockIdx.x == 0 && threadIdx.x == 0) {
     *a.omin = r.omin;
     *a.omax = r.omax;
+  }
+}
+
+// ---- broadcasting add ---------------------------------------------------------------
+
+constexpr int kMaxBroadcastDims = 6;
+
+struct BroadcastAddArgs {
+  AddArgs add;  // operands, ranges, calibration; n = number of output elements (< 2^32)
+  int nd;       // merged axes, innermost last
+  uint32_t dim[kMaxBroadcastDims];
+  uint32_t lstride[kMaxBroadcastDims], rstride[kMaxBroadcastDims];  // 0 on a broadcast axis
+  int lhs_unsigned, rhs_unsigned;
+};
+
+// dnnl_quantized_elemwise_add.cc:143-182 for operands of different shapes: the scales as for
+// the plain sum, but a uint8 operand next to an int8 one is taken as it is (the reorder to
+// int8 at half scale is only made on the same-shape route, :185-210)
+template <int OUT>
+__global__ __launch_bounds__(kThreads) void broadcast_add_kernel(BroadcastAddArgs p) {
+  const AddArgs& a = p.add;
+  const bool lu = p.lhs_unsigned != 0, ru = p.rhs_unsigned != 0;
+  const float a_absmax = maxabs(*a.lhs_min, *a.lhs_max);
+  const float b_absmax = maxabs(*a.rhs_min, *a.rhs_max);
+  const float a_scale = type_range(lu ? MXQ_UINT8 : MXQ_INT8) / a_absmax;
+  const float b_scale = type_range(ru ? MXQ_UINT8 : MXQ_INT8) / b_absmax;
+  const double out_range = type_range_wide(OUT);
+  float omin, omax, out_scale;
+  if (a.calibrated) {
+    omin = a.min_calib;
+    omax = a.max_calib;
+    out_scale = static_cast<float>(out_range / static_cast<double>(maxabs(omin, omax)));
+  } else {
+    omax = a_absmax + b_absmax;
+    omin = -omax;
+    out_scale = static_cast<float>(out_range / static_cast<double>(omax));
+  }
+  const float s0 = out_scale / a_scale, s1 = out_scale / b_scale;
+  if (blockIdx.x == 0 && threadIdx.x == 0) {
+    *a.omin = omin;
+    *a.omax = omax;
+  }
+  auto one = [&](uint32_t x, uint32_t y) {
+    const int xi = lu ? static_cast<int>(x) : static_cast<int>(static_cast<int8_t>(x));
+    const int yi = ru ? static_cast<int>(y) : static_cast<int>(static_cast<int8_t>(y));
+    return narrow<OUT>(static_cast<float>(xi) * s0 + static_cast<float>(yi) * s1);
+  };
+  const uint32_t n = static_cast<uint32_t>(a.n);
+  const uint32_t stride = gridDim.x * kThreads;
+  const int last = p.nd - 1;
+  if (a.vec_ok) {
+    // 16 outputs of one innermost run per lane; an operand that is broadcast along the
+    // innermost axis contributes one byte, the other 16
+    const uint32_t inner16 = p.dim[last] >> 4;
+    for (uint32_t q = blockIdx.x * kThreads + threadIdx.x; q < (n >> 4); q += stride) {
+      uint32_t rest = q / inner16;
+      const uint32_t c = (q - rest * inner16) << 4;
+      uint32_t lo = c * p.lstride[last], ro = c * p.rstride[last];
+      for (int d = last - 1; d >= 0; --d) {
+        const uint32_t up = rest / p.dim[d], k = rest - up * p.dim[d];
+        lo += k * p.lstride[d];
+        ro += k * p.rstride[d];
+        rest = up;
+      }
+      u4 x, y;
+      if (p.lstride[last]) {
+        x = *reinterpret_cast<const u4*>(a.lhs + lo);
+      } else {
+        const uint32_t b = a.lhs[lo] * 0x01010101u;
+        x = u4{b, b, b, b};
+      }
+      if (p.rstride[last]) {
+        y = *reinterpret_cast<const u4*>(a.rhs + ro);
+      } else {
+        const uint32_t b = a.rhs[ro] * 0x01010101u;
+        y = u4{b, b, b, b};
+      }
+      if (OUT == MXQ_INT32) {
+        i4* o = reinterpret_cast<i4*>(a.out) + size_t(q) * 4;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+          i4 v;
+#pragma unroll
+          for (int k = 0; k < 4; ++k) v[k] = one((x[w] >> (8 * k)) & 0xffu, (y[w] >> (8 * k)) & 0xffu);
+          o[w] = v;
+        }
+      } else {
+        u4 v;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+          uint32_t r[4];
+#pragma unroll
+          for (int k = 0; k < 4; ++k)
+            r[k] = static_cast<uint32_t>(one((x[w] >> (8 * k)) & 0xffu, (y[w] >> (8 * k)) & 0xffu));
+          v[w] = pack_low_bytes(r[0], r[1], r[2], r[3]);
+        }
+        reinterpret_cast<u4*>(a.out)[q] = v;
+      }
+    }
+    return;
+  }
+  for (uint32_t i = blockIdx.x * kThreads + threadIdx.x; i < n; i += stride) {
+    uint32_t rest = i, lo = 0, ro = 0;
+    for (int d = last; d >= 0; --d) {
+      const uint32_t up = rest / p.dim[d], k = rest - up * p.dim[d];
+      lo += k * p.lstride[d];
+      ro += k * p.rstride[d];
+      rest = up;
+    }
+    const int v = one(a.lhs[lo], a.rhs[ro]);
+    if (OUT == MXQ_INT32)
+      static_cast<int32_t*>(a.out)[i] = v;
+    else
+      static_cast<uint8_t*>(a.out)[i] = static_cast<uint8_t>(v);
   }
 }
 
@@ -794,6 +910,114 @@ int mxq_quantized_elemwise_add(void* stream, const void* lhs, int lhs_type, cons
     else MXQ_ADD(MXQ_INT8, false, false);
   }
 #undef MXQ_ADD
+  MXQ_LAUNCH_CHECK();
+  MXQ_API_END();
+}
+
+int mxq_quantized_broadcast_add(void* stream, const void* lhs, int lhs_type, int lhs_ndim,
+                                const int64_t* lhs_shape, const void* rhs, int rhs_type,
+                                int rhs_ndim, const int64_t* rhs_shape, const float* lhs_min,
+                                const float* lhs_max, const float* rhs_min, const float* rhs_max,
+                                void* out, int out_type, float* omin, float* omax,
+                                int calibrated, float min_calib, float max_calib) {
+  MXQ_API_BEGIN();
+  MXQ_CHECK(lhs_ndim >= 0 && rhs_ndim >= 0 && (lhs_ndim == 0 || lhs_shape != nullptr) &&
+                (rhs_ndim == 0 || rhs_shape != nullptr),
+            "null shape pointer");
+  // numpy broadcasting: shapes aligned at the last axis, an extent of 1 stretches
+  const int nd = lhs_ndim > rhs_ndim ? lhs_ndim : rhs_ndim;
+  std::vector<int64_t> ls(nd, 1), rs(nd, 1), os(nd, 1);
+  for (int i = 0; i < lhs_ndim; ++i) ls[nd - lhs_ndim + i] = lhs_shape[i];
+  for (int i = 0; i < rhs_ndim; ++i) rs[nd - rhs_ndim + i] = rhs_shape[i];
+  bool same = lhs_ndim == rhs_ndim;
+  size_t n = 1;
+  for (int i = 0; i < nd; ++i) {
+    MXQ_CHECK(ls[i] >= 0 && rs[i] >= 0, "negative extent");
+    MXQ_CHECK(ls[i] == rs[i] || ls[i] == 1 || rs[i] == 1,
+              "operands could not be broadcast together: axis " << i << " has " << ls[i]
+                                                                << " and " << rs[i]);
+    os[i] = ls[i] == 1 ? rs[i] : ls[i];
+    same = same && ls[i] == rs[i];
+    n *= static_cast<size_t>(os[i]);
+  }
+  // equal shapes take the plain sum, as the reference does
+  if (same)
+    return mxq_quantized_elemwise_add(stream, lhs, lhs_type, rhs, rhs_type, lhs_min, lhs_max,
+                                      rhs_min, rhs_max, out, out_type, omin, omax, n, calibrated,
+                                      min_calib, max_calib);
+  MXQ_CHECK(byte_type(lhs_type) && byte_type(rhs_type),
+            "quantized_npi_add takes int8 or uint8 inputs, got " << lhs_type << " and "
+                                                                 << rhs_type);
+  const int want = !calibrated ? MXQ_INT32 : (lhs_type == rhs_type ? lhs_type : MXQ_INT8);
+  MXQ_CHECK(out_type == want, "output type must be " << want << " for these inputs"
+                                                     << (calibrated ? " (calibrated)" : "")
+                                                     << ", got " << out_type);
+  MXQ_CHECK(lhs_min != nullptr && lhs_max != nullptr && rhs_min != nullptr && rhs_max != nullptr &&
+                omin != nullptr && omax != nullptr,
+            "null range pointer");
+  MXQ_CHECK(n < (size_t(1) << 32), "broadcast output of " << n << " elements: at most 2^32 - 1");
+  MXQ_CHECK(n == 0 || (lhs != nullptr && rhs != nullptr && out != nullptr), "null data pointer");
+  BroadcastAddArgs p;
+  AddArgs& a = p.add;
+  a.lhs = static_cast<const uint8_t*>(lhs);
+  a.rhs = static_cast<const uint8_t*>(rhs);
+  a.out = out;
+  a.n = n;
+  a.lhs_min = lhs_min; a.lhs_max = lhs_max; a.rhs_min = rhs_min; a.rhs_max = rhs_max;
+  a.omin = omin; a.omax = omax;
+  a.min_calib = min_calib; a.max_calib = max_calib;
+  a.calibrated = calibrated != 0;
+  p.lhs_unsigned = lhs_type == MXQ_UINT8;
+  p.rhs_unsigned = rhs_type == MXQ_UINT8;
+  // element strides of the contiguous operands (0 where the operand is stretched), then
+  // neighbouring axes with the same stretch pattern merged and unit axes dropped
+  std::vector<int64_t> lst(nd, 0), rst(nd, 0);
+  int64_t lacc = 1, racc = 1;
+  for (int i = nd - 1; i >= 0; --i) {
+    lst[i] = ls[i] == 1 ? 0 : lacc;
+    rst[i] = rs[i] == 1 ? 0 : racc;
+    lacc *= ls[i];
+    racc *= rs[i];
+  }
+  std::vector<int64_t> md, ml, mr;
+  for (int i = 0; i < nd; ++i) {
+    if (os[i] == 1) continue;
+    if (!md.empty() && ml.back() == lst[i] * os[i] && mr.back() == rst[i] * os[i]) {
+      md.back() *= os[i];
+      ml.back() = lst[i];
+      mr.back() = rst[i];
+    } else {
+      md.push_back(os[i]);
+      ml.push_back(lst[i]);
+      mr.push_back(rst[i]);
+    }
+  }
+  if (md.empty()) { md.push_back(1); ml.push_back(0); mr.push_back(0); }
+  MXQ_CHECK(static_cast<int>(md.size()) <= kMaxBroadcastDims,
+            "more than " << kMaxBroadcastDims << " axes after merging");
+  p.nd = static_cast<int>(md.size());
+  for (int i = 0; i < kMaxBroadcastDims; ++i) {
+    p.dim[i] = i < p.nd ? static_cast<uint32_t>(md[i]) : 1;
+    p.lstride[i] = i < p.nd ? static_cast<uint32_t>(ml[i]) : 0;
+    p.rstride[i] = i < p.nd ? static_cast<uint32_t>(mr[i]) : 0;
+  }
+  // 16 outputs per lane when innermost runs are whole 16-byte pieces: every run of an
+  // operand that is not stretched there then starts on a multiple of 16 elements
+  a.vec_ok = (md.back() % 16 == 0 && aligned16(out) &&
+              (ml.back() == 0 || aligned16(lhs)) && (mr.back() == 0 || aligned16(rhs)))
+                 ? 1 : 0;
+  if (n == 0) {
+    // ranges only
+    a.vec_ok = 0;
+  }
+  const int grid = grid_for(a.vec_ok ? (n + 15) / 16 : (n ? n : 1));
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (out_type == MXQ_INT32)
+    hipLaunchKernelGGL((broadcast_add_kernel<MXQ_INT32>), dim3(grid), dim3(kThreads), 0, s, p);
+  else if (out_type == MXQ_UINT8)
+    hipLaunchKernelGGL((broadcast_add_kernel<MXQ_UINT8>), dim3(grid), dim3(kThreads), 0, s, p);
+  else
+    hipLaunchKernelGGL((broadcast_add_kernel<MXQ_INT8>), dim3(grid), dim3(kThreads), 0, s, p);
   MXQ_LAUNCH_CHECK();
   MXQ_API_END();
 }

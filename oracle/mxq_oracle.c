@@ -392,10 +392,11 @@ static inline int32_t q_round_sat(float f, float lo, float hi) {
  * scales[i] = output_scale / scale_i (:180-182).  A uint8 operand next to an int8 one
  * is first reordered to int8 with scale 0.5 and its scale doubled (:189-210).
  * The sum itself is dnnl::sum: dst = saturate(round(s0 * a + s1 * b)). */
-void qref_elemwise_add(const void* lhs_, int lhs_unsigned, const void* rhs_, int rhs_unsigned,
-                       size_t n, float lhs_min, float lhs_max, float rhs_min, float rhs_max,
-                       int out_kind, int calibrated, float min_calib, float max_calib,
-                       void* out_, float* omin, float* omax) {
+static void elemwise_add_impl(const void* lhs_, int lhs_unsigned, const void* rhs_,
+                              int rhs_unsigned, size_t n, float lhs_min, float lhs_max,
+                              float rhs_min, float rhs_max, int out_kind, int calibrated,
+                              float min_calib, float max_calib, int halve_mixed, void* out_,
+                              float* omin, float* omax) {
   const float a_absmax = q_maxabs(lhs_min, lhs_max), b_absmax = q_maxabs(rhs_min, rhs_max);
   const float a_scale = q_type_range(lhs_unsigned) / a_absmax;
   const float b_scale = q_type_range(rhs_unsigned) / b_absmax;
@@ -411,7 +412,8 @@ void qref_elemwise_add(const void* lhs_, int lhs_unsigned, const void* rhs_, int
     output_scale = (float)(out_range / (double)output_max);
   }
   float s0 = output_scale / a_scale, s1 = output_scale / b_scale;
-  const int halve_a = lhs_unsigned && !rhs_unsigned, halve_b = rhs_unsigned && !lhs_unsigned;
+  const int halve_a = halve_mixed && lhs_unsigned && !rhs_unsigned;
+  const int halve_b = halve_mixed && rhs_unsigned && !lhs_unsigned;
   if (halve_a) s0 = (float)((double)s0 * (1.0 / 0.5));
   if (halve_b) s1 = (float)((double)s1 * (1.0 / 0.5));
   const float lo = out_kind == 0 ? -2147483648.0f : (out_kind == 1 ? -128.0f : 0.0f);
@@ -435,6 +437,26 @@ void qref_elemwise_add(const void* lhs_, int lhs_unsigned, const void* rhs_, int
   }
   *omin = output_min;
   *omax = output_max;
+}
+
+void qref_elemwise_add(const void* lhs_, int lhs_unsigned, const void* rhs_, int rhs_unsigned,
+                       size_t n, float lhs_min, float lhs_max, float rhs_min, float rhs_max,
+                       int out_kind, int calibrated, float min_calib, float max_calib,
+                       void* out_, float* omin, float* omax) {
+  elemwise_add_impl(lhs_, lhs_unsigned, rhs_, rhs_unsigned, n, lhs_min, lhs_max, rhs_min, rhs_max,
+                    out_kind, calibrated, min_calib, max_calib, 1, out_, omin, omax);
+}
+
+/* The same sum for operands the caller has already stretched to one shape, as
+ * _contrib_quantized_npi_add computes it when the shapes differ: dnnl::binary with the two
+ * scales, and no reorder of a uint8 operand to int8 (that is only made on the same-shape
+ * route, dnnl_quantized_elemwise_add.cc:183-210).  PARITY UNPINNED like qref_elemwise_add. */
+void qref_broadcast_add(const void* lhs_, int lhs_unsigned, const void* rhs_, int rhs_unsigned,
+                        size_t n, float lhs_min, float lhs_max, float rhs_min, float rhs_max,
+                        int out_kind, int calibrated, float min_calib, float max_calib,
+                        void* out_, float* omin, float* omax) {
+  elemwise_add_impl(lhs_, lhs_unsigned, rhs_, rhs_unsigned, n, lhs_min, lhs_max, rhs_min, rhs_max,
+                    out_kind, calibrated, min_calib, max_calib, 0, out_, omin, omax);
 }
 
 /* One input of dnnl_quantized_concat.cc:68-98 brought to the output's scale:

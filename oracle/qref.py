@@ -51,6 +51,7 @@ _lib.qref_relu_i8.argtypes = [_p, _sz, _p]
 _lib.qref_pool_nchw.argtypes = [_p, _i] + [_i] * 12 + [_i, _i, _p]
 _lib.qref_elemwise_add.argtypes = [_p, _i, _p, _i, _sz, _f, _f, _f, _f, _i, _i, _f, _f, _p, _pf,
                                    _pf]
+_lib.qref_broadcast_add.argtypes = _lib.qref_elemwise_add.argtypes
 _lib.qref_concat_rescale.argtypes = [_p, _i, _sz, _f, _f, _f, _f, _i, _p]
 _lib.qref_elemwise_mul.argtypes = [_p, _p, _sz, _f, _f, _f, _f, _i, _f, _f, _p, _pf, _pf]
 _lib.qref_quantize_asym.argtypes = [_p, _sz, _f, _f, _p, _pf, _pf]
@@ -300,6 +301,36 @@ def quantized_elemwise_add(lhs, rhs, lhs_min, lhs_max, rhs_min, rhs_max, min_cal
                            min_calib_range if calibrated else 0.0,
                            max_calib_range if calibrated else 0.0, _ptr(out),
                            ctypes.byref(omin), ctypes.byref(omax))
+    return out, np.float32(omin.value), np.float32(omax.value)
+
+
+def quantized_npi_add(lhs, rhs, lhs_min, lhs_max, rhs_min, rhs_max, min_calib_range=None,
+                      max_calib_range=None):
+    """_contrib_quantized_npi_add -> (out, min, max): operands of one shape take the plain sum;
+    others are stretched by numpy's rules and summed at their own scales
+    (dnnl_quantized_elemwise_add.cc:183-257)."""
+    if lhs.shape == rhs.shape:
+        return quantized_elemwise_add(lhs, rhs, lhs_min, lhs_max, rhs_min, rhs_max,
+                                      min_calib_range, max_calib_range)
+    for x in (lhs, rhs):
+        if x.dtype not in (np.int8, np.uint8):
+            raise TypeError("quantized_npi_add takes int8 or uint8")
+    a, b = np.broadcast_arrays(lhs, rhs)
+    a, b = np.ascontiguousarray(a), np.ascontiguousarray(b)
+    calibrated = min_calib_range is not None and max_calib_range is not None
+    if not calibrated:
+        out_dtype, kind = np.int32, 0
+    elif a.dtype == b.dtype:
+        out_dtype, kind = a.dtype, (1 if a.dtype == np.int8 else 2)
+    else:
+        out_dtype, kind = np.int8, 1
+    out = np.empty(a.shape, dtype=out_dtype)
+    omin, omax = ctypes.c_float(), ctypes.c_float()
+    _lib.qref_broadcast_add(_ptr(a), int(a.dtype == np.uint8), _ptr(b), int(b.dtype == np.uint8),
+                            a.size, lhs_min, lhs_max, rhs_min, rhs_max, kind, int(calibrated),
+                            min_calib_range if calibrated else 0.0,
+                            max_calib_range if calibrated else 0.0, _ptr(out),
+                            ctypes.byref(omin), ctypes.byref(omax))
     return out, np.float32(omin.value), np.float32(omax.value)
 
 

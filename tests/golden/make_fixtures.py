@@ -137,6 +137,10 @@ def cases():
     out.append(("_npx_quantized_transpose", dict(axes=(-1, 0, -2, 1)), [t, s(-1.0), s(1.0)]))
     out.append(("_npx_quantized_reshape", dict(newshape=(-2, -5, -6, 4, -1)),
                 [t, s(-1.0), s(1.0)]))
+    out.append(("_contrib_quantized_npi_add", dict(),
+                [bd, _u8(rng, (C, 1, 16)), s(-1.0), s(2.0), s(0.0), s(2.5)]))
+    out.append(("_contrib_quantized_npi_add", dict(min_calib_range=-3.5, max_calib_range=3.0),
+                [bd, _i8(rng, (1, C, 5, 1), -128), s(-1.0), s(2.0), s(-0.5), s(2.5)]))
     return out
 
 
@@ -175,6 +179,8 @@ def run_oracle(op, attrs, ins):
         res = oracle.quantized_flatten(ins[0], f(ins[1]), f(ins[2]))
     elif op == "_contrib_quantized_elemwise_add":
         res = oracle.quantized_elemwise_add(ins[0], ins[1], *[f(v) for v in ins[2:]], *cal)
+    elif op == "_contrib_quantized_npi_add":
+        res = oracle.quantized_npi_add(ins[0], ins[1], *[f(v) for v in ins[2:]], *cal)
     elif op == "_contrib_quantized_concat":
         n = attrs["num_args"]
         res = oracle.quantized_concat(ins[:n], [f(v) for v in ins[n::2]],

@@ -214,3 +214,43 @@ def test_concat_c_abi_rejects_bad_arguments():
     rc = lib.mxq_quantized_concat(st, 0, ptrs, types, mins, maxs, ext, 2, 1, P(o), 5, P(omn),
                                   P(omx))
     assert rc == -1 and b"at least one" in lib.mxq_last_error()
+
+
+# ---- quantized_npi_add (broadcasting) -------------------------------------------------------
+
+BROADCAST_SHAPES = [((4, 6), (1, 1)), ((1, 1, 1), (13, 74, 52)), ((3, 4, 56, 56), (1, 4, 1, 1)),
+                    ((32, 56, 64), (64,)), ((8, 1, 48), (1, 5, 1)), ((2, 3, 16, 32), (3, 1, 32)),
+                    ((7, 33), (7, 1)), ((5, 1, 4, 1, 16), (1, 3, 1, 2, 16)), ((6,), ()),
+                    ((0, 4), (1, 4)), ((64, 256), (64, 256))]
+
+
+@pytest.mark.parametrize("sa,sb", BROADCAST_SHAPES)
+@pytest.mark.parametrize("ta,tb", [(np.int8, np.int8), (np.uint8, np.uint8),
+                                   (np.int8, np.uint8), (np.uint8, np.int8)])
+@pytest.mark.parametrize("calib", [None, (-3.0, 2.5)])
+def test_quantized_npi_add_matches_oracle(sa, sb, ta, tb, calib):
+    import mxnet_amd
+    rng = np.random.default_rng(len(sa) * 7 + len(sb))
+    a = rng.integers(*((0, 256) if ta == np.uint8 else (-128, 128)), sa).astype(ta)
+    b = rng.integers(*((0, 256) if tb == np.uint8 else (-128, 128)), sb).astype(tb)
+    amin, amax, bmin, bmax = -1.3, 0.9, -0.2, 2.2
+    kw = {} if calib is None else {"min_calib_range": calib[0], "max_calib_range": calib[1]}
+    f32 = lambda v: torch.tensor([v], dtype=torch.float32, device="cuda")
+    dev = lambda x: torch.from_numpy(np.require(x, requirements="C")).cuda()
+    out, mn, mx = mxnet_amd.contrib.quantized_npi_add(dev(a), dev(b), f32(amin), f32(amax),
+                                                      f32(bmin), f32(bmax), **kw)
+    ref, rmn, rmx = oracle.quantized_npi_add(a, b, amin, amax, bmin, bmax, **kw)
+    assert tuple(out.shape) == ref.shape
+    got = out.cpu().numpy()
+    assert got.dtype == ref.dtype
+    np.testing.assert_array_equal(got, ref)
+    assert (mn.item(), mx.item()) == (rmn, rmx)
+
+
+def test_quantized_npi_add_refuses_shapes_that_do_not_broadcast():
+    import mxnet_amd
+    a = torch.zeros((3, 4), dtype=torch.int8, device="cuda")
+    b = torch.zeros((3, 5), dtype=torch.int8, device="cuda")
+    s = torch.ones(1, device="cuda")
+    with pytest.raises(mxnet_amd.operator.MXNetError, match="broadcast"):
+        mxnet_amd.contrib.quantized_npi_add(a, b, s, s, s, s)

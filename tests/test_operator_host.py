@@ -454,3 +454,24 @@ def test_numpy_namespace_reshape_and_transpose_inference():
         Node("_npx_quantized_transpose", axes=(0, 1, 3)).infer_shape([(2, 3, 4), None, None])
     with pytest.raises(MXNetError, match="number of axes"):
         Node("_npx_quantized_transpose", axes=(0, 1)).infer_shape([(2, 3, 4), None, None])
+
+
+def test_quantized_npi_add_registration_and_inference():
+    """quantized_elemwise_add.cc:141-189, quantized_elemwise_add-inl.h:58-70."""
+    n = "_contrib_quantized_npi_add"
+    assert op.has_attr(n, "FCompute<gpu>") and op.has_attr(n, "FNeedRequantize")
+    assert op.has_attr("_npx_quantized_npi_add", "FCompute<gpu>")
+    assert op.has_attr("_npi_add", "FQuantizedOp")
+    node = Node(n)
+    assert node.list_inputs() == ["lhs", "rhs", "lhs_min", "lhs_max", "rhs_min", "rhs_max"]
+    assert node.list_outputs() == ["output", "min_output", "max_output"]
+    for a, b, want in [((3, 4, 5), (4, 1), (3, 4, 5)), ((1, 1), (7, 2), (7, 2)),
+                       ((2, 0, 3), (1, 3), (2, 0, 3)), ((5,), (5,), (5,)), ((6, 1), (), (6, 1))]:
+        ins, outs = node.infer_shape([a, b] + [None] * 4)
+        assert outs == [want, (1,), (1,)] and ins[2:] == [(1,)] * 4
+    with pytest.raises(MXNetError, match="could not be broadcast"):
+        node.infer_shape([(2, 3), (2, 0, 3)] + [None] * 4)
+    assert node.infer_type([I8, U8] + [None] * 4)[1] == [I32, F32, F32]
+    cal = Node(n, min_calib_range=-1.0, max_calib_range=1.0)
+    assert cal.infer_type([U8, U8] + [None] * 4)[1] == [U8, F32, F32]
+    assert cal.infer_type([I8, U8] + [None] * 4)[1] == [I8, F32, F32]

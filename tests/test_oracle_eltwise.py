@@ -194,3 +194,72 @@ def test_concat_type_rule_and_mixed_types():
     assert out.dtype == np.uint8
     with pytest.raises(TypeError):
         qref.quantized_concat([u.astype(np.int32)], [0.0], [1.0], dim=0)
+
+
+# ---- quantized_npi_add (broadcasting) -------------------------------------------------------
+
+@pytest.mark.parametrize("shape,ta,tb,broadcast", [
+    ((4, 6), np.uint8, np.int8, None), ((13, 74, 52), np.uint8, np.uint8, None),
+    ((4, 6), np.uint8, np.int8, "A"), ((13, 74, 52), np.uint8, np.uint8, "B"),
+    ((3, 4, 56, 56), np.int8, np.uint8, "A"), ((32, 56, 64, 11), np.int8, np.int8, "B")])
+def test_reference_npi_add_test(shape, ta, tb, broadcast):
+    """check_quantized_npi_add (test_quantization.py:436-512): one operand may be all-ones
+    shaped; the dequantized int32 sum is within 2 of the float sum."""
+    rng = np.random.default_rng(7)
+    sa = (1,) * len(shape) if broadcast == "A" else shape
+    sb = (1,) * len(shape) if broadcast == "B" else shape
+    a, b = integers(rng, ta, sa), integers(rng, tb, sb)
+    (alo, ahi), (blo, bhi) = low_high(ta), low_high(tb)
+    out, mn, mx = qref.quantized_npi_add(a, b, alo, ahi, blo, bhi)
+    assert out.dtype == np.int32 and out.shape == shape
+    assert mx == F(ahi) + F(bhi) and mn == -mx
+    back = out.astype(np.float32) * mx / F(0x7fffffff)
+    want = a.astype(np.float32) + b.astype(np.float32)
+    assert np.abs(back - want).max() <= 2
+
+
+@pytest.mark.parametrize("ta,tb", [(np.int8, np.int8), (np.uint8, np.uint8),
+                                   (np.int8, np.uint8), (np.uint8, np.int8)])
+@pytest.mark.parametrize("calib", [None, (-3.0, 2.5)])
+def test_npi_add_rule_exactly(ta, tb, calib):
+    """Different shapes: saturate(nearest-even(float(a) * s0 + float(b) * s1)) on the stretched
+    operands, a uint8 operand next to an int8 one at its own scale (no halving); rationals."""
+    rng = np.random.default_rng(11)
+    a = rng.integers(*((0, 256) if ta == np.uint8 else (-128, 128)), (6, 1, 40)).astype(ta)
+    b = rng.integers(*((0, 256) if tb == np.uint8 else (-128, 128)), (5, 1)).astype(tb)
+    amin, amax, bmin, bmax = -1.3, 0.9, -0.2, 2.2
+    kw = {} if calib is None else {"min_calib_range": calib[0], "max_calib_range": calib[1]}
+    out, mn, mx = qref.quantized_npi_add(a, b, amin, amax, bmin, bmax, **kw)
+    assert out.shape == (6, 5, 40)
+    ra, rb = (F(255.5) if ta == np.uint8 else F(127.5)), (F(255.5) if tb == np.uint8 else F(127.5))
+    a_abs, b_abs = max(abs(F(amin)), abs(F(amax))), max(abs(F(bmin)), abs(F(bmax)))
+    if calib is None:
+        out_range, omax = 2147483647.0, F(a_abs + b_abs)
+        omin, lo, hi = -omax, -2 ** 31, 2147483520
+        assert out.dtype == np.int32
+    else:
+        unsigned_out = ta == tb and ta == np.uint8
+        out_range = 255.5 if unsigned_out else 127.5
+        omin, omax = F(calib[0]), F(calib[1])
+        lo, hi = (0, 255) if unsigned_out else (-128, 127)
+        assert out.dtype == (np.uint8 if unsigned_out else np.int8)
+    assert (mn, mx) == (omin, omax)
+    out_scale = F(out_range / float(max(abs(omin), abs(omax))))
+    s0, s1 = F(out_scale / F(ra / a_abs)), F(out_scale / F(rb / b_abs))
+    for i in range(6):
+        for j in range(5):
+            for k in range(0, 40, 3):
+                t = F(F(int(a[i, 0, k])) * s0) + F(F(int(b[j, 0])) * s1)
+                q = min(max(Fraction(float(F(t))), Fraction(lo)), Fraction(hi))
+                assert int(out[i, j, k]) == round_half_even(q), (i, j, k)
+
+
+def test_npi_add_same_shape_is_elemwise_add_and_bad_shapes_fail():
+    rng = np.random.default_rng(2)
+    a, b = integers(rng, np.uint8, (3, 17)), integers(rng, np.int8, (3, 17))
+    x = qref.quantized_npi_add(a, b, 0.0, 2.0, -1.0, 1.0)
+    y = qref.quantized_elemwise_add(a, b, 0.0, 2.0, -1.0, 1.0)
+    np.testing.assert_array_equal(x[0], y[0])
+    assert x[1:] == y[1:]
+    with pytest.raises(ValueError):
+        qref.quantized_npi_add(a, b[:, :5], 0.0, 2.0, -1.0, 1.0)
