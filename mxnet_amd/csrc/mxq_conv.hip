@@ -411,7 +411,7 @@ void conv_nhwc(void* stream, const int8_t* data, const int8_t* weight, const int
   MXQ_CHECK(min_data && max_data && min_weight && max_weight, "null input range pointer");
   MXQ_CHECK(omin && omax, "null output range pointer");
   MXQ_CHECK(bias == nullptr || (min_bias && max_bias), "bias given without its range");
-  MXQ_CHECK(out32 != nullptr || out8 != nullptr, "no output buffer");
+  MXQ_CHECK(N == 0 || out32 != nullptr || out8 != nullptr, "no output buffer");
   MXQ_CHECK(out8 == nullptr || (rmin && rmax), "fused requantize needs rmin/rmax");
   const int eh = dilate_h * (KH - 1) + 1, ew = dilate_w * (KW - 1) + 1;
   MXQ_CHECK(H + 2 * pad_h >= eh && W + 2 * pad_w >= ew, "kernel larger than padded input");
@@ -427,8 +427,8 @@ void conv_nhwc(void* stream, const int8_t* data, const int8_t* weight, const int
   MXQ_CHECK(M < (1LL << 31) && K < (1LL << 31), "problem too large for 32-bit tile indices");
   a.M = static_cast<int>(M);
   a.K = static_cast<int>(K);
-  if (a.M == 0) return;
-  MXQ_CHECK(data != nullptr && weight != nullptr, "null operand pointer");
+  MXQ_CHECK(a.M == 0 || O == 0 || (data != nullptr && weight != nullptr),
+            "null operand pointer");
   Epilogue& e = a.epi;
   e.bias = bias;
   e.min_data = min_data; e.max_data = max_data;
@@ -442,6 +442,11 @@ void conv_nhwc(void* stream, const int8_t* data, const int8_t* weight, const int
   e.plane = planar ? a.OH * a.OW : 0;
 
   hipStream_t s = static_cast<hipStream_t>(stream);
+  if (a.M == 0 || O == 0) {
+    // no output elements: launch_fc writes the range scalars alone
+    launch_fc(s, data, weight, a.M, O, C, O, e);
+    return;
+  }
   const bool aligned = (C % 16 == 0) && aligned16(data) && aligned16(weight);
   const long long data_bytes = static_cast<long long>(N) * H * W * C;
   const bool dma_ok = aligned && data_bytes < (1LL << 31) &&

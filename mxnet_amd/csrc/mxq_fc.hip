@@ -275,8 +275,16 @@ int num_cus() {
 //   41..44  as 21..24 with a 2-stage ring (short K)
 //   51..56  128-byte stages: 64x64 (2, 3 stages), 128x128 (2, 3), 256x256 (2), 256x128 (2)
 //   57..59  128x64 and 64x128 with 128-byte stages, 64x64 with 256-byte stages
+// an output without elements still owes its range scalars
+__global__ void gemm_ranges_kernel(Epilogue e) { epilogue_ranges(e); }
+
 void launch_fc(hipStream_t s, const int8_t* data, const int8_t* weight, int M, int N, int K,
                int ldo, const Epilogue& epi) {
+  if (M == 0 || N == 0) {
+    hipLaunchKernelGGL(gemm_ranges_kernel, dim3(1), dim3(1), 0, s, epi);
+    MXQ_LAUNCH_CHECK();
+    return;
+  }
   FcArgs a;
   a.data = data;
   a.weight = weight;
@@ -399,10 +407,10 @@ extern "C" int mxq_quantized_fc(void* stream, const int8_t* data, const int8_t* 
   MXQ_CHECK(min_data && max_data && min_weight && max_weight, "null input range pointer");
   MXQ_CHECK(omin && omax, "null output range pointer");
   MXQ_CHECK(bias == nullptr || (min_bias && max_bias), "bias given without its range");
-  MXQ_CHECK(out32 != nullptr || out8 != nullptr, "no output buffer");
+  MXQ_CHECK(M == 0 || N == 0 || out32 != nullptr || out8 != nullptr, "no output buffer");
   MXQ_CHECK(out8 == nullptr || (rmin && rmax), "fused requantize needs rmin/rmax");
-  if (M == 0 || N == 0) return 0;
-  MXQ_CHECK(data != nullptr && weight != nullptr, "null operand pointer");
+  MXQ_CHECK(M == 0 || N == 0 || K == 0 || (data != nullptr && weight != nullptr),
+            "null operand pointer");
   Epilogue e;
   e.bias = bias;
   e.min_data = min_data;

@@ -182,9 +182,9 @@ def quantized_fully_connected(data, weight, bias, min_data, max_data, min_weight
     data = _c(data, np.int8)
     weight = _c(weight, np.int8)
     if flatten:
-        d2 = data.reshape(data.shape[0], -1)
+        d2 = data.reshape(data.shape[0], int(np.prod(data.shape[1:], dtype=np.int64)))
     else:
-        d2 = data.reshape(-1, data.shape[-1])
+        d2 = data.reshape(int(np.prod(data.shape[:-1], dtype=np.int64)), data.shape[-1])
     mn, mx = range_for_multiplication(min_data, max_data, min_weight, max_weight)
     b32 = None
     if bias is not None:

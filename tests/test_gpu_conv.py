@@ -229,3 +229,16 @@ def test_conv_int32_written_as_nchw(capi, case, use_bias):
                                          (dilate, dilate))
     np.testing.assert_array_equal(out.cpu().numpy(), ro)
     assert (omin.item(), omax.item()) == (rmn, rmx)
+
+
+def test_conv_without_images_still_writes_its_range(capi):
+    x = torch.zeros((0, 8, 8, 16), dtype=torch.int8, device="cuda")
+    w = torch.ones((32, 3, 3, 16), dtype=torch.int8, device="cuda")
+    f = lambda v: torch.tensor([v], dtype=torch.float32, device="cuda")
+    res = capi.quantized_conv_nhwc(x, w, None, f(-1.0), f(1.0), f(-0.5), f(0.5), None, None,
+                                   stride=(1, 1), pad=(1, 1))
+    _, rmn, rmx = oracle.quantized_conv(np.zeros((0, 16, 8, 8), np.int8),
+                                        np.ones((32, 16, 3, 3), np.int8), None, -1.0, 1.0, -0.5,
+                                        0.5, pad=(1, 1))
+    assert tuple(res["out32"].shape) == (0, 8, 8, 32)
+    assert (res["omin"].item(), res["omax"].item()) == (rmn, rmx)

@@ -201,3 +201,19 @@ def test_fc_short_k_streaming_kernel_refuses_other_shapes(capi):
             run_fc(capi, d[:, :64].copy(), w[:, :64].copy(), None, 1.0, 1.0, 1.0)
     finally:
         mxnet_amd._lib.set_tuning("fc_config", 0)
+
+
+def test_fc_degenerate_extents(capi):
+    """No rows: nothing to compute, but the output range is still written.  K = 0: the
+    output is the rescaled bias alone."""
+    w = int8_uniform((24, 48), seed=1)
+    b = int8_uniform((24,), seed=2)
+    res = run_fc(capi, np.zeros((0, 48), np.int8), w, b, 1.0, 0.08, 0.5)
+    ro, rmn, rmx = oracle_fc(np.zeros((0, 48), np.int8), w, b, 1.0, 0.08, 0.5)
+    assert tuple(res["out32"].shape) == (0, 24)
+    assert (res["omin"].item(), res["omax"].item()) == (rmn, rmx)
+    d0, w0 = np.zeros((5, 0), np.int8), np.zeros((24, 0), np.int8)
+    res = run_fc(capi, d0, w0, b, 1.0, 0.08, 0.5)
+    ro, rmn, rmx = oracle_fc(d0, w0, b, 1.0, 0.08, 0.5)
+    np.testing.assert_array_equal(res["out32"].cpu().numpy(), ro)
+    assert (res["omin"].item(), res["omax"].item()) == (rmn, rmx)
