@@ -112,10 +112,12 @@ struct AddArgs {
 
 // LU / RU: the operand is uint8.  FAST: both scales are small enough that neither
 // product overflows, so no NaN can arise and the one-instruction clamp applies.
-template <int OUT, bool LU, bool RU>
+// HALVE: a uint8 operand next to an int8 one is first brought to int8 at half scale (the
+// same-shape sum); without it both operands keep their own scale (the broadcasting sum).
+template <int OUT, bool LU, bool RU, bool HALVE = true>
 struct AddRule {
   float s0, s1, omin, omax;
-  static constexpr bool kHalveL = LU && !RU, kHalveR = RU && !LU;
+  static constexpr bool kHalveL = HALVE && LU && !RU, kHalveR = HALVE && RU && !LU;
   __device__ __forceinline__ float sum(int a, int b) const {
     if (kHalveL) a = halve_u8(a);
     if (kHalveR) b = halve_u8(b);
@@ -140,9 +142,9 @@ struct AddRule {
 };
 
 // dnnl_quantized_elemwise_add.cc:143-210
-template <int OUT, bool LU, bool RU>
-__device__ __forceinline__ AddRule<OUT, LU, RU> add_rule(const AddArgs& a) {
-  AddRule<OUT, LU, RU> r;
+template <int OUT, bool LU, bool RU, bool HALVE = true>
+__device__ __forceinline__ AddRule<OUT, LU, RU, HALVE> add_rule(const AddArgs& a) {
+  AddRule<OUT, LU, RU, HALVE> r;
   const float a_absmax = maxabs(*a.lhs_min, *a.lhs_max);
   const float b_absmax = maxabs(*a.rhs_min, *a.rhs_max);
   const float a_scale = type_range(LU ? MXQ_UINT8 : MXQ_INT8) / a_absmax;
@@ -275,42 +277,148 @@ struct BroadcastAddArgs {
 // dnnl_quantized_elemwise_add.cc:143-182 for operands of different shapes: the scales as for
 // the plain sum, but a uint8 operand next to an int8 one is taken as it is (the reorder to
 // int8 at half scale is only made on the same-shape route, :185-210)
-template <int OUT>
+template <int OUT, bool LU, bool RU>
+using BroadcastRule = AddRule<OUT, LU, RU, false>;
+
+// 16 results from 16 bytes of each operand, stored as OUT
+template <int OUT, bool LU, bool RU, bool FAST>
+__device__ __forceinline__ void broadcast_store16(const BroadcastRule<OUT, LU, RU>& r, u4 x, u4 y,
+                                                  void* out, size_t piece) {
+  if (OUT == MXQ_INT32) {
+    i4* o = static_cast<i4*>(out) + piece * 4;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      i4 v;
+#pragma unroll
+      for (int k = 0; k < 4; ++k) v[k] = r.apply(byte_of<LU>(x[w], k), byte_of<RU>(y[w], k));
+      o[w] = v;  // a lane's 64 bytes: left to the cache to merge into whole lines
+    }
+  } else {
+    u4 v;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) v[w] = r.template apply4<FAST>(x[w], y[w]);
+    stream_store16(v, static_cast<u4*>(out) + piece);
+  }
+}
+
+// Innermost runs of at least 1 KiB in 16-byte pieces: one wave per 4 KiB of a run, so the
+// run's position in both operands is wave-uniform (scalar divisions, once per 4 KiB) and an
+// operand that is stretched along the run is one scalar byte.
+template <int OUT, bool LU, bool RU>
+__global__ __launch_bounds__(kThreads) void broadcast_add_rows_kernel(BroadcastAddArgs p) {
+  const AddArgs& a = p.add;
+  const BroadcastRule<OUT, LU, RU> r = add_rule<OUT, LU, RU, false>(a);
+  if (blockIdx.x == 0 && threadIdx.x == 0) {
+    *a.omin = r.omin;
+    *a.omax = r.omax;
+  }
+  const int last = p.nd - 1;
+  const uint32_t inner16 = p.dim[last] >> 4;
+  const uint32_t chunks = (inner16 + 255u) >> 8;
+  const uint32_t rows = static_cast<uint32_t>(a.n) / p.dim[last];
+  const uint32_t items = rows * chunks;
+  const uint32_t lane = threadIdx.x & 63u;
+  const uint32_t wave =
+      __builtin_amdgcn_readfirstlane(blockIdx.x * (kThreads / 64) + (threadIdx.x >> 6));
+  const uint32_t nwaves = gridDim.x * (kThreads / 64);
+  const bool fast = r.fast();
+  for (uint32_t item = wave; item < items; item += nwaves) {
+    const uint32_t row = item / chunks, k = item - row * chunks;
+    uint32_t rest = row, lo = 0, ro = 0;
+    for (int d = last - 1; d >= 0; --d) {
+      const uint32_t up = rest / p.dim[d], c = rest - up * p.dim[d];
+      lo += c * p.lstride[d];
+      ro += c * p.rstride[d];
+      rest = up;
+    }
+    if (OUT == MXQ_INT32) {
+      // a dword of each operand per lane and step: every store instruction writes 1 KiB of
+      // consecutive output
+      const uint32_t e0 = k << 12;  // first element of this piece within the run
+      const uint32_t left4 = (p.dim[last] - e0) >> 2;
+      const uint32_t lsplat = p.lstride[last] ? 0u : a.lhs[lo] * 0x01010101u;
+      const uint32_t rsplat = p.rstride[last] ? 0u : a.rhs[ro] * 0x01010101u;
+      const uint32_t* l4 = reinterpret_cast<const uint32_t*>(a.lhs + lo + e0);
+      const uint32_t* r4 = reinterpret_cast<const uint32_t*>(a.rhs + ro + e0);
+      i4* o4 = static_cast<i4*>(a.out) + ((size_t(row) * p.dim[last] + e0) >> 2);
+#pragma unroll
+      for (int jj = 0; jj < 16; jj += 4) {
+        uint32_t xs[4], ys[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const uint32_t g = (jj + j) * 64 + lane;
+          xs[j] = lsplat;
+          ys[j] = rsplat;
+          if (g < left4) {
+            if (p.lstride[last]) xs[j] = __builtin_nontemporal_load(l4 + g);
+            if (p.rstride[last]) ys[j] = __builtin_nontemporal_load(r4 + g);
+          }
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const uint32_t g = (jj + j) * 64 + lane;
+          if (g < left4) {
+            i4 v;
+#pragma unroll
+            for (int b = 0; b < 4; ++b) v[b] = r.apply(byte_of<LU>(xs[j], b), byte_of<RU>(ys[j], b));
+            __builtin_nontemporal_store(v, o4 + g);
+          }
+        }
+      }
+      continue;
+    }
+    const uint32_t left = inner16 - (k << 8);
+    const uint32_t c0 = (k << 8) + lane;
+    u4 x[4] = {}, y[4] = {};
+    if (p.lstride[last]) {
+      const u4* src = reinterpret_cast<const u4*>(a.lhs + lo) + c0;
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        if (lane + 64u * j < left) x[j] = __builtin_nontemporal_load(src + 64 * j);
+    } else {
+      const uint32_t b = a.lhs[lo] * 0x01010101u;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) x[j] = u4{b, b, b, b};
+    }
+    if (p.rstride[last]) {
+      const u4* src = reinterpret_cast<const u4*>(a.rhs + ro) + c0;
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        if (lane + 64u * j < left) y[j] = __builtin_nontemporal_load(src + 64 * j);
+    } else {
+      const uint32_t b = a.rhs[ro] * 0x01010101u;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) y[j] = u4{b, b, b, b};
+    }
+    const size_t piece0 = size_t(row) * inner16 + c0;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      if (lane + 64u * j < left) {
+        if (fast)
+          broadcast_store16<OUT, LU, RU, true>(r, x[j], y[j], a.out, piece0 + 64 * j);
+        else
+          broadcast_store16<OUT, LU, RU, false>(r, x[j], y[j], a.out, piece0 + 64 * j);
+      }
+    }
+  }
+}
+
+// Any other layout: 16 outputs of one innermost run per lane where runs are whole 16-byte
+// pieces, else one output per lane; positions by division.
+template <int OUT, bool LU, bool RU>
 __global__ __launch_bounds__(kThreads) void broadcast_add_kernel(BroadcastAddArgs p) {
   const AddArgs& a = p.add;
-  const bool lu = p.lhs_unsigned != 0, ru = p.rhs_unsigned != 0;
-  const float a_absmax = maxabs(*a.lhs_min, *a.lhs_max);
-  const float b_absmax = maxabs(*a.rhs_min, *a.rhs_max);
-  const float a_scale = type_range(lu ? MXQ_UINT8 : MXQ_INT8) / a_absmax;
-  const float b_scale = type_range(ru ? MXQ_UINT8 : MXQ_INT8) / b_absmax;
-  const double out_range = type_range_wide(OUT);
-  float omin, omax, out_scale;
-  if (a.calibrated) {
-    omin = a.min_calib;
-    omax = a.max_calib;
-    out_scale = static_cast<float>(out_range / static_cast<double>(maxabs(omin, omax)));
-  } else {
-    omax = a_absmax + b_absmax;
-    omin = -omax;
-    out_scale = static_cast<float>(out_range / static_cast<double>(omax));
-  }
-  const float s0 = out_scale / a_scale, s1 = out_scale / b_scale;
+  const BroadcastRule<OUT, LU, RU> r = add_rule<OUT, LU, RU, false>(a);
   if (blockIdx.x == 0 && threadIdx.x == 0) {
-    *a.omin = omin;
-    *a.omax = omax;
+    *a.omin = r.omin;
+    *a.omax = r.omax;
   }
-  auto one = [&](uint32_t x, uint32_t y) {
-    const int xi = lu ? static_cast<int>(x) : static_cast<int>(static_cast<int8_t>(x));
-    const int yi = ru ? static_cast<int>(y) : static_cast<int>(static_cast<int8_t>(y));
-    return narrow<OUT>(static_cast<float>(xi) * s0 + static_cast<float>(yi) * s1);
-  };
   const uint32_t n = static_cast<uint32_t>(a.n);
   const uint32_t stride = gridDim.x * kThreads;
   const int last = p.nd - 1;
   if (a.vec_ok) {
-    // 16 outputs of one innermost run per lane; an operand that is broadcast along the
-    // innermost axis contributes one byte, the other 16
     const uint32_t inner16 = p.dim[last] >> 4;
+    const bool fast = r.fast();
     for (uint32_t q = blockIdx.x * kThreads + threadIdx.x; q < (n >> 4); q += stride) {
       uint32_t rest = q / inner16;
       const uint32_t c = (q - rest * inner16) << 4;
@@ -334,27 +442,10 @@ __global__ __launch_bounds__(kThreads) void broadcast_add_kernel(BroadcastAddArg
         const uint32_t b = a.rhs[ro] * 0x01010101u;
         y = u4{b, b, b, b};
       }
-      if (OUT == MXQ_INT32) {
-        i4* o = reinterpret_cast<i4*>(a.out) + size_t(q) * 4;
-#pragma unroll
-        for (int w = 0; w < 4; ++w) {
-          i4 v;
-#pragma unroll
-          for (int k = 0; k < 4; ++k) v[k] = one((x[w] >> (8 * k)) & 0xffu, (y[w] >> (8 * k)) & 0xffu);
-          o[w] = v;
-        }
-      } else {
-        u4 v;
-#pragma unroll
-        for (int w = 0; w < 4; ++w) {
-          uint32_t r[4];
-#pragma unroll
-          for (int k = 0; k < 4; ++k)
-            r[k] = static_cast<uint32_t>(one((x[w] >> (8 * k)) & 0xffu, (y[w] >> (8 * k)) & 0xffu));
-          v[w] = pack_low_bytes(r[0], r[1], r[2], r[3]);
-        }
-        reinterpret_cast<u4*>(a.out)[q] = v;
-      }
+      if (fast)
+        broadcast_store16<OUT, LU, RU, true>(r, x, y, a.out, q);
+      else
+        broadcast_store16<OUT, LU, RU, false>(r, x, y, a.out, q);
     }
     return;
   }
@@ -366,7 +457,9 @@ __global__ __launch_bounds__(kThreads) void broadcast_add_kernel(BroadcastAddArg
       ro += k * p.rstride[d];
       rest = up;
     }
-    const int v = one(a.lhs[lo], a.rhs[ro]);
+    const int x = LU ? static_cast<int>(a.lhs[lo]) : static_cast<int>(static_cast<int8_t>(a.lhs[lo]));
+    const int y = RU ? static_cast<int>(a.rhs[ro]) : static_cast<int>(static_cast<int8_t>(a.rhs[ro]));
+    const int v = r.apply(x, y);
     if (OUT == MXQ_INT32)
       static_cast<int32_t*>(a.out)[i] = v;
     else
@@ -1010,14 +1103,32 @@ int mxq_quantized_broadcast_add(void* stream, const void* lhs, int lhs_type, int
     // ranges only
     a.vec_ok = 0;
   }
-  const int grid = grid_for(a.vec_ok ? (n + 15) / 16 : (n ? n : 1));
   hipStream_t s = static_cast<hipStream_t>(stream);
-  if (out_type == MXQ_INT32)
-    hipLaunchKernelGGL((broadcast_add_kernel<MXQ_INT32>), dim3(grid), dim3(kThreads), 0, s, p);
-  else if (out_type == MXQ_UINT8)
-    hipLaunchKernelGGL((broadcast_add_kernel<MXQ_UINT8>), dim3(grid), dim3(kThreads), 0, s, p);
-  else
-    hipLaunchKernelGGL((broadcast_add_kernel<MXQ_INT8>), dim3(grid), dim3(kThreads), 0, s, p);
+  const bool lu = p.lhs_unsigned != 0, ru = p.rhs_unsigned != 0;
+  const bool rows = a.vec_ok && md.back() >= 1024;
+  const int grid = rows ? 2 * grid_for((n / static_cast<size_t>(md.back())) *
+                                       ((static_cast<size_t>(md.back()) / 16 + 255) / 256) * 64)
+                        : grid_for(a.vec_ok ? (n + 15) / 16 : (n ? n : 1));
+#define MXQ_BCAST(O, L, R)                                                                   \
+  do {                                                                                       \
+    if (rows)                                                                                \
+      hipLaunchKernelGGL((broadcast_add_rows_kernel<O, L, R>), dim3(grid), dim3(kThreads), 0, \
+                         s, p);                                                              \
+    else                                                                                     \
+      hipLaunchKernelGGL((broadcast_add_kernel<O, L, R>), dim3(grid), dim3(kThreads), 0, s,  \
+                         p);                                                                 \
+  } while (0)
+  if (out_type == MXQ_INT32) {
+    if (lu) { if (ru) MXQ_BCAST(MXQ_INT32, true, true); else MXQ_BCAST(MXQ_INT32, true, false); }
+    else    { if (ru) MXQ_BCAST(MXQ_INT32, false, true); else MXQ_BCAST(MXQ_INT32, false, false); }
+  } else if (out_type == MXQ_UINT8) {
+    MXQ_BCAST(MXQ_UINT8, true, true);
+  } else {
+    if (lu) MXQ_BCAST(MXQ_INT8, true, false);
+    else if (ru) MXQ_BCAST(MXQ_INT8, false, true);
+    else MXQ_BCAST(MXQ_INT8, false, false);
+  }
+#undef MXQ_BCAST
   MXQ_LAUNCH_CHECK();
   MXQ_API_END();
 }

@@ -221,7 +221,10 @@ def test_concat_c_abi_rejects_bad_arguments():
 BROADCAST_SHAPES = [((4, 6), (1, 1)), ((1, 1, 1), (13, 74, 52)), ((3, 4, 56, 56), (1, 4, 1, 1)),
                     ((32, 56, 64), (64,)), ((8, 1, 48), (1, 5, 1)), ((2, 3, 16, 32), (3, 1, 32)),
                     ((7, 33), (7, 1)), ((5, 1, 4, 1, 16), (1, 3, 1, 2, 16)), ((6,), ()),
-                    ((0, 4), (1, 4)), ((64, 256), (64, 256))]
+                    ((0, 4), (1, 4)), ((64, 256), (64, 256)),
+                    # innermost runs of 1 KiB and more: the wave-per-run kernel, ragged pieces
+                    ((3, 5, 1040), (5, 1)), ((4, 2, 4112), (1, 2, 4112)), ((2, 3, 2048), (3, 1)),
+                    ((2, 1, 1024), (1, 3, 1024)), ((1, 1), (3, 5136))]
 
 
 @pytest.mark.parametrize("sa,sb", BROADCAST_SHAPES)
