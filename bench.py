@@ -52,6 +52,8 @@ MEASURED_TRAFFIC_BYTES = {
     "batch_norm": (2.0 * 32819.7 + 65536.0) * _KIB,             # bn_rows_kernel_nchw_64M.md
     "embedding": (2.0 * 31709.6 + 65535.8) * _KIB,              # embedding_kernel_bert_vocab.md
     "transpose": (2.0 * 32796.4 + 65536.1) * _KIB,              # permute_elem_kernel_attention_64M.md
+    "maxpool": (2.0 * 100388.0 + 50177.2) * _KIB,               # pool_lds_kernel_maxpool.md
+    "avgpool": (2.0 * 200728.0 + 8192.1) * _KIB,                # pool_lds_kernel_global_avgpool.md
     "resnet50_convs": 512.1e6,                                  # conv_stack_resnet50.md (19 launches)
 }
 
