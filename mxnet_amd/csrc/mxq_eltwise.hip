@@ -14,6 +14,7 @@
 // output is a byte type, 4 where it is int32 (so that every lane stores 16 bytes).
 #include <hip/hip_runtime.h>
 
+#include <type_traits>
 #include <vector>
 
 #include <cstdint>
@@ -331,74 +332,85 @@ __global__ __launch_bounds__(kThreads) void broadcast_add_rows_kernel(BroadcastA
       ro += c * p.rstride[d];
       rest = up;
     }
+    // Loads are unconditional and branch-free (indices clamped to the run, a stretched
+    // operand reads the other operand's bytes and discards them: at most one is stretched
+    // along the run): with loads inside branches the compiler drains the memory counter,
+    // stores included, before every batch.
+    const bool lrun = p.lstride[last] != 0, rrun = p.rstride[last] != 0;
+    const uint32_t lsplat = lrun ? 0u : a.lhs[lo] * 0x01010101u;
+    const uint32_t rsplat = rrun ? 0u : a.rhs[ro] * 0x01010101u;
+    const uint8_t* lbase = lrun ? a.lhs + lo : a.rhs + ro;
+    const uint8_t* rbase = rrun ? a.rhs + ro : a.lhs + lo;
     if (OUT == MXQ_INT32) {
       // a dword of each operand per lane and step: every store instruction writes 1 KiB of
       // consecutive output
       const uint32_t e0 = k << 12;  // first element of this piece within the run
       const uint32_t left4 = (p.dim[last] - e0) >> 2;
-      const uint32_t lsplat = p.lstride[last] ? 0u : a.lhs[lo] * 0x01010101u;
-      const uint32_t rsplat = p.rstride[last] ? 0u : a.rhs[ro] * 0x01010101u;
-      const uint32_t* l4 = reinterpret_cast<const uint32_t*>(a.lhs + lo + e0);
-      const uint32_t* r4 = reinterpret_cast<const uint32_t*>(a.rhs + ro + e0);
+      const uint32_t* l4 = reinterpret_cast<const uint32_t*>(lbase + e0);
+      const uint32_t* r4 = reinterpret_cast<const uint32_t*>(rbase + e0);
       i4* o4 = static_cast<i4*>(a.out) + ((size_t(row) * p.dim[last] + e0) >> 2);
-#pragma unroll
-      for (int jj = 0; jj < 16; jj += 4) {
+      for (int jj = 0; jj < 16 && static_cast<uint32_t>(jj) * 64u < left4; jj += 4) {
         uint32_t xs[4], ys[4];
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
           const uint32_t g = (jj + j) * 64 + lane;
-          xs[j] = lsplat;
-          ys[j] = rsplat;
-          if (g < left4) {
-            if (p.lstride[last]) xs[j] = __builtin_nontemporal_load(l4 + g);
-            if (p.rstride[last]) ys[j] = __builtin_nontemporal_load(r4 + g);
-          }
+          const uint32_t gc = g < left4 ? g : left4 - 1u;
+          const uint32_t xv = __builtin_nontemporal_load(l4 + gc);
+          const uint32_t yv = __builtin_nontemporal_load(r4 + gc);
+          xs[j] = lrun ? xv : lsplat;
+          ys[j] = rrun ? yv : rsplat;
         }
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
           const uint32_t g = (jj + j) * 64 + lane;
-          if (g < left4) {
-            i4 v;
+          i4 v;
 #pragma unroll
-            for (int b = 0; b < 4; ++b) v[b] = r.apply(byte_of<LU>(xs[j], b), byte_of<RU>(ys[j], b));
-            __builtin_nontemporal_store(v, o4 + g);
-          }
+          for (int b = 0; b < 4; ++b) v[b] = r.apply(byte_of<LU>(xs[j], b), byte_of<RU>(ys[j], b));
+          if (g < left4) __builtin_nontemporal_store(v, o4 + g);
         }
       }
       continue;
     }
     const uint32_t left = inner16 - (k << 8);
-    const uint32_t c0 = (k << 8) + lane;
-    u4 x[4] = {}, y[4] = {};
-    if (p.lstride[last]) {
-      const u4* src = reinterpret_cast<const u4*>(a.lhs + lo) + c0;
+    const uint32_t c0 = k << 8;
+    const u4* l16 = reinterpret_cast<const u4*>(lbase) + c0;
+    const u4* r16 = reinterpret_cast<const u4*>(rbase) + c0;
+    const size_t piece0 = size_t(row) * inner16 + c0 + lane;
+    // NB steps of 64 lanes x 16 bytes, all loads first, all results before the first store
+    // (the stores are opaque to the compiler's count of outstanding operations)
+    auto steps = [&](auto nb) {
+      constexpr int NB = decltype(nb)::value;
+      u4 x[NB], y[NB], v[NB];
 #pragma unroll
-      for (int j = 0; j < 4; ++j)
-        if (lane + 64u * j < left) x[j] = __builtin_nontemporal_load(src + 64 * j);
-    } else {
-      const uint32_t b = a.lhs[lo] * 0x01010101u;
-#pragma unroll
-      for (int j = 0; j < 4; ++j) x[j] = u4{b, b, b, b};
-    }
-    if (p.rstride[last]) {
-      const u4* src = reinterpret_cast<const u4*>(a.rhs + ro) + c0;
-#pragma unroll
-      for (int j = 0; j < 4; ++j)
-        if (lane + 64u * j < left) y[j] = __builtin_nontemporal_load(src + 64 * j);
-    } else {
-      const uint32_t b = a.rhs[ro] * 0x01010101u;
-#pragma unroll
-      for (int j = 0; j < 4; ++j) y[j] = u4{b, b, b, b};
-    }
-    const size_t piece0 = size_t(row) * inner16 + c0;
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      if (lane + 64u * j < left) {
-        if (fast)
-          broadcast_store16<OUT, LU, RU, true>(r, x[j], y[j], a.out, piece0 + 64 * j);
-        else
-          broadcast_store16<OUT, LU, RU, false>(r, x[j], y[j], a.out, piece0 + 64 * j);
+      for (int j = 0; j < NB; ++j) {
+        const uint32_t t = lane + 64u * j < left ? lane + 64u * j : left - 1u;
+        const u4 xv = __builtin_nontemporal_load(l16 + t);
+        const u4 yv = __builtin_nontemporal_load(r16 + t);
+        x[j] = lrun ? xv : u4{lsplat, lsplat, lsplat, lsplat};
+        y[j] = rrun ? yv : u4{rsplat, rsplat, rsplat, rsplat};
       }
+      if (fast) {
+#pragma unroll
+        for (int j = 0; j < NB; ++j)
+#pragma unroll
+          for (int w = 0; w < 4; ++w) v[j][w] = r.template apply4<true>(x[j][w], y[j][w]);
+      } else {
+#pragma unroll
+        for (int j = 0; j < NB; ++j)
+#pragma unroll
+          for (int w = 0; w < 4; ++w) v[j][w] = r.template apply4<false>(x[j][w], y[j][w]);
+      }
+#pragma unroll
+      for (int j = 0; j < NB; ++j)
+        if (lane + 64u * j < left) stream_store16(v[j], static_cast<u4*>(a.out) + piece0 + 64 * j);
+    };
+    if (OUT != MXQ_INT32) {
+      if (left > 128u)
+        steps(std::integral_constant<int, 4>());
+      else if (left > 64u)
+        steps(std::integral_constant<int, 2>());
+      else
+        steps(std::integral_constant<int, 1>());
     }
   }
 }
