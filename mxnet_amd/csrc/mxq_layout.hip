@@ -350,20 +350,38 @@ __global__ __launch_bounds__(kThreads) void permute_elem_kernel(ElemArgs e) {
     batch_offsets(a, z, in_off, out_off);
     const uint8_t* src = a.in + in_off;
     uint8_t* dst = a.out + out_off;
-    for (int c = threadIdx.x; c < pieces; c += kThreads) {
+    // at most 4 pieces per thread (T * T * E / 16 <= 1024): all loads first, unconditional
+    // (a piece outside the tensor reads the batch's first bytes and is dropped), then the
+    // LDS writes; the same for the way out
+    u4 v[4];
+    int slot[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int c = threadIdx.x + j * kThreads;
       const int b = c / run16, off = (c - b * run16) << 4;
-      if (b0 + b < a.B && a0 + off / E < a.A)
-        *reinterpret_cast<u4*>(tile + b * pitch + off) = *reinterpret_cast<const u4*>(
-            src + static_cast<size_t>((b0 + b) * a.b_in_stride + a0 * E + off));
+      const bool ok = c < pieces && b0 + b < a.B && a0 + off / E < a.A;
+      slot[j] = ok ? b * pitch + off : -1;
+      const size_t at = ok ? static_cast<size_t>((b0 + b) * a.b_in_stride + a0 * E + off) : 0;
+      v[j] = *reinterpret_cast<const u4*>(src + at);
     }
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      if (slot[j] >= 0) *reinterpret_cast<u4*>(tile + slot[j]) = v[j];
     __syncthreads();
-    for (int c = threadIdx.x; c < pieces; c += kThreads) {
+    size_t to[4];
+    bool put[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int c = threadIdx.x + j * kThreads;
       const int ar = c / run16, off = (c - ar * run16) << 4;
       const int b = off / E, within = off - b * E;
-      if (a0 + ar < a.A && b0 + b < a.B)
-        *reinterpret_cast<u4*>(dst + static_cast<size_t>((a0 + ar) * a.a_out_stride + b0 * E + off)) =
-            *reinterpret_cast<const u4*>(tile + b * pitch + ar * E + within);
+      put[j] = c < pieces && a0 + ar < a.A && b0 + b < a.B;
+      to[j] = static_cast<size_t>((a0 + ar) * a.a_out_stride + b0 * E + off);
+      v[j] = *reinterpret_cast<const u4*>(tile + (c < pieces ? b * pitch + ar * E + within : 0));
     }
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      if (put[j]) *reinterpret_cast<u4*>(dst + to[j]) = v[j];
     __syncthreads();
   }
   pass_range(a.imin, a.imax, a.omin, a.omax);
