@@ -34,27 +34,29 @@ INT8_PEAK_TOPS = 5000.0  # MI355X dense int8 MFMA
 
 # HBM bytes per step of the workload's kernels from `rocprofv3 --pmc FETCH_SIZE` and
 # `--pmc WRITE_SIZE` runs (KiB per dispatch; FETCH_SIZE x 2.00 per the copy-kernel
-# calibration, profiles/copy_calibration_64M.md); each entry names its summary under
-# profiles/.  None = not measured.
+# calibration, profiles/copy_calibration_64M.md), with the summary under profiles/ each
+# figure was read from: `roofline.traffic` is that profile's figure, not a counter read in
+# this run (`roofline.traffic_source` names the file); a workload without an entry reports
+# null.
 _KIB = 1024.0
 MEASURED_TRAFFIC_BYTES = {
-    "fc4096": (2.0 * 49309.8 + 16384.1) * _KIB,                 # fc_dma_kernel_4096.md
-    "quantize": (2.0 * 131102.5 + 65536.1) * _KIB,              # quantize_kernel_64M.md
-    "quantize_uncal": (2.0 * (131093.7 + 131139.1) + 65536.1) * _KIB,   # quantize_uncalibrated_64M.md
-    "requantize": (2.0 * 131104.8 + 65536.1) * _KIB,            # requantize_kernel_64M.md
-    "requantize_uncal": (2.0 * (131089.2 + 131139.2) + 65536.1) * _KIB,  # requantize_uncalibrated_64M.md
-    "dequantize": (2.0 * 32784.6 + 262224.7) * _KIB,            # dequantize_kernel_64M.md
-    "elemwise_add": (2.0 * 65570.1 + 262176.7) * _KIB,          # add_kernel_int32_64M.md
-    "elemwise_add_int8": (2.0 * 65583.7 + 65536.1) * _KIB,      # add_kernel_int8_64M.md
-    "concat": (2.0 * 32840.8 + 65536.1) * _KIB,                 # concat_kernel_64M.md
-    "elemwise_mul_int8": (2.0 * 65565.8 + 65536.1) * _KIB,      # mul_kernel_int8_64M.md
-    "quantize_asym": (2.0 * 131099.2 + 65536.1) * _KIB,         # quantize_asym_kernel_64M.md
-    "batch_norm": (2.0 * 32819.7 + 65536.0) * _KIB,             # bn_rows_kernel_nchw_64M.md
-    "embedding": (2.0 * 31709.6 + 65535.8) * _KIB,              # embedding_kernel_bert_vocab.md
-    "transpose": (2.0 * 32796.4 + 65536.1) * _KIB,              # permute_elem_kernel_attention_64M.md
-    "maxpool": (2.0 * 100388.0 + 50177.2) * _KIB,               # pool_lds_kernel_maxpool.md
-    "avgpool": (2.0 * 200728.0 + 8192.1) * _KIB,                # pool_lds_kernel_global_avgpool.md
-    "resnet50_convs": 512.1e6,                                  # conv_stack_resnet50.md (19 launches)
+    "fc4096": ((2.0 * 49309.8 + 16384.1) * _KIB, "profiles/fc_dma_kernel_4096.md"),
+    "quantize": ((2.0 * 131102.5 + 65536.1) * _KIB, "profiles/quantize_kernel_64M.md"),
+    "quantize_uncal": ((2.0 * (131093.7 + 131139.1) + 65536.1) * _KIB, "profiles/quantize_uncalibrated_64M.md"),
+    "requantize": ((2.0 * 131104.8 + 65536.1) * _KIB, "profiles/requantize_kernel_64M.md"),
+    "requantize_uncal": ((2.0 * (131089.2 + 131139.2) + 65536.1) * _KIB, "profiles/requantize_uncalibrated_64M.md"),
+    "dequantize": ((2.0 * 32784.6 + 262224.7) * _KIB, "profiles/dequantize_kernel_64M.md"),
+    "elemwise_add": ((2.0 * 65570.1 + 262176.7) * _KIB, "profiles/add_kernel_int32_64M.md"),
+    "elemwise_add_int8": ((2.0 * 65583.7 + 65536.1) * _KIB, "profiles/add_kernel_int8_64M.md"),
+    "concat": ((2.0 * 32840.8 + 65536.1) * _KIB, "profiles/concat_kernel_64M.md"),
+    "elemwise_mul_int8": ((2.0 * 65565.8 + 65536.1) * _KIB, "profiles/mul_kernel_int8_64M.md"),
+    "quantize_asym": ((2.0 * 131099.2 + 65536.1) * _KIB, "profiles/quantize_asym_kernel_64M.md"),
+    "batch_norm": ((2.0 * 32819.7 + 65536.0) * _KIB, "profiles/bn_rows_kernel_nchw_64M.md"),
+    "embedding": ((2.0 * 31709.6 + 65535.8) * _KIB, "profiles/embedding_kernel_bert_vocab.md"),
+    "transpose": ((2.0 * 32796.4 + 65536.1) * _KIB, "profiles/permute_elem_kernel_attention_64M.md"),
+    "maxpool": ((2.0 * 100388.0 + 50177.2) * _KIB, "profiles/pool_lds_kernel_maxpool.md"),
+    "avgpool": ((2.0 * 200728.0 + 8192.1) * _KIB, "profiles/pool_lds_kernel_global_avgpool.md"),
+    "resnet50_convs": (512.1e6, "profiles/conv_stack_resnet50.md"),
 }
 
 
@@ -65,6 +67,7 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=2000)
     ap.add_argument("--workload", default="fc4096",
                     choices=["fc4096", "fc8192", "quantize", "quantize_uncal", "quantize_uint8",
+                             "quantize_laplace", "quantize_uint8_uncal", "small_casts",
                              "requantize", "requantize_uncal", "dequantize", "copy", "maxpool", "avgpool",
                              "elemwise_add", "elemwise_add_int8", "concat", "elemwise_mul_int8", "quantize_asym",
                              "batch_norm", "embedding", "transpose", "resnet50_convs", "bert_fc_chain",
@@ -103,6 +106,7 @@ class FcWorkload:
         self.calib = (-r, r)
         self.out8 = torch.empty((S, S), dtype=torch.int8, device="cuda")
         self.sc = [torch.empty(1, device="cuda") for _ in range(4)]
+        self.ws = fc_workspace(torch, lib, S, S, S, True)
         self.lib = lib
         self.P = lambda t: ctypes.c_void_p(t.data_ptr())
         self.torch = torch
@@ -114,7 +118,7 @@ class FcWorkload:
                                        P(self.dmin), P(self.dmax), P(self.wmin), P(self.wmax),
                                        P(self.bmin), P(self.bmax), None, P(self.sc[0]),
                                        P(self.sc[1]), P(self.out8), P(self.sc[2]), P(self.sc[3]),
-                                       0, self.calib[0], self.calib[1])
+                                       0, self.calib[0], self.calib[1], *ws_args(self.ws))
         if rc != 0:
             raise RuntimeError(self.lib.mxq_last_error().decode())
 
@@ -145,6 +149,18 @@ class FcWorkload:
                                                                            dt)}
 
 
+def fc_workspace(torch, lib, M, N, K, fused):
+    """The scratch mxq_quantized_fc asks for on this shape (None when it would not split)."""
+    nbytes = lib.mxq_quantized_fc_workspace(M, N, K, int(fused))
+    return torch.empty(nbytes, dtype=torch.uint8, device="cuda") if nbytes else None
+
+
+def ws_args(ws):
+    if ws is None:
+        return None, 0
+    return ctypes.c_void_p(ws.data_ptr()), ws.numel()
+
+
 class CastWorkload:
     """Benchmark configuration 2: 64M-element flat tensors, buffers rotated so that the
     256 MB Infinity Cache cannot serve the reads."""
@@ -164,23 +180,35 @@ class CastWorkload:
         self.omin = torch.empty(1, device="cuda")
         self.omax = torch.empty(1, device="cuda")
         self.ws = torch.empty(lib.mxq_quantize_v2_workspace(n), dtype=torch.uint8, device="cuda")
-        if kind in ("quantize", "quantize_uncal", "quantize_uint8"):
+        if kind in ("quantize", "quantize_uncal", "quantize_uint8", "quantize_laplace",
+                    "quantize_uint8_uncal"):
             self.src = []
             for _ in range(self.NBUF):
-                x = torch.randn(n, device="cuda", generator=g)
+                if kind == "quantize_laplace":
+                    # Laplace(0, 1) by inversion of its distribution function
+                    u = torch.rand(n, device="cuda", generator=g) - 0.5
+                    x = -torch.sign(u) * torch.log1p(-2.0 * u.abs())
+                    del u
+                else:
+                    x = torch.randn(n, device="cuda", generator=g)
                 idx = torch.randint(0, n, (n // 10000,), device="cuda", generator=g)
                 sign = torch.randint(0, 2, (n // 10000,), device="cuda", generator=g) * 2 - 1
                 x[idx] = 50.0 * sign.to(torch.float32)
                 self.src.append(x)
             self.dst = [torch.empty(n, dtype=torch.uint8, device="cuda")
                         for _ in range(self.NBUF)]
-            self.bytes = (9.0 if kind == "quantize_uncal" else 5.0) * n
-            self.kernel = "quantize_kernel" + (" + minmax_f32_kernel"
-                                               if kind == "quantize_uncal" else "")
-            self.name = {"quantize": "quantize_v2 fp32->int8 calibrated (-50,50)",
+            uncal = kind in ("quantize_uncal", "quantize_uint8_uncal")
+            self.bytes = (9.0 if uncal else 5.0) * n
+            self.kernel = "quantize_kernel" + (" + minmax_f32_kernel" if uncal else "")
+            self.name = {"quantize": "quantize_v2 fp32->int8 calibrated (-50,50), N(0,1) input "
+                                     "with 0.01% outliers at +-50",
                          "quantize_uncal": "quantize_v2 fp32->int8 uncalibrated "
                                            "(on-device min/max)",
-                         "quantize_uint8": "quantize_v2 fp32->uint8 calibrated (-50,50)"}[kind]
+                         "quantize_uint8": "quantize_v2 fp32->uint8 calibrated (-50,50)",
+                         "quantize_laplace": "quantize_v2 fp32->int8 calibrated (-50,50), "
+                                             "Laplace(0,1) input with 0.01% outliers at +-50",
+                         "quantize_uint8_uncal": "quantize_v2 fp32->uint8 uncalibrated "
+                                                 "(on-device min/max)"}[kind]
         elif kind.startswith("requantize"):
             self.src = [torch.randint(-2 ** 28, 2 ** 28, (n,), device="cuda", generator=g,
                                       dtype=torch.int32) for _ in range(self.NBUF)]
@@ -311,9 +339,13 @@ class CastWorkload:
         self.i += 1
         st = ctypes.c_void_p(self.torch.cuda.current_stream().cuda_stream)
         kind = self.kind
-        if kind == "quantize":
+        if kind in ("quantize", "quantize_laplace"):
             rc = lib.mxq_quantize_v2(st, P(self.src[k]), P(self.dst[k]), P(self.omin),
                                      P(self.omax), n, 5, 1, -50.0, 50.0, None, 0)
+        elif kind == "quantize_uint8_uncal":
+            rc = lib.mxq_quantize_v2(st, P(self.src[k]), P(self.dst[k]), P(self.omin),
+                                     P(self.omax), n, 3, 0, 0.0, 0.0, P(self.ws),
+                                     self.ws.numel())
         elif kind == "quantize_uint8":
             rc = lib.mxq_quantize_v2(st, P(self.src[k]), P(self.dst[k]), P(self.omin),
                                      P(self.omax), n, 3, 1, -50.0, 50.0, None, 0)
@@ -392,8 +424,10 @@ class CastWorkload:
             x = self.src[0][:n].cpu().numpy()
         reps, t0 = 0, time.perf_counter()
         while True:
-            if kind == "quantize":
+            if kind in ("quantize", "quantize_laplace"):
                 oracle.quantize_v2(x, "int8", -50.0, 50.0)
+            elif kind == "quantize_uint8_uncal":
+                oracle.quantize_v2(x, "uint8")
             elif kind == "quantize_uint8":
                 oracle.quantize_v2(x, "uint8", -50.0, 50.0)
             elif kind == "quantize_uncal":
@@ -554,6 +588,69 @@ class GraphWorkload:
         return None
 
 
+class SmallCastsWorkload(GraphWorkload):
+    """The cast operators at the sizes they have inside benchmark configurations 1 and 5:
+    [128,1024] and [4096,768], [4096,2304], [4096,3072].  One step = calibrated quantize_v2,
+    calibrated requantize and dequantize of every size (12 launches in one graph).  The
+    operands of these sizes sit in the caches, so the table reports time per launch and the
+    algorithmic GB/s it amounts to, not a fraction of HBM peak worth quoting."""
+    SIZES = [(128, 1024), (4096, 768), (4096, 2304), (4096, 3072)]
+
+    def __init__(self, torch, lib):
+        self.kernel = "quantize_kernel / requantize_kernel / dequantize_kernel"
+        self.bound = "hbm"
+        self.name = "quantize_v2, requantize, dequantize at [128,1024], [4096,768], " \
+                    "[4096,2304], [4096,3072] (calibrated), 12 launches per step"
+        P = lambda t: ctypes.c_void_p(t.data_ptr())
+        g = torch.Generator(device="cuda").manual_seed(6)
+        self.bytes = 0.0
+        self.items = []
+        one = [torch.tensor([v], device="cuda") for v in (-1.0, 1.0)]
+        sc = [torch.empty(1, device="cuda") for _ in range(2)]
+        for (r, c) in self.SIZES:
+            n = r * c
+            x = torch.randn(n, device="cuda", generator=g)
+            a = torch.randint(-2 ** 28, 2 ** 28, (n,), device="cuda", generator=g,
+                              dtype=torch.int32)
+            q = torch.randint(-127, 128, (n,), device="cuda", generator=g, dtype=torch.int8)
+            o8 = torch.empty(n, dtype=torch.int8, device="cuda")
+            of = torch.empty(n, dtype=torch.float32, device="cuda")
+            self.items.append((n, x, a, q, o8, of))
+            self.bytes += 15.0 * n
+        self.keep = (one, sc)
+
+        def body(only=None):
+            st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+            j = 0
+            for (n, x, a, q, o8, of) in self.items:
+                calls = [
+                    lambda: lib.mxq_quantize_v2(st, P(x), P(o8), P(sc[0]), P(sc[1]), n, 5, 1,
+                                                -4.0, 4.0, None, 0),
+                    lambda: lib.mxq_requantize(st, P(a), P(one[0]), P(one[1]), P(o8), P(sc[0]),
+                                               P(sc[1]), n, 1, -0.1, 0.1, None, 0),
+                    lambda: lib.mxq_dequantize(st, P(q), 5, P(one[0]), P(one[1]), P(of), n)]
+                for call in calls:
+                    if only is None or only == j:
+                        if call() != 0:
+                            raise RuntimeError(lib.mxq_last_error().decode())
+                    j += 1
+        self.body = body
+        self.capture(torch, body)
+
+    def value(self, sec_per_step):
+        return self.bytes / sec_per_step / 1e9, "GB/s"
+
+    def per_layer(self, torch):
+        rows, j = [], 0
+        for (r, c) in self.SIZES:
+            for op in ("quantize_v2", "requantize", "dequantize"):
+                t = self.time_alone(torch, lambda: self.body(j), reps=20)
+                rows.append({"launch": "%s [%d,%d]" % (op, r, c), "us": round(t * 1e6, 2),
+                             "GB/s": round(5.0 * r * c / t / 1e9, 1)})
+                j += 1
+        return rows
+
+
 # ResNet-50 v1 bottleneck convolutions, batch 64: (H, Cin, Cout, kernel, stride)
 RESNET50_CONVS = [(56, 64, 64, 1, 1), (56, 64, 64, 3, 1), (56, 64, 256, 1, 1), (56, 256, 64, 1, 1),
                   (56, 256, 128, 1, 2), (28, 128, 128, 3, 1), (28, 128, 512, 1, 1),
@@ -588,25 +685,27 @@ class ConvStackWorkload(GraphWorkload):
             bq, bmin, bmax = capi.quantize(b, b.min().reshape(1), b.max().reshape(1), "int8")
             out8 = torch.empty((N, OH, OH, O), dtype=torch.int8, device="cuda")
             sc = [torch.empty(1, device="cuda") for _ in range(4)]
+            nws = lib.mxq_quantized_conv_workspace(N, H, H, C, O, k, k, s, s, pad, pad, 1, 1, 1)
+            ws = torch.empty(nws, dtype=torch.uint8, device="cuda") if nws else None
             # naive calibration: range of the fp32 output of this layer on a batch slice
             ref = torch.nn.functional.conv2d(x[:4].permute(0, 3, 1, 2), w.permute(0, 3, 1, 2), b,
                                              stride=s, padding=pad)
             r = float(ref.abs().max().item())
             self.layers.append((d, wq, bq, dmin, dmax, wmin, wmax, bmin, bmax, out8, sc,
-                                (N, H, H, C, O, k, k, s, s, pad, pad), r))
+                                (N, H, H, C, O, k, k, s, s, pad, pad), r, ws))
             self.ops += 2.0 * N * OH * OH * O * k * k * C
             del x, w, ref
 
         def body(only=None):
             st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
             for i, (d, wq, bq, dmin, dmax, wmin, wmax, bmin, bmax, out8, sc, geo,
-                    r) in enumerate(self.layers):
+                    r, ws) in enumerate(self.layers):
                 if only is not None and i != only:
                     continue
                 rc = lib.mxq_quantized_conv_nhwc(st, P(d), P(wq), P(bq), *geo, 1, 1, P(dmin),
                                                  P(dmax), P(wmin), P(wmax), P(bmin), P(bmax),
                                                  None, P(sc[0]), P(sc[1]), P(out8), P(sc[2]),
-                                                 P(sc[3]), 1, -r, r)
+                                                 P(sc[3]), 1, -r, r, *ws_args(ws))
                 if rc != 0:
                     raise RuntimeError(lib.mxq_last_error().decode())
         self.body = body
@@ -659,7 +758,8 @@ class BertChainWorkload(GraphWorkload):
                         acc=torch.empty((M, N), dtype=torch.int32, device="cuda"),
                         q8=torch.empty((M, N), dtype=torch.int8, device="cuda"),
                         y=torch.empty((M, N), dtype=torch.float32, device="cuda"),
-                        sc=[torch.empty(1, device="cuda") for _ in range(6)])
+                        sc=[torch.empty(1, device="cuda") for _ in range(6)],
+                        ws=fc_workspace(torch, lib, M, N, K, fused))
             self.layers.append((K, N, wq, bq, wmin, wmax, bmin, bmax, r, bufs))
             self.ops += 2.0 * M * N * K
             del w
@@ -677,7 +777,7 @@ class BertChainWorkload(GraphWorkload):
                         lib.mxq_quantized_fc(st, P(B["q"]), P(wq), P(bq), M, N, K, P(sc[0]),
                                              P(sc[1]), P(wmin), P(wmax), P(bmin), P(bmax), None,
                                              P(sc[2]), P(sc[3]), P(B["q8"]), P(sc[4]), P(sc[5]),
-                                             0, -r, r),
+                                             0, -r, r, *ws_args(B["ws"])),
                         lib.mxq_dequantize(st, P(B["q8"]), 5, P(sc[4]), P(sc[5]), P(B["y"]),
                                            M * N)]
                     if any(rcs):
@@ -688,7 +788,8 @@ class BertChainWorkload(GraphWorkload):
                                         -20.0, 20.0, None, 0),
                     lib.mxq_quantized_fc(st, P(B["q"]), P(wq), P(bq), M, N, K, P(sc[0]), P(sc[1]),
                                          P(wmin), P(wmax), P(bmin), P(bmax), P(B["acc"]),
-                                         P(sc[2]), P(sc[3]), None, None, None, 0, 0.0, 0.0),
+                                         P(sc[2]), P(sc[3]), None, None, None, 0, 0.0, 0.0,
+                                         *ws_args(B["ws"])),
                     lib.mxq_requantize(st, P(B["acc"]), P(sc[2]), P(sc[3]), P(B["q8"]), P(sc[4]),
                                        P(sc[5]), M * N, 1, -r, r, None, 0),
                     lib.mxq_dequantize(st, P(B["q8"]), 5, P(sc[4]), P(sc[5]), P(B["y"]), M * N)]
@@ -713,7 +814,7 @@ def mfma_context(torch, S):
     all, zero vs random operand bytes) and the vendor int8 GEMM (hipBLASLt through
     torch._int_mm, int32 output, no bias, no requantize) on the same operand shapes."""
     out = {}
-    path = os.path.join(ROOT, "mxnet_amd", "libmxq_probe.so")
+    path = os.path.join(ROOT, "bench_probe.so")
     if os.path.exists(path):
         probe = ctypes.CDLL(path)
         probe.mxq_probe_mfma_i8.restype = ctypes.c_double
@@ -771,6 +872,8 @@ def make_workload(name, torch, capi, lib):
         return BertChainWorkload(torch, capi, lib, fused=True)
     if name == "copy":
         return CopyWorkload(torch)
+    if name == "small_casts":
+        return SmallCastsWorkload(torch, lib)
     if name in ("maxpool", "avgpool"):
         return PoolWorkload(name, torch, lib)
     if name == "fc4096":
@@ -780,8 +883,33 @@ def make_workload(name, torch, capi, lib):
     return CastWorkload(name, torch, capi, lib)
 
 
+SETTLE_MS = 250.0
+
+
+def settle(torch, wl, min_gpu_ms=SETTLE_MS):
+    """Untimed steps of the same workload until at least `min_gpu_ms` of GPU time have
+    passed: over the first ~100 ms after an idle period the clocks have not settled and
+    every kernel here runs 5-15 % slower, whatever --warmup says.  Returns the GPU
+    milliseconds spent."""
+    spent, batch = 0.0, 8
+    while spent < min_gpu_ms:
+        e0 = torch.cuda.Event(enable_timing=True)
+        e1 = torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(batch):
+            wl.step()
+        e1.record()
+        torch.cuda.synchronize()
+        spent += e0.elapsed_time(e1)
+        batch = min(batch * 2, 4096)
+    return spent
+
+
 def timed_run(torch, wl, steps, warmup):
-    """Returns (wall seconds for `steps` steps, HIP-event seconds for the same steps)."""
+    """Returns (wall seconds for `steps` steps, HIP-event seconds for the same steps).
+    The events are recorded on the stream the kernels are launched on (torch's current
+    stream, whose handle every step passes to the C ABI)."""
+    wl.settle_ms = settle(torch, wl)
     for _ in range(warmup):
         wl.step()
     torch.cuda.synchronize()
@@ -806,7 +934,8 @@ def roofline_of(wl, event_s_per_launch, key=None):
         peak, unit = HBM_PEAK_GBS, "GB/s"
     return {"bound": wl.bound, "kernel": wl.kernel, "achieved": round(achieved, 1), "peak": peak,
             "unit": unit, "frac": round(achieved / peak, 4),
-            "traffic": MEASURED_TRAFFIC_BYTES.get(key),
+            "traffic": MEASURED_TRAFFIC_BYTES.get(key, (None, None))[0],
+            "traffic_source": MEASURED_TRAFFIC_BYTES.get(key, (None, None))[1],
             "avg_launch_us": round(event_s_per_launch * 1e6, 2)}
 
 
@@ -844,6 +973,7 @@ def main():
         "data": "synthetic",
         "config": {"workload": wl.name},
         "device": torch.cuda.get_device_name(0),
+        "settle_ms": round(wl.settle_ms, 1),
         "roofline": roofline_of(wl, ev / args.steps, args.workload),
     }
 
@@ -854,7 +984,8 @@ def main():
 
     if not args.no_cast_ops:
         rows = []
-        for kind in ["quantize", "quantize_uint8", "quantize_uncal", "requantize",
+        for kind in ["quantize", "quantize_laplace", "quantize_uint8", "quantize_uncal",
+                     "quantize_uint8_uncal", "small_casts", "requantize",
                      "requantize_uncal", "dequantize", "elemwise_add", "elemwise_add_int8",
                      "concat", "elemwise_mul_int8", "quantize_asym", "batch_norm", "embedding",
                      "transpose", "maxpool", "avgpool", "fc8192",
@@ -863,7 +994,7 @@ def main():
                 continue
             w2 = make_workload(kind, torch, capi, lib)
             steps2 = 300
-            wall2, ev2 = timed_run(torch, w2, steps2, 300)
+            wall2, ev2 = timed_run(torch, w2, steps2, 20)
             r = roofline_of(w2, ev2 / steps2, kind)
             r["workload"] = w2.name
             if isinstance(w2, GraphWorkload):

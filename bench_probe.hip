@@ -1,4 +1,4 @@
-// libmxq_probe.so - measurement aid for the benchmark, not part of the operator ABI.
+// bench_probe.so - measurement aid for the benchmark, not part of the operator ABI.
 //
 // mxq_probe_mfma_i8 runs v_mfma_i32_32x32x32_i8 back to back out of registers: no
 // LDS, no global memory in the loop, the register shape of the FC kernel's wave

@@ -8,7 +8,10 @@
  *   - takes plain device pointers, sizes and a raw hipStream_t (as void*; NULL
  *     is the default stream),
  *   - only enqueues work on that stream: no allocation, no free, no device or
- *     stream synchronisation, no retained state,
+ *     stream synchronisation, no retained state (the library has no mutable
+ *     process-wide variables; the entry points are re-entrant and may be called
+ *     concurrently from different threads on different streams, provided that
+ *     calls in flight at the same time do not share a workspace),
  *   - returns 0 on success and -1 on failure with the message available from
  *     mxq_last_error() on the calling thread (the convention of
  *     include/mxnet/c_api_error.h:39-58 in the reference).
@@ -27,7 +30,7 @@
 extern "C" {
 #endif
 
-#define MXQ_ABI_VERSION 1
+#define MXQ_ABI_VERSION 2
 
 /* element type codes = mshadow::TypeFlag (3rdparty/mshadow/mshadow/base.h:351-364) */
 #define MXQ_FLOAT32 0
@@ -263,13 +266,22 @@ int mxq_quantized_concat(void* stream, int num_args, const void* const* in, cons
  *               accumulator with the calibrated range (min_calib, max_calib),
  *               bit-identical to mxq_requantize on out32; relu != 0 clamps the
  *               int8 at zero; rmin/rmax receive the requantized range.
- * At least one of out32 / out8 must be given. */
+ * At least one of out32 / out8 must be given.
+ *   workspace   device scratch (16-byte aligned) or NULL.  Shapes with few output tiles and
+ *               a long K are split along K over several work-groups per tile, which leave
+ *               their int32 partial sums in the workspace (integer addition is
+ *               associative: the result is the unsplit one bit for bit); this is the
+ *               operator's kTempSpace (quantized_fully_connected.cc:369-372).
+ *               mxq_quantized_fc_workspace() returns the bytes with which the call takes
+ *               its fastest route (0 when it would not split; fused_int8_only != 0 says
+ *               that only out8 will be given); with less, or NULL, nothing is split. */
+size_t mxq_quantized_fc_workspace(int M, int N, int K, int fused_int8_only);
 int mxq_quantized_fc(void* stream, const int8_t* data, const int8_t* weight, const int8_t* bias,
                      int M, int N, int K, const float* min_data, const float* max_data,
                      const float* min_weight, const float* max_weight, const float* min_bias,
                      const float* max_bias, int32_t* out32, float* omin, float* omax,
                      int8_t* out8, float* rmin, float* rmax, int relu, float min_calib,
-                     float max_calib);
+                     float max_calib, void* workspace, size_t workspace_bytes);
 
 /* ---- _contrib_quantized_conv ----------------------------------------------
  * Replaces QuantizedCuDNNConvOp::Forward
@@ -278,7 +290,11 @@ int mxq_quantized_fc(void* stream, const int8_t* data, const int8_t* weight, con
  * kernel.  Operands are NHWC here (data [N,H,W,C], weight [O,KH,KW,C], output
  * [N,OH,OW,O]); the layout adapters below replace the three TransposeImpl calls
  * (:147-148,183) for callers holding the operator's NCHW tensors.  Epilogue
- * arguments as for mxq_quantized_fc. */
+ * and workspace arguments as for mxq_quantized_fc (the reference passes cuDNN its own
+ * workspace out of the operator's temp space, quantized_conv.cu:121-177). */
+size_t mxq_quantized_conv_workspace(int N, int H, int W, int C, int O, int KH, int KW,
+                                    int stride_h, int stride_w, int pad_h, int pad_w,
+                                    int dilate_h, int dilate_w, int fused_int8_only);
 int mxq_quantized_conv_nhwc(void* stream, const int8_t* data, const int8_t* weight,
                             const int8_t* bias, int N, int H, int W, int C, int O, int KH,
                             int KW, int stride_h, int stride_w, int pad_h, int pad_w,
@@ -287,7 +303,7 @@ int mxq_quantized_conv_nhwc(void* stream, const int8_t* data, const int8_t* weig
                             const float* max_weight, const float* min_bias,
                             const float* max_bias, int32_t* out32, float* omin, float* omax,
                             int8_t* out8, float* rmin, float* rmax, int relu, float min_calib,
-                            float max_calib);
+                            float max_calib, void* workspace, size_t workspace_bytes);
 /* The same convolution with the int32 output written as the operator's own layout,
  * [N,O,OH,OW]: the kernel's epilogue stores channel planes directly, which replaces the
  * third TransposeImpl (quantized_conv.cu:183) and the NHWC int32 buffer it reads. */
@@ -298,7 +314,8 @@ int mxq_quantized_conv_nhwc_out_nchw(void* stream, const int8_t* data, const int
                                      const float* min_data, const float* max_data,
                                      const float* min_weight, const float* max_weight,
                                      const float* min_bias, const float* max_bias,
-                                     int32_t* out32_nchw, float* omin, float* omax);
+                                     int32_t* out32_nchw, float* omin, float* omax,
+                                     void* workspace, size_t workspace_bytes);
 
 /* [N,C,H,W] int8 -> [N,H,W,C] int8 (also OIHW -> OHWI for the weight). */
 int mxq_nchw_to_nhwc_i8(void* stream, const int8_t* in, int8_t* out, int N, int C, int H, int W);

@@ -56,12 +56,14 @@ SIGNATURES = {
                                  [ctypes.c_int64] * 3 + [ctypes.c_double, _f, _f, _i, _p, _sz]),
     "mxq_quantized_concat": (_i, [_p, _i, _p, _p, _p, _p, _p, ctypes.c_int64, ctypes.c_int64, _p,
                                   _i, _p, _p]),
+    "mxq_quantized_fc_workspace": (_sz, [_i, _i, _i, _i]),
     "mxq_quantized_fc": (_i, [_p, _p, _p, _p, _i, _i, _i] + [_p] * 6 + [_p, _p, _p, _p, _p, _p,
-                              _i, _f, _f]),
+                              _i, _f, _f, _p, _sz]),
+    "mxq_quantized_conv_workspace": (_sz, [_i] * 14),
     "mxq_quantized_conv_nhwc": (_i, [_p, _p, _p, _p] + [_i] * 13 + [_p] * 6 +
-                                [_p, _p, _p, _p, _p, _p, _i, _f, _f]),
+                                [_p, _p, _p, _p, _p, _p, _i, _f, _f, _p, _sz]),
     "mxq_quantized_conv_nhwc_out_nchw": (_i, [_p, _p, _p, _p] + [_i] * 13 + [_p] * 6 +
-                                         [_p, _p, _p]),
+                                         [_p, _p, _p, _p, _sz]),
     "mxq_nchw_to_nhwc_i8": (_i, [_p, _p, _p, _i, _i, _i, _i]),
     "mxq_nchw_to_nhwc_pad_i8": (_i, [_p, _p, _p, _i, _i, _i, _i, _i]),
     "mxq_nchw_to_s2d_nhwc_i8": (_i, [_p, _p, _p, _i, _i, _i, _i, _i, _i, _i]),
@@ -73,9 +75,17 @@ for _name, (_res, _args) in SIGNATURES.items():
     _fn.restype = _res
     _fn.argtypes = _args
 
-# development knob, not part of include/mxq.h
-lib.mxq_set_tuning.restype = _i
-lib.mxq_set_tuning.argtypes = [ctypes.c_char_p, _i]
+# test-only twins of the FC and convolution entry points (tests/mxq_test_hooks.h, not part
+# of include/mxq.h): the same arguments followed by the tile configuration, the split-K
+# factor and, for the FC, the streaming kernel's work-groups per CU (0 = choose)
+TEST_HOOKS = {
+    "mxq_test_quantized_fc": (_i, SIGNATURES["mxq_quantized_fc"][1] + [_i, _i, _i]),
+    "mxq_test_quantized_conv_nhwc": (_i, SIGNATURES["mxq_quantized_conv_nhwc"][1] + [_i, _i]),
+}
+for _name, (_res, _args) in TEST_HOOKS.items():
+    _fn = getattr(lib, _name)
+    _fn.restype = _res
+    _fn.argtypes = _args
 
 
 def last_error():
@@ -85,8 +95,3 @@ def last_error():
 def check(rc):
     if rc != 0:
         raise MXQError(last_error())
-
-
-def set_tuning(key, value):
-    if lib.mxq_set_tuning(key.encode(), int(value)) != 0:
-        raise MXQError("unknown tuning key or bad value: %s=%r" % (key, value))

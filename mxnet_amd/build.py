@@ -55,14 +55,15 @@ def build(verbose=False):
     return LIB
 
 
-PROBE_LIB = os.path.join(HERE, "libmxq_probe.so")
+ROOT = os.path.dirname(HERE)
+PROBE_LIB = os.path.join(ROOT, "bench_probe.so")
 
 
 def build_probe(verbose=False):
-    """libmxq_probe.so: the register-only MFMA rate probe bench.py reports next to the
-    FC figures.  Kept out of libmxq_hip.so: it is not an operator."""
+    """bench_probe.so: the register-only MFMA rate probe bench.py reports next to the FC
+    figures.  A bench aid kept beside bench.py, not part of the operator library."""
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
-    cmd = [hipcc] + HIPCC_FLAGS + ["-shared", os.path.join(CSRC, "mxq_probe.hip"), "-o",
+    cmd = [hipcc] + HIPCC_FLAGS + ["-shared", os.path.join(ROOT, "bench_probe.hip"), "-o",
                                    PROBE_LIB]
     if verbose:
         print(" ".join(cmd), flush=True)
@@ -72,7 +73,7 @@ def build_probe(verbose=False):
     if text:
         print(text)
     if out.returncode != 0:
-        raise RuntimeError("hipcc failed: mxq_probe.hip")
+        raise RuntimeError("hipcc failed: bench_probe.hip")
     return PROBE_LIB
 
 

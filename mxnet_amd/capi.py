@@ -30,6 +30,11 @@ def _workspace(nbytes, dev):
     return torch.empty(nbytes, dtype=torch.uint8, device=dev)
 
 
+# scratch handed to the test-only entry points when a test pins a split-K factor: room for
+# the partial sums of every case the tests run (the launcher checks the size it needs)
+_SPLIT_WS_BYTES = 96 << 20
+
+
 def quantize_v2(data, out_type="int8", min_calib_range=None, max_calib_range=None):
     assert data.dtype == torch.float32
     calibrated = min_calib_range is not None and max_calib_range is not None
@@ -87,9 +92,10 @@ def dequantize(data, min_range, max_range):
 
 
 def quantized_fc(data, weight, bias, min_data, max_data, min_weight, max_weight, min_bias=None,
-                 max_bias=None, want_int32=True, calib=None, relu=False):
+                 max_bias=None, want_int32=True, calib=None, relu=False, force=None):
     """data int8 [M,K], weight int8 [N,K], bias int8 [N] or None.
-    Returns dict(out32, omin, omax[, out8, rmin, rmax])."""
+    Returns dict(out32, omin, omax[, out8, rmin, rmax]).  `force` = (cfg, splits,
+    stream_groups) goes through the test-only entry point that pins the kernel variant."""
     M, K = data.shape
     N, K2 = weight.shape
     assert K == K2
@@ -102,19 +108,28 @@ def quantized_fc(data, weight, bias, min_data, max_data, min_weight, max_weight,
         out8 = torch.empty((M, N), dtype=torch.int8, device=dev)
         rmin, rmax = _scalar(dev), _scalar(dev)
         lo, hi = float(calib[0]), float(calib[1])
-    check(lib.mxq_quantized_fc(_stream(), _ptr(data), _ptr(weight), _ptr(bias), M, N, K,
-                               _ptr(min_data), _ptr(max_data), _ptr(min_weight),
-                               _ptr(max_weight), _ptr(min_bias), _ptr(max_bias), _ptr(out32),
-                               _ptr(res["omin"]), _ptr(res["omax"]), _ptr(out8), _ptr(rmin),
-                               _ptr(rmax), int(relu), lo, hi))
+    args = [_stream(), _ptr(data), _ptr(weight), _ptr(bias), M, N, K, _ptr(min_data),
+            _ptr(max_data), _ptr(min_weight), _ptr(max_weight), _ptr(min_bias), _ptr(max_bias),
+            _ptr(out32), _ptr(res["omin"]), _ptr(res["omax"]), _ptr(out8), _ptr(rmin),
+            _ptr(rmax), int(relu), lo, hi]
+    if force is None:
+        wsb = lib.mxq_quantized_fc_workspace(M, N, K, int(not want_int32))
+        ws = _workspace(wsb, dev) if wsb else None
+        check(lib.mxq_quantized_fc(*args, _ptr(ws), wsb))
+    else:
+        cfg, splits, groups = force
+        wsb = _SPLIT_WS_BYTES if splits != 1 else 0
+        ws = _workspace(wsb, dev) if wsb else None
+        check(lib.mxq_test_quantized_fc(*args, _ptr(ws), wsb, cfg, splits, groups))
     res.update(out32=out32, out8=out8, rmin=rmin, rmax=rmax)
     return res
 
 
 def quantized_conv_nhwc(data, weight, bias, min_data, max_data, min_weight, max_weight,
                         min_bias=None, max_bias=None, stride=(1, 1), pad=(0, 0), dilate=(1, 1),
-                        want_int32=True, calib=None, relu=False):
-    """data int8 [N,H,W,C], weight int8 [O,KH,KW,C] -> out [N,OH,OW,O]."""
+                        want_int32=True, calib=None, relu=False, force=None):
+    """data int8 [N,H,W,C], weight int8 [O,KH,KW,C] -> out [N,OH,OW,O].  `force` = (cfg,
+    splits) goes through the test-only entry point that pins the kernel variant."""
     N, H, W, C = data.shape
     O, KH, KW, C2 = weight.shape
     assert C == C2
@@ -129,13 +144,20 @@ def quantized_conv_nhwc(data, weight, bias, min_data, max_data, min_weight, max_
         out8 = torch.empty((N, OH, OW, O), dtype=torch.int8, device=dev)
         rmin, rmax = _scalar(dev), _scalar(dev)
         lo, hi = float(calib[0]), float(calib[1])
-    check(lib.mxq_quantized_conv_nhwc(_stream(), _ptr(data), _ptr(weight), _ptr(bias), N, H, W,
-                                      C, O, KH, KW, stride[0], stride[1], pad[0], pad[1],
-                                      dilate[0], dilate[1], _ptr(min_data), _ptr(max_data),
-                                      _ptr(min_weight), _ptr(max_weight), _ptr(min_bias),
-                                      _ptr(max_bias), _ptr(out32), _ptr(res["omin"]),
-                                      _ptr(res["omax"]), _ptr(out8), _ptr(rmin), _ptr(rmax),
-                                      int(relu), lo, hi))
+    geo = [N, H, W, C, O, KH, KW, stride[0], stride[1], pad[0], pad[1], dilate[0], dilate[1]]
+    args = [_stream(), _ptr(data), _ptr(weight), _ptr(bias)] + geo + [
+        _ptr(min_data), _ptr(max_data), _ptr(min_weight), _ptr(max_weight), _ptr(min_bias),
+        _ptr(max_bias), _ptr(out32), _ptr(res["omin"]), _ptr(res["omax"]), _ptr(out8),
+        _ptr(rmin), _ptr(rmax), int(relu), lo, hi]
+    if force is None:
+        wsb = lib.mxq_quantized_conv_workspace(*geo, int(not want_int32))
+        ws = _workspace(wsb, dev) if wsb else None
+        check(lib.mxq_quantized_conv_nhwc(*args, _ptr(ws), wsb))
+    else:
+        cfg, splits = force
+        wsb = _SPLIT_WS_BYTES if splits != 1 else 0
+        ws = _workspace(wsb, dev) if wsb else None
+        check(lib.mxq_test_quantized_conv_nhwc(*args, _ptr(ws), wsb, cfg, splits))
     res.update(out32=out32, out8=out8, rmin=rmin, rmax=rmax)
     return res
 

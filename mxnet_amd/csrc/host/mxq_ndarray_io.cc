@@ -87,11 +87,14 @@ std::vector<int64_t> ReadShape(Reader* r, bool* unknown) {
   return shape;
 }
 
+// Product of the extents; a crafted file whose product wraps around is refused rather than
+// read into a buffer that no longer matches its shape.
 size_t Elements(const std::vector<int64_t>& shape) {
   size_t n = 1;
   for (const int64_t d : shape) {
     CHECK(d >= 0) << "Invalid NDArray file format (negative extent)";
-    n *= static_cast<size_t>(d);
+    CHECK(!__builtin_mul_overflow(n, static_cast<size_t>(d), &n))
+        << "Invalid NDArray file format (element count overflows)";
   }
   return n;
 }
@@ -100,7 +103,11 @@ void ReadBody(Reader* r, Array* a) {
   (void)r->Get<int32_t>();  // context: device type
   (void)r->Get<int32_t>();  //          device id
   a->dtype = r->Get<int32_t>();
-  a->data.resize(TypeSize(a->dtype) * Elements(a->shape));
+  size_t bytes = 0;
+  CHECK(!__builtin_mul_overflow(static_cast<size_t>(TypeSize(a->dtype)), Elements(a->shape),
+                                &bytes))
+      << "Invalid NDArray file format (byte count overflows)";
+  a->data.resize(bytes);
   if (!a->data.empty()) r->Read(a->data.data(), a->data.size());
   a->none = false;
 }
@@ -145,6 +152,14 @@ class Writer {
   }
   void Write(const void* p, size_t n) {
     CHECK(std::fwrite(p, 1, n, f_) == n) << "write failed";
+  }
+  // Flushes and closes; a full disk shows up here, not as a silently truncated file.
+  void Close() {
+    FILE* f = f_;
+    f_ = nullptr;
+    const int flushed = std::fflush(f);
+    const int closed = std::fclose(f);
+    CHECK(flushed == 0 && closed == 0) << "write failed (flush / close)";
   }
   template <typename T>
   void Put(T v) {
@@ -253,6 +268,7 @@ int mxq_ndlist_save(const char* path, int count, const char** names, const mxq_b
     w.Put<uint64_t>(len);
     w.Write(names[i], len);
   }
+  w.Close();
   IO_API_END();
 }
 

@@ -619,6 +619,12 @@ static void QuantizedFullyConnectedForwardGPU(const NodeAttrs& attrs, const OpCo
   const index_t n = wshape[0];
   CHECK_EQ(wshape[1], k);
   const int8_t* bias = param.no_bias ? nullptr : inputs[2].dptr<int8_t>();
+  // the operator's temp space (quantized_fully_connected.cc:369-372) carries the split-K
+  // partial sums of shapes with few output tiles and a long reduction
+  const size_t ws_bytes = mxq_quantized_fc_workspace(static_cast<int>(m), static_cast<int>(n),
+                                                     static_cast<int>(k), 0);
+  void* ws = nullptr;
+  if (ws_bytes != 0 && !ctx.requested.empty()) ws = ctx.requested[0].get_space(ws_bytes);
   MXQ_CALL(mxq_quantized_fc(
       raw_stream(ctx), inputs[0].dptr<int8_t>(), inputs[1].dptr<int8_t>(), bias,
       static_cast<int>(m), static_cast<int>(n), static_cast<int>(k),
@@ -626,7 +632,8 @@ static void QuantizedFullyConnectedForwardGPU(const NodeAttrs& attrs, const OpCo
       inputs[num_inputs + 2].dptr<float>(), inputs[num_inputs + 3].dptr<float>(),
       param.no_bias ? nullptr : inputs[7].dptr<float>(),
       param.no_bias ? nullptr : inputs[8].dptr<float>(), outputs[0].dptr<int32_t>(),
-      outputs[1].dptr<float>(), outputs[2].dptr<float>(), nullptr, nullptr, nullptr, 0, 0.f, 0.f));
+      outputs[1].dptr<float>(), outputs[2].dptr<float>(), nullptr, nullptr, nullptr, 0, 0.f, 0.f,
+      ws, ws != nullptr ? ws_bytes : 0));
 }
 
 // Temp space of the convolution: NHWC copies of data and weight plus the NHWC int32
@@ -670,21 +677,50 @@ static ConvS2D ConvSpaceToDepth(const ConvolutionParam& param, const TShape& d, 
   return r;
 }
 
+// The convolution as the kernel sees it: NHWC extents after channel padding or the
+// space-to-depth transform, and the bytes of the two operand copies in temp space.
+struct ConvKernelView {
+  ConvS2D s2d;
+  int H, W, C, KH, KW, sh, sw, ph, pw;
+  size_t d_bytes, w_bytes;  // rounded up to 256
+};
+static ConvKernelView ConvView(const ConvolutionParam& param, const TShape& d, const TShape& w,
+                               const TShape& o) {
+  auto up = [](size_t x) { return (x + 255) / 256 * 256; };
+  ConvKernelView v;
+  v.s2d = ConvSpaceToDepth(param, d, w, o);
+  const int N = d[0], C = d[1], O = w[0];
+  if (v.s2d.use) {
+    v.C = ConvPaddedChannels(4 * C);
+    v.H = v.s2d.H2; v.W = v.s2d.W2; v.KH = v.s2d.K2h; v.KW = v.s2d.K2w;
+    v.sh = v.sw = 1;
+    v.ph = v.s2d.pad_h; v.pw = v.s2d.pad_w;
+  } else {
+    v.C = ConvPaddedChannels(C);
+    v.H = d[2]; v.W = d[3]; v.KH = w[2]; v.KW = w[3];
+    v.sh = static_cast<int>(param.stride[0]); v.sw = static_cast<int>(param.stride[1]);
+    v.ph = static_cast<int>(param.pad[0]); v.pw = static_cast<int>(param.pad[1]);
+  }
+  v.d_bytes = up(static_cast<size_t>(N) * v.H * v.W * v.C);
+  v.w_bytes = up(static_cast<size_t>(O) * v.KH * v.KW * v.C);
+  return v;
+}
+
+// Bytes of split-K scratch the convolution kernel wants for this view (0: no split).
+static size_t ConvSplitBytes(const ConvolutionParam& param, const ConvKernelView& v, int N,
+                             int O) {
+  if (N <= 0 || O <= 0 || v.C <= 0) return 0;
+  return mxq_quantized_conv_workspace(N, v.H, v.W, v.C, O, v.KH, v.KW, v.sh, v.sw, v.ph, v.pw,
+                                      static_cast<int>(param.dilate[0]),
+                                      static_cast<int>(param.dilate[1]), 0);
+}
+
 static size_t QuantizedConvTempBytes(const ConvolutionParam& param, const TShape& d,
                                      const TShape& w, const TShape& o) {
-  auto up = [](size_t x) { return (x + 255) / 256 * 256; };
-  const ConvS2D s2d = ConvSpaceToDepth(param, d, w, o);
-  if (s2d.use) {
-    const size_t CP = static_cast<size_t>(ConvPaddedChannels(4 * static_cast<int>(d[1])));
-    return up(static_cast<size_t>(d[0]) * s2d.H2 * s2d.W2 * CP) +
-           up(static_cast<size_t>(w[0]) * s2d.K2h * s2d.K2w * CP);
-  }
-  const size_t C = static_cast<size_t>(d[1]);
-  const size_t scale_num = static_cast<size_t>(ConvPaddedChannels(static_cast<int>(C)));
-  const size_t d_bytes = C == 0 ? 0 : d.Size() / C * scale_num;
-  const size_t w_bytes = C == 0 ? 0 : w.Size() / C * scale_num;
+  const ConvKernelView v = ConvView(param, d, w, o);
   // the output is written in its own layout: no third buffer
-  return up(d_bytes) + up(w_bytes);
+  return v.d_bytes + v.w_bytes +
+         ConvSplitBytes(param, v, static_cast<int>(d[0]), static_cast<int>(w[0]));
 }
 
 // QuantizedConvForwardGPU, quantized_conv.cu:268-291
@@ -700,41 +736,32 @@ static void QuantizedConvForwardGPU(const NodeAttrs& attrs, const OpContext& ctx
   const TShape& w = inputs[1].shape_;
   const TShape& o = outputs[0].shape_;
   CHECK(!ctx.requested.empty()) << "quantized_conv needs its temp space resource";
-  auto up = [](size_t x) { return (x + 255) / 256 * 256; };
-  char* ws = ctx.requested[0].get_space(QuantizedConvTempBytes(param, d, w, o));
   const int N = d[0], C = d[1], H = d[2], W = d[3], O = w[0], KH = w[2], KW = w[3];
+  const ConvKernelView v = ConvView(param, d, w, o);
+  const size_t split_bytes = ConvSplitBytes(param, v, N, O);
+  char* ws = ctx.requested[0].get_space(v.d_bytes + v.w_bytes + split_bytes);
   void* stream = raw_stream(ctx);
   int8_t* d_nhwc = reinterpret_cast<int8_t*>(ws);
-  // the convolution as the kernel sees it
-  int cH = H, cW = W, cC = ConvPaddedChannels(C), cKH = KH, cKW = KW;
-  int sh = static_cast<int>(param.stride[0]), sw = static_cast<int>(param.stride[1]);
-  int ph = static_cast<int>(param.pad[0]), pw = static_cast<int>(param.pad[1]);
-  const ConvS2D s2d = ConvSpaceToDepth(param, d, w, o);
-  int8_t* w_ohwi;
-  if (s2d.use) {
-    cC = ConvPaddedChannels(4 * C);
-    cH = s2d.H2; cW = s2d.W2; cKH = s2d.K2h; cKW = s2d.K2w;
-    sh = sw = 1;
-    ph = s2d.pad_h; pw = s2d.pad_w;
-    w_ohwi = reinterpret_cast<int8_t*>(ws + up(static_cast<size_t>(N) * cH * cW * cC));
+  int8_t* w_ohwi = reinterpret_cast<int8_t*>(ws + v.d_bytes);
+  void* split_ws = split_bytes != 0 ? ws + v.d_bytes + v.w_bytes : nullptr;
+  if (v.s2d.use) {
     MXQ_CALL(mxq_nchw_to_s2d_nhwc_i8(stream, inputs[0].dptr<int8_t>(), d_nhwc, N, C, H, W,
-                                     s2d.off_h, s2d.off_w, cC));
+                                     v.s2d.off_h, v.s2d.off_w, v.C));
     MXQ_CALL(mxq_nchw_to_s2d_nhwc_i8(stream, inputs[1].dptr<int8_t>(), w_ohwi, O, C, KH, KW, 0, 0,
-                                     cC));
+                                     v.C));
   } else {
-    w_ohwi = reinterpret_cast<int8_t*>(ws + up(static_cast<size_t>(N) * H * W * cC));
-    MXQ_CALL(mxq_nchw_to_nhwc_pad_i8(stream, inputs[0].dptr<int8_t>(), d_nhwc, N, C, H, W, cC));
-    MXQ_CALL(mxq_nchw_to_nhwc_pad_i8(stream, inputs[1].dptr<int8_t>(), w_ohwi, O, C, KH, KW, cC));
+    MXQ_CALL(mxq_nchw_to_nhwc_pad_i8(stream, inputs[0].dptr<int8_t>(), d_nhwc, N, C, H, W, v.C));
+    MXQ_CALL(mxq_nchw_to_nhwc_pad_i8(stream, inputs[1].dptr<int8_t>(), w_ohwi, O, C, KH, KW, v.C));
   }
   const size_t ni = param.no_bias ? 2 : 3;
   MXQ_CALL(mxq_quantized_conv_nhwc_out_nchw(
-      stream, d_nhwc, w_ohwi, param.no_bias ? nullptr : inputs[2].dptr<int8_t>(), N, cH, cW, cC,
-      O, cKH, cKW, sh, sw, ph, pw, static_cast<int>(param.dilate[0]),
+      stream, d_nhwc, w_ohwi, param.no_bias ? nullptr : inputs[2].dptr<int8_t>(), N, v.H, v.W,
+      v.C, O, v.KH, v.KW, v.sh, v.sw, v.ph, v.pw, static_cast<int>(param.dilate[0]),
       static_cast<int>(param.dilate[1]),
       inputs[ni].dptr<float>(), inputs[ni + 1].dptr<float>(), inputs[ni + 2].dptr<float>(),
       inputs[ni + 3].dptr<float>(), param.no_bias ? nullptr : inputs[7].dptr<float>(),
       param.no_bias ? nullptr : inputs[8].dptr<float>(), outputs[0].dptr<int32_t>(),
-      outputs[1].dptr<float>(), outputs[2].dptr<float>()));
+      outputs[1].dptr<float>(), outputs[2].dptr<float>(), split_ws, split_bytes));
 }
 
 // _contrib_quantized_act: int8 relu, ranges pass through (dnnl_quantized_act.cc:33-45)
@@ -930,6 +957,22 @@ size_t MXQTempSpaceBytes(const NodeAttrs& attrs, const ShapeVector& in, const Sh
   if (name == "_contrib_requantize") return mxq_requantize_workspace(in[0].Size());
   if (name == "_contrib_quantized_conv")
     return QuantizedConvTempBytes(nnvm::get<ConvolutionParam>(attrs.parsed), in[0], in[1], out[0]);
+  if (name == "_contrib_quantized_fully_connected") {
+    // rows x reduction as QuantizedFullyConnectedForwardGPU reads them off the shapes
+    const auto& param = nnvm::get<FullyConnectedParam>(attrs.parsed);
+    const TShape& d = in[0];
+    if (d.ndim() < 1 || in[1].ndim() != 2) return 0;
+    index_t m, k;
+    if (param.flatten || d.ndim() == 2) {
+      m = d[0];
+      k = d.ProdShape(1, d.ndim());
+    } else {
+      k = d[d.ndim() - 1];
+      m = d.ProdShape(0, d.ndim() - 1);
+    }
+    return mxq_quantized_fc_workspace(static_cast<int>(m), static_cast<int>(in[1][0]),
+                                      static_cast<int>(k), 0);
+  }
   return 0;
 }
 

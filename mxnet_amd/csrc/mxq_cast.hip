@@ -30,8 +30,6 @@
 
 namespace mxq {
 
-int g_cast_blocks_per_cu = 2;  // tunable through mxq_set_tuning("cast_blocks_per_cu", v)
-
 namespace {
 
 typedef float f4 __attribute__((ext_vector_type(4)));
@@ -656,15 +654,8 @@ __global__ void passthrough_range_kernel(float* omin, float* omax, float lo, flo
 }
 
 int stream_grid(size_t work_items) {
-  int dev = 0;
-  MXQ_HIP(hipGetDevice(&dev));
-  static thread_local int cached_dev = -1, cached_cus = 0;
-  if (cached_dev != dev) {
-    MXQ_HIP(hipDeviceGetAttribute(&cached_cus, hipDeviceAttributeMultiprocessorCount, dev));
-    cached_dev = dev;
-  }
   size_t want = (work_items + kThreads - 1) / kThreads;
-  size_t cap = size_t(cached_cus) * size_t(g_cast_blocks_per_cu);
+  size_t cap = size_t(num_cus()) * size_t(kCastBlocksPerCu);
   if (want < 1) want = 1;
   return static_cast<int>(want < cap ? want : cap);
 }

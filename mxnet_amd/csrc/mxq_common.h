@@ -54,6 +54,14 @@ struct Error : public std::runtime_error {
   }                                          \
   return 0;
 
+// Compute units of the calling thread's current device (cached per thread and device).
+int num_cus();
+
+// Work-groups of 256 threads per CU the streaming kernels are launched with at most:
+// more resident waves lower the HBM bandwidth they reach (8 waves per CU: 6.0 TB/s,
+// 16: 5.5, 32 and more: 5.4 on a 256 MB cast).
+constexpr int kCastBlocksPerCu = 2;
+
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 }  // namespace mxq

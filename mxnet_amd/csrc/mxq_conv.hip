@@ -16,15 +16,14 @@
 
 #include "../../include/mxq.h"
 #include "mxq_common.h"
-#include "mxq_gemm.cuh"
+#include "mxq_gemm.h"
 #include "mxq_tiles.h"
 
 namespace mxq {
 
-int g_conv_config = 0;  // 0 = choose by shape
-
 void launch_fc(hipStream_t s, const int8_t* data, const int8_t* weight, int M, int N, int K,
-               int ldo, const Epilogue& epi);
+               int ldo, const Epilogue& epi, const GemmForce& force, const Workspace& ws);
+size_t fc_workspace_bytes(int M, int N, int K, bool fused8);
 
 namespace {
 
@@ -35,6 +34,7 @@ struct ConvArgs {
   int sh, sw, ph, pw, dh, dw, OH, OW;
   int M, K;  // N*OH*OW, KH*KW*C
   Epilogue epi;
+  SplitK sk;
 };
 
 // Activation loader: row = output pixel, chunk = 16 channels of one filter tap.
@@ -150,13 +150,16 @@ struct ConvIssuer {
   int C, H, W, KH, KW, dh, dw;
   v4i rsrc;
 
-  __device__ __forceinline__ void init(const ConvArgs& a, int row_begin, int wave, int lane) {
+  // kbeg: reduction index (a multiple of the stage depth) at which stage 0 starts
+  __device__ __forceinline__ void init(const ConvArgs& a, int row_begin, int wave, int lane,
+                                       int kbeg = 0) {
     C = a.C; H = a.H; W = a.W; KH = a.KH; KW = a.KW; dh = a.dh; dw = a.dw;
     rsrc = make_rsrc(a.data, static_cast<uint32_t>(a.N) * a.H * a.W * a.C);
     DmaLane<Cfg> g;
     g.init(wave, lane);
-    const int tap = g.c16 / C;
-    cc = g.c16 - tap * C;
+    const int k = kbeg + g.c16;
+    const int tap = k / C;
+    cc = k - tap * C;
     kh = tap / KW;
     kw = tap - kh * KW;
     retap();
@@ -204,8 +207,11 @@ template <class Cfg, int NS, int PIPE>
 __global__ __launch_bounds__(Cfg::kThreads, NS <= 2 ? Cfg::kMinWaves : 1) void conv_dma_kernel(ConvArgs p) {
   __shared__ __attribute__((aligned(16))) v4i lds[NS * Cfg::STAGE_SLOTS];
   const int tiles_m = (p.M + Cfg::BM - 1) / Cfg::BM, tiles_n = (p.O + Cfg::BN - 1) / Cfg::BN;
-  int tm, tn;
-  tile_coords(blockIdx.x, tiles_m, tiles_n, tm, tn);
+  int tm, tn, tile = 0, z = 0;
+  if (p.sk.splits > 1)
+    tile_coords_split(blockIdx.x, tiles_m, tiles_n, p.sk.splits, tm, tn, tile, z);
+  else
+    tile_coords(blockIdx.x, tiles_m, tiles_n, tm, tn);
   const int m0 = tm * Cfg::BM, n0 = tn * Cfg::BN;
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -213,18 +219,24 @@ __global__ __launch_bounds__(Cfg::kThreads, NS <= 2 ? Cfg::kMinWaves : 1) void c
   // what the epilogue needs is fetched while the first operand stages are in flight
   EpiPre pre;
   auto prefetch = [&]() { pre = epi_prefetch<Cfg>(p.epi, n0, p.O); };
+  // this work-group's K slice: stages [kt0, kt0 + KT) (all of them without a split)
+  const int kt_all = (p.K + Cfg::BK - 1) / Cfg::BK;
+  const int kt0 = z * p.sk.kt_per_split;
+  const int KT = (kt_all - kt0) < p.sk.kt_per_split ? (kt_all - kt0) : p.sk.kt_per_split;
+  const int kbeg = kt0 * Cfg::BK;
   ConvIssuer<Cfg, Cfg::A_CHUNKS> ai;
   RowIssuerBuffer<Cfg, Cfg::B_CHUNKS> bi;
-  ai.init(p, m0, wave, lane);
-  bi.init(p.weight, n0, p.O, p.K, wave, lane);
+  ai.init(p, m0, wave, lane, kbeg);
+  bi.init(p.weight, n0, p.O, p.K, wave, lane, kbeg);
 
   v16i acc[Cfg::MI][Cfg::NI];
-  gemm_mainloop_dma<Cfg, NS, PIPE>(acc, ai, bi, (p.K + Cfg::BK - 1) / Cfg::BK, lds, prefetch);
+  gemm_mainloop_dma<Cfg, NS, PIPE>(acc, ai, bi, KT, lds, prefetch);
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  if (blockIdx.x == 0 && threadIdx.x == 0) epilogue_ranges(p.epi);
+  if (p.sk.splits > 1 && !splitk_gather<Cfg>(acc, p.sk, tile, z)) return;
 
   gemm_epilogue_lds<Cfg, NS * Cfg::STAGE_SLOTS * 16>(acc, p.epi, pre, m0, n0, p.M, p.O,
                                                      static_cast<size_t>(p.O), lds);
-  if (blockIdx.x == 0 && threadIdx.x == 0) epilogue_ranges(p.epi);
 }
 
 typedef GemmCfg<256, 256, 64, 2, 4> CfgL8;   // 8 waves, wave tile 128 x 64
@@ -243,9 +255,13 @@ typedef GemmCfg<64, 128, 128, 2, 2> CfgQK;
 typedef GemmCfg<64, 64, 256, 2, 2> CfgSK2;
 
 template <class Cfg, int NS, int PIPE>
-void launch_dma(hipStream_t s, const ConvArgs& a) {
-  const int tiles = ((a.M + Cfg::BM - 1) / Cfg::BM) * ((a.O + Cfg::BN - 1) / Cfg::BN);
-  hipLaunchKernelGGL((conv_dma_kernel<Cfg, NS, PIPE>), dim3(tiles), dim3(Cfg::kThreads), 0, s, a);
+void launch_dma(hipStream_t s, ConvArgs a, int splits, const Workspace& ws) {
+  const long tiles =
+      static_cast<long>((a.M + Cfg::BM - 1) / Cfg::BM) * ((a.O + Cfg::BN - 1) / Cfg::BN);
+  splitk_setup<Cfg>(s, a.sk, tiles, a.K, splits, ws.ptr, ws.bytes);
+  hipLaunchKernelGGL((conv_dma_kernel<Cfg, NS, PIPE>),
+                     dim3(static_cast<unsigned>(tiles * a.sk.splits)), dim3(Cfg::kThreads), 0, s,
+                     a);
   MXQ_LAUNCH_CHECK();
 }
 
@@ -257,17 +273,6 @@ void launch_cfg(hipStream_t s, const ConvArgs& a, bool aligned) {
   else
     hipLaunchKernelGGL((conv_kernel<Cfg, false>), dim3(tiles), dim3(Cfg::kThreads), 0, s, a);
   MXQ_LAUNCH_CHECK();
-}
-
-int num_cus() {
-  int dev = 0;
-  MXQ_HIP(hipGetDevice(&dev));
-  static thread_local int cached_dev = -1, cached_cus = 0;
-  if (cached_dev != dev) {
-    MXQ_HIP(hipDeviceGetAttribute(&cached_cus, hipDeviceAttributeMultiprocessorCount, dev));
-    cached_dev = dev;
-  }
-  return cached_cus;
 }
 
 // ---- layout adapters ------------------------------------------------------------
@@ -396,6 +401,104 @@ void launch_transpose(hipStream_t s, const void* in, void* out, int B, int R, in
   MXQ_LAUNCH_CHECK();
 }
 
+// Output tile of a direct-to-LDS configuration of this file (what a split-K work-group
+// leaves in the workspace); false for the register-staged ones.
+bool conv_cfg_tile(int cfg, int& bm, int& bn) {
+  switch (cfg) {
+    case 11: case 16: case 35: bm = 256; bn = 256; return true;
+    case 12: case 22: case 36: bm = 256; bn = 128; return true;
+    case 13: case 23: bm = 256; bn = 64; return true;
+    case 14: case 24: case 33: case 34: bm = 128; bn = 128; return true;
+    case 15: case 25: case 31: case 32: case 39: bm = 64; bn = 64; return true;
+    case 37: bm = 128; bn = 64; return true;
+    case 38: bm = 64; bn = 128; return true;
+    default: return false;
+  }
+}
+
+struct ConvGeometry {
+  int N, H, W, C, O, KH, KW, sh, sw, ph, pw, dh, dw;
+  int OH, OW;
+  long long M, K;
+  bool is_fc;  // 1x1, unit stride, no padding: the FC of the flattened pixels
+};
+
+ConvGeometry conv_geometry(int N, int H, int W, int C, int O, int KH, int KW, int stride_h,
+                           int stride_w, int pad_h, int pad_w, int dilate_h, int dilate_w) {
+  MXQ_CHECK(N >= 0 && H > 0 && W > 0 && C > 0 && O > 0 && KH > 0 && KW > 0, "bad shape");
+  MXQ_CHECK(stride_h > 0 && stride_w > 0 && dilate_h > 0 && dilate_w > 0 && pad_h >= 0 &&
+                pad_w >= 0,
+            "bad stride/dilate/pad");
+  const int eh = dilate_h * (KH - 1) + 1, ew = dilate_w * (KW - 1) + 1;
+  MXQ_CHECK(H + 2 * pad_h >= eh && W + 2 * pad_w >= ew, "kernel larger than padded input");
+  ConvGeometry g = {N, H, W, C, O, KH, KW, stride_h, stride_w, pad_h, pad_w, dilate_h, dilate_w,
+                    0, 0, 0, 0, false};
+  g.OH = (H + 2 * pad_h - eh) / stride_h + 1;
+  g.OW = (W + 2 * pad_w - ew) / stride_w + 1;
+  g.M = static_cast<long long>(N) * g.OH * g.OW;
+  g.K = static_cast<long long>(KH) * KW * C;
+  MXQ_CHECK(g.M < (1LL << 31) && g.K < (1LL << 31), "problem too large for 32-bit tile indices");
+  g.is_fc = KH == 1 && KW == 1 && stride_h == 1 && stride_w == 1 && pad_h == 0 && pad_w == 0;
+  return g;
+}
+
+struct ConvPlan {
+  int cfg;
+  int splits;
+};
+
+// What conv_nhwc would launch for a convolution that does not reduce to the FC.  `aligned`:
+// C % 16 == 0 and 16-byte aligned operands.
+ConvPlan plan_conv(const ConvGeometry& g, bool aligned, const GemmForce& force) {
+  ConvPlan plan = {force.cfg, force.splits};
+  const int M = static_cast<int>(g.M), K = static_cast<int>(g.K), O = g.O;
+  const long long data_bytes = static_cast<long long>(g.N) * g.H * g.W * g.C;
+  const bool dma_ok = aligned && data_bytes < (1LL << 31) &&
+                      static_cast<long long>(O) * K < (1LL << 31);
+  if (plan.cfg == 0) {
+    const long cus = num_cus();
+    auto tiles = [&](int bm, int bn) {
+      return static_cast<long>((M + bm - 1) / bm) * ((O + bn - 1) / bn);
+    };
+    int auto_splits = 1;
+    if (dma_ok) {
+      switch (choose_tile(M, O, K, cus, true, &auto_splits)) {
+        case Tile::kL8: plan.cfg = 11; break;
+        case Tile::kW128x2: plan.cfg = 22; break;
+        case Tile::kW128K2: plan.cfg = 36; break;
+        case Tile::kM128x2: plan.cfg = 24; break;
+        case Tile::kM128K2: plan.cfg = 33; break;
+        case Tile::kS64x2: plan.cfg = 25; break;
+        case Tile::kS64x4: plan.cfg = 15; break;
+        case Tile::kS64K2: plan.cfg = 31; break;
+        case Tile::kR128K2: plan.cfg = 37; break;
+        case Tile::kQ128K2: plan.cfg = 38; break;
+        case Tile::kS64K4: plan.cfg = 39; break;
+      }
+    } else if (O > 128 && tiles(256, 256) >= cus) {
+      plan.cfg = 1;
+    } else if (O > 64 && tiles(256, 128) >= cus) {
+      plan.cfg = 2;
+    } else if (O <= 64 && tiles(256, 64) >= cus) {
+      plan.cfg = 3;
+    } else if (tiles(128, 128) >= cus) {
+      plan.cfg = 4;
+    } else {
+      plan.cfg = 5;
+    }
+    if (plan.splits == 0) plan.splits = auto_splits;
+  }
+  if (plan.splits <= 0) plan.splits = 1;
+  return plan;
+}
+
+size_t conv_plan_workspace(const ConvPlan& plan, const ConvGeometry& g) {
+  int bm, bn;
+  if (plan.splits <= 1 || !conv_cfg_tile(plan.cfg, bm, bn)) return 0;
+  const long tiles = static_cast<long>((g.M + bm - 1) / bm) * ((g.O + bn - 1) / bn);
+  return splitk_workspace_bytes(tiles, plan.splits, bm, bn);
+}
+
 // Both C entry points: `planar` writes out32 as [N][O][OH][OW] instead of [N][OH][OW][O].
 void conv_nhwc(void* stream, const int8_t* data, const int8_t* weight, const int8_t* bias, int N,
                int H, int W, int C, int O, int KH, int KW, int stride_h, int stride_w, int pad_h,
@@ -403,30 +506,27 @@ void conv_nhwc(void* stream, const int8_t* data, const int8_t* weight, const int
                const float* max_data, const float* min_weight, const float* max_weight,
                const float* min_bias, const float* max_bias, int32_t* out32, float* omin,
                float* omax, int8_t* out8, float* rmin, float* rmax, int relu, float min_calib,
-               float max_calib, bool planar) {
-  MXQ_CHECK(N >= 0 && H > 0 && W > 0 && C > 0 && O > 0 && KH > 0 && KW > 0, "bad shape");
-  MXQ_CHECK(stride_h > 0 && stride_w > 0 && dilate_h > 0 && dilate_w > 0 && pad_h >= 0 &&
-                pad_w >= 0,
-            "bad stride/dilate/pad");
+               float max_calib, bool planar, const GemmForce& force, const Workspace& ws) {
+  const ConvGeometry g = conv_geometry(N, H, W, C, O, KH, KW, stride_h, stride_w, pad_h, pad_w,
+                                       dilate_h, dilate_w);
   MXQ_CHECK(min_data && max_data && min_weight && max_weight, "null input range pointer");
   MXQ_CHECK(omin && omax, "null output range pointer");
   MXQ_CHECK(bias == nullptr || (min_bias && max_bias), "bias given without its range");
   MXQ_CHECK(N == 0 || out32 != nullptr || out8 != nullptr, "no output buffer");
   MXQ_CHECK(out8 == nullptr || (rmin && rmax), "fused requantize needs rmin/rmax");
-  const int eh = dilate_h * (KH - 1) + 1, ew = dilate_w * (KW - 1) + 1;
-  MXQ_CHECK(H + 2 * pad_h >= eh && W + 2 * pad_w >= ew, "kernel larger than padded input");
   ConvArgs a;
   a.data = data;
   a.weight = weight;
   a.N = N; a.H = H; a.W = W; a.C = C; a.O = O; a.KH = KH; a.KW = KW;
   a.sh = stride_h; a.sw = stride_w; a.ph = pad_h; a.pw = pad_w; a.dh = dilate_h; a.dw = dilate_w;
-  a.OH = (H + 2 * pad_h - eh) / stride_h + 1;
-  a.OW = (W + 2 * pad_w - ew) / stride_w + 1;
-  const long long M = static_cast<long long>(N) * a.OH * a.OW;
-  const long long K = static_cast<long long>(KH) * KW * C;
-  MXQ_CHECK(M < (1LL << 31) && K < (1LL << 31), "problem too large for 32-bit tile indices");
-  a.M = static_cast<int>(M);
-  a.K = static_cast<int>(K);
+  a.OH = g.OH;
+  a.OW = g.OW;
+  a.M = static_cast<int>(g.M);
+  a.K = static_cast<int>(g.K);
+  a.sk.splits = 1;
+  a.sk.kt_per_split = 1 << 30;
+  a.sk.counters = nullptr;
+  a.sk.partials = nullptr;
   MXQ_CHECK(a.M == 0 || O == 0 || (data != nullptr && weight != nullptr),
             "null operand pointer");
   Epilogue& e = a.epi;
@@ -444,77 +544,54 @@ void conv_nhwc(void* stream, const int8_t* data, const int8_t* weight, const int
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (a.M == 0 || O == 0) {
     // no output elements: launch_fc writes the range scalars alone
-    launch_fc(s, data, weight, a.M, O, C, O, e);
+    launch_fc(s, data, weight, a.M, O, C, O, e, GemmForce(), Workspace());
+    return;
+  }
+  // a 1x1, unit-stride, unpadded convolution is the FC of the flattened pixels
+  if (force.cfg == 0 && g.is_fc) {
+    launch_fc(s, data, weight, a.M, O, C, O, e, force, ws);
     return;
   }
   const bool aligned = (C % 16 == 0) && aligned16(data) && aligned16(weight);
   const long long data_bytes = static_cast<long long>(N) * H * W * C;
   const bool dma_ok = aligned && data_bytes < (1LL << 31) &&
                       static_cast<long long>(O) * a.K < (1LL << 31);
-  int cfg = g_conv_config;
-  // a 1x1, unit-stride, unpadded convolution is the FC of the flattened pixels
-  if (cfg == 0 && KH == 1 && KW == 1 && stride_h == 1 && stride_w == 1 && pad_h == 0 &&
-      pad_w == 0) {
-    launch_fc(s, data, weight, a.M, O, C, O, e);
-    return;
+  ConvPlan plan = plan_conv(g, aligned, force);
+  // a split the chooser proposed is dropped when the caller brought no room for it
+  if (force.splits == 0 && plan.splits > 1 &&
+      (ws.ptr == nullptr || !aligned16(ws.ptr) || ws.bytes < conv_plan_workspace(plan, g))) {
+    GemmForce unsplit = force;
+    unsplit.splits = 1;
+    plan = plan_conv(g, aligned, unsplit);
   }
-  if (cfg == 0) {
-    const long cus = num_cus();
-    auto tiles = [&](int bm, int bn) {
-      return static_cast<long>((a.M + bm - 1) / bm) * ((O + bn - 1) / bn);
-    };
-    if (dma_ok) {
-      switch (choose_tile(a.M, O, a.K, cus, true)) {
-        case Tile::kL8: cfg = 11; break;
-        case Tile::kW128x2: cfg = 22; break;
-        case Tile::kW128K2: cfg = 36; break;
-        case Tile::kM128x2: cfg = 24; break;
-        case Tile::kM128K2: cfg = 33; break;
-        case Tile::kS64x2: cfg = 25; break;
-        case Tile::kS64x4: cfg = 15; break;
-        case Tile::kS64K2: cfg = 31; break;
-        case Tile::kR128K2: cfg = 37; break;
-        case Tile::kQ128K2: cfg = 38; break;
-        case Tile::kS64K4: cfg = 39; break;
-      }
-    } else if (O > 128 && tiles(256, 256) >= cus) {
-      cfg = 1;
-    } else if (O > 64 && tiles(256, 128) >= cus) {
-      cfg = 2;
-    } else if (O <= 64 && tiles(256, 64) >= cus) {
-      cfg = 3;
-    } else if (tiles(128, 128) >= cus) {
-      cfg = 4;
-    } else {
-      cfg = 5;
-    }
-  }
+  const int cfg = plan.cfg, sp = plan.splits;
   if (cfg > 10) MXQ_CHECK(dma_ok, "shape does not qualify for the direct-to-LDS conv kernels");
+  if (cfg <= 10) MXQ_CHECK(sp <= 1, "the register-staged kernels have no split-K form");
   switch (cfg) {
     case 1: launch_cfg<CfgL8>(s, a, aligned); break;
     case 2: launch_cfg<CfgW128>(s, a, aligned); break;
     case 3: launch_cfg<CfgW64>(s, a, aligned); break;
     case 4: launch_cfg<CfgM>(s, a, aligned); break;
     case 5: launch_cfg<CfgS>(s, a, aligned); break;
-    case 11: launch_dma<CfgL8, 4, 2>(s, a); break;
-    case 12: launch_dma<CfgW128, 4, 2>(s, a); break;
-    case 13: launch_dma<CfgW64, 4, 2>(s, a); break;
-    case 14: launch_dma<CfgM, 4, 2>(s, a); break;
-    case 15: launch_dma<CfgS, 4, 2>(s, a); break;
-    case 16: launch_dma<CfgL4, 4, 2>(s, a); break;
-    case 31: launch_dma<CfgSK, 2, 0>(s, a); break;
-    case 32: launch_dma<CfgSK, 3, 0>(s, a); break;
-    case 33: launch_dma<CfgMK, 2, 0>(s, a); break;
-    case 34: launch_dma<CfgMK, 3, 0>(s, a); break;
-    case 35: launch_dma<CfgL8K, 2, 0>(s, a); break;
-    case 36: launch_dma<CfgW128K, 2, 0>(s, a); break;
-    case 37: launch_dma<CfgRK, 2, 0>(s, a); break;
-    case 38: launch_dma<CfgQK, 2, 0>(s, a); break;
-    case 39: launch_dma<CfgSK2, 2, 0>(s, a); break;
-    case 22: launch_dma<CfgW128, 2, 0>(s, a); break;
-    case 23: launch_dma<CfgW64, 2, 0>(s, a); break;
-    case 24: launch_dma<CfgM, 2, 0>(s, a); break;
-    case 25: launch_dma<CfgS, 2, 0>(s, a); break;
+    case 11: launch_dma<CfgL8, 4, 2>(s, a, sp, ws); break;
+    case 12: launch_dma<CfgW128, 4, 2>(s, a, sp, ws); break;
+    case 13: launch_dma<CfgW64, 4, 2>(s, a, sp, ws); break;
+    case 14: launch_dma<CfgM, 4, 2>(s, a, sp, ws); break;
+    case 15: launch_dma<CfgS, 4, 2>(s, a, sp, ws); break;
+    case 16: launch_dma<CfgL4, 4, 2>(s, a, sp, ws); break;
+    case 31: launch_dma<CfgSK, 2, 0>(s, a, sp, ws); break;
+    case 32: launch_dma<CfgSK, 3, 0>(s, a, sp, ws); break;
+    case 33: launch_dma<CfgMK, 2, 0>(s, a, sp, ws); break;
+    case 34: launch_dma<CfgMK, 3, 0>(s, a, sp, ws); break;
+    case 35: launch_dma<CfgL8K, 2, 0>(s, a, sp, ws); break;
+    case 36: launch_dma<CfgW128K, 2, 0>(s, a, sp, ws); break;
+    case 37: launch_dma<CfgRK, 2, 0>(s, a, sp, ws); break;
+    case 38: launch_dma<CfgQK, 2, 0>(s, a, sp, ws); break;
+    case 39: launch_dma<CfgSK2, 2, 0>(s, a, sp, ws); break;
+    case 22: launch_dma<CfgW128, 2, 0>(s, a, sp, ws); break;
+    case 23: launch_dma<CfgW64, 2, 0>(s, a, sp, ws); break;
+    case 24: launch_dma<CfgM, 2, 0>(s, a, sp, ws); break;
+    case 25: launch_dma<CfgS, 2, 0>(s, a, sp, ws); break;
     default: MXQ_CHECK(false, "unknown conv tile configuration " << cfg);
   }
 }
@@ -526,6 +603,21 @@ using namespace mxq;
 
 extern "C" {
 
+size_t mxq_quantized_conv_workspace(int N, int H, int W, int C, int O, int KH, int KW,
+                                    int stride_h, int stride_w, int pad_h, int pad_w,
+                                    int dilate_h, int dilate_w, int fused_int8_only) {
+  try {
+    const ConvGeometry g = conv_geometry(N, H, W, C, O, KH, KW, stride_h, stride_w, pad_h, pad_w,
+                                         dilate_h, dilate_w);
+    if (g.M == 0) return 0;
+    if (g.is_fc)
+      return fc_workspace_bytes(static_cast<int>(g.M), O, C, fused_int8_only != 0 && O % 16 == 0);
+    return conv_plan_workspace(plan_conv(g, C % 16 == 0, GemmForce()), g);
+  } catch (...) {
+    return 0;
+  }
+}
+
 int mxq_quantized_conv_nhwc(void* stream, const int8_t* data, const int8_t* weight,
                             const int8_t* bias, int N, int H, int W, int C, int O, int KH,
                             int KW, int stride_h, int stride_w, int pad_h, int pad_w,
@@ -534,11 +626,40 @@ int mxq_quantized_conv_nhwc(void* stream, const int8_t* data, const int8_t* weig
                             const float* max_weight, const float* min_bias,
                             const float* max_bias, int32_t* out32, float* omin, float* omax,
                             int8_t* out8, float* rmin, float* rmax, int relu, float min_calib,
-                            float max_calib) {
+                            float max_calib, void* workspace, size_t workspace_bytes) {
   MXQ_API_BEGIN();
+  Workspace ws;
+  ws.ptr = workspace;
+  ws.bytes = workspace_bytes;
   conv_nhwc(stream, data, weight, bias, N, H, W, C, O, KH, KW, stride_h, stride_w, pad_h, pad_w,
             dilate_h, dilate_w, min_data, max_data, min_weight, max_weight, min_bias, max_bias,
-            out32, omin, omax, out8, rmin, rmax, relu, min_calib, max_calib, false);
+            out32, omin, omax, out8, rmin, rmax, relu, min_calib, max_calib, false, GemmForce(),
+            ws);
+  MXQ_API_END();
+}
+
+// Test-only twin of mxq_quantized_conv_nhwc (declared in tests/mxq_test_hooks.h): the tile
+// configuration and the split-K factor come as arguments (0 = let the launcher choose).
+int mxq_test_quantized_conv_nhwc(void* stream, const int8_t* data, const int8_t* weight,
+                                 const int8_t* bias, int N, int H, int W, int C, int O, int KH,
+                                 int KW, int stride_h, int stride_w, int pad_h, int pad_w,
+                                 int dilate_h, int dilate_w, const float* min_data,
+                                 const float* max_data, const float* min_weight,
+                                 const float* max_weight, const float* min_bias,
+                                 const float* max_bias, int32_t* out32, float* omin,
+                                 float* omax, int8_t* out8, float* rmin, float* rmax, int relu,
+                                 float min_calib, float max_calib, void* workspace,
+                                 size_t workspace_bytes, int cfg, int splits) {
+  MXQ_API_BEGIN();
+  Workspace ws;
+  ws.ptr = workspace;
+  ws.bytes = workspace_bytes;
+  GemmForce force;
+  force.cfg = cfg;
+  force.splits = splits;
+  conv_nhwc(stream, data, weight, bias, N, H, W, C, O, KH, KW, stride_h, stride_w, pad_h, pad_w,
+            dilate_h, dilate_w, min_data, max_data, min_weight, max_weight, min_bias, max_bias,
+            out32, omin, omax, out8, rmin, rmax, relu, min_calib, max_calib, false, force, ws);
   MXQ_API_END();
 }
 
@@ -549,12 +670,16 @@ int mxq_quantized_conv_nhwc_out_nchw(void* stream, const int8_t* data, const int
                                      const float* min_data, const float* max_data,
                                      const float* min_weight, const float* max_weight,
                                      const float* min_bias, const float* max_bias,
-                                     int32_t* out32_nchw, float* omin, float* omax) {
+                                     int32_t* out32_nchw, float* omin, float* omax,
+                                     void* workspace, size_t workspace_bytes) {
   MXQ_API_BEGIN();
   MXQ_CHECK(out32_nchw != nullptr, "no output buffer");
+  Workspace ws;
+  ws.ptr = workspace;
+  ws.bytes = workspace_bytes;
   conv_nhwc(stream, data, weight, bias, N, H, W, C, O, KH, KW, stride_h, stride_w, pad_h, pad_w,
             dilate_h, dilate_w, min_data, max_data, min_weight, max_weight, min_bias, max_bias,
-            out32_nchw, omin, omax, nullptr, nullptr, nullptr, 0, 0.f, 0.f, true);
+            out32_nchw, omin, omax, nullptr, nullptr, nullptr, 0, 0.f, 0.f, true, GemmForce(), ws);
   MXQ_API_END();
 }
 

@@ -24,7 +24,6 @@
 
 namespace mxq {
 
-extern int g_cast_blocks_per_cu;  // mxq_cast.hip: work-groups per CU of the streaming kernels
 
 namespace {
 
@@ -945,15 +944,8 @@ __global__ __launch_bounds__(kThreads) void bn_rows_kernel(BnArgs a) {
 }
 
 int grid_for(size_t work_items) {
-  int dev = 0;
-  MXQ_HIP(hipGetDevice(&dev));
-  static thread_local int cached_dev = -1, cached_cus = 0;
-  if (cached_dev != dev) {
-    MXQ_HIP(hipDeviceGetAttribute(&cached_cus, hipDeviceAttributeMultiprocessorCount, dev));
-    cached_dev = dev;
-  }
   size_t want = (work_items + kThreads - 1) / kThreads;
-  const size_t cap = size_t(cached_cus) * size_t(g_cast_blocks_per_cu);
+  const size_t cap = size_t(num_cus()) * size_t(kCastBlocksPerCu);
   if (want < 1) want = 1;
   return static_cast<int>(want < cap ? want : cap);
 }

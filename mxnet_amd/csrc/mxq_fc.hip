@@ -11,13 +11,10 @@
 
 #include "../../include/mxq.h"
 #include "mxq_common.h"
-#include "mxq_gemm.cuh"
+#include "mxq_gemm.h"
 #include "mxq_tiles.h"
 
 namespace mxq {
-
-int g_fc_config = 0;  // 0 = choose by shape; 1.. force a tile configuration (tuning/tests)
-int g_fc_stream_groups = 2;  // work-groups per CU of the short-K streaming kernel when forced
 
 namespace {
 
@@ -27,6 +24,7 @@ struct FcArgs {
   int M, N, K;
   int ldo;               // output row pitch in elements (N for the FC)
   Epilogue epi;
+  SplitK sk;
 };
 
 template <class Cfg, bool ALIGNED>
@@ -59,8 +57,11 @@ template <class Cfg, int NS, int PIPE, bool BUF>
 __global__ __launch_bounds__(Cfg::kThreads, NS <= 2 ? Cfg::kMinWaves : 1) void fc_dma_kernel(FcArgs p) {
   __shared__ __attribute__((aligned(16))) v4i lds[NS * Cfg::STAGE_SLOTS];
   const int tiles_m = (p.M + Cfg::BM - 1) / Cfg::BM, tiles_n = (p.N + Cfg::BN - 1) / Cfg::BN;
-  int tm, tn;
-  tile_coords(blockIdx.x, tiles_m, tiles_n, tm, tn);
+  int tm, tn, tile = 0, z = 0;
+  if (p.sk.splits > 1)
+    tile_coords_split(blockIdx.x, tiles_m, tiles_n, p.sk.splits, tm, tn, tile, z);
+  else
+    tile_coords(blockIdx.x, tiles_m, tiles_n, tm, tn);
   const int m0 = tm * Cfg::BM, n0 = tn * Cfg::BN;
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -69,25 +70,30 @@ __global__ __launch_bounds__(Cfg::kThreads, NS <= 2 ? Cfg::kMinWaves : 1) void f
   EpiPre pre;
   auto prefetch = [&]() { pre = epi_prefetch<Cfg>(p.epi, n0, p.N); };
   v16i acc[Cfg::MI][Cfg::NI];
-  const int KT = (p.K + Cfg::BK - 1) / Cfg::BK;
+  // this work-group's K slice: stages [kt0, kt0 + KT) (all of them without a split)
+  const int kt_all = (p.K + Cfg::BK - 1) / Cfg::BK;
+  const int kt0 = z * p.sk.kt_per_split;
+  const int KT = (kt_all - kt0) < p.sk.kt_per_split ? (kt_all - kt0) : p.sk.kt_per_split;
+  const int kbeg = kt0 * Cfg::BK;
   if (BUF) {
     RowIssuerBuffer<Cfg, Cfg::A_CHUNKS> ai;
     RowIssuerBuffer<Cfg, Cfg::B_CHUNKS> bi;
-    ai.init(p.data, m0, p.M, p.K, wave, lane);
-    bi.init(p.weight, n0, p.N, p.K, wave, lane);
+    ai.init(p.data, m0, p.M, p.K, wave, lane, kbeg);
+    bi.init(p.weight, n0, p.N, p.K, wave, lane, kbeg);
     gemm_mainloop_dma<Cfg, NS, PIPE>(acc, ai, bi, KT, lds, prefetch);
   } else {
     RowIssuerGlobal<Cfg, Cfg::A_CHUNKS> ai;
     RowIssuerGlobal<Cfg, Cfg::B_CHUNKS> bi;
-    ai.init(p.data, m0, p.M, p.K, wave, lane);
-    bi.init(p.weight, n0, p.N, p.K, wave, lane);
+    ai.init(p.data, m0, p.M, p.K, wave, lane, kbeg);
+    bi.init(p.weight, n0, p.N, p.K, wave, lane, kbeg);
     gemm_mainloop_dma<Cfg, NS, PIPE>(acc, ai, bi, KT, lds, prefetch);
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  if (blockIdx.x == 0 && threadIdx.x == 0) epilogue_ranges(p.epi);
+  if (p.sk.splits > 1 && !splitk_gather<Cfg>(acc, p.sk, tile, z)) return;
 
   gemm_epilogue_lds<Cfg, NS * Cfg::STAGE_SLOTS * 16>(acc, p.epi, pre, m0, n0, p.M, p.N,
                                                      static_cast<size_t>(p.ldo), lds);
-  if (blockIdx.x == 0 && threadIdx.x == 0) epilogue_ranges(p.epi);
 }
 
 typedef GemmCfg<256, 256, 64, 2, 4> CfgL8;    // 8 waves, wave tile 128 x 64
@@ -236,10 +242,12 @@ void launch_stream(hipStream_t s, const FcArgs& a, long cus, int groups_per_cu) 
 }
 
 template <class Cfg, int NS, int PIPE, bool BUF>
-void launch_dma(hipStream_t s, const FcArgs& a) {
-  const int tiles = ((a.M + Cfg::BM - 1) / Cfg::BM) * ((a.N + Cfg::BN - 1) / Cfg::BN);
-  hipLaunchKernelGGL((fc_dma_kernel<Cfg, NS, PIPE, BUF>), dim3(tiles), dim3(Cfg::kThreads), 0,
-                     s, a);
+void launch_dma(hipStream_t s, FcArgs a, int splits, const Workspace& ws) {
+  const long tiles = static_cast<long>((a.M + Cfg::BM - 1) / Cfg::BM) * ((a.N + Cfg::BN - 1) / Cfg::BN);
+  splitk_setup<Cfg>(s, a.sk, tiles, a.K, splits, ws.ptr, ws.bytes);
+  hipLaunchKernelGGL((fc_dma_kernel<Cfg, NS, PIPE, BUF>),
+                     dim3(static_cast<unsigned>(tiles * a.sk.splits)), dim3(Cfg::kThreads), 0, s,
+                     a);
   MXQ_LAUNCH_CHECK();
 }
 
@@ -253,17 +261,6 @@ void launch_cfg(hipStream_t s, const FcArgs& a, bool aligned) {
   MXQ_LAUNCH_CHECK();
 }
 
-int num_cus() {
-  int dev = 0;
-  MXQ_HIP(hipGetDevice(&dev));
-  static thread_local int cached_dev = -1, cached_cus = 0;
-  if (cached_dev != dev) {
-    MXQ_HIP(hipDeviceGetAttribute(&cached_cus, hipDeviceAttributeMultiprocessorCount, dev));
-    cached_dev = dev;
-  }
-  return cached_cus;
-}
-
 }  // namespace
 
 // Tile configurations:
@@ -275,11 +272,93 @@ int num_cus() {
 //   41..44  as 21..24 with a 2-stage ring (short K)
 //   51..56  128-byte stages: 64x64 (2, 3 stages), 128x128 (2, 3), 256x256 (2), 256x128 (2)
 //   57..59  128x64 and 64x128 with 128-byte stages, 64x64 with 256-byte stages
+//   61, 62  the short-K streaming kernel with 64- / 128-column strips
+// Output tile of a direct-to-LDS configuration (what a split-K work-group leaves in the
+// workspace); false for every other configuration.
+bool fc_cfg_tile(int cfg, int& bm, int& bn) {
+  switch (cfg) {
+    case 11: case 12: case 14: case 16: case 31: case 32: case 55: bm = 256; bn = 256; return true;
+    case 21: case 41: case 56: bm = 256; bn = 128; return true;
+    case 22: case 42: bm = 256; bn = 64; return true;
+    case 23: case 43: case 53: case 54: bm = 128; bn = 128; return true;
+    case 24: case 44: case 51: case 52: case 59: bm = 64; bn = 64; return true;
+    case 57: bm = 128; bn = 64; return true;
+    case 58: bm = 64; bn = 128; return true;
+    default: return false;
+  }
+}
+
+struct FcPlan {
+  int cfg;
+  int splits;
+  int stream_groups;
+};
+
+// What launch_fc would run for this shape.  `aligned`: K % 16 == 0 and 16-byte aligned
+// operands; `fused8`: int8 output only, 16-byte aligned with a row pitch that is a
+// multiple of 16 (what the streaming kernel stores).
+FcPlan plan_fc(int M, int N, int K, bool aligned, bool fused8, const GemmForce& force) {
+  FcPlan plan = {force.cfg, force.splits, force.stream_groups > 0 ? force.stream_groups : 2};
+  const bool buf_ok = aligned && K >= 16 && static_cast<long long>(M) * K < (1LL << 31) &&
+                      static_cast<long long>(N) * K < (1LL << 31);
+  const bool glb_ok = buf_ok && (K % 64 == 0);
+  const long cus = num_cus();
+  if (plan.cfg == 0) {
+    auto tiles = [&](int bm, int bn) {
+      return static_cast<long>((M + bm - 1) / bm) * ((N + bn - 1) / bn);
+    };
+    int auto_splits = 1;
+    if (buf_ok) {
+      switch (choose_tile(M, N, K, cus, false, &auto_splits)) {
+        case Tile::kL8: plan.cfg = glb_ok ? 12 : 31; break;
+        case Tile::kW128x2: plan.cfg = 41; break;
+        case Tile::kW128K2: plan.cfg = 56; break;
+        case Tile::kM128x2: plan.cfg = 43; break;
+        case Tile::kM128K2: plan.cfg = 53; break;
+        case Tile::kS64x2: plan.cfg = 44; break;
+        case Tile::kS64x4: plan.cfg = 24; break;
+        case Tile::kS64K2: plan.cfg = 51; break;
+        case Tile::kR128K2: plan.cfg = 57; break;
+        case Tile::kQ128K2: plan.cfg = 58; break;
+        case Tile::kS64K4: plan.cfg = 59; break;
+      }
+    } else {
+      if (tiles(256, 256) >= cus)
+        plan.cfg = 1;
+      else if (tiles(128, 128) >= cus)
+        plan.cfg = 3;
+      else
+        plan.cfg = 4;
+    }
+    if (plan.splits == 0) plan.splits = auto_splits;
+    // the short-K streaming kernel: chosen for tall outputs of at most 256 columns
+    // (200704 x 64 -> 64: 8.5 us against 10.2; -> 256: 18.5 against 21.9; 200704 x 128 ->
+    // 128: 15.3 against 17.1); from 512 columns on the tiled kernels are level or ahead
+    const int stream_rows = K == 256 ? 128 : 256;
+    const bool stream_ok = aligned && fused8 && (K == 32 || K == 64 || K == 128 || K == 256) &&
+                           N % 64 == 0 && (N <= stream_rows || N % stream_rows == 0);
+    if (stream_ok && N <= 256 && K <= 128 && M >= 32768) {
+      plan.cfg = (N % 128 == 0) ? 62 : 61;
+      plan.splits = 1;
+      if (force.stream_groups <= 0) plan.stream_groups = K <= 64 ? 4 : 3;
+    }
+  }
+  if (plan.splits <= 0) plan.splits = 1;
+  return plan;
+}
+
+size_t fc_plan_workspace(const FcPlan& plan, int M, int N) {
+  int bm, bn;
+  if (plan.splits <= 1 || !fc_cfg_tile(plan.cfg, bm, bn)) return 0;
+  const long tiles = static_cast<long>((M + bm - 1) / bm) * ((N + bn - 1) / bn);
+  return splitk_workspace_bytes(tiles, plan.splits, bm, bn);
+}
+
 // an output without elements still owes its range scalars
 __global__ void gemm_ranges_kernel(Epilogue e) { epilogue_ranges(e); }
 
 void launch_fc(hipStream_t s, const int8_t* data, const int8_t* weight, int M, int N, int K,
-               int ldo, const Epilogue& epi) {
+               int ldo, const Epilogue& epi, const GemmForce& force, const Workspace& ws) {
   if (M == 0 || N == 0) {
     hipLaunchKernelGGL(gemm_ranges_kernel, dim3(1), dim3(1), 0, s, epi);
     MXQ_LAUNCH_CHECK();
@@ -293,116 +372,102 @@ void launch_fc(hipStream_t s, const int8_t* data, const int8_t* weight, int M, i
   a.K = K;
   a.ldo = ldo;
   a.epi = epi;
+  a.sk.splits = 1;
+  a.sk.kt_per_split = 1 << 30;
+  a.sk.counters = nullptr;
+  a.sk.partials = nullptr;
   const bool aligned = (K % 16 == 0) && aligned16(data) && aligned16(weight);
   // direct-to-LDS kernels: operands below 2 GiB; K a multiple of the 64-byte stage for
   // the global-load form, of 16 for the buffer-load form
   const bool buf_ok = aligned && K >= 16 && static_cast<long long>(M) * K < (1LL << 31) &&
                       static_cast<long long>(N) * K < (1LL << 31);
   const bool glb_ok = buf_ok && (K % 64 == 0);
-  int cfg = g_fc_config;
-  if (cfg == 0) {
-    const long cus = num_cus();
-    auto tiles = [&](int bm, int bn) {
-      return static_cast<long>((M + bm - 1) / bm) * ((N + bn - 1) / bn);
-    };
-    if (buf_ok) {
-      switch (choose_tile(M, N, K, cus)) {
-        case Tile::kL8: cfg = glb_ok ? 12 : 31; break;
-        case Tile::kW128x2: cfg = 41; break;
-        case Tile::kW128K2: cfg = 56; break;
-        case Tile::kM128x2: cfg = 43; break;
-        case Tile::kM128K2: cfg = 53; break;
-        case Tile::kS64x2: cfg = 44; break;
-        case Tile::kS64x4: cfg = 24; break;
-        case Tile::kS64K2: cfg = 51; break;
-        case Tile::kR128K2: cfg = 57; break;
-        case Tile::kQ128K2: cfg = 58; break;
-        case Tile::kS64K4: cfg = 59; break;
-      }
-    } else {
-      if (tiles(256, 256) >= cus)
-        cfg = 1;
-      else if (tiles(128, 128) >= cus)
-        cfg = 3;
-      else
-        cfg = 4;
-    }
+  const bool fused8 = epi.out32 == nullptr && epi.out8 != nullptr && ldo % 16 == 0 &&
+                      aligned16(epi.out8);
+  FcPlan plan = plan_fc(M, N, K, aligned, fused8, force);
+  // a split the chooser proposed is dropped when the caller brought no room for it
+  if (force.splits == 0 && plan.splits > 1 &&
+      (ws.ptr == nullptr || !aligned16(ws.ptr) || ws.bytes < fc_plan_workspace(plan, M, N))) {
+    GemmForce unsplit = force;
+    unsplit.splits = 1;
+    plan = plan_fc(M, N, K, aligned, fused8, unsplit);
   }
+  const int cfg = plan.cfg;
   if (cfg >= 11 && cfg <= 16) MXQ_CHECK(glb_ok, "shape does not qualify for the DMA kernels");
-  // 61 / 62: the short-K streaming kernel with 64- / 128-column strips
-  const int stream_rows = K == 256 ? 128 : 256;  // weight rows one work-group parks in LDS
-  const bool stream_ok = aligned && (K == 32 || K == 64 || K == 128 || K == 256) &&
-                         epi.out32 == nullptr && epi.out8 != nullptr && N % 64 == 0 &&
-                         (N <= stream_rows || N % stream_rows == 0) && ldo % 16 == 0 &&
-                         aligned16(epi.out8);
-  // chosen for tall outputs of at most 256 columns (200704 x 64 -> 64: 8.5 us against 10.2;
-  // -> 256: 18.5 against 21.9; 200704 x 128 -> 128: 15.3 against 17.1); from 512 columns on
-  // the tiled kernels are level or ahead
-  int stream_groups = g_fc_stream_groups;
-  if (g_fc_config == 0 && stream_ok && N <= 256 && K <= 128 && M >= 32768) {
-    cfg = (N % 128 == 0) ? 62 : 61;
-    stream_groups = K <= 64 ? 4 : 3;
-  }
   if (cfg == 61 || cfg == 62) {
+    const int stream_rows = K == 256 ? 128 : 256;  // weight rows one work-group parks in LDS
+    const bool stream_ok = aligned && fused8 && (K == 32 || K == 64 || K == 128 || K == 256) &&
+                           N % 64 == 0 && (N <= stream_rows || N % stream_rows == 0);
     MXQ_CHECK(stream_ok && (cfg == 61 || N % 128 == 0),
               "shape does not qualify for the short-K streaming kernel");
+    MXQ_CHECK(plan.stream_groups >= 1 && plan.stream_groups <= 16, "stream_groups out of range");
     const long cus = num_cus();
 #define MXQ_STREAM(NI)                                                          \
   do {                                                                          \
-    if (K == 32) launch_stream<1, NI>(s, a, cus, stream_groups);           \
-    else if (K == 64) launch_stream<2, NI>(s, a, cus, stream_groups);      \
-    else if (K == 128) launch_stream<4, NI>(s, a, cus, stream_groups);     \
-    else launch_stream<8, NI>(s, a, cus, stream_groups);                   \
+    if (K == 32) launch_stream<1, NI>(s, a, cus, plan.stream_groups);           \
+    else if (K == 64) launch_stream<2, NI>(s, a, cus, plan.stream_groups);      \
+    else if (K == 128) launch_stream<4, NI>(s, a, cus, plan.stream_groups);     \
+    else launch_stream<8, NI>(s, a, cus, plan.stream_groups);                   \
   } while (0)
     if (cfg == 61) MXQ_STREAM(2); else MXQ_STREAM(4);
 #undef MXQ_STREAM
     return;
   }
   if (cfg >= 21) MXQ_CHECK(buf_ok, "shape does not qualify for the buffer-load DMA kernels");
+  if (cfg < 11) MXQ_CHECK(plan.splits <= 1, "the register-staged kernels have no split-K form");
+  const int sp = plan.splits;
   switch (cfg) {
     case 1: launch_cfg<CfgL8>(s, a, aligned); break;
     case 2: launch_cfg<CfgL4>(s, a, aligned); break;
     case 3: launch_cfg<CfgM>(s, a, aligned); break;
     case 4: launch_cfg<CfgS>(s, a, aligned); break;
-    case 11: launch_dma<CfgL8, 4, 0, false>(s, a); break;
-    case 12: launch_dma<CfgL8, 4, 2, false>(s, a); break;
-    case 14: launch_dma<CfgL4, 4, 0, false>(s, a); break;
-    case 16: launch_dma<CfgL4, 4, 2, false>(s, a); break;
-    case 21: launch_dma<CfgW128, 4, 2, true>(s, a); break;
-    case 22: launch_dma<CfgW64, 4, 2, true>(s, a); break;
-    case 23: launch_dma<CfgM, 4, 2, true>(s, a); break;
-    case 24: launch_dma<CfgS, 4, 2, true>(s, a); break;
-    case 41: launch_dma<CfgW128, 2, 0, true>(s, a); break;
-    case 42: launch_dma<CfgW64, 2, 0, true>(s, a); break;
-    case 43: launch_dma<CfgM, 2, 0, true>(s, a); break;
-    case 44: launch_dma<CfgS, 2, 0, true>(s, a); break;
-    case 51: launch_dma<CfgSK, 2, 0, true>(s, a); break;
-    case 52: launch_dma<CfgSK, 3, 0, true>(s, a); break;
-    case 53: launch_dma<CfgMK, 2, 0, true>(s, a); break;
-    case 54: launch_dma<CfgMK, 3, 0, true>(s, a); break;
-    case 55: launch_dma<CfgL8K, 2, 0, true>(s, a); break;
-    case 56: launch_dma<CfgW128K, 2, 0, true>(s, a); break;
-    case 57: launch_dma<CfgRK, 2, 0, true>(s, a); break;
-    case 58: launch_dma<CfgQK, 2, 0, true>(s, a); break;
-    case 59: launch_dma<CfgSK2, 2, 0, true>(s, a); break;
-    case 31: launch_dma<CfgL8, 4, 2, true>(s, a); break;
-    case 32: launch_dma<CfgL4, 4, 2, true>(s, a); break;
+    case 11: launch_dma<CfgL8, 4, 0, false>(s, a, sp, ws); break;
+    case 12: launch_dma<CfgL8, 4, 2, false>(s, a, sp, ws); break;
+    case 14: launch_dma<CfgL4, 4, 0, false>(s, a, sp, ws); break;
+    case 16: launch_dma<CfgL4, 4, 2, false>(s, a, sp, ws); break;
+    case 21: launch_dma<CfgW128, 4, 2, true>(s, a, sp, ws); break;
+    case 22: launch_dma<CfgW64, 4, 2, true>(s, a, sp, ws); break;
+    case 23: launch_dma<CfgM, 4, 2, true>(s, a, sp, ws); break;
+    case 24: launch_dma<CfgS, 4, 2, true>(s, a, sp, ws); break;
+    case 41: launch_dma<CfgW128, 2, 0, true>(s, a, sp, ws); break;
+    case 42: launch_dma<CfgW64, 2, 0, true>(s, a, sp, ws); break;
+    case 43: launch_dma<CfgM, 2, 0, true>(s, a, sp, ws); break;
+    case 44: launch_dma<CfgS, 2, 0, true>(s, a, sp, ws); break;
+    case 51: launch_dma<CfgSK, 2, 0, true>(s, a, sp, ws); break;
+    case 52: launch_dma<CfgSK, 3, 0, true>(s, a, sp, ws); break;
+    case 53: launch_dma<CfgMK, 2, 0, true>(s, a, sp, ws); break;
+    case 54: launch_dma<CfgMK, 3, 0, true>(s, a, sp, ws); break;
+    case 55: launch_dma<CfgL8K, 2, 0, true>(s, a, sp, ws); break;
+    case 56: launch_dma<CfgW128K, 2, 0, true>(s, a, sp, ws); break;
+    case 57: launch_dma<CfgRK, 2, 0, true>(s, a, sp, ws); break;
+    case 58: launch_dma<CfgQK, 2, 0, true>(s, a, sp, ws); break;
+    case 59: launch_dma<CfgSK2, 2, 0, true>(s, a, sp, ws); break;
+    case 31: launch_dma<CfgL8, 4, 2, true>(s, a, sp, ws); break;
+    case 32: launch_dma<CfgL4, 4, 2, true>(s, a, sp, ws); break;
     default: MXQ_CHECK(false, "unknown fc tile configuration " << cfg);
   }
+}
+
+// Scratch bytes with which launch_fc takes its fastest route for this shape (0 when it
+// would not split).  Assumes 16-byte aligned operands.
+size_t fc_workspace_bytes(int M, int N, int K, bool fused8) {
+  if (M <= 0 || N <= 0 || K <= 0) return 0;
+  const FcPlan plan = plan_fc(M, N, K, K % 16 == 0, fused8, GemmForce());
+  return fc_plan_workspace(plan, M, N);
 }
 
 }  // namespace mxq
 
 using namespace mxq;
 
-extern "C" int mxq_quantized_fc(void* stream, const int8_t* data, const int8_t* weight,
-                                const int8_t* bias, int M, int N, int K, const float* min_data,
-                                const float* max_data, const float* min_weight,
-                                const float* max_weight, const float* min_bias,
-                                const float* max_bias, int32_t* out32, float* omin, float* omax,
-                                int8_t* out8, float* rmin, float* rmax, int relu,
-                                float min_calib, float max_calib) {
-  MXQ_API_BEGIN();
+namespace {
+
+void fc_entry(void* stream, const int8_t* data, const int8_t* weight, const int8_t* bias, int M,
+              int N, int K, const float* min_data, const float* max_data,
+              const float* min_weight, const float* max_weight, const float* min_bias,
+              const float* max_bias, int32_t* out32, float* omin, float* omax, int8_t* out8,
+              float* rmin, float* rmax, int relu, float min_calib, float max_calib,
+              void* workspace, size_t workspace_bytes, const GemmForce& force) {
   MXQ_CHECK(M >= 0 && N >= 0 && K >= 0, "negative dimension");
   MXQ_CHECK(min_data && max_data && min_weight && max_weight, "null input range pointer");
   MXQ_CHECK(omin && omax, "null output range pointer");
@@ -429,6 +494,58 @@ extern "C" int mxq_quantized_fc(void* stream, const int8_t* data, const int8_t* 
   float a = fabsf(min_calib), b = fabsf(max_calib);
   e.real_range = (a < b) ? b : a;
   e.plane = 0;
-  launch_fc(static_cast<hipStream_t>(stream), data, weight, M, N, K, N, e);
+  Workspace ws;
+  ws.ptr = workspace;
+  ws.bytes = workspace_bytes;
+  launch_fc(static_cast<hipStream_t>(stream), data, weight, M, N, K, N, e, force, ws);
+}
+
+}  // namespace
+
+extern "C" {
+
+size_t mxq_quantized_fc_workspace(int M, int N, int K, int fused_int8_only) {
+  try {
+    return fc_workspace_bytes(M, N, K, fused_int8_only != 0 && N % 16 == 0);
+  } catch (...) {
+    return 0;
+  }
+}
+
+int mxq_quantized_fc(void* stream, const int8_t* data, const int8_t* weight, const int8_t* bias,
+                     int M, int N, int K, const float* min_data, const float* max_data,
+                     const float* min_weight, const float* max_weight, const float* min_bias,
+                     const float* max_bias, int32_t* out32, float* omin, float* omax,
+                     int8_t* out8, float* rmin, float* rmax, int relu, float min_calib,
+                     float max_calib, void* workspace, size_t workspace_bytes) {
+  MXQ_API_BEGIN();
+  fc_entry(stream, data, weight, bias, M, N, K, min_data, max_data, min_weight, max_weight,
+           min_bias, max_bias, out32, omin, omax, out8, rmin, rmax, relu, min_calib, max_calib,
+           workspace, workspace_bytes, GemmForce());
   MXQ_API_END();
 }
+
+// Test-only twin of mxq_quantized_fc (declared in tests/mxq_test_hooks.h, not in the
+// operator header): the tile configuration, the split-K factor and the streaming kernel's
+// work-groups per CU come as arguments (0 = let the launcher choose), so tests can drive
+// every kernel variant on any shape without process-wide state.
+int mxq_test_quantized_fc(void* stream, const int8_t* data, const int8_t* weight,
+                          const int8_t* bias, int M, int N, int K, const float* min_data,
+                          const float* max_data, const float* min_weight,
+                          const float* max_weight, const float* min_bias, const float* max_bias,
+                          int32_t* out32, float* omin, float* omax, int8_t* out8, float* rmin,
+                          float* rmax, int relu, float min_calib, float max_calib,
+                          void* workspace, size_t workspace_bytes, int cfg, int splits,
+                          int stream_groups) {
+  MXQ_API_BEGIN();
+  GemmForce force;
+  force.cfg = cfg;
+  force.splits = splits;
+  force.stream_groups = stream_groups;
+  fc_entry(stream, data, weight, bias, M, N, K, min_data, max_data, min_weight, max_weight,
+           min_bias, max_bias, out32, omin, omax, out8, rmin, rmax, relu, min_calib, max_calib,
+           workspace, workspace_bytes, force);
+  MXQ_API_END();
+}
+
+}  // extern "C"

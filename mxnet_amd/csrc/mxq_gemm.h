@@ -27,14 +27,16 @@
 //   out32     = acc                                      optional
 //   out8      = FloatToQuantized(float(acc) * (max_out / 2^31), -R, R)   requantize-inl.h:89-105
 //               optionally max(out8, 0)
-#ifndef MXQ_GEMM_CUH_
-#define MXQ_GEMM_CUH_
+#ifndef MXQ_GEMM_H_
+#define MXQ_GEMM_H_
 
 #include <hip/hip_runtime.h>
 
 #include <type_traits>
 
 #include <cstdint>
+
+#include "mxq_common.h"
 
 namespace mxq {
 
@@ -173,11 +175,10 @@ struct GemmCfg {
 // 8 XCDs round-robin; remap so that each XCD (own L2) owns a contiguous run of
 // logical tile ids, and order logical ids in bands of GROUP tile-rows so the run
 // is a compact rectangle that shares activation rows and weight rows in L2.
-__device__ __forceinline__ void tile_coords(int bid, int tiles_m, int tiles_n, int& tm,
-                                            int& tn) {
-  const int total = tiles_m * tiles_n;
-  int lid = bid;
-  if ((total & 7) == 0) lid = (bid & 7) * (total >> 3) + (bid >> 3);
+__device__ __forceinline__ int xcd_remap(int bid, int total) {
+  return ((total & 7) == 0) ? (bid & 7) * (total >> 3) + (bid >> 3) : bid;
+}
+__device__ __forceinline__ void band_coords(int lid, int tiles_m, int tiles_n, int& tm, int& tn) {
   constexpr int GROUP = 4;
   const int band = GROUP * tiles_n;
   const int g = lid / band;
@@ -186,6 +187,21 @@ __device__ __forceinline__ void tile_coords(int bid, int tiles_m, int tiles_n, i
   const int in_band = lid - g * band;
   tm = first_m + in_band % rows;
   tn = in_band / rows;
+}
+__device__ __forceinline__ void tile_coords(int bid, int tiles_m, int tiles_n, int& tm,
+                                            int& tn) {
+  band_coords(xcd_remap(bid, tiles_m * tiles_n), tiles_m, tiles_n, tm, tn);
+}
+// The same for a grid of tiles x splits work-groups (split-K): consecutive logical ids walk
+// the tiles of one K slice, so the work-groups an XCD owns share operand rows in its L2.
+// `tile` is the tile's index in the counter and partial arrays.
+__device__ __forceinline__ void tile_coords_split(int bid, int tiles_m, int tiles_n, int splits,
+                                                  int& tm, int& tn, int& tile, int& z) {
+  const int tiles = tiles_m * tiles_n;
+  const int lid = xcd_remap(bid, tiles * splits);
+  z = lid / tiles;
+  tile = lid - z * tiles;
+  band_coords(tile, tiles_m, tiles_n, tm, tn);
 }
 
 // 16 bytes of row `row` at byte offset k0; zero outside [0,K).  With ALIGNED the
@@ -399,14 +415,15 @@ struct DmaLane {
 
 // K-contiguous row-major operand (FC activation, every weight) through
 // global_load_lds.  Needs K % BK == 0; rows past the end are clamped to the last
-// row (they only feed accumulators that are never stored).
+// row (they only feed accumulators that are never stored).  `kbeg` is the byte offset
+// inside a row at which stage 0 starts (the K slice of a split-K work-group).
 template <class Cfg, int INSTR>
 struct RowIssuerGlobal {
   uint32_t voff[INSTR];
   const int8_t* base;
   __device__ __forceinline__ void init(const int8_t* b, int row_begin, int rows, int K, int wave,
-                                       int lane) {
-    base = b;
+                                       int lane, int kbeg = 0) {
+    base = b + kbeg;
     DmaLane<Cfg> g;
     g.init(wave, lane);
 #pragma unroll
@@ -430,12 +447,12 @@ struct RowIssuerBuffer {
   int c16, K;
   v4i rsrc;
   __device__ __forceinline__ void init(const int8_t* b, int row_begin, int rows, int K_, int wave,
-                                       int lane) {
+                                       int lane, int kbeg = 0) {
     K = K_;
     rsrc = make_rsrc(b, static_cast<uint32_t>(rows) * static_cast<uint32_t>(K_));
     DmaLane<Cfg> g;
     g.init(wave, lane);
-    c16 = g.c16;
+    c16 = g.c16 + kbeg;
 #pragma unroll
     for (int i = 0; i < INSTR; ++i) {
       const int row = row_begin + g.row0 + i * DmaLane<Cfg>::kRowStep;
@@ -893,6 +910,133 @@ __device__ __forceinline__ void gemm_epilogue_lds(v16i (&acc)[Cfg::MI][Cfg::NI],
   }
 }
 
+// ---- split-K -------------------------------------------------------------------------
+// Shapes with few output tiles and a long reduction leave most CUs idle.  There `splits`
+// work-groups share one output tile, each reducing a slice of kt_per_split K stages.  Integer
+// accumulation is associative, so the sum of the slices is the unsplit result bit for bit.
+// Every work-group of a tile leaves its accumulators in the workspace (in lane order: the
+// work-group that reads them back has the same thread -> output mapping, so both sides
+// move whole 1 KiB runs per wave instruction and nothing is transposed), then takes a
+// ticket from the tile's counter; the one that draws the last ticket adds the other
+// slices to its own registers and runs the ordinary epilogue, the others exit.  No
+// work-group waits for another.
+//
+// Visibility across the XCDs' L2s without a fence: partials are written and read with
+// device-scope accesses (sc1: written through to, and read from, the level all XCDs
+// share), a work-group's stores have completed (vmcnt(0) on every lane, then the
+// barrier) before its thread 0 takes the ticket with a device-scope atomic, and the last
+// work-group issues its loads only after the atomic has returned.
+struct SplitK {
+  int splits;          // work-groups per output tile; 1 = no split
+  int kt_per_split;    // K stages per work-group
+  unsigned* counters;  // [tiles], zero when the kernel starts
+  int* partials;       // [tiles][splits][BM * BN]
+};
+
+inline size_t splitk_counter_bytes(long tiles) {
+  return (static_cast<size_t>(tiles) * 4 + 255) / 256 * 256;
+}
+inline size_t splitk_workspace_bytes(long tiles, int splits, int bm, int bn) {
+  if (splits <= 1) return 0;
+  return splitk_counter_bytes(tiles) + static_cast<size_t>(tiles) * splits * bm * bn * 4;
+}
+
+// (a template only so that every file including this header may define it)
+template <int kBlock>
+__global__ void splitk_zero_kernel(unsigned* counters, int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) counters[i] = 0u;
+}
+
+// Host side: turns the requested split count into the kernel's SplitK (never more slices
+// than K stages, no empty slice), carves the workspace and clears the counters on `s`.
+template <class Cfg>
+inline void splitk_setup(hipStream_t s, SplitK& sk, long tiles, int K, int splits, void* ws,
+                         size_t ws_bytes) {
+  const int KT = (K + Cfg::BK - 1) / Cfg::BK;
+  if (splits > KT) splits = KT;
+  if (splits < 1) splits = 1;
+  sk.kt_per_split = (KT + splits - 1) / splits;
+  if (sk.kt_per_split < 1) sk.kt_per_split = 1;
+  sk.splits = KT > 0 ? (KT + sk.kt_per_split - 1) / sk.kt_per_split : 1;
+  sk.counters = nullptr;
+  sk.partials = nullptr;
+  if (sk.splits <= 1) {
+    sk.splits = 1;
+    return;
+  }
+  const size_t need = splitk_workspace_bytes(tiles, sk.splits, Cfg::BM, Cfg::BN);
+  MXQ_CHECK(ws != nullptr && aligned16(ws), "split-K needs a 16-byte aligned workspace");
+  MXQ_CHECK(ws_bytes >= need, "split-K workspace too small: " << ws_bytes << " < " << need);
+  MXQ_CHECK(tiles * sk.splits < (1L << 30), "split-K grid too large");
+  sk.counters = static_cast<unsigned*>(ws);
+  sk.partials = reinterpret_cast<int*>(static_cast<char*>(ws) + splitk_counter_bytes(tiles));
+  hipLaunchKernelGGL(splitk_zero_kernel<256>, dim3(static_cast<unsigned>((tiles + 255) / 256)),
+                     dim3(256), 0, s, sk.counters, static_cast<int>(tiles));
+  MXQ_LAUNCH_CHECK();
+}
+
+// Device side, after the K loop of a split work-group.  Returns true in the work-group
+// that arrived last: its accumulators then hold the sum over all slices.
+template <class Cfg>
+__device__ __forceinline__ bool splitk_gather(v16i (&acc)[Cfg::MI][Cfg::NI], const SplitK& sk,
+                                              int tile, int z) {
+  constexpr int MI = Cfg::MI, NI = Cfg::NI, QUADS = MI * NI * 4;
+  constexpr int kTileInts = Cfg::BM * Cfg::BN;
+  static_assert(QUADS * 4 * Cfg::kThreads == kTileInts, "lane-order layout covers the tile");
+  constexpr int kDeviceScope = 16;  // sc1 in the buffer instructions' cache policy
+  constexpr int kRsrcFlags = 0x00020000;
+  const int tid = threadIdx.x;
+  __shared__ unsigned s_ticket;
+  int* tile_base = sk.partials + static_cast<size_t>(tile) * sk.splits * kTileInts;
+  {
+    const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(
+        tile_base + static_cast<size_t>(z) * kTileInts, 0, kTileInts * 4, kRsrcFlags);
+#pragma unroll
+    for (int mi = 0; mi < MI; ++mi)
+#pragma unroll
+      for (int ni = 0; ni < NI; ++ni)
+#pragma unroll
+        for (int vq = 0; vq < 4; ++vq) {
+          const v4i w = {acc[mi][ni][4 * vq], acc[mi][ni][4 * vq + 1], acc[mi][ni][4 * vq + 2],
+                         acc[mi][ni][4 * vq + 3]};
+          const int q = (mi * NI + ni) * 4 + vq;
+          __builtin_amdgcn_raw_buffer_store_b128(w, rs, (q * Cfg::kThreads + tid) * 16, 0,
+                                                 kDeviceScope);
+        }
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+  if (tid == 0)
+    s_ticket = __hip_atomic_fetch_add(sk.counters + tile, 1u, __ATOMIC_RELAXED,
+                                      __HIP_MEMORY_SCOPE_AGENT);
+  __syncthreads();
+  if (s_ticket != static_cast<unsigned>(sk.splits - 1)) return false;
+  for (int zz = 0; zz < sk.splits; ++zz) {
+    if (zz == z) continue;
+    const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(
+        tile_base + static_cast<size_t>(zz) * kTileInts, 0, kTileInts * 4, kRsrcFlags);
+#pragma unroll
+    for (int mi = 0; mi < MI; ++mi) {
+      v4i w[NI * 4];
+#pragma unroll
+      for (int j = 0; j < NI * 4; ++j)
+        w[j] = __builtin_amdgcn_raw_buffer_load_b128(
+            rs, ((mi * NI * 4 + j) * Cfg::kThreads + tid) * 16, 0, kDeviceScope);
+#pragma unroll
+      for (int ni = 0; ni < NI; ++ni)
+#pragma unroll
+        for (int vq = 0; vq < 4; ++vq)
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            acc[mi][ni][4 * vq + i] =
+                static_cast<int>(static_cast<uint32_t>(acc[mi][ni][4 * vq + i]) +
+                                 static_cast<uint32_t>(w[ni * 4 + vq][i]));
+    }
+  }
+  return true;
+}
+
 // Range scalars, written once per launch.
 __device__ __forceinline__ void epilogue_ranges(const Epilogue& e) {
   const EpiScalars s = epi_scalars(e);
@@ -905,4 +1049,4 @@ __device__ __forceinline__ void epilogue_ranges(const Epilogue& e) {
 }
 
 }  // namespace mxq
-#endif  // MXQ_GEMM_CUH_
+#endif  // MXQ_GEMM_H_

@@ -25,17 +25,6 @@ constexpr int kMaxDims = 8;
 
 typedef uint32_t u4 __attribute__((ext_vector_type(4)));
 
-int num_cus() {
-  int dev = 0;
-  MXQ_HIP(hipGetDevice(&dev));
-  static thread_local int cached_dev = -1, cached_cus = 0;
-  if (cached_dev != dev) {
-    MXQ_HIP(hipDeviceGetAttribute(&cached_cus, hipDeviceAttributeMultiprocessorCount, dev));
-    cached_dev = dev;
-  }
-  return cached_cus;
-}
-
 // Lanes that share one row: the smallest power of two that covers its `units` pieces,
 // at most a wave.
 int group_lanes(size_t units) {

@@ -13,7 +13,7 @@
 
 #include "../../include/mxq.h"
 #include "mxq_common.h"
-#include "mxq_gemm.cuh"
+#include "mxq_gemm.h"
 
 namespace mxq {
 namespace {
@@ -438,17 +438,6 @@ __global__ __launch_bounds__(256) void copy_bytes_kernel(const uint8_t* __restri
   }
 }
 
-int device_cus() {
-  int dev = 0;
-  MXQ_HIP(hipGetDevice(&dev));
-  static thread_local int cached_dev = -1, cached_cus = 0;
-  if (cached_dev != dev) {
-    MXQ_HIP(hipDeviceGetAttribute(&cached_cus, hipDeviceAttributeMultiprocessorCount, dev));
-    cached_dev = dev;
-  }
-  return cached_cus;
-}
-
 }  // namespace
 }  // namespace mxq
 
@@ -496,7 +485,7 @@ int mxq_quantized_pooling_nchw(void* stream, const void* in, int in_type, int N,
   a.is_unsigned = in_type == MXQ_UINT8;
   a.vec_ok = aligned16(in) ? 1 : 0;
   const long long plane_bytes = static_cast<long long>(H) * W;
-  const int cus = device_cus();
+  const int cus = num_cus();
   long long blocks = 0;
   bool direct = false;
   if (2 * plane_bytes <= kPoolLdsBytes) {
@@ -616,7 +605,7 @@ int mxq_quantized_flatten(void* stream, const void* in, const float* imin, const
   if (n_bytes != 0 && in != out) {
     const int vec_ok = aligned16(in) && aligned16(out);
     size_t g = (n_bytes / (vec_ok ? 16 : 1) + 255) / 256;
-    const size_t cap = static_cast<size_t>(device_cus()) * 8;
+    const size_t cap = static_cast<size_t>(num_cus()) * 8;
     if (g > cap) g = cap;
     if (g < 1) g = 1;
     hipLaunchKernelGGL(copy_bytes_kernel, dim3(static_cast<unsigned>(g)), dim3(256), 0, s,

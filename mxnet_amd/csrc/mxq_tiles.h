@@ -2,7 +2,26 @@
 #ifndef MXQ_TILES_H_
 #define MXQ_TILES_H_
 
+#include <cstddef>
+
 namespace mxq {
+
+// What a caller may pin instead of leaving it to the choosers below: a tile configuration
+// number of the launcher (0 = choose by shape), the number of work-groups that share one
+// output tile along K (0 = choose, 1 = no split) and, for the short-K streaming kernel,
+// its work-groups per CU (0 = choose).  The operator entry points pass the default; the
+// test-only entry points pass what the test asks for.
+struct GemmForce {
+  int cfg = 0;
+  int splits = 0;
+  int stream_groups = 0;
+};
+
+// Caller-provided scratch for the split-K route (may be null: then nothing is split).
+struct Workspace {
+  void* ptr = nullptr;
+  size_t bytes = 0;
+};
 
 enum class Tile {
   kL8,      // 256 x 256, 64-byte stages, 4-stage ring, pinned pipeline
@@ -34,7 +53,9 @@ enum class Tile {
 // `gather` says that the left operand is gathered pixel by pixel (convolution): the 64-row
 // tile then issues half as many gathers per wave and measures a few per cent ahead of the
 // 128-row one, which in turn is ahead for plain row-major operands.
-inline Tile choose_tile(long M, long N, long K, long cus, bool gather = false) {
+inline Tile choose_tile(long M, long N, long K, long cus, bool gather = false,
+                        int* splits = nullptr) {
+  if (splits != nullptr) *splits = 1;
   auto tiles = [&](long bm, long bn) { return ((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
   if (K > 256 && N > 128 && 16 * tiles(256, 256) >= 9 * cus) return Tile::kL8;
   if (N <= 64) return (K >= 4096) ? Tile::kS64x4 : Tile::kS64x2;

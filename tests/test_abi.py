@@ -21,8 +21,26 @@ def test_hip_library_exports_every_declared_symbol():
     for n in names:
         assert hasattr(lib, n), n
         assert n in mxnet_amd._lib.SIGNATURES, "no ctypes signature for " + n
-    assert mxnet_amd._lib.lib.mxq_abi_version() == 1
+    assert mxnet_amd._lib.lib.mxq_abi_version() == 2
     assert mxnet_amd._lib.last_error() == ""
+
+
+def test_hip_library_has_no_tuning_state():
+    """The launcher keeps no mutable process-wide configuration: the old tuning setter and
+    its globals are gone; forced kernel variants are arguments of the test-only entry
+    points (tests/mxq_test_hooks.h)."""
+    import subprocess
+    import mxnet_amd
+    out = subprocess.run(["nm", "-C", "--defined-only", mxnet_amd._lib.LIB_PATH],
+                         capture_output=True, text=True, check=True).stdout
+    assert "mxq_set_tuning" not in out
+    assert not re.findall(r"\bmxq::g_\w+", out)
+    for hook in mxnet_amd._lib.TEST_HOOKS:
+        assert hook in out
+        assert hook not in declared_functions("mxq.h")
+    hooks_h = open(os.path.join(ROOT, "tests", "mxq_test_hooks.h")).read()
+    for hook in mxnet_amd._lib.TEST_HOOKS:
+        assert hook in hooks_h
 
 
 def test_ops_library_exports_every_declared_symbol():
@@ -46,8 +64,10 @@ def test_argument_validation_needs_no_gpu():
     rc = lib.mxq_dequantize(None, p, 0, p, p, p, 4)
     assert rc == -1 and "int8 or uint8" in mxnet_amd._lib.last_error()
     rc = lib.mxq_quantized_fc(None, p, p, None, 4, 4, 16, p, p, p, p, None, None, None, p, p,
-                              None, None, None, 0, 0.0, 0.0)
+                              None, None, None, 0, 0.0, 0.0, None, 0)
     assert rc == -1 and "no output buffer" in mxnet_amd._lib.last_error()
+    # the workspace queries are host arithmetic
+    assert lib.mxq_quantized_fc_workspace(4, 4, 16, 0) == 0
     rc = lib.mxq_nhwc_to_nchw(None, p, p, 1, 1, 1, 1, 2)
     assert rc == -1 and "elem_bytes" in mxnet_amd._lib.last_error()
     assert lib.mxq_quantize_v2_workspace(1 << 26) >= 64

@@ -24,13 +24,15 @@ def f32(v):
     return dev(np.array([v], np.float32))
 
 
-def run_conv_nchw(capi, d, w, b, rd, rw, rb, stride, pad, dilate, calib=None, relu=False):
+def run_conv_nchw(capi, d, w, b, rd, rw, rb, stride, pad, dilate, calib=None, relu=False,
+                  force=None):
+    """force = (cfg, splits) pins the kernel variant through the test-only entry point."""
     dn = capi.nchw_to_nhwc_i8(dev(d))
     wn = capi.nchw_to_nhwc_i8(dev(w))
     res = capi.quantized_conv_nhwc(dn, wn, None if b is None else dev(b), f32(-rd), f32(rd),
                                    f32(-rw), f32(rw), None if b is None else f32(-rb),
                                    None if b is None else f32(rb), stride=stride, pad=pad,
-                                   dilate=dilate, calib=calib, relu=relu)
+                                   dilate=dilate, calib=calib, relu=relu, force=force)
     res["out32_nchw"] = capi.nhwc_to_nchw(res["out32"])
     if res["out8"] is not None:
         res["out8_nchw"] = capi.nhwc_to_nchw(res["out8"])
@@ -72,18 +74,12 @@ def test_conv_int32(capi, case, use_bias):
 @pytest.mark.parametrize("cfg", [1, 2, 3, 4, 5, 11, 12, 13, 14, 15, 16, 22, 23, 24, 25, 31, 32, 33, 34,
                                  35, 36, 37, 38, 39])
 def test_conv_every_tile_config(capi, cfg):
-    import mxnet_amd
     N, C, H, W, O, KH, KW, s, p, dl = (2, 32, 19, 19, 72, 3, 3, 1, 1, 1)
     d = int8_uniform((N, C, H, W), seed=cfg)
     w = int8_uniform((O, C, KH, KW), seed=cfg + 1)
     b = int8_uniform((O,), seed=cfg + 2)
-    mxnet_amd._lib.set_tuning("conv_config", cfg)
-    try:
-        res = run_conv_nchw(capi, d, w, b, 1.0, 1.0, 1.0, (s, s), (p, p), (dl, dl),
-                            calib=(-0.02, 0.02), relu=True)
-        torch.cuda.synchronize()
-    finally:
-        mxnet_amd._lib.set_tuning("conv_config", 0)
+    res = run_conv_nchw(capi, d, w, b, 1.0, 1.0, 1.0, (s, s), (p, p), (dl, dl),
+                        calib=(-0.02, 0.02), relu=True, force=(cfg, 1))
     ro, rmn, rmx = oracle.quantized_conv(d, w, b, -1.0, 1.0, -1.0, 1.0, -1.0, 1.0, (s, s),
                                          (p, p), (dl, dl))
     np.testing.assert_array_equal(res["out32_nchw"].cpu().numpy(), ro)
@@ -100,23 +96,42 @@ def test_conv_every_tile_config(capi, cfg):
 def test_conv_direct_to_lds_configs(capi, cfg, case):
     """The buffer-load kernels on shapes that stress the tap bookkeeping: C = 16 (four
     taps per 64-byte stage), C = 48 (taps straddle stages), stride 2, dilation, K tails."""
-    import mxnet_amd
     N, C, H, W, O, KH, KW, s, p, dl = case
     d = int8_uniform((N, C, H, W), seed=cfg + C)
     w = int8_uniform((O, C, KH, KW), seed=cfg + O)
     b = int8_uniform((O,), seed=cfg)
-    mxnet_amd._lib.set_tuning("conv_config", cfg)
-    try:
-        res = run_conv_nchw(capi, d, w, b, 1.0, 1.0, 1.0, (s, s), (p, p), (dl, dl),
-                            calib=(-0.05, 0.04), relu=False)
-        torch.cuda.synchronize()
-    finally:
-        mxnet_amd._lib.set_tuning("conv_config", 0)
+    res = run_conv_nchw(capi, d, w, b, 1.0, 1.0, 1.0, (s, s), (p, p), (dl, dl),
+                        calib=(-0.05, 0.04), relu=False, force=(cfg, 1))
     ro, rmn, rmx = oracle.quantized_conv(d, w, b, -1.0, 1.0, -1.0, 1.0, -1.0, 1.0, (s, s),
                                          (p, p), (dl, dl))
     np.testing.assert_array_equal(res["out32_nchw"].cpu().numpy(), ro)
     rq, qmn, qmx = oracle.requantize(ro, rmn, rmx, -0.05, 0.04)
     np.testing.assert_array_equal(res["out8_nchw"].cpu().numpy(), rq)
+
+
+# split-K through the convolution kernels: the K slices start in the middle of the
+# (kh, kw, c) walk (C = 16: four taps per 64-byte stage; C = 48: taps straddle stages),
+# stride 2, dilation, K tails, more splits than stages
+@pytest.mark.parametrize("cfg", [11, 12, 13, 14, 15, 16, 22, 23, 24, 25, 31, 32, 33, 34, 35, 36, 37,
+                                 38, 39])
+@pytest.mark.parametrize("case,splits", [((2, 16, 9, 11, 40, 3, 3, 1, 1, 1), 2),
+                                         ((1, 48, 8, 8, 24, 5, 3, 2, 2, 1), 3),
+                                         ((2, 64, 14, 14, 96, 1, 1, 2, 0, 1), 2),
+                                         ((1, 16, 12, 12, 20, 3, 3, 1, 2, 2), 9),
+                                         ((3, 128, 7, 7, 130, 3, 3, 1, 1, 1), 4),
+                                         ((1, 512, 7, 7, 192, 3, 3, 1, 1, 1), 6)])
+def test_conv_split_k(capi, cfg, case, splits):
+    N, C, H, W, O, KH, KW, s, p, dl = case
+    d = int8_uniform((N, C, H, W), seed=cfg + C + 1)
+    w = int8_uniform((O, C, KH, KW), seed=cfg + O + 1)
+    b = int8_uniform((O,), seed=cfg + 1)
+    res = run_conv_nchw(capi, d, w, b, 1.0, 1.0, 1.0, (s, s), (p, p), (dl, dl),
+                        calib=(-0.05, 0.04), relu=True, force=(cfg, splits))
+    ro, rmn, rmx = oracle.quantized_conv(d, w, b, -1.0, 1.0, -1.0, 1.0, -1.0, 1.0, (s, s),
+                                         (p, p), (dl, dl))
+    np.testing.assert_array_equal(res["out32_nchw"].cpu().numpy(), ro)
+    rq, qmn, qmx = oracle.requantize(ro, rmn, rmx, -0.05, 0.04)
+    np.testing.assert_array_equal(res["out8_nchw"].cpu().numpy(), oracle.relu_i8(rq))
 
 
 def test_layout_adapters(capi):
@@ -222,7 +237,7 @@ def test_conv_int32_written_as_nchw(capi, case, use_bias):
     rc = lib.mxq_quantized_conv_nhwc_out_nchw(
         st, P(dn), P(wn), P(bd), N, H, W, C, O, KH, KW, stride, stride, pad, pad, dilate, dilate,
         P(sc[0]), P(sc[1]), P(sc[2]), P(sc[3]), P(sc[4]) if use_bias else None,
-        P(sc[5]) if use_bias else None, P(out), P(omin), P(omax))
+        P(sc[5]) if use_bias else None, P(out), P(omin), P(omax), None, 0)
     assert rc == 0, lib.mxq_last_error()
     ro, rmn, rmx = oracle.quantized_conv(d, w, b, -1.0, 1.0, -0.5, 0.5, -2.0 if use_bias else None,
                                          2.0 if use_bias else None, (stride, stride), (pad, pad),

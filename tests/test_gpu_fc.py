@@ -24,11 +24,13 @@ def f32(v):
     return dev(np.array([v], np.float32))
 
 
-def run_fc(capi, d, w, b, rd, rw, rb, calib=None, relu=False, want_int32=True):
+def run_fc(capi, d, w, b, rd, rw, rb, calib=None, relu=False, want_int32=True, force=None):
+    """force = (cfg, splits, stream_groups) pins the kernel variant through the test-only
+    entry point; None is the operator's own entry point."""
     return capi.quantized_fc(dev(d), dev(w), None if b is None else dev(b), f32(-rd), f32(rd),
                              f32(-rw), f32(rw), None if b is None else f32(-rb),
                              None if b is None else f32(rb), want_int32=want_int32, calib=calib,
-                             relu=relu)
+                             relu=relu, force=force)
 
 
 def oracle_fc(d, w, b, rd, rw, rb):
@@ -67,16 +69,10 @@ def test_fc_every_tile_config(capi, cfg, M, K, N):
         pytest.skip("the global-load direct-to-LDS kernels need K % 64 == 0")
     if cfg > 20 and K % 16 != 0:
         pytest.skip("the buffer-load direct-to-LDS kernels need K % 16 == 0")
-    import mxnet_amd
     d = int8_uniform((M, K), seed=cfg + M)
     w = int8_uniform((N, K), seed=cfg + N + 7)
     b = int8_uniform((N,), seed=cfg)
-    mxnet_amd._lib.set_tuning("fc_config", cfg)
-    try:
-        res = run_fc(capi, d, w, b, 2.0, 0.1, 1.0, calib=(-30.0, 28.0))
-        torch.cuda.synchronize()
-    finally:
-        mxnet_amd._lib.set_tuning("fc_config", 0)
+    res = run_fc(capi, d, w, b, 2.0, 0.1, 1.0, calib=(-30.0, 28.0), force=(cfg, 1, 0))
     ro, rmn, rmx = oracle_fc(d, w, b, 2.0, 0.1, 1.0)
     np.testing.assert_array_equal(res["out32"].cpu().numpy(), ro)
     rq, qmn, qmx = oracle.requantize(ro, rmn, rmx, -30.0, 28.0)
@@ -168,7 +164,6 @@ def test_fc_short_k_streaming_kernel(capi, cfg, M, K, N, relu, use_bias):
     int8 output against requantize(oracle int32), ragged M, one to several column groups."""
     if cfg == 62 and N % 128 != 0:
         pytest.skip("128-column strips need N % 128 == 0")
-    import mxnet_amd
     d = int8_uniform((M, K), seed=cfg + M)
     w = int8_uniform((N, K), seed=K + N, lo=-40, hi=40)
     b = int8_uniform((N,), seed=N) if use_bias else None
@@ -176,12 +171,8 @@ def test_fc_short_k_streaming_kernel(capi, cfg, M, K, N, relu, use_bias):
     ro, rmn, rmx = oracle_fc(d, w, b, rd, rw, rb)
     fl = ro.astype(np.float64) * (float(rmx) / 2147483648.0)
     R = float(np.percentile(np.abs(fl), 98.0))
-    mxnet_amd._lib.set_tuning("fc_config", cfg)
-    try:
-        res = run_fc(capi, d, w, b, rd, rw, rb, calib=(-R, 0.9 * R), relu=relu, want_int32=False)
-        torch.cuda.synchronize()
-    finally:
-        mxnet_amd._lib.set_tuning("fc_config", 0)
+    res = run_fc(capi, d, w, b, rd, rw, rb, calib=(-R, 0.9 * R), relu=relu, want_int32=False,
+                 force=(cfg, 1, 2))
     rq, qmn, qmx = oracle.requantize(ro, rmn, rmx, -R, 0.9 * R)
     if relu:
         rq = oracle.relu_i8(rq)
@@ -193,14 +184,76 @@ def test_fc_short_k_streaming_kernel(capi, cfg, M, K, N, relu, use_bias):
 def test_fc_short_k_streaming_kernel_refuses_other_shapes(capi):
     import mxnet_amd
     d, w = int8_uniform((64, 96), seed=1), int8_uniform((64, 96), seed=2)
-    mxnet_amd._lib.set_tuning("fc_config", 61)
-    try:
-        with pytest.raises(mxnet_amd._lib.MXQError, match="short-K"):
-            run_fc(capi, d, w, None, 1.0, 1.0, 1.0, calib=(-1.0, 1.0), want_int32=False)
-        with pytest.raises(mxnet_amd._lib.MXQError, match="short-K"):   # int32 output wanted
-            run_fc(capi, d[:, :64].copy(), w[:, :64].copy(), None, 1.0, 1.0, 1.0)
-    finally:
-        mxnet_amd._lib.set_tuning("fc_config", 0)
+    with pytest.raises(mxnet_amd._lib.MXQError, match="short-K"):
+        run_fc(capi, d, w, None, 1.0, 1.0, 1.0, calib=(-1.0, 1.0), want_int32=False,
+               force=(61, 1, 2))
+    with pytest.raises(mxnet_amd._lib.MXQError, match="short-K"):   # int32 output wanted
+        run_fc(capi, d[:, :64].copy(), w[:, :64].copy(), None, 1.0, 1.0, 1.0, force=(61, 1, 2))
+
+
+# every direct-to-LDS configuration, split along K over 2 .. 5 work-groups per tile: the
+# int32 sum and the fused int8 output must not depend on the split (integer addition is
+# associative).  Shapes: tile-aligned, ragged M / N, K not a multiple of the stage depth,
+# more splits than K stages (clamped), one stage per split.
+@pytest.mark.parametrize("cfg", [11, 12, 14, 16, 21, 22, 23, 24, 31, 32, 41, 42, 43, 44, 51, 52, 53,
+                                 54, 55, 56, 57, 58, 59])
+@pytest.mark.parametrize("M,K,N,splits", [(512, 1024, 512, 2), (300, 2064, 270, 3),
+                                          (70, 4096, 33, 5), (257, 208, 64, 4),
+                                          (1024, 1536, 520, 4), (64, 128, 64, 2)])
+def test_fc_split_k(capi, cfg, M, K, N, splits):
+    if 10 < cfg < 20 and K % 64 != 0:
+        pytest.skip("the global-load direct-to-LDS kernels need K % 64 == 0")
+    d = int8_uniform((M, K), seed=cfg + M + 1)
+    w = int8_uniform((N, K), seed=cfg + N + 3)
+    b = int8_uniform((N,), seed=cfg + 5)
+    res = run_fc(capi, d, w, b, 2.0, 0.1, 1.0, calib=(-30.0, 28.0), force=(cfg, splits, 0))
+    ro, rmn, rmx = oracle_fc(d, w, b, 2.0, 0.1, 1.0)
+    np.testing.assert_array_equal(res["out32"].cpu().numpy(), ro)
+    rq, qmn, qmx = oracle.requantize(ro, rmn, rmx, -30.0, 28.0)
+    np.testing.assert_array_equal(res["out8"].cpu().numpy(), rq)
+    assert (res["omin"].item(), res["omax"].item()) == (rmn, rmx)
+
+
+def test_fc_split_k_workspace_reuse(capi):
+    """The same workspace handed to split launches of different data back to back: every
+    launch must read the partial sums of its own work-groups, not an earlier launch's
+    (stale lines in another XCD's L2), and clear its own counters."""
+    import ctypes
+    from mxnet_amd._lib import lib, check
+    M, K, N = 640, 3072, 384
+    ws = torch.empty(64 << 20, dtype=torch.uint8, device="cuda")
+    one = [f32(v) for v in (-1.0, 1.0, -0.1, 0.1)]
+    out = torch.empty((M, N), dtype=torch.int32, device="cuda")
+    om = [torch.empty(1, device="cuda") for _ in range(2)]
+    P = lambda t: ctypes.c_void_p(t.data_ptr())
+    st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    for it in range(12):
+        d = int8_uniform((M, K), seed=100 + it)
+        w = int8_uniform((N, K), seed=200 + it)
+        cfg, splits = [(53, 4), (43, 6), (12, 3), (58, 8)][it % 4]
+        dd, wd = dev(d), dev(w)   # kept alive until the result has been read back
+        check(lib.mxq_test_quantized_fc(st, P(dd), P(wd), None, M, N, K, P(one[0]),
+                                        P(one[1]), P(one[2]), P(one[3]), None, None, P(out),
+                                        P(om[0]), P(om[1]), None, None, None, 0, 0.0, 0.0,
+                                        P(ws), ws.numel(), cfg, splits, 0))
+        ro, _, _ = oracle_fc(d, w, None, 1.0, 0.1, 1.0)
+        np.testing.assert_array_equal(out.cpu().numpy(), ro)
+
+
+def test_fc_split_k_needs_workspace(capi):
+    import mxnet_amd
+    d, w = int8_uniform((256, 1024), seed=1), int8_uniform((256, 1024), seed=2)
+    args = [dev(d), dev(w), None, f32(-1.0), f32(1.0), f32(-1.0), f32(1.0)]
+    import ctypes
+    from mxnet_amd._lib import lib
+    out = torch.empty((256, 256), dtype=torch.int32, device="cuda")
+    om = [torch.empty(1, device="cuda") for _ in range(2)]
+    P = lambda t: ctypes.c_void_p(t.data_ptr())
+    rc = lib.mxq_test_quantized_fc(None, P(args[0]), P(args[1]), None, 256, 256, 1024, P(args[3]),
+                                   P(args[4]), P(args[5]), P(args[6]), None, None, P(out),
+                                   P(om[0]), P(om[1]), None, None, None, 0, 0.0, 0.0, None, 0,
+                                   53, 4, 0)
+    assert rc != 0 and "workspace" in mxnet_amd._lib.last_error()
 
 
 def test_fc_degenerate_extents(capi):

@@ -40,9 +40,22 @@ def cast_input(seed):
     return x
 
 
+def laplace_input(seed):
+    """Laplace(0,1) (by inversion) with 0.01 % of the positions at +-50."""
+    g = torch.Generator(device="cuda").manual_seed(seed)
+    u = torch.rand(N_CAST, device="cuda", generator=g) - 0.5
+    x = -torch.sign(u) * torch.log1p(-2.0 * u.abs())
+    del u
+    idx = torch.randint(0, N_CAST, (N_CAST // 10000,), device="cuda", generator=g)
+    sign = torch.randint(0, 2, (N_CAST // 10000,), device="cuda", generator=g) * 2 - 1
+    x[idx] = 50.0 * sign.to(torch.float32)
+    return x
+
+
+@pytest.mark.parametrize("dist", ["normal", "laplace"])
 @pytest.mark.parametrize("calib", [None, (-50.0, 50.0), (-4.0, 4.0)])
-def test_quantize_v2_64m(capi, calib):
-    x = cast_input(1)
+def test_quantize_v2_64m(capi, calib, dist):
+    x = cast_input(1) if dist == "normal" else laplace_input(11)
     kw = {} if calib is None else {"min_calib_range": calib[0], "max_calib_range": calib[1]}
     q, mn, mx = capi.quantize_v2(x, "int8", **kw)
     ref, rmn, rmx = oracle.quantize_v2(x.cpu().numpy(), "int8", *(calib or ()))
@@ -50,11 +63,21 @@ def test_quantize_v2_64m(capi, calib):
     assert np.array_equal(q.cpu().numpy(), ref)
 
 
-def test_quantize_v2_uint8_64m(capi):
-    x = cast_input(2)
-    lo, hi = float(x.min()), float(x.max())
-    q, mn, mx = capi.quantize_v2(x, "uint8", min_calib_range=lo, max_calib_range=hi)
-    ref, rmn, rmx = oracle.quantize_v2(x.cpu().numpy(), "uint8", lo, hi)
+@pytest.mark.parametrize("dist", ["normal", "laplace"])
+@pytest.mark.parametrize("calibrated", [True, False])
+def test_quantize_v2_uint8_64m(capi, calibrated, dist):
+    """fp32 -> uint8 over the data's own range: given as the calibrated range, or found by
+    the on-device min/max reduction (uncalibrated)."""
+    x = cast_input(2) if dist == "normal" else laplace_input(12)
+    xn = x.cpu().numpy()
+    if calibrated:
+        lo, hi = float(x.min()), float(x.max())
+        q, mn, mx = capi.quantize_v2(x, "uint8", min_calib_range=lo, max_calib_range=hi)
+        ref, rmn, rmx = oracle.quantize_v2(xn, "uint8", lo, hi)
+    else:
+        q, mn, mx = capi.quantize_v2(x, "uint8")
+        ref, rmn, rmx = oracle.quantize_v2(xn, "uint8")
+        assert (rmn, rmx) == (float(xn.min()), float(xn.max()))
     assert (mn.item(), mx.item()) == (rmn, rmx)
     assert np.array_equal(q.cpu().numpy(), ref)
 
@@ -120,6 +143,24 @@ def check_fc(capi, M, K, N, seed):
     assert torch.equal(res["out8"], torch.clamp(q, min=0))
     assert (res["rmin"].item(), res["rmax"].item()) == (mn.item(), mx.item())
     assert int(res["out8"].max()) == 127 and 0.2 < float((res["out8"] > 0).float().mean()) < 0.8
+    # ... and the oracle's own chain on the sampled rows: int8 bias rescaled to int32,
+    # exact accumulation, requantize, relu
+    acc_o, omin_o, omax_o = oracle.quantized_fully_connected(
+        d1[rows].cpu().numpy(), w.cpu().numpy(), b.cpu().numpy(), -1.0, 1.0, -1.0, 1.0, -1.0, 1.0)
+    assert np.array_equal(res["out32"][rows].cpu().numpy(), acc_o)
+    assert (res["omin"].item(), res["omax"].item()) == (omin_o, omax_o)
+    q_o, qmn_o, qmx_o = oracle.requantize(acc_o, omin_o, omax_o, -c, c)
+    assert np.array_equal(res["out8"][rows].cpu().numpy(), oracle.relu_i8(q_o))
+    assert (res["rmin"].item(), res["rmax"].item()) == (qmn_o, qmx_o)
+    # the form the benchmark times: int8 output only (no int32 store)
+    fused = capi.quantized_fc(d1, w, b, *args, -one, one, calib=(-c, c), relu=True,
+                              want_int32=False)
+    assert torch.equal(fused["out8"], res["out8"])
+    assert (fused["omin"].item(), fused["omax"].item()) == (omin_o, omax_o)
+
+
+def test_fc_4096(capi):
+    check_fc(capi, 4096, 4096, 4096, seed=4)
 
 
 def test_fc_8192(capi):

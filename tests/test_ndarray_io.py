@@ -102,3 +102,21 @@ def test_malformed_files(tmp_path):
         nd.load(path)
     with pytest.raises(MXNetError, match="cannot open"):
         nd.load(str(tmp_path / "missing.params"))
+
+
+def test_shape_whose_element_count_overflows_is_refused(tmp_path):
+    """A crafted record whose extents multiply to more than 2^64 must not be read into a
+    buffer sized by the wrapped product."""
+    import struct
+    from mxnet_amd import ndarray as nd
+    path = tmp_path / "overflow.params"
+    with open(path, "wb") as f:
+        f.write(struct.pack("<QQQ", 0x112, 0, 1))           # list magic, reserved, one array
+        f.write(struct.pack("<Ii", 0xF993FAC9, 0))           # V2 record, default storage
+        f.write(struct.pack("<i", 3))
+        f.write(struct.pack("<qqq", 1 << 32, 1 << 32, 2))    # 2^65 elements
+        f.write(struct.pack("<iii", 1, 0, 5))                # cpu(0), int8
+        f.write(b"\0" * 16)
+        f.write(struct.pack("<Q", 0))
+    with pytest.raises(Exception, match="overflow"):
+        nd.load(str(path))
