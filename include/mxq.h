@@ -60,6 +60,20 @@ int mxq_quantize_v2(void* stream, const float* in, void* out, float* omin, float
                     size_t n, int out_type, int calibrated, float min_calib, float max_calib,
                     void* workspace, size_t workspace_bytes);
 
+/* mxq_quantize_v2 for callers that cannot allocate (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc) and bring no workspace: the reduction
+ * partials of the uncalibrated path live in a 16 KiB array inside the library's device
+ * image (one copy per GPU, held until the process ends).  It has no counterpart in the
+ * reference, whose operator always draws its temp space from the framework's resource
+ * pool.  Same arguments and results as mxq_quantize_v2 without the workspace; n is
+ * limited to 2^31 elements (a larger n is refused with an error).  The call allocates and
+ * frees nothing.  All calls on one GPU share that GPU's array: calls that overlap in time
+ * on one GPU (different streams) race on it and must be serialised by the caller; calls
+ * on one stream, or on different GPUs, are safe. */
+int mxq_quantize_v2_noalloc(void* stream, const float* in, void* out, float* omin, float* omax,
+                            size_t n, int out_type, int calibrated, float min_calib,
+                            float max_calib);
+
 /* ---- _contrib_quantize (v1) ---------------------------------------------
  * Replaces QuantizeCompute<gpu> (src/operator/quantization/quantize-inl.h:90-131):
  * same kernels, the range arrives as two device scalars. */

@@ -32,6 +32,7 @@ SIGNATURES = {
     "mxq_abi_version": (_i, []),
     "mxq_quantize_v2_workspace": (_sz, [_sz]),
     "mxq_quantize_v2": (_i, [_p, _p, _p, _p, _p, _sz, _i, _i, _f, _f, _p, _sz]),
+    "mxq_quantize_v2_noalloc": (_i, [_p, _p, _p, _p, _p, _sz, _i, _i, _f, _f]),
     "mxq_quantize": (_i, [_p, _p, _p, _p, _p, _p, _p, _sz, _i]),
     "mxq_quantize_v2_passthrough": (_i, [_p, _p, _p, _p, _p, _sz, _i, _i, _f, _f]),
     "mxq_requantize_workspace": (_sz, [_sz]),

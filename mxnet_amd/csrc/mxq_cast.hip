@@ -21,6 +21,7 @@
 // 256 threads per CU (more resident waves lower the achieved HBM bandwidth).
 #include <hip/hip_runtime.h>
 
+#include <atomic>
 #include <cmath>
 #include <cstdint>
 #include <cstring>
@@ -44,6 +45,16 @@ constexpr int kUnroll = 4;             // 16-byte segments in flight per lane
 constexpr int kMaxParts = 1024;
 constexpr int kPartWords = 4;
 constexpr size_t kWsBytes = size_t(kMaxParts) * kPartWords * 4;
+
+// The reduction partials of mxq_quantize_v2_noalloc: library-owned device memory for callers
+// that can neither allocate nor bring a workspace.  Every GPU the library runs on holds its
+// own copy of this array at its own address until the process ends.  In host code the
+// name below is only a handle for hipGetSymbolAddress; kernels are given the address that
+// call returns (cached per device in g_noalloc_ptr).
+static __device__ __align__(256) uint32_t scratch[kMaxParts * kPartWords];
+constexpr int kMaxDevices = 64;
+std::atomic<uint32_t*> g_noalloc_ptr[kMaxDevices];
+constexpr size_t kNoAllocMaxElements = size_t(1) << 31;
 
 __device__ __forceinline__ float maxabs(float a, float b) {
   float x = fabsf(a), y = fabsf(b);
@@ -665,6 +676,22 @@ int reduce_grid(size_t n) {
   return g < kMaxParts ? g : kMaxParts;
 }
 
+// Address of `scratch` on the calling thread's current device; looked up once per device.
+uint32_t* noalloc_scratch() {
+  int dev = 0;
+  MXQ_HIP(hipGetDevice(&dev));
+  MXQ_CHECK(dev >= 0 && dev < kMaxDevices, "device index " << dev << " out of range");
+  uint32_t* p = g_noalloc_ptr[dev].load(std::memory_order_acquire);
+  if (p == nullptr) {
+    void* addr = nullptr;
+    MXQ_HIP(hipGetSymbolAddress(&addr, HIP_SYMBOL(scratch)));
+    MXQ_CHECK(addr != nullptr, "no device address for the scratch array");
+    p = static_cast<uint32_t*>(addr);
+    g_noalloc_ptr[dev].store(p, std::memory_order_release);
+  }
+  return p;
+}
+
 uint32_t* carve(void* workspace, size_t bytes) {
   MXQ_CHECK(workspace != nullptr, "the uncalibrated path needs a workspace");
   MXQ_CHECK(bytes >= kWsBytes, "workspace too small: " << bytes << " < " << kWsBytes);
@@ -731,6 +758,20 @@ int mxq_quantize_v2(void* stream, const float* in, void* out, float* omin, float
     launch_quantize(s, in, out, omin, omax, n, out_type, 0.f, 0.f, nullptr, nullptr, parts,
                     grid);
   }
+  MXQ_API_END();
+}
+
+int mxq_quantize_v2_noalloc(void* stream, const float* in, void* out, float* omin, float* omax,
+                            size_t n, int out_type, int calibrated, float min_calib,
+                            float max_calib) {
+  MXQ_API_BEGIN();
+  MXQ_CHECK(n <= kNoAllocMaxElements,
+            "mxq_quantize_v2_noalloc takes at most " << kNoAllocMaxElements << " elements, got "
+                                                     << n);
+  uint32_t* parts = calibrated ? nullptr : noalloc_scratch();
+  const int rc = mxq_quantize_v2(stream, in, out, omin, omax, n, out_type, calibrated, min_calib,
+                                 max_calib, parts, parts != nullptr ? kWsBytes : 0);
+  if (rc != 0) return rc;
   MXQ_API_END();
 }
 
