@@ -210,28 +210,38 @@ __global__ __launch_bounds__(kThreads) void add_kernel(AddArgs a) {
   size_t done = 0;
   if (a.vec_ok) {
     if (OUT == MXQ_INT32) {
-      // 4 elements per lane: a dword of each operand in, 16 bytes out
+      // Write-dominated (2 bytes in, 4 out): as in the dequantize kernel a wave owns whole
+      // 4 KiB runs of the output; lane l takes the dwords l, l + 64, l + 128, l + 192 of
+      // each operand's 1 KiB and issues four device-scope 16-byte stores back to back,
+      // each instruction writing 1 KiB of consecutive addresses (69.6 -> 66.9 us at 64 M
+      // elements against 16-byte segments a grid-stride apart).
       const size_t nq = a.n >> 2;
       const uint32_t* l4 = reinterpret_cast<const uint32_t*>(a.lhs);
       const uint32_t* r4 = reinterpret_cast<const uint32_t*>(a.rhs);
       i4* o4 = reinterpret_cast<i4*>(a.out);
-      size_t q = t0;
-      for (; q + 3 * stride < nq; q += 4 * stride) {
-        uint32_t x[4], y[4];
+      constexpr int kRun = 256, kPer = kRun / 64, kWaves = kThreads / 64;
+      const size_t runs = nq / kRun;
+      const int lane = threadIdx.x & 63;
+      const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+      for (size_t run = size_t(blockIdx.x) * kWaves + wave; run < runs;
+           run += size_t(gridDim.x) * kWaves) {
+        uint32_t x[kPer], y[kPer];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          x[j] = __builtin_nontemporal_load(l4 + q + j * stride);
-          y[j] = __builtin_nontemporal_load(r4 + q + j * stride);
+        for (int j = 0; j < kPer; ++j) {
+          x[j] = __builtin_nontemporal_load(l4 + run * kRun + j * 64 + lane);
+          y[j] = __builtin_nontemporal_load(r4 + run * kRun + j * 64 + lane);
         }
+        const __amdgpu_buffer_rsrc_t dst =
+            __builtin_amdgcn_make_buffer_rsrc(o4 + run * kRun, 0, kRun * 16, 0x00020000);
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
+        for (int j = 0; j < kPer; ++j) {
           i4 v;
 #pragma unroll
           for (int k = 0; k < 4; ++k) v[k] = r.apply(byte_of<LU>(x[j], k), byte_of<RU>(y[j], k));
-          __builtin_nontemporal_store(v, o4 + q + j * stride);
+          __builtin_amdgcn_raw_buffer_store_b128(v, dst, (j * 64 + lane) * 16, 0, 16 /* sc1 */);
         }
       }
-      for (; q < nq; q += stride) {
+      for (size_t q = runs * kRun + t0; q < nq; q += stride) {
         const uint32_t x = l4[q], y = r4[q];
         i4 v;
 #pragma unroll
