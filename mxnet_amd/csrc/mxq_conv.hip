@@ -239,6 +239,216 @@ __global__ __launch_bounds__(Cfg::kThreads, NS <= 2 ? Cfg::kMinWaves : 1) void c
                                                      static_cast<size_t>(p.O), lds);
 }
 
+// ---- 3 x 3 convolution over 64 channels with the weights parked in LDS --------------
+// A layer like ResNet's 56 x 56, 64 -> 64 has a short reduction (K = 576) and a weight
+// tensor of 36 KB: as an implicit GEMM every tile is prologue and epilogue, and the nine
+// taps re-fetch every input pixel nine times.  Here a work-group of 8 waves parks the whole
+// weight tensor in LDS once; after that one barrier every wave works on its own.  An item
+// is R consecutive output rows of one image: the wave brings their R + 2 input rows (with
+// the zero halo left and right, zero rows above and below the image) into its private LDS
+// patch with buffer loads ... lds, then for each output row runs the 9 taps x 2 k-steps x
+// (2 x 2) MFMAs out of LDS, adds the bias, requantizes and stores the row; the int8 tile is
+// transposed through the patch row that has just become dead.  No barrier per K step,
+// every input row is fetched (R + 2) / R times instead of nine, and with two waves per SIMD
+// one wave's fetch and epilogue overlap the other's MFMAs.  int8 output with the fused
+// requantize only (the form the quantized graph runs with a calibrated convolution);
+// everything else takes the tiled kernels.
+constexpr int kRowsC = 64;        // input channels = bytes per pixel
+constexpr int kRowsO = 64;        // output channels
+constexpr int kRowsPitch = 60;    // patch pixels per row
+constexpr int kRowsMaxW = kRowsPitch - 2;
+constexpr int kRowsWaves = 8;
+
+// (row & 3) ^ (row >> 2 & 3): spreads the 16-byte pieces of the transposed int8 tile (row
+// pitch 64 bytes) over the banks for the column-wise writes and the row-wise reads alike
+__device__ __forceinline__ int tile_swz(int row) { return (row ^ (row >> 2)) & 3; }
+
+template <int R>
+__global__ __launch_bounds__(64 * kRowsWaves, 1) void conv3x3_rows_kernel(ConvArgs p) {
+  constexpr int CH = kRowsC / 16;                       // 16-byte chunks per pixel
+  constexpr int kPatchPixels = (R + 2) * kRowsPitch;
+  constexpr int kFetches = (kPatchPixels + 15) / 16;    // buffer loads of 16 pixels each
+  __shared__ __attribute__((aligned(16))) v4i wl[9 * kRowsO * CH];               // 36 KB
+  __shared__ __attribute__((aligned(16))) v4i patch_all[kRowsWaves * kPatchPixels * CH];
+  __shared__ __attribute__((aligned(16))) int sbias[kRowsO];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  v4i* patch = patch_all + wave * kPatchPixels * CH;
+  const uint32_t patch_addr = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(patch));
+  const v4i rsrc = make_rsrc(p.data, static_cast<uint32_t>(p.N) * p.H * p.W * kRowsC);
+  const int chunks_per_image = (p.OH + R - 1) / R;
+  const int items = p.N * chunks_per_image;
+  // lane geometry of the fetches: flat patch pixel 16 * j + lane / 4, chunk slot lane % 4
+  auto fetch = [&](int item) {
+    const int n = item / chunks_per_image, oh0 = (item - n * chunks_per_image) * R;
+#pragma unroll
+    for (int j = 0; j < kFetches; ++j) {
+      const int flat = 16 * j + (lane >> 2);
+      const int row = flat / kRowsPitch, px = flat - row * kRowsPitch;
+      const int ih = oh0 + row - 1, iw = px - 1;
+      const int chunk = (lane & 3) ^ swz<CH>(px);
+      const bool ok = static_cast<unsigned>(ih) < static_cast<unsigned>(p.H) &&
+                      static_cast<unsigned>(iw) < static_cast<unsigned>(p.W);
+      const uint32_t off =
+          ok ? static_cast<uint32_t>(((n * p.H + ih) * p.W + iw) * kRowsC + chunk * 16)
+             : kOutOfRange;
+      if (flat < kPatchPixels) dma_buffer(patch_addr + j * 1024, off, rsrc);
+    }
+  };
+  int item = blockIdx.x * kRowsWaves + wave;
+  if (item < items) fetch(item);  // on its way while the weights are staged
+
+  // weights [o][tap][c] -> LDS [tap][o][chunk ^ swz(o)], straight into LDS as well: fetch
+  // j fills the 16 rows (tap, o) = 16 * j ... + 15, lane / 4 the row, lane % 4 the slot
+  {
+    const v4i wrsrc = make_rsrc(p.weight, 9 * kRowsO * kRowsC);
+    const uint32_t wl_addr = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(wl));
+    constexpr int kWeightFetches = 9 * kRowsO / 16;  // 36
+    for (int j = wave; j < kWeightFetches; j += kRowsWaves) {
+      const int row = 16 * j + (lane >> 2);
+      const int t = row / kRowsO, o = row - t * kRowsO;
+      const int chunk = (lane & 3) ^ swz<CH>(o);
+      dma_buffer(wl_addr + j * 1024, static_cast<uint32_t>((o * 9 + t) * kRowsC + chunk * 16),
+                 wrsrc);
+    }
+  }
+  const EpiScalars s = epi_scalars(p.epi);
+  if (tid < kRowsO) sbias[tid] = epi_bias32(p.epi, s, tid);
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+
+  const int lrow = lane & 31, lgrp = lane >> 5;
+  const bool relu = p.epi.relu != 0;
+  // patch pixel of output column mi * 32 + lrow under tap column kw; columns past the row
+  // (their results are never stored) are kept inside it
+  int apx[2][3];
+#pragma unroll
+  for (int mi = 0; mi < 2; ++mi)
+#pragma unroll
+    for (int kw = 0; kw < 3; ++kw) {
+      const int px = mi * 32 + lrow + kw;
+      apx[mi][kw] = px < kRowsPitch ? px : kRowsPitch - 1;
+    }
+  for (; item < items; item += gridDim.x * kRowsWaves) {
+    const int n = item / chunks_per_image, oh0 = (item - n * chunks_per_image) * R;
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      if (oh0 + r >= p.OH) break;
+      v16i acc[2][2];
+#pragma unroll
+      for (int mi = 0; mi < 2; ++mi)
+#pragma unroll
+        for (int ni = 0; ni < 2; ++ni)
+#pragma unroll
+          for (int v = 0; v < 16; ++v) acc[mi][ni][v] = 0;
+#pragma unroll
+      for (int kh = 0; kh < 3; ++kh)
+#pragma unroll
+        for (int kw = 0; kw < 3; ++kw)
+#pragma unroll
+          for (int ks = 0; ks < 2; ++ks) {
+            v4i fa[2], fb[2];
+#pragma unroll
+            for (int mi = 0; mi < 2; ++mi) {
+              const int px = apx[mi][kw];
+              fa[mi] = patch[((r + kh) * kRowsPitch + px) * CH + ((ks * 2 + lgrp) ^ swz<CH>(px))];
+            }
+#pragma unroll
+            for (int ni = 0; ni < 2; ++ni)
+              fb[ni] = wl[((kh * 3 + kw) * kRowsO + ni * 32 + lrow) * CH +
+                          ((ks * 2 + lgrp) ^ swz<CH>(lrow))];
+#pragma unroll
+            for (int mi = 0; mi < 2; ++mi)
+#pragma unroll
+              for (int ni = 0; ni < 2; ++ni)
+                acc[mi][ni] =
+                    __builtin_amdgcn_mfma_i32_32x32x32_i8(fb[ni], fa[mi], acc[mi][ni], 0, 0, 0);
+          }
+      // patch row r is dead now (output row r + 1 starts at patch row r + 1): the int8 tile
+      // of up to 58 pixels x 64 channels is transposed through it, 64 bytes per pixel
+      char* stage = reinterpret_cast<char*>(patch + r * kRowsPitch * CH);
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+      __builtin_amdgcn_wave_barrier();
+      auto requantize_tile = [&](auto with_relu) {
+#pragma unroll
+        for (int mi = 0; mi < 2; ++mi) {
+          const int px = mi * 32 + lrow;
+#pragma unroll
+          for (int ni = 0; ni < 2; ++ni)
+#pragma unroll
+            for (int vq = 0; vq < 4; ++vq) {
+              const int nl = ni * 32 + 8 * vq + 4 * lgrp;
+              const v4i b = *reinterpret_cast<const v4i*>(sbias + nl);
+              int q[4];
+#pragma unroll
+              for (int i = 0; i < 4; ++i) {
+                const int v = static_cast<int>(static_cast<uint32_t>(acc[mi][ni][4 * vq + i]) +
+                                               static_cast<uint32_t>(b[i]));
+                q[i] = decltype(with_relu)::value ? epi_requant_relu(v, s)
+                                                  : epi_requant(v, s, -127.0f);
+              }
+              if (px < p.OW)
+                *reinterpret_cast<uint32_t*>(stage + px * kRowsO +
+                                             (((nl >> 4) ^ tile_swz(px)) << 4) + (nl & 15)) =
+                    pack_bytes(q[0], q[1], q[2], q[3]);
+            }
+        }
+      };
+      if (relu)
+        requantize_tile(std::true_type());
+      else
+        requantize_tile(std::false_type());
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+      __builtin_amdgcn_wave_barrier();
+      int8_t* orow = p.epi.out8 +
+                     (static_cast<size_t>(n) * p.OH + oh0 + r) * p.OW * kRowsO;
+#pragma unroll
+      for (int it = 0; it < 4; ++it) {
+        const int px = it * 16 + (lane >> 2), c16 = lane & 3;
+        if (px < p.OW) {
+          const v4i val =
+              *reinterpret_cast<const v4i*>(stage + px * kRowsO + ((c16 ^ tile_swz(px)) << 4));
+          *reinterpret_cast<v4i*>(orow + px * kRowsO + c16 * 16) = val;
+        }
+      }
+    }
+    // the next item's fetches overwrite the patch: every LDS read above must have returned
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_wave_barrier();
+    const int next = item + gridDim.x * kRowsWaves;
+    if (next < items) fetch(next);
+  }
+  if (blockIdx.x == 0 && threadIdx.x == 0) epilogue_ranges(p.epi);
+}
+
+bool conv3x3_rows_ok(const ConvArgs& a) {
+  const long long data_bytes = static_cast<long long>(a.N) * a.H * a.W * a.C;
+  return a.KH == 3 && a.KW == 3 && a.sh == 1 && a.sw == 1 && a.ph == 1 && a.pw == 1 &&
+         a.dh == 1 && a.dw == 1 && a.C == kRowsC && a.O == kRowsO && a.W <= kRowsMaxW &&
+         a.epi.out32 == nullptr && a.epi.out8 != nullptr && aligned16(a.data) &&
+         aligned16(a.weight) && aligned16(a.epi.out8) && data_bytes < (1LL << 31);
+}
+
+void launch_conv3x3_rows(hipStream_t s, const ConvArgs& a) {
+  const long cus = num_cus();
+  // two output rows per item once that still gives most waves of the chip an item: a third
+  // fewer input rows to fetch per output row
+  const long items2 = static_cast<long>(a.N) * ((a.OH + 1) / 2);
+  const bool two = 5 * items2 >= 3 * kRowsWaves * cus;
+  const long items = two ? items2 : static_cast<long>(a.N) * a.OH;
+  long grid = (items + kRowsWaves - 1) / kRowsWaves;
+  if (grid > cus) grid = cus;
+  if (two)
+    hipLaunchKernelGGL(conv3x3_rows_kernel<2>, dim3(static_cast<unsigned>(grid)),
+                       dim3(64 * kRowsWaves), 0, s, a);
+  else
+    hipLaunchKernelGGL(conv3x3_rows_kernel<1>, dim3(static_cast<unsigned>(grid)),
+                       dim3(64 * kRowsWaves), 0, s, a);
+  MXQ_LAUNCH_CHECK();
+}
+
 typedef GemmCfg<256, 256, 64, 2, 4> CfgL8;   // 8 waves, wave tile 128 x 64
 typedef GemmCfg<256, 128, 64, 4, 2> CfgW128; // 8 waves, wave tile 64 x 64
 typedef GemmCfg<256, 64, 64, 4, 1> CfgW64;   // 4 waves, wave tile 64 x 64
@@ -563,6 +773,15 @@ void conv_nhwc(void* stream, const int8_t* data, const int8_t* weight, const int
     GemmForce unsplit = force;
     unsplit.splits = 1;
     plan = plan_conv(g, aligned, unsplit);
+  }
+  // 61: the parked-weights row kernel (3 x 3 over 64 -> 64 channels, fused int8 output);
+  // chosen for it whenever the launch has rows for every wave of the chip
+  if (plan.cfg == 61 || (force.cfg == 0 && conv3x3_rows_ok(a) &&
+                         static_cast<long>(a.N) * a.OH >= 1L * kRowsWaves * num_cus())) {
+    MXQ_CHECK(conv3x3_rows_ok(a), "shape does not qualify for the parked-weights 3x3 kernel");
+    MXQ_CHECK(plan.splits <= 1 || force.splits == 0, "the 3x3 row kernel has no split-K form");
+    launch_conv3x3_rows(s, a);
+    return;
   }
   const int cfg = plan.cfg, sp = plan.splits;
   if (cfg > 10) MXQ_CHECK(dma_ok, "shape does not qualify for the direct-to-LDS conv kernels");

@@ -25,15 +25,17 @@ def f32(v):
 
 
 def run_conv_nchw(capi, d, w, b, rd, rw, rb, stride, pad, dilate, calib=None, relu=False,
-                  force=None):
+                  force=None, want_int32=True):
     """force = (cfg, splits) pins the kernel variant through the test-only entry point."""
     dn = capi.nchw_to_nhwc_i8(dev(d))
     wn = capi.nchw_to_nhwc_i8(dev(w))
     res = capi.quantized_conv_nhwc(dn, wn, None if b is None else dev(b), f32(-rd), f32(rd),
                                    f32(-rw), f32(rw), None if b is None else f32(-rb),
                                    None if b is None else f32(rb), stride=stride, pad=pad,
-                                   dilate=dilate, calib=calib, relu=relu, force=force)
-    res["out32_nchw"] = capi.nhwc_to_nchw(res["out32"])
+                                   dilate=dilate, calib=calib, relu=relu, force=force,
+                                   want_int32=want_int32)
+    if want_int32:
+        res["out32_nchw"] = capi.nhwc_to_nchw(res["out32"])
     if res["out8"] is not None:
         res["out8_nchw"] = capi.nhwc_to_nchw(res["out8"])
     return res
@@ -132,6 +134,41 @@ def test_conv_split_k(capi, cfg, case, splits):
     np.testing.assert_array_equal(res["out32_nchw"].cpu().numpy(), ro)
     rq, qmn, qmx = oracle.requantize(ro, rmn, rmx, -0.05, 0.04)
     np.testing.assert_array_equal(res["out8_nchw"].cpu().numpy(), oracle.relu_i8(rq))
+
+
+# the parked-weights 3 x 3 kernel (64 -> 64 channels, one output row per wave item): odd
+# extents, a single column, the widest row it takes, rows shorter than one MFMA block, more
+# rows than waves, with and without bias and relu
+@pytest.mark.parametrize("N,H,W", [(2, 56, 56), (3, 7, 9), (1, 5, 58), (2, 13, 1), (5, 3, 33),
+                                   (1, 1, 1), (70, 6, 31), (6, 56, 56), (24, 7, 40)])
+@pytest.mark.parametrize("relu,use_bias", [(True, True), (False, True), (True, False)])
+@pytest.mark.parametrize("forced", [True, False])
+def test_conv3x3_parked_weights(capi, N, H, W, relu, use_bias, forced):
+    d = int8_uniform((N, 64, H, W), seed=N + H + W)
+    w = int8_uniform((64, 64, 3, 3), seed=H + 1, lo=-50, hi=50)
+    b = int8_uniform((64,), seed=W + 2) if use_bias else None
+    ro, rmn, rmx = oracle.quantized_conv(d, w, b, -1.0, 1.0, -1.0, 1.0,
+                                         -1.0 if use_bias else None, 1.0 if use_bias else None,
+                                         (1, 1), (1, 1), (1, 1))
+    fl = ro.astype(np.float64) * (float(rmx) / 2147483648.0)
+    R = float(np.percentile(np.abs(fl), 98.0)) or 1.0
+    res = run_conv_nchw(capi, d, w, b, 1.0, 1.0, 1.0, (1, 1), (1, 1), (1, 1), calib=(-R, 0.9 * R),
+                        relu=relu, force=(61, 1) if forced else None, want_int32=False)
+    rq, qmn, qmx = oracle.requantize(ro, rmn, rmx, -R, 0.9 * R)
+    if relu:
+        rq = oracle.relu_i8(rq)
+    np.testing.assert_array_equal(res["out8_nchw"].cpu().numpy(), rq)
+    assert (res["omin"].item(), res["omax"].item()) == (rmn, rmx)
+    assert (res["rmin"].item(), res["rmax"].item()) == (qmn, qmx)
+
+
+def test_conv3x3_parked_weights_refuses_other_shapes(capi):
+    import mxnet_amd
+    d = int8_uniform((1, 32, 8, 8), seed=1)
+    w = int8_uniform((64, 32, 3, 3), seed=2)
+    with pytest.raises(mxnet_amd._lib.MXQError, match="parked-weights"):
+        run_conv_nchw(capi, d, w, None, 1.0, 1.0, 1.0, (1, 1), (1, 1), (1, 1), calib=(-1.0, 1.0),
+                      force=(61, 1), want_int32=False)
 
 
 def test_layout_adapters(capi):
