@@ -684,6 +684,7 @@ ConvPlan plan_conv(const ConvGeometry& g, bool aligned, const GemmForce& force) 
         case Tile::kR128K2: plan.cfg = 37; break;
         case Tile::kQ128K2: plan.cfg = 38; break;
         case Tile::kS64K4: plan.cfg = 39; break;
+        case Tile::kW192K2: plan.cfg = 11; break;  // not proposed for gathered operands
       }
     } else if (O > 128 && tiles(256, 256) >= cus) {
       plan.cfg = 1;

@@ -110,6 +110,7 @@ typedef GemmCfg<64, 64, 128, 2, 2> CfgSK;      // 4 waves, wave tile 32 x 32
 typedef GemmCfg<128, 64, 128, 2, 2> CfgRK;     // 4 waves, wave tile 64 x 32
 typedef GemmCfg<64, 128, 128, 2, 2> CfgQK;     // 4 waves, wave tile 32 x 64
 typedef GemmCfg<64, 64, 256, 2, 2> CfgSK2;     // 256-byte stages for very long K
+typedef GemmCfg<256, 192, 128, 4, 2> CfgW192K; // 8 waves, wave tile 64 x 96
 
 // Short-K form (K = 32, 64, 128 or 256; int8 output only).  With one or two K steps a tile of
 // the kernels above is all prologue and epilogue: a round of DMA latency, two barriers, and
@@ -272,6 +273,7 @@ void launch_cfg(hipStream_t s, const FcArgs& a, bool aligned) {
 //   41..44  as 21..24 with a 2-stage ring (short K)
 //   51..56  128-byte stages: 64x64 (2, 3 stages), 128x128 (2, 3), 256x256 (2), 256x128 (2)
 //   57..59  128x64 and 64x128 with 128-byte stages, 64x64 with 256-byte stages
+//   60      256x192 with 128-byte stages (outputs whose width is a multiple of 192)
 //   61, 62  the short-K streaming kernel with 64- / 128-column strips
 // Output tile of a direct-to-LDS configuration (what a split-K work-group leaves in the
 // workspace); false for every other configuration.
@@ -284,6 +286,7 @@ bool fc_cfg_tile(int cfg, int& bm, int& bn) {
     case 24: case 44: case 51: case 52: case 59: bm = 64; bn = 64; return true;
     case 57: bm = 128; bn = 64; return true;
     case 58: bm = 64; bn = 128; return true;
+    case 60: bm = 256; bn = 192; return true;
     default: return false;
   }
 }
@@ -321,6 +324,7 @@ FcPlan plan_fc(int M, int N, int K, bool aligned, bool fused8, const GemmForce& 
         case Tile::kR128K2: plan.cfg = 57; break;
         case Tile::kQ128K2: plan.cfg = 58; break;
         case Tile::kS64K4: plan.cfg = 59; break;
+        case Tile::kW192K2: plan.cfg = 60; break;
       }
     } else {
       if (tiles(256, 256) >= cus)
@@ -442,6 +446,7 @@ void launch_fc(hipStream_t s, const int8_t* data, const int8_t* weight, int M, i
     case 57: launch_dma<CfgRK, 2, 0, true>(s, a, sp, ws); break;
     case 58: launch_dma<CfgQK, 2, 0, true>(s, a, sp, ws); break;
     case 59: launch_dma<CfgSK2, 2, 0, true>(s, a, sp, ws); break;
+    case 60: launch_dma<CfgW192K, 2, 0, true>(s, a, sp, ws); break;
     case 31: launch_dma<CfgL8, 4, 2, true>(s, a, sp, ws); break;
     case 32: launch_dma<CfgL4, 4, 2, true>(s, a, sp, ws); break;
     default: MXQ_CHECK(false, "unknown fc tile configuration " << cfg);

@@ -899,9 +899,15 @@ __device__ __forceinline__ void gemm_epilogue_lds(v16i (&acc)[Cfg::MI][Cfg::NI],
     // instructions in order, the wait makes the writes complete first
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     __builtin_amdgcn_wave_barrier();
+    // 16-byte pieces of the staged tile in row-major order, 64 per store instruction (a
+    // wave tile of 96 columns has 6 pieces per row: the last instruction is then partial)
+    constexpr int kPieces = TM * LPR;
 #pragma unroll
-    for (int it = 0; it < TM / RPI; ++it) {
-      const int rr = it * RPI + lane / LPR, c16 = lane % LPR;
+    for (int it = 0; it < (kPieces + 63) / 64; ++it) {
+      const int piece = it * 64 + lane;
+      const int rr = (64 % LPR == 0) ? it * RPI + lane / LPR : piece / LPR;
+      const int c16 = (64 % LPR == 0) ? lane % LPR : piece - rr * LPR;
+      if (kPieces % 64 != 0 && piece >= kPieces) continue;
       const v4i val = *reinterpret_cast<const v4i*>(stage + rr * LD + c16 * 16);
       const int m = m_base + rr, n = n_base + c16 * 16;
       if (m < M && n < N)

@@ -60,7 +60,7 @@ def test_fc_int32(capi, M, K, N, use_bias):
 
 
 @pytest.mark.parametrize("cfg", [1, 2, 3, 4, 11, 12, 14, 16, 21, 22, 23, 24, 31, 32, 41, 42, 43, 44,
-                                 51, 52, 53, 54, 55, 56, 57, 58, 59])
+                                 51, 52, 53, 54, 55, 56, 57, 58, 59, 60])
 @pytest.mark.parametrize("M,K,N", [(512, 512, 512), (300, 208, 270), (70, 444, 33),
                                    (300, 192, 270), (1, 64, 1), (1024, 1024, 520),
                                    (130, 16, 70), (257, 80, 64)])
@@ -196,7 +196,7 @@ def test_fc_short_k_streaming_kernel_refuses_other_shapes(capi):
 # associative).  Shapes: tile-aligned, ragged M / N, K not a multiple of the stage depth,
 # more splits than K stages (clamped), one stage per split.
 @pytest.mark.parametrize("cfg", [11, 12, 14, 16, 21, 22, 23, 24, 31, 32, 41, 42, 43, 44, 51, 52, 53,
-                                 54, 55, 56, 57, 58, 59])
+                                 54, 55, 56, 57, 58, 59, 60])
 @pytest.mark.parametrize("M,K,N,splits", [(512, 1024, 512, 2), (300, 2064, 270, 3),
                                           (70, 4096, 33, 5), (257, 208, 64, 4),
                                           (1024, 1536, 520, 4), (64, 128, 64, 2)])
