@@ -118,7 +118,7 @@ def quantized_fc(data, weight, bias, min_data, max_data, min_weight, max_weight,
         check(lib.mxq_quantized_fc(*args, _ptr(ws), wsb))
     else:
         cfg, splits, groups = force
-        wsb = _SPLIT_WS_BYTES if splits != 1 else 0
+        wsb = _SPLIT_WS_BYTES if splits > 1 else 0
         ws = _workspace(wsb, dev) if wsb else None
         check(lib.mxq_test_quantized_fc(*args, _ptr(ws), wsb, cfg, splits, groups))
     res.update(out32=out32, out8=out8, rmin=rmin, rmax=rmax)
@@ -155,7 +155,7 @@ def quantized_conv_nhwc(data, weight, bias, min_data, max_data, min_weight, max_
         check(lib.mxq_quantized_conv_nhwc(*args, _ptr(ws), wsb))
     else:
         cfg, splits = force
-        wsb = _SPLIT_WS_BYTES if splits != 1 else 0
+        wsb = _SPLIT_WS_BYTES if splits > 1 else 0
         ws = _workspace(wsb, dev) if wsb else None
         check(lib.mxq_test_quantized_conv_nhwc(*args, _ptr(ws), wsb, cfg, splits))
     res.update(out32=out32, out8=out8, rmin=rmin, rmax=rmax)

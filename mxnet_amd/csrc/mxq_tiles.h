@@ -65,7 +65,24 @@ inline Tile choose_tile(long M, long N, long K, long cus, bool gather = false,
       4 * tiles(256, 192) >= 3 * cus && tiles(256, 192) > tiles(256, 256))
     return Tile::kW192K2;
   if (K > 256 && N > 128 && 16 * tiles(256, 256) >= 9 * cus) return Tile::kL8;
-  if (N <= 64) return (K >= 4096) ? Tile::kS64x4 : Tile::kS64x2;
+  // Split-K: an output of few 64 x 64 tiles under a very long reduction (a fully-connected
+  // layer at small batch: 256 x 8192 -> 800, 64 x 25088 -> 4096) leaves most CUs idle and
+  // each tile walks thousands of K bytes alone.  Up to four work-groups share a tile then
+  // (18.3 -> 12.9 us and 63.5 -> 27 us on those two).  The price is a counter-clearing
+  // launch and the partial sums' round trip through memory (about 2 us plus 1 us per 4 MB),
+  // which is why shapes with more tiles or a shorter K are left alone: on the ResNet-50 and
+  // BERT layers every split measured slower than the unsplit kernel.
+  auto few_tile_splits = [&]() {
+    const long t = tiles(64, 64);
+    if (splits == nullptr || K < 8192 || 2 * t > cus) return;
+    long sp = cus / t;
+    if (sp > 4) sp = 4;
+    if (sp >= 2) *splits = static_cast<int>(sp);
+  };
+  if (N <= 64) {
+    if (K >= 4096) few_tile_splits();
+    return (K >= 4096) ? Tile::kS64x4 : Tile::kS64x2;
+  }
   if (4 * tiles(256, 128) >= 3 * cus) return (K >= 512) ? Tile::kW128K2 : Tile::kW128x2;
   if (tiles(128, 128) >= cus) return (K >= 256) ? Tile::kM128K2 : Tile::kM128x2;
   if (K < 512) return Tile::kS64x2;
@@ -82,6 +99,7 @@ inline Tile choose_tile(long M, long N, long K, long cus, bool gather = false,
   }
   // 256-byte stages once K is long enough to leave them several steps (3136 x 4608 -> 512:
   // 15.8 us against 19.8 us)
+  if (K >= 4096) few_tile_splits();
   return (K >= 4096) ? Tile::kS64K4 : Tile::kS64K2;
 }
 

@@ -240,6 +240,24 @@ def test_fc_split_k_workspace_reuse(capi):
         np.testing.assert_array_equal(out.cpu().numpy(), ro)
 
 
+def test_fc_split_is_chosen_for_few_tiles_and_long_k(capi):
+    """The launcher's own choice: the reference's small-batch test shape (256 x 8192 -> 800)
+    asks for a split-K workspace and gives the oracle's result with it and without it; the
+    square and BERT shapes ask for none."""
+    from mxnet_amd._lib import lib
+    assert lib.mxq_quantized_fc_workspace(256, 800, 8192, 0) > 0
+    assert lib.mxq_quantized_fc_workspace(4096, 4096, 4096, 1) == 0
+    assert lib.mxq_quantized_fc_workspace(4096, 2304, 768, 1) == 0
+    d = int8_uniform((256, 8192), seed=5)
+    w = int8_uniform((800, 8192), seed=6)
+    b = int8_uniform((800,), seed=7)
+    ro, rmn, rmx = oracle_fc(d, w, b, 1.0, 0.08, 0.5)
+    res = run_fc(capi, d, w, b, 1.0, 0.08, 0.5)                 # with the workspace
+    np.testing.assert_array_equal(res["out32"].cpu().numpy(), ro)
+    res = run_fc(capi, d, w, b, 1.0, 0.08, 0.5, force=(0, 0, 0))  # chooser, no workspace
+    np.testing.assert_array_equal(res["out32"].cpu().numpy(), ro)
+
+
 def test_fc_split_k_needs_workspace(capi):
     import mxnet_amd
     d, w = int8_uniform((256, 1024), seed=1), int8_uniform((256, 1024), seed=2)
