@@ -97,10 +97,14 @@ inline Tile choose_tile(long M, long N, long K, long cus, bool gather = false,
     if (q_fits && (gather || !r_fits)) return Tile::kQ128K2;
     return r_fits ? Tile::kR128K2 : Tile::kQ128K2;
   }
-  // 256-byte stages once K is long enough to leave them several steps (3136 x 4608 -> 512:
-  // 15.8 us against 19.8 us)
+  // Fewer than two 64 x 64 tiles per CU are left: 256-byte stages once K leaves them four
+  // steps (3136 x 4608 -> 512: 15.8 us against 19.8 us).  With so few work-groups per CU a
+  // deeper stage is what keeps bytes in flight, which counts most when the operands come
+  // from HBM: inside the 19-layer ResNet stack (every layer reads operands last touched
+  // 300 us earlier) 3136 x 2048 -> 512 is 3.6 us and the strided 3136 x 1024 -> 512 2.4 us
+  // faster this way, and level with 128-byte stages when the operands are cache-warm.
   if (K >= 4096) few_tile_splits();
-  return (K >= 4096) ? Tile::kS64K4 : Tile::kS64K2;
+  return (K >= 1024) ? Tile::kS64K4 : Tile::kS64K2;
 }
 
 }  // namespace mxq
