@@ -336,13 +336,19 @@ __global__ __launch_bounds__(64 * kRowsWaves, 1) void conv3x3_rows_kernel(ConvAr
 #pragma unroll
     for (int r = 0; r < R; ++r) {
       if (oh0 + r >= p.OH) break;
+      // accumulators start at the int32 bias of their columns, read from LDS straight into
+      // the registers the MFMAs add to: no bias add in the epilogue
       v16i acc[2][2];
 #pragma unroll
-      for (int mi = 0; mi < 2; ++mi)
+      for (int ni = 0; ni < 2; ++ni)
 #pragma unroll
-        for (int ni = 0; ni < 2; ++ni)
+        for (int vq = 0; vq < 4; ++vq) {
+          const v4i b = *reinterpret_cast<const v4i*>(sbias + ni * 32 + 8 * vq + 4 * lgrp);
 #pragma unroll
-          for (int v = 0; v < 16; ++v) acc[mi][ni][v] = 0;
+          for (int mi = 0; mi < 2; ++mi)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) acc[mi][ni][4 * vq + i] = b[i];
+        }
 #pragma unroll
       for (int kh = 0; kh < 3; ++kh)
 #pragma unroll
@@ -380,12 +386,10 @@ __global__ __launch_bounds__(64 * kRowsWaves, 1) void conv3x3_rows_kernel(ConvAr
 #pragma unroll
             for (int vq = 0; vq < 4; ++vq) {
               const int nl = ni * 32 + 8 * vq + 4 * lgrp;
-              const v4i b = *reinterpret_cast<const v4i*>(sbias + nl);
               int q[4];
 #pragma unroll
               for (int i = 0; i < 4; ++i) {
-                const int v = static_cast<int>(static_cast<uint32_t>(acc[mi][ni][4 * vq + i]) +
-                                               static_cast<uint32_t>(b[i]));
+                const int v = acc[mi][ni][4 * vq + i];
                 q[i] = decltype(with_relu)::value ? epi_requant_relu(v, s)
                                                   : epi_requant(v, s, -127.0f);
               }

@@ -169,11 +169,17 @@ __global__ __launch_bounds__(256, 2) void fc_stream_kernel(FcArgs p, int bn, int
     const int tile = item / strips;
     const int s0 = (item - tile * strips) * TN;  // first column of the strip inside the group's
     const int m_base = tile * 32;
+    // the accumulators start at the int32 bias of their columns (read from LDS straight
+    // into the registers the MFMAs add to): the epilogue has no bias add left
     v16i acc[NI];
 #pragma unroll
     for (int ni = 0; ni < NI; ++ni)
 #pragma unroll
-      for (int v = 0; v < 16; ++v) acc[ni][v] = 0;
+      for (int vq = 0; vq < 4; ++vq) {
+        const v4i b = *reinterpret_cast<const v4i*>(sbias + s0 + ni * 32 + 8 * vq + 4 * lgrp);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc[ni][4 * vq + i] = b[i];
+      }
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks)
 #pragma unroll
@@ -188,12 +194,10 @@ __global__ __launch_bounds__(256, 2) void fc_stream_kernel(FcArgs p, int bn, int
 #pragma unroll
         for (int vq = 0; vq < 4; ++vq) {
           const int nl = ni * 32 + 8 * vq + 4 * lgrp;
-          const v4i b = *reinterpret_cast<const v4i*>(sbias + s0 + nl);
           int q[4];
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
-            const int v = static_cast<int>(static_cast<uint32_t>(acc[ni][4 * vq + i]) +
-                                           static_cast<uint32_t>(b[i]));
+            const int v = acc[ni][4 * vq + i];
             q[i] = decltype(with_relu)::value ? epi_requant_relu(v, s) : epi_requant(v, s, -127.0f);
           }
           *reinterpret_cast<uint32_t*>(stage + lrow * LD + nl) = pack_bytes(q[0], q[1], q[2], q[3]);
