@@ -1,0 +1,119 @@
+"""Seeded random shapes through the operators' own entry points (the launcher chooses the
+kernel): every route the tile chooser can take for small and mid-size problems, with ragged
+extents, K tails, stride / pad / dilation mixes, against the CPU oracle bit for bit."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from tests.data_gen import int8_uniform
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def capi():
+    import mxnet_amd
+    return mxnet_amd.capi
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def f32(v):
+    return dev(np.array([v], np.float32))
+
+
+def fc_shapes():
+    rng = np.random.default_rng(20240611)
+    shapes = []
+    for _ in range(60):
+        M = int(rng.integers(1, 700))
+        N = int(rng.integers(1, 700))
+        K = int(rng.choice([rng.integers(1, 300), 16 * rng.integers(1, 40), 64 * rng.integers(1, 24)]))
+        shapes.append((M, N, K))
+    # chooser corner cases: widths that are multiples of 192, tall and narrow, few tiles
+    # under a long K (split-K with the workspace the entry point asks for), one row
+    shapes += [(512, 384, 512), (300, 192, 1024), (2048, 64, 64), (4100, 128, 128),
+               (64, 320, 8192), (40, 130, 9000), (1, 1000, 4096), (700, 1, 48)]
+    return shapes
+
+
+@pytest.mark.parametrize("M,N,K", fc_shapes())
+def test_fc_random_shape(capi, M, N, K):
+    d = int8_uniform((M, K), seed=M * 7 + K)
+    w = int8_uniform((N, K), seed=N * 5 + K + 1)
+    b = int8_uniform((N,), seed=N + 3) if (M + N + K) % 3 else None
+    rd, rw, rb = 1.5, 0.2, 0.7
+    relu = bool((M + K) % 2)
+    ro, rmn, rmx = oracle.quantized_fully_connected(d, w, b, -rd, rd, -rw, rw,
+                                                    None if b is None else -rb,
+                                                    None if b is None else rb)
+    fl = ro.astype(np.float64) * (float(rmx) / 2147483648.0)
+    R = float(np.percentile(np.abs(fl), 97.0)) or 1.0   # 3 % of the outputs saturate
+    res = capi.quantized_fc(dev(d), dev(w), None if b is None else dev(b), f32(-rd), f32(rd),
+                            f32(-rw), f32(rw), None if b is None else f32(-rb),
+                            None if b is None else f32(rb), want_int32=True,
+                            calib=(-R, 0.8 * R), relu=relu)
+    np.testing.assert_array_equal(res["out32"].cpu().numpy(), ro)
+    assert (res["omin"].item(), res["omax"].item()) == (rmn, rmx)
+    rq, qmn, qmx = oracle.requantize(ro, rmn, rmx, -R, 0.8 * R)
+    if relu:
+        rq = oracle.relu_i8(rq)
+    np.testing.assert_array_equal(res["out8"].cpu().numpy(), rq)
+    assert (res["rmin"].item(), res["rmax"].item()) == (qmn, qmx)
+    # the fused form alone (no int32 output) takes other kernels for some shapes
+    res8 = capi.quantized_fc(dev(d), dev(w), None if b is None else dev(b), f32(-rd), f32(rd),
+                             f32(-rw), f32(rw), None if b is None else f32(-rb),
+                             None if b is None else f32(rb), want_int32=False,
+                             calib=(-R, 0.8 * R), relu=relu)
+    np.testing.assert_array_equal(res8["out8"].cpu().numpy(), rq)
+
+
+def conv_cases():
+    rng = np.random.default_rng(77)
+    cases = []
+    while len(cases) < 40:
+        N = int(rng.integers(1, 4))
+        C = int(rng.choice([3, 4, 16, 20, 32, 48, 64, 128]))
+        H = int(rng.integers(3, 20))
+        W = int(rng.integers(3, 20))
+        O = int(rng.choice([8, 24, 64, 70, 128, 200]))
+        KH = int(rng.choice([1, 3, 5]))
+        KW = int(rng.choice([1, 3]))
+        s = int(rng.choice([1, 2]))
+        p = int(rng.integers(0, 3))
+        dl = int(rng.choice([1, 1, 2]))
+        if (H + 2 * p - dl * (KH - 1) - 1) < 0 or (W + 2 * p - dl * (KW - 1) - 1) < 0:
+            continue
+        cases.append((N, C, H, W, O, KH, KW, s, p, dl))
+    return cases
+
+
+@pytest.mark.parametrize("case", conv_cases())
+def test_conv_random_geometry(capi, case):
+    N, C, H, W, O, KH, KW, s, p, dl = case
+    d = int8_uniform((N, C, H, W), seed=C + H * 3 + W)
+    w = int8_uniform((O, C, KH, KW), seed=O + KH + 11)
+    b = int8_uniform((O,), seed=O + 1) if (N + C + O) % 2 else None
+    relu = bool((H + W) % 2)
+    ro, rmn, rmx = oracle.quantized_conv(d, w, b, -1.0, 1.0, -1.0, 1.0,
+                                         None if b is None else -1.0,
+                                         None if b is None else 1.0, (s, s), (p, p), (dl, dl))
+    fl = ro.astype(np.float64) * (float(rmx) / 2147483648.0)
+    R = float(np.percentile(np.abs(fl), 97.0)) or 1.0
+    dn, wn = capi.nchw_to_nhwc_i8(dev(d)), capi.nchw_to_nhwc_i8(dev(w))
+    one = [f32(-1.0), f32(1.0)]
+    res = capi.quantized_conv_nhwc(dn, wn, None if b is None else dev(b), one[0], one[1], one[0],
+                                   one[1], None if b is None else one[0],
+                                   None if b is None else one[1], stride=(s, s), pad=(p, p),
+                                   dilate=(dl, dl), calib=(-R, 0.8 * R), relu=relu,
+                                   want_int32=True)
+    np.testing.assert_array_equal(capi.nhwc_to_nchw(res["out32"]).cpu().numpy(), ro)
+    rq, qmn, qmx = oracle.requantize(ro, rmn, rmx, -R, 0.8 * R)
+    if relu:
+        rq = oracle.relu_i8(rq)
+    np.testing.assert_array_equal(capi.nhwc_to_nchw(res["out8"]).cpu().numpy(), rq)
+    assert (res["omin"].item(), res["omax"].item()) == (rmn, rmx)
+    assert (res["rmin"].item(), res["rmax"].item()) == (qmn, qmx)
