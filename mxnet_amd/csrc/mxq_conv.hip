@@ -318,7 +318,7 @@ __global__ __launch_bounds__(64 * kRowsWaves, 1) void conv3x3_rows_kernel(ConvAr
   __syncthreads();
 
   const int lrow = lane & 31, lgrp = lane >> 5;
-  const bool relu = p.epi.relu != 0;
+  const bool relu = p.epi.relu != 0, stream8 = p.epi.stream8 != 0;
   // patch pixel of output column mi * 32 + lrow under tap column kw; columns past the row
   // (their results are never stored) are kept inside it
   int apx[2][3];
@@ -408,15 +408,21 @@ __global__ __launch_bounds__(64 * kRowsWaves, 1) void conv3x3_rows_kernel(ConvAr
       __builtin_amdgcn_wave_barrier();
       int8_t* orow = p.epi.out8 +
                      (static_cast<size_t>(n) * p.OH + oh0 + r) * p.OW * kRowsO;
+      auto store_row = [&](auto stream) {
 #pragma unroll
-      for (int it = 0; it < 4; ++it) {
-        const int px = it * 16 + (lane >> 2), c16 = lane & 3;
-        if (px < p.OW) {
-          const v4i val =
-              *reinterpret_cast<const v4i*>(stage + px * kRowsO + ((c16 ^ tile_swz(px)) << 4));
-          *reinterpret_cast<v4i*>(orow + px * kRowsO + c16 * 16) = val;
+        for (int it = 0; it < 4; ++it) {
+          const int px = it * 16 + (lane >> 2), c16 = lane & 3;
+          if (px < p.OW) {
+            const v4i val =
+                *reinterpret_cast<const v4i*>(stage + px * kRowsO + ((c16 ^ tile_swz(px)) << 4));
+            epi_store16<decltype(stream)::value>(val, orow + px * kRowsO + c16 * 16);
+          }
         }
-      }
+      };
+      if (stream8)
+        store_row(std::true_type());
+      else
+        store_row(std::false_type());
     }
     // the next item's fetches overwrite the patch: every LDS read above must have returned
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
@@ -755,6 +761,7 @@ void conv_nhwc(void* stream, const int8_t* data, const int8_t* weight, const int
   float x = fabsf(min_calib), y = fabsf(max_calib);
   e.real_range = (x < y) ? y : x;
   e.plane = planar ? a.OH * a.OW : 0;
+  e.stream8 = epi_stream_rows(a.M);
 
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (a.M == 0 || O == 0) {

@@ -161,7 +161,7 @@ __global__ __launch_bounds__(256, 2) void fc_stream_kernel(FcArgs p, int bn, int
   int item = blockIdx.x * 4 + wave;
   v4i fa[KS];
   if (item < items) load_a(item, fa);
-  const bool relu = p.epi.relu != 0;
+  const bool relu = p.epi.relu != 0, stream8 = p.epi.stream8 != 0;
   for (; item < items; item += step) {
     v4i fa_next[KS];
     const bool more = item + step < items;
@@ -211,15 +211,21 @@ __global__ __launch_bounds__(256, 2) void fc_stream_kernel(FcArgs p, int bn, int
     // order, the wait makes the writes complete first
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     __builtin_amdgcn_wave_barrier();
+    auto store_tile = [&](auto stream) {
 #pragma unroll
-    for (int it = 0; it < 32 / RPI; ++it) {
-      const int rr = it * RPI + lane / LPR, c16 = lane % LPR;
-      const v4i val = *reinterpret_cast<const v4i*>(stage + rr * LD + c16 * 16);
-      const int m = m_base + rr;
-      if (m < p.M)
-        *reinterpret_cast<v4i*>(p.epi.out8 + static_cast<size_t>(m) * p.ldo + n_begin + s0 +
-                                c16 * 16) = val;
-    }
+      for (int it = 0; it < 32 / RPI; ++it) {
+        const int rr = it * RPI + lane / LPR, c16 = lane % LPR;
+        const v4i val = *reinterpret_cast<const v4i*>(stage + rr * LD + c16 * 16);
+        const int m = m_base + rr;
+        if (m < p.M)
+          epi_store16<decltype(stream)::value>(
+              val, p.epi.out8 + static_cast<size_t>(m) * p.ldo + n_begin + s0 + c16 * 16);
+      }
+    };
+    if (stream8)
+      store_tile(std::true_type());
+    else
+      store_tile(std::false_type());
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     __builtin_amdgcn_wave_barrier();
     if (more) {
@@ -380,6 +386,7 @@ void launch_fc(hipStream_t s, const int8_t* data, const int8_t* weight, int M, i
   a.K = K;
   a.ldo = ldo;
   a.epi = epi;
+  a.epi.stream8 = epi_stream_rows(M);
   a.sk.splits = 1;
   a.sk.kt_per_split = 1 << 30;
   a.sk.counters = nullptr;

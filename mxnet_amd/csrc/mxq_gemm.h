@@ -63,7 +63,35 @@ struct Epilogue {
   // and out32 is written planar, [M / plane][N][plane] (NCHW for an NHWC convolution);
   // only out32 has this form.
   int plane;
+  // out8 is written with non-temporal stores (see epi_stream_rows)
+  int stream8;
 };
+
+// Outputs of at least this many rows are written with non-temporal stores: plain stores
+// leave the int8 tiles as dirty lines in the XCDs' L2s, where they displace the operand
+// rows other tiles of the launch still share and have to be written back when the next
+// launch needs the space.  The 19 layers of the ResNet-50 stack at batch 64, each on
+// operands of its own: 304-309 us with plain stores, 263 us with every layer streaming,
+// 267 us from 8192 rows on, 277 us from 32768 rows on (one box, two rounds each).  The layer
+// that consumes the output then reads it from memory instead of the memory-side cache,
+// which it only forgives when the producer's gain is large: measured on producer ->
+// consumer pairs (second layer reading what the first wrote, six rotating sets; 1x1 -> 1x1,
+// 1x1 -> 3x3 and 3x3 -> 1x1 at batch 64), streaming changes the pair's time by -14 ... 0 %
+// at 200704 and 50176 rows, -3 ... +5 % at 12544 rows, +1 ... +11 % at 3136 and 4096 rows
+// (BERT's 4096 x 3072 -> 768).  The threshold keeps the first group only.
+constexpr int kEpiStreamRows = 32768;
+inline int epi_stream_rows(long long rows) { return rows >= kEpiStreamRows ? 1 : 0; }
+
+// 16 bytes of the int8 output tile.  The flavour is a compile-time parameter and callers
+// branch around whole store loops: two stores to one address that differ only in the
+// non-temporal hint are merged into a plain one by the compiler.
+template <bool STREAM>
+__device__ __forceinline__ void epi_store16(v4i val, void* p) {
+  if (STREAM)
+    __builtin_nontemporal_store(val, reinterpret_cast<v4i*>(p));
+  else
+    *reinterpret_cast<v4i*>(p) = val;
+}
 
 __device__ __forceinline__ float dev_maxabs(float a, float b) {
   float x = fabsf(a), y = fabsf(b);
@@ -901,18 +929,24 @@ __device__ __forceinline__ void gemm_epilogue_lds(v16i (&acc)[Cfg::MI][Cfg::NI],
     __builtin_amdgcn_wave_barrier();
     // 16-byte pieces of the staged tile in row-major order, 64 per store instruction (a
     // wave tile of 96 columns has 6 pieces per row: the last instruction is then partial)
-    constexpr int kPieces = TM * LPR;
+    auto store_tile = [&](auto stream) {
+      constexpr int kPieces = TM * LPR;
 #pragma unroll
-    for (int it = 0; it < (kPieces + 63) / 64; ++it) {
-      const int piece = it * 64 + lane;
-      const int rr = (64 % LPR == 0) ? it * RPI + lane / LPR : piece / LPR;
-      const int c16 = (64 % LPR == 0) ? lane % LPR : piece - rr * LPR;
-      if (kPieces % 64 != 0 && piece >= kPieces) continue;
-      const v4i val = *reinterpret_cast<const v4i*>(stage + rr * LD + c16 * 16);
-      const int m = m_base + rr, n = n_base + c16 * 16;
-      if (m < M && n < N)
-        *reinterpret_cast<v4i*>(e.out8 + static_cast<size_t>(m) * ldo + n) = val;
-    }
+      for (int it = 0; it < (kPieces + 63) / 64; ++it) {
+        const int piece = it * 64 + lane;
+        const int rr = (64 % LPR == 0) ? it * RPI + lane / LPR : piece / LPR;
+        const int c16 = (64 % LPR == 0) ? lane % LPR : piece - rr * LPR;
+        if (kPieces % 64 != 0 && piece >= kPieces) continue;
+        const v4i val = *reinterpret_cast<const v4i*>(stage + rr * LD + c16 * 16);
+        const int m = m_base + rr, n = n_base + c16 * 16;
+        if (m < M && n < N)
+          epi_store16<decltype(stream)::value>(val, e.out8 + static_cast<size_t>(m) * ldo + n);
+      }
+    };
+    if (e.stream8)
+      store_tile(std::true_type());
+    else
+      store_tile(std::false_type());
   }
 }
 
