@@ -333,7 +333,9 @@ __global__ __launch_bounds__(64 * kRowsWaves, 1) void conv3x3_rows_kernel(ConvAr
     const int n = item / chunks_per_image, oh0 = (item - n * chunks_per_image) * R;
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __builtin_amdgcn_wave_barrier();
-#pragma unroll
+    // a real loop: the second row re-runs the first row's instructions out of the
+    // instruction cache instead of fetching a second copy of them
+#pragma unroll 1
     for (int r = 0; r < R; ++r) {
       if (oh0 + r >= p.OH) break;
       // accumulators start at the int32 bias of their columns, read from LDS straight into
