@@ -238,7 +238,7 @@ __global__ __launch_bounds__(kThreads) void add_kernel(AddArgs a) {
           i4 v;
 #pragma unroll
           for (int k = 0; k < 4; ++k) v[k] = r.apply(byte_of<LU>(x[j], k), byte_of<RU>(y[j], k));
-          __builtin_amdgcn_raw_buffer_store_b128(v, dst, (j * 64 + lane) * 16, 0, 16 /* sc1 */);
+          __builtin_amdgcn_raw_buffer_store_b128(v, dst, (j * 64 + lane) * 16, 0, 18 /* sc1 + nt */);
         }
       }
       for (size_t q = runs * kRun + t0; q < nq; q += stride) {
