@@ -208,7 +208,7 @@ __global__ __launch_bounds__(Cfg::kThreads, NS <= 2 ? Cfg::kMinWaves : 1) void c
   __shared__ __attribute__((aligned(16))) v4i lds[NS * Cfg::STAGE_SLOTS];
   const int tiles_m = (p.M + Cfg::BM - 1) / Cfg::BM, tiles_n = (p.O + Cfg::BN - 1) / Cfg::BN;
   int tm, tn, tile = 0, z = 0;
-  if (p.sk.splits > 1)
+  if (__builtin_expect(p.sk.splits > 1, 0))
     tile_coords_split(blockIdx.x, tiles_m, tiles_n, p.sk.splits, tm, tn, tile, z);
   else
     tile_coords(blockIdx.x, tiles_m, tiles_n, tm, tn);
@@ -233,7 +233,7 @@ __global__ __launch_bounds__(Cfg::kThreads, NS <= 2 ? Cfg::kMinWaves : 1) void c
   gemm_mainloop_dma<Cfg, NS, PIPE>(acc, ai, bi, KT, lds, prefetch);
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   if (blockIdx.x == 0 && threadIdx.x == 0) epilogue_ranges(p.epi);
-  if (p.sk.splits > 1 && !splitk_gather<Cfg>(acc, p.sk, tile, z)) return;
+  if (__builtin_expect(p.sk.splits > 1, 0) && !splitk_gather<Cfg>(acc, p.sk, tile, z)) return;
 
   gemm_epilogue_lds<Cfg, NS * Cfg::STAGE_SLOTS * 16>(acc, p.epi, pre, m0, n0, p.M, p.O,
                                                      static_cast<size_t>(p.O), lds);
