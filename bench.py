@@ -70,7 +70,8 @@ def parse_args():
                              "quantize_laplace", "quantize_uint8_uncal", "small_casts",
                              "requantize", "requantize_uncal", "dequantize", "copy", "maxpool", "avgpool",
                              "elemwise_add", "elemwise_add_int8", "concat", "elemwise_mul_int8", "quantize_asym",
-                             "batch_norm", "embedding", "transpose", "resnet50_convs", "bert_fc_chain",
+                             "batch_norm", "embedding", "transpose", "resnet50_convs", "resnet50_chain",
+                             "bert_fc_chain",
                              "bert_fc_chain_fused"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-cast-ops", action="store_true")
@@ -726,6 +727,109 @@ class ConvStackWorkload(GraphWorkload):
 BERT_FCS = [(768, 2304), (768, 768), (768, 3072), (3072, 768)]
 
 
+class ResNetChainWorkload(GraphWorkload):
+    """The bottleneck body of ResNet-50 v1 at batch 64 as one producer -> consumer chain (the 19
+    shapes of configuration 4 in the order and number a forward pass runs them): 16 blocks of
+    conv1x1 (+relu) -> conv3x3 (+relu) -> conv1x1, a projection conv1x1 on the shortcut of the
+    first block of each stage, quantized_elemwise_add of the two branches (int8 out, calibrated)
+    and quantized ReLU; stride on the first 1x1 of a stage as in the reference's model zoo
+    (python/mxnet/gluon/model_zoo/vision/resnet.py:108-123).  Every layer reads what the layer
+    before it wrote.  NHWC int8, requantize fused into every convolution, calibration ranges
+    from one pass with int32 outputs over the same synthetic input.  52 convolutions + 16 adds +
+    16 relus per step; stem, pooling and the classifier are not part of it."""
+    STAGES = [(3, 64, 256, 1), (4, 128, 512, 2), (6, 256, 1024, 2), (3, 512, 2048, 2)]
+
+    def __init__(self, torch, capi, lib):
+        self.kernel = "conv / fc kernels, add_kernel, relu"
+        self.bound = "mfma"
+        self.name = "ResNet-50 v1 bottleneck body as a chain (52 convolutions + 16 residual " \
+                    "adds + relus), batch 64, NHWC int8, requantize fused"
+        P = lambda t: ctypes.c_void_p(t.data_ptr()) if t is not None else None
+        g = torch.Generator(device="cuda").manual_seed(44)
+        N, H = 64, 56
+        x = torch.randn((N, H, H, 64), device="cuda", generator=g).clamp_(min=0.0)
+        cur, cmin, cmax = capi.quantize_v2(x, "int8")
+        del x
+        self.calls, self.ops, self.keep = [], 0.0, []
+        f1 = lambda v: torch.tensor([v], dtype=torch.float32, device="cuda")
+
+        def conv(inp, imin, imax, H, C, O, k, s, relu):
+            """Adds one fused convolution to the chain; returns its int8 output and range."""
+            pad = 1 if k == 3 else 0
+            OH = (H + 2 * pad - k) // s + 1
+            w = torch.randn((O, k, k, C), device="cuda", generator=g) * (2.0 / (k * k * C)) ** 0.5
+            wq, wmin, wmax = capi.quantize(w, w.min().reshape(1), w.max().reshape(1), "int8")
+            b = torch.randn((O,), device="cuda", generator=g) * 0.1
+            bq, bmin, bmax = capi.quantize(b, b.min().reshape(1), b.max().reshape(1), "int8")
+            del w, b
+            # calibration: the float range of this layer's int32 output on the chain's own data
+            res = capi.quantized_conv_nhwc(inp, wq, bq, imin, imax, wmin, wmax, bmin, bmax,
+                                           stride=(s, s), pad=(pad, pad), want_int32=True)
+            r = float(res["out32"].abs().max().item()) * float(res["omax"].item()) / 2147483648.0
+            r = max(r, 1e-6)
+            del res
+            out8 = torch.empty((N, OH, OH, O), dtype=torch.int8, device="cuda")
+            sc = [torch.empty(1, device="cuda") for _ in range(4)]
+            geo = (N, H, H, C, O, k, k, s, s, pad, pad)
+            nws = lib.mxq_quantized_conv_workspace(*geo, 1, 1, 1)
+            ws = torch.empty(nws, dtype=torch.uint8, device="cuda") if nws else None
+            args = (P(inp), P(wq), P(bq), *geo, 1, 1, P(imin), P(imax), P(wmin), P(wmax), P(bmin),
+                    P(bmax), None, P(sc[0]), P(sc[1]), P(out8), P(sc[2]), P(sc[3]), int(relu), -r,
+                    r, *ws_args(ws))
+            self.calls.append((lib.mxq_quantized_conv_nhwc, args))
+            self.keep.append((inp, wq, bq, imin, imax, wmin, wmax, bmin, bmax, out8, sc, ws))
+            self.ops += 2.0 * N * OH * OH * O * k * k * C
+            st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+            if lib.mxq_quantized_conv_nhwc(st, *args):
+                raise RuntimeError(lib.mxq_last_error().decode())
+            return out8, sc[2], sc[3], OH
+
+        for (blocks, mid, out, stride) in self.STAGES:
+            for bi in range(blocks):
+                s = stride if bi == 0 else 1
+                C = cur.shape[3]
+                a, amin, amax, H1 = conv(cur, cmin, cmax, H, C, mid, 1, s, True)
+                b, bmin_, bmax_, _ = conv(a, amin, amax, H1, mid, mid, 3, 1, True)
+                c, cmin_, cmax_, _ = conv(b, bmin_, bmax_, H1, mid, out, 1, 1, False)
+                if bi == 0:
+                    sh, smin, smax, _ = conv(cur, cmin, cmax, H, C, out, 1, s, False)
+                else:
+                    sh, smin, smax = cur, cmin, cmax
+                # residual sum, int8 out with a calibrated range, then the quantized ReLU
+                fa = capi.dequantize(c, cmin_, cmax_) + capi.dequantize(sh, smin, smax)
+                r = max(float(fa.abs().max().item()), 1e-6)
+                del fa
+                y = torch.empty_like(c)
+                ysc = [torch.empty(1, device="cuda") for _ in range(4)]
+                z = torch.empty_like(c)
+                add_args = (P(c), 5, P(sh), 5, P(cmin_), P(cmax_), P(smin), P(smax), P(y), 5,
+                            P(ysc[0]), P(ysc[1]), c.numel(), 1, -r, r)
+                relu_args = (P(y), P(ysc[0]), P(ysc[1]), P(z), P(ysc[2]), P(ysc[3]), y.numel())
+                self.calls.append((lib.mxq_quantized_elemwise_add, add_args))
+                self.calls.append((lib.mxq_quantized_relu, relu_args))
+                self.keep.append((c, sh, y, z, ysc))
+                st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+                for fn, args in self.calls[-2:]:
+                    if fn(st, *args):
+                        raise RuntimeError(lib.mxq_last_error().decode())
+                cur, cmin, cmax, H = z, ysc[2], ysc[3], H1
+        torch.cuda.synchronize()
+        self.images = N
+
+        def body():
+            st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+            for fn, args in self.calls:
+                if fn(st, *args):
+                    raise RuntimeError(lib.mxq_last_error().decode())
+        self.graph_body = body
+        self.capture(torch, body)
+
+    def per_layer(self, torch):
+        t = self.time_alone(torch, self.graph_body, reps=1, replays=50)
+        return [{"chain": "whole body", "us": round(t * 1e6, 1),
+                 "images_per_s": round(self.images / t, 0), "launches": len(self.calls)}]
+
+
 class BertChainWorkload(GraphWorkload):
     """Benchmark configuration 5: BERT-base FC shapes at M = 32 x 128 = 4096; per layer calibrated
     quantize_v2 -> quantized_fully_connected (+ int8 bias) -> requantize -> dequantize, as
@@ -866,6 +970,8 @@ def mfma_context(torch, S):
 def make_workload(name, torch, capi, lib):
     if name == "resnet50_convs":
         return ConvStackWorkload(torch, capi, lib)
+    if name == "resnet50_chain":
+        return ResNetChainWorkload(torch, capi, lib)
     if name == "bert_fc_chain":
         return BertChainWorkload(torch, capi, lib)
     if name == "bert_fc_chain_fused":
@@ -989,7 +1095,7 @@ def main():
                      "requantize_uncal", "dequantize", "elemwise_add", "elemwise_add_int8",
                      "concat", "elemwise_mul_int8", "quantize_asym", "batch_norm", "embedding",
                      "transpose", "maxpool", "avgpool", "fc8192",
-                     "resnet50_convs", "bert_fc_chain", "bert_fc_chain_fused"]:
+                     "resnet50_convs", "resnet50_chain", "bert_fc_chain", "bert_fc_chain_fused"]:
             if kind == args.workload:
                 continue
             w2 = make_workload(kind, torch, capi, lib)

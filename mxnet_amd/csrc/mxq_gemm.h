@@ -70,16 +70,19 @@ struct Epilogue {
 // Outputs of at least this many rows are written with non-temporal stores: plain stores
 // leave the int8 tiles as dirty lines in the XCDs' L2s, where they displace the operand
 // rows other tiles of the launch still share and have to be written back when the next
-// launch needs the space.  The 19 layers of the ResNet-50 stack at batch 64, each on
-// operands of its own: 304-309 us with plain stores, 263 us with every layer streaming,
-// 267 us from 8192 rows on, 277 us from 32768 rows on (one box, two rounds each).  The layer
-// that consumes the output then reads it from memory instead of the memory-side cache,
-// which it only forgives when the producer's gain is large: measured on producer ->
-// consumer pairs (second layer reading what the first wrote, six rotating sets; 1x1 -> 1x1,
-// 1x1 -> 3x3 and 3x3 -> 1x1 at batch 64), streaming changes the pair's time by -14 ... 0 %
-// at 200704 and 50176 rows, -3 ... +5 % at 12544 rows, +1 ... +11 % at 3136 and 4096 rows
-// (BERT's 4096 x 3072 -> 768).  The threshold keeps the first group only.
-constexpr int kEpiStreamRows = 32768;
+// launch needs the space.  The layer that consumes the output then reads it from memory
+// instead of the memory-side cache.  Measured at batch 64 (one box each, two rounds):
+//   the 19 ResNet-50 layers on operands of their own: plain 304-309 us, streaming from
+//     32768 rows 277, from 8192 rows 267, every layer 263;
+//   the ResNet-50 bottleneck body as a real chain (52 convolutions, every layer reading
+//     what the one before wrote): plain 1095 us, from 32768 rows 1074, from 8192 rows 1065,
+//     every layer 1064.5;
+//   producer -> consumer pairs (1x1 -> 1x1, 1x1 -> 3x3, 3x3 -> 1x1): -14 ... 0 % for the
+//     pair at 200704 and 50176 rows, -3 ... +5 % at 12544 rows, +1 ... +11 % at 3136 and
+//     4096 rows; BERT's chain at 4096 rows (a dequantize consumes each output) +2.5 %.
+// 8192 keeps everything from 14 x 14 planes at batch 64 up and leaves the 4096-row
+// fully-connected layers alone.
+constexpr int kEpiStreamRows = 8192;
 inline int epi_stream_rows(long long rows) { return rows >= kEpiStreamRows ? 1 : 0; }
 
 // 16 bytes of the int8 output tile.  The flavour is a compile-time parameter and callers
