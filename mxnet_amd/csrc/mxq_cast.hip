@@ -664,7 +664,19 @@ __global__ __launch_bounds__(kThreads) void relu_i8_kernel(const int8_t* __restr
     const size_t n16 = n >> 4;
     const u4* in16 = reinterpret_cast<const u4*>(in);
     u4* out16 = reinterpret_cast<u4*>(out);
-    for (size_t q = t0; q < n16; q += stride) {
+    // four 16-byte pieces a grid stride apart in flight per lane
+    size_t q = t0;
+    for (; q + 3 * stride < n16; q += 4 * stride) {
+      u4 w[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) w[j] = nt_load(in16 + q + j * stride);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        u4 r = {relu4(w[j].x), relu4(w[j].y), relu4(w[j].z), relu4(w[j].w)};
+        nt_store(r, out16 + q + j * stride);
+      }
+    }
+    for (; q < n16; q += stride) {
       u4 w = nt_load(in16 + q);
       u4 r = {relu4(w.x), relu4(w.y), relu4(w.z), relu4(w.w)};
       nt_store(r, out16 + q);
@@ -946,7 +958,7 @@ int mxq_quantized_relu(void* stream, const int8_t* in, const float* imin, const 
             "null range pointer");
   MXQ_CHECK(n == 0 || (in != nullptr && out != nullptr), "null data pointer");
   const bool vec = aligned16(in) && aligned16(out);
-  const int grid = stream_grid(n == 0 ? 1 : (vec ? (n + 15) / 16 : n));
+  const int grid = stream_grid(n == 0 ? 1 : (vec ? (n + 15) / 16 : n), n);
   hipLaunchKernelGGL(relu_i8_kernel, dim3(grid), dim3(kThreads), 0,
                      static_cast<hipStream_t>(stream), in, out, n, imin, imax, omin, omax, vec);
   MXQ_LAUNCH_CHECK();

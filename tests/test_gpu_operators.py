@@ -239,8 +239,12 @@ def test_quantized_conv_channel_counts_off_16(contrib, shape, filters, kernel, s
     assert (mn.item(), mx.item()) == (rmn, rmx)
 
 
-def test_quantized_act(contrib):
-    q = np.random.default_rng(8).integers(-128, 128, size=(5, 1000), dtype=np.int8)
+# sizes: below one pass of the grid, the unrolled loop with a remainder and a ragged tail,
+# many passes of the unrolled loop
+@pytest.mark.parametrize("shape", [(5, 1000), (1, 1), (3, 1000003), (64, 28, 28, 512),
+                                   ((1 << 25) + 17,)])
+def test_quantized_act(contrib, shape):
+    q = np.random.default_rng(8).integers(-128, 128, size=shape, dtype=np.int8)
     out, mn, mx = contrib.quantized_act(dev(q), scalar(-2.5), scalar(2.5), act_type="relu")
     np.testing.assert_array_equal(out.cpu().numpy(), np.maximum(q, 0))
     assert (mn.item(), mx.item()) == (-2.5, 2.5)
