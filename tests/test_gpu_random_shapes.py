@@ -37,6 +37,10 @@ def fc_shapes():
     # under a long K (split-K with the workspace the entry point asks for), one row
     shapes += [(512, 384, 512), (300, 192, 1024), (2048, 64, 64), (4100, 128, 128),
                (64, 320, 8192), (40, 130, 9000), (1, 1000, 4096), (700, 1, 48)]
+    # either side of the row count from which the int8 tiles are written with streaming
+    # stores (8192), ragged there, through the tiled, the short-K and the fallback kernels
+    shapes += [(8191, 64, 48), (8192, 128, 64), (8200, 80, 256), (9000, 256, 64),
+               (33000, 64, 128), (8193, 100, 37)]
     return shapes
 
 
@@ -88,6 +92,10 @@ def conv_cases():
         if (H + 2 * p - dl * (KH - 1) - 1) < 0 or (W + 2 * p - dl * (KW - 1) - 1) < 0:
             continue
         cases.append((N, C, H, W, O, KH, KW, s, p, dl))
+    # more than 8192 output pixels: the streaming-store flavour of the tiled kernels, ragged
+    # last tiles
+    cases += [(3, 16, 64, 64, 32, 3, 3, 1, 1, 1), (2, 64, 70, 58, 64, 3, 3, 1, 1, 1),
+              (5, 32, 45, 41, 48, 1, 1, 1, 0, 1), (9, 64, 62, 60, 24, 3, 3, 2, 1, 1)]
     return cases
 
 
