@@ -1,0 +1,109 @@
+"""The entry points under HIP graph capture: a chain of them is recorded once and replayed
+several times on new input contents (written into the captured buffers between replays, with
+the program's own eager work and synchronisations in between); every replay must give what
+the oracle gives for that input.  Covers the launches that carry state between kernels of
+one call: the uncalibrated casts (reduction partials in a workspace, or in the library's own
+array for the no-allocation entry point) and a split-K fully-connected layer (tile counters
+cleared by a kernel of the same call, partial sums in the workspace)."""
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from tests.data_gen import int8_uniform
+
+pytestmark = pytest.mark.gpu
+
+
+def P(t):
+    return ctypes.c_void_p(t.data_ptr()) if t is not None else None
+
+
+def scalar():
+    return torch.empty(1, dtype=torch.float32, device="cuda")
+
+
+def test_replays_follow_their_inputs():
+    import mxnet_amd
+    lib = mxnet_amd._lib.lib
+    M, K, N = 256, 8192, 800          # the launcher splits this one along K
+    n = M * K
+    x = torch.empty(n, dtype=torch.float32, device="cuda")
+    q = torch.empty((M, K), dtype=torch.int8, device="cuda")
+    q2 = torch.empty((M, K), dtype=torch.int8, device="cuda")
+    qr = [scalar() for _ in range(4)]
+    w_np = int8_uniform((N, K), seed=5)
+    b_np = int8_uniform((N,), seed=6)
+    w, b = torch.from_numpy(w_np).cuda(), torch.from_numpy(b_np).cuda()
+    wr = [torch.tensor([v], device="cuda") for v in (-0.3, 0.3, -0.9, 0.9)]
+    acc = torch.empty((M, N), dtype=torch.int32, device="cuda")
+    out8 = torch.empty((M, N), dtype=torch.int8, device="cuda")
+    fr = [scalar() for _ in range(4)]
+    r8 = torch.empty((M, N), dtype=torch.int8, device="cuda")
+    rr = [scalar() for _ in range(2)]
+    y = torch.empty((M, N), dtype=torch.float32, device="cuda")
+    ws_q = torch.empty(lib.mxq_quantize_v2_workspace(n), dtype=torch.uint8, device="cuda")
+    ws_r = torch.empty(lib.mxq_requantize_workspace(M * N), dtype=torch.uint8, device="cuda")
+    nfc = lib.mxq_quantized_fc_workspace(M, N, K, 0)
+    assert nfc > 0, "this shape is expected to ask for a split-K workspace"
+    ws_fc = torch.empty(nfc, dtype=torch.uint8, device="cuda")
+    calib = 40.0
+
+    def body():
+        st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+        rcs = [
+            # uncalibrated quantize: partials in the caller's workspace ...
+            lib.mxq_quantize_v2(st, P(x), P(q), P(qr[0]), P(qr[1]), n, 5, 0, 0.0, 0.0, P(ws_q),
+                                ws_q.numel()),
+            # ... and in the library's own array
+            lib.mxq_quantize_v2_noalloc(st, P(x), P(q2), P(qr[2]), P(qr[3]), n, 5, 0, 0.0, 0.0),
+            lib.mxq_quantized_fc(st, P(q), P(w), P(b), M, N, K, P(qr[0]), P(qr[1]), P(wr[0]),
+                                 P(wr[1]), P(wr[2]), P(wr[3]), P(acc), P(fr[0]), P(fr[1]),
+                                 P(out8), P(fr[2]), P(fr[3]), 0, -calib, calib, P(ws_fc),
+                                 ws_fc.numel()),
+            # uncalibrated requantize of the int32 output
+            lib.mxq_requantize(st, P(acc), P(fr[0]), P(fr[1]), P(r8), P(rr[0]), P(rr[1]), M * N,
+                               0, 0.0, 0.0, P(ws_r), ws_r.numel()),
+            lib.mxq_dequantize(st, P(r8), 5, P(rr[0]), P(rr[1]), P(y), M * N),
+        ]
+        assert not any(rcs), mxnet_amd._lib.last_error()
+
+    rng = np.random.default_rng(3)
+    first = rng.standard_normal(n).astype(np.float32)
+    x.copy_(torch.from_numpy(first))
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        body()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        body()
+
+    for it in range(4):
+        data = (rng.standard_normal(n) * (1.0 + it)).astype(np.float32)
+        data[it] = 7.0 * (it + 1)                     # the range changes with every replay
+        x.copy_(torch.from_numpy(data))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        oq, omn, omx = oracle.quantize_v2(data, "int8")
+        np.testing.assert_array_equal(q.cpu().numpy().ravel(), oq)
+        np.testing.assert_array_equal(q2.cpu().numpy().ravel(), oq)
+        assert (qr[0].item(), qr[1].item()) == (omn, omx)
+        assert (qr[2].item(), qr[3].item()) == (omn, omx)
+        ro, rmn, rmx = oracle.quantized_fully_connected(oq.reshape(M, K), w_np, b_np, omn, omx,
+                                                        -0.3, 0.3, -0.9, 0.9)
+        np.testing.assert_array_equal(acc.cpu().numpy(), ro)
+        assert (fr[0].item(), fr[1].item()) == (rmn, rmx)
+        fq, fmn, fmx = oracle.requantize(ro, rmn, rmx, -calib, calib)
+        np.testing.assert_array_equal(out8.cpu().numpy(), fq)
+        uq, umn, umx = oracle.requantize(ro, rmn, rmx)
+        np.testing.assert_array_equal(r8.cpu().numpy(), uq)
+        assert (rr[0].item(), rr[1].item()) == (umn, umx)
+        np.testing.assert_array_equal(y.cpu().numpy(), oracle.dequantize(uq, umn, umx))
+        # the program's own eager work between replays
+        (x * 2.0).sum().item()
