@@ -72,7 +72,8 @@ def parse_args():
                              "elemwise_add", "elemwise_add_int8", "concat", "elemwise_mul_int8", "quantize_asym",
                              "batch_norm", "embedding", "transpose", "resnet50_convs", "resnet50_chain",
                              "bert_fc_chain",
-                             "bert_fc_chain_fused"])
+                             "bert_fc_chain_fused",
+                             "bert_fc_chain_f32"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-cast-ops", action="store_true")
     return ap.parse_args()
@@ -840,7 +841,11 @@ class BertChainWorkload(GraphWorkload):
         self.bound = "mfma"
         self.name = "BERT-base FC chain M=4096: 768->2304, 768->768, 768->3072, 3072->768, " \
                     "quantize_v2 -> quantized_fc -> requantize -> dequantize per layer"
-        if fused:
+        if fused == "f32":
+            self.kernel = "quantize + fc_dma (requantize and dequantize in the epilogue) kernels"
+            self.name = self.name.replace("quantized_fc -> requantize -> dequantize",
+                                          "quantized_fc with requantize and dequantize fused")
+        elif fused:
             self.kernel = "quantize + fc_dma (requantize in the epilogue) + dequantize kernels"
             self.name = self.name.replace("quantized_fc -> requantize",
                                           "quantized_fc with the requantize fused")
@@ -863,7 +868,7 @@ class BertChainWorkload(GraphWorkload):
                         q8=torch.empty((M, N), dtype=torch.int8, device="cuda"),
                         y=torch.empty((M, N), dtype=torch.float32, device="cuda"),
                         sc=[torch.empty(1, device="cuda") for _ in range(6)],
-                        ws=fc_workspace(torch, lib, M, N, K, fused))
+                        ws=fc_workspace(torch, lib, M, N, K, fused is True))
             self.layers.append((K, N, wq, bq, wmin, wmax, bmin, bmax, r, bufs))
             self.ops += 2.0 * M * N * K
             del w
@@ -874,6 +879,17 @@ class BertChainWorkload(GraphWorkload):
                 if only is not None and i != only:
                     continue
                 sc = B["sc"]
+                if fused == "f32":
+                    rcs = [
+                        lib.mxq_quantize_v2(st, P(B["x"]), P(B["q"]), P(sc[0]), P(sc[1]), M * K,
+                                            5, 1, -20.0, 20.0, None, 0),
+                        lib.mxq_quantized_fc_f32(st, P(B["q"]), P(wq), P(bq), M, N, K, P(sc[0]),
+                                                 P(sc[1]), P(wmin), P(wmax), P(bmin), P(bmax),
+                                                 P(B["y"]), P(sc[2]), P(sc[3]), P(sc[4]),
+                                                 P(sc[5]), 0, -r, r, *ws_args(B["ws"]))]
+                    if any(rcs):
+                        raise RuntimeError(lib.mxq_last_error().decode())
+                    continue
                 if fused:
                     rcs = [
                         lib.mxq_quantize_v2(st, P(B["x"]), P(B["q"]), P(sc[0]), P(sc[1]), M * K,
@@ -976,6 +992,8 @@ def make_workload(name, torch, capi, lib):
         return BertChainWorkload(torch, capi, lib)
     if name == "bert_fc_chain_fused":
         return BertChainWorkload(torch, capi, lib, fused=True)
+    if name == "bert_fc_chain_f32":
+        return BertChainWorkload(torch, capi, lib, fused="f32")
     if name == "copy":
         return CopyWorkload(torch)
     if name == "small_casts":
@@ -1095,7 +1113,8 @@ def main():
                      "requantize_uncal", "dequantize", "elemwise_add", "elemwise_add_int8",
                      "concat", "elemwise_mul_int8", "quantize_asym", "batch_norm", "embedding",
                      "transpose", "maxpool", "avgpool", "fc8192",
-                     "resnet50_convs", "resnet50_chain", "bert_fc_chain", "bert_fc_chain_fused"]:
+                     "resnet50_convs", "resnet50_chain", "bert_fc_chain", "bert_fc_chain_fused",
+                     "bert_fc_chain_f32"]:
             if kind == args.workload:
                 continue
             w2 = make_workload(kind, torch, capi, lib)

@@ -297,6 +297,23 @@ int mxq_quantized_fc(void* stream, const int8_t* data, const int8_t* weight, con
                      int8_t* out8, float* rmin, float* rmax, int relu, float min_calib,
                      float max_calib, void* workspace, size_t workspace_bytes);
 
+/* _contrib_quantized_fully_connected -> _contrib_requantize -> _contrib_dequantize in one
+ * launch: the three operators a quantized graph runs where a float consumer follows the
+ * layer (quantized_fully_connected.cu:58-138, requantize-inl.h:89-125 with a calibrated
+ * range, dequantize-inl.h:64-75).  out_f32 [M,N] receives float(q) * (R / 127) with q the
+ * requantized int8 value and R = max(|min_calib|, |max_calib|): bit-identical to
+ * mxq_dequantize(mxq_requantize(out32)) element by element; relu != 0 clamps q at zero
+ * first.  omin/omax and rmin/rmax are written as by mxq_quantized_fc.  The int8 tensor
+ * between the operators is never stored.  Workspace as for mxq_quantized_fc (size it with
+ * fused_int8_only = 0). */
+int mxq_quantized_fc_f32(void* stream, const int8_t* data, const int8_t* weight,
+                         const int8_t* bias, int M, int N, int K, const float* min_data,
+                         const float* max_data, const float* min_weight, const float* max_weight,
+                         const float* min_bias, const float* max_bias, float* out_f32,
+                         float* omin, float* omax, float* rmin, float* rmax, int relu,
+                         float min_calib, float max_calib, void* workspace,
+                         size_t workspace_bytes);
+
 /* ---- _contrib_quantized_conv ----------------------------------------------
  * Replaces QuantizedCuDNNConvOp::Forward
  * (src/operator/quantization/quantized_conv.cu:101-219): the NHWC int8

@@ -60,6 +60,8 @@ SIGNATURES = {
     "mxq_quantized_fc_workspace": (_sz, [_i, _i, _i, _i]),
     "mxq_quantized_fc": (_i, [_p, _p, _p, _p, _i, _i, _i] + [_p] * 6 + [_p, _p, _p, _p, _p, _p,
                               _i, _f, _f, _p, _sz]),
+    "mxq_quantized_fc_f32": (_i, [_p, _p, _p, _p, _i, _i, _i] + [_p] * 6 + [_p, _p, _p, _p, _p,
+                                  _i, _f, _f, _p, _sz]),
     "mxq_quantized_conv_workspace": (_sz, [_i] * 14),
     "mxq_quantized_conv_nhwc": (_i, [_p, _p, _p, _p] + [_i] * 13 + [_p] * 6 +
                                 [_p, _p, _p, _p, _p, _p, _i, _f, _f, _p, _sz]),
@@ -81,6 +83,7 @@ for _name, (_res, _args) in SIGNATURES.items():
 # factor and, for the FC, the streaming kernel's work-groups per CU (0 = choose)
 TEST_HOOKS = {
     "mxq_test_quantized_fc": (_i, SIGNATURES["mxq_quantized_fc"][1] + [_i, _i, _i]),
+    "mxq_test_quantized_fc_f32": (_i, SIGNATURES["mxq_quantized_fc_f32"][1] + [_i, _i]),
     "mxq_test_quantized_conv_nhwc": (_i, SIGNATURES["mxq_quantized_conv_nhwc"][1] + [_i, _i]),
 }
 for _name, (_res, _args) in TEST_HOOKS.items():

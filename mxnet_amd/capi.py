@@ -125,6 +125,33 @@ def quantized_fc(data, weight, bias, min_data, max_data, min_weight, max_weight,
     return res
 
 
+def quantized_fc_f32(data, weight, bias, min_data, max_data, min_weight, max_weight,
+                     min_bias=None, max_bias=None, calib=(-1.0, 1.0), relu=False, force=None):
+    """quantized_fc -> requantize over `calib` -> dequantize in one launch.  Returns
+    dict(outf, omin, omax, rmin, rmax).  `force` = (cfg, splits) pins the kernel variant
+    through the test-only entry point."""
+    M, K = data.shape
+    N, K2 = weight.shape
+    assert K == K2
+    dev = data.device
+    res = {k: _scalar(dev) for k in ("omin", "omax", "rmin", "rmax")}
+    res["outf"] = torch.empty((M, N), dtype=torch.float32, device=dev)
+    args = [_stream(), _ptr(data), _ptr(weight), _ptr(bias), M, N, K, _ptr(min_data),
+            _ptr(max_data), _ptr(min_weight), _ptr(max_weight), _ptr(min_bias), _ptr(max_bias),
+            _ptr(res["outf"]), _ptr(res["omin"]), _ptr(res["omax"]), _ptr(res["rmin"]),
+            _ptr(res["rmax"]), int(relu), float(calib[0]), float(calib[1])]
+    if force is None:
+        wsb = lib.mxq_quantized_fc_workspace(M, N, K, 0)
+        ws = _workspace(wsb, dev) if wsb else None
+        check(lib.mxq_quantized_fc_f32(*args, _ptr(ws), wsb))
+    else:
+        cfg, splits = force
+        wsb = _SPLIT_WS_BYTES if splits > 1 else 0
+        ws = _workspace(wsb, dev) if wsb else None
+        check(lib.mxq_test_quantized_fc_f32(*args, _ptr(ws), wsb, cfg, splits))
+    return res
+
+
 def quantized_conv_nhwc(data, weight, bias, min_data, max_data, min_weight, max_weight,
                         min_bias=None, max_bias=None, stride=(1, 1), pad=(0, 0), dilate=(1, 1),
                         want_int32=True, calib=None, relu=False, force=None):

@@ -757,7 +757,7 @@ void conv_nhwc(void* stream, const int8_t* data, const int8_t* weight, const int
   e.min_data = min_data; e.max_data = max_data;
   e.min_weight = min_weight; e.max_weight = max_weight;
   e.min_bias = min_bias; e.max_bias = max_bias;
-  e.out32 = out32; e.out8 = out8;
+  e.out32 = out32; e.out8 = out8; e.outf = nullptr;
   e.omin = omin; e.omax = omax; e.rmin = rmin; e.rmax = rmax;
   e.relu = relu;
   float x = fabsf(min_calib), y = fabsf(max_calib);

@@ -397,8 +397,8 @@ void launch_fc(hipStream_t s, const int8_t* data, const int8_t* weight, int M, i
   const bool buf_ok = aligned && K >= 16 && static_cast<long long>(M) * K < (1LL << 31) &&
                       static_cast<long long>(N) * K < (1LL << 31);
   const bool glb_ok = buf_ok && (K % 64 == 0);
-  const bool fused8 = epi.out32 == nullptr && epi.out8 != nullptr && ldo % 16 == 0 &&
-                      aligned16(epi.out8);
+  const bool fused8 = epi.out32 == nullptr && epi.outf == nullptr && epi.out8 != nullptr &&
+                      ldo % 16 == 0 && aligned16(epi.out8);
   FcPlan plan = plan_fc(M, N, K, aligned, fused8, force);
   // a split the chooser proposed is dropped when the caller brought no room for it
   if (force.splits == 0 && plan.splits > 1 &&
@@ -482,14 +482,16 @@ void fc_entry(void* stream, const int8_t* data, const int8_t* weight, const int8
               int N, int K, const float* min_data, const float* max_data,
               const float* min_weight, const float* max_weight, const float* min_bias,
               const float* max_bias, int32_t* out32, float* omin, float* omax, int8_t* out8,
-              float* rmin, float* rmax, int relu, float min_calib, float max_calib,
-              void* workspace, size_t workspace_bytes, const GemmForce& force) {
+              float* out_f32, float* rmin, float* rmax, int relu, float min_calib,
+              float max_calib, void* workspace, size_t workspace_bytes, const GemmForce& force) {
   MXQ_CHECK(M >= 0 && N >= 0 && K >= 0, "negative dimension");
   MXQ_CHECK(min_data && max_data && min_weight && max_weight, "null input range pointer");
   MXQ_CHECK(omin && omax, "null output range pointer");
   MXQ_CHECK(bias == nullptr || (min_bias && max_bias), "bias given without its range");
-  MXQ_CHECK(M == 0 || N == 0 || out32 != nullptr || out8 != nullptr, "no output buffer");
-  MXQ_CHECK(out8 == nullptr || (rmin && rmax), "fused requantize needs rmin/rmax");
+  MXQ_CHECK(M == 0 || N == 0 || out32 != nullptr || out8 != nullptr || out_f32 != nullptr,
+            "no output buffer");
+  MXQ_CHECK((out8 == nullptr && out_f32 == nullptr) || (rmin && rmax),
+            "fused requantize needs rmin/rmax");
   MXQ_CHECK(M == 0 || N == 0 || K == 0 || (data != nullptr && weight != nullptr),
             "null operand pointer");
   Epilogue e;
@@ -502,6 +504,7 @@ void fc_entry(void* stream, const int8_t* data, const int8_t* weight, const int8
   e.max_bias = max_bias;
   e.out32 = out32;
   e.out8 = out8;
+  e.outf = out_f32;
   e.omin = omin;
   e.omax = omax;
   e.rmin = rmin;
@@ -536,8 +539,8 @@ int mxq_quantized_fc(void* stream, const int8_t* data, const int8_t* weight, con
                      float max_calib, void* workspace, size_t workspace_bytes) {
   MXQ_API_BEGIN();
   fc_entry(stream, data, weight, bias, M, N, K, min_data, max_data, min_weight, max_weight,
-           min_bias, max_bias, out32, omin, omax, out8, rmin, rmax, relu, min_calib, max_calib,
-           workspace, workspace_bytes, GemmForce());
+           min_bias, max_bias, out32, omin, omax, out8, nullptr, rmin, rmax, relu, min_calib,
+           max_calib, workspace, workspace_bytes, GemmForce());
   MXQ_API_END();
 }
 
@@ -559,8 +562,45 @@ int mxq_test_quantized_fc(void* stream, const int8_t* data, const int8_t* weight
   force.splits = splits;
   force.stream_groups = stream_groups;
   fc_entry(stream, data, weight, bias, M, N, K, min_data, max_data, min_weight, max_weight,
-           min_bias, max_bias, out32, omin, omax, out8, rmin, rmax, relu, min_calib, max_calib,
-           workspace, workspace_bytes, force);
+           min_bias, max_bias, out32, omin, omax, out8, nullptr, rmin, rmax, relu, min_calib,
+           max_calib, workspace, workspace_bytes, force);
+  MXQ_API_END();
+}
+
+int mxq_quantized_fc_f32(void* stream, const int8_t* data, const int8_t* weight,
+                         const int8_t* bias, int M, int N, int K, const float* min_data,
+                         const float* max_data, const float* min_weight, const float* max_weight,
+                         const float* min_bias, const float* max_bias, float* out_f32,
+                         float* omin, float* omax, float* rmin, float* rmax, int relu,
+                         float min_calib, float max_calib, void* workspace,
+                         size_t workspace_bytes) {
+  MXQ_API_BEGIN();
+  MXQ_CHECK(M == 0 || N == 0 || out_f32 != nullptr, "no output buffer");
+  fc_entry(stream, data, weight, bias, M, N, K, min_data, max_data, min_weight, max_weight,
+           min_bias, max_bias, nullptr, omin, omax, nullptr, out_f32, rmin, rmax, relu,
+           min_calib, max_calib, workspace, workspace_bytes, GemmForce());
+  MXQ_API_END();
+}
+
+// Test-only twin of mxq_quantized_fc_f32 with the tile configuration and the split-K factor
+// pinned (tests/mxq_test_hooks.h).
+int mxq_test_quantized_fc_f32(void* stream, const int8_t* data, const int8_t* weight,
+                              const int8_t* bias, int M, int N, int K, const float* min_data,
+                              const float* max_data, const float* min_weight,
+                              const float* max_weight, const float* min_bias,
+                              const float* max_bias, float* out_f32, float* omin, float* omax,
+                              float* rmin, float* rmax, int relu, float min_calib,
+                              float max_calib, void* workspace, size_t workspace_bytes, int cfg,
+                              int splits) {
+  MXQ_API_BEGIN();
+  MXQ_CHECK(M == 0 || N == 0 || out_f32 != nullptr, "no output buffer");
+  GemmForce force;
+  force.cfg = cfg;
+  force.splits = splits;
+  force.stream_groups = 0;
+  fc_entry(stream, data, weight, bias, M, N, K, min_data, max_data, min_weight, max_weight,
+           min_bias, max_bias, nullptr, omin, omax, nullptr, out_f32, rmin, rmax, relu,
+           min_calib, max_calib, workspace, workspace_bytes, force);
   MXQ_API_END();
 }
 

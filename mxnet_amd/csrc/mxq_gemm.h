@@ -53,6 +53,9 @@ struct Epilogue {
   const float* max_bias;
   int32_t* out32;          // [M][ldo] or null
   int8_t* out8;            // [M][ldo] or null
+  // [M][ldo] or null: the int8 result above taken back to float, q * (R / 127), i.e.
+  // what dequantize makes of the requantized output (dequantize-inl.h:64-75)
+  float* outf;
   float* omin;             // int32 output range
   float* omax;
   float* rmin;             // requantized range (only with out8)
@@ -107,6 +110,7 @@ struct EpiScalars {
   float foq, fbq;  // float per int32 level / per int8 bias level
   float in_scale;  // max_out / 2^31
   float qscale;    // 127 / R
+  float dqscale;   // R / 127: float per int8 level of the requantized output
 };
 
 __device__ __forceinline__ EpiScalars epi_scalars(const Epilogue& e) {
@@ -122,6 +126,7 @@ __device__ __forceinline__ EpiScalars epi_scalars(const Epilogue& e) {
     s.fbq = static_cast<float>(static_cast<double>(dev_maxabs(*e.min_bias, *e.max_bias)) / 127.0);
   s.in_scale = dev_maxabs(-s.max_out, s.max_out) / 2147483648.0f;
   s.qscale = 127.0f / dev_maxabs(-e.real_range, e.real_range);
+  s.dqscale = dev_maxabs(-e.real_range, e.real_range) / 127.0f;
   return s;
 }
 
@@ -151,6 +156,13 @@ __device__ __forceinline__ int epi_requant_relu(int acc, const EpiScalars& s) {
   float f = static_cast<float>(acc) * s.in_scale;
   float u = f * s.qscale + 0.5f;
   return static_cast<int>(__builtin_amdgcn_fmed3f(u, 0.0f, 127.0f));
+}
+
+// The requantized int8 value taken back to float (an int8 dequantize over the calibrated
+// range): float(q) * (R / 127), as bits.  The detour through the integer keeps +0 for a
+// magnitude that truncates to zero from below.
+__device__ __forceinline__ int epi_dequant_bits(int q, const EpiScalars& s) {
+  return __builtin_bit_cast(int, static_cast<float>(q) * s.dqscale);
 }
 
 // {a,b,c,d} low bytes -> one dword (a in byte 0).
@@ -688,18 +700,32 @@ __device__ __forceinline__ void gemm_epilogue(v16i (&acc)[Cfg::MI][Cfg::NI], con
               if (n + i < N) e.out32[off + i] = v[i];
           }
         }
-        if (e.out8 != nullptr) {
+        if (e.out8 != nullptr || e.outf != nullptr) {
           int q[4];
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
             q[i] = epi_requant(v[i], s, e.relu ? 0.0f : -127.0f);
           }
-          if (full) {
-            *reinterpret_cast<uint32_t*>(e.out8 + off) = pack_bytes(q[0], q[1], q[2], q[3]);
-          } else {
+          if (e.out8 != nullptr) {
+            if (full) {
+              *reinterpret_cast<uint32_t*>(e.out8 + off) = pack_bytes(q[0], q[1], q[2], q[3]);
+            } else {
 #pragma unroll
-            for (int i = 0; i < 4; ++i)
-              if (n + i < N) e.out8[off + i] = static_cast<int8_t>(q[i]);
+              for (int i = 0; i < 4; ++i)
+                if (n + i < N) e.out8[off + i] = static_cast<int8_t>(q[i]);
+            }
+          }
+          if (e.outf != nullptr) {
+            int* of = reinterpret_cast<int*>(e.outf);
+            if (full && (reinterpret_cast<uintptr_t>(e.outf) & 15u) == 0) {
+              v4i w = {epi_dequant_bits(q[0], s), epi_dequant_bits(q[1], s),
+                       epi_dequant_bits(q[2], s), epi_dequant_bits(q[3], s)};
+              *reinterpret_cast<v4i*>(of + off) = w;
+            } else {
+#pragma unroll
+              for (int i = 0; i < 4; ++i)
+                if (n + i < N) of[off + i] = epi_dequant_bits(q[i], s);
+            }
           }
         }
       }
@@ -768,7 +794,10 @@ __device__ __forceinline__ void gemm_epilogue_lds(v16i (&acc)[Cfg::MI][Cfg::NI],
   const bool fast32 = e.out32 == nullptr ||
                       ((N % 4 == 0) && (ldo % 4 == 0) &&
                        ((reinterpret_cast<uintptr_t>(e.out32) & 15u) == 0));
-  if (__builtin_expect(!(fast8 && fast32), 0)) {
+  const bool fastf = e.outf == nullptr ||
+                     ((N % 4 == 0) && (ldo % 4 == 0) &&
+                      ((reinterpret_cast<uintptr_t>(e.outf) & 15u) == 0));
+  if (__builtin_expect(!(fast8 && fast32 && fastf), 0)) {
     gemm_epilogue<Cfg>(acc, e, m_base, n_base, M, N, ldo);
     return;
   }
@@ -798,72 +827,21 @@ __device__ __forceinline__ void gemm_epilogue_lds(v16i (&acc)[Cfg::MI][Cfg::NI],
     }
   }
 
-  // Branch weights only place code: the fused int8 path, the one short launches take, stays
-  // contiguous, which shortens the instruction fetch of a launch whose code is cold (19-layer
-  // ResNet stack 264.8 -> 260.4 us; int32-output launches +0.4 %).
-  if (__builtin_expect(e.out32 != nullptr, 0)) {
+  // A 32-bit output, row-major: `quad(mi, ni, vq)` gives the 4 adjacent columns a lane holds
+  // of MFMA tile (mi, ni).  One 32 x 32 tile at a time through the wave's scratch: stored
+  // directly a lane's quads touch 32 rows with 32 bytes each; read back, 8 lanes cover one
+  // 128-byte row and a store instruction writes 8 whole cache lines.
+  auto store_rows32 = [&](int* out, auto quad) {
     if (kStage32) {
-      // One 32 x 32 MFMA tile at a time through the wave's scratch: a lane holds 4
-      // adjacent columns of one row per register quad, which stored directly touches 32
-      // rows with 32 bytes each; read back, 8 lanes cover one 128-byte row and a store
-      // instruction writes 8 whole cache lines.
       int* t32 = reinterpret_cast<int*>(stage);
 #pragma unroll
       for (int mi = 0; mi < MI; ++mi) {
 #pragma unroll
         for (int ni = 0; ni < NI; ++ni) {
-          if (e.plane > 0) {
-            // planar: the tile goes into the scratch channel-major (a lane's 16 values are
-            // one pixel of 16 channels; 32 lanes write 32 adjacent dwords), so that read
-            // back a lane holds 4 adjacent pixels of one channel and 8 lanes cover the
-            // tile's 32 pixels = one 128-byte run of that channel's plane (two runs where
-            // the tile straddles two images)
 #pragma unroll
-            for (int vq = 0; vq < 4; ++vq)
-#pragma unroll
-              for (int i = 0; i < 4; ++i)
-                t32[(8 * vq + 4 * lgrp + i) * Scratch::kPitch32 + lrow] = acc[mi][ni][4 * vq + i];
-            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-            __builtin_amdgcn_wave_barrier();
-            const int c = lane >> 3, p4 = (lane & 7) * 4;
-            v4i col[4];
-#pragma unroll
-            for (int it = 0; it < 4; ++it)
-              col[it] = *reinterpret_cast<const v4i*>(t32 + (it * 8 + c) * Scratch::kPitch32 + p4);
-            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-            __builtin_amdgcn_wave_barrier();
-            const int m0 = m_base + mi * 32 + p4;
-            const int img = m0 / e.plane, pix = m0 - img * e.plane;
-            const bool quad = (e.plane & 3) == 0;  // then 4 | pix and the quad is in one image
-#pragma unroll
-            for (int it = 0; it < 4; ++it) {
-              const int n = n_base + ni * 32 + it * 8 + c;
-              if (n >= N) continue;
-              if (quad) {
-                if (m0 < M)
-                  *reinterpret_cast<v4i*>(e.out32 + (static_cast<size_t>(img) * N + n) * e.plane +
-                                          pix) = col[it];
-              } else {
-                int im = img, px = pix;
-#pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                  if (m0 + j < M)
-                    e.out32[(static_cast<size_t>(im) * N + n) * e.plane + px] = col[it][j];
-                  if (++px == e.plane) {
-                    px = 0;
-                    ++im;
-                  }
-                }
-              }
-            }
-            continue;
-          }
-#pragma unroll
-          for (int vq = 0; vq < 4; ++vq) {
-            const v4i w = {acc[mi][ni][4 * vq], acc[mi][ni][4 * vq + 1], acc[mi][ni][4 * vq + 2],
-                           acc[mi][ni][4 * vq + 3]};
-            *reinterpret_cast<v4i*>(t32 + lrow * Scratch::kPitch32 + 8 * vq + 4 * lgrp) = w;
-          }
+          for (int vq = 0; vq < 4; ++vq)
+            *reinterpret_cast<v4i*>(t32 + lrow * Scratch::kPitch32 + 8 * vq + 4 * lgrp) =
+                quad(mi, ni, vq);
           asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
           __builtin_amdgcn_wave_barrier();
           v4i back[4];
@@ -879,7 +857,82 @@ __device__ __forceinline__ void gemm_epilogue_lds(v16i (&acc)[Cfg::MI][Cfg::NI],
             const int m = m_base + mi * 32 + it * 8 + (lane >> 3);
             const int n = n_base + ni * 32 + (lane & 7) * 4;
             if (m < M && n < N)
-              *reinterpret_cast<v4i*>(e.out32 + static_cast<size_t>(m) * ldo + n) = back[it];
+              *reinterpret_cast<v4i*>(out + static_cast<size_t>(m) * ldo + n) = back[it];
+          }
+        }
+      }
+    } else {
+#pragma unroll
+      for (int ni = 0; ni < NI; ++ni)
+#pragma unroll
+        for (int vq = 0; vq < 4; ++vq)
+#pragma unroll
+          for (int mi = 0; mi < MI; ++mi) {
+            const int m = m_base + mi * 32 + lrow, n = n_base + ni * 32 + 8 * vq + 4 * lgrp;
+            if (m < M && n < N)
+              *reinterpret_cast<v4i*>(out + static_cast<size_t>(m) * ldo + n) = quad(mi, ni, vq);
+          }
+    }
+  };
+  auto acc_quad = [&](int mi, int ni, int vq) {
+    return v4i{acc[mi][ni][4 * vq], acc[mi][ni][4 * vq + 1], acc[mi][ni][4 * vq + 2],
+               acc[mi][ni][4 * vq + 3]};
+  };
+
+  // Branch weights only place code: the fused int8 path, the one short launches take, stays
+  // contiguous, which shortens the instruction fetch of a launch whose code is cold (19-layer
+  // ResNet stack 264.8 -> 260.4 us; int32-output launches +0.4 %).
+  if (__builtin_expect(e.out32 != nullptr, 0)) {
+    if (e.plane == 0) {
+      store_rows32(e.out32, acc_quad);
+    } else if (kStage32) {
+      // planar: the tile goes into the scratch channel-major (a lane's 16 values are
+      // one pixel of 16 channels; 32 lanes write 32 adjacent dwords), so that read
+      // back a lane holds 4 adjacent pixels of one channel and 8 lanes cover the
+      // tile's 32 pixels = one 128-byte run of that channel's plane (two runs where
+      // the tile straddles two images)
+      int* t32 = reinterpret_cast<int*>(stage);
+#pragma unroll
+      for (int mi = 0; mi < MI; ++mi) {
+#pragma unroll
+        for (int ni = 0; ni < NI; ++ni) {
+#pragma unroll
+          for (int vq = 0; vq < 4; ++vq)
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+              t32[(8 * vq + 4 * lgrp + i) * Scratch::kPitch32 + lrow] = acc[mi][ni][4 * vq + i];
+          asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+          __builtin_amdgcn_wave_barrier();
+          const int c = lane >> 3, p4 = (lane & 7) * 4;
+          v4i col[4];
+#pragma unroll
+          for (int it = 0; it < 4; ++it)
+            col[it] = *reinterpret_cast<const v4i*>(t32 + (it * 8 + c) * Scratch::kPitch32 + p4);
+          asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+          __builtin_amdgcn_wave_barrier();
+          const int m0 = m_base + mi * 32 + p4;
+          const int img = m0 / e.plane, pix = m0 - img * e.plane;
+          const bool quad = (e.plane & 3) == 0;  // then 4 | pix and the quad is in one image
+#pragma unroll
+          for (int it = 0; it < 4; ++it) {
+            const int n = n_base + ni * 32 + it * 8 + c;
+            if (n >= N) continue;
+            if (quad) {
+              if (m0 < M)
+                *reinterpret_cast<v4i*>(e.out32 + (static_cast<size_t>(img) * N + n) * e.plane +
+                                        pix) = col[it];
+            } else {
+              int im = img, px = pix;
+#pragma unroll
+              for (int j = 0; j < 4; ++j) {
+                if (m0 + j < M)
+                  e.out32[(static_cast<size_t>(im) * N + n) * e.plane + px] = col[it][j];
+                if (++px == e.plane) {
+                  px = 0;
+                  ++im;
+                }
+              }
+            }
           }
         }
       }
@@ -892,19 +945,35 @@ __device__ __forceinline__ void gemm_epilogue_lds(v16i (&acc)[Cfg::MI][Cfg::NI],
           for (int mi = 0; mi < MI; ++mi) {
             const int m = m_base + mi * 32 + lrow, n = n_base + ni * 32 + 8 * vq + 4 * lgrp;
             if (m < M && n < N) {
-              const v4i w = {acc[mi][ni][4 * vq], acc[mi][ni][4 * vq + 1],
-                             acc[mi][ni][4 * vq + 2], acc[mi][ni][4 * vq + 3]};
-              if (e.plane > 0) {
-                const int img = m / e.plane, pix = m - img * e.plane;
+              const v4i w = acc_quad(mi, ni, vq);
+              const int img = m / e.plane, pix = m - img * e.plane;
 #pragma unroll
-                for (int i = 0; i < 4; ++i)  // N % 4 == 0 on this path
-                  e.out32[(static_cast<size_t>(img) * N + (n + i)) * e.plane + pix] = w[i];
-              } else {
-                *reinterpret_cast<v4i*>(e.out32 + static_cast<size_t>(m) * ldo + n) = w;
-              }
+              for (int i = 0; i < 4; ++i)  // N % 4 == 0 on this path
+                e.out32[(static_cast<size_t>(img) * N + (n + i)) * e.plane + pix] = w[i];
             }
           }
     }
+  }
+
+  // the requantized result as float: requantize, then the int8 dequantize over the
+  // calibrated range, element by element in registers
+  if (e.outf != nullptr) {
+    auto dequantized_tile = [&](auto relu) {
+      store_rows32(reinterpret_cast<int*>(e.outf), [&](int mi, int ni, int vq) {
+        v4i w;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int q = decltype(relu)::value ? epi_requant_relu(acc[mi][ni][4 * vq + i], s)
+                                              : epi_requant(acc[mi][ni][4 * vq + i], s, -127.0f);
+          w[i] = epi_dequant_bits(q, s);
+        }
+        return w;
+      });
+    };
+    if (e.relu)
+      dequantized_tile(std::true_type());
+    else
+      dequantized_tile(std::false_type());
   }
 
   if (e.out8 != nullptr) {
@@ -1088,7 +1157,8 @@ __device__ __forceinline__ void epilogue_ranges(const Epilogue& e) {
   const EpiScalars s = epi_scalars(e);
   *e.omin = -s.max_out;
   *e.omax = s.max_out;
-  if (e.out8 != nullptr && e.rmin != nullptr) {
+  // also for an output without elements, whose buffer pointer may be null
+  if (e.rmin != nullptr && e.rmax != nullptr) {
     *e.rmin = -e.real_range;
     *e.rmax = e.real_range;
   }

@@ -28,6 +28,16 @@ int mxq_test_quantized_fc(void* stream, const int8_t* data, const int8_t* weight
                           void* workspace, size_t workspace_bytes, int cfg, int splits,
                           int stream_groups);
 
+/* mxq_quantized_fc_f32 with the tile configuration and the split-K factor pinned. */
+int mxq_test_quantized_fc_f32(void* stream, const int8_t* data, const int8_t* weight,
+                              const int8_t* bias, int M, int N, int K, const float* min_data,
+                              const float* max_data, const float* min_weight,
+                              const float* max_weight, const float* min_bias,
+                              const float* max_bias, float* out_f32, float* omin, float* omax,
+                              float* rmin, float* rmax, int relu, float min_calib,
+                              float max_calib, void* workspace, size_t workspace_bytes, int cfg,
+                              int splits);
+
 /* mxq_quantized_conv_nhwc with the tile configuration (mxq_conv.hip lists them) and the
  * split-K factor pinned. */
 int mxq_test_quantized_conv_nhwc(void* stream, const int8_t* data, const int8_t* weight,

@@ -288,3 +288,90 @@ def test_fc_degenerate_extents(capi):
     ro, rmn, rmx = oracle_fc(d0, w0, b, 1.0, 0.08, 0.5)
     np.testing.assert_array_equal(res["out32"].cpu().numpy(), ro)
     assert (res["omin"].item(), res["omax"].item()) == (rmn, rmx)
+
+
+# ---- quantized_fc -> requantize -> dequantize in one launch ---------------------------------
+def oracle_fc_f32(d, w, b, rd, rw, rb, calib, relu):
+    """The three reference operators one after the other."""
+    ro, rmn, rmx = oracle_fc(d, w, b, rd, rw, rb)
+    rq, qmn, qmx = oracle.requantize(ro, rmn, rmx, *calib)
+    if relu:
+        rq = oracle.relu_i8(rq)
+    return oracle.dequantize(rq, qmn, qmx), (rmn, rmx), (qmn, qmx)
+
+
+def check_fc_f32(capi, d, w, b, calib, relu, force=None):
+    rd, rw, rb = 2.0, 0.1, 1.0
+    res = capi.quantized_fc_f32(dev(d), dev(w), None if b is None else dev(b), f32(-rd), f32(rd),
+                                f32(-rw), f32(rw), None if b is None else f32(-rb),
+                                None if b is None else f32(rb), calib=calib, relu=relu,
+                                force=force)
+    ref, r32, r8 = oracle_fc_f32(d, w, b, rd, rw, rb, calib, relu)
+    got = res["outf"].cpu().numpy()
+    # bit for bit, the sign of a zero included
+    np.testing.assert_array_equal(got.view(np.uint32), ref.view(np.uint32))
+    assert (res["omin"].item(), res["omax"].item()) == r32
+    assert (res["rmin"].item(), res["rmax"].item()) == r8
+
+
+@pytest.mark.parametrize("M,K,N", SHAPES + [(4096, 768, 768), (512, 3072, 772), (100, 64, 6)])
+@pytest.mark.parametrize("relu", [False, True])
+def test_fc_dequantized_output(capi, M, K, N, relu):
+    d = int8_uniform((M, K), seed=M + K + 2)
+    w = int8_uniform((N, K), seed=N + K + 3)
+    b = int8_uniform((N,), seed=N + 4) if (M + N) % 2 else None
+    ro, rmn, rmx = oracle_fc(d, w, b, 2.0, 0.1, 1.0)
+    fl = ro.astype(np.float64) * (float(rmx) / 2147483648.0)
+    R = float(np.percentile(np.abs(fl), 98.0)) or 1.0
+    check_fc_f32(capi, d, w, b, (-R, 0.85 * R), relu)
+
+
+@pytest.mark.parametrize("cfg", [1, 2, 3, 4, 11, 12, 14, 16, 21, 22, 23, 24, 31, 32, 41, 42, 43, 44,
+                                 51, 52, 53, 54, 55, 56, 57, 58, 59, 60])
+@pytest.mark.parametrize("M,K,N,splits", [(512, 512, 512, 1), (300, 192, 270, 1), (70, 448, 36, 1),
+                                          (257, 208, 64, 1), (300, 2064, 272, 3)])
+def test_fc_dequantized_output_every_tile_config(capi, cfg, M, K, N, splits):
+    if 10 < cfg < 20 and K % 64 != 0:
+        pytest.skip("the global-load direct-to-LDS kernels need K % 64 == 0")
+    if cfg < 10 and splits > 1:
+        pytest.skip("the register-staged kernels have no split-K form")
+    d = int8_uniform((M, K), seed=cfg + M + 11)
+    w = int8_uniform((N, K), seed=cfg + N + 13)
+    b = int8_uniform((N,), seed=cfg + 17)
+    check_fc_f32(capi, d, w, b, (-30.0, 28.0), bool(cfg % 2), force=(cfg, splits))
+
+
+def test_fc_dequantized_output_matches_the_three_kernels(capi):
+    """The fused launch against this library's own quantized_fc -> requantize -> dequantize."""
+    M, K, N = 4096, 768, 2304
+    d = int8_uniform((M, K), seed=31)
+    w = int8_uniform((N, K), seed=32, lo=-30, hi=30)
+    b = int8_uniform((N,), seed=33)
+    ranges = [f32(-1.0), f32(1.0), f32(-0.08), f32(0.08), f32(-0.5), f32(0.5)]
+    dd, wd, bd = dev(d), dev(w), dev(b)
+    res = capi.quantized_fc(dd, wd, bd, *ranges, want_int32=True)
+    fl = res["out32"].float() * (res["omax"].item() / 2147483648.0)
+    R = float(fl.abs().quantile(0.99).item())
+    q, qmn, qmx = capi.requantize(res["out32"], res["omin"], res["omax"], min_calib_range=-R,
+                                  max_calib_range=R)
+    y = capi.dequantize(q, qmn, qmx)
+    fused = capi.quantized_fc_f32(dd, wd, bd, *ranges, calib=(-R, R))
+    assert torch.equal(fused["outf"].view(torch.int32), y.view(torch.int32))
+    assert (fused["rmin"].item(), fused["rmax"].item()) == (qmn.item(), qmx.item())
+
+
+def test_fc_dequantized_output_degenerate(capi):
+    # no rows: only the range scalars are written
+    res = capi.quantized_fc_f32(torch.empty((0, 64), dtype=torch.int8, device="cuda"),
+                                dev(int8_uniform((32, 64), seed=1)), None, f32(-1.0), f32(1.0),
+                                f32(-1.0), f32(1.0), calib=(-2.0, 3.0))
+    assert res["outf"].shape == (0, 32)
+    assert (res["rmin"].item(), res["rmax"].item()) == (-3.0, 3.0)
+    # K = 0: every output is the requantized, dequantized bias
+    b = int8_uniform((40,), seed=2)
+    check_fc_f32(capi, np.zeros((5, 0), np.int8), np.zeros((40, 0), np.int8), b, (-0.5, 0.5),
+                 False)
+    from mxnet_amd._lib import last_error, lib
+    rc = lib.mxq_quantized_fc_f32(None, None, None, None, 4, 4, 16, None, None, None, None, None,
+                                  None, None, None, None, None, None, 0, 0.0, 1.0, None, 0)
+    assert rc != 0 and "no output buffer" in last_error()
