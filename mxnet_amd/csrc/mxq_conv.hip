@@ -388,17 +388,12 @@ __global__ __launch_bounds__(64 * kRowsWaves, 1) void conv3x3_rows_kernel(ConvAr
 #pragma unroll
             for (int vq = 0; vq < 4; ++vq) {
               const int nl = ni * 32 + 8 * vq + 4 * lgrp;
-              int q[4];
-#pragma unroll
-              for (int i = 0; i < 4; ++i) {
-                const int v = acc[mi][ni][4 * vq + i];
-                q[i] = decltype(with_relu)::value ? epi_requant_relu(v, s)
-                                                  : epi_requant(v, s, -127.0f);
-              }
+              const uint32_t w = epi_requant_pack<decltype(with_relu)::value>(
+                  acc[mi][ni][4 * vq], acc[mi][ni][4 * vq + 1], acc[mi][ni][4 * vq + 2],
+                  acc[mi][ni][4 * vq + 3], s);
               if (px < p.OW)
                 *reinterpret_cast<uint32_t*>(stage + px * kRowsO +
-                                             (((nl >> 4) ^ tile_swz(px)) << 4) + (nl & 15)) =
-                    pack_bytes(q[0], q[1], q[2], q[3]);
+                                             (((nl >> 4) ^ tile_swz(px)) << 4) + (nl & 15)) = w;
             }
         }
       };

@@ -27,7 +27,7 @@ struct FcArgs {
   SplitK sk;
 };
 
-template <class Cfg, bool ALIGNED>
+template <class Cfg, bool ALIGNED, bool F32OUT>
 __global__ __launch_bounds__(Cfg::kThreads, Cfg::kMinWaves) void fc_kernel(FcArgs p) {
   __shared__ __attribute__((aligned(16))) v4i lds[2][Cfg::STAGE_SLOTS];
   const int wave = threadIdx.x >> 6;
@@ -45,7 +45,7 @@ __global__ __launch_bounds__(Cfg::kThreads, Cfg::kMinWaves) void fc_kernel(FcArg
   v16i acc[Cfg::MI][Cfg::NI];
   gemm_mainloop<Cfg>(acc, af, bf, (p.K + Cfg::BK - 1) / Cfg::BK, lds);
 
-  gemm_epilogue<Cfg>(acc, p.epi, m0 + wm * Cfg::TM, n0 + wn * Cfg::TN, p.M, p.N,
+  gemm_epilogue<Cfg, F32OUT>(acc, p.epi, m0 + wm * Cfg::TM, n0 + wn * Cfg::TN, p.M, p.N,
                      static_cast<size_t>(p.ldo));
   if (blockIdx.x == 0 && threadIdx.x == 0) epilogue_ranges(p.epi);
 }
@@ -53,7 +53,9 @@ __global__ __launch_bounds__(Cfg::kThreads, Cfg::kMinWaves) void fc_kernel(FcArg
 // Direct-to-LDS variant (see gemm_mainloop_dma); launch_fc() picks it when the
 // operands qualify.  BUF selects buffer loads (any K % 16 == 0, zero-filled tails)
 // over global loads (K % 64 == 0, clamped rows).
-template <class Cfg, int NS, int PIPE, bool BUF>
+// F32OUT builds the float output (FcArgs::epi.outf) in: a kernel of its own, so that the int8
+// and int32 forms do not carry its code.
+template <class Cfg, int NS, int PIPE, bool BUF, bool F32OUT>
 __global__ __launch_bounds__(Cfg::kThreads, NS <= 2 ? Cfg::kMinWaves : 1) void fc_dma_kernel(FcArgs p) {
   __shared__ __attribute__((aligned(16))) v4i lds[NS * Cfg::STAGE_SLOTS];
   const int tiles_m = (p.M + Cfg::BM - 1) / Cfg::BM, tiles_n = (p.N + Cfg::BN - 1) / Cfg::BN;
@@ -92,7 +94,7 @@ __global__ __launch_bounds__(Cfg::kThreads, NS <= 2 ? Cfg::kMinWaves : 1) void f
   if (blockIdx.x == 0 && threadIdx.x == 0) epilogue_ranges(p.epi);
   if (__builtin_expect(p.sk.splits > 1, 0) && !splitk_gather<Cfg>(acc, p.sk, tile, z)) return;
 
-  gemm_epilogue_lds<Cfg, NS * Cfg::STAGE_SLOTS * 16>(acc, p.epi, pre, m0, n0, p.M, p.N,
+  gemm_epilogue_lds<Cfg, NS * Cfg::STAGE_SLOTS * 16, F32OUT>(acc, p.epi, pre, m0, n0, p.M, p.N,
                                                      static_cast<size_t>(p.ldo), lds);
 }
 
@@ -194,13 +196,10 @@ __global__ __launch_bounds__(256, 2) void fc_stream_kernel(FcArgs p, int bn, int
 #pragma unroll
         for (int vq = 0; vq < 4; ++vq) {
           const int nl = ni * 32 + 8 * vq + 4 * lgrp;
-          int q[4];
-#pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            const int v = acc[ni][4 * vq + i];
-            q[i] = decltype(with_relu)::value ? epi_requant_relu(v, s) : epi_requant(v, s, -127.0f);
-          }
-          *reinterpret_cast<uint32_t*>(stage + lrow * LD + nl) = pack_bytes(q[0], q[1], q[2], q[3]);
+          *reinterpret_cast<uint32_t*>(stage + lrow * LD + nl) =
+              epi_requant_pack<decltype(with_relu)::value>(acc[ni][4 * vq], acc[ni][4 * vq + 1],
+                                                           acc[ni][4 * vq + 2],
+                                                           acc[ni][4 * vq + 3], s);
         }
     };
     if (relu)
@@ -256,19 +255,29 @@ template <class Cfg, int NS, int PIPE, bool BUF>
 void launch_dma(hipStream_t s, FcArgs a, int splits, const Workspace& ws) {
   const long tiles = static_cast<long>((a.M + Cfg::BM - 1) / Cfg::BM) * ((a.N + Cfg::BN - 1) / Cfg::BN);
   splitk_setup<Cfg>(s, a.sk, tiles, a.K, splits, ws.ptr, ws.bytes);
-  hipLaunchKernelGGL((fc_dma_kernel<Cfg, NS, PIPE, BUF>),
-                     dim3(static_cast<unsigned>(tiles * a.sk.splits)), dim3(Cfg::kThreads), 0, s,
-                     a);
+  if (a.epi.outf != nullptr)
+    hipLaunchKernelGGL((fc_dma_kernel<Cfg, NS, PIPE, BUF, true>),
+                       dim3(static_cast<unsigned>(tiles * a.sk.splits)), dim3(Cfg::kThreads), 0,
+                       s, a);
+  else
+    hipLaunchKernelGGL((fc_dma_kernel<Cfg, NS, PIPE, BUF, false>),
+                       dim3(static_cast<unsigned>(tiles * a.sk.splits)), dim3(Cfg::kThreads), 0,
+                       s, a);
   MXQ_LAUNCH_CHECK();
 }
 
 template <class Cfg>
 void launch_cfg(hipStream_t s, const FcArgs& a, bool aligned) {
   const int tiles = ((a.M + Cfg::BM - 1) / Cfg::BM) * ((a.N + Cfg::BN - 1) / Cfg::BN);
-  if (aligned)
-    hipLaunchKernelGGL((fc_kernel<Cfg, true>), dim3(tiles), dim3(Cfg::kThreads), 0, s, a);
+  const bool f32 = a.epi.outf != nullptr;
+  if (aligned && f32)
+    hipLaunchKernelGGL((fc_kernel<Cfg, true, true>), dim3(tiles), dim3(Cfg::kThreads), 0, s, a);
+  else if (aligned)
+    hipLaunchKernelGGL((fc_kernel<Cfg, true, false>), dim3(tiles), dim3(Cfg::kThreads), 0, s, a);
+  else if (f32)
+    hipLaunchKernelGGL((fc_kernel<Cfg, false, true>), dim3(tiles), dim3(Cfg::kThreads), 0, s, a);
   else
-    hipLaunchKernelGGL((fc_kernel<Cfg, false>), dim3(tiles), dim3(Cfg::kThreads), 0, s, a);
+    hipLaunchKernelGGL((fc_kernel<Cfg, false, false>), dim3(tiles), dim3(Cfg::kThreads), 0, s, a);
   MXQ_LAUNCH_CHECK();
 }
 

@@ -174,6 +174,19 @@ __device__ __forceinline__ uint32_t pack_bytes(int a, int b, int c, int d) {
   return lo | hi;
 }
 
+// Four requantized outputs as one dword (first in byte 0).  (Converting the relu'd values as
+// unsigned and or-ing them without byte masks saves a quarter instruction per output and
+// measures the same: 19-layer stack 261.7 against 260.3 us.)
+template <bool RELU>
+__device__ __forceinline__ uint32_t epi_requant_pack(int a0, int a1, int a2, int a3,
+                                                     const EpiScalars& s) {
+  if (RELU)
+    return pack_bytes(epi_requant_relu(a0, s), epi_requant_relu(a1, s), epi_requant_relu(a2, s),
+                      epi_requant_relu(a3, s));
+  return pack_bytes(epi_requant(a0, s, -127.0f), epi_requant(a1, s, -127.0f),
+                    epi_requant(a2, s, -127.0f), epi_requant(a3, s, -127.0f));
+}
+
 // Bank-spreading XOR for the chunk index.  A fragment read is 32 consecutive
 // rows at one logical chunk, 16 bytes per lane.  For CH = 4 the function is a
 // bijection of row bits (1,2) for fixed bits (0,3) and of bits (2,3) for fixed
@@ -657,7 +670,9 @@ __device__ __forceinline__ void gemm_mainloop_dma(v16i (&acc)[Cfg::MI][Cfg::NI],
 }
 
 // Stores one wave's accumulators.  m_base/n_base: origin of the wave tile.
-template <class Cfg>
+// F32OUT: the kernel can also write Epilogue::outf (only the fully-connected kernels are
+// built that way; elsewhere the code for it is left out, which keeps cold kernels short).
+template <class Cfg, bool F32OUT = false>
 __device__ __forceinline__ void gemm_epilogue(v16i (&acc)[Cfg::MI][Cfg::NI], const Epilogue& e,
                                               int m_base, int n_base, int M, int N,
                                               size_t ldo) {
@@ -700,7 +715,7 @@ __device__ __forceinline__ void gemm_epilogue(v16i (&acc)[Cfg::MI][Cfg::NI], con
               if (n + i < N) e.out32[off + i] = v[i];
           }
         }
-        if (e.out8 != nullptr || e.outf != nullptr) {
+        if (e.out8 != nullptr || (F32OUT && e.outf != nullptr)) {
           int q[4];
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
@@ -715,7 +730,7 @@ __device__ __forceinline__ void gemm_epilogue(v16i (&acc)[Cfg::MI][Cfg::NI], con
                 if (n + i < N) e.out8[off + i] = static_cast<int8_t>(q[i]);
             }
           }
-          if (e.outf != nullptr) {
+          if (F32OUT && e.outf != nullptr) {
             int* of = reinterpret_cast<int*>(e.outf);
             if (full && (reinterpret_cast<uintptr_t>(e.outf) & 15u) == 0) {
               v4i w = {epi_dequant_bits(q[0], s), epi_dequant_bits(q[1], s),
@@ -771,7 +786,7 @@ struct EpiScratch {
   static constexpr int kNeed32 = Cfg::BN * 4 + kWaves * kPerWave;
 };
 
-template <class Cfg, int RING_BYTES>
+template <class Cfg, int RING_BYTES, bool F32OUT = false>
 __device__ __forceinline__ void gemm_epilogue_lds(v16i (&acc)[Cfg::MI][Cfg::NI],
                                                   const Epilogue& e, const EpiPre& pre, int m0,
                                                   int n0, int M, int N, size_t ldo,
@@ -794,11 +809,11 @@ __device__ __forceinline__ void gemm_epilogue_lds(v16i (&acc)[Cfg::MI][Cfg::NI],
   const bool fast32 = e.out32 == nullptr ||
                       ((N % 4 == 0) && (ldo % 4 == 0) &&
                        ((reinterpret_cast<uintptr_t>(e.out32) & 15u) == 0));
-  const bool fastf = e.outf == nullptr ||
+  const bool fastf = !F32OUT || e.outf == nullptr ||
                      ((N % 4 == 0) && (ldo % 4 == 0) &&
                       ((reinterpret_cast<uintptr_t>(e.outf) & 15u) == 0));
   if (__builtin_expect(!(fast8 && fast32 && fastf), 0)) {
-    gemm_epilogue<Cfg>(acc, e, m_base, n_base, M, N, ldo);
+    gemm_epilogue<Cfg, F32OUT>(acc, e, m_base, n_base, M, N, ldo);
     return;
   }
   char* lds = reinterpret_cast<char*>(lds_v);
@@ -957,7 +972,7 @@ __device__ __forceinline__ void gemm_epilogue_lds(v16i (&acc)[Cfg::MI][Cfg::NI],
 
   // the requantized result as float: requantize, then the int8 dequantize over the
   // calibrated range, element by element in registers
-  if (e.outf != nullptr) {
+  if (F32OUT && e.outf != nullptr) {
     auto dequantized_tile = [&](auto relu) {
       store_rows32(reinterpret_cast<int*>(e.outf), [&](int mi, int ni, int vq) {
         v4i w;
@@ -985,13 +1000,10 @@ __device__ __forceinline__ void gemm_epilogue_lds(v16i (&acc)[Cfg::MI][Cfg::NI],
 #pragma unroll
           for (int mi = 0; mi < MI; ++mi) {
             const int nl = ni * 32 + 8 * vq + 4 * lgrp, ml = mi * 32 + lrow;
-            int q[4];
-#pragma unroll
-            for (int i = 0; i < 4; ++i)
-              q[i] = decltype(relu)::value ? epi_requant_relu(acc[mi][ni][4 * vq + i], s)
-                                           : epi_requant(acc[mi][ni][4 * vq + i], s, -127.0f);
             *reinterpret_cast<uint32_t*>(stage + ml * LD + nl) =
-                pack_bytes(q[0], q[1], q[2], q[3]);
+                epi_requant_pack<decltype(relu)::value>(acc[mi][ni][4 * vq], acc[mi][ni][4 * vq + 1],
+                                                        acc[mi][ni][4 * vq + 2],
+                                                        acc[mi][ni][4 * vq + 3], s);
           }
     };
     if (e.relu)
