@@ -73,6 +73,13 @@ def test_fc_random_shape(capi, M, N, K):
                              None if b is None else f32(rb), want_int32=False,
                              calib=(-R, 0.8 * R), relu=relu)
     np.testing.assert_array_equal(res8["out8"].cpu().numpy(), rq)
+    # requantize and dequantize both in the launch: the float the three operators give
+    resf = capi.quantized_fc_f32(dev(d), dev(w), None if b is None else dev(b), f32(-rd), f32(rd),
+                                 f32(-rw), f32(rw), None if b is None else f32(-rb),
+                                 None if b is None else f32(rb), calib=(-R, 0.8 * R), relu=relu)
+    ref = oracle.dequantize(rq, qmn, qmx)
+    np.testing.assert_array_equal(resf["outf"].cpu().numpy().view(np.uint32), ref.view(np.uint32))
+    assert (resf["rmin"].item(), resf["rmax"].item()) == (qmn, qmx)
 
 
 def conv_cases():
