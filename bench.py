@@ -40,7 +40,7 @@ INT8_PEAK_TOPS = 5000.0  # MI355X dense int8 MFMA
 # null.
 _KIB = 1024.0
 MEASURED_TRAFFIC_BYTES = {
-    "fc4096": ((2.0 * 49289.3 + 16384.1) * _KIB, "profiles/fc_dma_kernel_4096.md"),
+    "fc4096": ((2.0 * 49277.4 + 16384.1) * _KIB, "profiles/fc_dma_kernel_4096.md"),
     "quantize": ((2.0 * 131102.5 + 65536.1) * _KIB, "profiles/quantize_kernel_64M.md"),
     "quantize_uncal": ((2.0 * (131093.7 + 131139.1) + 65536.1) * _KIB, "profiles/quantize_uncalibrated_64M.md"),
     "requantize": ((2.0 * 131104.8 + 65536.1) * _KIB, "profiles/requantize_kernel_64M.md"),
