@@ -71,6 +71,7 @@ def parse_args():
                              "requantize", "requantize_uncal", "dequantize", "copy", "maxpool", "avgpool",
                              "elemwise_add", "elemwise_add_int8", "concat", "elemwise_mul_int8", "quantize_asym",
                              "batch_norm", "embedding", "transpose", "resnet50_convs", "resnet50_chain",
+                             "resnet50_chain_fused",
                              "bert_fc_chain",
                              "bert_fc_chain_fused",
                              "bert_fc_chain_f32"])
@@ -740,11 +741,16 @@ class ResNetChainWorkload(GraphWorkload):
     16 relus per step; stem, pooling and the classifier are not part of it."""
     STAGES = [(3, 64, 256, 1), (4, 128, 512, 2), (6, 256, 1024, 2), (3, 512, 2048, 2)]
 
-    def __init__(self, torch, capi, lib):
+    def __init__(self, torch, capi, lib, fused_sum=False):
         self.kernel = "conv / fc kernels, add_kernel, relu"
         self.bound = "mfma"
         self.name = "ResNet-50 v1 bottleneck body as a chain (52 convolutions + 16 residual " \
                     "adds + relus), batch 64, NHWC int8, requantize fused"
+        if fused_sum:
+            self.kernel = "conv / fc kernels, the residual sum and its relu in the epilogue of " \
+                          "each block's last 1x1 convolution"
+            self.name += ", residual add + relu fused into the block's last convolution " \
+                         "(mxq_quantized_fc_sum)"
         P = lambda t: ctypes.c_void_p(t.data_ptr()) if t is not None else None
         g = torch.Generator(device="cuda").manual_seed(44)
         N, H = 64, 56
@@ -754,8 +760,10 @@ class ResNetChainWorkload(GraphWorkload):
         self.calls, self.ops, self.keep = [], 0.0, []
         f1 = lambda v: torch.tensor([v], dtype=torch.float32, device="cuda")
 
-        def conv(inp, imin, imax, H, C, O, k, s, relu):
-            """Adds one fused convolution to the chain; returns its int8 output and range."""
+        def conv(inp, imin, imax, H, C, O, k, s, relu, record=True):
+            """Adds one fused convolution to the chain; returns its int8 output and range
+            (record=False: runs it once for the calibration of what follows, outside the
+            chain, and also returns what a fused call needs)."""
             pad = 1 if k == 3 else 0
             OH = (H + 2 * pad - k) // s + 1
             w = torch.randn((O, k, k, C), device="cuda", generator=g) * (2.0 / (k * k * C)) ** 0.5
@@ -777,12 +785,15 @@ class ResNetChainWorkload(GraphWorkload):
             args = (P(inp), P(wq), P(bq), *geo, 1, 1, P(imin), P(imax), P(wmin), P(wmax), P(bmin),
                     P(bmax), None, P(sc[0]), P(sc[1]), P(out8), P(sc[2]), P(sc[3]), int(relu), -r,
                     r, *ws_args(ws))
-            self.calls.append((lib.mxq_quantized_conv_nhwc, args))
+            if record:
+                self.calls.append((lib.mxq_quantized_conv_nhwc, args))
             self.keep.append((inp, wq, bq, imin, imax, wmin, wmax, bmin, bmax, out8, sc, ws))
             self.ops += 2.0 * N * OH * OH * O * k * k * C
             st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
             if lib.mxq_quantized_conv_nhwc(st, *args):
                 raise RuntimeError(lib.mxq_last_error().decode())
+            if not record:
+                return out8, sc[2], sc[3], OH, (wq, bq, wmin, wmax, bmin, bmax, r, ws)
             return out8, sc[2], sc[3], OH
 
         for (blocks, mid, out, stride) in self.STAGES:
@@ -791,11 +802,15 @@ class ResNetChainWorkload(GraphWorkload):
                 C = cur.shape[3]
                 a, amin, amax, H1 = conv(cur, cmin, cmax, H, C, mid, 1, s, True)
                 b, bmin_, bmax_, _ = conv(a, amin, amax, H1, mid, mid, 3, 1, True)
-                c, cmin_, cmax_, _ = conv(b, bmin_, bmax_, H1, mid, out, 1, 1, False)
                 if bi == 0:
                     sh, smin, smax, _ = conv(cur, cmin, cmax, H, C, out, 1, s, False)
                 else:
                     sh, smin, smax = cur, cmin, cmax
+                if fused_sum:
+                    c, cmin_, cmax_, _, (wq3, bq3, w3min, w3max, b3min, b3max, r3, ws3) = conv(
+                        b, bmin_, bmax_, H1, mid, out, 1, 1, False, record=False)
+                else:
+                    c, cmin_, cmax_, _ = conv(b, bmin_, bmax_, H1, mid, out, 1, 1, False)
                 # residual sum, int8 out with a calibrated range, then the quantized ReLU
                 fa = capi.dequantize(c, cmin_, cmax_) + capi.dequantize(sh, smin, smax)
                 r = max(float(fa.abs().max().item()), 1e-6)
@@ -803,6 +818,34 @@ class ResNetChainWorkload(GraphWorkload):
                 y = torch.empty_like(c)
                 ysc = [torch.empty(1, device="cuda") for _ in range(4)]
                 z = torch.empty_like(c)
+                if fused_sum:
+                    # the block's last 1x1 convolution is the FC of its flattened pixels
+                    Mrows = N * H1 * H1
+                    fargs = (P(b), P(wq3), P(bq3), Mrows, out, mid, P(bmin_), P(bmax_), P(w3min),
+                             P(w3max), P(b3min), P(b3max), P(sh), P(smin), P(smax), P(z),
+                             P(ysc[0]), P(ysc[1]), P(ysc[2]), P(ysc[3]), -r3, r3, -r, r, 1,
+                             *ws_args(ws3))
+                    self.calls.append((lib.mxq_quantized_fc_sum, fargs))
+                    self.keep.append((c, sh, y, z, ysc))
+                    st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+                    if lib.mxq_quantized_fc_sum(st, *fargs):
+                        raise RuntimeError(lib.mxq_last_error().decode())
+                    # the three operators on the same tensors must give the same bytes
+                    z3 = torch.empty_like(c)
+                    zsc = [torch.empty(1, device="cuda") for _ in range(4)]
+                    rcs = [lib.mxq_quantized_elemwise_add(st, P(c), 5, P(sh), 5, P(cmin_),
+                                                          P(cmax_), P(smin), P(smax), P(y), 5,
+                                                          P(zsc[0]), P(zsc[1]), c.numel(), 1,
+                                                          -r, r),
+                           lib.mxq_quantized_relu(st, P(y), P(zsc[0]), P(zsc[1]), P(z3),
+                                                  P(zsc[2]), P(zsc[3]), y.numel())]
+                    if any(rcs):
+                        raise RuntimeError(lib.mxq_last_error().decode())
+                    if not torch.equal(z, z3):
+                        raise RuntimeError("fused residual sum differs from the three operators")
+                    del z3
+                    cur, cmin, cmax, H = z, ysc[2], ysc[3], H1
+                    continue
                 add_args = (P(c), 5, P(sh), 5, P(cmin_), P(cmax_), P(smin), P(smax), P(y), 5,
                             P(ysc[0]), P(ysc[1]), c.numel(), 1, -r, r)
                 relu_args = (P(y), P(ysc[0]), P(ysc[1]), P(z), P(ysc[2]), P(ysc[3]), y.numel())
@@ -988,6 +1031,8 @@ def make_workload(name, torch, capi, lib):
         return ConvStackWorkload(torch, capi, lib)
     if name == "resnet50_chain":
         return ResNetChainWorkload(torch, capi, lib)
+    if name == "resnet50_chain_fused":
+        return ResNetChainWorkload(torch, capi, lib, fused_sum=True)
     if name == "bert_fc_chain":
         return BertChainWorkload(torch, capi, lib)
     if name == "bert_fc_chain_fused":
@@ -1113,8 +1158,8 @@ def main():
                      "requantize_uncal", "dequantize", "elemwise_add", "elemwise_add_int8",
                      "concat", "elemwise_mul_int8", "quantize_asym", "batch_norm", "embedding",
                      "transpose", "maxpool", "avgpool", "fc8192",
-                     "resnet50_convs", "resnet50_chain", "bert_fc_chain", "bert_fc_chain_fused",
-                     "bert_fc_chain_f32"]:
+                     "resnet50_convs", "resnet50_chain", "resnet50_chain_fused", "bert_fc_chain",
+                     "bert_fc_chain_fused", "bert_fc_chain_f32"]:
             if kind == args.workload:
                 continue
             w2 = make_workload(kind, torch, capi, lib)

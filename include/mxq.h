@@ -314,6 +314,29 @@ int mxq_quantized_fc_f32(void* stream, const int8_t* data, const int8_t* weight,
                          float min_calib, float max_calib, void* workspace,
                          size_t workspace_bytes);
 
+/* _contrib_quantized_fully_connected -> _contrib_requantize -> _contrib_quantized_elemwise_add
+ * (-> _contrib_quantized_act) in one launch: a layer whose requantized int8 output is added
+ * to a second int8 tensor of the same shape, the residual sum of a bottleneck block
+ * (quantized_fully_connected.cu:58-138, requantize-inl.h:89-125,
+ * quantized_elemwise_add.cc:30-134 / dnnl/dnnl_quantized_elemwise_add.cc:134-257 with a
+ * calibrated int8 output, quantized_activation.cc:84-120).  In NHWC a 1x1 unit-stride
+ * unpadded convolution is this call on the flattened pixels (M = N*H*W, K = C, N = O).
+ *   residual       int8 [M,N], range (min_residual, max_residual)
+ *   min/max_calib  the layer's own requantization range, as for mxq_quantized_fc
+ *   sum_*_calib    the sum's calibrated range; rmin / rmax receive it
+ *   sum_relu != 0  clamps the sum at zero
+ * out8 is bit-identical to mxq_quantized_elemwise_add(out8 of mxq_quantized_fc, residual)
+ * followed by mxq_quantized_relu; neither intermediate tensor is stored.  Workspace as for
+ * mxq_quantized_fc with fused_int8_only = 1. */
+int mxq_quantized_fc_sum(void* stream, const int8_t* data, const int8_t* weight,
+                         const int8_t* bias, int M, int N, int K, const float* min_data,
+                         const float* max_data, const float* min_weight, const float* max_weight,
+                         const float* min_bias, const float* max_bias, const int8_t* residual,
+                         const float* min_residual, const float* max_residual, int8_t* out8,
+                         float* omin, float* omax, float* rmin, float* rmax, float min_calib,
+                         float max_calib, float sum_min_calib, float sum_max_calib, int sum_relu,
+                         void* workspace, size_t workspace_bytes);
+
 /* ---- _contrib_quantized_conv ----------------------------------------------
  * Replaces QuantizedCuDNNConvOp::Forward
  * (src/operator/quantization/quantized_conv.cu:101-219): the NHWC int8

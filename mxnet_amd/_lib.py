@@ -62,6 +62,8 @@ SIGNATURES = {
                               _i, _f, _f, _p, _sz]),
     "mxq_quantized_fc_f32": (_i, [_p, _p, _p, _p, _i, _i, _i] + [_p] * 6 + [_p, _p, _p, _p, _p,
                                   _i, _f, _f, _p, _sz]),
+    "mxq_quantized_fc_sum": (_i, [_p, _p, _p, _p, _i, _i, _i] + [_p] * 6 + [_p, _p, _p] +
+                             [_p, _p, _p, _p, _p, _f, _f, _f, _f, _i, _p, _sz]),
     "mxq_quantized_conv_workspace": (_sz, [_i] * 14),
     "mxq_quantized_conv_nhwc": (_i, [_p, _p, _p, _p] + [_i] * 13 + [_p] * 6 +
                                 [_p, _p, _p, _p, _p, _p, _i, _f, _f, _p, _sz]),
@@ -83,6 +85,7 @@ for _name, (_res, _args) in SIGNATURES.items():
 # factor and, for the FC, the streaming kernel's work-groups per CU (0 = choose)
 TEST_HOOKS = {
     "mxq_test_quantized_fc": (_i, SIGNATURES["mxq_quantized_fc"][1] + [_i, _i, _i]),
+    "mxq_test_quantized_fc_sum": (_i, SIGNATURES["mxq_quantized_fc_sum"][1] + [_i, _i, _i]),
     "mxq_test_quantized_fc_f32": (_i, SIGNATURES["mxq_quantized_fc_f32"][1] + [_i, _i]),
     "mxq_test_quantized_conv_nhwc": (_i, SIGNATURES["mxq_quantized_conv_nhwc"][1] + [_i, _i]),
 }

@@ -152,6 +152,36 @@ def quantized_fc_f32(data, weight, bias, min_data, max_data, min_weight, max_wei
     return res
 
 
+def quantized_fc_sum(data, weight, bias, residual, min_data, max_data, min_weight, max_weight,
+                     min_bias, max_bias, min_residual, max_residual, calib, sum_calib,
+                     sum_relu=False, force=None):
+    """quantized_fc -> requantize over `calib` -> elemwise_add with `residual` over `sum_calib`
+    (-> relu) in one launch.  Returns dict(out8, omin, omax, rmin, rmax).  `force` = (cfg,
+    splits, stream_groups) pins the kernel variant through the test-only entry point."""
+    M, K = data.shape
+    N, K2 = weight.shape
+    assert K == K2 and tuple(residual.shape) == (M, N) and residual.dtype == torch.int8
+    dev = data.device
+    res = {k: _scalar(dev) for k in ("omin", "omax", "rmin", "rmax")}
+    res["out8"] = torch.empty((M, N), dtype=torch.int8, device=dev)
+    args = [_stream(), _ptr(data), _ptr(weight), _ptr(bias), M, N, K, _ptr(min_data),
+            _ptr(max_data), _ptr(min_weight), _ptr(max_weight), _ptr(min_bias), _ptr(max_bias),
+            _ptr(residual), _ptr(min_residual), _ptr(max_residual), _ptr(res["out8"]),
+            _ptr(res["omin"]), _ptr(res["omax"]), _ptr(res["rmin"]), _ptr(res["rmax"]),
+            float(calib[0]), float(calib[1]), float(sum_calib[0]), float(sum_calib[1]),
+            int(sum_relu)]
+    if force is None:
+        wsb = lib.mxq_quantized_fc_workspace(M, N, K, 1)
+        ws = _workspace(wsb, dev) if wsb else None
+        check(lib.mxq_quantized_fc_sum(*args, _ptr(ws), wsb))
+    else:
+        cfg, splits, groups = force
+        wsb = _SPLIT_WS_BYTES if splits > 1 else 0
+        ws = _workspace(wsb, dev) if wsb else None
+        check(lib.mxq_test_quantized_fc_sum(*args, _ptr(ws), wsb, cfg, splits, groups))
+    return res
+
+
 def quantized_conv_nhwc(data, weight, bias, min_data, max_data, min_weight, max_weight,
                         min_bias=None, max_bias=None, stride=(1, 1), pad=(0, 0), dilate=(1, 1),
                         want_int32=True, calib=None, relu=False, force=None):

@@ -753,6 +753,8 @@ void conv_nhwc(void* stream, const int8_t* data, const int8_t* weight, const int
   e.min_weight = min_weight; e.max_weight = max_weight;
   e.min_bias = min_bias; e.max_bias = max_bias;
   e.out32 = out32; e.out8 = out8; e.outf = nullptr;
+  e.res = nullptr; e.res_min = nullptr; e.res_max = nullptr;
+  e.sum_min_calib = 0.f; e.sum_max_calib = 0.f; e.sum_relu = 0; e.with_sum = 0;
   e.omin = omin; e.omax = omax; e.rmin = rmin; e.rmax = rmax;
   e.relu = relu;
   float x = fabsf(min_calib), y = fabsf(max_calib);

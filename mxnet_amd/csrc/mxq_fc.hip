@@ -27,7 +27,7 @@ struct FcArgs {
   SplitK sk;
 };
 
-template <class Cfg, bool ALIGNED, bool F32OUT>
+template <class Cfg, bool ALIGNED, int MODE>
 __global__ __launch_bounds__(Cfg::kThreads, Cfg::kMinWaves) void fc_kernel(FcArgs p) {
   __shared__ __attribute__((aligned(16))) v4i lds[2][Cfg::STAGE_SLOTS];
   const int wave = threadIdx.x >> 6;
@@ -45,17 +45,17 @@ __global__ __launch_bounds__(Cfg::kThreads, Cfg::kMinWaves) void fc_kernel(FcArg
   v16i acc[Cfg::MI][Cfg::NI];
   gemm_mainloop<Cfg>(acc, af, bf, (p.K + Cfg::BK - 1) / Cfg::BK, lds);
 
-  gemm_epilogue<Cfg, F32OUT>(acc, p.epi, m0 + wm * Cfg::TM, n0 + wn * Cfg::TN, p.M, p.N,
+  gemm_epilogue<Cfg, MODE>(acc, p.epi, m0 + wm * Cfg::TM, n0 + wn * Cfg::TN, p.M, p.N,
                      static_cast<size_t>(p.ldo));
-  if (blockIdx.x == 0 && threadIdx.x == 0) epilogue_ranges(p.epi);
+  if (blockIdx.x == 0 && threadIdx.x == 0) epilogue_ranges<MODE>(p.epi);
 }
 
 // Direct-to-LDS variant (see gemm_mainloop_dma); launch_fc() picks it when the
 // operands qualify.  BUF selects buffer loads (any K % 16 == 0, zero-filled tails)
 // over global loads (K % 64 == 0, clamped rows).
-// F32OUT builds the float output (FcArgs::epi.outf) in: a kernel of its own, so that the int8
-// and int32 forms do not carry its code.
-template <class Cfg, int NS, int PIPE, bool BUF, bool F32OUT>
+// MODE (kEpiPlain / kEpiF32 / kEpiSum) builds the float output or the residual sum in: kernels
+// of their own, so that the int8 and int32 forms do not carry their code.
+template <class Cfg, int NS, int PIPE, bool BUF, int MODE>
 __global__ __launch_bounds__(Cfg::kThreads, NS <= 2 ? Cfg::kMinWaves : 1) void fc_dma_kernel(FcArgs p) {
   __shared__ __attribute__((aligned(16))) v4i lds[NS * Cfg::STAGE_SLOTS];
   const int tiles_m = (p.M + Cfg::BM - 1) / Cfg::BM, tiles_n = (p.N + Cfg::BN - 1) / Cfg::BN;
@@ -70,7 +70,7 @@ __global__ __launch_bounds__(Cfg::kThreads, NS <= 2 ? Cfg::kMinWaves : 1) void f
 
   // what the epilogue needs is fetched while the first operand stages are in flight
   EpiPre pre;
-  auto prefetch = [&]() { pre = epi_prefetch<Cfg>(p.epi, n0, p.N); };
+  auto prefetch = [&]() { pre = epi_prefetch<Cfg, MODE>(p.epi, n0, p.N); };
   v16i acc[Cfg::MI][Cfg::NI];
   // this work-group's K slice: stages [kt0, kt0 + KT) (all of them without a split)
   const int kt_all = (p.K + Cfg::BK - 1) / Cfg::BK;
@@ -91,11 +91,11 @@ __global__ __launch_bounds__(Cfg::kThreads, NS <= 2 ? Cfg::kMinWaves : 1) void f
     gemm_mainloop_dma<Cfg, NS, PIPE>(acc, ai, bi, KT, lds, prefetch);
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-  if (blockIdx.x == 0 && threadIdx.x == 0) epilogue_ranges(p.epi);
+  if (blockIdx.x == 0 && threadIdx.x == 0) epilogue_ranges<MODE>(p.epi);
   if (__builtin_expect(p.sk.splits > 1, 0) && !splitk_gather<Cfg>(acc, p.sk, tile, z)) return;
 
-  gemm_epilogue_lds<Cfg, NS * Cfg::STAGE_SLOTS * 16, F32OUT>(acc, p.epi, pre, m0, n0, p.M, p.N,
-                                                     static_cast<size_t>(p.ldo), lds);
+  gemm_epilogue_lds<Cfg, NS * Cfg::STAGE_SLOTS * 16, MODE>(acc, p.epi, pre, m0, n0, p.M, p.N,
+                                                           static_cast<size_t>(p.ldo), lds);
 }
 
 typedef GemmCfg<256, 256, 64, 2, 4> CfgL8;    // 8 waves, wave tile 128 x 64
@@ -123,7 +123,8 @@ typedef GemmCfg<256, 192, 128, 4, 2> CfgW192K; // 8 waves, wave tile 64 x 96
 // the next item's fragment requested before the current one is multiplied, weights read from
 // LDS, then the fused epilogue and a transpose of the int8 tile through the wave's own LDS
 // scratch.  No barrier after the weights are staged; waves only meet the memory system.
-template <int KS, int NI>
+// SUM: the residual operand FcArgs::epi.res is added to the int8 tile on its way out.
+template <int KS, int NI, bool SUM>
 __global__ __launch_bounds__(256, 2) void fc_stream_kernel(FcArgs p, int bn, int strips) {
   constexpr int K = 32 * KS, CH = 2 * KS;  // bytes and 16-byte chunks per row
   constexpr int TN = 32 * NI, LD = TN + 16;
@@ -142,6 +143,11 @@ __global__ __launch_bounds__(256, 2) void fc_stream_kernel(FcArgs p, int bn, int
         p.weight + static_cast<size_t>(n_begin + r) * K + c * 16);
   }
   const EpiScalars s = epi_scalars(p.epi);
+  SumRule rule = {0.0f, 0.0f, 1};
+  if (SUM)
+    rule = sum_rule(dev_maxabs(-p.epi.real_range, p.epi.real_range),
+                    dev_maxabs(*p.epi.res_min, *p.epi.res_max), p.epi.sum_min_calib,
+                    p.epi.sum_max_calib);
   if (tid < cols) sbias[tid] = epi_bias32(p.epi, s, n_begin + tid);
   __syncthreads();
 
@@ -171,6 +177,18 @@ __global__ __launch_bounds__(256, 2) void fc_stream_kernel(FcArgs p, int bn, int
     const int tile = item / strips;
     const int s0 = (item - tile * strips) * TN;  // first column of the strip inside the group's
     const int m_base = tile * 32;
+    // the residual operand's pieces of this tile, in the layout the tile leaves in
+    v4i resv[32 / RPI];
+    if (SUM) {
+#pragma unroll
+      for (int it = 0; it < 32 / RPI; ++it) {
+        const int m = m_base + it * RPI + lane / LPR;
+        resv[it] = v4i{0, 0, 0, 0};
+        if (m < p.M)
+          resv[it] = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(
+              p.epi.res + static_cast<size_t>(m) * p.ldo + n_begin + s0 + (lane % LPR) * 16));
+      }
+    }
     // the accumulators start at the int32 bias of their columns (read from LDS straight
     // into the registers the MFMAs add to): the epilogue has no bias add left
     v16i acc[NI];
@@ -210,21 +228,40 @@ __global__ __launch_bounds__(256, 2) void fc_stream_kernel(FcArgs p, int bn, int
     // order, the wait makes the writes complete first
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     __builtin_amdgcn_wave_barrier();
-    auto store_tile = [&](auto stream) {
+    auto store_tile = [&](auto stream, auto sum_relu, auto sum_fast) {
 #pragma unroll
       for (int it = 0; it < 32 / RPI; ++it) {
         const int rr = it * RPI + lane / LPR, c16 = lane % LPR;
-        const v4i val = *reinterpret_cast<const v4i*>(stage + rr * LD + c16 * 16);
+        v4i val = *reinterpret_cast<const v4i*>(stage + rr * LD + c16 * 16);
+        if (SUM) {
+#pragma unroll
+          for (int w = 0; w < 4; ++w)
+            val[w] = static_cast<int>(
+                sum4<decltype(sum_relu)::value, decltype(sum_fast)::value>(
+                    static_cast<uint32_t>(val[w]), static_cast<uint32_t>(resv[it][w]), rule));
+        }
         const int m = m_base + rr;
         if (m < p.M)
           epi_store16<decltype(stream)::value>(
               val, p.epi.out8 + static_cast<size_t>(m) * p.ldo + n_begin + s0 + c16 * 16);
       }
     };
-    if (stream8)
-      store_tile(std::true_type());
-    else
-      store_tile(std::false_type());
+    auto store_flavour = [&](auto sum_relu, auto sum_fast) {
+      if (stream8)
+        store_tile(std::true_type(), sum_relu, sum_fast);
+      else
+        store_tile(std::false_type(), sum_relu, sum_fast);
+    };
+    if (SUM && !rule.fast) {
+      if (p.epi.sum_relu)
+        store_flavour(std::true_type(), std::integral_constant<bool, !SUM>());
+      else
+        store_flavour(std::false_type(), std::integral_constant<bool, !SUM>());
+    } else if (SUM && p.epi.sum_relu) {
+      store_flavour(std::true_type(), std::true_type());
+    } else {
+      store_flavour(std::false_type(), std::true_type());
+    }
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     __builtin_amdgcn_wave_barrier();
     if (more) {
@@ -232,11 +269,13 @@ __global__ __launch_bounds__(256, 2) void fc_stream_kernel(FcArgs p, int bn, int
       for (int ks = 0; ks < KS; ++ks) fa[ks] = fa_next[ks];
     }
   }
-  if (blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0) epilogue_ranges(p.epi);
+  if (blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0) epilogue_ranges<SUM ? kEpiSum : kEpiPlain>(p.epi);
 }
 
 template <int KS, int NI>
 void launch_stream(hipStream_t s, const FcArgs& a, long cus, int groups_per_cu) {
+  // the residual operand is read in 16-byte pieces, like the output is written
+  MXQ_CHECK(a.epi.res == nullptr || aligned16(a.epi.res), "unaligned residual operand");
   constexpr int TN = 32 * NI;
   const int max_rows = KS <= 4 ? 256 : 128;
   const int bn = a.N < max_rows ? a.N : max_rows;
@@ -246,8 +285,12 @@ void launch_stream(hipStream_t s, const FcArgs& a, long cus, int groups_per_cu) 
   long gx = cus * groups_per_cu / ny;
   if (gx < 1) gx = 1;
   if (gx * 4 > items) gx = (items + 3) / 4;
-  hipLaunchKernelGGL((fc_stream_kernel<KS, NI>), dim3(static_cast<unsigned>(gx), ny), dim3(256), 0,
-                     s, a, bn, strips);
+  if (a.epi.res != nullptr)
+    hipLaunchKernelGGL((fc_stream_kernel<KS, NI, true>), dim3(static_cast<unsigned>(gx), ny),
+                       dim3(256), 0, s, a, bn, strips);
+  else
+    hipLaunchKernelGGL((fc_stream_kernel<KS, NI, false>), dim3(static_cast<unsigned>(gx), ny),
+                       dim3(256), 0, s, a, bn, strips);
   MXQ_LAUNCH_CHECK();
 }
 
@@ -255,29 +298,39 @@ template <class Cfg, int NS, int PIPE, bool BUF>
 void launch_dma(hipStream_t s, FcArgs a, int splits, const Workspace& ws) {
   const long tiles = static_cast<long>((a.M + Cfg::BM - 1) / Cfg::BM) * ((a.N + Cfg::BN - 1) / Cfg::BN);
   splitk_setup<Cfg>(s, a.sk, tiles, a.K, splits, ws.ptr, ws.bytes);
-  if (a.epi.outf != nullptr)
-    hipLaunchKernelGGL((fc_dma_kernel<Cfg, NS, PIPE, BUF, true>),
-                       dim3(static_cast<unsigned>(tiles * a.sk.splits)), dim3(Cfg::kThreads), 0,
-                       s, a);
-  else
-    hipLaunchKernelGGL((fc_dma_kernel<Cfg, NS, PIPE, BUF, false>),
-                       dim3(static_cast<unsigned>(tiles * a.sk.splits)), dim3(Cfg::kThreads), 0,
-                       s, a);
+  const dim3 grid(static_cast<unsigned>(tiles * a.sk.splits));
+  switch (epi_mode(a.epi)) {
+    case kEpiF32:
+      hipLaunchKernelGGL((fc_dma_kernel<Cfg, NS, PIPE, BUF, kEpiF32>), grid, dim3(Cfg::kThreads),
+                         0, s, a);
+      break;
+    case kEpiSum:
+      hipLaunchKernelGGL((fc_dma_kernel<Cfg, NS, PIPE, BUF, kEpiSum>), grid, dim3(Cfg::kThreads),
+                         0, s, a);
+      break;
+    default:
+      hipLaunchKernelGGL((fc_dma_kernel<Cfg, NS, PIPE, BUF, kEpiPlain>), grid,
+                         dim3(Cfg::kThreads), 0, s, a);
+  }
   MXQ_LAUNCH_CHECK();
 }
 
 template <class Cfg>
 void launch_cfg(hipStream_t s, const FcArgs& a, bool aligned) {
   const int tiles = ((a.M + Cfg::BM - 1) / Cfg::BM) * ((a.N + Cfg::BN - 1) / Cfg::BN);
-  const bool f32 = a.epi.outf != nullptr;
-  if (aligned && f32)
-    hipLaunchKernelGGL((fc_kernel<Cfg, true, true>), dim3(tiles), dim3(Cfg::kThreads), 0, s, a);
-  else if (aligned)
-    hipLaunchKernelGGL((fc_kernel<Cfg, true, false>), dim3(tiles), dim3(Cfg::kThreads), 0, s, a);
-  else if (f32)
-    hipLaunchKernelGGL((fc_kernel<Cfg, false, true>), dim3(tiles), dim3(Cfg::kThreads), 0, s, a);
-  else
-    hipLaunchKernelGGL((fc_kernel<Cfg, false, false>), dim3(tiles), dim3(Cfg::kThreads), 0, s, a);
+  const int mode = epi_mode(a.epi);
+#define MXQ_FC_KERNEL(ALIGNED, MODE) \
+  hipLaunchKernelGGL((fc_kernel<Cfg, ALIGNED, MODE>), dim3(tiles), dim3(Cfg::kThreads), 0, s, a)
+  if (aligned) {
+    if (mode == kEpiF32) MXQ_FC_KERNEL(true, kEpiF32);
+    else if (mode == kEpiSum) MXQ_FC_KERNEL(true, kEpiSum);
+    else MXQ_FC_KERNEL(true, kEpiPlain);
+  } else {
+    if (mode == kEpiF32) MXQ_FC_KERNEL(false, kEpiF32);
+    else if (mode == kEpiSum) MXQ_FC_KERNEL(false, kEpiSum);
+    else MXQ_FC_KERNEL(false, kEpiPlain);
+  }
+#undef MXQ_FC_KERNEL
   MXQ_LAUNCH_CHECK();
 }
 
@@ -378,7 +431,7 @@ size_t fc_plan_workspace(const FcPlan& plan, int M, int N) {
 }
 
 // an output without elements still owes its range scalars
-__global__ void gemm_ranges_kernel(Epilogue e) { epilogue_ranges(e); }
+__global__ void gemm_ranges_kernel(Epilogue e) { epilogue_ranges<kEpiSum>(e); }
 
 void launch_fc(hipStream_t s, const int8_t* data, const int8_t* weight, int M, int N, int K,
                int ldo, const Epilogue& epi, const GemmForce& force, const Workspace& ws) {
@@ -407,7 +460,8 @@ void launch_fc(hipStream_t s, const int8_t* data, const int8_t* weight, int M, i
                       static_cast<long long>(N) * K < (1LL << 31);
   const bool glb_ok = buf_ok && (K % 64 == 0);
   const bool fused8 = epi.out32 == nullptr && epi.outf == nullptr && epi.out8 != nullptr &&
-                      ldo % 16 == 0 && aligned16(epi.out8);
+                      ldo % 16 == 0 && aligned16(epi.out8) &&
+                      (epi.res == nullptr || aligned16(epi.res));
   FcPlan plan = plan_fc(M, N, K, aligned, fused8, force);
   // a split the chooser proposed is dropped when the caller brought no room for it
   if (force.splits == 0 && plan.splits > 1 &&
@@ -487,12 +541,22 @@ using namespace mxq;
 
 namespace {
 
+// The residual sum fused behind the requantization (mxq_quantized_fc_sum).
+struct SumArgs {
+  const int8_t* res;
+  const float* res_min;
+  const float* res_max;
+  float min_calib, max_calib;
+  int relu;
+};
+
 void fc_entry(void* stream, const int8_t* data, const int8_t* weight, const int8_t* bias, int M,
               int N, int K, const float* min_data, const float* max_data,
               const float* min_weight, const float* max_weight, const float* min_bias,
               const float* max_bias, int32_t* out32, float* omin, float* omax, int8_t* out8,
               float* out_f32, float* rmin, float* rmax, int relu, float min_calib,
-              float max_calib, void* workspace, size_t workspace_bytes, const GemmForce& force) {
+              float max_calib, void* workspace, size_t workspace_bytes, const GemmForce& force,
+              const SumArgs* sum = nullptr) {
   MXQ_CHECK(M >= 0 && N >= 0 && K >= 0, "negative dimension");
   MXQ_CHECK(min_data && max_data && min_weight && max_weight, "null input range pointer");
   MXQ_CHECK(omin && omax, "null output range pointer");
@@ -514,6 +578,26 @@ void fc_entry(void* stream, const int8_t* data, const int8_t* weight, const int8
   e.out32 = out32;
   e.out8 = out8;
   e.outf = out_f32;
+  e.res = nullptr;
+  e.res_min = e.res_max = nullptr;
+  e.sum_min_calib = e.sum_max_calib = 0.f;
+  e.sum_relu = 0;
+  e.with_sum = 0;
+  if (sum != nullptr) {
+    MXQ_CHECK((M == 0 || N == 0 || out8 != nullptr) && out32 == nullptr && out_f32 == nullptr,
+              "the fused sum writes the int8 output only");
+    MXQ_CHECK(sum->res_min && sum->res_max, "null residual range pointer");
+    MXQ_CHECK(M == 0 || N == 0 || sum->res != nullptr, "null residual operand");
+    if (M != 0 && N != 0) {  // without elements only the ranges are written
+      e.res = sum->res;
+      e.res_min = sum->res_min;
+      e.res_max = sum->res_max;
+    }
+    e.sum_min_calib = sum->min_calib;
+    e.sum_max_calib = sum->max_calib;
+    e.sum_relu = sum->relu;
+    e.with_sum = 1;
+  }
   e.omin = omin;
   e.omax = omax;
   e.rmin = rmin;
@@ -588,6 +672,48 @@ int mxq_quantized_fc_f32(void* stream, const int8_t* data, const int8_t* weight,
   fc_entry(stream, data, weight, bias, M, N, K, min_data, max_data, min_weight, max_weight,
            min_bias, max_bias, nullptr, omin, omax, nullptr, out_f32, rmin, rmax, relu,
            min_calib, max_calib, workspace, workspace_bytes, GemmForce());
+  MXQ_API_END();
+}
+
+int mxq_quantized_fc_sum(void* stream, const int8_t* data, const int8_t* weight,
+                         const int8_t* bias, int M, int N, int K, const float* min_data,
+                         const float* max_data, const float* min_weight, const float* max_weight,
+                         const float* min_bias, const float* max_bias, const int8_t* residual,
+                         const float* min_residual, const float* max_residual, int8_t* out8,
+                         float* omin, float* omax, float* rmin, float* rmax, float min_calib,
+                         float max_calib, float sum_min_calib, float sum_max_calib, int sum_relu,
+                         void* workspace, size_t workspace_bytes) {
+  MXQ_API_BEGIN();
+  const SumArgs sum = {residual, min_residual, max_residual, sum_min_calib, sum_max_calib,
+                       sum_relu};
+  fc_entry(stream, data, weight, bias, M, N, K, min_data, max_data, min_weight, max_weight,
+           min_bias, max_bias, nullptr, omin, omax, out8, nullptr, rmin, rmax, 0, min_calib,
+           max_calib, workspace, workspace_bytes, GemmForce(), &sum);
+  MXQ_API_END();
+}
+
+// Test-only twin of mxq_quantized_fc_sum with the kernel variant pinned
+// (tests/mxq_test_hooks.h).
+int mxq_test_quantized_fc_sum(void* stream, const int8_t* data, const int8_t* weight,
+                              const int8_t* bias, int M, int N, int K, const float* min_data,
+                              const float* max_data, const float* min_weight,
+                              const float* max_weight, const float* min_bias,
+                              const float* max_bias, const int8_t* residual,
+                              const float* min_residual, const float* max_residual,
+                              int8_t* out8, float* omin, float* omax, float* rmin, float* rmax,
+                              float min_calib, float max_calib, float sum_min_calib,
+                              float sum_max_calib, int sum_relu, void* workspace,
+                              size_t workspace_bytes, int cfg, int splits, int stream_groups) {
+  MXQ_API_BEGIN();
+  const SumArgs sum = {residual, min_residual, max_residual, sum_min_calib, sum_max_calib,
+                       sum_relu};
+  GemmForce force;
+  force.cfg = cfg;
+  force.splits = splits;
+  force.stream_groups = stream_groups;
+  fc_entry(stream, data, weight, bias, M, N, K, min_data, max_data, min_weight, max_weight,
+           min_bias, max_bias, nullptr, omin, omax, out8, nullptr, rmin, rmax, 0, min_calib,
+           max_calib, workspace, workspace_bytes, force, &sum);
   MXQ_API_END();
 }
 

@@ -37,6 +37,7 @@
 #include <cstdint>
 
 #include "mxq_common.h"
+#include "mxq_sum.h"
 
 namespace mxq {
 
@@ -56,6 +57,16 @@ struct Epilogue {
   // [M][ldo] or null: the int8 result above taken back to float, q * (R / 127), i.e.
   // what dequantize makes of the requantized output (dequantize-inl.h:64-75)
   float* outf;
+  // int8 [M][ldo] or null: a second operand that is added to the requantized int8 result
+  // before it is stored (the residual sum that follows the layer, then optionally the int8
+  // relu): out8 = relu?(add(requantize(acc), res)) over the calibrated range
+  // (sum_min_calib, sum_max_calib), which rmin / rmax then receive.
+  const int8_t* res;
+  const float* res_min;    // device scalars: the range of res
+  const float* res_max;
+  float sum_min_calib, sum_max_calib;
+  int sum_relu;
+  int with_sum;            // rmin / rmax report the sum's range (also for an empty output)
   float* omin;             // int32 output range
   float* omax;
   float* rmin;             // requantized range (only with out8)
@@ -670,9 +681,18 @@ __device__ __forceinline__ void gemm_mainloop_dma(v16i (&acc)[Cfg::MI][Cfg::NI],
 }
 
 // Stores one wave's accumulators.  m_base/n_base: origin of the wave tile.
-// F32OUT: the kernel can also write Epilogue::outf (only the fully-connected kernels are
-// built that way; elsewhere the code for it is left out, which keeps cold kernels short).
-template <class Cfg, bool F32OUT = false>
+// What a kernel's epilogue is built for besides the int32 and int8 outputs.  Only the
+// fully-connected kernels are built with the extras, each as an instantiation of its own:
+// elsewhere their code is left out, which keeps cold kernels short.
+constexpr int kEpiPlain = 0;  // out32 and / or out8
+constexpr int kEpiF32 = 1;    // Epilogue::outf
+constexpr int kEpiSum = 2;    // out8 with Epilogue::res added
+
+inline int epi_mode(const Epilogue& e) {
+  return e.outf != nullptr ? kEpiF32 : (e.res != nullptr ? kEpiSum : kEpiPlain);
+}
+
+template <class Cfg, int MODE = kEpiPlain>
 __device__ __forceinline__ void gemm_epilogue(v16i (&acc)[Cfg::MI][Cfg::NI], const Epilogue& e,
                                               int m_base, int n_base, int M, int N,
                                               size_t ldo) {
@@ -715,13 +735,27 @@ __device__ __forceinline__ void gemm_epilogue(v16i (&acc)[Cfg::MI][Cfg::NI], con
               if (n + i < N) e.out32[off + i] = v[i];
           }
         }
-        if (e.out8 != nullptr || (F32OUT && e.outf != nullptr)) {
+        if (e.out8 != nullptr || (MODE == kEpiF32 && e.outf != nullptr)) {
           int q[4];
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
             q[i] = epi_requant(v[i], s, e.relu ? 0.0f : -127.0f);
           }
-          if (e.out8 != nullptr) {
+          if (MODE == kEpiSum && e.res != nullptr && e.out8 != nullptr) {
+            const SumRule r = sum_rule(dev_maxabs(-e.real_range, e.real_range),
+                                       dev_maxabs(*e.res_min, *e.res_max), e.sum_min_calib,
+                                       e.sum_max_calib);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+              if (n + i < N) {
+                // the overflow-safe form serves every rule on this rarely taken path
+                const int b = static_cast<int>(e.res[off + i]);
+                const uint32_t v8 = e.sum_relu ? sum_one<true, false>(q[i], b, r)
+                                               : sum_one<false, false>(q[i], b, r);
+                e.out8[off + i] = static_cast<int8_t>(v8 & 0xffu);
+              }
+            }
+          } else if (e.out8 != nullptr) {
             if (full) {
               *reinterpret_cast<uint32_t*>(e.out8 + off) = pack_bytes(q[0], q[1], q[2], q[3]);
             } else {
@@ -730,7 +764,7 @@ __device__ __forceinline__ void gemm_epilogue(v16i (&acc)[Cfg::MI][Cfg::NI], con
                 if (n + i < N) e.out8[off + i] = static_cast<int8_t>(q[i]);
             }
           }
-          if (F32OUT && e.outf != nullptr) {
+          if (MODE == kEpiF32 && e.outf != nullptr) {
             int* of = reinterpret_cast<int*>(e.outf);
             if (full && (reinterpret_cast<uintptr_t>(e.outf) & 15u) == 0) {
               v4i w = {epi_dequant_bits(q[0], s), epi_dequant_bits(q[1], s),
@@ -760,12 +794,17 @@ __device__ __forceinline__ void gemm_epilogue(v16i (&acc)[Cfg::MI][Cfg::NI], con
 struct EpiPre {
   EpiScalars s;
   int bias32;
+  SumRule sum;  // the residual sum's scales (kernels built for it)
 };
-template <class Cfg>
+template <class Cfg, int MODE = kEpiPlain>
 __device__ __forceinline__ EpiPre epi_prefetch(const Epilogue& e, int n0, int N) {
   static_assert(Cfg::kThreads >= Cfg::BN, "one thread per tile column");
   EpiPre p;
   p.s = epi_scalars(e);
+  p.sum = SumRule{0.0f, 0.0f, 1};
+  if (MODE == kEpiSum && e.res != nullptr)
+    p.sum = sum_rule(dev_maxabs(-e.real_range, e.real_range),
+                     dev_maxabs(*e.res_min, *e.res_max), e.sum_min_calib, e.sum_max_calib);
   const int t = threadIdx.x;
   p.bias32 = (t < Cfg::BN && n0 + t < N) ? epi_bias32(e, p.s, n0 + t) : 0;
   return p;
@@ -786,7 +825,7 @@ struct EpiScratch {
   static constexpr int kNeed32 = Cfg::BN * 4 + kWaves * kPerWave;
 };
 
-template <class Cfg, int RING_BYTES, bool F32OUT = false>
+template <class Cfg, int RING_BYTES, int MODE = kEpiPlain>
 __device__ __forceinline__ void gemm_epilogue_lds(v16i (&acc)[Cfg::MI][Cfg::NI],
                                                   const Epilogue& e, const EpiPre& pre, int m0,
                                                   int n0, int M, int N, size_t ldo,
@@ -809,11 +848,16 @@ __device__ __forceinline__ void gemm_epilogue_lds(v16i (&acc)[Cfg::MI][Cfg::NI],
   const bool fast32 = e.out32 == nullptr ||
                       ((N % 4 == 0) && (ldo % 4 == 0) &&
                        ((reinterpret_cast<uintptr_t>(e.out32) & 15u) == 0));
-  const bool fastf = !F32OUT || e.outf == nullptr ||
+  // the sum's scales; a rule whose products could overflow goes the general way with the
+  // unaligned outputs
+  const SumRule rule = pre.sum;
+  const bool fasts = MODE != kEpiSum || e.res == nullptr ||
+                     (((reinterpret_cast<uintptr_t>(e.res) & 15u) == 0) && rule.fast);
+  const bool fastf = MODE != kEpiF32 || e.outf == nullptr ||
                      ((N % 4 == 0) && (ldo % 4 == 0) &&
                       ((reinterpret_cast<uintptr_t>(e.outf) & 15u) == 0));
-  if (__builtin_expect(!(fast8 && fast32 && fastf), 0)) {
-    gemm_epilogue<Cfg, F32OUT>(acc, e, m_base, n_base, M, N, ldo);
+  if (__builtin_expect(!(fast8 && fast32 && fastf && fasts), 0)) {
+    gemm_epilogue<Cfg, MODE>(acc, e, m_base, n_base, M, N, ldo);
     return;
   }
   char* lds = reinterpret_cast<char*>(lds_v);
@@ -972,7 +1016,7 @@ __device__ __forceinline__ void gemm_epilogue_lds(v16i (&acc)[Cfg::MI][Cfg::NI],
 
   // the requantized result as float: requantize, then the int8 dequantize over the
   // calibrated range, element by element in registers
-  if (F32OUT && e.outf != nullptr) {
+  if (MODE == kEpiF32 && e.outf != nullptr) {
     auto dequantized_tile = [&](auto relu) {
       store_rows32(reinterpret_cast<int*>(e.outf), [&](int mi, int ni, int vq) {
         v4i w;
@@ -992,6 +1036,27 @@ __device__ __forceinline__ void gemm_epilogue_lds(v16i (&acc)[Cfg::MI][Cfg::NI],
   }
 
   if (e.out8 != nullptr) {
+    // the staged tile leaves in 16-byte pieces in row-major order, 64 per store instruction
+    // (a wave tile of 96 columns has 6 pieces per row: the last instruction is then partial)
+    constexpr int kPieces = TM * LPR;
+    constexpr int kIters = (kPieces + 63) / 64;
+    // the residual operand's pieces are fetched now, behind the requantization's arithmetic
+    v4i resv[MODE == kEpiSum ? kIters : 1];
+    if constexpr (MODE == kEpiSum) {
+      if (e.res != nullptr) {
+#pragma unroll
+        for (int it = 0; it < kIters; ++it) {
+          const int piece = it * 64 + lane;
+          const int rr = (64 % LPR == 0) ? it * RPI + lane / LPR : piece / LPR;
+          const int c16 = (64 % LPR == 0) ? lane % LPR : piece - rr * LPR;
+          const int m = m_base + rr, n = n_base + c16 * 16;
+          resv[it] = v4i{0, 0, 0, 0};
+          if ((kPieces % 64 == 0 || piece < kPieces) && m < M && n < N)
+            resv[it] = __builtin_nontemporal_load(
+                reinterpret_cast<const v4i*>(e.res + static_cast<size_t>(m) * ldo + n));
+        }
+      }
+    }
     auto requantize_tile = [&](auto relu) {
 #pragma unroll
       for (int ni = 0; ni < NI; ++ni)
@@ -1014,26 +1079,46 @@ __device__ __forceinline__ void gemm_epilogue_lds(v16i (&acc)[Cfg::MI][Cfg::NI],
     // instructions in order, the wait makes the writes complete first
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     __builtin_amdgcn_wave_barrier();
-    // 16-byte pieces of the staged tile in row-major order, 64 per store instruction (a
-    // wave tile of 96 columns has 6 pieces per row: the last instruction is then partial)
-    auto store_tile = [&](auto stream) {
-      constexpr int kPieces = TM * LPR;
+    auto store_tile = [&](auto stream, auto sum_mode) {
+      constexpr int SM = decltype(sum_mode)::value;  // 0 no sum, 1 sum, 2 sum + relu
 #pragma unroll
-      for (int it = 0; it < (kPieces + 63) / 64; ++it) {
+      for (int it = 0; it < kIters; ++it) {
         const int piece = it * 64 + lane;
         const int rr = (64 % LPR == 0) ? it * RPI + lane / LPR : piece / LPR;
         const int c16 = (64 % LPR == 0) ? lane % LPR : piece - rr * LPR;
         if (kPieces % 64 != 0 && piece >= kPieces) continue;
-        const v4i val = *reinterpret_cast<const v4i*>(stage + rr * LD + c16 * 16);
+        v4i val = *reinterpret_cast<const v4i*>(stage + rr * LD + c16 * 16);
+        if constexpr (SM != 0) {
+#pragma unroll
+          for (int w = 0; w < 4; ++w)
+            val[w] = static_cast<int>(sum4<SM == 2, true>(
+                static_cast<uint32_t>(val[w]), static_cast<uint32_t>(resv[it][w]), rule));
+        }
         const int m = m_base + rr, n = n_base + c16 * 16;
         if (m < M && n < N)
           epi_store16<decltype(stream)::value>(val, e.out8 + static_cast<size_t>(m) * ldo + n);
       }
     };
+    if constexpr (MODE == kEpiSum) {
+      if (e.res != nullptr) {
+        if (e.stream8) {
+          if (e.sum_relu)
+            store_tile(std::true_type(), std::integral_constant<int, 2>());
+          else
+            store_tile(std::true_type(), std::integral_constant<int, 1>());
+        } else {
+          if (e.sum_relu)
+            store_tile(std::false_type(), std::integral_constant<int, 2>());
+          else
+            store_tile(std::false_type(), std::integral_constant<int, 1>());
+        }
+        return;
+      }
+    }
     if (e.stream8)
-      store_tile(std::true_type());
+      store_tile(std::true_type(), std::integral_constant<int, 0>());
     else
-      store_tile(std::false_type());
+      store_tile(std::false_type(), std::integral_constant<int, 0>());
   }
 }
 
@@ -1165,14 +1250,22 @@ __device__ __forceinline__ bool splitk_gather(v16i (&acc)[Cfg::MI][Cfg::NI], con
 }
 
 // Range scalars, written once per launch.
+// MODE as for the epilogues: only a kernel built for the residual sum looks at its fields
+// (three more scalar registers, which some of the tiled kernels do not have to spare).
+template <int MODE = kEpiPlain>
 __device__ __forceinline__ void epilogue_ranges(const Epilogue& e) {
   const EpiScalars s = epi_scalars(e);
   *e.omin = -s.max_out;
   *e.omax = s.max_out;
   // also for an output without elements, whose buffer pointer may be null
   if (e.rmin != nullptr && e.rmax != nullptr) {
-    *e.rmin = -e.real_range;
-    *e.rmax = e.real_range;
+    if (MODE == kEpiSum && e.with_sum) {  // the sum's calibrated range, as quantized_elemwise_add reports it
+      *e.rmin = e.sum_min_calib;
+      *e.rmax = e.sum_max_calib;
+    } else {
+      *e.rmin = -e.real_range;
+      *e.rmax = e.real_range;
+    }
   }
 }
 

@@ -38,6 +38,19 @@ int mxq_test_quantized_fc_f32(void* stream, const int8_t* data, const int8_t* we
                               float max_calib, void* workspace, size_t workspace_bytes, int cfg,
                               int splits);
 
+/* mxq_quantized_fc_sum with the tile configuration, the split-K factor and the streaming
+ * kernel's work-groups per CU pinned. */
+int mxq_test_quantized_fc_sum(void* stream, const int8_t* data, const int8_t* weight,
+                              const int8_t* bias, int M, int N, int K, const float* min_data,
+                              const float* max_data, const float* min_weight,
+                              const float* max_weight, const float* min_bias,
+                              const float* max_bias, const int8_t* residual,
+                              const float* min_residual, const float* max_residual,
+                              int8_t* out8, float* omin, float* omax, float* rmin, float* rmax,
+                              float min_calib, float max_calib, float sum_min_calib,
+                              float sum_max_calib, int sum_relu, void* workspace,
+                              size_t workspace_bytes, int cfg, int splits, int stream_groups);
+
 /* mxq_quantized_conv_nhwc with the tile configuration (mxq_conv.hip lists them) and the
  * split-K factor pinned. */
 int mxq_test_quantized_conv_nhwc(void* stream, const int8_t* data, const int8_t* weight,

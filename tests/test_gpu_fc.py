@@ -375,3 +375,120 @@ def test_fc_dequantized_output_degenerate(capi):
     rc = lib.mxq_quantized_fc_f32(None, None, None, None, 4, 4, 16, None, None, None, None, None,
                                   None, None, None, None, None, None, 0, 0.0, 1.0, None, 0)
     assert rc != 0 and "no output buffer" in last_error()
+
+
+# ---- quantized_fc -> requantize -> elemwise_add (-> relu) in one launch -----------------------
+def oracle_fc_sum(d, w, b, res, calib, res_range, sum_calib, sum_relu):
+    """The reference's operators one after the other."""
+    rd, rw, rb = 2.0, 0.1, 1.0
+    ro, rmn, rmx = oracle_fc(d, w, b, rd, rw, rb)
+    rq, qmn, qmx = oracle.requantize(ro, rmn, rmx, *calib)
+    out, omn, omx = oracle.quantized_elemwise_add(rq, res, qmn, qmx, -res_range, res_range,
+                                                  min_calib_range=sum_calib[0],
+                                                  max_calib_range=sum_calib[1])
+    if sum_relu:
+        out = oracle.relu_i8(out)
+    return out, (rmn, rmx), (omn, omx)
+
+
+def check_fc_sum(capi, d, w, b, res, calib, res_range, sum_calib, sum_relu, force=None):
+    rd, rw, rb = 2.0, 0.1, 1.0
+    got = capi.quantized_fc_sum(dev(d), dev(w), None if b is None else dev(b), dev(res), f32(-rd),
+                                f32(rd), f32(-rw), f32(rw), None if b is None else f32(-rb),
+                                None if b is None else f32(rb), f32(-res_range), f32(res_range),
+                                calib, sum_calib, sum_relu=sum_relu, force=force)
+    ref, r32, rsum = oracle_fc_sum(d, w, b, res, calib, res_range, sum_calib, sum_relu)
+    np.testing.assert_array_equal(got["out8"].cpu().numpy(), ref)
+    assert (got["omin"].item(), got["omax"].item()) == r32
+    assert (got["rmin"].item(), got["rmax"].item()) == rsum
+
+
+def sum_case(M, K, N, seed):
+    d = int8_uniform((M, K), seed=seed)
+    w = int8_uniform((N, K), seed=seed + 1)
+    b = int8_uniform((N,), seed=seed + 2) if (M + N) % 2 else None
+    res = int8_uniform((M, N), seed=seed + 3)
+    ro, rmn, rmx = oracle_fc(d, w, b, 2.0, 0.1, 1.0)
+    fl = ro.astype(np.float64) * (float(rmx) / 2147483648.0)
+    R = float(np.percentile(np.abs(fl), 98.0)) or 1.0
+    return d, w, b, res, R
+
+
+@pytest.mark.parametrize("M,K,N", SHAPES + [(4096, 64, 256), (40000, 64, 64), (33000, 128, 128),
+                                            (3136, 512, 2048), (100, 64, 6)])
+@pytest.mark.parametrize("sum_relu", [False, True])
+def test_fc_residual_sum(capi, M, K, N, sum_relu):
+    d, w, b, res, R = sum_case(M, K, N, seed=M + K + N)
+    # the residual's range and the sum's range chosen so that part of the sums saturate
+    check_fc_sum(capi, d, w, b, res, (-R, 0.85 * R), 0.7 * R, (-0.9 * R, 1.1 * R), sum_relu)
+
+
+@pytest.mark.parametrize("cfg", [1, 2, 3, 4, 11, 12, 14, 16, 21, 22, 23, 24, 31, 32, 41, 42, 43, 44,
+                                 51, 52, 53, 54, 55, 56, 57, 58, 59, 60])
+@pytest.mark.parametrize("M,K,N,splits", [(512, 512, 512, 1), (300, 192, 272, 1), (70, 448, 36, 1),
+                                          (257, 208, 64, 1), (300, 2064, 272, 3)])
+def test_fc_residual_sum_every_tile_config(capi, cfg, M, K, N, splits):
+    if 10 < cfg < 20 and K % 64 != 0:
+        pytest.skip("the global-load direct-to-LDS kernels need K % 64 == 0")
+    if cfg < 10 and splits > 1:
+        pytest.skip("the register-staged kernels have no split-K form")
+    d, w, b, res, R = sum_case(M, K, N, seed=cfg + M)
+    check_fc_sum(capi, d, w, b, res, (-R, 0.85 * R), 0.7 * R, (-0.9 * R, 1.1 * R), bool(cfg % 2),
+                 force=(cfg, splits, 0))
+
+
+@pytest.mark.parametrize("cfg,M,K,N", [(61, 4096, 64, 64), (62, 5000, 64, 256), (61, 777, 32, 192),
+                                       (62, 2100, 128, 128), (62, 300, 256, 256)])
+@pytest.mark.parametrize("sum_relu", [False, True])
+def test_fc_residual_sum_streaming_kernel(capi, cfg, M, K, N, sum_relu):
+    d, w, b, res, R = sum_case(M, K, N, seed=cfg + N)
+    check_fc_sum(capi, d, w, b, res, (-R, 0.85 * R), 0.7 * R, (-0.9 * R, 1.1 * R), sum_relu,
+                 force=(cfg, 1, 0))
+
+
+def test_fc_residual_sum_huge_scales_and_misalignment(capi):
+    """A residual range so large that the products could overflow takes the overflow-safe
+    rule; a residual or output that is not 16-byte aligned takes the general epilogue."""
+    d, w, b, res, R = sum_case(300, 192, 272, seed=5)
+    check_fc_sum(capi, d, w, b, res, (-R, R), 3e38, (-1e-8, 1e-8), True)
+    check_fc_sum(capi, d, w, b, res, (-R, R), 1e-30, (-3e38, 3e38), False)
+    # misaligned residual: a view that starts 1 byte into a larger buffer
+    rd, rw = 2.0, 0.1
+    buf = torch.empty(res.size + 16, dtype=torch.int8, device="cuda")
+    view = buf[1:1 + res.size].view(res.shape)
+    view.copy_(dev(res))
+    got = capi.quantized_fc_sum(dev(d), dev(w), None if b is None else dev(b), view, f32(-rd),
+                                f32(rd), f32(-rw), f32(rw), None if b is None else f32(-1.0),
+                                None if b is None else f32(1.0), f32(-0.7 * R), f32(0.7 * R),
+                                (-R, R), (-R, R), sum_relu=True)
+    ref, _, _ = oracle_fc_sum(d, w, b, res, (-R, R), 0.7 * R, (-R, R), True)
+    np.testing.assert_array_equal(got["out8"].cpu().numpy(), ref)
+
+
+def test_fc_residual_sum_matches_the_three_kernels(capi, ):
+    """Against this library's own quantized_fc -> elemwise_add -> relu on a ResNet shape."""
+    import mxnet_amd
+    M, K, N = 50176, 128, 512
+    d, w, b, res, R = sum_case(M, K, N, seed=9)
+    ranges = [f32(-2.0), f32(2.0), f32(-0.1), f32(0.1)]
+    bias_r = [None, None] if b is None else [f32(-1.0), f32(1.0)]
+    dd, wd, bd, rs = dev(d), dev(w), None if b is None else dev(b), dev(res)
+    one = capi.quantized_fc(dd, wd, bd, *ranges, *bias_r, want_int32=False, calib=(-R, R))
+    s8, smn, smx = mxnet_amd.contrib.quantized_elemwise_add(
+        one["out8"], rs, one["rmin"], one["rmax"], f32(-0.7 * R), f32(0.7 * R),
+        min_calib_range=-R, max_calib_range=R)
+    s8 = torch.clamp(s8, min=0)
+    fused = capi.quantized_fc_sum(dd, wd, bd, rs, *ranges, *bias_r, f32(-0.7 * R), f32(0.7 * R),
+                                  (-R, R), (-R, R), sum_relu=True)
+    assert torch.equal(fused["out8"], s8)
+    assert (fused["rmin"].item(), fused["rmax"].item()) == (smn.item(), smx.item())
+
+
+def test_fc_residual_sum_degenerate(capi):
+    res = capi.quantized_fc_sum(torch.empty((0, 64), dtype=torch.int8, device="cuda"),
+                                dev(int8_uniform((32, 64), seed=1)), None,
+                                torch.empty((0, 32), dtype=torch.int8, device="cuda"), f32(-1.0),
+                                f32(1.0), f32(-1.0), f32(1.0), None, None, f32(-1.0), f32(1.0),
+                                (-2.0, 3.0), (-4.0, 5.0))
+    assert res["out8"].shape == (0, 32)
+    assert (res["rmin"].item(), res["rmax"].item()) == (-4.0, 5.0)
