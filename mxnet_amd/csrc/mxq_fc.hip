@@ -372,7 +372,9 @@ struct FcPlan {
 // What launch_fc would run for this shape.  `aligned`: K % 16 == 0 and 16-byte aligned
 // operands; `fused8`: int8 output only, 16-byte aligned with a row pitch that is a
 // multiple of 16 (what the streaming kernel stores).
-FcPlan plan_fc(int M, int N, int K, bool aligned, bool fused8, const GemmForce& force) {
+// `sum`: the residual-sum form, whose epilogue does twice the arithmetic per output.
+FcPlan plan_fc(int M, int N, int K, bool aligned, bool fused8, const GemmForce& force,
+               bool sum = false) {
   FcPlan plan = {force.cfg, force.splits, force.stream_groups > 0 ? force.stream_groups : 2};
   const bool buf_ok = aligned && K >= 16 && static_cast<long long>(M) * K < (1LL << 31) &&
                       static_cast<long long>(N) * K < (1LL << 31);
@@ -407,6 +409,17 @@ FcPlan plan_fc(int M, int N, int K, bool aligned, bool fused8, const GemmForce& 
         plan.cfg = 4;
     }
     if (plan.splits == 0) plan.splits = auto_splits;
+    // With the residual sum in the epilogue the balance moves (sweeps of every configuration
+    // per layer inside the chained ResNet-50 body at batch 64): where the plain form takes
+    // 256 x 128 tiles on 64-byte stages, 256 x 256 tiles on 128-byte stages are ahead once
+    // they cover 0.56 of the CUs (12544 x 256 -> 1024: -1.9 us per layer) and 128 x 128
+    // tiles otherwise (50176 x 128 -> 512: -1.2 us per layer).
+    if (sum && plan.cfg == 41) {
+      if (K >= 256 && N > 128 && 16 * tiles(256, 256) >= 9 * cus)
+        plan.cfg = 55;
+      else
+        plan.cfg = 43;
+    }
     // the short-K streaming kernel: chosen for tall outputs of at most 256 columns
     // (200704 x 64 -> 64: 8.5 us against 10.2; -> 256: 18.5 against 21.9; 200704 x 128 ->
     // 128: 15.3 against 17.1); from 512 columns on the tiled kernels are level or ahead
@@ -417,6 +430,12 @@ FcPlan plan_fc(int M, int N, int K, bool aligned, bool fused8, const GemmForce& 
       plan.cfg = (N % 128 == 0) ? 62 : 61;
       plan.splits = 1;
       if (force.stream_groups <= 0) plan.stream_groups = K <= 64 ? 4 : 3;
+      // the sum's extra registers and arithmetic favour the 64-column strips with more
+      // groups in flight (200704 x 64 -> 256 inside the chain: -7 us per layer)
+      if (sum && K <= 64) {
+        plan.cfg = 61;
+        if (force.stream_groups <= 0) plan.stream_groups = 5;
+      }
     }
   }
   if (plan.splits <= 0) plan.splits = 1;
@@ -462,13 +481,14 @@ void launch_fc(hipStream_t s, const int8_t* data, const int8_t* weight, int M, i
   const bool fused8 = epi.out32 == nullptr && epi.outf == nullptr && epi.out8 != nullptr &&
                       ldo % 16 == 0 && aligned16(epi.out8) &&
                       (epi.res == nullptr || aligned16(epi.res));
-  FcPlan plan = plan_fc(M, N, K, aligned, fused8, force);
+  const bool sum = epi.res != nullptr;
+  FcPlan plan = plan_fc(M, N, K, aligned, fused8, force, sum);
   // a split the chooser proposed is dropped when the caller brought no room for it
   if (force.splits == 0 && plan.splits > 1 &&
       (ws.ptr == nullptr || !aligned16(ws.ptr) || ws.bytes < fc_plan_workspace(plan, M, N))) {
     GemmForce unsplit = force;
     unsplit.splits = 1;
-    plan = plan_fc(M, N, K, aligned, fused8, unsplit);
+    plan = plan_fc(M, N, K, aligned, fused8, unsplit, sum);
   }
   const int cfg = plan.cfg;
   if (cfg >= 11 && cfg <= 16) MXQ_CHECK(glb_ok, "shape does not qualify for the DMA kernels");
