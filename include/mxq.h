@@ -326,7 +326,8 @@ int mxq_quantized_fc_f32(void* stream, const int8_t* data, const int8_t* weight,
  *   sum_*_calib    the sum's calibrated range; rmin / rmax receive it
  *   sum_relu != 0  clamps the sum at zero
  * out8 is bit-identical to mxq_quantized_elemwise_add(out8 of mxq_quantized_fc, residual)
- * followed by mxq_quantized_relu; neither intermediate tensor is stored.  Workspace as for
+ * followed by mxq_quantized_relu; neither intermediate tensor is stored.  out8 may be the
+ * residual's own buffer (the shortcut updated in place).  Workspace as for
  * mxq_quantized_fc with fused_int8_only = 1. */
 int mxq_quantized_fc_sum(void* stream, const int8_t* data, const int8_t* weight,
                          const int8_t* bias, int M, int N, int K, const float* min_data,

@@ -492,3 +492,25 @@ def test_fc_residual_sum_degenerate(capi):
                                 (-2.0, 3.0), (-4.0, 5.0))
     assert res["out8"].shape == (0, 32)
     assert (res["rmin"].item(), res["rmax"].item()) == (-4.0, 5.0)
+
+
+@pytest.mark.parametrize("M,K,N", [(50176, 128, 512), (40000, 64, 256), (300, 208, 100)])
+def test_fc_residual_sum_in_place(capi, M, K, N):
+    """The output may be the residual operand's own buffer (the sum updates the shortcut in
+    place): every piece is read before the tile that owns it is stored."""
+    import ctypes
+    from mxnet_amd._lib import check, lib
+    d, w, b, res, R = sum_case(M, K, N, seed=M + 1)
+    ref, _, _ = oracle_fc_sum(d, w, b, res, (-R, R), 0.7 * R, (-R, 1.2 * R), True)
+    dd, wd, rs = dev(d), dev(w), dev(res)
+    bd = None if b is None else dev(b)
+    sc = [f32(v) for v in (-2.0, 2.0, -0.1, 0.1, -1.0, 1.0, -0.7 * R, 0.7 * R)]
+    out = [torch.empty(1, device="cuda") for _ in range(4)]
+    P = lambda t: None if t is None else ctypes.c_void_p(t.data_ptr())
+    st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    check(lib.mxq_quantized_fc_sum(st, P(dd), P(wd), P(bd), M, N, K, P(sc[0]), P(sc[1]), P(sc[2]),
+                                   P(sc[3]), P(sc[4]) if b is not None else None,
+                                   P(sc[5]) if b is not None else None, P(rs), P(sc[6]), P(sc[7]),
+                                   P(rs), P(out[0]), P(out[1]), P(out[2]), P(out[3]), -R, R, -R,
+                                   1.2 * R, 1, None, 0))
+    np.testing.assert_array_equal(rs.cpu().numpy(), ref)
