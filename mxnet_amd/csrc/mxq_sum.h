@@ -52,6 +52,20 @@ __device__ __forceinline__ uint32_t sum_one(int a, int b, const SumRule& r) {
 // Four int8 pairs (x: left operand, y: right operand, byte k of each) -> four int8 results.
 template <bool RELU, bool FAST>
 __device__ __forceinline__ uint32_t sum4(uint32_t x, uint32_t y, const SumRule& r) {
+  if (RELU && FAST) {
+    // results in [0, 127]: v_cvt_pk_u8_f32 rounds to nearest even, saturates and places the
+    // byte in one instruction (instead of the 1.5 * 2^23 add and three quarters of a pack)
+    uint32_t w = 0;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const int a = static_cast<int>(static_cast<int8_t>((x >> (8 * k)) & 0xffu));
+      const int b = static_cast<int>(static_cast<int8_t>((y >> (8 * k)) & 0xffu));
+      const float p = static_cast<float>(a) * r.s0;
+      const float q = static_cast<float>(b) * r.s1;
+      w = __builtin_amdgcn_cvt_pk_u8_f32(__builtin_amdgcn_fmed3f(p + q, 0.0f, 127.0f), k, w);
+    }
+    return w;
+  }
   uint32_t q[4];
 #pragma unroll
   for (int k = 0; k < 4; ++k) {
