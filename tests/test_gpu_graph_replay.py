@@ -4,7 +4,8 @@ the program's own eager work and synchronisations in between); every replay must
 the oracle gives for that input.  Covers the launches that carry state between kernels of
 one call: the uncalibrated casts (reduction partials in a workspace, or in the library's own
 array for the no-allocation entry point) and a split-K fully-connected layer (tile counters
-cleared by a kernel of the same call, partial sums in the workspace)."""
+cleared by a kernel of the same call, partial sums in the workspace), also in its
+float-output and residual-sum forms."""
 import ctypes
 
 import numpy as np
@@ -49,6 +50,18 @@ def test_replays_follow_their_inputs():
     nfc = lib.mxq_quantized_fc_workspace(M, N, K, 0)
     assert nfc > 0, "this shape is expected to ask for a split-K workspace"
     ws_fc = torch.empty(nfc, dtype=torch.uint8, device="cuda")
+    # the float-output and residual-sum forms of the same split layer, each with a workspace
+    # of its own (launches of one graph may not share one)
+    ws_f32 = torch.empty(nfc, dtype=torch.uint8, device="cuda")
+    ws_sum = torch.empty(lib.mxq_quantized_fc_workspace(M, N, K, 1), dtype=torch.uint8,
+                         device="cuda")
+    yf = torch.empty((M, N), dtype=torch.float32, device="cuda")
+    ff = [scalar() for _ in range(4)]
+    res_np = int8_uniform((M, N), seed=8)
+    res = torch.from_numpy(res_np).cuda()
+    res_r = [torch.tensor([v], device="cuda") for v in (-30.0, 30.0)]
+    s8 = torch.empty((M, N), dtype=torch.int8, device="cuda")
+    fs = [scalar() for _ in range(4)]
     calib = 40.0
 
     def body():
@@ -67,6 +80,14 @@ def test_replays_follow_their_inputs():
             lib.mxq_requantize(st, P(acc), P(fr[0]), P(fr[1]), P(r8), P(rr[0]), P(rr[1]), M * N,
                                0, 0.0, 0.0, P(ws_r), ws_r.numel()),
             lib.mxq_dequantize(st, P(r8), 5, P(rr[0]), P(rr[1]), P(y), M * N),
+            lib.mxq_quantized_fc_f32(st, P(q), P(w), P(b), M, N, K, P(qr[0]), P(qr[1]), P(wr[0]),
+                                     P(wr[1]), P(wr[2]), P(wr[3]), P(yf), P(ff[0]), P(ff[1]),
+                                     P(ff[2]), P(ff[3]), 0, -calib, calib, P(ws_f32),
+                                     ws_f32.numel()),
+            lib.mxq_quantized_fc_sum(st, P(q), P(w), P(b), M, N, K, P(qr[0]), P(qr[1]), P(wr[0]),
+                                     P(wr[1]), P(wr[2]), P(wr[3]), P(res), P(res_r[0]),
+                                     P(res_r[1]), P(s8), P(fs[0]), P(fs[1]), P(fs[2]), P(fs[3]),
+                                     -calib, calib, -50.0, 45.0, 1, P(ws_sum), ws_sum.numel()),
         ]
         assert not any(rcs), mxnet_amd._lib.last_error()
 
@@ -105,5 +126,11 @@ def test_replays_follow_their_inputs():
         np.testing.assert_array_equal(r8.cpu().numpy(), uq)
         assert (rr[0].item(), rr[1].item()) == (umn, umx)
         np.testing.assert_array_equal(y.cpu().numpy(), oracle.dequantize(uq, umn, umx))
+        np.testing.assert_array_equal(yf.cpu().numpy().view(np.uint32),
+                                      oracle.dequantize(fq, fmn, fmx).view(np.uint32))
+        sq, smn, smx = oracle.quantized_elemwise_add(fq, res_np, fmn, fmx, -30.0, 30.0,
+                                                     min_calib_range=-50.0, max_calib_range=45.0)
+        np.testing.assert_array_equal(s8.cpu().numpy(), oracle.relu_i8(sq))
+        assert (fs[2].item(), fs[3].item()) == (smn, smx)
         # the program's own eager work between replays
         (x * 2.0).sum().item()
