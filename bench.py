@@ -67,6 +67,7 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=2000)
     ap.add_argument("--workload", default="fc4096",
                     choices=["fc4096", "fc8192", "quantize", "quantize_uncal", "quantize_uint8",
+                             "quantize_v1", "quantized_act",
                              "quantize_laplace", "quantize_uint8_uncal", "small_casts",
                              "requantize", "requantize_uncal", "dequantize", "copy", "maxpool", "avgpool",
                              "elemwise_add", "elemwise_add_int8", "concat", "elemwise_mul_int8", "quantize_asym",
@@ -225,6 +226,25 @@ class CastWorkload:
             self.name = ("requantize int32->int8 " +
                          ("uncalibrated (on-device min/max)" if kind == "requantize_uncal"
                           else "calibrated (-0.1,0.1)"))
+        elif kind == "quantize_v1":
+            self.src = [torch.randn(n, device="cuda", generator=g).clamp_(-4.0, 4.0)
+                        for _ in range(self.NBUF)]
+            self.dst = [torch.empty(n, dtype=torch.int8, device="cuda")
+                        for _ in range(self.NBUF)]
+            self.imin = torch.tensor([-4.0], device="cuda")
+            self.imax = torch.tensor([4.0], device="cuda")
+            self.bytes = 5.0 * n
+            self.kernel = "quantize_kernel"
+            self.name = "quantize (v1) fp32->int8, range (-4,4) given as inputs"
+        elif kind == "quantized_act":
+            self.src = [torch.randint(-127, 128, (n,), device="cuda", generator=g,
+                                      dtype=torch.int8) for _ in range(self.NBUF)]
+            self.dst = [torch.empty(n, dtype=torch.int8, device="cuda") for _ in range(self.NBUF)]
+            self.imin = torch.tensor([-3.0], device="cuda")
+            self.imax = torch.tensor([3.0], device="cuda")
+            self.bytes = 2.0 * n
+            self.kernel = "relu_i8_kernel"
+            self.name = "quantized_act relu int8->int8"
         elif kind == "dequantize":
             self.src = [torch.randint(-127, 128, (n,), device="cuda", generator=g,
                                       dtype=torch.int8) for _ in range(self.NBUF)]
@@ -356,6 +376,12 @@ class CastWorkload:
             rc = lib.mxq_quantize_v2(st, P(self.src[k]), P(self.dst[k]), P(self.omin),
                                      P(self.omax), n, 5, 0, 0.0, 0.0, P(self.ws),
                                      self.ws.numel())
+        elif kind == "quantize_v1":
+            rc = lib.mxq_quantize(st, P(self.src[k]), P(self.imin), P(self.imax), P(self.dst[k]),
+                                  P(self.omin), P(self.omax), n, 5)
+        elif kind == "quantized_act":
+            rc = lib.mxq_quantized_relu(st, P(self.src[k]), P(self.imin), P(self.imax),
+                                        P(self.dst[k]), P(self.omin), P(self.omax), n)
         elif kind == "requantize":
             rc = lib.mxq_requantize(st, P(self.src[k]), P(self.imin), P(self.imax),
                                     P(self.dst[k]), P(self.omin), P(self.omax), n, 1, -0.1, 0.1,
@@ -435,6 +461,10 @@ class CastWorkload:
                 oracle.quantize_v2(x, "uint8", -50.0, 50.0)
             elif kind == "quantize_uncal":
                 oracle.quantize_v2(x, "int8")
+            elif kind == "quantize_v1":
+                oracle.quantize(x, -4.0, 4.0)
+            elif kind == "quantized_act":
+                oracle.relu_i8(x)
             elif kind == "requantize":
                 oracle.requantize(x, -1.0, 1.0, -0.1, 0.1)
             elif kind == "requantize_uncal":
@@ -1154,7 +1184,8 @@ def main():
     if not args.no_cast_ops:
         rows = []
         for kind in ["quantize", "quantize_laplace", "quantize_uint8", "quantize_uncal",
-                     "quantize_uint8_uncal", "small_casts", "requantize",
+                     "quantize_uint8_uncal", "quantize_v1", "quantized_act", "small_casts",
+                     "requantize",
                      "requantize_uncal", "dequantize", "elemwise_add", "elemwise_add_int8",
                      "concat", "elemwise_mul_int8", "quantize_asym", "batch_norm", "embedding",
                      "transpose", "maxpool", "avgpool", "fc8192",
