@@ -45,8 +45,8 @@ MEASURED_TRAFFIC_BYTES = {
     "quantize_uncal": ((2.0 * (131093.7 + 131139.1) + 65536.1) * _KIB, "profiles/quantize_uncalibrated_64M.md"),
     "requantize": ((2.0 * 131104.8 + 65536.1) * _KIB, "profiles/requantize_kernel_64M.md"),
     "requantize_uncal": ((2.0 * (131089.2 + 131139.2) + 65536.1) * _KIB, "profiles/requantize_uncalibrated_64M.md"),
-    "dequantize": ((2.0 * 32785.5 + 262144.0) * _KIB, "profiles/dequantize_kernel_64M.md"),
-    "elemwise_add": ((2.0 * 65570.5 + 262144.1) * _KIB, "profiles/add_kernel_int32_64M.md"),
+    "dequantize": ((2.0 * 32782.0 + 262144.0) * _KIB, "profiles/dequantize_chunk_kernel_64M.md"),
+    "elemwise_add": ((2.0 * 65557.2 + 262144.1) * _KIB, "profiles/add32_chunk_kernel_64M.md"),
     "elemwise_add_int8": ((2.0 * 65583.7 + 65536.1) * _KIB, "profiles/add_kernel_int8_64M.md"),
     "concat": ((2.0 * 32840.8 + 65536.1) * _KIB, "profiles/concat_kernel_64M.md"),
     "elemwise_mul_int8": ((2.0 * 65565.8 + 65536.1) * _KIB, "profiles/mul_kernel_int8_64M.md"),
@@ -253,7 +253,7 @@ class CastWorkload:
             self.imin = torch.tensor([-3.0], device="cuda")
             self.imax = torch.tensor([3.0], device="cuda")
             self.bytes = 5.0 * n
-            self.kernel = "dequantize_kernel"
+            self.kernel = "dequantize_chunk_kernel"
             self.name = "dequantize int8->fp32"
         elif kind in ("elemwise_add", "elemwise_add_int8"):
             self.src = [torch.randint(-127, 128, (n,), device="cuda", generator=g,
@@ -265,7 +265,7 @@ class CastWorkload:
             self.imin = torch.tensor([-3.0], device="cuda")
             self.imax = torch.tensor([3.0], device="cuda")
             self.bytes = (6.0 if kind == "elemwise_add" else 3.0) * n
-            self.kernel = "add_kernel"
+            self.kernel = "add32_chunk_kernel" if kind == "elemwise_add" else "add_kernel"
             self.name = ("quantized_elemwise_add int8+int8->" +
                          ("int32" if kind == "elemwise_add" else "int8 calibrated (-5,5)"))
         elif kind == "concat":

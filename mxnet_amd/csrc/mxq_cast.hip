@@ -423,6 +423,65 @@ constexpr int kDeqRunQuads = 256;   // 16-byte pieces of one wave's output run (
 constexpr int kStreamOut = 18;
 constexpr int kRsrcFlags = 0x00020000;
 
+// One contiguous chunk per work-group, no loop: every lane requests its two dwords of the
+// chunk's 4 KiB of input (512 lanes, a lane's dwords 2 KiB apart), then converts and writes
+// the chunk's 16 KiB of output with two 16-byte stores.  From 16 M elements on this is the
+// fastest pattern measured for the widening cast (64 M: 50.3 us against 56.3 us for 4 KiB
+// runs per wave of a grid-stride kernel; 256 M: 196 against 237 us); exactly two pieces per
+// lane matter (one: 60.7 us, three: 57.5, four: 58.9 at 64 M), the thread count little (128 /
+// 256 / 512 / 1024 threads: 51.6 / 51.5 / 50.3 / 54.3 us).
+constexpr int kDeqChunkThreads = 512;
+constexpr int kDeqChunkPieces = 2;
+constexpr size_t kDeqChunkMinElements = size_t(1) << 24;
+
+template <bool UNSIGNED>
+__global__ __launch_bounds__(kDeqChunkThreads) void dequantize_chunk_kernel(
+    const uint8_t* __restrict__ in, float* __restrict__ out, size_t n,
+    const float* __restrict__ imin, const float* __restrict__ imax) {
+  const float lo = *imin, hi = *imax;
+  const float scale = UNSIGNED ? (hi - lo) / (255.0f - 0.0f) : maxabs(hi, lo) / 127.0f;
+  auto conv = [&](uint32_t byte) -> float {
+    if (UNSIGNED) {
+      float p = static_cast<float>(byte) * scale;
+      return p + lo;
+    } else {
+      return static_cast<float>(static_cast<int>(static_cast<int8_t>(byte))) * scale;
+    }
+  };
+  const size_t nquad = n >> 2;
+  const size_t base = size_t(blockIdx.x) * (kDeqChunkPieces * kDeqChunkThreads);
+  const uint32_t* in4 = reinterpret_cast<const uint32_t*>(in);
+  uint32_t w[kDeqChunkPieces];
+#pragma unroll
+  for (int j = 0; j < kDeqChunkPieces; ++j) {
+    const size_t q = base + size_t(j) * kDeqChunkThreads + threadIdx.x;
+    w[j] = q < nquad ? nt_load(in4 + q) : 0u;
+  }
+  // the descriptor ends with the tensor: pieces past the last whole quad are dropped
+  const size_t left = nquad > base ? nquad - base : 0;
+  const uint32_t bytes = left >= size_t(kDeqChunkPieces) * kDeqChunkThreads
+                             ? kDeqChunkPieces * kDeqChunkThreads * 16
+                             : static_cast<uint32_t>(left * 16);
+  const __amdgpu_buffer_rsrc_t dst = __builtin_amdgcn_make_buffer_rsrc(
+      reinterpret_cast<f4*>(out) + base, 0, bytes, kRsrcFlags);
+#pragma unroll
+  for (int j = 0; j < kDeqChunkPieces; ++j) {
+    f4 y;
+    y.x = conv(w[j] & 0xffu);
+    y.y = conv((w[j] >> 8) & 0xffu);
+    y.z = conv((w[j] >> 16) & 0xffu);
+    y.w = conv(w[j] >> 24);
+    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(i4, y), dst,
+                                           (j * kDeqChunkThreads + threadIdx.x) * 16, 0,
+                                           kStreamOut);
+  }
+  // the ragged tail (< 4 elements)
+  if (blockIdx.x == 0) {
+    const size_t i = (nquad << 2) + threadIdx.x;
+    if (i < n) out[i] = conv(in[i]);
+  }
+}
+
 template <bool UNSIGNED, bool VEC>
 __global__ __launch_bounds__(kThreads) void dequantize_kernel(const uint8_t* __restrict__ in,
                                                               float* __restrict__ out, size_t n,
@@ -977,6 +1036,19 @@ int mxq_dequantize(void* stream, const void* in, int in_type, const float* imin,
   const bool vec = aligned16(out) && ((reinterpret_cast<uintptr_t>(in) & 3u) == 0);
   const int grid = stream_grid(vec ? (n + 3) / 4 : n, n, true);
   const uint8_t* i8 = static_cast<const uint8_t*>(in);
+  if (vec && n >= kDeqChunkMinElements) {
+    const size_t per = size_t(kDeqChunkPieces) * kDeqChunkThreads;
+    const size_t chunks = ((n >> 2) + per - 1) / per;
+    MXQ_CHECK(chunks < (size_t(1) << 31), "tensor too large for one launch");
+    if (in_type == MXQ_UINT8)
+      hipLaunchKernelGGL(dequantize_chunk_kernel<true>, dim3(static_cast<unsigned>(chunks)),
+                         dim3(kDeqChunkThreads), 0, s, i8, out, n, imin, imax);
+    else
+      hipLaunchKernelGGL(dequantize_chunk_kernel<false>, dim3(static_cast<unsigned>(chunks)),
+                         dim3(kDeqChunkThreads), 0, s, i8, out, n, imin, imax);
+    MXQ_LAUNCH_CHECK();
+    return 0;
+  }
 #define MXQ_D(U, V) \
   hipLaunchKernelGGL((dequantize_kernel<U, V>), dim3(grid), dim3(kThreads), 0, s, i8, out, n, \
                      imin, imax)

@@ -202,6 +202,60 @@ __device__ __forceinline__ void add_bytes(const AddArgs& a, const AddRule<OUT, L
   }
 }
 
+// The int32 sum of large tensors: one contiguous chunk per work-group, no loop.  Every lane
+// requests its two dwords of each operand (512 lanes, a lane's dwords 2 KiB apart), then adds
+// and writes the chunk's 16 KiB of output with two 16-byte stores.  As for the widening cast,
+// this is the fastest pattern measured for a write-dominated stream (64 M elements: 62.8 us
+// against 69.0 us for 4 KiB runs per wave of a grid-stride kernel; one, four or eight dwords
+// per lane: 67.2 / 68.4 / 67.4 us).
+constexpr int kAddChunkThreads = 512;
+constexpr int kAddChunkPieces = 2;
+constexpr size_t kAddChunkMinElements = size_t(1) << 24;
+
+template <bool LU, bool RU>
+__global__ __launch_bounds__(kAddChunkThreads) void add32_chunk_kernel(AddArgs a) {
+  const AddRule<MXQ_INT32, LU, RU> r = add_rule<MXQ_INT32, LU, RU>(a);
+  const size_t nq = a.n >> 2;
+  const size_t base = size_t(blockIdx.x) * (kAddChunkPieces * kAddChunkThreads);
+  const uint32_t* l4 = reinterpret_cast<const uint32_t*>(a.lhs);
+  const uint32_t* r4 = reinterpret_cast<const uint32_t*>(a.rhs);
+  uint32_t x[kAddChunkPieces], y[kAddChunkPieces];
+#pragma unroll
+  for (int j = 0; j < kAddChunkPieces; ++j) {
+    const size_t q = base + size_t(j) * kAddChunkThreads + threadIdx.x;
+    x[j] = q < nq ? __builtin_nontemporal_load(l4 + q) : 0u;
+    y[j] = q < nq ? __builtin_nontemporal_load(r4 + q) : 0u;
+  }
+  // the descriptor ends with the tensor: pieces past the last whole quad are dropped
+  const size_t left = nq > base ? nq - base : 0;
+  const uint32_t bytes = left >= size_t(kAddChunkPieces) * kAddChunkThreads
+                             ? kAddChunkPieces * kAddChunkThreads * 16
+                             : static_cast<uint32_t>(left * 16);
+  const __amdgpu_buffer_rsrc_t dst = __builtin_amdgcn_make_buffer_rsrc(
+      reinterpret_cast<i4*>(a.out) + base, 0, bytes, 0x00020000);
+#pragma unroll
+  for (int j = 0; j < kAddChunkPieces; ++j) {
+    i4 v;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) v[k] = r.apply(byte_of<LU>(x[j], k), byte_of<RU>(y[j], k));
+    __builtin_amdgcn_raw_buffer_store_b128(v, dst, (j * kAddChunkThreads + threadIdx.x) * 16, 0,
+                                           18 /* sc1 + nt */);
+  }
+  if (blockIdx.x == 0) {
+    // the ragged tail (< 4 elements) and the range
+    const size_t i = (nq << 2) + threadIdx.x;
+    if (i < a.n) {
+      const int xv = LU ? static_cast<int>(a.lhs[i]) : static_cast<int>(static_cast<int8_t>(a.lhs[i]));
+      const int yv = RU ? static_cast<int>(a.rhs[i]) : static_cast<int>(static_cast<int8_t>(a.rhs[i]));
+      static_cast<int32_t*>(a.out)[i] = r.apply(xv, yv);
+    }
+    if (threadIdx.x == 0) {
+      *a.omin = r.omin;
+      *a.omax = r.omax;
+    }
+  }
+}
+
 template <int OUT, bool LU, bool RU>
 __global__ __launch_bounds__(kThreads) void add_kernel(AddArgs a) {
   const AddRule<OUT, LU, RU> r = add_rule<OUT, LU, RU>(a);
@@ -1006,7 +1060,19 @@ int mxq_quantized_elemwise_add(void* stream, const void* lhs, int lhs_type, cons
   const bool lu = lhs_type == MXQ_UINT8, ru = rhs_type == MXQ_UINT8;
 #define MXQ_ADD(O, L, R) \
   hipLaunchKernelGGL((add_kernel<O, L, R>), dim3(grid), dim3(kThreads), 0, s, a)
-  if (out_type == MXQ_INT32) {
+  if (out_type == MXQ_INT32 && a.vec_ok && n >= kAddChunkMinElements) {
+    const size_t per = size_t(kAddChunkPieces) * kAddChunkThreads;
+    const size_t chunks = ((n >> 2) + per - 1) / per;
+    MXQ_CHECK(chunks < (size_t(1) << 31), "tensor too large for one launch");
+    const dim3 cg(static_cast<unsigned>(chunks)), cb(kAddChunkThreads);
+    if (lu) {
+      if (ru) hipLaunchKernelGGL((add32_chunk_kernel<true, true>), cg, cb, 0, s, a);
+      else hipLaunchKernelGGL((add32_chunk_kernel<true, false>), cg, cb, 0, s, a);
+    } else {
+      if (ru) hipLaunchKernelGGL((add32_chunk_kernel<false, true>), cg, cb, 0, s, a);
+      else hipLaunchKernelGGL((add32_chunk_kernel<false, false>), cg, cb, 0, s, a);
+    }
+  } else if (out_type == MXQ_INT32) {
     if (lu) { if (ru) MXQ_ADD(MXQ_INT32, true, true); else MXQ_ADD(MXQ_INT32, true, false); }
     else    { if (ru) MXQ_ADD(MXQ_INT32, false, true); else MXQ_ADD(MXQ_INT32, false, false); }
   } else if (out_type == MXQ_UINT8) {

@@ -102,6 +102,56 @@ def test_dequantize_64m(capi):
     assert np.array_equal(got.view(np.uint32), ref.view(np.uint32))
 
 
+@pytest.mark.parametrize("dtype", ["int8", "uint8"])
+@pytest.mark.parametrize("n", [(1 << 24), (1 << 24) + 1, (1 << 24) + 1023 * 4 + 3,
+                               (1 << 25) - 4097, 3 * (1 << 23) + 2048 * 4])
+def test_dequantize_chunk_kernel_edges(capi, dtype, n):
+    """From 16 M elements on the widening cast runs one chunk of 2048 quads per work-group:
+    last chunks that are full, hold one quad, end one quad short, and ragged tails of 1-3
+    elements, for both input types."""
+    g = torch.Generator(device="cuda").manual_seed(n % 1000)
+    if dtype == "int8":
+        q = torch.randint(-128, 128, (n,), device="cuda", generator=g, dtype=torch.int8)
+        lo, hi = -3.0, 2.5
+    else:
+        q = torch.randint(0, 256, (n,), device="cuda", generator=g, dtype=torch.uint8)
+        lo, hi = -1.0, 7.0
+    guard = torch.full((n + 64,), 7.5, dtype=torch.float32, device="cuda")
+    y = guard[:n]
+    from mxnet_amd._lib import check, lib
+    import ctypes
+    code = 5 if dtype == "int8" else 3
+    rlo, rhi = f32(lo), f32(hi)   # kept alive across the call
+    check(lib.mxq_dequantize(ctypes.c_void_p(torch.cuda.current_stream().cuda_stream),
+                             ctypes.c_void_p(q.data_ptr()), code,
+                             ctypes.c_void_p(rlo.data_ptr()), ctypes.c_void_p(rhi.data_ptr()),
+                             ctypes.c_void_p(y.data_ptr()), n))
+    torch.cuda.synchronize()
+    ref = oracle.dequantize(q.cpu().numpy(), lo, hi)
+    assert np.array_equal(y.cpu().numpy().view(np.uint32), ref.view(np.uint32))
+    assert bool((guard[n:] == 7.5).all()), "wrote past the end"
+
+
+@pytest.mark.parametrize("lu,ru", [(False, False), (True, False), (False, True), (True, True)])
+@pytest.mark.parametrize("n", [(1 << 24), (1 << 24) + 3, (1 << 24) + 1023 * 4 + 1,
+                               (1 << 25) - 4097])
+def test_elemwise_add_int32_chunk_kernel_edges(contrib, lu, ru, n):
+    """From 16 M elements on the int32 sum runs one chunk of 2048 quads per work-group: full
+    and partial last chunks, ragged tails, every operand type pair."""
+    g = torch.Generator(device="cuda").manual_seed(n % 997 + 2 * lu + ru)
+    def operand(unsigned):
+        if unsigned:
+            return torch.randint(0, 256, (n,), device="cuda", generator=g, dtype=torch.uint8)
+        return torch.randint(-128, 128, (n,), device="cuda", generator=g, dtype=torch.int8)
+    a, b = operand(lu), operand(ru)
+    rng = (-1.5, 2.0, -0.75, 0.5)
+    out, mn, mx = contrib.quantized_elemwise_add(a, b, *[f32(v) for v in rng])
+    ref, rmn, rmx = oracle.quantized_elemwise_add(a.cpu().numpy(), b.cpu().numpy(), *rng)
+    assert out.dtype == torch.int32
+    assert (mn.item(), mx.item()) == (rmn, rmx)
+    assert np.array_equal(out.cpu().numpy(), ref)
+
+
 def test_elemwise_add_64m(contrib):
     g = torch.Generator(device="cuda").manual_seed(5)
     a = torch.randint(-127, 128, (N_CAST,), device="cuda", generator=g, dtype=torch.int8)
