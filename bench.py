@@ -72,7 +72,7 @@ def parse_args():
                              "requantize", "requantize_uncal", "dequantize", "copy", "maxpool", "avgpool",
                              "elemwise_add", "elemwise_add_int8", "concat", "elemwise_mul_int8", "quantize_asym",
                              "batch_norm", "embedding", "transpose", "resnet50_convs", "resnet50_chain",
-                             "resnet50_chain_fused",
+                             "resnet50_chain_fused", "resnet50_chain_unfused",
                              "bert_fc_chain",
                              "bert_fc_chain_fused",
                              "bert_fc_chain_f32"])
@@ -771,11 +771,18 @@ class ResNetChainWorkload(GraphWorkload):
     16 relus per step; stem, pooling and the classifier are not part of it."""
     STAGES = [(3, 64, 256, 1), (4, 128, 512, 2), (6, 256, 1024, 2), (3, 512, 2048, 2)]
 
-    def __init__(self, torch, capi, lib, fused_sum=False):
+    def __init__(self, torch, capi, lib, fused_sum=False, unfused=False):
         self.kernel = "conv / fc kernels, add_kernel, relu"
         self.bound = "mfma"
         self.name = "ResNet-50 v1 bottleneck body as a chain (52 convolutions + 16 residual " \
                     "adds + relus), batch 64, NHWC int8, requantize fused"
+        if unfused:
+            # the operator sequence of the graph the reference's pass emits: every convolution
+            # writes int32, a _contrib_requantize node narrows it, relu is a node of its own
+            self.kernel = "conv / fc kernels (int32 out), requantize, relu, add_kernel"
+            self.name = "ResNet-50 v1 bottleneck body as the reference's graph runs it: " \
+                        "quantized_conv (int32) -> requantize -> quantized_act per layer, " \
+                        "elemwise_add + act per block, batch 64, NHWC"
         if fused_sum:
             self.kernel = "conv / fc kernels, the residual sum and its relu in the epilogue of " \
                           "each block's last 1x1 convolution"
@@ -810,6 +817,32 @@ class ResNetChainWorkload(GraphWorkload):
             out8 = torch.empty((N, OH, OH, O), dtype=torch.int8, device="cuda")
             sc = [torch.empty(1, device="cuda") for _ in range(4)]
             geo = (N, H, H, C, O, k, k, s, s, pad, pad)
+            if unfused:
+                acc = torch.empty((N, OH, OH, O), dtype=torch.int32, device="cuda")
+                tmp8 = torch.empty_like(out8) if relu else out8
+                sc += [torch.empty(1, device="cuda") for _ in range(2)]
+                nws = lib.mxq_quantized_conv_workspace(*geo, 1, 1, 0)
+                ws = torch.empty(nws, dtype=torch.uint8, device="cuda") if nws else None
+                seq = [(lib.mxq_quantized_conv_nhwc,
+                        (P(inp), P(wq), P(bq), *geo, 1, 1, P(imin), P(imax), P(wmin), P(wmax),
+                         P(bmin), P(bmax), P(acc), P(sc[0]), P(sc[1]), None, None, None, 0, 0.0,
+                         0.0, *ws_args(ws))),
+                       (lib.mxq_requantize,
+                        (P(acc), P(sc[0]), P(sc[1]), P(tmp8), P(sc[4] if relu else sc[2]),
+                         P(sc[5] if relu else sc[3]), acc.numel(), 1, -r, r, None, 0))]
+                if relu:
+                    seq.append((lib.mxq_quantized_relu,
+                                (P(tmp8), P(sc[4]), P(sc[5]), P(out8), P(sc[2]), P(sc[3]),
+                                 out8.numel())))
+                self.calls += seq
+                self.keep.append((inp, wq, bq, imin, imax, wmin, wmax, bmin, bmax, out8, sc, ws,
+                                  acc, tmp8))
+                self.ops += 2.0 * N * OH * OH * O * k * k * C
+                st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+                for fn, a_ in seq:
+                    if fn(st, *a_):
+                        raise RuntimeError(lib.mxq_last_error().decode())
+                return out8, sc[2], sc[3], OH
             nws = lib.mxq_quantized_conv_workspace(*geo, 1, 1, 1)
             ws = torch.empty(nws, dtype=torch.uint8, device="cuda") if nws else None
             args = (P(inp), P(wq), P(bq), *geo, 1, 1, P(imin), P(imax), P(wmin), P(wmax), P(bmin),
@@ -1063,6 +1096,8 @@ def make_workload(name, torch, capi, lib):
         return ResNetChainWorkload(torch, capi, lib)
     if name == "resnet50_chain_fused":
         return ResNetChainWorkload(torch, capi, lib, fused_sum=True)
+    if name == "resnet50_chain_unfused":
+        return ResNetChainWorkload(torch, capi, lib, unfused=True)
     if name == "bert_fc_chain":
         return BertChainWorkload(torch, capi, lib)
     if name == "bert_fc_chain_fused":
@@ -1189,7 +1224,8 @@ def main():
                      "requantize_uncal", "dequantize", "elemwise_add", "elemwise_add_int8",
                      "concat", "elemwise_mul_int8", "quantize_asym", "batch_norm", "embedding",
                      "transpose", "maxpool", "avgpool", "fc8192",
-                     "resnet50_convs", "resnet50_chain", "resnet50_chain_fused", "bert_fc_chain",
+                     "resnet50_convs", "resnet50_chain_unfused", "resnet50_chain", "resnet50_chain_fused",
+                     "bert_fc_chain",
                      "bert_fc_chain_fused", "bert_fc_chain_f32"]:
             if kind == args.workload:
                 continue
