@@ -750,6 +750,52 @@ __global__ __launch_bounds__(kThreads) void relu_i8_kernel(const int8_t* __restr
   }
 }
 
+// The relu of large tensors: one contiguous 32 KiB chunk per work-group, no loop; every lane
+// requests its eight 16-byte pieces (4 KiB apart), then clamps and stores them.  64 M
+// elements: 23.2 -> 21.6 us against the grid-stride kernel (two builds, one box); 16 or 64 KiB
+// chunks and 64 ... 1024 lanes stay at 22.6-25.9 us.  At 51 M elements the gain is 3 % alone
+// and nothing inside the chained ResNet-50 body, below that the grid-stride kernel with its
+// size-dependent grid is level or ahead: taken from 64 M elements on.
+constexpr int kReluChunkPieces = 8;
+constexpr size_t kReluChunkMinElements = size_t(1) << 26;
+
+__global__ __launch_bounds__(kThreads) void relu_chunk_kernel(const int8_t* __restrict__ in,
+                                                              int8_t* __restrict__ out, size_t n,
+                                                              const float* __restrict__ imin,
+                                                              const float* __restrict__ imax,
+                                                              float* __restrict__ omin,
+                                                              float* __restrict__ omax) {
+  typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+  auto relu4 = [](uint32_t w) -> uint32_t {
+    uint32_t neg = (w >> 7) & 0x01010101u;
+    return w & ((neg * 0xffu) ^ 0xffffffffu);
+  };
+  const size_t n16 = n >> 4;
+  const size_t base = size_t(blockIdx.x) * (kReluChunkPieces * kThreads);
+  const u4* in16 = reinterpret_cast<const u4*>(in);
+  u4* out16 = reinterpret_cast<u4*>(out);
+  u4 w[kReluChunkPieces];
+#pragma unroll
+  for (int j = 0; j < kReluChunkPieces; ++j) {
+    const size_t q = base + size_t(j) * kThreads + threadIdx.x;
+    w[j] = q < n16 ? nt_load(in16 + q) : u4{0, 0, 0, 0};
+  }
+#pragma unroll
+  for (int j = 0; j < kReluChunkPieces; ++j) {
+    const size_t q = base + size_t(j) * kThreads + threadIdx.x;
+    const u4 r = {relu4(w[j].x), relu4(w[j].y), relu4(w[j].z), relu4(w[j].w)};
+    if (q < n16) nt_store(r, out16 + q);
+  }
+  if (blockIdx.x == 0) {
+    const size_t i = (n16 << 4) + threadIdx.x;
+    if (i < n) out[i] = in[i] > 0 ? in[i] : 0;
+    if (threadIdx.x == 0) {
+      *omin = *imin;
+      *omax = *imax;
+    }
+  }
+}
+
 __global__ void passthrough_range_kernel(float* omin, float* omax, float lo, float hi) {
   *omin = lo;
   *omax = hi;
@@ -1017,6 +1063,15 @@ int mxq_quantized_relu(void* stream, const int8_t* in, const float* imin, const 
             "null range pointer");
   MXQ_CHECK(n == 0 || (in != nullptr && out != nullptr), "null data pointer");
   const bool vec = aligned16(in) && aligned16(out);
+  if (vec && n >= kReluChunkMinElements) {
+    const size_t per = size_t(kReluChunkPieces) * kThreads;
+    const size_t chunks = ((n >> 4) + per - 1) / per;
+    MXQ_CHECK(chunks < (size_t(1) << 31), "tensor too large for one launch");
+    hipLaunchKernelGGL(relu_chunk_kernel, dim3(static_cast<unsigned>(chunks)), dim3(kThreads), 0,
+                       static_cast<hipStream_t>(stream), in, out, n, imin, imax, omin, omax);
+    MXQ_LAUNCH_CHECK();
+    return 0;
+  }
   const int grid = stream_grid(n == 0 ? 1 : (vec ? (n + 15) / 16 : n), n);
   hipLaunchKernelGGL(relu_i8_kernel, dim3(grid), dim3(kThreads), 0,
                      static_cast<hipStream_t>(stream), in, out, n, imin, imax, omin, omax, vec);

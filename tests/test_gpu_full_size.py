@@ -152,6 +152,29 @@ def test_elemwise_add_int32_chunk_kernel_edges(contrib, lu, ru, n):
     assert np.array_equal(out.cpu().numpy(), ref)
 
 
+@pytest.mark.parametrize("n", [(1 << 26), (1 << 26) + 5, (1 << 26) + 2047 * 16 + 15,
+                               (1 << 26) + 2048 * 16 + 1])
+def test_quantized_act_chunk_kernel_edges(contrib, n):
+    """From 64 M elements on the relu runs one chunk of 2048 16-byte pieces per work-group:
+    full and partial last chunks, ragged tails."""
+    g = torch.Generator(device="cuda").manual_seed(n % 991)
+    guard = torch.randint(-128, 128, (n + 64,), device="cuda", generator=g, dtype=torch.int8)
+    x = guard[:n]
+    out_buf = torch.full((n + 64,), 77, dtype=torch.int8, device="cuda")
+    import ctypes
+    from mxnet_amd._lib import check, lib
+    lo, hi, omn, omx = f32(-2.0), f32(3.0), f32(0.0), f32(0.0)
+    P = lambda t: ctypes.c_void_p(t.data_ptr())
+    check(lib.mxq_quantized_relu(ctypes.c_void_p(torch.cuda.current_stream().cuda_stream), P(x),
+                                 P(lo), P(hi), P(out_buf), P(omn), P(omx), n))
+    torch.cuda.synchronize()
+    assert torch.equal(out_buf[:n], torch.clamp(x, min=0))
+    assert bool((out_buf[n:] == 77).all()), "wrote past the end"
+    assert (omn.item(), omx.item()) == (-2.0, 3.0)
+    ref = oracle.relu_i8(x[:1 << 20].cpu().numpy())
+    assert np.array_equal(out_buf[:1 << 20].cpu().numpy(), ref)
+
+
 def test_elemwise_add_64m(contrib):
     g = torch.Generator(device="cuda").manual_seed(5)
     a = torch.randint(-127, 128, (N_CAST,), device="cuda", generator=g, dtype=torch.int8)
