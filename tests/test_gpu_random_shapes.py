@@ -80,6 +80,20 @@ def test_fc_random_shape(capi, M, N, K):
     ref = oracle.dequantize(rq, qmn, qmx)
     np.testing.assert_array_equal(resf["outf"].cpu().numpy().view(np.uint32), ref.view(np.uint32))
     assert (resf["rmin"].item(), resf["rmax"].item()) == (qmn, qmx)
+    # the residual sum (and its relu) behind the requantization
+    res8 = int8_uniform((M, N), seed=M + N + 9)
+    ro2, _, _ = oracle.requantize(ro, rmn, rmx, -R, 0.8 * R)       # no relu before the sum
+    sref, smn, smx = oracle.quantized_elemwise_add(ro2, res8, qmn, qmx, -0.6 * R, 0.6 * R,
+                                                   min_calib_range=-R, max_calib_range=1.1 * R)
+    if relu:
+        sref = oracle.relu_i8(sref)
+    ress = capi.quantized_fc_sum(dev(d), dev(w), None if b is None else dev(b), dev(res8),
+                                 f32(-rd), f32(rd), f32(-rw), f32(rw),
+                                 None if b is None else f32(-rb), None if b is None else f32(rb),
+                                 f32(-0.6 * R), f32(0.6 * R), (-R, 0.8 * R), (-R, 1.1 * R),
+                                 sum_relu=relu)
+    np.testing.assert_array_equal(ress["out8"].cpu().numpy(), sref)
+    assert (ress["rmin"].item(), ress["rmax"].item()) == (smn, smx)
 
 
 def conv_cases():
