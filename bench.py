@@ -48,12 +48,12 @@ MEASURED_TRAFFIC_BYTES = {
     "dequantize": ((2.0 * 32782.0 + 262144.0) * _KIB, "profiles/dequantize_chunk_kernel_64M.md"),
     "elemwise_add": ((2.0 * 65557.2 + 262144.1) * _KIB, "profiles/add32_chunk_kernel_64M.md"),
     "elemwise_add_int8": ((2.0 * 65583.7 + 65536.1) * _KIB, "profiles/add_kernel_int8_64M.md"),
-    "concat": ((2.0 * 32840.8 + 65536.1) * _KIB, "profiles/concat_kernel_64M.md"),
+    "concat": ((2.0 * 32890.0 + 65536.1) * _KIB, "profiles/concat_kernel_64M.md"),
     "elemwise_mul_int8": ((2.0 * 65565.8 + 65536.1) * _KIB, "profiles/mul_kernel_int8_64M.md"),
     "quantize_asym": ((2.0 * 131099.2 + 65536.1) * _KIB, "profiles/quantize_asym_kernel_64M.md"),
-    "batch_norm": ((2.0 * 32819.7 + 65536.0) * _KIB, "profiles/bn_rows_kernel_nchw_64M.md"),
+    "batch_norm": ((2.0 * 32815.5 + 65536.0) * _KIB, "profiles/bn_rows_kernel_nchw_64M.md"),
     "embedding": ((2.0 * 31709.6 + 65535.8) * _KIB, "profiles/embedding_kernel_bert_vocab.md"),
-    "transpose": ((2.0 * 32796.4 + 65536.1) * _KIB, "profiles/permute_elem_kernel_attention_64M.md"),
+    "transpose": ((2.0 * 32800.1 + 65548.3) * _KIB, "profiles/permute_elem_direct_kernel_attention_64M.md"),
     "maxpool": ((2.0 * 100388.0 + 50177.2) * _KIB, "profiles/pool_lds_kernel_maxpool.md"),
     "avgpool": ((2.0 * 200728.0 + 8192.1) * _KIB, "profiles/pool_lds_kernel_global_avgpool.md"),
     "resnet50_convs": (521.8e6, "profiles/conv_stack_resnet50.md"),
@@ -243,7 +243,7 @@ class CastWorkload:
             self.imin = torch.tensor([-3.0], device="cuda")
             self.imax = torch.tensor([3.0], device="cuda")
             self.bytes = 2.0 * n
-            self.kernel = "relu_i8_kernel"
+            self.kernel = "relu_chunk_kernel"
             self.name = "quantized_act relu int8->int8"
         elif kind == "dequantize":
             self.src = [torch.randint(-127, 128, (n,), device="cuda", generator=g,
@@ -350,7 +350,7 @@ class CastWorkload:
             self.c_shape = (ctypes.c_int64 * 4)(*self.shape)
             self.c_axes = (ctypes.c_int * 4)(0, 2, 1, 3)
             self.bytes = 2.0 * n
-            self.kernel = "permute_elem_kernel"
+            self.kernel = "permute_elem_direct_kernel"
             self.name = "quantized_transpose int8 %s axes (0,2,1,3)" % (self.shape,)
         else:
             raise ValueError(kind)

@@ -376,6 +376,58 @@ __global__ __launch_bounds__(kThreads) void permute_elem_kernel(ElemArgs e) {
   pass_range(a.imin, a.imax, a.omin, a.omax);
 }
 
+// The same swap for runs of 16, 32, 64, 128 or 256 bytes without LDS: the 64 lanes of a wave
+// are (16-byte piece of the run) x (2^sa_shift runs along A) x (2^sb_shift runs along B), so
+// one load instruction reads 2^sa_shift consecutive runs of the input for each of its B
+// positions and one store instruction writes 2^sb_shift consecutive runs of the output for
+// each of its A positions: at least 128 contiguous bytes on both sides.  A lane moves
+// kElemDirectPieces pieces that follow one another along B; one wave per tile, no loop.
+constexpr int kElemDirectPieces = 2;
+
+struct ElemDirectArgs {
+  TileArgs t;  // A / B count runs; a_out_stride / b_in_stride in bytes; tiles_a = tiles along A
+  unsigned tiles_b;
+  int e16_shift, sa_shift, sb_shift;
+};
+
+__global__ __launch_bounds__(kThreads) void permute_elem_direct_kernel(ElemDirectArgs e) {
+  const TileArgs& a = e.t;
+  const uint32_t lane = threadIdx.x & 63u;
+  const uint32_t within = lane & ((1u << e.e16_shift) - 1u);
+  const uint32_t asub = (lane >> e.e16_shift) & ((1u << e.sa_shift) - 1u);
+  const uint32_t bsub = lane >> (e.e16_shift + e.sa_shift);
+  const uint64_t per_batch = uint64_t(a.tiles_a) * e.tiles_b;
+  const uint64_t wave = uint64_t(blockIdx.x) * (kThreads / 64) +
+                        __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  if (wave < per_batch * static_cast<uint64_t>(a.batches)) {
+    const uint64_t z = wave / per_batch, rem = wave - z * per_batch;
+    const uint64_t tb = rem / a.tiles_a, ta = rem - tb * a.tiles_a;
+    size_t in_off, out_off;
+    batch_offsets(a, static_cast<int64_t>(z), in_off, out_off);
+    const int64_t ai = static_cast<int64_t>(ta << e.sa_shift) + asub;
+    const int64_t b0 = static_cast<int64_t>((tb * kElemDirectPieces) << e.sb_shift) + bsub;
+    const int E = 16 << e.e16_shift;
+    const uint8_t* src = a.in + in_off + static_cast<size_t>(ai) * E + 16 * within;
+    uint8_t* dst = a.out + out_off + static_cast<size_t>(ai * a.a_out_stride) + 16 * within;
+    u4 v[kElemDirectPieces];
+#pragma unroll
+    for (int j = 0; j < kElemDirectPieces; ++j) {
+      const int64_t b = b0 + (int64_t(j) << e.sb_shift);
+      v[j] = (ai < a.A && b < a.B)
+                 ? __builtin_nontemporal_load(
+                       reinterpret_cast<const u4*>(src + static_cast<size_t>(b * a.b_in_stride)))
+                 : u4{0, 0, 0, 0};
+    }
+#pragma unroll
+    for (int j = 0; j < kElemDirectPieces; ++j) {
+      const int64_t b = b0 + (int64_t(j) << e.sb_shift);
+      if (ai < a.A && b < a.B)
+        __builtin_nontemporal_store(v[j], reinterpret_cast<u4*>(dst + static_cast<size_t>(b) * E));
+    }
+  }
+  pass_range(a.imin, a.imax, a.omin, a.omax);
+}
+
 __global__ void range_only_kernel(const float* imin, const float* imax, float* omin, float* omax) {
   *omin = *imin;
   *omax = *imax;
@@ -538,6 +590,32 @@ int mxq_quantized_transpose(void* stream, const void* in, const float* imin, con
           t.p_out_stride[t.p.nd] = out_stride[d];
           t.batches *= oe[d];
           ++t.p.nd;
+        }
+        const int e16 = e.E >> 4;
+        if ((e16 & (e16 - 1)) == 0 && e16 <= 16) {
+          // power-of-two runs: straight through registers
+          ElemDirectArgs d;
+          d.t = t;
+          d.e16_shift = __builtin_ctz(e16);
+          const int run_shift = 6 - d.e16_shift;  // runs per wave instruction
+          d.sa_shift = (run_shift + 1) / 2;
+          d.sb_shift = run_shift - d.sa_shift;
+          const int64_t da_tiles = (t.A + (int64_t(1) << d.sa_shift) - 1) >> d.sa_shift;
+          const int64_t per_b = int64_t(kElemDirectPieces) << d.sb_shift;
+          const int64_t db_tiles = (t.B + per_b - 1) / per_b;
+          const int64_t waves_per_group = kThreads / 64;
+          if (da_tiles < (int64_t(1) << 31) && db_tiles < (int64_t(1) << 31) &&
+              t.batches < (int64_t(1) << 40) / (da_tiles * db_tiles + 1)) {
+            const int64_t groups = (da_tiles * db_tiles * t.batches + waves_per_group - 1) / waves_per_group;
+            if (groups < (int64_t(1) << 31)) {
+              d.t.tiles_a = static_cast<unsigned>(da_tiles);
+              d.tiles_b = static_cast<unsigned>(db_tiles);
+              hipLaunchKernelGGL(permute_elem_direct_kernel, dim3(static_cast<unsigned>(groups)),
+                                 dim3(kThreads), 0, s, d);
+              MXQ_LAUNCH_CHECK();
+              return 0;
+            }
+          }
         }
         const int64_t ta = (t.A + e.T - 1) / e.T, tb = (t.B + e.T - 1) / e.T;
         if (ta * tb < (int64_t(1) << 31)) {

@@ -175,6 +175,36 @@ def test_quantized_act_chunk_kernel_edges(contrib, n):
     assert np.array_equal(out_buf[:1 << 20].cpu().numpy(), ref)
 
 
+CONCAT_EDGE_CASES = [
+    # (shapes, axis, dtype, (min, max) per input)
+    ([((1 << 25) + 16,), ((1 << 25) + 4096 * 16 - 16,)], 0, np.int8, [(-1.0, 1.0), (-2.0, 2.0)]),
+    ([(8, 3, 1 << 20), (8, 0, 1 << 20), (8, 5, (1 << 20))], 1, np.int8,
+     [(-1.0, 0.5), (-1.0, 1.0), (-3.0, 4.0)]),
+    ([(4, (1 << 23) + 48), (4, (1 << 23) + 16 * 1023)], 1, np.uint8, [(0.0, 1.0), (0.0, 2.5)]),
+    ([(2, 1 << 24, 2), (2, (1 << 24) + 8, 2)], 1, np.int8, [(-2.0, 2.0), (-2.0, 2.0)]),
+]
+
+
+@pytest.mark.parametrize("case", range(len(CONCAT_EDGE_CASES)))
+def test_concat_chunk_kernel_edges(contrib, case):
+    """From 64 MiB per launch, with every input 16-byte aligned, concat runs one chunk of 1024
+    16-byte pieces per work-group: partial last chunks, several rows with a pitch, an empty
+    input between two others, uint8, and equal ranges (the byte copy)."""
+    shapes, axis, dtype, ranges = CONCAT_EDGE_CASES[case]
+    rng = np.random.default_rng(100 + case)
+    lo, hi = (0, 256) if dtype == np.uint8 else (-128, 128)
+    xs = [rng.integers(lo, hi, size=s, dtype=np.int64).astype(dtype) for s in shapes]
+    args = [torch.from_numpy(x).cuda() for x in xs]
+    for mn, mx in ranges:
+        args += [f32(mn), f32(mx)]
+    out, omn, omx = contrib.quantized_concat(*args, num_args=len(xs), dim=axis)
+    ref, rmn, rmx = oracle.quantized_concat(xs, [r[0] for r in ranges], [r[1] for r in ranges],
+                                            dim=axis)
+    assert tuple(out.shape) == ref.shape
+    assert (omn.item(), omx.item()) == (rmn, rmx)
+    assert np.array_equal(out.cpu().numpy(), ref)
+
+
 def test_elemwise_add_64m(contrib):
     g = torch.Generator(device="cuda").manual_seed(5)
     a = torch.randint(-127, 128, (N_CAST,), device="cuda", generator=g, dtype=torch.int8)

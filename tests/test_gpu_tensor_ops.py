@@ -241,6 +241,10 @@ def test_transpose_every_permutation(contrib, shape, axes):
     ((3, 37, 19, 48), (0, 2, 1, 3)),        # runs of 48 bytes, ragged tiles of runs
     ((2, 9, 50, 16), (0, 2, 1, 3)),         # runs of 16 bytes
     ((5, 8, 9, 256), (0, 2, 1, 3)),         # runs of 256 bytes
+    ((3, 13, 21, 128), (0, 2, 1, 3)),       # runs of 128 bytes, both swapped axes ragged
+    ((3, 35, 9, 64), (0, 2, 1, 3)),         # runs of 64 bytes, ragged
+    ((2, 33, 17, 32), (0, 2, 1, 3)),        # runs of 32 bytes, ragged
+    ((9, 4, 11, 64), (2, 1, 0, 3)),         # the outermost axis swaps with the third
     ((2, 11, 3, 20, 32), (0, 3, 2, 1, 4)),  # an axis between the two that swap
     ((3, 1000, 10, 16), (2, 1, 0, 3)),      # one of the two axes too short for run tiles
     ((3, 32, 52), (0, 2, 1)),               # dword / 16-byte friendly, partial tiles
