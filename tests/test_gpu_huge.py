@@ -1,5 +1,5 @@
-"""Tensors past the 32-bit marks: more than 2^32 elements through the casts and the
-element-wise sum, operands and outputs of 2 GiB and more through the fully-connected and
+"""Tensors past the 32-bit marks: more than 2^32 elements through the casts, the relu, the
+element-wise sum, concat and transpose, operands and outputs of 2 GiB and more through the fully-connected and
 convolution launchers (the direct-to-LDS kernels address operands with 32-bit offsets, so
 the launchers must route these elsewhere).  The oracle recomputes windows that sit on the
 marks (start, 2^31, 2^32, end); every other element is covered by a size-independent
@@ -153,6 +153,67 @@ def test_elemwise_add_past_4g_elements(contrib):
             part, _, _ = contrib.quantized_elemwise_add(a8[s:e], b8[s:e], *scal, **kw)
             assert torch.equal(out[s:e], part), f"piece at {s}"
         del out
+
+
+def test_quantized_act_past_4g_elements(contrib):
+    g = torch.Generator(device="cuda").manual_seed(12)
+    x = torch.randint(-128, 128, (N_BIG,), dtype=torch.int8, device="cuda", generator=g)
+    out, mn, mx = contrib.quantized_act(x, f32(-2.0), f32(3.0), act_type="relu")
+    torch.cuda.synchronize()
+    assert (mn.item(), mx.item()) == (-2.0, 3.0)
+    for s, e in windows(N_BIG):
+        np.testing.assert_array_equal(out[s:e].cpu().numpy(), oracle.relu_i8(x[s:e].cpu().numpy()),
+                                      err_msg=f"window {s}")
+    for s, e in pieces(N_BIG):
+        assert torch.equal(out[s:e], torch.clamp(x[s:e], min=0)), f"piece at {s}"
+
+
+def test_concat_past_4g_bytes(contrib):
+    """Two rows of two inputs, 2^30 + 4096 + 16 bytes per row and input: the output passes
+    2^32 bytes, one input is rescaled to the hull of the ranges and one is copied."""
+    L = (1 << 30) + 4096 + 16
+    g = torch.Generator(device="cuda").manual_seed(13)
+    a = torch.randint(-128, 128, (2, L), dtype=torch.int8, device="cuda", generator=g)
+    b = torch.randint(-128, 128, (2, L), dtype=torch.int8, device="cuda", generator=g)
+    rng = [(-1.0, 0.5), (-2.0, 2.0)]
+    scal = [f32(v) for r in rng for v in r]
+    out, mn, mx = contrib.quantized_concat(a, b, *scal, num_args=2, dim=1)
+    torch.cuda.synchronize()
+    assert tuple(out.shape) == (2, 2 * L)
+    for s in (0, (1 << 29), L - WIN):
+        cols = slice(s, s + WIN)
+        ref, rmn, rmx = oracle.quantized_concat([a[:, cols].cpu().numpy(), b[:, cols].cpu().numpy()],
+                                                [r[0] for r in rng], [r[1] for r in rng], dim=1)
+        assert (mn.item(), mx.item()) == (rmn, rmx)
+        got = torch.cat([out[:, cols], out[:, L + s:L + s + WIN]], dim=1)
+        np.testing.assert_array_equal(got.cpu().numpy(), ref, err_msg=f"columns from {s}")
+    step = 1 << 26
+    for s in range(0, L, step):
+        cols = slice(s, min(s + step, L))
+        part, _, _ = contrib.quantized_concat(a[:, cols].contiguous(), b[:, cols].contiguous(),
+                                              *scal, num_args=2, dim=1)
+        w = part.shape[1] // 2
+        assert torch.equal(out[:, cols], part[:, :w]), f"first input, columns from {s}"
+        assert torch.equal(out[:, L + cols.start:L + cols.stop], part[:, w:]), \
+            f"second input, columns from {s}"
+
+
+def test_transpose_past_4g_bytes(contrib):
+    """(batch, seq, heads, 64) -> (batch, heads, seq, 64) over more than 2^32 bytes: pure byte
+    movement, so torch's own permute is an independent check of every byte; the oracle
+    recomputes the first and the last batch entry."""
+    shape = (33, 4096, 512, 64)
+    g = torch.Generator(device="cuda").manual_seed(14)
+    x = torch.randint(-128, 128, shape, dtype=torch.int8, device="cuda", generator=g)
+    out, mn, mx = contrib.quantized_transpose(x, f32(-1.5), f32(2.5), axes=(0, 2, 1, 3))
+    torch.cuda.synchronize()
+    assert tuple(out.shape) == (33, 512, 4096, 64)
+    for n in (0, 32):
+        ref, rmn, rmx = oracle.quantized_transpose(x[n:n + 1].cpu().numpy(), -1.5, 2.5, (0, 2, 1, 3))
+        np.testing.assert_array_equal(out[n:n + 1].cpu().numpy(), ref, err_msg=f"batch entry {n}")
+        assert (mn.item(), mx.item()) == (rmn, rmx)
+    for n in range(shape[0]):
+        assert torch.equal(out[n], x[n].permute(1, 0, 2)), f"batch entry {n}"
 
 
 def fc_reference(d, w, b, rows, calib, relu):
