@@ -54,6 +54,8 @@ MEASURED_TRAFFIC_BYTES = {
     "batch_norm": ((2.0 * 32815.5 + 65536.0) * _KIB, "profiles/bn_rows_kernel_nchw_64M.md"),
     "embedding": ((2.0 * 31709.6 + 65535.8) * _KIB, "profiles/embedding_kernel_bert_vocab.md"),
     "transpose": ((2.0 * 32800.1 + 65548.3) * _KIB, "profiles/permute_elem_direct_kernel_attention_64M.md"),
+    "transpose_to_nhwc": ((2.0 * 32797.6 + 65541.4) * _KIB, "profiles/permute_tile16_kernel_to_nhwc_64M.md"),
+    "transpose_to_nchw": ((2.0 * 32797.6 + 65538.6) * _KIB, "profiles/permute_tile16_kernel_to_nchw_64M.md"),
     "maxpool": ((2.0 * 100388.0 + 50177.2) * _KIB, "profiles/pool_lds_kernel_maxpool.md"),
     "avgpool": ((2.0 * 200728.0 + 8192.1) * _KIB, "profiles/pool_lds_kernel_global_avgpool.md"),
     "resnet50_convs": (521.8e6, "profiles/conv_stack_resnet50.md"),
@@ -71,7 +73,8 @@ def parse_args():
                              "quantize_laplace", "quantize_uint8_uncal", "small_casts",
                              "requantize", "requantize_uncal", "dequantize", "copy", "maxpool", "avgpool",
                              "elemwise_add", "elemwise_add_int8", "concat", "elemwise_mul_int8", "quantize_asym",
-                             "batch_norm", "embedding", "transpose", "resnet50_convs", "resnet50_chain",
+                             "batch_norm", "embedding", "transpose", "transpose_to_nhwc", "transpose_to_nchw",
+                             "resnet50_convs", "resnet50_chain",
                              "resnet50_chain_fused", "resnet50_chain_unfused",
                              "bert_fc_chain",
                              "bert_fc_chain_fused",
@@ -339,19 +342,25 @@ class CastWorkload:
             self.bytes = (2.0 * 768 + 4.0) * self.rows
             self.kernel = "embedding_kernel"
             self.name = "quantized_embedding, 30522 x 768 int8 table, %d int32 ids" % self.rows
-        elif kind == "transpose":
-            # attention layout change (batch, seq, heads, 64) -> (batch, heads, seq, 64)
-            self.shape = (n // (512 * 16 * 64), 512, 16, 64)
+        elif kind in ("transpose", "transpose_to_nhwc", "transpose_to_nchw"):
+            # attention layout change (batch, seq, heads, 64) -> (batch, heads, seq, 64), or
+            # the layout change at a convolution's boundary, NCHW <-> NHWC of 256 x 64 x 64
+            self.shape, self.axes = {
+                "transpose": ((n // (512 * 16 * 64), 512, 16, 64), (0, 2, 1, 3)),
+                "transpose_to_nhwc": ((n // (256 * 64 * 64), 256, 64, 64), (0, 2, 3, 1)),
+                "transpose_to_nchw": ((n // (256 * 64 * 64), 64, 64, 256), (0, 3, 1, 2)),
+            }[kind]
             self.src = [torch.randint(-127, 128, self.shape, device="cuda", generator=g,
                                       dtype=torch.int8) for _ in range(self.NBUF)]
             self.dst = [torch.empty(n, dtype=torch.int8, device="cuda") for _ in range(self.NBUF)]
             self.imin = torch.tensor([-1.0], device="cuda")
             self.imax = torch.tensor([1.0], device="cuda")
             self.c_shape = (ctypes.c_int64 * 4)(*self.shape)
-            self.c_axes = (ctypes.c_int * 4)(0, 2, 1, 3)
+            self.c_axes = (ctypes.c_int * 4)(*self.axes)
             self.bytes = 2.0 * n
-            self.kernel = "permute_elem_direct_kernel"
-            self.name = "quantized_transpose int8 %s axes (0,2,1,3)" % (self.shape,)
+            self.kernel = "permute_elem_direct_kernel" if kind == "transpose" else "permute_tile16_kernel"
+            self.name = "quantized_transpose int8 %s axes (%s)" % (
+                self.shape, ",".join(str(a) for a in self.axes))
         else:
             raise ValueError(kind)
         self.name += ", %d elements" % n
@@ -423,7 +432,7 @@ class CastWorkload:
             rc = lib.mxq_quantized_embedding(st, P(self.src[k]), 4, P(self.table), P(self.imin),
                                              P(self.imax), P(self.dst[k]), P(self.omin),
                                              P(self.omax), self.rows, 30522, 768)
-        elif kind == "transpose":
+        elif kind.startswith("transpose"):
             rc = lib.mxq_quantized_transpose(st, P(self.src[k]), P(self.imin), P(self.imax),
                                              P(self.dst[k]), P(self.omin), P(self.omax), 4,
                                              self.c_shape, self.c_axes)
@@ -444,8 +453,8 @@ class CastWorkload:
             n = (n // 768) * 768
             x = self.src[0][:n // 768].cpu().numpy()
             table = self.table.cpu().numpy()
-        elif kind == "transpose":
-            x = self.src[0][:n // (512 * 16 * 64)].cpu().numpy()
+        elif kind.startswith("transpose"):
+            x = self.src[0][:n // (self.shape[1] * self.shape[2] * self.shape[3])].cpu().numpy()
         elif kind == "batch_norm":
             x = self.src[0][:n].cpu().numpy().reshape(-1, self.channels, self.inner)
             bn = [t.cpu().numpy() for t in (self.gamma, self.beta, self.mean, self.var)]
@@ -483,8 +492,8 @@ class CastWorkload:
                 oracle.quantized_batch_norm(x, *bn, -3.0, 3.0, -6.0, 6.0, relu=True)
             elif kind == "embedding":
                 oracle.quantized_embedding(x, table, -1.0, 1.0)
-            elif kind == "transpose":
-                oracle.quantized_transpose(x, -1.0, 1.0, (0, 2, 1, 3))
+            elif kind.startswith("transpose"):
+                oracle.quantized_transpose(x, -1.0, 1.0, self.axes)
             else:
                 oracle.dequantize(x, -3.0, 3.0)
             reps += 1
@@ -1223,7 +1232,8 @@ def main():
                      "requantize",
                      "requantize_uncal", "dequantize", "elemwise_add", "elemwise_add_int8",
                      "concat", "elemwise_mul_int8", "quantize_asym", "batch_norm", "embedding",
-                     "transpose", "maxpool", "avgpool", "fc8192",
+                     "transpose", "transpose_to_nhwc", "transpose_to_nchw", "maxpool", "avgpool",
+                     "fc8192",
                      "resnet50_convs", "resnet50_chain_unfused", "resnet50_chain", "resnet50_chain_fused",
                      "bert_fc_chain",
                      "bert_fc_chain_fused", "bert_fc_chain_f32"]:

@@ -255,39 +255,45 @@ __device__ __forceinline__ void batch_offsets(const TileArgs& a, int64_t z, size
 }
 
 // The same for friendly strides (A % 4 == 0 and every input stride a multiple of 4; B % 16
-// == 0 and every output stride a multiple of 16; aligned pointers): 64 (B) x 128 (A) bytes
+// == 0 and every output stride a multiple of 16; aligned pointers): TB (B) x 128 (A) bytes
 // per tile, every thread loads dwords along A (a wave reads whole 128-byte runs), transposes
 // 4 x 4 bytes in registers with v_perm and parks the result in LDS, from where 16-byte
-// pieces of the output rows leave.
+// pieces of the output rows leave.  TB = 128 makes the output runs whole cache lines too.
+template <int TB>
 __global__ __launch_bounds__(kThreads) void permute_tile4_kernel(TileArgs a) {
-  constexpr int kPitch = 17;  // dwords per transposed row: 64 bytes + 4 of padding
+  constexpr int kPitch = TB / 4 + 1;  // dwords per transposed row: TB bytes + 4 of padding
+  constexpr int kPasses = TB / 32;
   __shared__ uint32_t tile[128 * kPitch];
   const int t = threadIdx.x;
   const int64_t tb = blockIdx.x / a.tiles_a, ta = blockIdx.x - tb * a.tiles_a;
-  const int64_t a0 = ta * 128, b0 = tb * 64;
+  const int64_t a0 = ta * 128, b0 = tb * TB;
   const int sq = t & 31;
   for (int64_t z = blockIdx.y; z < a.batches; z += gridDim.y) {
     size_t in_off, out_off;
     batch_offsets(a, z, in_off, out_off);
     const uint8_t* src = a.in + in_off;
     uint8_t* dst = a.out + out_off;
+    const int64_t aa = a0 + 4 * sq;
+    // every dword of the thread first, then the byte transposes and the LDS writes
+    uint32_t w[kPasses][4];
 #pragma unroll
-    for (int pass = 0; pass < 2; ++pass) {
-      const int rq = (t >> 5) + 8 * pass;
-      const int64_t aa = a0 + 4 * sq;
-      uint32_t w[4];
+    for (int pass = 0; pass < kPasses; ++pass)
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        const int64_t b = b0 + 4 * rq + j;
-        w[j] = (b < a.B && aa < a.A)
-                   ? *reinterpret_cast<const uint32_t*>(src + static_cast<size_t>(b * a.b_in_stride + aa))
-                   : 0u;
+        const int64_t b = b0 + 4 * ((t >> 5) + 8 * pass) + j;
+        w[pass][j] = (b < a.B && aa < a.A)
+                         ? __builtin_nontemporal_load(reinterpret_cast<const uint32_t*>(
+                               src + static_cast<size_t>(b * a.b_in_stride + aa)))
+                         : 0u;
       }
+#pragma unroll
+    for (int pass = 0; pass < kPasses; ++pass) {
+      const int rq = (t >> 5) + 8 * pass;
       // x[i] = byte i of w[0..3]
-      const uint32_t t0 = __builtin_amdgcn_perm(w[1], w[0], 0x05010400u);
-      const uint32_t t1 = __builtin_amdgcn_perm(w[1], w[0], 0x07030602u);
-      const uint32_t t2 = __builtin_amdgcn_perm(w[3], w[2], 0x05010400u);
-      const uint32_t t3 = __builtin_amdgcn_perm(w[3], w[2], 0x07030602u);
+      const uint32_t t0 = __builtin_amdgcn_perm(w[pass][1], w[pass][0], 0x05010400u);
+      const uint32_t t1 = __builtin_amdgcn_perm(w[pass][1], w[pass][0], 0x07030602u);
+      const uint32_t t2 = __builtin_amdgcn_perm(w[pass][3], w[pass][2], 0x05010400u);
+      const uint32_t t3 = __builtin_amdgcn_perm(w[pass][3], w[pass][2], 0x07030602u);
       tile[(4 * sq + 0) * kPitch + rq] = __builtin_amdgcn_perm(t2, t0, 0x05040100u);
       tile[(4 * sq + 1) * kPitch + rq] = __builtin_amdgcn_perm(t2, t0, 0x07060302u);
       tile[(4 * sq + 2) * kPitch + rq] = __builtin_amdgcn_perm(t3, t1, 0x05040100u);
@@ -295,17 +301,78 @@ __global__ __launch_bounds__(kThreads) void permute_tile4_kernel(TileArgs a) {
     }
     __syncthreads();
     const int64_t left = a.B - b0;
-    const int nb = left < 64 ? static_cast<int>(left) : 64;  // bytes per output row (16 | nb)
-    const int per_row = nb >> 4;                              // 16-byte pieces per row: 1..4
+    const int nb = left < TB ? static_cast<int>(left) : TB;  // bytes per output row (16 | nb)
+    const int per_row = nb >> 4;                              // 16-byte pieces per row
     const int pieces = 128 * per_row;
     for (int c = t; c < pieces; c += kThreads) {
-      const int sl = per_row == 4 ? (c >> 2) : (per_row == 2 ? (c >> 1) : (per_row == 1 ? c : c / 3));
+      const int sl = per_row == TB / 16 ? c / (TB / 16) : c / per_row;
       const int k = c - sl * per_row;
-      if (a0 + sl >= a.A) continue;
-      u4 v;
+      if (a0 + sl < a.A) {
+        u4 v;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) v[i] = tile[sl * kPitch + 4 * k + i];
-      *reinterpret_cast<u4*>(dst + static_cast<size_t>((a0 + sl) * a.a_out_stride + b0 + 16 * k)) = v;
+        for (int i = 0; i < 4; ++i) v[i] = tile[sl * kPitch + 4 * k + i];
+        __builtin_nontemporal_store(
+            v, reinterpret_cast<u4*>(dst + static_cast<size_t>((a0 + sl) * a.a_out_stride + b0 + 16 * k)));
+      }
+    }
+    __syncthreads();
+  }
+  pass_range(a.imin, a.imax, a.omin, a.omax);
+}
+
+// The same with 16-byte loads (A % 16 == 0 and every input stride a multiple of 16 as well):
+// a thread takes 16 bytes along A of four consecutive B rows, so the 128 x 128-byte tile
+// costs it four load instructions instead of sixteen; 8 lanes cover a row's 128 bytes.
+__global__ __launch_bounds__(kThreads) void permute_tile16_kernel(TileArgs a) {
+  constexpr int kPitch = 33;  // dwords per transposed row: 128 bytes + 4 of padding
+  __shared__ uint32_t tile[128 * kPitch];
+  const int t = threadIdx.x;
+  const int64_t tb = blockIdx.x / a.tiles_a, ta = blockIdx.x - tb * a.tiles_a;
+  const int64_t a0 = ta * 128, b0 = tb * 128;
+  const int sq = t & 7, rq = t >> 3;
+  for (int64_t z = blockIdx.y; z < a.batches; z += gridDim.y) {
+    size_t in_off, out_off;
+    batch_offsets(a, z, in_off, out_off);
+    const uint8_t* src = a.in + in_off;
+    uint8_t* dst = a.out + out_off;
+    const int64_t aa = a0 + 16 * sq;
+    u4 w[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int64_t b = b0 + 4 * rq + j;
+      w[j] = (b < a.B && aa < a.A)
+                 ? __builtin_nontemporal_load(reinterpret_cast<const u4*>(
+                       src + static_cast<size_t>(b * a.b_in_stride + aa)))
+                 : u4{0, 0, 0, 0};
+    }
+#pragma unroll
+    for (int d = 0; d < 4; ++d) {
+      // x[i] = byte i of w[0..3][d]
+      const uint32_t t0 = __builtin_amdgcn_perm(w[1][d], w[0][d], 0x05010400u);
+      const uint32_t t1 = __builtin_amdgcn_perm(w[1][d], w[0][d], 0x07030602u);
+      const uint32_t t2 = __builtin_amdgcn_perm(w[3][d], w[2][d], 0x05010400u);
+      const uint32_t t3 = __builtin_amdgcn_perm(w[3][d], w[2][d], 0x07030602u);
+      const int row = 16 * sq + 4 * d;
+      tile[(row + 0) * kPitch + rq] = __builtin_amdgcn_perm(t2, t0, 0x05040100u);
+      tile[(row + 1) * kPitch + rq] = __builtin_amdgcn_perm(t2, t0, 0x07060302u);
+      tile[(row + 2) * kPitch + rq] = __builtin_amdgcn_perm(t3, t1, 0x05040100u);
+      tile[(row + 3) * kPitch + rq] = __builtin_amdgcn_perm(t3, t1, 0x07060302u);
+    }
+    __syncthreads();
+    const int64_t left = a.B - b0;
+    const int nb = left < 128 ? static_cast<int>(left) : 128;  // bytes per output row (16 | nb)
+    const int per_row = nb >> 4;
+    const int pieces = 128 * per_row;
+    for (int c = t; c < pieces; c += kThreads) {
+      const int sl = per_row == 8 ? c >> 3 : c / per_row;
+      const int k = c - sl * per_row;
+      if (a0 + sl < a.A) {
+        u4 v;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) v[i] = tile[sl * kPitch + 4 * k + i];
+        __builtin_nontemporal_store(
+            v, reinterpret_cast<u4*>(dst + static_cast<size_t>((a0 + sl) * a.a_out_stride + b0 + 16 * k)));
+      }
     }
     __syncthreads();
   }
@@ -678,13 +745,22 @@ int mxq_quantized_transpose(void* stream, const void* in, const float* imin, con
   for (int d = 0; d < a.p.nd; ++d)
     friendly = friendly && (a.p.in_stride[d] % 4 == 0) && (a.p_out_stride[d] % 16 == 0);
   if (friendly) {
-    const int64_t fa = (a.A + 127) / 128, fb = (a.B + 63) / 64;
+    // output rows of 128 bytes per tile (whole cache lines on both sides) where B has them
+    // and A fills the tile's 128 columns (with 64 the larger tile idles half its lanes)
+    const int tile_b = (a.B >= 128 && a.A >= 128) ? 128 : 64;
+    const int64_t fa = (a.A + 127) / 128, fb = (a.B + tile_b - 1) / tile_b;
     if (fa * fb < (int64_t(1) << 31)) {
       a.tiles_a = static_cast<unsigned>(fa);
       const int64_t fy = a.batches < 65535 ? a.batches : 65535;
-      hipLaunchKernelGGL(permute_tile4_kernel,
-                         dim3(static_cast<unsigned>(fa * fb), static_cast<unsigned>(fy)),
-                         dim3(kThreads), 0, s, a);
+      const dim3 grid(static_cast<unsigned>(fa * fb), static_cast<unsigned>(fy));
+      bool friendly16 = (a.A % 16 == 0) && (a.b_in_stride % 16 == 0);
+      for (int d = 0; d < a.p.nd; ++d) friendly16 = friendly16 && (a.p.in_stride[d] % 16 == 0);
+      if (tile_b == 128 && friendly16)
+        hipLaunchKernelGGL(permute_tile16_kernel, grid, dim3(kThreads), 0, s, a);
+      else if (tile_b == 128)
+        hipLaunchKernelGGL(permute_tile4_kernel<128>, grid, dim3(kThreads), 0, s, a);
+      else
+        hipLaunchKernelGGL(permute_tile4_kernel<64>, grid, dim3(kThreads), 0, s, a);
       MXQ_LAUNCH_CHECK();
       return 0;
     }

@@ -177,7 +177,10 @@ def test_layout_adapters(capi):
     np.testing.assert_array_equal(y.cpu().numpy(), x.transpose(0, 2, 3, 1))
     z = capi.nhwc_to_nchw(y)
     np.testing.assert_array_equal(z.cpu().numpy(), x)
-    for shape in ((2, 8, 8, 64), (3, 4, 12, 20), (1, 16, 16, 132)):   # int8 NHWC -> NCHW, dword kernel
+    # int8 NHWC -> NCHW: the dword kernel, and from 128 pixels with 16 | C the 16-byte one
+    # (ragged last tiles in both directions)
+    for shape in ((2, 8, 8, 64), (3, 4, 12, 20), (1, 16, 16, 132), (2, 16, 8, 144),
+                  (2, 13, 12, 272), (1, 56, 56, 256)):
         v8 = int8_uniform(shape, seed=4)
         z8 = capi.nhwc_to_nchw(dev(v8))
         np.testing.assert_array_equal(z8.cpu().numpy(), v8.transpose(0, 3, 1, 2))
@@ -193,7 +196,8 @@ def test_layout_adapters(capi):
     for shape, cp in (((3, 5, 7, 9), 16), ((2, 3, 70, 33), 16), ((1, 70, 5, 5), 80),
                       ((2, 16, 4, 4), 16), ((2, 3, 8, 8), 16), ((2, 64, 12, 12), 64),
                       ((3, 70, 4, 8), 80), ((2, 130, 16, 4), 144), ((1, 40, 4, 4), 48),
-                      ((2, 20, 10, 30), 32)):
+                      ((2, 20, 10, 30), 32), ((2, 256, 12, 12), 256), ((1, 200, 20, 12), 208),
+                      ((2, 128, 56, 56), 128)):
         x = int8_uniform(shape, seed=3)
         n, c, h, w = shape
         out = torch.full((n, h, w, cp), 77, dtype=torch.int8, device="cuda")

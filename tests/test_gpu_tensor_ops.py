@@ -249,6 +249,9 @@ def test_transpose_every_permutation(contrib, shape, axes):
     ((3, 1000, 10, 16), (2, 1, 0, 3)),      # one of the two axes too short for run tiles
     ((3, 32, 52), (0, 2, 1)),               # dword / 16-byte friendly, partial tiles
     ((3, 20, 48), (0, 2, 1)),               # output rows not a multiple of 16
+    ((2, 144, 132), (0, 2, 1)),             # dword loads, 128-byte output rows, a 16-byte last tile
+    ((2, 176, 160), (0, 2, 1)),             # 16-byte loads, a last tile of three pieces per row
+    ((3, 5, 256, 144), (1, 0, 3, 2)),       # 16-byte loads under two permuted outer axes
     ((2, 3, 130, 260), (1, 0, 3, 2)),
     ((0, 5, 3), (2, 0, 1)),                 # empty
     ((7,), (0,)),
