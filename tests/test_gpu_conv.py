@@ -180,7 +180,8 @@ def test_layout_adapters(capi):
     # int8 NHWC -> NCHW: the dword kernel, and from 128 pixels with 16 | C the 16-byte one
     # (ragged last tiles in both directions)
     for shape in ((2, 8, 8, 64), (3, 4, 12, 20), (1, 16, 16, 132), (2, 16, 8, 144),
-                  (2, 13, 12, 272), (1, 56, 56, 256)):
+                  (2, 13, 12, 272), (1, 56, 56, 256), (3, 14, 14, 256), (2, 10, 15, 144),
+                  (2, 14, 14, 1040)):   # the last three: planes of 4 | H*W bytes, dword stores
         v8 = int8_uniform(shape, seed=4)
         z8 = capi.nhwc_to_nchw(dev(v8))
         np.testing.assert_array_equal(z8.cpu().numpy(), v8.transpose(0, 3, 1, 2))
