@@ -323,6 +323,7 @@ __global__ __launch_bounds__(kThreads) void permute_tile4_kernel(TileArgs a) {
 // The same with 16-byte loads (A % 16 == 0 and every input stride a multiple of 16 as well):
 // a thread takes 16 bytes along A of four consecutive B rows, so the 128 x 128-byte tile
 // costs it four load instructions instead of sixteen; 8 lanes cover a row's 128 bytes.
+template <int PIECE>
 __global__ __launch_bounds__(kThreads) void permute_tile16_kernel(TileArgs a) {
   constexpr int kPitch = 33;  // dwords per transposed row: 128 bytes + 4 of padding
   __shared__ uint32_t tile[128 * kPitch];
@@ -360,18 +361,23 @@ __global__ __launch_bounds__(kThreads) void permute_tile16_kernel(TileArgs a) {
     }
     __syncthreads();
     const int64_t left = a.B - b0;
-    const int nb = left < 128 ? static_cast<int>(left) : 128;  // bytes per output row (16 | nb)
-    const int per_row = nb >> 4;
+    const int nb = left < 128 ? static_cast<int>(left) : 128;  // bytes per output row (PIECE | nb)
+    const int per_row = nb / PIECE;
     const int pieces = 128 * per_row;
     for (int c = t; c < pieces; c += kThreads) {
-      const int sl = per_row == 8 ? c >> 3 : c / per_row;
+      const int sl = per_row == 128 / PIECE ? c / (128 / PIECE) : c / per_row;
       const int k = c - sl * per_row;
       if (a0 + sl < a.A) {
-        u4 v;
+        uint8_t* to = dst + static_cast<size_t>((a0 + sl) * a.a_out_stride + b0 + PIECE * k);
+        if (PIECE == 16) {
+          u4 v;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) v[i] = tile[sl * kPitch + 4 * k + i];
-        __builtin_nontemporal_store(
-            v, reinterpret_cast<u4*>(dst + static_cast<size_t>((a0 + sl) * a.a_out_stride + b0 + 16 * k)));
+          for (int i = 0; i < 4; ++i) v[i] = tile[sl * kPitch + 4 * k + i];
+          __builtin_nontemporal_store(v, reinterpret_cast<u4*>(to));
+        } else {
+          // output rows of 4 | B bytes (14 x 14 planes): dword pieces
+          __builtin_nontemporal_store(tile[sl * kPitch + k], reinterpret_cast<uint32_t*>(to));
+        }
       }
     }
     __syncthreads();
@@ -744,6 +750,26 @@ int mxq_quantized_transpose(void* stream, const void* in, const float* imin, con
                   (a.a_out_stride % 16 == 0) && aligned16(in) && aligned16(out);
   for (int d = 0; d < a.p.nd; ++d)
     friendly = friendly && (a.p.in_stride[d] % 4 == 0) && (a.p_out_stride[d] % 16 == 0);
+  {
+    // 16-byte loads with dword stores: output rows and strides that are multiples of 4 only
+    bool in16 = (a.A % 16 == 0) && (a.b_in_stride % 16 == 0) && aligned16(in);
+    bool out4 = (a.B % 4 == 0) && (a.a_out_stride % 4 == 0) &&
+                (reinterpret_cast<uintptr_t>(out) & 3u) == 0;
+    for (int d = 0; d < a.p.nd; ++d) {
+      in16 = in16 && (a.p.in_stride[d] % 16 == 0);
+      out4 = out4 && (a.p_out_stride[d] % 4 == 0);
+    }
+    const int64_t fa = (a.A + 127) / 128, fb = (a.B + 127) / 128;
+    if (!friendly && in16 && out4 && a.A >= 128 && a.B >= 128 && fa * fb < (int64_t(1) << 31)) {
+      a.tiles_a = static_cast<unsigned>(fa);
+      const int64_t fy = a.batches < 65535 ? a.batches : 65535;
+      hipLaunchKernelGGL(permute_tile16_kernel<4>,
+                         dim3(static_cast<unsigned>(fa * fb), static_cast<unsigned>(fy)),
+                         dim3(kThreads), 0, s, a);
+      MXQ_LAUNCH_CHECK();
+      return 0;
+    }
+  }
   if (friendly) {
     // output rows of 128 bytes per tile (whole cache lines on both sides) where B has them
     // and A fills the tile's 128 columns (with 64 the larger tile idles half its lanes)
@@ -756,7 +782,7 @@ int mxq_quantized_transpose(void* stream, const void* in, const float* imin, con
       bool friendly16 = (a.A % 16 == 0) && (a.b_in_stride % 16 == 0);
       for (int d = 0; d < a.p.nd; ++d) friendly16 = friendly16 && (a.p.in_stride[d] % 16 == 0);
       if (tile_b == 128 && friendly16)
-        hipLaunchKernelGGL(permute_tile16_kernel, grid, dim3(kThreads), 0, s, a);
+        hipLaunchKernelGGL(permute_tile16_kernel<16>, grid, dim3(kThreads), 0, s, a);
       else if (tile_b == 128)
         hipLaunchKernelGGL(permute_tile4_kernel<128>, grid, dim3(kThreads), 0, s, a);
       else

@@ -252,6 +252,8 @@ def test_transpose_every_permutation(contrib, shape, axes):
     ((2, 144, 132), (0, 2, 1)),             # dword loads, 128-byte output rows, a 16-byte last tile
     ((2, 176, 160), (0, 2, 1)),             # 16-byte loads, a last tile of three pieces per row
     ((3, 5, 256, 144), (1, 0, 3, 2)),       # 16-byte loads under two permuted outer axes
+    ((3, 14, 14, 256), (0, 3, 1, 2)),       # planes of 196 bytes: 16-byte loads, dword stores
+    ((2, 132, 144), (0, 2, 1)),             # the same with a 4-byte last tile
     ((2, 3, 130, 260), (1, 0, 3, 2)),
     ((0, 5, 3), (2, 0, 1)),                 # empty
     ((7,), (0,)),
