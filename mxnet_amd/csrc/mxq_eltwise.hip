@@ -903,17 +903,24 @@ struct BnArgs {
 // one factor and one offset per channel in the units of the int8 input and output; then the
 // library's own normalisation over mean 0 and variance 1, which divides the factor by
 // sqrt(1 + eps) once more.
+__device__ __forceinline__ void bn_channel(const BnArgs& a, uint32_t c, float max_abs_data,
+                                           float max_abs_output, float unit_std, float& factor,
+                                           float& offset) {
+  const float invstd = static_cast<float>(1.0 / sqrt(static_cast<double>(a.var[c]) + a.eps));
+  const float w = a.gamma[c] * invstd * max_abs_data / max_abs_output;
+  offset = (a.beta[c] - a.mean[c] * a.gamma[c] * invstd) * 127.5f / max_abs_output;
+  factor = w / unit_std;
+}
+
 __global__ __launch_bounds__(kThreads) void bn_table_kernel(BnArgs a) {
   const float max_abs_data = maxabs(*a.min_data, *a.max_data);
   const float max_abs_output = maxabs(a.min_calib, a.max_calib);
   const float unit_std = sqrtf(1.0f + static_cast<float>(a.eps));
   for (uint32_t c = blockIdx.x * kThreads + threadIdx.x; c < a.channels;
        c += gridDim.x * kThreads) {
-    const float invstd =
-        static_cast<float>(1.0 / sqrt(static_cast<double>(a.var[c]) + a.eps));
-    const float w = a.gamma[c] * invstd * max_abs_data / max_abs_output;
-    const float b = (a.beta[c] - a.mean[c] * a.gamma[c] * invstd) * 127.5f / max_abs_output;
-    a.table[c] = w / unit_std;
+    float w, b;
+    bn_channel(a, c, max_abs_data, max_abs_output, unit_std, w, b);
+    a.table[c] = w;
     a.table[a.channels + c] = b;
   }
   if (blockIdx.x == 0 && threadIdx.x == 0) {
@@ -1006,8 +1013,20 @@ __global__ __launch_bounds__(kThreads) void bn_kernel(BnArgs a) {
 // Rows of at least 1 KiB (inner % 16 == 0): one wave per 4 KiB piece of a row, so the channel,
 // its factor and offset are wave-uniform (scalar loads, no per-lane division) and a lane keeps
 // four 16-byte loads in flight.
-template <bool IN_U>
+// OWN_TABLE: no table kernel ran; every wave folds its channel's four parameters itself (the
+// same function, so the same factor and offset) and the first thread passes the range on.
+template <bool IN_U, bool OWN_TABLE>
 __global__ __launch_bounds__(kThreads) void bn_rows_kernel(BnArgs a) {
+  float max_abs_data = 0.f, max_abs_output = 0.f, unit_std = 0.f;
+  if (OWN_TABLE) {
+    max_abs_data = maxabs(*a.min_data, *a.max_data);
+    max_abs_output = maxabs(a.min_calib, a.max_calib);
+    unit_std = sqrtf(1.0f + static_cast<float>(a.eps));
+    if (blockIdx.x == 0 && threadIdx.x == 0) {
+      *a.omin = a.min_calib;
+      *a.omax = a.max_calib;
+    }
+  }
   const uint32_t inner16 = a.inner >> 4;
   const uint32_t chunks = (inner16 + 255u) >> 8;
   const uint32_t rows = static_cast<uint32_t>(a.n / a.inner);
@@ -1022,7 +1041,13 @@ __global__ __launch_bounds__(kThreads) void bn_rows_kernel(BnArgs a) {
   for (uint32_t item = wave; item < items; item += nwaves) {
     const uint32_t row = item / chunks, k = item - row * chunks;
     const uint32_t c = row % a.channels;
-    const float w = a.table[c], b = a.table[a.channels + c];
+    float w, b;
+    if (OWN_TABLE) {
+      bn_channel(a, c, max_abs_data, max_abs_output, unit_std, w, b);
+    } else {
+      w = a.table[c];
+      b = a.table[a.channels + c];
+    }
     const uint32_t left = inner16 - (k << 8);
     const size_t base = size_t(row) * inner16 + (k << 8) + lane;
     u4 x[4] = {};
@@ -1333,6 +1358,20 @@ int mxq_quantized_batch_norm(void* stream, const void* data, int data_type, cons
   MXQ_CHECK(a.n == 0 || (data != nullptr && out != nullptr), "null data pointer");
   a.vec_ok = (inner % 16 == 0 && a.n < (size_t(1) << 32) && aligned16(data) && aligned16(out)) ? 1 : 0;
   hipStream_t s = static_cast<hipStream_t>(stream);
+  // large tensors of long rows: one launch, the waves fold their channel's parameters
+  // themselves (a piece of 4 KiB per wave pays for the double-precision 1/sqrt many times over)
+#ifndef BN_NO_OWN
+  if (a.vec_ok && inner >= 1024 && a.n >= (size_t(1) << 26)) {
+    const size_t waves = (a.n / a.inner) * ((a.inner / 16 + 255) / 256);
+    const int grid = static_cast<int>((waves + kThreads / 64 - 1) / (kThreads / 64));
+    if (data_type == MXQ_UINT8)
+      hipLaunchKernelGGL((bn_rows_kernel<true, true>), dim3(grid), dim3(kThreads), 0, s, a);
+    else
+      hipLaunchKernelGGL((bn_rows_kernel<false, true>), dim3(grid), dim3(kThreads), 0, s, a);
+    MXQ_LAUNCH_CHECK();
+    return 0;
+  }
+#endif
   hipLaunchKernelGGL(bn_table_kernel, dim3((a.channels + kThreads - 1) / kThreads < 64
                                                ? (a.channels + kThreads - 1) / kThreads
                                                : 64),
@@ -1347,9 +1386,9 @@ int mxq_quantized_batch_norm(void* stream, const void* data, int data_type, cons
     if (a.n >= (size_t(1) << 26))
       grid = static_cast<int>((waves + kThreads / 64 - 1) / (kThreads / 64));
     if (data_type == MXQ_UINT8)
-      hipLaunchKernelGGL((bn_rows_kernel<true>), dim3(grid), dim3(kThreads), 0, s, a);
+      hipLaunchKernelGGL((bn_rows_kernel<true, false>), dim3(grid), dim3(kThreads), 0, s, a);
     else
-      hipLaunchKernelGGL((bn_rows_kernel<false>), dim3(grid), dim3(kThreads), 0, s, a);
+      hipLaunchKernelGGL((bn_rows_kernel<false, false>), dim3(grid), dim3(kThreads), 0, s, a);
   } else {
     const int grid = 2 * grid_for(a.vec_ok ? (a.n + 15) / 16 : a.n);
     if (data_type == MXQ_UINT8)

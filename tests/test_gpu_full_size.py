@@ -205,6 +205,36 @@ def test_concat_chunk_kernel_edges(contrib, case):
     assert np.array_equal(out.cpu().numpy(), ref)
 
 
+@pytest.mark.parametrize("dtype,relu", [(np.int8, True), (np.uint8, False)])
+def test_batch_norm_64m_one_launch(contrib, dtype, relu):
+    """From 64 M elements with rows of at least 1 KiB the batch norm is one launch whose waves
+    fold their channel's parameters themselves: the oracle on the first and last image, and
+    every image against the two-launch form (per-channel table) that smaller calls take."""
+    N, C, H, W = 64, 256, 64, 64
+    g = torch.Generator(device="cuda").manual_seed(31)
+    lo, hi = (0, 256) if dtype == np.uint8 else (-128, 128)
+    x = torch.randint(lo, hi, (N, C, H, W), device="cuda", generator=g,
+                      dtype=torch.uint8 if dtype == np.uint8 else torch.int8)
+    rng = np.random.default_rng(32)
+    gamma = rng.uniform(0.5, 2.0, C).astype(np.float32)
+    beta = rng.normal(0, 0.5, C).astype(np.float32)
+    mean = rng.normal(0, 0.3, C).astype(np.float32)
+    var = rng.uniform(0.3, 2.0, C).astype(np.float32)
+    rd = (0.0, 3.1) if dtype == np.uint8 else (-2.7, 3.1)
+    par = [torch.from_numpy(v).cuda() for v in (gamma, beta, mean, var)]
+    kw = dict(eps=2e-5, axis=1, min_calib_range=-6.5, max_calib_range=7.25, relu=relu)
+    out, mn, mx = contrib.quantized_batch_norm(x, *par, f32(rd[0]), f32(rd[1]), **kw)
+    for n in (0, N - 1):
+        ref, rmn, rmx = oracle.quantized_batch_norm(x[n:n + 1].cpu().numpy(), gamma, beta, mean,
+                                                    var, rd[0], rd[1], -6.5, 7.25, eps=2e-5,
+                                                    axis=1, relu=relu)
+        assert np.array_equal(out[n:n + 1].cpu().numpy(), ref), f"image {n}"
+        assert (mn.item(), mx.item()) == (rmn, rmx)
+    for n0 in range(0, N, 16):
+        part, _, _ = contrib.quantized_batch_norm(x[n0:n0 + 16], *par, f32(rd[0]), f32(rd[1]), **kw)
+        assert torch.equal(out[n0:n0 + 16], part), f"images from {n0}"
+
+
 def test_elemwise_add_64m(contrib):
     g = torch.Generator(device="cuda").manual_seed(5)
     a = torch.randint(-127, 128, (N_CAST,), device="cuda", generator=g, dtype=torch.int8)
