@@ -207,9 +207,10 @@ def test_concat_chunk_kernel_edges(contrib, case):
 
 @pytest.mark.parametrize("dtype,relu", [(np.int8, True), (np.uint8, False)])
 def test_batch_norm_64m_one_launch(contrib, dtype, relu):
-    """From 64 M elements with rows of at least 1 KiB the batch norm is one launch whose waves
-    fold their channel's parameters themselves: the oracle on the first and last image, and
-    every image against the two-launch form (per-channel table) that smaller calls take."""
+    """With rows of 2 KiB and more the batch norm is one launch whose waves fold their channel's
+    parameters themselves, from 64 M elements on a grid of one piece per wave: the oracle on
+    the first and last image, and every block of 16 images against a call of its own (the
+    capped grid whose waves stride over the pieces)."""
     N, C, H, W = 64, 256, 64, 64
     g = torch.Generator(device="cuda").manual_seed(31)
     lo, hi = (0, 256) if dtype == np.uint8 else (-128, 128)
