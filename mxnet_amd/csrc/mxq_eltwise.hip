@@ -1010,22 +1010,22 @@ __global__ __launch_bounds__(kThreads) void bn_kernel(BnArgs a) {
   }
 }
 
-// Rows of at least 1 KiB (inner % 16 == 0): one wave per 4 KiB piece of a row, so the channel,
-// its factor and offset are wave-uniform (scalar loads, no per-lane division) and a lane keeps
+constexpr int64_t kBnRowsMin = 2048;
+
+// Rows of at least kBnRowsMin bytes (inner % 16 == 0): one wave per 4 KiB piece of a row, so
+// the channel, its factor and offset are wave-uniform (no per-lane division) and a lane keeps
 // four 16-byte loads in flight.
-// OWN_TABLE: no table kernel ran; every wave folds its channel's four parameters itself (the
-// same function, so the same factor and offset) and the first thread passes the range on.
-template <bool IN_U, bool OWN_TABLE>
+// No table kernel runs in front of this one: every wave folds its channel's four parameters
+// itself (the function the table kernel calls, so the same factor and offset; one
+// double-precision 1/sqrt per piece of up to 4 KiB) and the first thread passes the range on.
+template <bool IN_U>
 __global__ __launch_bounds__(kThreads) void bn_rows_kernel(BnArgs a) {
-  float max_abs_data = 0.f, max_abs_output = 0.f, unit_std = 0.f;
-  if (OWN_TABLE) {
-    max_abs_data = maxabs(*a.min_data, *a.max_data);
-    max_abs_output = maxabs(a.min_calib, a.max_calib);
-    unit_std = sqrtf(1.0f + static_cast<float>(a.eps));
-    if (blockIdx.x == 0 && threadIdx.x == 0) {
-      *a.omin = a.min_calib;
-      *a.omax = a.max_calib;
-    }
+  const float max_abs_data = maxabs(*a.min_data, *a.max_data);
+  const float max_abs_output = maxabs(a.min_calib, a.max_calib);
+  const float unit_std = sqrtf(1.0f + static_cast<float>(a.eps));
+  if (blockIdx.x == 0 && threadIdx.x == 0) {
+    *a.omin = a.min_calib;
+    *a.omax = a.max_calib;
   }
   const uint32_t inner16 = a.inner >> 4;
   const uint32_t chunks = (inner16 + 255u) >> 8;
@@ -1042,12 +1042,7 @@ __global__ __launch_bounds__(kThreads) void bn_rows_kernel(BnArgs a) {
     const uint32_t row = item / chunks, k = item - row * chunks;
     const uint32_t c = row % a.channels;
     float w, b;
-    if (OWN_TABLE) {
-      bn_channel(a, c, max_abs_data, max_abs_output, unit_std, w, b);
-    } else {
-      w = a.table[c];
-      b = a.table[a.channels + c];
-    }
+    bn_channel(a, c, max_abs_data, max_abs_output, unit_std, w, b);
     const uint32_t left = inner16 - (k << 8);
     const size_t base = size_t(row) * inner16 + (k << 8) + lane;
     u4 x[4] = {};
@@ -1358,20 +1353,20 @@ int mxq_quantized_batch_norm(void* stream, const void* data, int data_type, cons
   MXQ_CHECK(a.n == 0 || (data != nullptr && out != nullptr), "null data pointer");
   a.vec_ok = (inner % 16 == 0 && a.n < (size_t(1) << 32) && aligned16(data) && aligned16(out)) ? 1 : 0;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  // rows of 2 KiB and more: ONE launch, the waves fold their channel's parameters themselves
-  // (a double-precision 1/sqrt per piece of up to 4 KiB; with 1 KiB rows it costs more than
-  // the table kernel's launch: 64 x 512 x 1024 takes 30.4 us that way against 28.4 us).
-  // Twice the work-groups per CU of the narrowing kernels, as for concat (measured fastest);
-  // from 64 M elements one piece per wave and no loop.
-  if (a.n != 0 && a.vec_ok && inner >= 2048) {
+  // Rows of kBnRowsMin bytes and more: ONE launch, a wave per piece of a row of up to 4 KiB,
+  // the waves fold their channel's parameters themselves.  Twice the work-groups per CU of
+  // the narrowing kernels, as for concat (measured fastest); from 64 M elements one piece per
+  // wave and no loop.  Shorter rows fill too little of a wave's four 1 KiB pieces (64 x 512
+  // x 1024: 28.6 us that way, 18.4 us with 16 bytes per lane and the channel by division).
+  if (a.n != 0 && a.vec_ok && inner >= kBnRowsMin) {
     const size_t waves = (a.n / a.inner) * ((a.inner / 16 + 255) / 256);
     int grid = 2 * grid_for(waves * 64);
     if (a.n >= (size_t(1) << 26))
       grid = static_cast<int>((waves + kThreads / 64 - 1) / (kThreads / 64));
     if (data_type == MXQ_UINT8)
-      hipLaunchKernelGGL((bn_rows_kernel<true, true>), dim3(grid), dim3(kThreads), 0, s, a);
+      hipLaunchKernelGGL((bn_rows_kernel<true>), dim3(grid), dim3(kThreads), 0, s, a);
     else
-      hipLaunchKernelGGL((bn_rows_kernel<false, true>), dim3(grid), dim3(kThreads), 0, s, a);
+      hipLaunchKernelGGL((bn_rows_kernel<false>), dim3(grid), dim3(kThreads), 0, s, a);
     MXQ_LAUNCH_CHECK();
     return 0;
   }
@@ -1381,18 +1376,7 @@ int mxq_quantized_batch_norm(void* stream, const void* data, int data_type, cons
                      dim3(kThreads), 0, s, a);
   MXQ_LAUNCH_CHECK();
   if (a.n == 0) return 0;
-  if (a.vec_ok && inner >= 1024) {
-    const size_t waves = (a.n / a.inner) * ((a.inner / 16 + 255) / 256);
-    // twice the work-groups per CU of the narrowing kernels, as for concat: measured fastest
-    // from 64 M elements one 4 KiB piece per wave and no loop (24.4 -> 23.9 us there)
-    int grid = 2 * grid_for(waves * 64);
-    if (a.n >= (size_t(1) << 26))
-      grid = static_cast<int>((waves + kThreads / 64 - 1) / (kThreads / 64));
-    if (data_type == MXQ_UINT8)
-      hipLaunchKernelGGL((bn_rows_kernel<true, false>), dim3(grid), dim3(kThreads), 0, s, a);
-    else
-      hipLaunchKernelGGL((bn_rows_kernel<false, false>), dim3(grid), dim3(kThreads), 0, s, a);
-  } else {
+  {
     const int grid = 2 * grid_for(a.vec_ok ? (a.n + 15) / 16 : a.n);
     if (data_type == MXQ_UINT8)
       hipLaunchKernelGGL((bn_kernel<true>), dim3(grid), dim3(kThreads), 0, s, a);
