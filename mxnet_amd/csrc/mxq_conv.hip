@@ -16,6 +16,7 @@
 
 #include "../../include/mxq.h"
 #include "mxq_common.h"
+#include "mxq_thin_transpose.h"
 #include "mxq_gemm.h"
 #include "mxq_tiles.h"
 
@@ -631,6 +632,18 @@ __global__ __launch_bounds__(256) void transpose_i8_wide_kernel(const uint8_t* _
   }
 }
 
+// A thin extent (at most 64 bytes, e.g. 7 x 7 planes) beside a long one that is a multiple of
+// 128: see thin_transpose_tile.  One matrix per blockIdx.y.
+template <bool THIN_IN>
+__global__ __launch_bounds__(256) void transpose_i8_thin_kernel(const uint8_t* __restrict__ in,
+                                                                uint8_t* __restrict__ out,
+                                                                int L, int T) {
+  __shared__ __attribute__((aligned(16))) uint8_t flat[128 * 64];
+  const size_t plane = static_cast<size_t>(L) * T;
+  thin_transpose_tile<THIN_IN>(in + blockIdx.y * plane, out + blockIdx.y * plane, L, T,
+                               blockIdx.x * 128, flat);
+}
+
 // Space-to-depth by 2 while going from planes to pixels: out[b][h2][w2][(dh*2+dw)*C + c] =
 // in[b][c][2*h2 - off_h + dh][2*w2 - off_w + dw] (zero outside the plane), the channel run
 // of every output pixel zero-padded to CP bytes.  A stride-2 convolution over few channels
@@ -694,6 +707,23 @@ void launch_transpose(hipStream_t s, const void* in, void* out, int B, int R, in
                        static_cast<const uint8_t*>(in), static_cast<uint8_t*>(out), R, S, RP);
     MXQ_LAUNCH_CHECK();
     return;
+  }
+  if (sizeof(T) == 1 && RP == R && aligned16(in) && aligned16(out)) {
+    // a thin extent (<= 64) beside a long one that is a multiple of 128
+    const bool thin_in = S <= 64 && R % 128 == 0;
+    const bool thin_out = R <= 64 && S % 128 == 0;
+    if (thin_in || thin_out) {
+      const int L = thin_in ? R : S, thin = thin_in ? S : R;
+      dim3 grid(L / 128, B);
+      if (thin_in)
+        hipLaunchKernelGGL(transpose_i8_thin_kernel<true>, grid, dim3(256), 0, s,
+                           static_cast<const uint8_t*>(in), static_cast<uint8_t*>(out), L, thin);
+      else
+        hipLaunchKernelGGL(transpose_i8_thin_kernel<false>, grid, dim3(256), 0, s,
+                           static_cast<const uint8_t*>(in), static_cast<uint8_t*>(out), L, thin);
+      MXQ_LAUNCH_CHECK();
+      return;
+    }
   }
   dim3 grid((S + 63) / 64, (RP + 63) / 64, B);
   hipLaunchKernelGGL((transpose_kernel<T>), grid, dim3(256), 0, s, static_cast<const T*>(in),

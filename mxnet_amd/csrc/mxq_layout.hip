@@ -15,6 +15,7 @@
 
 #include "../../include/mxq.h"
 #include "mxq_common.h"
+#include "mxq_thin_transpose.h"
 
 namespace mxq {
 
@@ -385,6 +386,22 @@ __global__ __launch_bounds__(kThreads) void permute_tile16_kernel(TileArgs a) {
   pass_range(a.imin, a.imax, a.omin, a.omax);
 }
 
+// The innermost axis moves and one of the two extents is thin (at most 64 bytes, e.g. planes
+// of 7 x 7) while the other is a multiple of 128, both matrices dense ([B][A] in, [A][B] out):
+// see thin_transpose_tile.  Batches along blockIdx.y.
+template <bool THIN_IN>
+__global__ __launch_bounds__(kThreads) void permute_thin_kernel(TileArgs a) {
+  __shared__ __attribute__((aligned(16))) uint8_t flat[128 * 64];
+  const int L = static_cast<int>(THIN_IN ? a.B : a.A), T = static_cast<int>(THIN_IN ? a.A : a.B);
+  for (int64_t z = blockIdx.y; z < a.batches; z += gridDim.y) {
+    size_t in_off, out_off;
+    batch_offsets(a, z, in_off, out_off);
+    thin_transpose_tile<THIN_IN>(a.in + in_off, a.out + out_off, L, T, blockIdx.x * 128, flat);
+    __syncthreads();
+  }
+  pass_range(a.imin, a.imax, a.omin, a.omax);
+}
+
 // The innermost run of E bytes (16 | E, E <= 256) stays whole but the two axes around it
 // swap neighbours (attention's (batch, seq, heads, E) <-> (batch, heads, seq, E)): rows of
 // such short runs copied one by one touch half cache lines on one side.  Here T x T runs
@@ -750,6 +767,25 @@ int mxq_quantized_transpose(void* stream, const void* in, const float* imin, con
                   (a.a_out_stride % 16 == 0) && aligned16(in) && aligned16(out);
   for (int d = 0; d < a.p.nd; ++d)
     friendly = friendly && (a.p.in_stride[d] % 4 == 0) && (a.p_out_stride[d] % 16 == 0);
+  {
+    // a thin extent beside a long one, dense matrices, every batch on a 16-byte mark
+    bool marks = aligned16(in) && aligned16(out) && a.b_in_stride == a.A && a.a_out_stride == a.B;
+    for (int d = 0; d < a.p.nd; ++d)
+      marks = marks && (a.p.in_stride[d] % 16 == 0) && (a.p_out_stride[d] % 16 == 0);
+    const bool thin_in = a.A <= 64 && a.B % 128 == 0;   // input [B][A], A thin
+    const bool thin_out = a.B <= 64 && a.A % 128 == 0;  // input [B][A], B thin
+    const int64_t longer = thin_in ? a.B : a.A;
+    if (!friendly && marks && (thin_in || thin_out) && longer / 128 < (int64_t(1) << 31)) {
+      const int64_t gy = a.batches < 65535 ? a.batches : 65535;
+      const dim3 grid(static_cast<unsigned>(longer / 128), static_cast<unsigned>(gy));
+      if (thin_in)
+        hipLaunchKernelGGL(permute_thin_kernel<true>, grid, dim3(kThreads), 0, s, a);
+      else
+        hipLaunchKernelGGL(permute_thin_kernel<false>, grid, dim3(kThreads), 0, s, a);
+      MXQ_LAUNCH_CHECK();
+      return 0;
+    }
+  }
   {
     // 16-byte loads with dword stores: output rows and strides that are multiples of 4 only
     bool in16 = (a.A % 16 == 0) && (a.b_in_stride % 16 == 0) && aligned16(in);

@@ -181,7 +181,9 @@ def test_layout_adapters(capi):
     # (ragged last tiles in both directions)
     for shape in ((2, 8, 8, 64), (3, 4, 12, 20), (1, 16, 16, 132), (2, 16, 8, 144),
                   (2, 13, 12, 272), (1, 56, 56, 256), (3, 14, 14, 256), (2, 10, 15, 144),
-                  (2, 14, 14, 1040)):   # the last three: planes of 4 | H*W bytes, dword stores
+                  (2, 14, 14, 1040),    # the last three: planes of 4 | H*W bytes, dword stores
+                  (3, 7, 7, 256), (2, 5, 5, 128), (2, 3, 3, 384), (2, 1, 1, 128),
+                  (2, 7, 9, 128)):      # thin planes (at most 64 bytes) beside 128 | C
         v8 = int8_uniform(shape, seed=4)
         z8 = capi.nhwc_to_nchw(dev(v8))
         np.testing.assert_array_equal(z8.cpu().numpy(), v8.transpose(0, 3, 1, 2))
@@ -198,7 +200,8 @@ def test_layout_adapters(capi):
                       ((2, 16, 4, 4), 16), ((2, 3, 8, 8), 16), ((2, 64, 12, 12), 64),
                       ((3, 70, 4, 8), 80), ((2, 130, 16, 4), 144), ((1, 40, 4, 4), 48),
                       ((2, 20, 10, 30), 32), ((2, 256, 12, 12), 256), ((1, 200, 20, 12), 208),
-                      ((2, 128, 56, 56), 128)):
+                      ((2, 128, 56, 56), 128), ((3, 256, 7, 7), 256), ((2, 128, 5, 5), 128),
+                      ((2, 384, 3, 3), 384), ((2, 128, 1, 1), 128), ((2, 128, 7, 9), 128)):
         x = int8_uniform(shape, seed=3)
         n, c, h, w = shape
         out = torch.full((n, h, w, cp), 77, dtype=torch.int8, device="cuda")

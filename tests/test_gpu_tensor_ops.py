@@ -254,6 +254,11 @@ def test_transpose_every_permutation(contrib, shape, axes):
     ((3, 5, 256, 144), (1, 0, 3, 2)),       # 16-byte loads under two permuted outer axes
     ((3, 14, 14, 256), (0, 3, 1, 2)),       # planes of 196 bytes: 16-byte loads, dword stores
     ((2, 132, 144), (0, 2, 1)),             # the same with a 4-byte last tile
+    ((3, 7, 7, 256), (0, 3, 1, 2)),         # planes of 49 bytes out: the thin-extent kernel
+    ((3, 256, 7, 7), (0, 2, 3, 1)),         # and in
+    ((2, 3, 128, 5), (1, 0, 3, 2)),         # the same under two permuted outer axes
+    ((2, 25, 384), (0, 2, 1)),
+    ((128, 1), (1, 0)),
     ((2, 3, 130, 260), (1, 0, 3, 2)),
     ((0, 5, 3), (2, 0, 1)),                 # empty
     ((7,), (0,)),
