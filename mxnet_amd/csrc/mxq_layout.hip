@@ -775,7 +775,7 @@ int mxq_quantized_transpose(void* stream, const void* in, const float* imin, con
     const bool thin_in = a.A <= 64 && a.B % 128 == 0;   // input [B][A], A thin
     const bool thin_out = a.B <= 64 && a.A % 128 == 0;  // input [B][A], B thin
     const int64_t longer = thin_in ? a.B : a.A;
-    if (!friendly && marks && (thin_in || thin_out) && longer / 128 < (int64_t(1) << 31)) {
+    if (!friendly && marks && (thin_in || thin_out) && longer < (int64_t(1) << 31)) {
       const int64_t gy = a.batches < 65535 ? a.batches : 65535;
       const dim3 grid(static_cast<unsigned>(longer / 128), static_cast<unsigned>(gy));
       if (thin_in)
