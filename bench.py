@@ -54,6 +54,7 @@ MEASURED_TRAFFIC_BYTES = {
     "batch_norm": ((2.0 * 32838.0 + 65536.1) * _KIB, "profiles/bn_rows_kernel_nchw_64M.md"),
     "embedding": ((2.0 * 31709.6 + 65535.8) * _KIB, "profiles/embedding_kernel_bert_vocab.md"),
     "transpose": ((2.0 * 32800.1 + 65548.3) * _KIB, "profiles/permute_elem_direct_kernel_attention_64M.md"),
+    "quantized_act": ((2.0 * 32791.8 + 65575.3) * _KIB, "profiles/relu_chunk_kernel_64M.md"),
     "transpose_to_nhwc": ((2.0 * 32797.6 + 65541.4) * _KIB, "profiles/permute_tile16_kernel_to_nhwc_64M.md"),
     "transpose_to_nchw": ((2.0 * 32797.6 + 65538.6) * _KIB, "profiles/permute_tile16_kernel_to_nchw_64M.md"),
     "maxpool": ((2.0 * 100388.0 + 50177.2) * _KIB, "profiles/pool_lds_kernel_maxpool.md"),
