@@ -187,7 +187,7 @@ CONCAT_EDGE_CASES = [
 
 @pytest.mark.parametrize("case", range(len(CONCAT_EDGE_CASES)))
 def test_concat_chunk_kernel_edges(contrib, case):
-    """From 64 MiB per launch, with every input 16-byte aligned, concat runs one chunk of 1024
+    """From 16 MiB per launch, with every input 16-byte aligned, concat runs one chunk of 1024
     16-byte pieces per work-group: partial last chunks, several rows with a pitch, an empty
     input between two others, uint8, and equal ranges (the byte copy)."""
     shapes, axis, dtype, ranges = CONCAT_EDGE_CASES[case]
