@@ -75,7 +75,7 @@ def parse_args():
                              "requantize", "requantize_uncal", "dequantize", "copy", "maxpool", "avgpool",
                              "elemwise_add", "elemwise_add_int8", "concat", "elemwise_mul_int8", "quantize_asym",
                              "batch_norm", "embedding", "transpose", "transpose_to_nhwc", "transpose_to_nchw",
-                             "resnet50_convs", "resnet50_chain",
+                             "resnet50_convs", "resnet50_convs_operator", "resnet50_chain",
                              "resnet50_chain_fused", "resnet50_chain_unfused",
                              "bert_fc_chain",
                              "bert_fc_chain_fused",
@@ -766,6 +766,65 @@ class ConvStackWorkload(GraphWorkload):
         return rows
 
 
+class ConvOperatorWorkload(GraphWorkload):
+    """The same 19 ResNet-50 layers at batch 64 under the reference operator's own contract
+    (quantized_conv.cu:101-219): NCHW int8 data and OIHW int8 weights in, NCHW int32 out.  Per
+    layer: both operands brought to NHWC (the two TransposeImpl calls of the reference), then
+    the convolution whose epilogue writes int32 channel planes (no third transpose)."""
+
+    def __init__(self, torch, capi, lib):
+        self.kernel = "transpose_i8 kernels + conv / fc kernels (int32 NCHW out)"
+        self.bound = "mfma"
+        self.name = "ResNet-50 v1 bottleneck conv stack (19 distinct layers), batch 64, as the " \
+                    "operator sees it: NCHW int8 in, layout adapters, NCHW int32 out"
+        P = lambda t: ctypes.c_void_p(t.data_ptr())
+        g = torch.Generator(device="cuda").manual_seed(4)
+        N = 64
+        self.layers, self.ops = [], 0.0
+        one = [torch.tensor([v], device="cuda") for v in (-1.0, 1.0)]
+        for (H, C, O, k, s) in RESNET50_CONVS:
+            pad = 1 if k == 3 else 0
+            OH = (H + 2 * pad - k) // s + 1
+            d = torch.randint(-127, 128, (N, C, H, H), device="cuda", generator=g, dtype=torch.int8)
+            w = torch.randint(-127, 128, (O, C, k, k), device="cuda", generator=g, dtype=torch.int8)
+            b = torch.randint(-127, 128, (O,), device="cuda", generator=g, dtype=torch.int8)
+            dn = torch.empty((N, H, H, C), dtype=torch.int8, device="cuda")
+            wn = torch.empty((O, k, k, C), dtype=torch.int8, device="cuda")
+            out = torch.empty((N, O, OH, OH), dtype=torch.int32, device="cuda")
+            sc = [torch.empty(1, device="cuda") for _ in range(2)]
+            nws = lib.mxq_quantized_conv_workspace(N, H, H, C, O, k, k, s, s, pad, pad, 1, 1, 0)
+            ws = torch.empty(nws, dtype=torch.uint8, device="cuda") if nws else None
+            self.layers.append((d, w, b, dn, wn, out, sc, (N, H, H, C, O, k, k, s, s, pad, pad), ws))
+            self.ops += 2.0 * N * OH * OH * O * k * k * C
+
+        def body(only=None):
+            st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+            for i, (d, w, b, dn, wn, out, sc, geo, ws) in enumerate(self.layers):
+                if only is not None and i != only:
+                    continue
+                N_, H_, W_, C_, O_, k_ = geo[0], geo[1], geo[2], geo[3], geo[4], geo[5]
+                rc = lib.mxq_nchw_to_nhwc_pad_i8(st, P(d), P(dn), N_, C_, H_, W_, C_)
+                rc = rc or lib.mxq_nchw_to_nhwc_pad_i8(st, P(w), P(wn), O_, C_, k_, k_, C_)
+                rc = rc or lib.mxq_quantized_conv_nhwc_out_nchw(
+                    st, P(dn), P(wn), P(b), *geo, 1, 1, P(one[0]), P(one[1]), P(one[0]),
+                    P(one[1]), P(one[0]), P(one[1]), P(out), P(sc[0]), P(sc[1]), *ws_args(ws))
+                if rc != 0:
+                    raise RuntimeError(lib.mxq_last_error().decode())
+        self.body = body
+        self.capture(torch, body)
+
+    def per_layer(self, torch):
+        rows = []
+        for i, (H, C, O, k, s) in enumerate(RESNET50_CONVS):
+            pad = 1 if k == 3 else 0
+            OH = (H + 2 * pad - k) // s + 1
+            ops = 2.0 * 64 * OH * OH * O * k * k * C
+            t = self.time_alone(torch, lambda: self.body(i))
+            rows.append({"layer": "%dx%d %d->%d k%d s%d" % (H, H, C, O, k, s),
+                         "us": round(t * 1e6, 2), "TOPS": round(ops / t / 1e12, 1)})
+        return rows
+
+
 BERT_FCS = [(768, 2304), (768, 768), (768, 3072), (3072, 768)]
 
 
@@ -1102,6 +1161,8 @@ def mfma_context(torch, S):
 def make_workload(name, torch, capi, lib):
     if name == "resnet50_convs":
         return ConvStackWorkload(torch, capi, lib)
+    if name == "resnet50_convs_operator":
+        return ConvOperatorWorkload(torch, capi, lib)
     if name == "resnet50_chain":
         return ResNetChainWorkload(torch, capi, lib)
     if name == "resnet50_chain_fused":
@@ -1235,7 +1296,8 @@ def main():
                      "concat", "elemwise_mul_int8", "quantize_asym", "batch_norm", "embedding",
                      "transpose", "transpose_to_nhwc", "transpose_to_nchw", "maxpool", "avgpool",
                      "fc8192",
-                     "resnet50_convs", "resnet50_chain_unfused", "resnet50_chain", "resnet50_chain_fused",
+                     "resnet50_convs", "resnet50_convs_operator", "resnet50_chain_unfused",
+                     "resnet50_chain", "resnet50_chain_fused",
                      "bert_fc_chain",
                      "bert_fc_chain_fused", "bert_fc_chain_f32"]:
             if kind == args.workload:

@@ -632,6 +632,14 @@ __global__ __launch_bounds__(256) void transpose_i8_wide_kernel(const uint8_t* _
   }
 }
 
+__global__ __launch_bounds__(256) void copy16_kernel(const uint8_t* __restrict__ in,
+                                                     uint8_t* __restrict__ out, size_t pieces) {
+  typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+  const size_t stride = static_cast<size_t>(gridDim.x) * 256;
+  for (size_t q = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x; q < pieces; q += stride)
+    reinterpret_cast<u4*>(out)[q] = reinterpret_cast<const u4*>(in)[q];
+}
+
 // A thin extent (at most 64 bytes, e.g. 7 x 7 planes) beside a long one that is a multiple of
 // 128: see thin_transpose_tile.  One matrix per blockIdx.y.
 template <bool THIN_IN>
@@ -712,6 +720,17 @@ void launch_transpose(hipStream_t s, const void* in, void* out, int B, int R, in
     // a thin extent (<= 64) beside a long one that is a multiple of 128
     const bool thin_in = S <= 64 && R % 128 == 0;
     const bool thin_out = R <= 64 && S % 128 == 0;
+    if ((thin_in && S == 1) || (thin_out && R == 1)) {
+      // a thin extent of 1 (the weights of a 1 x 1 convolution): the transpose is a copy
+      const size_t pieces = static_cast<size_t>(B) * R * S / 16;  // 128 | R * S
+      const size_t want = (pieces + 255) / 256;
+      const size_t cap = static_cast<size_t>(num_cus()) * 8;
+      hipLaunchKernelGGL(copy16_kernel, dim3(static_cast<unsigned>(want < cap ? want : cap)),
+                         dim3(256), 0, s, static_cast<const uint8_t*>(in),
+                         static_cast<uint8_t*>(out), pieces);
+      MXQ_LAUNCH_CHECK();
+      return;
+    }
     if (thin_in || thin_out) {
       const int L = thin_in ? R : S, thin = thin_in ? S : R;
       dim3 grid(L / 128, B);

@@ -962,35 +962,41 @@ __device__ __forceinline__ void gemm_epilogue_lds(v16i (&acc)[Cfg::MI][Cfg::NI],
               t32[(8 * vq + 4 * lgrp + i) * Scratch::kPitch32 + lrow] = acc[mi][ni][4 * vq + i];
           asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
           __builtin_amdgcn_wave_barrier();
-          const int c = lane >> 3, p4 = (lane & 7) * 4;
-          v4i col[4];
+          if ((e.plane & 3) == 0) {
+            // 4 | plane: 4 | pix and a lane's four pixels lie in one image
+            const int c = lane >> 3, p4 = (lane & 7) * 4;
+            v4i col[4];
 #pragma unroll
-          for (int it = 0; it < 4; ++it)
-            col[it] = *reinterpret_cast<const v4i*>(t32 + (it * 8 + c) * Scratch::kPitch32 + p4);
-          asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-          __builtin_amdgcn_wave_barrier();
-          const int m0 = m_base + mi * 32 + p4;
-          const int img = m0 / e.plane, pix = m0 - img * e.plane;
-          const bool quad = (e.plane & 3) == 0;  // then 4 | pix and the quad is in one image
+            for (int it = 0; it < 4; ++it)
+              col[it] = *reinterpret_cast<const v4i*>(t32 + (it * 8 + c) * Scratch::kPitch32 + p4);
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            __builtin_amdgcn_wave_barrier();
+            const int m0 = m_base + mi * 32 + p4;
+            const int img = m0 / e.plane, pix = m0 - img * e.plane;
 #pragma unroll
-          for (int it = 0; it < 4; ++it) {
-            const int n = n_base + ni * 32 + it * 8 + c;
-            if (n >= N) continue;
-            if (quad) {
-              if (m0 < M)
+            for (int it = 0; it < 4; ++it) {
+              const int n = n_base + ni * 32 + it * 8 + c;
+              if (n < N && m0 < M)
                 *reinterpret_cast<v4i*>(e.out32 + (static_cast<size_t>(img) * N + n) * e.plane +
                                         pix) = col[it];
-            } else {
-              int im = img, px = pix;
+            }
+          } else {
+            // any other plane (7 x 7): a lane takes one pixel of the tile's 32, a store
+            // instruction two channels, so that it still writes runs of up to 128 bytes
+            // (broken only where the tile passes from one image to the next)
+            const int p = lane & 31, c2 = lane >> 5;
+            int col[16];
 #pragma unroll
-              for (int j = 0; j < 4; ++j) {
-                if (m0 + j < M)
-                  e.out32[(static_cast<size_t>(im) * N + n) * e.plane + px] = col[it][j];
-                if (++px == e.plane) {
-                  px = 0;
-                  ++im;
-                }
-              }
+            for (int it = 0; it < 16; ++it) col[it] = t32[(it * 2 + c2) * Scratch::kPitch32 + p];
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            __builtin_amdgcn_wave_barrier();
+            const int m = m_base + mi * 32 + p;
+            const int img = m / e.plane, pix = m - img * e.plane;
+#pragma unroll
+            for (int it = 0; it < 16; ++it) {
+              const int n = n_base + ni * 32 + it * 2 + c2;
+              if (n < N && m < M)
+                e.out32[(static_cast<size_t>(img) * N + n) * e.plane + pix] = col[it];
             }
           }
         }
