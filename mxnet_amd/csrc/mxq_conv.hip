@@ -575,15 +575,30 @@ __global__ __launch_bounds__(256) void transpose_i8_kernel(const uint8_t* __rest
 // The same on 128 rows x 128 columns with 16-byte loads (S % 16 == 0, S and RP >= 128,
 // 16-byte aligned input as well): a thread takes 16 bytes along S of four consecutive rows, four load
 // instructions instead of sixteen, and the output runs are whole 128-byte lines.
+struct WideOrder {
+  unsigned tiles_s, tiles_r, total, per_xcd;
+};
+
 template <int PIECE>
 __global__ __launch_bounds__(256) void transpose_i8_wide_kernel(const uint8_t* __restrict__ in,
                                                                 uint8_t* __restrict__ out,
-                                                                int R, int S, int RP) {
+                                                                int R, int S, int RP,
+                                                                WideOrder o) {
   typedef uint32_t u4 __attribute__((ext_vector_type(4)));
   constexpr int kPitch = 33;  // dwords per transposed row: 128 bytes + 4 of padding
   __shared__ uint32_t tile[128 * kPitch];
-  const size_t b = blockIdx.z;
-  const int r0 = blockIdx.y * 128, s0 = blockIdx.x * 128;
+  // the tile sequence runs along S first, then R, then the batch; with o.per_xcd != 0 the
+  // round-robin of work-group ids over the 8 XCDs is undone, so that every XCD owns a
+  // contiguous range of it and tiles that share input cache lines meet in one L2
+  unsigned item = blockIdx.x;
+  if (o.per_xcd != 0) {
+    item = (blockIdx.x & 7u) * o.per_xcd + (blockIdx.x >> 3);
+    if (item >= o.total) return;
+  }
+  const unsigned rest = item / o.tiles_s, ts = item - rest * o.tiles_s;
+  const unsigned bq = rest / o.tiles_r, tr = rest - bq * o.tiles_r;
+  const size_t b = bq;
+  const int r0 = tr * 128, s0 = ts * 128;
   const int t = threadIdx.x;
   const uint8_t* src = in + b * static_cast<size_t>(R) * S;
   uint8_t* dst = out + b * static_cast<size_t>(RP) * S;
@@ -680,15 +695,23 @@ __global__ __launch_bounds__(256) void s2d_nhwc_kernel(const int8_t* __restrict_
   }
 }
 
-// (Undoing the round-robin of work-group ids over the XCDs, so that every XCD owns a
-// contiguous range of tiles and neighbours that share cache lines meet in one L2, helps
-// planes whose rows do not start on 128-byte marks by 5-15 % and costs aligned ones 10 %:
-// not kept.)
+// Input rows that do not start on 128-byte marks (56 x 56 and 28 x 28 planes on the way to
+// pixels) share cache lines between neighbouring tiles along S: there the round-robin of
+// work-group ids over the XCDs is undone (64 x 256 x 56 x 56: 22.6 -> 21.1 us, 64 x 512 x 28 x 28:
+// 14.3 -> 12.1 us).  Rows on the marks lose 10 % that way (64 x 64 planes: 25.6 -> 28.9 us) and
+// the way back to planes gains nothing reliably, so those keep the plain order.
 template <int PIECE>
 void launch_wide(hipStream_t s, const void* in, void* out, int B, int R, int S, int RP) {
-  dim3 wide((S + 127) / 128, (RP + 127) / 128, B);
-  hipLaunchKernelGGL(transpose_i8_wide_kernel<PIECE>, wide, dim3(256), 0, s,
-                     static_cast<const uint8_t*>(in), static_cast<uint8_t*>(out), R, S, RP);
+  WideOrder o;
+  o.tiles_s = static_cast<unsigned>((S + 127) / 128);
+  o.tiles_r = static_cast<unsigned>((RP + 127) / 128);
+  const unsigned long long total = 1ull * o.tiles_s * o.tiles_r * static_cast<unsigned>(B);
+  MXQ_CHECK(total < (1ull << 31) - 8, "transpose grid too large");
+  o.total = static_cast<unsigned>(total);
+  o.per_xcd = (S % 128 != 0) ? (o.total + 7u) / 8u : 0u;
+  const unsigned grid = o.per_xcd != 0 ? o.per_xcd * 8u : o.total;
+  hipLaunchKernelGGL(transpose_i8_wide_kernel<PIECE>, dim3(grid), dim3(256), 0, s,
+                     static_cast<const uint8_t*>(in), static_cast<uint8_t*>(out), R, S, RP, o);
   MXQ_LAUNCH_CHECK();
 }
 
