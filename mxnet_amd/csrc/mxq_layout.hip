@@ -178,6 +178,9 @@ struct TileArgs {
   int64_t a_out_stride, b_in_stride;
   int64_t batches;    // product of p.out_extent
   unsigned tiles_a;   // tiles along A
+  // permute_tile16_kernel only: when per_xcd != 0 the grid is one-dimensional, tiles and
+  // batches in one sequence (A fastest) of which every XCD owns a contiguous range
+  unsigned tiles_ab = 0, xcd_total = 0, per_xcd = 0;
 };
 
 // The innermost axis moves: 64 (B) x 64 (A) bytes per tile through LDS.  Reads run along A,
@@ -329,10 +332,21 @@ __global__ __launch_bounds__(kThreads) void permute_tile16_kernel(TileArgs a) {
   constexpr int kPitch = 33;  // dwords per transposed row: 128 bytes + 4 of padding
   __shared__ uint32_t tile[128 * kPitch];
   const int t = threadIdx.x;
-  const int64_t tb = blockIdx.x / a.tiles_a, ta = blockIdx.x - tb * a.tiles_a;
+  unsigned tile_id = blockIdx.x;
+  int64_t z0 = blockIdx.y, z_step = gridDim.y;
+  if (a.per_xcd != 0) {
+    // work-group ids go round the 8 XCDs: undone, so that tiles which share input cache
+    // lines (rows of A that miss the 128-byte marks) meet in one L2
+    const unsigned item = (blockIdx.x & 7u) * a.per_xcd + (blockIdx.x >> 3);
+    if (item >= a.xcd_total) return;  // (work-group 0 is item 0: the range is still passed on)
+    z0 = item / a.tiles_ab;
+    tile_id = item - static_cast<unsigned>(z0) * a.tiles_ab;
+    z_step = a.batches;
+  }
+  const int64_t tb = tile_id / a.tiles_a, ta = tile_id - tb * a.tiles_a;
   const int64_t a0 = ta * 128, b0 = tb * 128;
   const int sq = t & 7, rq = t >> 3;
-  for (int64_t z = blockIdx.y; z < a.batches; z += gridDim.y) {
+  for (int64_t z = z0; z < a.batches; z += z_step) {
     size_t in_off, out_off;
     batch_offsets(a, z, in_off, out_off);
     const uint8_t* src = a.in + in_off;
@@ -817,7 +831,16 @@ int mxq_quantized_transpose(void* stream, const void* in, const float* imin, con
       const dim3 grid(static_cast<unsigned>(fa * fb), static_cast<unsigned>(fy));
       bool friendly16 = (a.A % 16 == 0) && (a.b_in_stride % 16 == 0);
       for (int d = 0; d < a.p.nd; ++d) friendly16 = friendly16 && (a.p.in_stride[d] % 16 == 0);
-      if (tile_b == 128 && friendly16)
+      if (tile_b == 128 && friendly16 && a.A % 128 != 0 && a.batches <= 65535 &&
+          fa * fb * a.batches < (int64_t(1) << 31) - 8) {
+        // rows of A that miss the 128-byte marks (56 x 56, 28 x 28 planes): XCD-aware order,
+        // measured on the convolution's adapters (22.6 -> 21.1 us, 14.3 -> 12.1 us); rows on
+        // the marks lose 10 % with it and keep the plain grid
+        a.tiles_ab = static_cast<unsigned>(fa * fb);
+        a.xcd_total = static_cast<unsigned>(fa * fb * a.batches);
+        a.per_xcd = (a.xcd_total + 7u) / 8u;
+        hipLaunchKernelGGL(permute_tile16_kernel<16>, dim3(a.per_xcd * 8u), dim3(kThreads), 0, s, a);
+      } else if (tile_b == 128 && friendly16)
         hipLaunchKernelGGL(permute_tile16_kernel<16>, grid, dim3(kThreads), 0, s, a);
       else if (tile_b == 128)
         hipLaunchKernelGGL(permute_tile4_kernel<128>, grid, dim3(kThreads), 0, s, a);
