@@ -30,7 +30,7 @@
 extern "C" {
 #endif
 
-#define MXQ_ABI_VERSION 2
+#define MXQ_ABI_VERSION 3
 
 /* element type codes = mshadow::TypeFlag (3rdparty/mshadow/mshadow/base.h:351-364) */
 #define MXQ_FLOAT32 0
@@ -371,6 +371,30 @@ int mxq_quantized_conv_nhwc_out_nchw(void* stream, const int8_t* data, const int
                                      const float* min_bias, const float* max_bias,
                                      int32_t* out32_nchw, float* omin, float* omax,
                                      void* workspace, size_t workspace_bytes);
+
+/* _contrib_quantized_conv on the operator's own tensors: data int8 [N,C,H,W], weight int8
+ * [O,C,KH,KW], bias int8 [O] or NULL, out32 int32 [N,O,OH,OW] -- everything
+ * QuantizedCuDNNConvOp::Forward does between its inputs and its outputs
+ * (src/operator/quantization/quantized_conv.cu:101-219, layout rule quantized_conv.cc:38-45),
+ * the three TransposeImpl calls included (:145-148,183).  1 x 1 convolutions over planes of
+ * 16 | OH*OW bytes and 16 | C channels run on the NCHW tensors as they are (strided ones
+ * after their used pixels were gathered into the workspace); every other geometry goes
+ * through the layout adapters and mxq_quantized_conv_nhwc_out_nchw inside this call.
+ * `workspace` (16-byte aligned) must hold mxq_quantized_conv_nchw_workspace() bytes: the
+ * operator's kTempSpace (quantized_conv.cu:121-160 asks for three tensor copies plus
+ * cuDNN's workspace there; 0 here for a unit-stride 1 x 1 layer).  operands_aligned16 != 0
+ * says that data and weight both start on 16-byte marks, as a framework's allocations do;
+ * with 0 the query returns what the adapter route needs, which every geometry can take. */
+size_t mxq_quantized_conv_nchw_workspace(int N, int C, int H, int W, int O, int KH, int KW,
+                                         int stride_h, int stride_w, int pad_h, int pad_w,
+                                         int dilate_h, int dilate_w, int operands_aligned16);
+int mxq_quantized_conv_nchw(void* stream, const int8_t* data, const int8_t* weight,
+                            const int8_t* bias, int N, int C, int H, int W, int O, int KH, int KW,
+                            int stride_h, int stride_w, int pad_h, int pad_w, int dilate_h,
+                            int dilate_w, const float* min_data, const float* max_data,
+                            const float* min_weight, const float* max_weight,
+                            const float* min_bias, const float* max_bias, int32_t* out32,
+                            float* omin, float* omax, void* workspace, size_t workspace_bytes);
 
 /* [N,C,H,W] int8 -> [N,H,W,C] int8 (also OIHW -> OHWI for the weight). */
 int mxq_nchw_to_nhwc_i8(void* stream, const int8_t* in, int8_t* out, int N, int C, int H, int W);

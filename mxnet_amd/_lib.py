@@ -69,6 +69,9 @@ SIGNATURES = {
                                 [_p, _p, _p, _p, _p, _p, _i, _f, _f, _p, _sz]),
     "mxq_quantized_conv_nhwc_out_nchw": (_i, [_p, _p, _p, _p] + [_i] * 13 + [_p] * 6 +
                                          [_p, _p, _p, _p, _sz]),
+    "mxq_quantized_conv_nchw_workspace": (_sz, [_i] * 14),
+    "mxq_quantized_conv_nchw": (_i, [_p, _p, _p, _p] + [_i] * 13 + [_p] * 6 +
+                                [_p, _p, _p, _p, _sz]),
     "mxq_nchw_to_nhwc_i8": (_i, [_p, _p, _p, _i, _i, _i, _i]),
     "mxq_nchw_to_nhwc_pad_i8": (_i, [_p, _p, _p, _i, _i, _i, _i, _i]),
     "mxq_nchw_to_s2d_nhwc_i8": (_i, [_p, _p, _p, _i, _i, _i, _i, _i, _i, _i]),
@@ -88,6 +91,7 @@ TEST_HOOKS = {
     "mxq_test_quantized_fc_sum": (_i, SIGNATURES["mxq_quantized_fc_sum"][1] + [_i, _i, _i]),
     "mxq_test_quantized_fc_f32": (_i, SIGNATURES["mxq_quantized_fc_f32"][1] + [_i, _i]),
     "mxq_test_quantized_conv_nhwc": (_i, SIGNATURES["mxq_quantized_conv_nhwc"][1] + [_i, _i]),
+    "mxq_test_quantized_conv_nchw": (_i, SIGNATURES["mxq_quantized_conv_nchw"][1] + [_i]),
 }
 for _name, (_res, _args) in TEST_HOOKS.items():
     _fn = getattr(lib, _name)

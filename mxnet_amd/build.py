@@ -8,7 +8,7 @@ CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libmxq_hip.so")
 
 HIP_SOURCES = ["mxq_capi.hip", "mxq_cast.hip", "mxq_fc.hip", "mxq_fc_plain.hip", "mxq_fc_f32.hip",
-               "mxq_fc_sum.hip", "mxq_conv.hip", "mxq_pool.hip",
+               "mxq_fc_sum.hip", "mxq_conv.hip", "mxq_conv_nchw.hip", "mxq_pool.hip",
                "mxq_eltwise.hip", "mxq_layout.hip"]
 
 HIPCC_FLAGS = [

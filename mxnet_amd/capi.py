@@ -219,6 +219,36 @@ def quantized_conv_nhwc(data, weight, bias, min_data, max_data, min_weight, max_
     return res
 
 
+def quantized_conv_nchw(data, weight, bias, min_data, max_data, min_weight, max_weight,
+                        min_bias=None, max_bias=None, stride=(1, 1), pad=(0, 0), dilate=(1, 1),
+                        cfg=None, out=None):
+    """The operator's contract: data int8 [N,C,H,W], weight int8 [O,C,KH,KW] -> int32
+    [N,O,OH,OW].  `cfg` pins the route through the test-only entry point (1 = layout
+    adapters, 71... = a tile of the NCHW 1x1 kernel)."""
+    N, C, H, W = data.shape
+    O, C2, KH, KW = weight.shape
+    assert C == C2
+    OH = (H + 2 * pad[0] - (dilate[0] * (KH - 1) + 1)) // stride[0] + 1
+    OW = (W + 2 * pad[1] - (dilate[1] * (KW - 1) + 1)) // stride[1] + 1
+    dev = data.device
+    res = {"omin": _scalar(dev), "omax": _scalar(dev)}
+    out32 = out if out is not None else torch.empty((N, O, OH, OW), dtype=torch.int32, device=dev)
+    geo = [N, C, H, W, O, KH, KW, stride[0], stride[1], pad[0], pad[1], dilate[0], dilate[1]]
+    both_aligned = data.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0 and cfg != 1
+    wsb = lib.mxq_quantized_conv_nchw_workspace(*geo, int(both_aligned))
+    ws = _workspace(wsb, dev) if wsb else None
+    args = [_stream(), _ptr(data), _ptr(weight), _ptr(bias)] + geo + [
+        _ptr(min_data), _ptr(max_data), _ptr(min_weight), _ptr(max_weight), _ptr(min_bias),
+        _ptr(max_bias), _ptr(out32), _ptr(res["omin"]), _ptr(res["omax"]), _ptr(ws), wsb]
+    if cfg is None:
+        check(lib.mxq_quantized_conv_nchw(*args))
+    else:
+        check(lib.mxq_test_quantized_conv_nchw(*args, int(cfg)))
+    res["out32"] = out32
+    res["workspace_bytes"] = wsb
+    return res
+
+
 def nchw_to_nhwc_i8(x):
     N, C, H, W = x.shape
     out = torch.empty((N, H, W, C), dtype=torch.int8, device=x.device)

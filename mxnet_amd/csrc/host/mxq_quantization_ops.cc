@@ -636,91 +636,21 @@ static void QuantizedFullyConnectedForwardGPU(const NodeAttrs& attrs, const OpCo
       ws, ws != nullptr ? ws_bytes : 0));
 }
 
-// Temp space of the convolution: NHWC copies of data and weight plus the NHWC int32
-// result (the reference asks for the same three buffers plus cuDNN's workspace,
-// quantized_conv.cu:121-160).
-// Channels are zero-padded to a multiple of 16 while the operands are brought to NHWC:
-// the kernel's direct-to-LDS path needs 16-byte channel runs, and e.g. a 3-channel 7x7
-// stem runs three times faster on 16 channels (13 of them zero) than through the
-// byte-granular fallback.
-static int ConvPaddedChannels(int C) { return (C + 15) / 16 * 16; }
-
-// A stride-2 convolution over at most 4 channels (an image stem) is run as the unit-stride
-// convolution over the space-to-depth form of its operands (see mxq_nchw_to_s2d_nhwc_i8):
-// 4 * C real channels out of 16 instead of C out of 16.
-struct ConvS2D {
-  bool use;
-  int off_h, off_w;  // pad mod 2
-  int H2, W2;        // extents of the transformed image
-  int K2h, K2w;      // transformed window
-  int pad_h, pad_w;  // transformed padding
-};
-static ConvS2D ConvSpaceToDepth(const ConvolutionParam& param, const TShape& d, const TShape& w,
-                                const TShape& o) {
-  ConvS2D r = {};
-  const int C = d[1], H = d[2], W = d[3], KH = w[2], KW = w[3];
-  if (C > 4 || param.stride[0] != 2 || param.stride[1] != 2 || param.dilate[0] != 1 ||
-      param.dilate[1] != 1 || KH < 2 || KW < 2)
-    return r;
-  const int ph = param.pad[0], pw = param.pad[1];
-  r.off_h = ph & 1;
-  r.off_w = pw & 1;
-  r.H2 = (H + r.off_h + 1) / 2;
-  r.W2 = (W + r.off_w + 1) / 2;
-  r.K2h = (KH + 1) / 2;
-  r.K2w = (KW + 1) / 2;
-  r.pad_h = (ph - r.off_h) / 2;
-  r.pad_w = (pw - r.off_w) / 2;
-  // the transformed problem must produce exactly the operator's output extent
-  r.use = r.H2 + 2 * r.pad_h - r.K2h + 1 == static_cast<int>(o[2]) &&
-          r.W2 + 2 * r.pad_w - r.K2w + 1 == static_cast<int>(o[3]);
-  return r;
-}
-
-// The convolution as the kernel sees it: NHWC extents after channel padding or the
-// space-to-depth transform, and the bytes of the two operand copies in temp space.
-struct ConvKernelView {
-  ConvS2D s2d;
-  int H, W, C, KH, KW, sh, sw, ph, pw;
-  size_t d_bytes, w_bytes;  // rounded up to 256
-};
-static ConvKernelView ConvView(const ConvolutionParam& param, const TShape& d, const TShape& w,
-                               const TShape& o) {
-  auto up = [](size_t x) { return (x + 255) / 256 * 256; };
-  ConvKernelView v;
-  v.s2d = ConvSpaceToDepth(param, d, w, o);
-  const int N = d[0], C = d[1], O = w[0];
-  if (v.s2d.use) {
-    v.C = ConvPaddedChannels(4 * C);
-    v.H = v.s2d.H2; v.W = v.s2d.W2; v.KH = v.s2d.K2h; v.KW = v.s2d.K2w;
-    v.sh = v.sw = 1;
-    v.ph = v.s2d.pad_h; v.pw = v.s2d.pad_w;
-  } else {
-    v.C = ConvPaddedChannels(C);
-    v.H = d[2]; v.W = d[3]; v.KH = w[2]; v.KW = w[3];
-    v.sh = static_cast<int>(param.stride[0]); v.sw = static_cast<int>(param.stride[1]);
-    v.ph = static_cast<int>(param.pad[0]); v.pw = static_cast<int>(param.pad[1]);
-  }
-  v.d_bytes = up(static_cast<size_t>(N) * v.H * v.W * v.C);
-  v.w_bytes = up(static_cast<size_t>(O) * v.KH * v.KW * v.C);
-  return v;
-}
-
-// Bytes of split-K scratch the convolution kernel wants for this view (0: no split).
-static size_t ConvSplitBytes(const ConvolutionParam& param, const ConvKernelView& v, int N,
-                             int O) {
-  if (N <= 0 || O <= 0 || v.C <= 0) return 0;
-  return mxq_quantized_conv_workspace(N, v.H, v.W, v.C, O, v.KH, v.KW, v.sh, v.sw, v.ph, v.pw,
-                                      static_cast<int>(param.dilate[0]),
-                                      static_cast<int>(param.dilate[1]), 0);
-}
-
+// Temp space of the convolution: what mxq_quantized_conv_nchw wants for the geometry.  The
+// reference asks for NHWC copies of data, weight and output plus cuDNN's workspace
+// (quantized_conv.cu:121-160); here a unit-stride 1x1 layer runs on the NCHW tensors as
+// they are and needs none, a strided 1x1 layer the pixels it reads, every other geometry
+// the two operand copies (channels zero-padded to a multiple of 16 on the way) and, for
+// few tiles under a long reduction, the split-K partial sums.
 static size_t QuantizedConvTempBytes(const ConvolutionParam& param, const TShape& d,
-                                     const TShape& w, const TShape& o) {
-  const ConvKernelView v = ConvView(param, d, w, o);
-  // the output is written in its own layout: no third buffer
-  return v.d_bytes + v.w_bytes +
-         ConvSplitBytes(param, v, static_cast<int>(d[0]), static_cast<int>(w[0]));
+                                     const TShape& w, bool operands_aligned16) {
+  return mxq_quantized_conv_nchw_workspace(
+      static_cast<int>(d[0]), static_cast<int>(d[1]), static_cast<int>(d[2]),
+      static_cast<int>(d[3]), static_cast<int>(w[0]), static_cast<int>(w[2]),
+      static_cast<int>(w[3]), static_cast<int>(param.stride[0]),
+      static_cast<int>(param.stride[1]), static_cast<int>(param.pad[0]),
+      static_cast<int>(param.pad[1]), static_cast<int>(param.dilate[0]),
+      static_cast<int>(param.dilate[1]), operands_aligned16 ? 1 : 0);
 }
 
 // QuantizedConvForwardGPU, quantized_conv.cu:268-291
@@ -734,34 +664,26 @@ static void QuantizedConvForwardGPU(const NodeAttrs& attrs, const OpContext& ctx
   CHECK_EQ(outputs.size(), 3U);
   const TShape& d = inputs[0].shape_;
   const TShape& w = inputs[1].shape_;
-  const TShape& o = outputs[0].shape_;
-  CHECK(!ctx.requested.empty()) << "quantized_conv needs its temp space resource";
   const int N = d[0], C = d[1], H = d[2], W = d[3], O = w[0], KH = w[2], KW = w[3];
-  const ConvKernelView v = ConvView(param, d, w, o);
-  const size_t split_bytes = ConvSplitBytes(param, v, N, O);
-  char* ws = ctx.requested[0].get_space(v.d_bytes + v.w_bytes + split_bytes);
-  void* stream = raw_stream(ctx);
-  int8_t* d_nhwc = reinterpret_cast<int8_t*>(ws);
-  int8_t* w_ohwi = reinterpret_cast<int8_t*>(ws + v.d_bytes);
-  void* split_ws = split_bytes != 0 ? ws + v.d_bytes + v.w_bytes : nullptr;
-  if (v.s2d.use) {
-    MXQ_CALL(mxq_nchw_to_s2d_nhwc_i8(stream, inputs[0].dptr<int8_t>(), d_nhwc, N, C, H, W,
-                                     v.s2d.off_h, v.s2d.off_w, v.C));
-    MXQ_CALL(mxq_nchw_to_s2d_nhwc_i8(stream, inputs[1].dptr<int8_t>(), w_ohwi, O, C, KH, KW, 0, 0,
-                                     v.C));
-  } else {
-    MXQ_CALL(mxq_nchw_to_nhwc_pad_i8(stream, inputs[0].dptr<int8_t>(), d_nhwc, N, C, H, W, v.C));
-    MXQ_CALL(mxq_nchw_to_nhwc_pad_i8(stream, inputs[1].dptr<int8_t>(), w_ohwi, O, C, KH, KW, v.C));
+  auto on16 = [](const void* q) { return (reinterpret_cast<uintptr_t>(q) & 15u) == 0; };
+  const size_t ws_bytes =
+      QuantizedConvTempBytes(param, d, w, on16(inputs[0].dptr_) && on16(inputs[1].dptr_));
+  char* ws = nullptr;
+  if (ws_bytes != 0) {
+    CHECK(!ctx.requested.empty()) << "quantized_conv needs its temp space resource";
+    ws = ctx.requested[0].get_space(ws_bytes);
   }
   const size_t ni = param.no_bias ? 2 : 3;
-  MXQ_CALL(mxq_quantized_conv_nhwc_out_nchw(
-      stream, d_nhwc, w_ohwi, param.no_bias ? nullptr : inputs[2].dptr<int8_t>(), N, v.H, v.W,
-      v.C, O, v.KH, v.KW, v.sh, v.sw, v.ph, v.pw, static_cast<int>(param.dilate[0]),
-      static_cast<int>(param.dilate[1]),
+  MXQ_CALL(mxq_quantized_conv_nchw(
+      raw_stream(ctx), inputs[0].dptr<int8_t>(), inputs[1].dptr<int8_t>(),
+      param.no_bias ? nullptr : inputs[2].dptr<int8_t>(), N, C, H, W, O, KH, KW,
+      static_cast<int>(param.stride[0]), static_cast<int>(param.stride[1]),
+      static_cast<int>(param.pad[0]), static_cast<int>(param.pad[1]),
+      static_cast<int>(param.dilate[0]), static_cast<int>(param.dilate[1]),
       inputs[ni].dptr<float>(), inputs[ni + 1].dptr<float>(), inputs[ni + 2].dptr<float>(),
       inputs[ni + 3].dptr<float>(), param.no_bias ? nullptr : inputs[7].dptr<float>(),
       param.no_bias ? nullptr : inputs[8].dptr<float>(), outputs[0].dptr<int32_t>(),
-      outputs[1].dptr<float>(), outputs[2].dptr<float>(), split_ws, split_bytes));
+      outputs[1].dptr<float>(), outputs[2].dptr<float>(), ws, ws_bytes));
 }
 
 // _contrib_quantized_act: int8 relu, ranges pass through (dnnl_quantized_act.cc:33-45)
@@ -956,7 +878,7 @@ size_t MXQTempSpaceBytes(const NodeAttrs& attrs, const ShapeVector& in, const Sh
   if (name == "_contrib_quantize_v2") return mxq_quantize_v2_workspace(in[0].Size());
   if (name == "_contrib_requantize") return mxq_requantize_workspace(in[0].Size());
   if (name == "_contrib_quantized_conv")
-    return QuantizedConvTempBytes(nnvm::get<ConvolutionParam>(attrs.parsed), in[0], in[1], out[0]);
+    return QuantizedConvTempBytes(nnvm::get<ConvolutionParam>(attrs.parsed), in[0], in[1], false);
   if (name == "_contrib_quantized_fully_connected") {
     // rows x reduction as QuantizedFullyConnectedForwardGPU reads them off the shapes
     const auto& param = nnvm::get<FullyConnectedParam>(attrs.parsed);

@@ -1,0 +1,532 @@
+// _contrib_quantized_conv on the operator's own tensors: NCHW int8 data, OIHW int8
+// weights, NCHW int32 output (src/operator/quantization/quantized_conv.cc:38-45).  The
+// reference's GPU operator brings both operands to NHWC with two TransposeImpl calls,
+// runs cuDNN, and transposes the result back (quantized_conv.cu:145-148,183).  Here a
+// 1 x 1 convolution, which is most of a bottleneck network, never leaves NCHW:
+//
+//   out[n][o][p] = bias32[o] + sum_c W[o][c] * X[n][c][p]        p = pixel of the plane
+//
+// per image is a GEMM whose activation operand lies "K-major" in memory: channel rows of
+// contiguous pixels.  A work-group stages [BK channels] x [BP pixels] slabs of the plane
+// straight into LDS (buffer_load ... lds, 16 bytes of one channel row per lane) and reads
+// the MFMA fragments out of them with the transposing LDS load of gfx950
+// (ds_read_b64_tr_b8): 16 lanes that point at 8 channel rows x 16 pixels get back, per
+// lane, one pixel's 8 consecutive channels, which is the operand layout
+// v_mfma_i32_32x32x32_i8 wants.  The weights [O][C] are already K-contiguous (OIHW of a
+// 1 x 1 window is OHWI) and take the same path as in the fully-connected kernel.  In the
+// result a lane holds one pixel and registers hold channels, so every store instruction
+// writes two 128-byte runs of two channel planes: the int32 output goes to its NCHW place
+// straight from the accumulators.  No adapter launch, no second copy of any tensor.
+//
+// Strided 1 x 1 convolutions first gather the pixels they use into a compact NCHW tensor
+// (a quarter of the input for stride 2) in the caller's workspace and then run the same
+// kernel.  Everything else (3 x 3, padded, planes whose size is no multiple of 16 bytes)
+// takes the NHWC kernels of mxq_conv.hip behind the layout adapters.
+#include <hip/hip_runtime.h>
+
+#include <cmath>
+#include <cstdint>
+
+#include "../../include/mxq.h"
+#include "mxq_common.h"
+#include "mxq_gemm.h"
+#include "mxq_tiles.h"
+
+namespace mxq {
+namespace {
+
+struct PlaneArgs {
+  const int8_t* data;    // [N][C][P]
+  const int8_t* weight;  // [O][C]
+  int N, C, P, O;
+  int tiles_p, tiles_o;
+  Epilogue epi;          // bias, input ranges, out32 ([N][O][P]), omin / omax
+};
+
+// Tile of BP pixels of one image x BO output channels; BK channels per stage.  The names
+// CH / BK / kThreads are what DmaLane and RowIssuerBuffer (mxq_gemm.h) read for the weight
+// operand.
+template <int BP_, int BO_, int BK_, int WP_, int WO_>
+struct PlaneCfg {
+  static constexpr int BP = BP_, BO = BO_, BK = BK_, WP = WP_, WO = WO_;
+  static constexpr int NW = WP * WO, kThreads = 64 * NW;
+  static constexpr int CHP = BP / 16;      // 16-byte pixel chunks per channel row
+  static constexpr int CH = BK / 16;       // 16-byte chunks per weight row
+  static constexpr int TP = BP / WP, TO = BO / WO;
+  static constexpr int MI = TP / 32, NI = TO / 32, KS = BK / 32;
+  static constexpr int A_SLOTS = BK * CHP, B_SLOTS = BO * CH;
+  static constexpr int STAGE_SLOTS = A_SLOTS + B_SLOTS;
+  static constexpr int A_INSTR = A_SLOTS / (64 * NW), B_INSTR = B_SLOTS / (64 * NW);
+  static_assert(BP % (32 * WP) == 0 && BO % (32 * WO) == 0, "wave tile");
+  static_assert(A_SLOTS % (64 * NW) == 0 && B_SLOTS % (64 * NW) == 0, "loader");
+  static_assert(CHP == 4 || CHP == 8, "pixel-chunk swizzle");
+  static_assert(CH == 4 || CH == 8, "fragment addressing of the weight operand");
+};
+
+// Where pixel chunk pc of channel row c sits in its row: pc ^ plane_swz(c).  A transposing
+// read touches, per 16 lanes, one 16-byte chunk of 8 consecutive rows, and two such groups
+// (chunks pc and pc + 1, pc even) go through the LDS together: the XOR makes those 16
+// pieces hit 16 different bank groups.  Rows of 128 bytes: the row's low three bits; rows
+// of 64 bytes (four rows per 256 bytes of banks): bit 2 of the row moves the chunk by two.
+template <int CHP>
+__device__ __forceinline__ int plane_swz(int c) {
+  return CHP == 8 ? (c & 7) : ((c >> 1) & 2);
+}
+
+typedef int v2i __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ v2i lds_read_tr8(const char* p) {
+  return __builtin_amdgcn_ds_read_tr8_b64_v2i32(
+      (v2i __attribute__((address_space(3)))*)(p));
+}
+
+template <class Cfg, int NS>
+__global__ __launch_bounds__(Cfg::kThreads, 2) void conv1x1_planes_kernel(PlaneArgs p) {
+  constexpr int BP = Cfg::BP, BK = Cfg::BK, CHP = Cfg::CHP, CH = Cfg::CH, NW = Cfg::NW;
+  constexpr int MI = Cfg::MI, NI = Cfg::NI, KS = Cfg::KS;
+  constexpr int AI = Cfg::A_INSTR, BI = Cfg::B_INSTR, CPT = AI + BI;
+  constexpr int STAGE_BYTES = Cfg::STAGE_SLOTS * 16, A_BYTES = Cfg::A_SLOTS * 16;
+  static_assert((NS - 2) * CPT < 64, "vmcnt range");
+  __shared__ __attribute__((aligned(16))) v4i lds[NS * Cfg::STAGE_SLOTS];
+  __shared__ __attribute__((aligned(16))) int sbias[Cfg::BO];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wp = wave / Cfg::WO, wo = wave % Cfg::WO;
+
+  // tile order: the output-channel tiles of one pixel slab are neighbours, and the
+  // round-robin of work-group ids over the XCDs is undone so that they meet in one L2
+  const int total = p.N * p.tiles_p * p.tiles_o;
+  const int lid = xcd_remap(blockIdx.x, total);
+  const int to = lid % p.tiles_o;
+  const int rest = lid / p.tiles_o;
+  const int tp = rest % p.tiles_p, n = rest / p.tiles_p;
+  const int p0 = tp * BP, o0 = to * Cfg::BO;
+
+  // activation loads: slot q of a stage (16 bytes) = channel row q / CHP, chunk q % CHP
+  const v4i arsrc = make_rsrc(p.data, static_cast<uint32_t>(p.N) * p.C * p.P);
+  uint32_t a_off[AI];
+  int a_c[AI];
+#pragma unroll
+  for (int j = 0; j < AI; ++j) {
+    const int q = (j * NW + wave) * 64 + lane;
+    const int c = q / CHP, pc = (q % CHP) ^ plane_swz<CHP>(c);
+    a_c[j] = c;
+    a_off[j] = (static_cast<uint32_t>(n) * p.C + c) * p.P + p0 + pc * 16;
+  }
+  RowIssuerBuffer<Cfg, BI> bi;
+  bi.init(p.weight, o0, p.O, p.C, wave, lane, 0);
+  const uint32_t lds0 = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(lds));
+  const int KT = (p.C + BK - 1) / BK;
+  auto issue = [&](int stage) {
+    if (stage >= KT) return;
+    const uint32_t sb = lds0 + static_cast<uint32_t>(stage % NS) * STAGE_BYTES;
+#pragma unroll
+    for (int j = 0; j < AI; ++j) {
+      const int c = stage * BK + a_c[j];
+      const uint32_t off =
+          c < p.C ? a_off[j] + static_cast<uint32_t>(stage * BK) * p.P : kOutOfRange;
+      dma_buffer(sb + (j * NW + wave) * 1024, off, arsrc);
+    }
+#pragma unroll
+    for (int j = 0; j < BI; ++j) bi.issue(j, stage, sb + A_BYTES + (j * NW + wave) * 1024);
+  };
+
+  // fragment addresses.  Activation: lane = 16 * G + s reads 8 bytes of channel row
+  // 16 * (G / 2) + s / 2 (+ 32 * ks + 8 * t) at pixel 16 * (G % 2) + 8 * (s % 2) of MFMA
+  // tile mi; the transposing load hands lane l the 8 channels of pixel l % 32, and two
+  // such loads (t = 0, 1) make the 16 bytes of k-group l / 32.
+  const int G = lane >> 4, s16 = lane & 15;
+  const int crow = 16 * (G >> 1) + (s16 >> 1);
+  int a_frag[MI];
+#pragma unroll
+  for (int mi = 0; mi < MI; ++mi) {
+    const int pc = (wp * Cfg::TP + 32 * mi) / 16 + (G & 1);
+    a_frag[mi] = crow * BP + ((pc ^ plane_swz<CHP>(crow)) << 4) + 8 * (s16 & 1);
+  }
+  const int frow = lane & 31, fgrp = lane >> 5;
+  const int rb = wo * Cfg::TO + frow;
+  int fb0[KS];
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) fb0[ks] = rb * CH + ((ks * 2 + fgrp) ^ swz<CH>(rb));
+
+  v16i acc[MI][NI];
+#pragma unroll
+  for (int mi = 0; mi < MI; ++mi)
+#pragma unroll
+    for (int ni = 0; ni < NI; ++ni)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[mi][ni][v] = 0;
+
+#pragma unroll
+  for (int st = 0; st < NS - 1; ++st) issue(st);
+  // what the epilogue needs, behind the first operand fetch
+  const EpiScalars es = epi_scalars(p.epi);
+  if (tid < Cfg::BO) sbias[tid] = (o0 + tid < p.O) ? epi_bias32(p.epi, es, o0 + tid) : 0;
+
+  for (int kt = 0; kt < KT; ++kt) {
+    const int newest = (kt + NS - 2) < (KT - 1) ? (kt + NS - 2) : (KT - 1);
+    wait_ahead<CPT, NS - 2>(newest - kt);
+    __builtin_amdgcn_s_barrier();
+    issue(kt + NS - 1);
+    const char* sa = reinterpret_cast<const char*>(lds) + (kt % NS) * STAGE_BYTES;
+    const v4i* sbw = reinterpret_cast<const v4i*>(sa + A_BYTES);
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      v4i fa[MI], fb[NI];
+#pragma unroll
+      for (int mi = 0; mi < MI; ++mi) {
+        const v2i lo = lds_read_tr8(sa + a_frag[mi] + (32 * ks) * BP);
+        const v2i hi = lds_read_tr8(sa + a_frag[mi] + (32 * ks + 8) * BP);
+        fa[mi] = v4i{lo.x, lo.y, hi.x, hi.y};
+      }
+#pragma unroll
+      for (int ni = 0; ni < NI; ++ni) fb[ni] = sbw[fb0[ks] + ni * 32 * CH];
+#pragma unroll
+      for (int mi = 0; mi < MI; ++mi)
+#pragma unroll
+        for (int ni = 0; ni < NI; ++ni)
+          acc[mi][ni] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fb[ni], fa[mi], acc[mi][ni], 0, 0, 0);
+    }
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  if (blockIdx.x == 0 && tid == 0) epilogue_ranges(p.epi);
+  __syncthreads();  // sbias (written before the loop; K = 0 would skip its barriers)
+
+  // lane = pixel, register = channel 8 * (v / 4) + 4 * (lane / 32) + v % 4 of the MFMA
+  // tile: a store instruction writes 32 consecutive int32 of two channel planes
+  const int px_base = p0 + wp * Cfg::TP + frow;
+  int32_t* out_img = p.epi.out32 + static_cast<size_t>(n) * p.O * p.P;
+#pragma unroll
+  for (int ni = 0; ni < NI; ++ni) {
+#pragma unroll
+    for (int vq = 0; vq < 4; ++vq) {
+      const int ol = wo * Cfg::TO + ni * 32 + 8 * vq + 4 * fgrp;  // channel inside the tile
+      const v4i b = *reinterpret_cast<const v4i*>(sbias + ol);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int o = o0 + ol + i;
+        if (o < p.O) {
+          int32_t* plane = out_img + static_cast<size_t>(o) * p.P;
+#pragma unroll
+          for (int mi = 0; mi < MI; ++mi) {
+            const int px = px_base + 32 * mi;
+            if (px < p.P)
+              plane[px] = static_cast<int>(static_cast<uint32_t>(acc[mi][ni][4 * vq + i]) +
+                                           static_cast<uint32_t>(b[i]));
+          }
+        }
+      }
+    }
+  }
+}
+
+// out[b][oh][ow] = in[b][oh * sh][ow * sw] over B = N * C planes: the pixels a strided
+// 1 x 1 convolution without padding reads, compacted.  FAST: sw == 2, 4 | OW and rows on
+// dword marks, a thread makes one dword of output from two of input.
+template <bool FAST>
+__global__ __launch_bounds__(256) void subsample_planes_kernel(const uint8_t* __restrict__ in,
+                                                               uint8_t* __restrict__ out, int H,
+                                                               int W, int OH, int OW, int sh,
+                                                               int sw, size_t items) {
+  const size_t stride = static_cast<size_t>(gridDim.x) * 256;
+  for (size_t i = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x; i < items; i += stride) {
+    if (FAST) {
+      const int q = OW / 4;
+      const int x = static_cast<int>(i % q);
+      const size_t t = i / q;
+      const int oh = static_cast<int>(t % OH);
+      const size_t b = t / OH;
+      const uint8_t* src = in + (b * H + static_cast<size_t>(oh) * sh) * W + 8 * x;
+      const uint32_t lo = *reinterpret_cast<const uint32_t*>(src);
+      const uint32_t hi = *reinterpret_cast<const uint32_t*>(src + 4);
+      // bytes 0 and 2 of each dword
+      const uint32_t v = __builtin_amdgcn_perm(hi, lo, 0x06040200u);
+      *reinterpret_cast<uint32_t*>(out + (b * OH + oh) * OW + 4 * x) = v;
+    } else {
+      const int ow = static_cast<int>(i % OW);
+      const size_t t = i / OW;
+      const int oh = static_cast<int>(t % OH);
+      const size_t b = t / OH;
+      out[i] = in[(b * H + static_cast<size_t>(oh) * sh) * W + static_cast<size_t>(ow) * sw];
+    }
+  }
+}
+
+void launch_subsample(hipStream_t s, const int8_t* in, int8_t* out, long long planes, int H,
+                      int W, int OH, int OW, int sh, int sw) {
+  const bool fast = sw == 2 && OW % 4 == 0 && W % 4 == 0 &&
+                    (reinterpret_cast<uintptr_t>(in) & 3u) == 0 &&
+                    (reinterpret_cast<uintptr_t>(out) & 3u) == 0 && 8 * (OW / 4) <= W;
+  const size_t items = static_cast<size_t>(planes) * OH * (fast ? OW / 4 : OW);
+  if (items == 0) return;
+  size_t grid = (items + 255) / 256;
+  const size_t cap = static_cast<size_t>(num_cus()) * 16;
+  if (grid > cap) grid = cap;
+  if (fast)
+    hipLaunchKernelGGL(subsample_planes_kernel<true>, dim3(static_cast<unsigned>(grid)),
+                       dim3(256), 0, s, reinterpret_cast<const uint8_t*>(in),
+                       reinterpret_cast<uint8_t*>(out), H, W, OH, OW, sh, sw, items);
+  else
+    hipLaunchKernelGGL(subsample_planes_kernel<false>, dim3(static_cast<unsigned>(grid)),
+                       dim3(256), 0, s, reinterpret_cast<const uint8_t*>(in),
+                       reinterpret_cast<uint8_t*>(out), H, W, OH, OW, sh, sw, items);
+  MXQ_LAUNCH_CHECK();
+}
+
+typedef PlaneCfg<128, 128, 64, 2, 2> PlaneM;   // 4 waves, wave tile 64 pixels x 64 channels
+typedef PlaneCfg<128, 64, 64, 2, 2> PlaneN64;  // 4 waves, wave tile 64 x 32
+typedef PlaneCfg<64, 128, 64, 2, 2> PlaneP64;  // 4 waves, wave tile 32 x 64
+typedef PlaneCfg<64, 64, 64, 2, 2> PlaneS;     // 4 waves, wave tile 32 x 32
+typedef PlaneCfg<128, 256, 64, 2, 4> PlaneW;   // 8 waves, wave tile 64 x 64
+
+template <class Cfg>
+void launch_planes(hipStream_t s, PlaneArgs a) {
+  a.tiles_p = (a.P + Cfg::BP - 1) / Cfg::BP;
+  a.tiles_o = (a.O + Cfg::BO - 1) / Cfg::BO;
+  const long long total = 1LL * a.N * a.tiles_p * a.tiles_o;
+  MXQ_CHECK(total < (1LL << 31), "grid too large");
+  hipLaunchKernelGGL((conv1x1_planes_kernel<Cfg, 2>), dim3(static_cast<unsigned>(total)),
+                     dim3(Cfg::kThreads), 0, s, a);
+  MXQ_LAUNCH_CHECK();
+}
+
+// The route a convolution takes.
+enum class Route {
+  kPlanes,        // 1 x 1, unit stride: the NCHW kernel on the operator's own tensors
+  kPlanesStrided, // 1 x 1, strided: gather the used pixels, then the NCHW kernel
+  kSpaceToDepth,  // few-channel stride-2 stem through mxq_nchw_to_s2d_nhwc_i8
+  kAdapters       // NHWC copies of both operands, NHWC kernel writing NCHW planes
+};
+
+int padded_channels(int C) { return (C + 15) / 16 * 16; }
+size_t up256(size_t x) { return (x + 255) / 256 * 256; }
+
+struct NchwPlan {
+  Route route;
+  int OH, OW;
+  // kSpaceToDepth
+  int off_h, off_w, H2, W2, K2h, K2w, pad2_h, pad2_w;
+  // NHWC view of the adapter routes
+  int vC;
+  bool weight_in_place;    // 1 x 1 window over C % 16 == 0 channels: OIHW is OHWI already
+  size_t d_bytes, w_bytes, split_bytes;
+};
+
+NchwPlan plan_nchw(int N, int C, int H, int W, int O, int KH, int KW, int sh, int sw, int ph,
+                   int pw, int dh, int dw, bool operands_aligned) {
+  MXQ_CHECK(N >= 0 && C > 0 && H > 0 && W > 0 && O > 0 && KH > 0 && KW > 0, "bad shape");
+  MXQ_CHECK(sh > 0 && sw > 0 && dh > 0 && dw > 0 && ph >= 0 && pw >= 0, "bad stride/dilate/pad");
+  const int eh = dh * (KH - 1) + 1, ew = dw * (KW - 1) + 1;
+  MXQ_CHECK(H + 2 * ph >= eh && W + 2 * pw >= ew, "kernel larger than padded input");
+  NchwPlan pl = {};
+  pl.OH = (H + 2 * ph - eh) / sh + 1;
+  pl.OW = (W + 2 * pw - ew) / sw + 1;
+  const long long P = 1LL * pl.OH * pl.OW;
+  const bool one = KH == 1 && KW == 1 && ph == 0 && pw == 0;
+  const bool small = 1LL * N * C * P < (1LL << 31) && 1LL * O * C < (1LL << 31) &&
+                     1LL * N * C * H * W < (1LL << 31);
+  if (one && operands_aligned && C % 16 == 0 && P % 16 == 0 && small) {
+    if (sh == 1 && sw == 1) {
+      pl.route = Route::kPlanes;
+      return pl;
+    }
+    pl.route = Route::kPlanesStrided;
+    pl.d_bytes = up256(static_cast<size_t>(N) * C * P);
+    return pl;
+  }
+  // a stride-2 convolution over at most 4 channels (an image stem) runs as the unit-stride
+  // convolution over the space-to-depth form of its operands: 4 * C real channels out of 16
+  // instead of C out of 16
+  if (C <= 4 && sh == 2 && sw == 2 && dh == 1 && dw == 1 && KH >= 2 && KW >= 2) {
+    pl.off_h = ph & 1;
+    pl.off_w = pw & 1;
+    pl.H2 = (H + pl.off_h + 1) / 2;
+    pl.W2 = (W + pl.off_w + 1) / 2;
+    pl.K2h = (KH + 1) / 2;
+    pl.K2w = (KW + 1) / 2;
+    pl.pad2_h = (ph - pl.off_h) / 2;
+    pl.pad2_w = (pw - pl.off_w) / 2;
+    // only when the transformed problem gives exactly the operator's output extent
+    if (pl.H2 + 2 * pl.pad2_h - pl.K2h + 1 == pl.OH && pl.W2 + 2 * pl.pad2_w - pl.K2w + 1 == pl.OW) {
+      pl.route = Route::kSpaceToDepth;
+      pl.vC = padded_channels(4 * C);
+      pl.d_bytes = up256(static_cast<size_t>(N) * pl.H2 * pl.W2 * pl.vC);
+      pl.w_bytes = up256(static_cast<size_t>(O) * pl.K2h * pl.K2w * pl.vC);
+      pl.split_bytes = mxq_quantized_conv_workspace(N, pl.H2, pl.W2, pl.vC, O, pl.K2h, pl.K2w, 1,
+                                                    1, pl.pad2_h, pl.pad2_w, 1, 1, 0);
+      return pl;
+    }
+  }
+  pl.route = Route::kAdapters;
+  pl.vC = padded_channels(C);
+  pl.weight_in_place = KH == 1 && KW == 1 && C % 16 == 0 && operands_aligned;
+  pl.d_bytes = up256(static_cast<size_t>(N) * H * W * pl.vC);
+  pl.w_bytes = pl.weight_in_place ? 0 : up256(static_cast<size_t>(O) * KH * KW * pl.vC);
+  pl.split_bytes =
+      mxq_quantized_conv_workspace(N, H, W, pl.vC, O, KH, KW, sh, sw, ph, pw, dh, dw, 0);
+  return pl;
+}
+
+// The entry points of the adapter routes are this library's own C functions: their error
+// text is already on the thread when they fail.
+#define MXQ_FORWARD(call)                                      \
+  do {                                                         \
+    if ((call) != 0) throw ::mxq::Error(mxq_last_error());     \
+  } while (0)
+
+void conv_nchw(void* stream, const int8_t* data, const int8_t* weight, const int8_t* bias, int N,
+               int C, int H, int W, int O, int KH, int KW, int sh, int sw, int ph, int pw, int dh,
+               int dw, const float* min_data, const float* max_data, const float* min_weight,
+               const float* max_weight, const float* min_bias, const float* max_bias,
+               int32_t* out32, float* omin, float* omax, void* workspace, size_t workspace_bytes,
+               int cfg) {
+  MXQ_CHECK(min_data && max_data && min_weight && max_weight, "null input range pointer");
+  MXQ_CHECK(omin && omax, "null output range pointer");
+  MXQ_CHECK(bias == nullptr || (min_bias && max_bias), "bias given without its range");
+  MXQ_CHECK(N == 0 || (data != nullptr && weight != nullptr && out32 != nullptr),
+            "null tensor pointer");
+  if (N == 0) {
+    // no output elements: the range scalars alone
+    MXQ_FORWARD(mxq_quantized_conv_nhwc(stream, data, weight, bias, 0, H, W, C, O, KH, KW, sh, sw,
+                                        ph, pw, dh, dw, min_data, max_data, min_weight,
+                                        max_weight, min_bias, max_bias, out32, omin, omax,
+                                        nullptr, nullptr, nullptr, 0, 0.f, 0.f, nullptr, 0));
+    return;
+  }
+  // cfg 1 pins the adapter route; 71.. pin a tile of the NCHW kernel
+  const bool aligned = aligned16(data) && aligned16(weight) && cfg != 1;
+  NchwPlan pl = plan_nchw(N, C, H, W, O, KH, KW, sh, sw, ph, pw, dh, dw, aligned);
+  MXQ_CHECK(cfg < 70 || pl.route == Route::kPlanes || pl.route == Route::kPlanesStrided,
+            "shape does not qualify for the NCHW 1x1 kernel");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  char* ws = static_cast<char*>(workspace);
+  const size_t need = pl.d_bytes + pl.w_bytes;
+  MXQ_CHECK(need == 0 || (ws != nullptr && aligned16(ws) && workspace_bytes >= need),
+            "workspace too small: " << workspace_bytes << " < " << need
+                                    << " (see mxq_quantized_conv_nchw_workspace)");
+
+  if (pl.route == Route::kPlanes || pl.route == Route::kPlanesStrided) {
+    const int8_t* planes = data;
+    if (pl.route == Route::kPlanesStrided) {
+      launch_subsample(s, data, reinterpret_cast<int8_t*>(ws), 1LL * N * C, H, W, pl.OH, pl.OW,
+                       sh, sw);
+      planes = reinterpret_cast<const int8_t*>(ws);
+    }
+    PlaneArgs a = {};
+    a.data = planes;
+    a.weight = weight;
+    a.N = N; a.C = C; a.P = pl.OH * pl.OW; a.O = O;
+    Epilogue& e = a.epi;
+    e = Epilogue();
+    e.bias = bias;
+    e.min_data = min_data; e.max_data = max_data;
+    e.min_weight = min_weight; e.max_weight = max_weight;
+    e.min_bias = min_bias; e.max_bias = max_bias;
+    e.out32 = out32;
+    e.omin = omin; e.omax = omax;
+    int pick = cfg;
+    if (pick < 70) {
+      const long cus = num_cus();
+      const long slabs128 = 1L * N * ((a.P + 127) / 128);
+      if (O <= 64)
+        pick = 72;
+      else if (O % 256 == 0 && slabs128 * (O / 256) >= 2 * cus)
+        pick = 75;
+      else if (slabs128 * ((O + 127) / 128) >= 2 * cus)
+        pick = 71;
+      else
+        pick = 73;
+    }
+    switch (pick) {
+      case 71: launch_planes<PlaneM>(s, a); break;
+      case 72: launch_planes<PlaneN64>(s, a); break;
+      case 73: launch_planes<PlaneP64>(s, a); break;
+      case 74: launch_planes<PlaneS>(s, a); break;
+      case 75: launch_planes<PlaneW>(s, a); break;
+      default: MXQ_CHECK(false, "unknown NCHW tile configuration " << pick);
+    }
+    return;
+  }
+
+  int8_t* d_nhwc = reinterpret_cast<int8_t*>(ws);
+  int8_t* w_ohwi = reinterpret_cast<int8_t*>(ws + pl.d_bytes);
+  const size_t split_room = workspace_bytes - need;
+  void* split_ws = split_room != 0 ? ws + need : nullptr;
+  if (pl.route == Route::kSpaceToDepth) {
+    MXQ_FORWARD(mxq_nchw_to_s2d_nhwc_i8(stream, data, d_nhwc, N, C, H, W, pl.off_h, pl.off_w,
+                                        pl.vC));
+    MXQ_FORWARD(mxq_nchw_to_s2d_nhwc_i8(stream, weight, w_ohwi, O, C, KH, KW, 0, 0, pl.vC));
+    MXQ_FORWARD(mxq_quantized_conv_nhwc_out_nchw(
+        stream, d_nhwc, w_ohwi, bias, N, pl.H2, pl.W2, pl.vC, O, pl.K2h, pl.K2w, 1, 1, pl.pad2_h,
+        pl.pad2_w, 1, 1, min_data, max_data, min_weight, max_weight, min_bias, max_bias, out32,
+        omin, omax, split_ws, split_room));
+    return;
+  }
+  MXQ_FORWARD(mxq_nchw_to_nhwc_pad_i8(stream, data, d_nhwc, N, C, H, W, pl.vC));
+  const int8_t* wk = weight;
+  if (!pl.weight_in_place) {
+    MXQ_FORWARD(mxq_nchw_to_nhwc_pad_i8(stream, weight, w_ohwi, O, C, KH, KW, pl.vC));
+    wk = w_ohwi;
+  }
+  MXQ_FORWARD(mxq_quantized_conv_nhwc_out_nchw(
+      stream, d_nhwc, wk, bias, N, H, W, pl.vC, O, KH, KW, sh, sw, ph, pw, dh, dw, min_data,
+      max_data, min_weight, max_weight, min_bias, max_bias, out32, omin, omax, split_ws,
+      split_room));
+}
+
+}  // namespace
+}  // namespace mxq
+
+using namespace mxq;
+
+extern "C" {
+
+size_t mxq_quantized_conv_nchw_workspace(int N, int C, int H, int W, int O, int KH, int KW,
+                                         int stride_h, int stride_w, int pad_h, int pad_w,
+                                         int dilate_h, int dilate_w, int operands_aligned16) {
+  try {
+    if (N <= 0) return 0;
+    const NchwPlan b = plan_nchw(N, C, H, W, O, KH, KW, stride_h, stride_w, pad_h, pad_w,
+                                 dilate_h, dilate_w, false);
+    const size_t nb = b.d_bytes + b.w_bytes + b.split_bytes;
+    if (operands_aligned16 == 0) return nb;
+    const NchwPlan a = plan_nchw(N, C, H, W, O, KH, KW, stride_h, stride_w, pad_h, pad_w,
+                                 dilate_h, dilate_w, true);
+    return a.d_bytes + a.w_bytes + a.split_bytes;
+  } catch (...) {
+    return 0;
+  }
+}
+
+int mxq_quantized_conv_nchw(void* stream, const int8_t* data, const int8_t* weight,
+                            const int8_t* bias, int N, int C, int H, int W, int O, int KH, int KW,
+                            int stride_h, int stride_w, int pad_h, int pad_w, int dilate_h,
+                            int dilate_w, const float* min_data, const float* max_data,
+                            const float* min_weight, const float* max_weight,
+                            const float* min_bias, const float* max_bias, int32_t* out32,
+                            float* omin, float* omax, void* workspace, size_t workspace_bytes) {
+  MXQ_API_BEGIN();
+  conv_nchw(stream, data, weight, bias, N, C, H, W, O, KH, KW, stride_h, stride_w, pad_h, pad_w,
+            dilate_h, dilate_w, min_data, max_data, min_weight, max_weight, min_bias, max_bias,
+            out32, omin, omax, workspace, workspace_bytes, 0);
+  MXQ_API_END();
+}
+
+// Test-only twin (declared in tests/mxq_test_hooks.h): cfg 1 pins the route through the
+// layout adapters, 71 ... 75 a tile of the NCHW kernel, 0 leaves the choice to the launcher.
+int mxq_test_quantized_conv_nchw(void* stream, const int8_t* data, const int8_t* weight,
+                                 const int8_t* bias, int N, int C, int H, int W, int O, int KH,
+                                 int KW, int stride_h, int stride_w, int pad_h, int pad_w,
+                                 int dilate_h, int dilate_w, const float* min_data,
+                                 const float* max_data, const float* min_weight,
+                                 const float* max_weight, const float* min_bias,
+                                 const float* max_bias, int32_t* out32, float* omin, float* omax,
+                                 void* workspace, size_t workspace_bytes, int cfg) {
+  MXQ_API_BEGIN();
+  conv_nchw(stream, data, weight, bias, N, C, H, W, O, KH, KW, stride_h, stride_w, pad_h, pad_w,
+            dilate_h, dilate_w, min_data, max_data, min_weight, max_weight, min_bias, max_bias,
+            out32, omin, omax, workspace, workspace_bytes, cfg);
+  MXQ_API_END();
+}
+
+}  // extern "C"

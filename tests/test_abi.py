@@ -21,7 +21,7 @@ def test_hip_library_exports_every_declared_symbol():
     for n in names:
         assert hasattr(lib, n), n
         assert n in mxnet_amd._lib.SIGNATURES, "no ctypes signature for " + n
-    assert mxnet_amd._lib.lib.mxq_abi_version() == 2
+    assert mxnet_amd._lib.lib.mxq_abi_version() == 3
     assert mxnet_amd._lib.last_error() == ""
 
 

@@ -1,0 +1,149 @@
+"""Parity of mxq_quantized_conv_nchw (the convolution on the operator's own NCHW / OIHW
+tensors, int32 NCHW out) with the CPU oracle: the 1x1 kernel that reads channel planes with
+the transposing LDS load, its strided form, and the adapter route behind the same call."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from tests.data_gen import int8_uniform
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def capi():
+    import mxnet_amd
+    return mxnet_amd.capi
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def f32(v):
+    return dev(np.array([v], np.float32))
+
+
+def run(capi, case, use_bias, cfg=None, guard=True):
+    N, C, H, W, O, KH, KW, s, p, dl = case
+    d = int8_uniform((N, C, H, W), seed=sum(case))
+    w = int8_uniform((O, C, KH, KW), seed=sum(case) + 1)
+    b = int8_uniform((O,), seed=O) if use_bias else None
+    rd, rw, rb = 3.0, 0.2, 1.5
+    eh, ew = dl * (KH - 1) + 1, dl * (KW - 1) + 1
+    OH, OW = (H + 2 * p - eh) // s + 1, (W + 2 * p - ew) // s + 1
+    # the output sits between two guard bands that must come back untouched
+    n_out = N * O * OH * OW
+    flat = torch.full((n_out + 512,), 0x5A5A5A5A, dtype=torch.int32, device="cuda")
+    out = flat[256:256 + n_out].view(N, O, OH, OW)
+    res = capi.quantized_conv_nchw(dev(d), dev(w), None if b is None else dev(b), f32(-rd),
+                                   f32(rd), f32(-rw), f32(rw), None if b is None else f32(-rb),
+                                   None if b is None else f32(rb), stride=(s, s), pad=(p, p),
+                                   dilate=(dl, dl), cfg=cfg, out=out)
+    ro, rmn, rmx = oracle.quantized_conv(d, w, b, -rd, rd, -rw, rw, None if b is None else -rb,
+                                         None if b is None else rb, (s, s), (p, p), (dl, dl))
+    np.testing.assert_array_equal(res["out32"].cpu().numpy(), ro)
+    assert (res["omin"].item(), res["omax"].item()) == (rmn, rmx)
+    g = flat.cpu().numpy()
+    assert (g[:256] == 0x5A5A5A5A).all() and (g[256 + n_out:] == 0x5A5A5A5A).all()
+    return res
+
+
+# (N, C, H, W, O, KH, KW, stride, pad, dilate): 1x1 layers whose planes are whole 16-byte runs
+PLANE_CASES = [
+    (2, 64, 56, 56, 64, 1, 1, 1, 0, 1),     # ResNet stage 1: 3136-pixel planes, one K stage
+    (2, 64, 56, 56, 256, 1, 1, 1, 0, 1),
+    (2, 256, 56, 56, 64, 1, 1, 1, 0, 1),    # four K stages
+    (3, 128, 28, 28, 512, 1, 1, 1, 0, 1),   # 784-pixel planes: the last tile is 16 pixels
+    (2, 512, 28, 28, 128, 1, 1, 1, 0, 1),
+    (3, 48, 8, 12, 40, 1, 1, 1, 0, 1),      # K tail (48 of 64 channels), O % 32 != 0, 96 pixels
+    (1, 16, 4, 4, 8, 1, 1, 1, 0, 1),        # one 16-pixel chunk, everything smaller than a tile
+    (5, 80, 16, 16, 136, 1, 1, 1, 0, 1),    # two K stages with a tail, O one past a tile
+]
+
+
+@pytest.mark.parametrize("case", PLANE_CASES)
+@pytest.mark.parametrize("use_bias", [False, True])
+def test_conv_nchw_planes(capi, case, use_bias):
+    res = run(capi, case, use_bias)
+    assert res["workspace_bytes"] == 0  # nothing is copied for a unit-stride 1x1 layer
+
+
+@pytest.mark.parametrize("cfg", [71, 72, 73, 74, 75])
+@pytest.mark.parametrize("case", [PLANE_CASES[2], PLANE_CASES[3], PLANE_CASES[5], PLANE_CASES[7]])
+def test_conv_nchw_every_plane_tile(capi, cfg, case):
+    run(capi, case, True, cfg=cfg)
+
+
+STRIDED_CASES = [
+    (2, 256, 56, 56, 128, 1, 1, 2, 0, 1),   # ResNet downsampling: 28 x 28 = 784 output pixels
+    (2, 256, 56, 56, 512, 1, 1, 2, 0, 1),
+    (2, 32, 16, 24, 48, 1, 1, 2, 0, 1),     # 8 x 12 output
+    (2, 32, 15, 31, 48, 1, 1, 2, 0, 1),     # odd extents: 8 x 16 output, rows off the dword marks
+    (1, 16, 24, 24, 16, 1, 1, 3, 0, 1),     # stride 3: the byte-wise gather
+]
+
+
+@pytest.mark.parametrize("case", STRIDED_CASES)
+def test_conv_nchw_strided_planes(capi, case):
+    res = run(capi, case, True)
+    N, C, H, W, _, _, _, s = case[:8]
+    gathered = N * C * ((H - 1) // s + 1) * ((W - 1) // s + 1)
+    assert res["workspace_bytes"] == (gathered + 255) // 256 * 256  # the pixels it reads, once
+
+
+# everything else goes through the adapters inside the same call
+ADAPTER_CASES = [
+    (3, 4, 28, 28, 128, 3, 3, 1, 1, 1),     # the reference's test shape
+    (2, 64, 56, 56, 64, 3, 3, 1, 1, 1),
+    (2, 128, 28, 28, 128, 3, 3, 1, 1, 1),
+    (2, 256, 14, 14, 1024, 1, 1, 1, 0, 1),  # 196-pixel planes: 1x1 weights used in place
+    (2, 1024, 14, 14, 512, 1, 1, 2, 0, 1),  # 49-pixel output planes
+    (1, 512, 7, 7, 2048, 1, 1, 1, 0, 1),
+    (1, 3, 32, 32, 16, 7, 7, 2, 3, 1),      # stem: space-to-depth route
+    (2, 20, 9, 11, 36, 5, 3, 1, 2, 1),      # C % 16 != 0
+    (2, 24, 8, 8, 32, 1, 1, 1, 0, 1),       # 1x1 with C % 16 != 0
+    (2, 16, 8, 8, 32, 1, 1, 1, 1, 1),       # padded 1x1
+    (1, 16, 12, 12, 20, 3, 3, 1, 2, 2),     # dilation
+]
+
+
+@pytest.mark.parametrize("case", ADAPTER_CASES)
+@pytest.mark.parametrize("use_bias", [False, True])
+def test_conv_nchw_other_geometries(capi, case, use_bias):
+    run(capi, case, use_bias)
+
+
+@pytest.mark.parametrize("case", [PLANE_CASES[0], PLANE_CASES[3], STRIDED_CASES[0]])
+def test_conv_nchw_routes_agree(capi, case):
+    """The NCHW kernel and the adapter route (pinned through the test-only entry point)
+    write the same tensor."""
+    a = run(capi, case, True)
+    b = run(capi, case, True, cfg=1)
+    assert torch.equal(a["out32"], b["out32"])
+
+
+def test_conv_nchw_unaligned_operands_take_the_adapters(capi):
+    """A data pointer off the 16-byte marks cannot feed the direct-to-LDS loads."""
+    case = (2, 64, 8, 8, 64, 1, 1, 1, 0, 1)
+    N, C, H, W, O = case[:5]
+    d = int8_uniform((N, C, H, W), seed=1)
+    w = int8_uniform((O, C, 1, 1), seed=2)
+    buf = torch.zeros(d.size + 16, dtype=torch.int8, device="cuda")
+    view = buf[4:4 + d.size].view(N, C, H, W)
+    view.copy_(dev(d))
+    res = capi.quantized_conv_nchw(view, dev(w), None, f32(-1.0), f32(1.0), f32(-1.0), f32(1.0))
+    ro, _, _ = oracle.quantized_conv(d, w, None, -1.0, 1.0, -1.0, 1.0)
+    np.testing.assert_array_equal(res["out32"].cpu().numpy(), ro)
+
+
+def test_conv_nchw_without_images(capi):
+    x = torch.zeros((0, 16, 8, 8), dtype=torch.int8, device="cuda")
+    w = torch.ones((32, 16, 1, 1), dtype=torch.int8, device="cuda")
+    res = capi.quantized_conv_nchw(x, w, None, f32(-1.0), f32(1.0), f32(-0.5), f32(0.5))
+    _, rmn, rmx = oracle.quantized_conv(np.zeros((0, 16, 8, 8), np.int8),
+                                        np.ones((32, 16, 1, 1), np.int8), None, -1.0, 1.0, -0.5,
+                                        0.5)
+    assert tuple(res["out32"].shape) == (0, 32, 8, 8)
+    assert (res["omin"].item(), res["omax"].item()) == (rmn, rmx)
