@@ -90,7 +90,8 @@ def parse_args():
                              "requantize", "requantize_uncal", "dequantize", "copy", "maxpool", "avgpool",
                              "elemwise_add", "elemwise_add_int8", "concat", "elemwise_mul_int8", "quantize_asym",
                              "batch_norm", "embedding", "transpose", "transpose_to_nhwc", "transpose_to_nchw",
-                             "resnet50_convs", "resnet50_convs_operator", "resnet50_chain",
+                             "resnet50_convs", "resnet50_convs_operator",
+                             "resnet50_convs_operator_adapters", "resnet50_chain",
                              "resnet50_chain_fused", "resnet50_chain_unfused",
                              "bert_fc_chain",
                              "bert_fc_chain_fused",
@@ -783,15 +784,17 @@ class ConvStackWorkload(GraphWorkload):
 
 class ConvOperatorWorkload(GraphWorkload):
     """The same 19 ResNet-50 layers at batch 64 under the reference operator's own contract
-    (quantized_conv.cu:101-219): NCHW int8 data and OIHW int8 weights in, NCHW int32 out.  Per
-    layer: both operands brought to NHWC (the two TransposeImpl calls of the reference), then
-    the convolution whose epilogue writes int32 channel planes (no third transpose)."""
+    (quantized_conv.cu:101-219): NCHW int8 data and OIHW int8 weights in, NCHW int32 out,
+    through mxq_quantized_conv_nchw, the one call the registered _contrib_quantized_conv
+    makes.  `route` pins every layer to one route through the test-only entry point
+    (1 = the layout adapters, as the reference's two TransposeImpl calls)."""
 
-    def __init__(self, torch, capi, lib):
-        self.kernel = "transpose_i8 kernels + conv / fc kernels (int32 NCHW out)"
+    def __init__(self, torch, capi, lib, route=0):
+        self.kernel = "conv1x1_planes_kernel (NCHW 1x1) + adapters / conv_dma_kernel (3x3, small planes), int32 NCHW out"
         self.bound = "mfma"
         self.name = "ResNet-50 v1 bottleneck conv stack (19 distinct layers), batch 64, as the " \
-                    "operator sees it: NCHW int8 in, layout adapters, NCHW int32 out"
+                    "operator sees it: NCHW int8 in, NCHW int32 out" + \
+                    (" (every layer through the layout adapters)" if route == 1 else "")
         P = lambda t: ctypes.c_void_p(t.data_ptr())
         g = torch.Generator(device="cuda").manual_seed(4)
         N = 64
@@ -803,26 +806,26 @@ class ConvOperatorWorkload(GraphWorkload):
             d = torch.randint(-127, 128, (N, C, H, H), device="cuda", generator=g, dtype=torch.int8)
             w = torch.randint(-127, 128, (O, C, k, k), device="cuda", generator=g, dtype=torch.int8)
             b = torch.randint(-127, 128, (O,), device="cuda", generator=g, dtype=torch.int8)
-            dn = torch.empty((N, H, H, C), dtype=torch.int8, device="cuda")
-            wn = torch.empty((O, k, k, C), dtype=torch.int8, device="cuda")
             out = torch.empty((N, O, OH, OH), dtype=torch.int32, device="cuda")
             sc = [torch.empty(1, device="cuda") for _ in range(2)]
-            nws = lib.mxq_quantized_conv_workspace(N, H, H, C, O, k, k, s, s, pad, pad, 1, 1, 0)
+            geo = (N, C, H, H, O, k, k, s, s, pad, pad, 1, 1)
+            nws = lib.mxq_quantized_conv_nchw_workspace(*geo, 0 if route == 1 else 1)
             ws = torch.empty(nws, dtype=torch.uint8, device="cuda") if nws else None
-            self.layers.append((d, w, b, dn, wn, out, sc, (N, H, H, C, O, k, k, s, s, pad, pad), ws))
+            self.layers.append((d, w, b, out, sc, geo, ws))
             self.ops += 2.0 * N * OH * OH * O * k * k * C
 
         def body(only=None):
             st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
-            for i, (d, w, b, dn, wn, out, sc, geo, ws) in enumerate(self.layers):
+            for i, (d, w, b, out, sc, geo, ws) in enumerate(self.layers):
                 if only is not None and i != only:
                     continue
-                N_, H_, W_, C_, O_, k_ = geo[0], geo[1], geo[2], geo[3], geo[4], geo[5]
-                rc = lib.mxq_nchw_to_nhwc_pad_i8(st, P(d), P(dn), N_, C_, H_, W_, C_)
-                rc = rc or lib.mxq_nchw_to_nhwc_pad_i8(st, P(w), P(wn), O_, C_, k_, k_, C_)
-                rc = rc or lib.mxq_quantized_conv_nhwc_out_nchw(
-                    st, P(dn), P(wn), P(b), *geo, 1, 1, P(one[0]), P(one[1]), P(one[0]),
-                    P(one[1]), P(one[0]), P(one[1]), P(out), P(sc[0]), P(sc[1]), *ws_args(ws))
+                args = [st, P(d), P(w), P(b)] + list(geo) + [
+                    P(one[0]), P(one[1]), P(one[0]), P(one[1]), P(one[0]), P(one[1]), P(out),
+                    P(sc[0]), P(sc[1])] + list(ws_args(ws))
+                if route == 0:
+                    rc = lib.mxq_quantized_conv_nchw(*args)
+                else:
+                    rc = lib.mxq_test_quantized_conv_nchw(*args, route)
                 if rc != 0:
                     raise RuntimeError(lib.mxq_last_error().decode())
         self.body = body
@@ -1178,6 +1181,8 @@ def make_workload(name, torch, capi, lib):
         return ConvStackWorkload(torch, capi, lib)
     if name == "resnet50_convs_operator":
         return ConvOperatorWorkload(torch, capi, lib)
+    if name == "resnet50_convs_operator_adapters":
+        return ConvOperatorWorkload(torch, capi, lib, route=1)
     if name == "resnet50_chain":
         return ResNetChainWorkload(torch, capi, lib)
     if name == "resnet50_chain_fused":

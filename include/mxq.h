@@ -376,15 +376,17 @@ int mxq_quantized_conv_nhwc_out_nchw(void* stream, const int8_t* data, const int
  * [O,C,KH,KW], bias int8 [O] or NULL, out32 int32 [N,O,OH,OW] -- everything
  * QuantizedCuDNNConvOp::Forward does between its inputs and its outputs
  * (src/operator/quantization/quantized_conv.cu:101-219, layout rule quantized_conv.cc:38-45),
- * the three TransposeImpl calls included (:145-148,183).  1 x 1 convolutions over planes of
- * 16 | OH*OW bytes and 16 | C channels run on the NCHW tensors as they are (strided ones
- * after their used pixels were gathered into the workspace); every other geometry goes
- * through the layout adapters and mxq_quantized_conv_nhwc_out_nchw inside this call.
+ * the three TransposeImpl calls included (:145-148,183).  Unpadded 1 x 1 convolutions over
+ * 16 | C channels never leave the channel-plane layout and need no workspace (strided ones
+ * and planes that are no multiple of 16 bytes through a gathering loader in the same
+ * kernel); every other geometry goes through the layout adapters and
+ * mxq_quantized_conv_nhwc_out_nchw inside this call.
  * `workspace` (16-byte aligned) must hold mxq_quantized_conv_nchw_workspace() bytes: the
  * operator's kTempSpace (quantized_conv.cu:121-160 asks for three tensor copies plus
- * cuDNN's workspace there; 0 here for a unit-stride 1 x 1 layer).  operands_aligned16 != 0
+ * cuDNN's workspace there; 0 here for an unpadded 1 x 1 layer).  operands_aligned16 != 0
  * says that data and weight both start on 16-byte marks, as a framework's allocations do;
- * with 0 the query returns what the adapter route needs, which every geometry can take. */
+ * with 0 the query returns enough for the adapter route as well, which every geometry and
+ * alignment can take. */
 size_t mxq_quantized_conv_nchw_workspace(int N, int C, int H, int W, int O, int KH, int KW,
                                          int stride_h, int stride_w, int pad_h, int pad_w,
                                          int dilate_h, int dilate_w, int operands_aligned16);

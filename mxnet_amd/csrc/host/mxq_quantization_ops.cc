@@ -638,8 +638,8 @@ static void QuantizedFullyConnectedForwardGPU(const NodeAttrs& attrs, const OpCo
 
 // Temp space of the convolution: what mxq_quantized_conv_nchw wants for the geometry.  The
 // reference asks for NHWC copies of data, weight and output plus cuDNN's workspace
-// (quantized_conv.cu:121-160); here a unit-stride 1x1 layer runs on the NCHW tensors as
-// they are and needs none, a strided 1x1 layer the pixels it reads, every other geometry
+// (quantized_conv.cu:121-160); here an unpadded 1x1 layer over 16 | C channels runs on the
+// NCHW tensors as they are and needs none, every other geometry
 // the two operand copies (channels zero-padded to a multiple of 16 on the way) and, for
 // few tiles under a long reduction, the split-K partial sums.
 static size_t QuantizedConvTempBytes(const ConvolutionParam& param, const TShape& d,

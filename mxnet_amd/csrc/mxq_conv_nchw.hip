@@ -18,10 +18,14 @@
 // writes two 128-byte runs of two channel planes: the int32 output goes to its NCHW place
 // straight from the accumulators.  No adapter launch, no second copy of any tensor.
 //
-// Strided 1 x 1 convolutions first gather the pixels they use into a compact NCHW tensor
-// (a quarter of the input for stride 2) in the caller's workspace and then run the same
-// kernel.  Everything else (3 x 3, padded, planes whose size is no multiple of 16 bytes)
-// takes the NHWC kernels of mxq_conv.hip behind the layout adapters.
+// Strided 1 x 1 convolutions, and planes whose size is no multiple of 16 bytes (14 x 14,
+// 7 x 7), run in the same kernel with a gathering loader: a thread fetches the four pixels
+// of its LDS dword from wherever the stride puts them (one 8-byte load and a v_perm for
+// stride 2 over rows of 4 | OW pixels, the plane's own dwords for unit stride, bytes
+// otherwise) and the operand becomes the matrix [C][N * OH * OW] whose pixel tiles run
+// across image boundaries.  No workspace, no pre-pass: a strided layer reads only the
+// cache lines it uses.  Everything else (3 x 3, padded 1 x 1, C % 16 != 0) takes the NHWC
+// kernels of mxq_conv.hip behind the layout adapters.
 #include <hip/hip_runtime.h>
 
 #include <cmath>
@@ -35,17 +39,25 @@
 namespace mxq {
 namespace {
 
+// The activation operand as rows of one channel each.  GM == 0 (native): image n, channel
+// c, pixel p at data[n * img_stride + c * row_stride + p], planes of 16 | P bytes read as they
+// lie, pixel tiles inside one image.  GM != 0 (gathered): the operand is the matrix
+// [C][N * P] whose column n * P + oh * OW + ow is input pixel (oh * sh, ow * sw) of image n --
+// what a strided layer reads, or a plane whose size is no multiple of 16 -- and pixel tiles
+// run over the columns regardless of where one image ends.
 struct PlaneArgs {
-  const int8_t* data;    // [N][C][P]
+  const int8_t* data;
   const int8_t* weight;  // [O][C]
-  int N, C, P, O;
-  int tiles_p, tiles_o;
+  int N, C, P, O;        // P = output pixels per image
+  int img_stride, row_stride;   // native
+  int H, W, OW, sh, sw;         // gathered: input plane, output row length, strides
+  uint32_t data_bytes;   // extent of the activation tensor
+  int tiles_p, tiles_o;  // pixel tiles (per image if native, per matrix if gathered), channel tiles
   Epilogue epi;          // bias, input ranges, out32 ([N][O][P]), omin / omax
 };
 
-// Tile of BP pixels of one image x BO output channels; BK channels per stage.  The names
-// CH / BK / kThreads are what DmaLane and RowIssuerBuffer (mxq_gemm.h) read for the weight
-// operand.
+// Tile of BP pixels x BO output channels; BK channels per stage.  The names CH / BK /
+// kThreads are what DmaLane and RowIssuerBuffer (mxq_gemm.h) read for the weight operand.
 template <int BP_, int BO_, int BK_, int WP_, int WO_>
 struct PlaneCfg {
   static constexpr int BP = BP_, BO = BO_, BK = BK_, WP = WP_, WO = WO_;
@@ -57,20 +69,27 @@ struct PlaneCfg {
   static constexpr int A_SLOTS = BK * CHP, B_SLOTS = BO * CH;
   static constexpr int STAGE_SLOTS = A_SLOTS + B_SLOTS;
   static constexpr int A_INSTR = A_SLOTS / (64 * NW), B_INSTR = B_SLOTS / (64 * NW);
+  // gathered operand: a thread owns one group of 4 consecutive pixels (one LDS dword per
+  // channel) and every TPG-th channel of a stage
+  static constexpr int GROUPS = BP / 4, TPG = kThreads / GROUPS, CPS = BK / TPG;
   static_assert(BP % (32 * WP) == 0 && BO % (32 * WO) == 0, "wave tile");
   static_assert(A_SLOTS % (64 * NW) == 0 && B_SLOTS % (64 * NW) == 0, "loader");
-  static_assert(CHP == 4 || CHP == 8, "pixel-chunk swizzle");
+  static_assert(CHP == 4 || CHP == 8 || CHP == 16, "pixel-chunk swizzle");
   static_assert(CH == 4 || CH == 8, "fragment addressing of the weight operand");
+  static_assert(kThreads % GROUPS == 0 && BK % TPG == 0 && TPG % 8 == 0,
+                "gathering loader: a thread's channels share their low three bits");
 };
 
 // Where pixel chunk pc of channel row c sits in its row: pc ^ plane_swz(c).  A transposing
 // read touches, per 16 lanes, one 16-byte chunk of 8 consecutive rows, and two such groups
 // (chunks pc and pc + 1, pc even) go through the LDS together: the XOR makes those 16
 // pieces hit 16 different bank groups.  Rows of 128 bytes: the row's low three bits; rows
-// of 64 bytes (four rows per 256 bytes of banks): bit 2 of the row moves the chunk by two.
+// of 64 bytes (four rows per 256 bytes of banks): bit 2 of the row moves the chunk by two;
+// rows of 256 bytes (every row on the same banks): twice the row's low three bits, so that
+// one group takes the even and the other the odd chunks.
 template <int CHP>
 __device__ __forceinline__ int plane_swz(int c) {
-  return CHP == 8 ? (c & 7) : ((c >> 1) & 2);
+  return CHP == 8 ? (c & 7) : (CHP == 16 ? 2 * (c & 7) : ((c >> 1) & 2));
 }
 
 typedef int v2i __attribute__((ext_vector_type(2)));
@@ -80,13 +99,20 @@ __device__ __forceinline__ v2i lds_read_tr8(const char* p) {
       (v2i __attribute__((address_space(3)))*)(p));
 }
 
-template <class Cfg, int NS>
+// How a gathered operand's four pixels of a group are fetched.
+constexpr int kNative = 0;      // not gathered: 16-byte direct-to-LDS loads
+constexpr int kGatherDword = 1; // unit stride, planes on dword marks: the plane's own dwords
+constexpr int kGatherPair = 2;  // sw == 2, 4 | OW, rows on 8-byte marks: 8 bytes and a v_perm
+constexpr int kGatherBytes = 3; // anything else: byte by byte
+
+template <class Cfg, int NS, int GM>
 __global__ __launch_bounds__(Cfg::kThreads, 2) void conv1x1_planes_kernel(PlaneArgs p) {
   constexpr int BP = Cfg::BP, BK = Cfg::BK, CHP = Cfg::CHP, CH = Cfg::CH, NW = Cfg::NW;
   constexpr int MI = Cfg::MI, NI = Cfg::NI, KS = Cfg::KS;
-  constexpr int AI = Cfg::A_INSTR, BI = Cfg::B_INSTR, CPT = AI + BI;
+  constexpr int AI = GM == kNative ? Cfg::A_INSTR : 0, BI = Cfg::B_INSTR, CPT = AI + BI;
   constexpr int STAGE_BYTES = Cfg::STAGE_SLOTS * 16, A_BYTES = Cfg::A_SLOTS * 16;
   static_assert((NS - 2) * CPT < 64, "vmcnt range");
+  static_assert(GM == kNative || NS == 2, "the gathering loader works one stage ahead");
   __shared__ __attribute__((aligned(16))) v4i lds[NS * Cfg::STAGE_SLOTS];
   __shared__ __attribute__((aligned(16))) int sbias[Cfg::BO];
   const int tid = threadIdx.x, lane = tid & 63;
@@ -95,28 +121,34 @@ __global__ __launch_bounds__(Cfg::kThreads, 2) void conv1x1_planes_kernel(PlaneA
 
   // tile order: the output-channel tiles of one pixel slab are neighbours, and the
   // round-robin of work-group ids over the XCDs is undone so that they meet in one L2
-  const int total = p.N * p.tiles_p * p.tiles_o;
+  constexpr bool gathered = GM != kNative;
+  const int images = gathered ? 1 : p.N;
+  const int total = images * p.tiles_p * p.tiles_o;
   const int lid = xcd_remap(blockIdx.x, total);
   const int to = lid % p.tiles_o;
   const int rest = lid / p.tiles_o;
   const int tp = rest % p.tiles_p, n = rest / p.tiles_p;
   const int p0 = tp * BP, o0 = to * Cfg::BO;
+  const int KT = (p.C + BK - 1) / BK;
+  const uint32_t lds0 = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(lds));
 
-  // activation loads: slot q of a stage (16 bytes) = channel row q / CHP, chunk q % CHP
-  const v4i arsrc = make_rsrc(p.data, static_cast<uint32_t>(p.N) * p.C * p.P);
-  uint32_t a_off[AI];
-  int a_c[AI];
+  // native activation loads: slot q of a stage (16 bytes) = channel row q / CHP, chunk q % CHP
+  const v4i arsrc = make_rsrc(p.data, p.data_bytes);
+  uint32_t a_off[AI > 0 ? AI : 1];
+  int a_c[AI > 0 ? AI : 1];
+  if constexpr (!gathered) {
 #pragma unroll
-  for (int j = 0; j < AI; ++j) {
-    const int q = (j * NW + wave) * 64 + lane;
-    const int c = q / CHP, pc = (q % CHP) ^ plane_swz<CHP>(c);
-    a_c[j] = c;
-    a_off[j] = (static_cast<uint32_t>(n) * p.C + c) * p.P + p0 + pc * 16;
+    for (int j = 0; j < AI; ++j) {
+      const int q = (j * NW + wave) * 64 + lane;
+      const int c = q / CHP, pc = (q % CHP) ^ plane_swz<CHP>(c);
+      a_c[j] = c;
+      a_off[j] = static_cast<uint32_t>(n) * p.img_stride +
+                 static_cast<uint32_t>(c) * p.row_stride + p0 + pc * 16;
+    }
   }
   RowIssuerBuffer<Cfg, BI> bi;
   bi.init(p.weight, o0, p.O, p.C, wave, lane, 0);
-  const uint32_t lds0 = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(lds));
-  const int KT = (p.C + BK - 1) / BK;
+  // direct-to-LDS loads of a stage: the weights, and the native activation slab
   auto issue = [&](int stage) {
     if (stage >= KT) return;
     const uint32_t sb = lds0 + static_cast<uint32_t>(stage % NS) * STAGE_BYTES;
@@ -124,11 +156,63 @@ __global__ __launch_bounds__(Cfg::kThreads, 2) void conv1x1_planes_kernel(PlaneA
     for (int j = 0; j < AI; ++j) {
       const int c = stage * BK + a_c[j];
       const uint32_t off =
-          c < p.C ? a_off[j] + static_cast<uint32_t>(stage * BK) * p.P : kOutOfRange;
+          c < p.C ? a_off[j] + static_cast<uint32_t>(stage * BK) * p.row_stride : kOutOfRange;
       dma_buffer(sb + (j * NW + wave) * 1024, off, arsrc);
     }
 #pragma unroll
     for (int j = 0; j < BI; ++j) bi.issue(j, stage, sb + A_BYTES + (j * NW + wave) * 1024);
+  };
+
+  // gathered activation loads: this thread's pixel group and first channel of a stage
+  constexpr int CPS = Cfg::CPS, TPG = Cfg::TPG;
+  const int grp = tid % Cfg::GROUPS, cs = tid / Cfg::GROUPS;
+  const int plane_in = p.H * p.W;
+  int goff[4] = {0, 0, 0, 0};   // byte offsets of the group's pixels in channel 0 of the tensor
+  if constexpr (gathered) {
+    const long long V = 1LL * p.N * p.P;
+#pragma unroll
+    for (int j = 0; j < (GM == kGatherBytes ? 4 : 1); ++j) {
+      const long long v = 1LL * p0 + 4 * grp + j;
+      const int vv = v < V ? static_cast<int>(v) : 0;   // columns past the end read pixel 0
+      const int img = vv / p.P, px = vv - img * p.P;
+      const int oh = px / p.OW, ow = px - oh * p.OW;
+      goff[j] = img * p.C * plane_in + oh * p.sh * p.W + ow * p.sw;
+    }
+  }
+  uint32_t areg[gathered ? CPS : 1];
+  auto gather = [&](int stage) {
+    if constexpr (gathered) {
+#pragma unroll
+      for (int i = 0; i < CPS; ++i) {
+        int c = stage * BK + cs + TPG * i;
+        c = c < p.C ? c : p.C - 1;   // the weights' zero K tail cancels whatever these rows hold
+        const int8_t* row = p.data + static_cast<size_t>(c) * plane_in;
+        if (GM == kGatherDword) {
+          areg[i] = *reinterpret_cast<const uint32_t*>(row + goff[0]);
+        } else if (GM == kGatherPair) {
+          typedef uint32_t u2 __attribute__((ext_vector_type(2)));
+          const u2 w = *reinterpret_cast<const u2*>(row + goff[0]);
+          areg[i] = __builtin_amdgcn_perm(w.y, w.x, 0x06040200u);
+        } else {
+          const uint32_t b0 = static_cast<uint8_t>(row[goff[0]]);
+          const uint32_t b1 = static_cast<uint8_t>(row[goff[1]]);
+          const uint32_t b2 = static_cast<uint8_t>(row[goff[2]]);
+          const uint32_t b3 = static_cast<uint8_t>(row[goff[3]]);
+          areg[i] = b0 | (b1 << 8) | (b2 << 16) | (b3 << 24);
+        }
+      }
+    }
+  };
+  // LDS dword of (channel row cs + TPG * i, pixel group grp): TPG is a multiple of 8, so the
+  // row's swizzle is that of cs for every i
+  const int gslot = cs * BP + ((((grp >> 2) ^ plane_swz<CHP>(cs))) << 4) + ((grp & 3) << 2);
+  auto stash = [&](int stage) {
+    if constexpr (gathered) {
+      char* sa = reinterpret_cast<char*>(lds) + (stage % NS) * STAGE_BYTES;
+#pragma unroll
+      for (int i = 0; i < CPS; ++i)
+        *reinterpret_cast<uint32_t*>(sa + gslot + TPG * i * BP) = areg[i];
+    }
   };
 
   // fragment addresses.  Activation: lane = 16 * G + s reads 8 bytes of channel row
@@ -157,17 +241,7 @@ __global__ __launch_bounds__(Cfg::kThreads, 2) void conv1x1_planes_kernel(PlaneA
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[mi][ni][v] = 0;
 
-#pragma unroll
-  for (int st = 0; st < NS - 1; ++st) issue(st);
-  // what the epilogue needs, behind the first operand fetch
-  const EpiScalars es = epi_scalars(p.epi);
-  if (tid < Cfg::BO) sbias[tid] = (o0 + tid < p.O) ? epi_bias32(p.epi, es, o0 + tid) : 0;
-
-  for (int kt = 0; kt < KT; ++kt) {
-    const int newest = (kt + NS - 2) < (KT - 1) ? (kt + NS - 2) : (KT - 1);
-    wait_ahead<CPT, NS - 2>(newest - kt);
-    __builtin_amdgcn_s_barrier();
-    issue(kt + NS - 1);
+  auto compute = [&](int kt) {
     const char* sa = reinterpret_cast<const char*>(lds) + (kt % NS) * STAGE_BYTES;
     const v4i* sbw = reinterpret_cast<const v4i*>(sa + A_BYTES);
 #pragma unroll
@@ -187,15 +261,65 @@ __global__ __launch_bounds__(Cfg::kThreads, 2) void conv1x1_planes_kernel(PlaneA
         for (int ni = 0; ni < NI; ++ni)
           acc[mi][ni] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fb[ni], fa[mi], acc[mi][ni], 0, 0, 0);
     }
+  };
+
+  if constexpr (!gathered) {
+#pragma unroll
+    for (int st = 0; st < NS - 1; ++st) issue(st);
+  } else {
+    gather(0);
+    issue(0);
+  }
+  // what the epilogue needs, behind the first operand fetch
+  const EpiScalars es = epi_scalars(p.epi);
+  if (tid < Cfg::BO) sbias[tid] = (o0 + tid < p.O) ? epi_bias32(p.epi, es, o0 + tid) : 0;
+
+  if constexpr (!gathered) {
+    for (int kt = 0; kt < KT; ++kt) {
+      const int newest = (kt + NS - 2) < (KT - 1) ? (kt + NS - 2) : (KT - 1);
+      wait_ahead<CPT, NS - 2>(newest - kt);
+      __builtin_amdgcn_s_barrier();
+      issue(kt + NS - 1);
+      compute(kt);
+    }
+  } else {
+    // one stage ahead: the registers and the weights' direct loads of stage kt + 1 are on
+    // their way while stage kt is multiplied; both have landed (vmcnt counts them together)
+    // before the registers go to LDS and the barrier publishes the stage
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    stash(0);
+    __syncthreads();
+    for (int kt = 0; kt < KT; ++kt) {
+      if (kt + 1 < KT) {
+        gather(kt + 1);
+        issue(kt + 1);
+      }
+      compute(kt);
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      if (kt + 1 < KT) stash(kt + 1);
+      __syncthreads();
+    }
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   if (blockIdx.x == 0 && tid == 0) epilogue_ranges(p.epi);
-  __syncthreads();  // sbias (written before the loop; K = 0 would skip its barriers)
+  __syncthreads();  // sbias
 
   // lane = pixel, register = channel 8 * (v / 4) + 4 * (lane / 32) + v % 4 of the MFMA
-  // tile: a store instruction writes 32 consecutive int32 of two channel planes
-  const int px_base = p0 + wp * Cfg::TP + frow;
-  int32_t* out_img = p.epi.out32 + static_cast<size_t>(n) * p.O * p.P;
+  // tile: a store instruction writes 32 consecutive int32 of two channel planes (fewer
+  // where a gathered tile passes from one image to the next)
+  size_t obase[MI];   // offset of (image, channel 0, pixel) in out32
+  bool ovalid[MI];
+#pragma unroll
+  for (int mi = 0; mi < MI; ++mi) {
+    const int v = p0 + wp * Cfg::TP + 32 * mi + frow;
+    int img = n, px = v;
+    if (gathered) {
+      img = v / p.P;
+      px = v - img * p.P;
+    }
+    ovalid[mi] = img < p.N && px < p.P;
+    obase[mi] = static_cast<size_t>(img) * p.O * p.P + px;
+  }
 #pragma unroll
   for (int ni = 0; ni < NI; ++ni) {
 #pragma unroll
@@ -206,13 +330,12 @@ __global__ __launch_bounds__(Cfg::kThreads, 2) void conv1x1_planes_kernel(PlaneA
       for (int i = 0; i < 4; ++i) {
         const int o = o0 + ol + i;
         if (o < p.O) {
-          int32_t* plane = out_img + static_cast<size_t>(o) * p.P;
+          int32_t* plane = p.epi.out32 + static_cast<size_t>(o) * p.P;
 #pragma unroll
           for (int mi = 0; mi < MI; ++mi) {
-            const int px = px_base + 32 * mi;
-            if (px < p.P)
-              plane[px] = static_cast<int>(static_cast<uint32_t>(acc[mi][ni][4 * vq + i]) +
-                                           static_cast<uint32_t>(b[i]));
+            if (ovalid[mi])
+              plane[obase[mi]] = static_cast<int>(static_cast<uint32_t>(acc[mi][ni][4 * vq + i]) +
+                                                  static_cast<uint32_t>(b[i]));
           }
         }
       }
@@ -220,80 +343,43 @@ __global__ __launch_bounds__(Cfg::kThreads, 2) void conv1x1_planes_kernel(PlaneA
   }
 }
 
-// out[b][oh][ow] = in[b][oh * sh][ow * sw] over B = N * C planes: the pixels a strided
-// 1 x 1 convolution without padding reads, compacted.  FAST: sw == 2, 4 | OW and rows on
-// dword marks, a thread makes one dword of output from two of input.
-template <bool FAST>
-__global__ __launch_bounds__(256) void subsample_planes_kernel(const uint8_t* __restrict__ in,
-                                                               uint8_t* __restrict__ out, int H,
-                                                               int W, int OH, int OW, int sh,
-                                                               int sw, size_t items) {
-  const size_t stride = static_cast<size_t>(gridDim.x) * 256;
-  for (size_t i = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x; i < items; i += stride) {
-    if (FAST) {
-      const int q = OW / 4;
-      const int x = static_cast<int>(i % q);
-      const size_t t = i / q;
-      const int oh = static_cast<int>(t % OH);
-      const size_t b = t / OH;
-      const uint8_t* src = in + (b * H + static_cast<size_t>(oh) * sh) * W + 8 * x;
-      const uint32_t lo = *reinterpret_cast<const uint32_t*>(src);
-      const uint32_t hi = *reinterpret_cast<const uint32_t*>(src + 4);
-      // bytes 0 and 2 of each dword
-      const uint32_t v = __builtin_amdgcn_perm(hi, lo, 0x06040200u);
-      *reinterpret_cast<uint32_t*>(out + (b * OH + oh) * OW + 4 * x) = v;
-    } else {
-      const int ow = static_cast<int>(i % OW);
-      const size_t t = i / OW;
-      const int oh = static_cast<int>(t % OH);
-      const size_t b = t / OH;
-      out[i] = in[(b * H + static_cast<size_t>(oh) * sh) * W + static_cast<size_t>(ow) * sw];
-    }
-  }
-}
-
-void launch_subsample(hipStream_t s, const int8_t* in, int8_t* out, long long planes, int H,
-                      int W, int OH, int OW, int sh, int sw) {
-  const bool fast = sw == 2 && OW % 4 == 0 && W % 4 == 0 &&
-                    (reinterpret_cast<uintptr_t>(in) & 3u) == 0 &&
-                    (reinterpret_cast<uintptr_t>(out) & 3u) == 0 && 8 * (OW / 4) <= W;
-  const size_t items = static_cast<size_t>(planes) * OH * (fast ? OW / 4 : OW);
-  if (items == 0) return;
-  size_t grid = (items + 255) / 256;
-  const size_t cap = static_cast<size_t>(num_cus()) * 16;
-  if (grid > cap) grid = cap;
-  if (fast)
-    hipLaunchKernelGGL(subsample_planes_kernel<true>, dim3(static_cast<unsigned>(grid)),
-                       dim3(256), 0, s, reinterpret_cast<const uint8_t*>(in),
-                       reinterpret_cast<uint8_t*>(out), H, W, OH, OW, sh, sw, items);
-  else
-    hipLaunchKernelGGL(subsample_planes_kernel<false>, dim3(static_cast<unsigned>(grid)),
-                       dim3(256), 0, s, reinterpret_cast<const uint8_t*>(in),
-                       reinterpret_cast<uint8_t*>(out), H, W, OH, OW, sh, sw, items);
-  MXQ_LAUNCH_CHECK();
-}
-
 typedef PlaneCfg<128, 128, 64, 2, 2> PlaneM;   // 4 waves, wave tile 64 pixels x 64 channels
 typedef PlaneCfg<128, 64, 64, 2, 2> PlaneN64;  // 4 waves, wave tile 64 x 32
 typedef PlaneCfg<64, 128, 64, 2, 2> PlaneP64;  // 4 waves, wave tile 32 x 64
 typedef PlaneCfg<64, 64, 64, 2, 2> PlaneS;     // 4 waves, wave tile 32 x 32
 typedef PlaneCfg<128, 256, 64, 2, 4> PlaneW;   // 8 waves, wave tile 64 x 64
+typedef PlaneCfg<256, 128, 64, 4, 2> PlaneH;   // 8 waves, wave tile 64 x 64
+typedef PlaneCfg<256, 256, 64, 2, 4> PlaneL;   // 8 waves, wave tile 128 x 64
 
 template <class Cfg>
-void launch_planes(hipStream_t s, PlaneArgs a) {
-  a.tiles_p = (a.P + Cfg::BP - 1) / Cfg::BP;
+void launch_planes(hipStream_t s, PlaneArgs a, int gm) {
+  const long long cols = gm != kNative ? 1LL * a.N * a.P : a.P;
+  a.tiles_p = static_cast<int>((cols + Cfg::BP - 1) / Cfg::BP);
   a.tiles_o = (a.O + Cfg::BO - 1) / Cfg::BO;
-  const long long total = 1LL * a.N * a.tiles_p * a.tiles_o;
+  const long long total = 1LL * (gm != kNative ? 1 : a.N) * a.tiles_p * a.tiles_o;
   MXQ_CHECK(total < (1LL << 31), "grid too large");
-  hipLaunchKernelGGL((conv1x1_planes_kernel<Cfg, 2>), dim3(static_cast<unsigned>(total)),
-                     dim3(Cfg::kThreads), 0, s, a);
+  const dim3 grid(static_cast<unsigned>(total)), block(Cfg::kThreads);
+  if (gm == kGatherDword) {
+    hipLaunchKernelGGL((conv1x1_planes_kernel<Cfg, 2, kGatherDword>), grid, block, 0, s, a);
+  } else if (gm == kGatherPair) {
+    hipLaunchKernelGGL((conv1x1_planes_kernel<Cfg, 2, kGatherPair>), grid, block, 0, s, a);
+  } else if (gm == kGatherBytes) {
+    hipLaunchKernelGGL((conv1x1_planes_kernel<Cfg, 2, kGatherBytes>), grid, block, 0, s, a);
+  } else if (a.C <= 2 * Cfg::BK) {
+    // a reduction of up to two stages needs no deeper ring; a longer one is read from HBM
+    // once and wants several stages in flight per work-group
+    hipLaunchKernelGGL((conv1x1_planes_kernel<Cfg, 2, kNative>), grid, block, 0, s, a);
+  } else {
+    hipLaunchKernelGGL((conv1x1_planes_kernel<Cfg, 4, kNative>), grid, block, 0, s, a);
+  }
   MXQ_LAUNCH_CHECK();
 }
 
 // The route a convolution takes.
 enum class Route {
-  kPlanes,        // 1 x 1, unit stride: the NCHW kernel on the operator's own tensors
-  kPlanesStrided, // 1 x 1, strided: gather the used pixels, then the NCHW kernel
+  kPlanes,        // 1 x 1, unit stride, 16 | plane: the NCHW kernel on the operator's own tensors
+  kPlanesGather,  // any other unpadded 1 x 1: the same kernel, its loader gathering the pixels
+                  // the layer reads
   kSpaceToDepth,  // few-channel stride-2 stem through mxq_nchw_to_s2d_nhwc_i8
   kAdapters       // NHWC copies of both operands, NHWC kernel writing NCHW planes
 };
@@ -325,13 +411,8 @@ NchwPlan plan_nchw(int N, int C, int H, int W, int O, int KH, int KW, int sh, in
   const bool one = KH == 1 && KW == 1 && ph == 0 && pw == 0;
   const bool small = 1LL * N * C * P < (1LL << 31) && 1LL * O * C < (1LL << 31) &&
                      1LL * N * C * H * W < (1LL << 31);
-  if (one && operands_aligned && C % 16 == 0 && P % 16 == 0 && small) {
-    if (sh == 1 && sw == 1) {
-      pl.route = Route::kPlanes;
-      return pl;
-    }
-    pl.route = Route::kPlanesStrided;
-    pl.d_bytes = up256(static_cast<size_t>(N) * C * P);
+  if (one && operands_aligned && C % 16 == 0 && small) {
+    pl.route = (sh == 1 && sw == 1 && P % 16 == 0) ? Route::kPlanes : Route::kPlanesGather;
     return pl;
   }
   // a stride-2 convolution over at most 4 channels (an image stem) runs as the unit-stride
@@ -396,7 +477,7 @@ void conv_nchw(void* stream, const int8_t* data, const int8_t* weight, const int
   // cfg 1 pins the adapter route; 71.. pin a tile of the NCHW kernel
   const bool aligned = aligned16(data) && aligned16(weight) && cfg != 1;
   NchwPlan pl = plan_nchw(N, C, H, W, O, KH, KW, sh, sw, ph, pw, dh, dw, aligned);
-  MXQ_CHECK(cfg < 70 || pl.route == Route::kPlanes || pl.route == Route::kPlanesStrided,
+  MXQ_CHECK(cfg < 70 || pl.route == Route::kPlanes || pl.route == Route::kPlanesGather,
             "shape does not qualify for the NCHW 1x1 kernel");
   hipStream_t s = static_cast<hipStream_t>(stream);
   char* ws = static_cast<char*>(workspace);
@@ -405,17 +486,27 @@ void conv_nchw(void* stream, const int8_t* data, const int8_t* weight, const int
             "workspace too small: " << workspace_bytes << " < " << need
                                     << " (see mxq_quantized_conv_nchw_workspace)");
 
-  if (pl.route == Route::kPlanes || pl.route == Route::kPlanesStrided) {
-    const int8_t* planes = data;
-    if (pl.route == Route::kPlanesStrided) {
-      launch_subsample(s, data, reinterpret_cast<int8_t*>(ws), 1LL * N * C, H, W, pl.OH, pl.OW,
-                       sh, sw);
-      planes = reinterpret_cast<const int8_t*>(ws);
-    }
+  if (pl.route == Route::kPlanes || pl.route == Route::kPlanesGather) {
     PlaneArgs a = {};
-    a.data = planes;
-    a.weight = weight;
     a.N = N; a.C = C; a.P = pl.OH * pl.OW; a.O = O;
+    a.data = data;
+    a.weight = weight;
+    a.data_bytes = static_cast<uint32_t>(N) * C * H * W;
+    int gm = kNative;
+    if (pl.route == Route::kPlanesGather) {
+      a.H = H; a.W = W; a.OW = pl.OW; a.sh = sh; a.sw = sw;
+      const int plane_in = H * W;
+      if (sh == 1 && sw == 1 && plane_in % 4 == 0)
+        gm = kGatherDword;
+      else if (sw == 2 && pl.OW % 4 == 0 && (sh * W) % 8 == 0 && plane_in % 8 == 0 &&
+               2 * pl.OW <= W)
+        gm = kGatherPair;
+      else
+        gm = kGatherBytes;
+    } else {
+      a.img_stride = C * a.P;
+      a.row_stride = a.P;
+    }
     Epilogue& e = a.epi;
     e = Epilogue();
     e.bias = bias;
@@ -427,22 +518,40 @@ void conv_nchw(void* stream, const int8_t* data, const int8_t* weight, const int
     int pick = cfg;
     if (pick < 70) {
       const long cus = num_cus();
-      const long slabs128 = 1L * N * ((a.P + 127) / 128);
-      if (O <= 64)
-        pick = 72;
-      else if (O % 256 == 0 && slabs128 * (O / 256) >= 2 * cus)
-        pick = 75;
-      else if (slabs128 * ((O + 127) / 128) >= 2 * cus)
-        pick = 71;
-      else
-        pick = 73;
+      // columns a pixel tile may run over: a gathered operand is one long row per channel
+      const long long cols = gm != kNative ? 1LL * N * a.P : a.P;
+      const long long rows = gm != kNative ? 1 : N;
+      auto tiles = [&](int bp, int bo) {
+        return rows * ((cols + bp - 1) / bp) * ((O + bo - 1) / bo);
+      };
+      auto padded = [&](int bp) { return (cols + bp - 1) / bp * bp; };
+      if (C >= 256 && O >= 256 && 100 * padded(256) <= 104 * padded(128) &&
+          16 * tiles(256, 256) >= 9 * cus) {
+        pick = 78;  // a real GEMM: the wave tile whose LDS traffic the matrix pipe can hide
+      } else if (C >= 256 && O >= 128 && 100 * padded(256) <= 104 * padded(128) &&
+                 4 * tiles(256, 128) >= 3 * cus) {
+        pick = 77;
+      } else {
+        // pixel tile: 128 unless 64 wastes clearly fewer MFMA rows on the last tile;
+        // channel tile: the widest that still gives every CU two work-groups
+        int bp = (cols <= 64 || 100 * padded(64) < 96 * padded(128)) ? 64 : 128;
+        int bo = 64;
+        if (O > 64) {
+          bo = 128;
+          if (bp == 128 && O >= 256 && tiles(128, 256) >= 2 * cus) bo = 256;
+          if (bp == 128 && tiles(128, bo) < cus) bp = 64;
+        }
+        pick = bp == 128 ? (bo == 64 ? 72 : (bo == 128 ? 71 : 75)) : (bo == 64 ? 74 : 73);
+      }
     }
     switch (pick) {
-      case 71: launch_planes<PlaneM>(s, a); break;
-      case 72: launch_planes<PlaneN64>(s, a); break;
-      case 73: launch_planes<PlaneP64>(s, a); break;
-      case 74: launch_planes<PlaneS>(s, a); break;
-      case 75: launch_planes<PlaneW>(s, a); break;
+      case 71: launch_planes<PlaneM>(s, a, gm); break;
+      case 72: launch_planes<PlaneN64>(s, a, gm); break;
+      case 73: launch_planes<PlaneP64>(s, a, gm); break;
+      case 74: launch_planes<PlaneS>(s, a, gm); break;
+      case 75: launch_planes<PlaneW>(s, a, gm); break;
+      case 77: launch_planes<PlaneH>(s, a, gm); break;
+      case 78: launch_planes<PlaneL>(s, a, gm); break;
       default: MXQ_CHECK(false, "unknown NCHW tile configuration " << pick);
     }
     return;
@@ -489,10 +598,12 @@ size_t mxq_quantized_conv_nchw_workspace(int N, int C, int H, int W, int O, int 
     const NchwPlan b = plan_nchw(N, C, H, W, O, KH, KW, stride_h, stride_w, pad_h, pad_w,
                                  dilate_h, dilate_w, false);
     const size_t nb = b.d_bytes + b.w_bytes + b.split_bytes;
-    if (operands_aligned16 == 0) return nb;
     const NchwPlan a = plan_nchw(N, C, H, W, O, KH, KW, stride_h, stride_w, pad_h, pad_w,
                                  dilate_h, dilate_w, true);
-    return a.d_bytes + a.w_bytes + a.split_bytes;
+    const size_t na = a.d_bytes + a.w_bytes + a.split_bytes;
+    // without the promise: enough for either route
+    if (operands_aligned16 == 0) return na > nb ? na : nb;
+    return na;
   } catch (...) {
     return 0;
   }
@@ -513,7 +624,7 @@ int mxq_quantized_conv_nchw(void* stream, const int8_t* data, const int8_t* weig
 }
 
 // Test-only twin (declared in tests/mxq_test_hooks.h): cfg 1 pins the route through the
-// layout adapters, 71 ... 75 a tile of the NCHW kernel, 0 leaves the choice to the launcher.
+// layout adapters, 71 ... 78 a tile of the NCHW kernel, 0 leaves the choice to the launcher.
 int mxq_test_quantized_conv_nchw(void* stream, const int8_t* data, const int8_t* weight,
                                  const int8_t* bias, int N, int C, int H, int W, int O, int KH,
                                  int KW, int stride_h, int stride_w, int pad_h, int pad_w,
