@@ -377,13 +377,14 @@ int mxq_quantized_conv_nhwc_out_nchw(void* stream, const int8_t* data, const int
  * QuantizedCuDNNConvOp::Forward does between its inputs and its outputs
  * (src/operator/quantization/quantized_conv.cu:101-219, layout rule quantized_conv.cc:38-45),
  * the three TransposeImpl calls included (:145-148,183).  Unpadded 1 x 1 convolutions over
- * 16 | C channels never leave the channel-plane layout and need no workspace (strided ones
- * and planes that are no multiple of 16 bytes through a gathering loader in the same
- * kernel); every other geometry goes through the layout adapters and
+ * 16 | C channels never leave the channel-plane layout (strided ones and planes that are
+ * no multiple of 16 bytes through a gathering loader in the same kernel or, where that
+ * would fetch single bytes, after the pixels they read were gathered into the workspace);
+ * every other geometry goes through the layout adapters and
  * mxq_quantized_conv_nhwc_out_nchw inside this call.
  * `workspace` (16-byte aligned) must hold mxq_quantized_conv_nchw_workspace() bytes: the
  * operator's kTempSpace (quantized_conv.cu:121-160 asks for three tensor copies plus
- * cuDNN's workspace there; 0 here for an unpadded 1 x 1 layer).  operands_aligned16 != 0
+ * cuDNN's workspace there; 0 here for most unpadded 1 x 1 layers).  operands_aligned16 != 0
  * says that data and weight both start on 16-byte marks, as a framework's allocations do;
  * with 0 the query returns enough for the adapter route as well, which every geometry and
  * alignment can take. */

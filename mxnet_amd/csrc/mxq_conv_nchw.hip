@@ -24,8 +24,10 @@
 // stride 2 over rows of 4 | OW pixels, the plane's own dwords for unit stride, bytes
 // otherwise) and the operand becomes the matrix [C][N * OH * OW] whose pixel tiles run
 // across image boundaries.  No workspace, no pre-pass: a strided layer reads only the
-// cache lines it uses.  Everything else (3 x 3, padded 1 x 1, C % 16 != 0) takes the NHWC
-// kernels of mxq_conv.hip behind the layout adapters.
+// cache lines it uses.  Where that loader would have to fetch single bytes (odd rows, 7 x 7
+// planes) a pre-pass gathers the pixels into one row per channel in the caller's workspace
+// first and the kernel reads that with its 16-byte loads.  Everything else (3 x 3, padded
+// 1 x 1, C % 16 != 0) takes the NHWC kernels of mxq_conv.hip behind the layout adapters.
 #include <hip/hip_runtime.h>
 
 #include <cmath>
@@ -50,6 +52,9 @@ struct PlaneArgs {
   const int8_t* weight;  // [O][C]
   int N, C, P, O;        // P = output pixels per image
   int img_stride, row_stride;   // native
+  int pitch;             // native, 0: pixel tiles inside one image.  > 0: a pre-gathered
+                         // operand (gather_planes_kernel), one row per channel over the whole
+                         // batch with image n's P pixels at columns n * pitch ...; img_stride 0
   int H, W, OW, sh, sw;         // gathered: input plane, output row length, strides
   uint32_t data_bytes;   // extent of the activation tensor
   int tiles_p, tiles_o;  // pixel tiles (per image if native, per matrix if gathered), channel tiles
@@ -104,6 +109,8 @@ constexpr int kNative = 0;      // not gathered: 16-byte direct-to-LDS loads
 constexpr int kGatherDword = 1; // unit stride, planes on dword marks: the plane's own dwords
 constexpr int kGatherPair = 2;  // sw == 2, 4 | OW, rows on 8-byte marks: 8 bytes and a v_perm
 constexpr int kGatherBytes = 3; // anything else: byte by byte
+constexpr int kGatherPair2 = 4; // sw == 2, 2 | OW, rows on dword marks: two dwords (two pixels
+                                // each, a pair never leaves its row) and a v_perm
 
 template <class Cfg, int NS, int GM>
 __global__ __launch_bounds__(Cfg::kThreads, 2) void conv1x1_planes_kernel(PlaneArgs p) {
@@ -122,7 +129,9 @@ __global__ __launch_bounds__(Cfg::kThreads, 2) void conv1x1_planes_kernel(PlaneA
   // tile order: the output-channel tiles of one pixel slab are neighbours, and the
   // round-robin of work-group ids over the XCDs is undone so that they meet in one L2
   constexpr bool gathered = GM != kNative;
-  const int images = gathered ? 1 : p.N;
+  const bool flat = gathered || p.pitch != 0;   // pixel tiles run over the whole batch
+  const int pitch = gathered ? p.P : p.pitch;   // columns per image then
+  const int images = flat ? 1 : p.N;
   const int total = images * p.tiles_p * p.tiles_o;
   const int lid = xcd_remap(blockIdx.x, total);
   const int to = lid % p.tiles_o;
@@ -171,7 +180,7 @@ __global__ __launch_bounds__(Cfg::kThreads, 2) void conv1x1_planes_kernel(PlaneA
   if constexpr (gathered) {
     const long long V = 1LL * p.N * p.P;
 #pragma unroll
-    for (int j = 0; j < (GM == kGatherBytes ? 4 : 1); ++j) {
+    for (int j = 0; j < ((GM == kGatherBytes || GM == kGatherPair2) ? 4 : 1); ++j) {
       const long long v = 1LL * p0 + 4 * grp + j;
       const int vv = v < V ? static_cast<int>(v) : 0;   // columns past the end read pixel 0
       const int img = vv / p.P, px = vv - img * p.P;
@@ -193,6 +202,10 @@ __global__ __launch_bounds__(Cfg::kThreads, 2) void conv1x1_planes_kernel(PlaneA
           typedef uint32_t u2 __attribute__((ext_vector_type(2)));
           const u2 w = *reinterpret_cast<const u2*>(row + goff[0]);
           areg[i] = __builtin_amdgcn_perm(w.y, w.x, 0x06040200u);
+        } else if (GM == kGatherPair2) {
+          const uint32_t w0 = *reinterpret_cast<const uint32_t*>(row + goff[0]);
+          const uint32_t w1 = *reinterpret_cast<const uint32_t*>(row + goff[2]);
+          areg[i] = __builtin_amdgcn_perm(w1, w0, 0x06040200u);
         } else {
           const uint32_t b0 = static_cast<uint8_t>(row[goff[0]]);
           const uint32_t b1 = static_cast<uint8_t>(row[goff[1]]);
@@ -304,18 +317,78 @@ __global__ __launch_bounds__(Cfg::kThreads, 2) void conv1x1_planes_kernel(PlaneA
   if (blockIdx.x == 0 && tid == 0) epilogue_ranges(p.epi);
   __syncthreads();  // sbias
 
-  // lane = pixel, register = channel 8 * (v / 4) + 4 * (lane / 32) + v % 4 of the MFMA
-  // tile: a store instruction writes 32 consecutive int32 of two channel planes (fewer
-  // where a gathered tile passes from one image to the next)
+  // In the accumulators a lane holds one pixel and registers hold channels
+  // (8 * (v / 4) + 4 * (lane / 32) + v % 4 of the MFMA tile).
+  if ((p.P & 3) == 0 && (reinterpret_cast<uintptr_t>(p.epi.out32) & 15u) == 0) {
+    // Planes of whole 16-byte runs: the wave's tile goes through its share of the (now free)
+    // stage ring, channel-major, and leaves with 16 bytes per lane along the pixels, so a
+    // store instruction writes runs of 4 * TP bytes of 256 / TP channel planes instead of two
+    // runs of 128 bytes (measured on store-only kernels of this shape: 2.9 -> 4.8 TB/s for
+    // 14 x 14 planes, 4.2 -> 5.0 for 28 x 28).  A group of four pixels never straddles two
+    // images because 4 | P.
+    constexpr int TP = Cfg::TP, LP = TP + 8;   // row pitch in dwords: lanes 32-63 write four
+                                               // rows further down, 32 banks away
+    constexpr int RING = NS * STAGE_BYTES;
+    constexpr int CHB = (32 * LP * 4 * NW <= RING) ? 32 : ((16 * LP * 4 * NW <= RING) ? 16 : 8);
+    static_assert(CHB * LP * 4 * NW <= RING, "stage ring too small for the epilogue's tile");
+    constexpr int LPR = TP / 4, RPI = 64 / LPR;   // lanes per channel row, rows per instruction
+    int* t32 = reinterpret_cast<int*>(lds) + wave * (CHB * LP);
+    const int px4 = (lane % LPR) * 4, r0 = lane / LPR;
+    const int v = p0 + wp * TP + px4;
+    int img = n, px = v;
+    if (flat) {
+      img = v / pitch;
+      px = v - img * pitch;
+    }
+    const bool ok = img < p.N && px < p.P;
+    int32_t* obase = p.epi.out32 + static_cast<size_t>(img) * p.O * p.P + px;
+#pragma unroll
+    for (int ni = 0; ni < NI; ++ni) {
+#pragma unroll
+      for (int part = 0; part < 32 / CHB; ++part) {
+#pragma unroll
+        for (int vq = 0; vq < 4; ++vq) {
+          if ((8 * vq) / CHB != part) continue;
+          const int ol = wo * Cfg::TO + ni * 32 + 8 * vq + 4 * fgrp;  // channel inside the tile
+          const v4i b = *reinterpret_cast<const v4i*>(sbias + ol);
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int mi = 0; mi < MI; ++mi)
+              t32[((8 * vq) % CHB + 4 * fgrp + i) * LP + 32 * mi + frow] =
+                  static_cast<int>(static_cast<uint32_t>(acc[mi][ni][4 * vq + i]) +
+                                   static_cast<uint32_t>(b[i]));
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        __builtin_amdgcn_wave_barrier();
+        v4i back[CHB / RPI];
+#pragma unroll
+        for (int it = 0; it < CHB / RPI; ++it)
+          back[it] = *reinterpret_cast<const v4i*>(t32 + (it * RPI + r0) * LP + px4);
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int it = 0; it < CHB / RPI; ++it) {
+          const int o = o0 + wo * Cfg::TO + ni * 32 + part * CHB + it * RPI + r0;
+          if (ok && o < p.O)
+            *reinterpret_cast<v4i*>(obase + static_cast<size_t>(o) * p.P) = back[it];
+        }
+      }
+    }
+    return;
+  }
+  // Any other plane (7 x 7): dword stores straight from the accumulators, a store
+  // instruction writes 32 consecutive int32 of two channel planes (fewer where a tile
+  // passes from one image to the next)
   size_t obase[MI];   // offset of (image, channel 0, pixel) in out32
   bool ovalid[MI];
 #pragma unroll
   for (int mi = 0; mi < MI; ++mi) {
     const int v = p0 + wp * Cfg::TP + 32 * mi + frow;
     int img = n, px = v;
-    if (gathered) {
-      img = v / p.P;
-      px = v - img * p.P;
+    if (flat) {
+      img = v / pitch;
+      px = v - img * pitch;
     }
     ovalid[mi] = img < p.N && px < p.P;
     obase[mi] = static_cast<size_t>(img) * p.O * p.P + px;
@@ -343,6 +416,125 @@ __global__ __launch_bounds__(Cfg::kThreads, 2) void conv1x1_planes_kernel(PlaneA
   }
 }
 
+// ---- pre-pass for gathered operands that would need byte loads --------------------------
+// out[c][n * pitch + oh * OW + ow] = in[n][c][oh * sh][ow * sw]: the pixels a 1 x 1
+// convolution without padding reads, as one row of `row_stride` bytes per channel over the
+// whole batch (columns past a plane's OH * OW pixels are not written).  Used where the
+// kernel's own gathering loader would have to fetch single bytes (odd rows, 7 x 7 planes):
+// the pre-pass costs one launch and the kernel then reads 16-byte pieces through its ring.
+// Work is cut into pieces "2^lg consecutive dwords of one plane" (2^lg = the power of two
+// that covers a plane's dwords, at most 64); a group of 2^lg lanes walks `run` consecutive
+// pieces, so the divisions that find its first plane are paid once per thread and every
+// later piece is found by counting.  kGatherItems pieces are requested before any is stored,
+// and every load is unconditional (a lane past the plane or past the run reads the plane's
+// first bytes and drops them): loads inside branches are waited for one by one.  One piece
+// per thread with its divisions took 22 us for the 51 MB of a 64 x 256 x 56 x 56 input, a
+// plane per wave 11-15 us for the 6-13 MB tensors of 14 x 14 and 7 x 7 planes (65 K to
+// 131 K short waves); this form 8 us.  ow_magic = ceil(2^32 / OW) finds a pixel's row,
+// exact below 2^16.
+constexpr int kGatherItems = 4;
+
+struct GatherArgs {
+  const uint8_t* in;
+  uint8_t* out;
+  int C, H, W, OW, P, sh, sw, pitch, row_stride;
+  unsigned planes;
+  int lg;              // lanes per group = 1 << lg
+  int pieces;          // pieces per plane = ceil(pitch / 4 / lanes per group)
+  unsigned run;        // consecutive pieces per group
+  unsigned total;      // planes * pieces
+  uint32_t ow_magic;
+};
+
+__global__ __launch_bounds__(256) void gather_planes_kernel(GatherArgs a) {
+  const unsigned slot = blockIdx.x * 256u + threadIdx.x;
+  const unsigned group = slot >> a.lg, lane = slot & ((1u << a.lg) - 1u);
+  unsigned q = group * a.run;
+  if (q >= a.total) return;
+  const unsigned q_end = (q + a.run < a.total) ? q + a.run : a.total;
+  // position of the first piece
+  unsigned b = q / static_cast<unsigned>(a.pieces);
+  int piece = static_cast<int>(q - b * a.pieces);
+  unsigned n = b / static_cast<unsigned>(a.C);
+  int c = static_cast<int>(b - n * a.C);
+  const int per = a.pitch >> 2, plane_in = a.H * a.W;
+  const uint8_t* src = a.in + static_cast<size_t>(b) * plane_in;
+  while (q < q_end) {
+    uint32_t v[kGatherItems];
+    uint8_t* to[kGatherItems];
+    bool ok[kGatherItems];
+#pragma unroll
+    for (int u = 0; u < kGatherItems; ++u) {
+      const int dd = (piece << a.lg) + static_cast<int>(lane);
+      ok[u] = q < q_end && dd < per && 4 * dd < a.P;
+      to[u] = a.out + static_cast<size_t>(c) * a.row_stride + static_cast<size_t>(n) * a.pitch +
+              4 * dd;
+      const int p4 = ok[u] ? 4 * dd : 0;
+      int oh = static_cast<int>(__umulhi(static_cast<uint32_t>(p4), a.ow_magic));
+      int ow = p4 - oh * a.OW;
+      uint32_t bytes[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const bool in_plane = p4 + j < a.P;
+        bytes[j] = src[in_plane ? oh * a.sh * a.W + ow * a.sw : 0];
+        bytes[j] = in_plane ? bytes[j] : 0u;
+        if (++ow == a.OW) {
+          ow = 0;
+          ++oh;
+        }
+      }
+      v[u] = bytes[0] | (bytes[1] << 8) | (bytes[2] << 16) | (bytes[3] << 24);
+      // the next piece (the pointer only moves while q < q_end, so it stays in the tensor)
+      ++q;
+      if (q < q_end) {
+        if (++piece == a.pieces) {
+          piece = 0;
+          src += plane_in;
+          if (++c == a.C) {
+            c = 0;
+            ++n;
+          }
+        }
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < kGatherItems; ++u)
+      if (ok[u]) *reinterpret_cast<uint32_t*>(to[u]) = v[u];
+  }
+}
+
+constexpr int kGatherMaxPlane = 1 << 16;  // pixels per gathered plane (the row division)
+
+void launch_gather(hipStream_t s, const int8_t* in, int8_t* out, int N, int C, int H, int W,
+                   int OH, int OW, int sh, int sw, int pitch, int row_stride) {
+  const long long planes = 1LL * N * C;
+  if (planes == 0 || pitch == 0) return;
+  MXQ_CHECK(OH * OW < kGatherMaxPlane, "plane too large for the gather");
+  GatherArgs a;
+  a.in = reinterpret_cast<const uint8_t*>(in);
+  a.out = reinterpret_cast<uint8_t*>(out);
+  a.C = C; a.H = H; a.W = W; a.OW = OW; a.P = OH * OW; a.sh = sh; a.sw = sw;
+  a.pitch = pitch; a.row_stride = row_stride;
+  a.planes = static_cast<unsigned>(planes);
+  a.lg = 0;
+  while (a.lg < 6 && (1 << a.lg) < pitch / 4) ++a.lg;
+  a.pieces = (pitch / 4 + (1 << a.lg) - 1) >> a.lg;
+  const long long total = planes * a.pieces;
+  MXQ_CHECK(total < (1LL << 31), "too many planes");
+  a.total = static_cast<unsigned>(total);
+  // groups: about 16 waves per CU, each group with at least 2 * kGatherItems pieces
+  const long long groups_per_wave = 64 >> a.lg;
+  long long groups = 16LL * num_cus() * groups_per_wave;
+  long long run = (total + groups - 1) / groups;
+  if (run < 2 * kGatherItems) run = 2 * kGatherItems;
+  a.run = static_cast<unsigned>(run);
+  groups = (total + run - 1) / run;
+  a.ow_magic = static_cast<uint32_t>(((1ULL << 32) + OW - 1) / OW);
+  const unsigned grid = static_cast<unsigned>(((groups << a.lg) + 255) / 256);
+  hipLaunchKernelGGL(gather_planes_kernel, dim3(grid), dim3(256), 0, s, a);
+  MXQ_LAUNCH_CHECK();
+}
+
 typedef PlaneCfg<128, 128, 64, 2, 2> PlaneM;   // 4 waves, wave tile 64 pixels x 64 channels
 typedef PlaneCfg<128, 64, 64, 2, 2> PlaneN64;  // 4 waves, wave tile 64 x 32
 typedef PlaneCfg<64, 128, 64, 2, 2> PlaneP64;  // 4 waves, wave tile 32 x 64
@@ -353,10 +545,11 @@ typedef PlaneCfg<256, 256, 64, 2, 4> PlaneL;   // 8 waves, wave tile 128 x 64
 
 template <class Cfg>
 void launch_planes(hipStream_t s, PlaneArgs a, int gm) {
-  const long long cols = gm != kNative ? 1LL * a.N * a.P : a.P;
+  const bool flat = gm != kNative || a.pitch != 0;
+  const long long cols = gm != kNative ? 1LL * a.N * a.P : (flat ? 1LL * a.N * a.pitch : a.P);
   a.tiles_p = static_cast<int>((cols + Cfg::BP - 1) / Cfg::BP);
   a.tiles_o = (a.O + Cfg::BO - 1) / Cfg::BO;
-  const long long total = 1LL * (gm != kNative ? 1 : a.N) * a.tiles_p * a.tiles_o;
+  const long long total = 1LL * (flat ? 1 : a.N) * a.tiles_p * a.tiles_o;
   MXQ_CHECK(total < (1LL << 31), "grid too large");
   const dim3 grid(static_cast<unsigned>(total)), block(Cfg::kThreads);
   if (gm == kGatherDword) {
@@ -365,6 +558,8 @@ void launch_planes(hipStream_t s, PlaneArgs a, int gm) {
     hipLaunchKernelGGL((conv1x1_planes_kernel<Cfg, 2, kGatherPair>), grid, block, 0, s, a);
   } else if (gm == kGatherBytes) {
     hipLaunchKernelGGL((conv1x1_planes_kernel<Cfg, 2, kGatherBytes>), grid, block, 0, s, a);
+  } else if (gm == kGatherPair2) {
+    hipLaunchKernelGGL((conv1x1_planes_kernel<Cfg, 2, kGatherPair2>), grid, block, 0, s, a);
   } else if (a.C <= 2 * Cfg::BK) {
     // a reduction of up to two stages needs no deeper ring; a longer one is read from HBM
     // once and wants several stages in flight per work-group
@@ -380,6 +575,8 @@ enum class Route {
   kPlanes,        // 1 x 1, unit stride, 16 | plane: the NCHW kernel on the operator's own tensors
   kPlanesGather,  // any other unpadded 1 x 1: the same kernel, its loader gathering the pixels
                   // the layer reads
+  kPlanesPrepass, // ... or, where that loader would fetch single bytes, after a pre-pass that
+                  // gathers them into one row per channel
   kSpaceToDepth,  // few-channel stride-2 stem through mxq_nchw_to_s2d_nhwc_i8
   kAdapters       // NHWC copies of both operands, NHWC kernel writing NCHW planes
 };
@@ -394,6 +591,8 @@ struct NchwPlan {
   int off_h, off_w, H2, W2, K2h, K2w, pad2_h, pad2_w;
   // NHWC view of the adapter routes
   int vC;
+  int gather_mode;         // kPlanesGather: how the loader fetches a group's four pixels
+  int pitch, row_stride;   // kPlanesPrepass: columns per image and bytes per channel row
   bool weight_in_place;    // 1 x 1 window over C % 16 == 0 channels: OIHW is OHWI already
   size_t d_bytes, w_bytes, split_bytes;
 };
@@ -412,7 +611,35 @@ NchwPlan plan_nchw(int N, int C, int H, int W, int O, int KH, int KW, int sh, in
   const bool small = 1LL * N * C * P < (1LL << 31) && 1LL * O * C < (1LL << 31) &&
                      1LL * N * C * H * W < (1LL << 31);
   if (one && operands_aligned && C % 16 == 0 && small) {
-    pl.route = (sh == 1 && sw == 1 && P % 16 == 0) ? Route::kPlanes : Route::kPlanesGather;
+    if (sh == 1 && sw == 1 && P % 16 == 0) {
+      pl.route = Route::kPlanes;
+      return pl;
+    }
+    // The gathering loader works one stage ahead out of registers; the pre-pass costs a launch
+    // and a copy of what the layer reads but feeds the kernel's four-stage ring.  Measured
+    // on the ResNet-50 layers at batch 64: the loader wins while the weight matrix is small
+    // (256 -> 128 / 2: 34 -> 28 us, 1024 -> 256 at 14 x 14: 24 -> 20 us), the ring once the
+    // layer is a real GEMM (512 -> 1024 / 2 at 28 x 28: 38 us against 53 us).
+    const int plane_in = H * W;
+    const long long pitch = (P + 3) / 4 * 4, row = (1LL * N * pitch + 15) / 16 * 16;
+    const bool prepass_ok = P < kGatherMaxPlane && 1LL * C * row < (1LL << 31);
+    const bool light = 1LL * O * C <= 256 * 1024 || !prepass_ok;
+    int mode = kGatherBytes;
+    if (sh == 1 && sw == 1 && plane_in % 4 == 0)
+      mode = kGatherDword;
+    else if (sw == 2 && pl.OW % 4 == 0 && (sh * W) % 8 == 0 && plane_in % 8 == 0 && 2 * pl.OW <= W)
+      mode = kGatherPair;
+    else if (sw == 2 && pl.OW % 2 == 0 && (sh * W) % 4 == 0 && plane_in % 4 == 0 && 2 * pl.OW <= W)
+      mode = kGatherPair2;
+    if ((mode != kGatherBytes && light) || !prepass_ok) {
+      pl.route = Route::kPlanesGather;
+      pl.gather_mode = mode;
+      return pl;
+    }
+    pl.route = Route::kPlanesPrepass;
+    pl.pitch = static_cast<int>(pitch);
+    pl.row_stride = static_cast<int>(row);
+    pl.d_bytes = up256(static_cast<size_t>(C) * row);
     return pl;
   }
   // a stride-2 convolution over at most 4 channels (an image stem) runs as the unit-stride
@@ -477,7 +704,9 @@ void conv_nchw(void* stream, const int8_t* data, const int8_t* weight, const int
   // cfg 1 pins the adapter route; 71.. pin a tile of the NCHW kernel
   const bool aligned = aligned16(data) && aligned16(weight) && cfg != 1;
   NchwPlan pl = plan_nchw(N, C, H, W, O, KH, KW, sh, sw, ph, pw, dh, dw, aligned);
-  MXQ_CHECK(cfg < 70 || pl.route == Route::kPlanes || pl.route == Route::kPlanesGather,
+  const bool planes_route = pl.route == Route::kPlanes || pl.route == Route::kPlanesGather ||
+                            pl.route == Route::kPlanesPrepass;
+  MXQ_CHECK(cfg < 70 || planes_route,
             "shape does not qualify for the NCHW 1x1 kernel");
   hipStream_t s = static_cast<hipStream_t>(stream);
   char* ws = static_cast<char*>(workspace);
@@ -486,7 +715,7 @@ void conv_nchw(void* stream, const int8_t* data, const int8_t* weight, const int
             "workspace too small: " << workspace_bytes << " < " << need
                                     << " (see mxq_quantized_conv_nchw_workspace)");
 
-  if (pl.route == Route::kPlanes || pl.route == Route::kPlanesGather) {
+  if (planes_route) {
     PlaneArgs a = {};
     a.N = N; a.C = C; a.P = pl.OH * pl.OW; a.O = O;
     a.data = data;
@@ -495,14 +724,15 @@ void conv_nchw(void* stream, const int8_t* data, const int8_t* weight, const int
     int gm = kNative;
     if (pl.route == Route::kPlanesGather) {
       a.H = H; a.W = W; a.OW = pl.OW; a.sh = sh; a.sw = sw;
-      const int plane_in = H * W;
-      if (sh == 1 && sw == 1 && plane_in % 4 == 0)
-        gm = kGatherDword;
-      else if (sw == 2 && pl.OW % 4 == 0 && (sh * W) % 8 == 0 && plane_in % 8 == 0 &&
-               2 * pl.OW <= W)
-        gm = kGatherPair;
-      else
-        gm = kGatherBytes;
+      gm = pl.gather_mode;
+    } else if (pl.route == Route::kPlanesPrepass) {
+      launch_gather(s, data, reinterpret_cast<int8_t*>(ws), N, C, H, W, pl.OH, pl.OW, sh, sw,
+                    pl.pitch, pl.row_stride);
+      a.data = reinterpret_cast<const int8_t*>(ws);
+      a.img_stride = 0;
+      a.row_stride = pl.row_stride;
+      a.pitch = pl.pitch;
+      a.data_bytes = static_cast<uint32_t>(C) * pl.row_stride;
     } else {
       a.img_stride = C * a.P;
       a.row_stride = a.P;
@@ -519,8 +749,9 @@ void conv_nchw(void* stream, const int8_t* data, const int8_t* weight, const int
     if (pick < 70) {
       const long cus = num_cus();
       // columns a pixel tile may run over: a gathered operand is one long row per channel
-      const long long cols = gm != kNative ? 1LL * N * a.P : a.P;
-      const long long rows = gm != kNative ? 1 : N;
+      const bool flat = gm != kNative || a.pitch != 0;
+      const long long cols = gm != kNative ? 1LL * N * a.P : (flat ? 1LL * N * a.pitch : a.P);
+      const long long rows = flat ? 1 : N;
       auto tiles = [&](int bp, int bo) {
         return rows * ((cols + bp - 1) / bp) * ((O + bo - 1) / bo);
       };

@@ -90,13 +90,24 @@ STRIDED_CASES = [
     (3, 512, 7, 7, 2048, 1, 1, 1, 0, 1),    # 7 x 7 planes repacked, O in 256-wide tiles
     (2, 48, 5, 3, 40, 1, 1, 1, 0, 1),       # 15 pixels
     (2, 16, 9, 7, 24, 1, 1, (2), 0, 1),     # 5 x 4 = 20 pixels
+    (3, 32, 12, 12, 72, 1, 1, 2, 0, 1),     # 6 x 6: pairs of pixels, 36 per plane
+    (2, 64, 20, 12, 32, 1, 1, 2, 0, 1),     # 10 x 6
 ]
 
 
 @pytest.mark.parametrize("case", STRIDED_CASES)
 def test_conv_nchw_strided_planes(capi, case):
     res = run(capi, case, True)
-    assert res["workspace_bytes"] == 0  # the loader gathers: no pre-pass, no copy
+    N, C, H, W, O, _, _, s = case[:8]
+    OH, OW = (H - 1) // s + 1, (W - 1) // s + 1
+    dwords = s == 1 and (H * W) % 4 == 0
+    pairs = s == 2 and OW % 4 == 0 and (s * W) % 8 == 0 and (H * W) % 8 == 0 and 2 * OW <= W
+    pairs2 = s == 2 and OW % 2 == 0 and (s * W) % 4 == 0 and (H * W) % 4 == 0 and 2 * OW <= W
+    if (dwords or pairs or pairs2) and O * C <= 256 * 1024:
+        assert res["workspace_bytes"] == 0  # the kernel's loader gathers: no pre-pass, no copy
+    else:
+        row = (N * ((OH * OW + 3) // 4 * 4) + 15) // 16 * 16  # one row per channel over the batch
+        assert res["workspace_bytes"] == (C * row + 255) // 256 * 256  # the pixels it reads, once
 
 
 # everything else goes through the adapters inside the same call
@@ -139,6 +150,21 @@ def test_conv_nchw_unaligned_operands_take_the_adapters(capi):
     res = capi.quantized_conv_nchw(view, dev(w), None, f32(-1.0), f32(1.0), f32(-1.0), f32(1.0))
     ro, _, _ = oracle.quantized_conv(d, w, None, -1.0, 1.0, -1.0, 1.0)
     np.testing.assert_array_equal(res["out32"].cpu().numpy(), ro)
+
+
+def test_conv_nchw_output_off_the_16_byte_marks(capi):
+    """An int32 output that starts 4 bytes past a 16-byte mark takes the dword stores."""
+    case = (2, 64, 8, 8, 96, 1, 1, 1, 0, 1)
+    N, C, H, W, O = case[:5]
+    d = int8_uniform((N, C, H, W), seed=5)
+    w = int8_uniform((O, C, 1, 1), seed=6)
+    flat = torch.zeros(N * O * H * W + 8, dtype=torch.int32, device="cuda")
+    out = flat[1:1 + N * O * H * W].view(N, O, H, W)
+    res = capi.quantized_conv_nchw(dev(d), dev(w), None, f32(-1.0), f32(1.0), f32(-1.0), f32(1.0),
+                                   out=out)
+    ro, _, _ = oracle.quantized_conv(d, w, None, -1.0, 1.0, -1.0, 1.0)
+    np.testing.assert_array_equal(res["out32"].cpu().numpy(), ro)
+    assert flat[0].item() == 0 and flat[-1].item() == 0
 
 
 def test_conv_nchw_without_images(capi):

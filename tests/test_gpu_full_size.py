@@ -342,3 +342,33 @@ def test_resnet50_conv_batch64(capi, H, C, O, k, s):
     assert torch.equal(res["out8"], torch.clamp(q_all, min=0))
     frac = float((res["out8"] > 0).float().mean())
     assert 0.2 < frac < 0.8 and int(res["out8"].max()) == 127
+
+
+@pytest.mark.parametrize("H,C,O,k,s", RESNET50_CONVS)
+def test_resnet50_conv_batch64_through_the_operator(capi, contrib, H, C, O, k, s):
+    """The same 19 layers at batch 64 through the registered _contrib_quantized_conv: NCHW int8
+    data and OIHW int8 weights in, int32 NCHW out, temp space sized by the operator host.  The
+    first and last image against the oracle, every image against the NHWC entry point's
+    result brought to NCHW by torch (another kernel, another layout, another epilogue)."""
+    batch, pad = 64, (1 if k == 3 else 0)
+    g = torch.Generator(device="cuda").manual_seed(3 * H + C + O + k)
+    d = torch.randint(-127, 128, (batch, C, H, H), device="cuda", generator=g, dtype=torch.int8)
+    w = torch.randint(-127, 128, (O, C, k, k), device="cuda", generator=g, dtype=torch.int8)
+    b = torch.randint(-127, 128, (O,), device="cuda", generator=g, dtype=torch.int8)
+    one = f32(1.0)
+    out, mn, mx = contrib.quantized_conv(d, w, b, -one, one, -one, one, -one, one,
+                                         kernel=(k, k), stride=(s, s), dilate=(1, 1),
+                                         pad=(pad, pad), num_filter=O, no_bias=False,
+                                         layout="NCHW")
+    OH = (H + 2 * pad - k) // s + 1
+    assert out.dtype == torch.int32 and tuple(out.shape) == (batch, O, OH, OH)
+    images = [0, batch - 1]
+    acc, omin, omax = oracle.quantized_conv(d[images].cpu().numpy(), w.cpu().numpy(),
+                                            b.cpu().numpy(), -1.0, 1.0, -1.0, 1.0, -1.0, 1.0,
+                                            stride=(s, s), pad=(pad, pad))
+    assert np.array_equal(out[images].cpu().numpy(), acc)
+    assert (mn.item(), mx.item()) == (omin, omax)
+    ref = capi.quantized_conv_nhwc(d.permute(0, 2, 3, 1).contiguous(),
+                                   w.permute(0, 2, 3, 1).contiguous(), b, -one, one, -one, one,
+                                   -one, one, stride=(s, s), pad=(pad, pad))
+    assert torch.equal(out, ref["out32"].permute(0, 3, 1, 2))
