@@ -69,7 +69,10 @@ int mxq_quantize_v2(void* stream, const float* in, void* out, float* omin, float
  * limited to 2^31 elements (a larger n is refused with an error).  The call allocates and
  * frees nothing.  All calls on one GPU share that GPU's array: calls that overlap in time
  * on one GPU (different streams) race on it and must be serialised by the caller; calls
- * on one stream, or on different GPUs, are safe. */
+ * on one stream, or on different GPUs, are safe.  The first uncalibrated call on a GPU
+ * looks the array's address up (hipGetDevice, hipGetSymbolAddress: host runtime calls that
+ * may load the code object); make that first call outside any stream capture, every later
+ * call on that GPU only launches kernels and may be captured. */
 int mxq_quantize_v2_noalloc(void* stream, const float* in, void* out, float* omin, float* omax,
                             size_t n, int out_type, int calibrated, float min_calib,
                             float max_calib);
@@ -326,7 +329,9 @@ int mxq_quantized_fc_f32(void* stream, const int8_t* data, const int8_t* weight,
  *   sum_*_calib    the sum's calibrated range; rmin / rmax receive it
  *   sum_relu != 0  clamps the sum at zero
  * out8 is bit-identical to mxq_quantized_elemwise_add(out8 of mxq_quantized_fc, residual)
- * followed by mxq_quantized_relu; neither intermediate tensor is stored.  out8 may be the
+ * followed by mxq_quantized_relu; neither intermediate tensor is stored.  (The element
+ * rounding of the sum is this library's own choice: in the reference it happens inside
+ * oneDNN and its parity is unpinned, as for mxq_quantized_elemwise_add.)  out8 may be the
  * residual's own buffer (the shortcut updated in place).  Workspace as for
  * mxq_quantized_fc with fused_int8_only = 1. */
 int mxq_quantized_fc_sum(void* stream, const int8_t* data, const int8_t* weight,

@@ -48,6 +48,9 @@ int mxq_node_num_outputs(void* node, int* out);
 /* comma-separated names; the string lives as long as the node */
 int mxq_node_input_names(void* node, const char** out);
 int mxq_node_output_names(void* node, const char** out);
+/* FGradient: "operator:node name" of the gradient node made for every input, comma-separated
+ * ("" for an operator registered without one); the string lives as long as the node */
+int mxq_node_gradient_names(void* node, const char** out);
 
 /* FInferShape / FInferType: unknown shapes have ndim -1, unknown types are -1;
  * both arrays are updated in place. */

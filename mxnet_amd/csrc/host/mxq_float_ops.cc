@@ -156,6 +156,13 @@ NNVM_REGISTER_OP(SoftmaxOutput)
                                      })
     .set_attr<nnvm::FListOutputNames>("FListOutputNames", OneOutput);
 
+// the operator MakeZeroGradNodes (src/operator/operator_common.h:430-444) names as the
+// gradient of an inference-only operator
+NNVM_REGISTER_OP(zeros_like)
+    .set_num_inputs(1)
+    .set_num_outputs(1)
+    .set_attr<nnvm::FListInputNames>("FListInputNames", DataOnly);
+
 // src/operator/nn/dropout.cc:64-110
 NNVM_REGISTER_OP(Dropout)
     .set_num_inputs(1)

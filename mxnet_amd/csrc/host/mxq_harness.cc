@@ -24,7 +24,7 @@ thread_local std::string tl_error;
 struct Node {
   nnvm::NodeAttrs attrs;
   mxnet::OpStatePtr state;
-  std::string in_names, out_names;
+  std::string in_names, out_names, grad_names;
 };
 
 #define OPS_API_BEGIN() try {
@@ -125,6 +125,24 @@ int mxq_node_input_names(void* node, const char** out) {
 int mxq_node_output_names(void* node, const char** out) {
   *out = static_cast<Node*>(node)->out_names.c_str();
   return 0;
+}
+
+int mxq_node_gradient_names(void* node, const char** out) {
+  OPS_API_BEGIN();
+  Node* n = static_cast<Node*>(node);
+  static auto& fgrad = *new auto(nnvm::Op::GetAttr<nnvm::FGradient>("FGradient"));
+  n->grad_names.clear();
+  if (fgrad.count(n->attrs.op)) {
+    nnvm::ObjectPtr fwd = nnvm::Node::Create();
+    fwd->attrs = n->attrs;
+    std::vector<std::string> names;
+    for (const nnvm::NodeEntry& e : fgrad[n->attrs.op](fwd, {}))
+      names.push_back((e.node->op() != nullptr ? e.node->op()->name : std::string("?")) + ":" +
+                      e.node->attrs.name);
+    n->grad_names = join(names);
+  }
+  *out = n->grad_names.c_str();
+  OPS_API_END();
 }
 
 int mxq_node_infer_shape(void* node, int num_in, int* in_ndim, int64_t* in_shape, int num_out,

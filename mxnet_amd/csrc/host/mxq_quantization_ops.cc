@@ -939,6 +939,7 @@ NNVM_REGISTER_OP(_contrib_quantize_v2)
     .set_attr<FNeedCalibrateInput>("FNeedCalibrateInput",
                                    [](const NodeAttrs&) { return std::vector<int>{0}; })
     .set_attr<FResourceRequest>("FResourceRequest", TempSpaceUnlessCalibrated<QuantizeV2Param>)
+    .set_attr<nnvm::FGradient>("FGradient", MakeZeroGradNodes)
     .add_argument("data", "NDArray-or-Symbol", "A ndarray/symbol of type `float32`")
     .add_arguments(QuantizeV2Param::__FIELDS__());
 
@@ -985,6 +986,7 @@ NNVM_REGISTER_OP(_contrib_requantize)
     .set_attr<FNeedCalibrateInput>("FNeedCalibrateInput",
                                    [](const NodeAttrs&) { return std::vector<int>{0}; })
     .set_attr<FResourceRequest>("FResourceRequest", TempSpaceUnlessCalibrated<RequantizeParam>)
+    .set_attr<nnvm::FGradient>("FGradient", MakeZeroGradNodes)
     .add_argument("data", "NDArray-or-Symbol", "A ndarray/symbol of type `int32`")
     .add_argument("min_range", "NDArray-or-Symbol",
                   "The original minimum scalar value in the form of float32 used for quantizing "
@@ -1010,6 +1012,7 @@ NNVM_REGISTER_OP(_contrib_dequantize)
     .set_attr<FInferStorageType>("FInferStorageType", DefaultStorageType)
     .set_attr<FCreateOpState>("FCreateOpState", CreateDequantizeState)
     .set_attr<FStatefulCompute>("FStatefulCompute<gpu>", DequantizeForwardGPU)
+    .set_attr<nnvm::FGradient>("FGradient", MakeZeroGradNodes)
     .add_argument("data", "NDArray-or-Symbol", "A ndarray/symbol of type `uint8`")
     .add_argument("min_range", "NDArray-or-Symbol",
                   "The minimum scalar value possibly produced for the input in float32")
@@ -1045,6 +1048,7 @@ NNVM_REGISTER_OP(_contrib_quantized_fully_connected)
                                 [](const NodeAttrs&) {
                                   return std::vector<ResourceRequest>{ResourceRequest::kTempSpace};
                                 })
+    .set_attr<nnvm::FGradient>("FGradient", MakeZeroGradNodes)
     .add_argument("data", "NDArray-or-Symbol", "Input data.")
     .add_argument("weight", "NDArray-or-Symbol", "weight.")
     .add_argument("bias", "NDArray-or-Symbol", "bias.")
@@ -1085,6 +1089,7 @@ NNVM_REGISTER_OP(_contrib_quantized_conv)
                                 })
     .set_attr<FNeedRequantize>("FNeedRequantize", [](const NodeAttrs&) { return true; })
     .set_attr<FCompute>("FCompute<gpu>", QuantizedConvForwardGPU)
+    .set_attr<nnvm::FGradient>("FGradient", MakeZeroGradNodes)
     .add_argument("data", "NDArray-or-Symbol", "Input data.")
     .add_argument("weight", "NDArray-or-Symbol", "weight.")
     .add_argument("bias", "NDArray-or-Symbol", "bias.")

@@ -405,12 +405,27 @@ typedef std::function<std::vector<uint32_t>(const NodeAttrs&)> FMutateInputs;
 
 // What FQuantizedOp hands back in the reference is a graph node; only its attributes
 // (operator, name, dict, parsed struct) are ever looked at.
+struct Node;
+typedef std::shared_ptr<Node> ObjectPtr;
+// include/nnvm/node.h: output `index` of `node`
+struct NodeEntry {
+  ObjectPtr node;
+  uint32_t index = 0;
+  uint32_t version = 0;
+};
 struct Node {
   NodeAttrs attrs;
+  std::vector<NodeEntry> inputs;
+  std::vector<ObjectPtr> control_deps;
   const Op* op() const { return attrs.op; }
+  uint32_t num_inputs() const {
+    return attrs.op != nullptr ? attrs.op->NumInputs(attrs) : static_cast<uint32_t>(inputs.size());
+  }
   static std::shared_ptr<Node> Create() { return std::make_shared<Node>(); }
 };
-typedef std::shared_ptr<Node> ObjectPtr;
+// include/nnvm/op_attr_types.h: the gradient of a node as new nodes, one entry per input
+typedef std::function<std::vector<NodeEntry>(const ObjectPtr&, const std::vector<NodeEntry>&)>
+    FGradient;
 
 }  // namespace nnvm
 
@@ -449,6 +464,26 @@ typedef std::function<bool(const NodeAttrs&, const size_t, const std::string)> F
 typedef std::function<bool(const NodeAttrs&, const size_t)> FAvoidDequantizeOutput;
 
 namespace op {
+
+// src/operator/operator_common.h:430-444: the quantized operators are inference-only, their
+// gradient with respect to every input is a zeros_like node named after the forward node.
+inline std::vector<nnvm::NodeEntry> MakeZeroGradNodes(const nnvm::ObjectPtr& n,
+                                                      const std::vector<nnvm::NodeEntry>&) {
+  const uint32_t count = n->num_inputs();
+  std::vector<nnvm::NodeEntry> grads;
+  for (uint32_t i = 0; i < count; ++i) {
+    nnvm::ObjectPtr z = nnvm::Node::Create();
+    z->attrs.op = nnvm::Op::Find("zeros_like");
+    z->attrs.name = n->attrs.name + (count == 1 ? std::string("_backward")
+                                                 : "_in" + std::to_string(i) + "_backward");
+    if (i < n->inputs.size()) z->inputs.push_back(n->inputs[i]);
+    z->control_deps.push_back(n);
+    nnvm::NodeEntry e;
+    e.node = z;
+    grads.push_back(e);
+  }
+  return grads;
+}
 
 struct InferShapeError : public dmlc::Error {
   int index;

@@ -719,7 +719,10 @@ template <typename T>
 void launch_transpose(hipStream_t s, const void* in, void* out, int B, int R, int S, int RP) {
   if (B == 0 || RP == 0 || S == 0) return;
   MXQ_CHECK(RP >= R, "padded extent below the extent");
-  MXQ_CHECK(B <= 65535 && (RP + 63) / 64 <= 65535, "transpose grid too large");
+  // only the kernels that put batches and row tiles on grid.y / grid.z have their limit
+  auto check_yz = [&]() {
+    MXQ_CHECK(B <= 65535 && (RP + 63) / 64 <= 65535, "transpose grid too large");
+  };
   if (sizeof(T) == 1 && S % 16 == 0 && S >= 128 && RP >= 128 && RP % 4 == 0 && RP % 16 != 0 &&
       aligned16(in) && (reinterpret_cast<uintptr_t>(out) & 3u) == 0) {
     launch_wide<4>(s, in, out, B, R, S, RP);
@@ -733,6 +736,7 @@ void launch_transpose(hipStream_t s, const void* in, void* out, int B, int R, in
       launch_wide<16>(s, in, out, B, R, S, RP);
       return;
     }
+    check_yz();
     dim3 grid128((S + 127) / 128, (RP + 63) / 64, B);
     hipLaunchKernelGGL(transpose_i8_kernel, grid128, dim3(256), 0, s,
                        static_cast<const uint8_t*>(in), static_cast<uint8_t*>(out), R, S, RP);
@@ -756,6 +760,7 @@ void launch_transpose(hipStream_t s, const void* in, void* out, int B, int R, in
     }
     if (thin_in || thin_out) {
       const int L = thin_in ? R : S, thin = thin_in ? S : R;
+      MXQ_CHECK(B <= 65535, "transpose grid too large");
       dim3 grid(L / 128, B);
       if (thin_in)
         hipLaunchKernelGGL(transpose_i8_thin_kernel<true>, grid, dim3(256), 0, s,
@@ -767,6 +772,7 @@ void launch_transpose(hipStream_t s, const void* in, void* out, int B, int R, in
       return;
     }
   }
+  check_yz();
   dim3 grid((S + 63) / 64, (RP + 63) / 64, B);
   hipLaunchKernelGGL((transpose_kernel<T>), grid, dim3(256), 0, s, static_cast<const T*>(in),
                      static_cast<T*>(out), R, S, RP);
@@ -1023,6 +1029,7 @@ int mxq_quantized_conv_nhwc(void* stream, const int8_t* data, const int8_t* weig
   MXQ_API_END();
 }
 
+#ifdef MXQ_TEST_HOOKS
 // Test-only twin of mxq_quantized_conv_nhwc (declared in tests/mxq_test_hooks.h): the tile
 // configuration and the split-K factor come as arguments (0 = let the launcher choose).
 int mxq_test_quantized_conv_nhwc(void* stream, const int8_t* data, const int8_t* weight,
@@ -1047,6 +1054,7 @@ int mxq_test_quantized_conv_nhwc(void* stream, const int8_t* data, const int8_t*
             out32, omin, omax, out8, rmin, rmax, relu, min_calib, max_calib, false, force, ws);
   MXQ_API_END();
 }
+#endif  // MXQ_TEST_HOOKS
 
 int mxq_quantized_conv_nhwc_out_nchw(void* stream, const int8_t* data, const int8_t* weight,
                                      const int8_t* bias, int N, int H, int W, int C, int O,

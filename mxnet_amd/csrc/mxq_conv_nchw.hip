@@ -854,6 +854,7 @@ int mxq_quantized_conv_nchw(void* stream, const int8_t* data, const int8_t* weig
   MXQ_API_END();
 }
 
+#ifdef MXQ_TEST_HOOKS
 // Test-only twin (declared in tests/mxq_test_hooks.h): cfg 1 pins the route through the
 // layout adapters, 71 ... 78 a tile of the NCHW kernel, 0 leaves the choice to the launcher.
 int mxq_test_quantized_conv_nchw(void* stream, const int8_t* data, const int8_t* weight,
@@ -870,5 +871,6 @@ int mxq_test_quantized_conv_nchw(void* stream, const int8_t* data, const int8_t*
             out32, omin, omax, workspace, workspace_bytes, cfg);
   MXQ_API_END();
 }
+#endif  // MXQ_TEST_HOOKS
 
 }  // extern "C"

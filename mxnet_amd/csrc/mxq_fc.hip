@@ -193,11 +193,17 @@ void launch_fc(hipStream_t s, const int8_t* data, const int8_t* weight, int M, i
 }
 
 // Scratch bytes with which launch_fc takes its fastest route for this shape (0 when it
-// would not split).  Assumes 16-byte aligned operands.
+// would not split).  Assumes 16-byte aligned operands.  The residual-sum form plans its tile
+// on its own (plan_fc's `sum`), so the figure is the larger of the two plans: a workspace
+// sized by this query serves mxq_quantized_fc and mxq_quantized_fc_sum alike.
 size_t fc_workspace_bytes(int M, int N, int K, bool fused8) {
   if (M <= 0 || N <= 0 || K <= 0) return 0;
-  const FcPlan plan = plan_fc(M, N, K, K % 16 == 0, fused8, GemmForce());
-  return fc_plan_workspace(plan, M, N);
+  const size_t plain =
+      fc_plan_workspace(plan_fc(M, N, K, K % 16 == 0, fused8, GemmForce(), false), M, N);
+  if (!fused8) return plain;
+  const size_t sum =
+      fc_plan_workspace(plan_fc(M, N, K, K % 16 == 0, true, GemmForce(), true), M, N);
+  return plain > sum ? plain : sum;
 }
 
 }  // namespace mxq
@@ -302,6 +308,7 @@ int mxq_quantized_fc(void* stream, const int8_t* data, const int8_t* weight, con
   MXQ_API_END();
 }
 
+#ifdef MXQ_TEST_HOOKS
 // Test-only twin of mxq_quantized_fc (declared in tests/mxq_test_hooks.h, not in the
 // operator header): the tile configuration, the split-K factor and the streaming kernel's
 // work-groups per CU come as arguments (0 = let the launcher choose), so tests can drive
@@ -324,6 +331,7 @@ int mxq_test_quantized_fc(void* stream, const int8_t* data, const int8_t* weight
            max_calib, workspace, workspace_bytes, force);
   MXQ_API_END();
 }
+#endif  // MXQ_TEST_HOOKS
 
 int mxq_quantized_fc_f32(void* stream, const int8_t* data, const int8_t* weight,
                          const int8_t* bias, int M, int N, int K, const float* min_data,
@@ -357,6 +365,7 @@ int mxq_quantized_fc_sum(void* stream, const int8_t* data, const int8_t* weight,
   MXQ_API_END();
 }
 
+#ifdef MXQ_TEST_HOOKS
 // Test-only twin of mxq_quantized_fc_sum with the kernel variant pinned
 // (tests/mxq_test_hooks.h).
 int mxq_test_quantized_fc_sum(void* stream, const int8_t* data, const int8_t* weight,
@@ -381,7 +390,9 @@ int mxq_test_quantized_fc_sum(void* stream, const int8_t* data, const int8_t* we
            max_calib, workspace, workspace_bytes, force, &sum);
   MXQ_API_END();
 }
+#endif  // MXQ_TEST_HOOKS
 
+#ifdef MXQ_TEST_HOOKS
 // Test-only twin of mxq_quantized_fc_f32 with the tile configuration and the split-K factor
 // pinned (tests/mxq_test_hooks.h).
 int mxq_test_quantized_fc_f32(void* stream, const int8_t* data, const int8_t* weight,
@@ -403,5 +414,6 @@ int mxq_test_quantized_fc_f32(void* stream, const int8_t* data, const int8_t* we
            min_calib, max_calib, workspace, workspace_bytes, force);
   MXQ_API_END();
 }
+#endif  // MXQ_TEST_HOOKS
 
 }  // extern "C"

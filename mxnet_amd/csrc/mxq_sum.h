@@ -1,8 +1,11 @@
-// The residual sum as an epilogue step: int8 + int8 -> int8 over a calibrated range, the
-// arithmetic of _contrib_quantized_elemwise_add (src/operator/quantization/
-// quantized_elemwise_add.cc:30-134, dnnl/dnnl_quantized_elemwise_add.cc:134-257) restated
-// exactly as add_kernel in mxq_eltwise.hip evaluates it, optionally followed by the int8
-// relu of _contrib_quantized_act (quantized_activation.cc:84-120).  A kernel that holds the
+// The residual sum as an epilogue step: int8 + int8 -> int8 over a calibrated range,
+// optionally followed by the int8 relu of _contrib_quantized_act
+// (quantized_activation.cc:84-120).  It mirrors add_kernel in mxq_eltwise.hip and the CPU
+// oracle bit for bit.  The scales come from the reference's own files
+// (src/operator/quantization/quantized_elemwise_add.cc:30-134,
+// dnnl/dnnl_quantized_elemwise_add.cc:134-257); the element arithmetic itself (two float
+// products, one sum, nearest-even, saturation, NaN -> 0) happens inside oneDNN in the
+// reference and is not pinned by anything in its tree: parity unpinned, as for add_kernel.  A kernel that holds the
 // left operand in registers applies it to 16-byte pieces on their way out.
 #ifndef MXQ_SUM_H_
 #define MXQ_SUM_H_

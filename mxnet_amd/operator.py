@@ -42,6 +42,7 @@ OPS_SIGNATURES = {
     "mxq_node_num_outputs": (_i, [_p, _pi]),
     "mxq_node_input_names": (_i, [_p, _pps]),
     "mxq_node_output_names": (_i, [_p, _pps]),
+    "mxq_node_gradient_names": (_i, [_p, _pps]),
     "mxq_node_infer_shape": (_i, [_p, _i, _pi, _pl, _i, _pi, _pl]),
     "mxq_node_infer_type": (_i, [_p, _i, _pi, _i, _pi]),
     "mxq_node_temp_bytes": (_i, [_p, _i, _pb, _i, _pb, ctypes.POINTER(_sz)]),
@@ -143,6 +144,12 @@ class Node:
         s = ctypes.c_char_p()
         _check(ops.mxq_node_output_names(self._h, ctypes.byref(s)))
         return s.value.decode().split(",") if s.value else []
+
+    def gradient_nodes(self):
+        """(operator, node name) of the gradient node FGradient makes for every input."""
+        s = ctypes.c_char_p()
+        _check(ops.mxq_node_gradient_names(self._h, ctypes.byref(s)))
+        return [tuple(x.split(":", 1)) for x in s.value.decode().split(",")] if s.value else []
 
     def infer_shape(self, in_shapes, out_shapes=None):
         """Shapes are tuples or None (unknown).  Returns (in_shapes, out_shapes)."""

@@ -108,3 +108,21 @@ def test_bench_refuses_more_than_one_gpu():
     r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"],
                        capture_output=True, text=True, timeout=120)
     assert r.returncode == 2 and "one GPU" in r.stderr
+
+
+def test_fc_workspace_query_covers_both_epilogue_forms():
+    """mxq_quantized_fc_workspace is host arithmetic: the fused-int8 figure is what both
+    mxq_quantized_fc and mxq_quantized_fc_sum (which plans its own tile) may ask for, so it is
+    never below the int32 form's figure where both split."""
+    import mxnet_amd
+    lib = mxnet_amd._lib.lib
+    import random
+    rnd = random.Random(5)
+    for _ in range(200):
+        M, N, K = rnd.choice([1, 64, 256, 4096, 50176]), rnd.choice([64, 256, 800, 4096]), \
+            rnd.choice([64, 576, 4096, 8192, 25088])
+        fused = lib.mxq_quantized_fc_workspace(M, N, K, 1)
+        plain = lib.mxq_quantized_fc_workspace(M, N, K, 0)
+        assert fused % 256 == 0 and plain % 256 == 0
+        assert fused >= plain or plain == 0 or fused == 0
+    assert lib.mxq_quantized_fc_workspace(4096, 4096, 4096, 1) == 0

@@ -39,6 +39,22 @@ def test_registry_names_aliases_and_gpu_attributes():
         Node("_contrib_does_not_exist")
 
 
+def test_inference_only_operators_have_zero_gradients():
+    """FGradient = MakeZeroGradNodes on the five operators (quantize_v2.cc:108, requantize.cc:94,
+    dequantize.cc:95, quantized_fully_connected.cc:362, quantized_conv.cc:221): one zeros_like
+    node per input, named as operator_common.h:430-444 names them."""
+    for n in ["_contrib_quantize_v2", "_contrib_requantize", "_contrib_dequantize",
+              "_contrib_quantized_fully_connected", "_contrib_quantized_conv"]:
+        assert op.has_attr(n, "FGradient")
+    q = Node("_contrib_quantize_v2", name="q0", out_type="int8")
+    assert q.gradient_nodes() == [("zeros_like", "q0_backward")]
+    fc = Node("_contrib_quantized_fully_connected", name="fc1", num_hidden=8, no_bias=True)
+    assert fc.gradient_nodes() == [("zeros_like", "fc1_in%d_backward" % i) for i in range(6)]
+    conv = Node("_contrib_quantized_conv", name="c", kernel=(1, 1), num_filter=8)
+    assert len(conv.gradient_nodes()) == 9 and conv.gradient_nodes()[8][1] == "c_in8_backward"
+    assert Node("_contrib_quantized_act", act_type="relu").gradient_nodes() == []
+
+
 def test_input_output_names():
     n = Node("_contrib_quantized_fully_connected", num_hidden=8)
     assert n.num_inputs == 9 and n.num_outputs == 3
