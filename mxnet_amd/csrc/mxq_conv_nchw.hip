@@ -636,11 +636,15 @@ NchwPlan plan_nchw(int N, int C, int H, int W, int O, int KH, int KW, int sh, in
       pl.gather_mode = mode;
       return pl;
     }
-    pl.route = Route::kPlanesPrepass;
-    pl.pitch = static_cast<int>(pitch);
-    pl.row_stride = static_cast<int>(row);
-    pl.d_bytes = up256(static_cast<size_t>(C) * row);
-    return pl;
+    // (a pre-pass in front of a very long reduction over few pixels loses to the adapters,
+    // whose kernel has the deeper stages: 2048 -> 512 at 7 x 7 24.8 against 21.6 us)
+    if (!(C >= 2048 && 1LL * N * P <= 4096)) {
+      pl.route = Route::kPlanesPrepass;
+      pl.pitch = static_cast<int>(pitch);
+      pl.row_stride = static_cast<int>(row);
+      pl.d_bytes = up256(static_cast<size_t>(C) * row);
+      return pl;
+    }
   }
   // a stride-2 convolution over at most 4 channels (an image stem) runs as the unit-stride
   // convolution over the space-to-depth form of its operands: 4 * C real channels out of 16
@@ -755,24 +759,24 @@ void conv_nchw(void* stream, const int8_t* data, const int8_t* weight, const int
       auto tiles = [&](int bp, int bo) {
         return rows * ((cols + bp - 1) / bp) * ((O + bo - 1) / bo);
       };
-      auto padded = [&](int bp) { return (cols + bp - 1) / bp * bp; };
-      if (C >= 256 && O >= 256 && 100 * padded(256) <= 104 * padded(128) &&
-          16 * tiles(256, 256) >= 9 * cus) {
-        pick = 78;  // a real GEMM: the wave tile whose LDS traffic the matrix pipe can hide
-      } else if (C >= 256 && O >= 128 && 100 * padded(256) <= 104 * padded(128) &&
+      auto padded = [&](int bp) { return rows * ((cols + bp - 1) / bp * bp); };
+      // From per-layer sweeps of every tile on the ResNet-50 layers at batch 64 (operands
+      // rotated): 64 output channels take the 128 x 64 tile; a layer with a long reduction
+      // whose 256 x 128 tiles cover three quarters of the chip takes those (256 -> 128 / 2:
+      // 19.8 us against 20.9; 512 -> 2048 at 7 x 7: 19.6 against 22); everything else
+      // 128 x 128, shrunk to 64 pixels and then 64 channels while there is less than one
+      // tile per CU (1024 -> 512 at 7 x 7: 16.3 us on 64 x 64 against 19.2).  The 256-column
+      // tiles never measured ahead by more than the run-to-run spread.
+      if (O <= 64) {
+        pick = (tiles(128, 64) >= cus || cols > 64) ? 72 : 74;
+      } else if (C >= 256 && 100 * padded(256) <= 104 * padded(128) &&
                  4 * tiles(256, 128) >= 3 * cus) {
         pick = 77;
       } else {
-        // pixel tile: 128 unless 64 wastes clearly fewer MFMA rows on the last tile;
-        // channel tile: the widest that still gives every CU two work-groups
-        int bp = (cols <= 64 || 100 * padded(64) < 96 * padded(128)) ? 64 : 128;
-        int bo = 64;
-        if (O > 64) {
-          bo = 128;
-          if (bp == 128 && O >= 256 && tiles(128, 256) >= 2 * cus) bo = 256;
-          if (bp == 128 && tiles(128, bo) < cus) bp = 64;
-        }
-        pick = bp == 128 ? (bo == 64 ? 72 : (bo == 128 ? 71 : 75)) : (bo == 64 ? 74 : 73);
+        int bp = 128, bo = 128;
+        if (tiles(bp, bo) < cus) bp = 64;
+        if (tiles(bp, bo) < cus) bo = 64;
+        pick = bp == 128 ? 71 : (bo == 128 ? 73 : 74);
       }
     }
     switch (pick) {
