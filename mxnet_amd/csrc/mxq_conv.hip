@@ -457,6 +457,203 @@ void launch_conv3x3_rows(hipStream_t s, const ConvArgs& a) {
   MXQ_LAUNCH_CHECK();
 }
 
+// ---- 3 x 3 convolution with the input patch resident in LDS -------------------------
+// The implicit GEMM above stages every input pixel nine times, once per tap, through the
+// CU's 64 bytes per clock from L1 into LDS, which is what bounds every tile below 256 x 256.
+// Here a work-group takes 128 consecutive output pixels (in (n, oh, ow) order, regardless
+// of where a row or an image ends) and 128 output channels, brings the input rows those
+// pixels touch into LDS ONCE -- "virtual rows" n * (H + 2) + ih + 1, so that the zero rows
+// above and below an image are rows like any other and a tile that passes from one image
+// to the next still reads a contiguous range -- and forms the nine taps' activation
+// fragments by address arithmetic: the patch pixel of output pixel (n, oh, ow) under tap
+// (kh, kw) is pp0 + kh * (W + 2) + kw.  Only the weights go through the stage ring (128
+// rows x 128 bytes per stage: one tap's 128 channels), so a K step moves half the bytes of
+// the implicit GEMM's and the ring is half as large: two work-groups of 8 waves share a CU
+// and one's loads and epilogue overlap the other's MFMAs.  Stride 1, pad 1, no dilation,
+// C a multiple of 128; int8 fused or int32 output through the common epilogue.
+constexpr int kPatchBytes = 40 * 1024;   // room for the patch of one tile
+#ifdef MXQ_STAMPS
+__device__ long long mxq_dbg_stamps[8 * 4096];
+#define MXQ_STAMP(k)                                                                  \
+  do {                                                                                \
+    if (lane == 0 && wave == 0 && blockIdx.x < 4096)                                  \
+      mxq_dbg_stamps[blockIdx.x * 8 + (k)] = __builtin_readcyclecounter();            \
+  } while (0)
+#else
+#define MXQ_STAMP(k)
+#endif
+typedef GemmCfg<128, 128, 128, 4, 2> CfgPatch;  // 8 waves, wave tile 32 pixels x 64 channels
+
+template <int NS>
+__global__ __launch_bounds__(512, 2) void conv3x3_patch_kernel(ConvArgs p) {
+  typedef CfgPatch Cfg;
+  constexpr int BM = Cfg::BM, BN = Cfg::BN, BK = Cfg::BK, CHW = Cfg::CH;   // CHW: chunks per weight row of a stage
+  constexpr int NW = 8, BI = Cfg::B_CHUNKS, KS = Cfg::KS, NI = Cfg::NI;
+  constexpr int STAGE_BYTES = BN * BK, RING_BYTES = NS * STAGE_BYTES;
+  static_assert(Cfg::MI == 1 && NI == 2 && BI == 2, "wave tile 32 x 64");
+  __shared__ __attribute__((aligned(16))) v4i lds[(kPatchBytes + RING_BYTES) / 16];
+  char* patch = reinterpret_cast<char*>(lds);
+  char* ring = patch + kPatchBytes;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave / Cfg::WN, wn = wave % Cfg::WN;
+  MXQ_STAMP(4);
+  const int tiles_m = (p.M + BM - 1) / BM, tiles_n = (p.O + BN - 1) / BN;
+  // channel tiles of one pixel tile are neighbours (they share the patch's cache lines)
+  const int lid = xcd_remap(blockIdx.x, tiles_m * tiles_n);
+  const int tn = lid % tiles_n, tm = lid / tiles_n;
+  const int m0 = tm * BM, n0 = tn * BN;
+  const int PW = p.W + 2, CH = p.C >> 4;   // patch pixels per row, 16-byte chunks per pixel
+  const int ohow = p.OH * p.OW;
+
+  // the range of virtual rows this tile touches
+  const int ma = m0, mb = (m0 + BM - 1 < p.M) ? m0 + BM - 1 : p.M - 1;
+  const int na = ma / ohow, oha = (ma - na * ohow) / p.OW;
+  const int nb = mb / ohow, ohb = (mb - nb * ohow) / p.OW;
+  const int vr0 = na * (p.H + 2) + oha;
+  const int rows = nb * (p.H + 2) + ohb + 2 - vr0 + 1;
+
+  // The patch: a row of it is RP pixels (the W + 2 real ones padded so that a row is whole
+  // load instructions of 64 slots: the row of an instruction is then wave-uniform and no lane
+  // divides anything), chunk j of patch pixel pp at slot pp * CH + (j ^ patch_swz(pp)).  A
+  // fragment read is 16 consecutive pixels per LDS pass; with 128-byte pixels two of them
+  // fill the banks once, so the XOR advances every second pixel, with wider pixels every one.
+  const int ch_shift = __builtin_ctz(CH);
+  const int per_row = (PW * CH + 63) >> 6;        // load instructions per patch row
+  const int RP = (per_row << 6) >> ch_shift;      // pixels per patch row
+  const int swz_shift = CH == 8 ? 1 : 0;
+  auto patch_swz = [&](int pixel) { return (pixel >> swz_shift) & (CH - 1); };
+  {
+    const v4i rsrc = make_rsrc(p.data, static_cast<uint32_t>(p.N) * p.H * p.W * p.C);
+    const uint32_t patch_addr = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(patch));
+    const int instrs = rows * per_row;
+    for (int it = wave; it < instrs; it += NW) {
+      const int r = it / per_row, part = it - r * per_row;    // wave-uniform
+      const int vabs = vr0 + r;
+      const int n = vabs / (p.H + 2), ih = vabs - n * (p.H + 2) - 1;
+      const bool row_ok = n < p.N && static_cast<unsigned>(ih) < static_cast<unsigned>(p.H);
+      const int q = part * 64 + lane;                          // slot inside the row
+      const int px = q >> ch_shift, pp = r * RP + px;
+      const int j = (q & (CH - 1)) ^ patch_swz(pp);
+      const int iw = px - 1;
+      const bool ok = row_ok && static_cast<unsigned>(iw) < static_cast<unsigned>(p.W);
+      const uint32_t off =
+          ok ? static_cast<uint32_t>(((n * p.H + ih) * p.W + iw) * p.C + 16 * j) : kOutOfRange;
+      dma_buffer(patch_addr + it * 1024, off, rsrc);
+    }
+  }
+  // the weights: stage s = tap s / (C / BK), channel block s % (C / BK); OHWI rows are K-contiguous
+  RowIssuerBuffer<Cfg, BI> bi;
+  bi.init(p.weight, n0, p.O, p.K, wave, lane, 0);
+  const uint32_t ring_addr = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(ring));
+  const int KT = p.K / BK;
+  auto issue = [&](int stage) {
+    if (stage >= KT) return;
+    const uint32_t sb = ring_addr + static_cast<uint32_t>(stage % NS) * STAGE_BYTES;
+#pragma unroll
+    for (int j = 0; j < BI; ++j) bi.issue(j, stage, sb + (j * NW + wave) * 1024);
+  };
+#pragma unroll
+  for (int st = 0; st < NS - 1; ++st) issue(st);
+  MXQ_STAMP(5);
+  EpiPre pre = epi_prefetch<Cfg>(p.epi, n0, p.O);
+  MXQ_STAMP(6);
+
+  // this lane's output pixel and its patch pixel under tap (0, 0)
+  const int frow = lane & 31, fgrp = lane >> 5;
+  int m = m0 + wm * Cfg::TM + frow;
+  m = m < p.M ? m : p.M - 1;   // rows past the end repeat the last pixel; never stored
+  const int n = m / ohow, rem = m - n * ohow;
+  const int oh = rem / p.OW, ow = rem - oh * p.OW;
+  const int pp0 = (n * (p.H + 2) + oh - vr0) * RP + ow;
+  const int rb = wn * Cfg::TN + frow;
+  int fb0[KS];
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) fb0[ks] = rb * CHW + ((ks * 2 + fgrp) ^ swz<CHW>(rb));
+
+  v16i acc[1][NI];
+#pragma unroll
+  for (int ni = 0; ni < NI; ++ni)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) acc[0][ni][v] = 0;
+
+  const int blocks = p.C / BK;   // stages per tap
+  int tap = 0, cblk = 0, pp = pp0;   // of the stage computed next
+  MXQ_STAMP(0);
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the patch and the first stages
+  MXQ_STAMP(1);
+  for (int kt = 0; kt < KT; ++kt) {
+    if (kt > 0) {
+      const int newest = (kt + NS - 2) < (KT - 1) ? (kt + NS - 2) : (KT - 1);
+      wait_ahead<BI, NS - 2>(newest - kt);
+    }
+    __builtin_amdgcn_s_barrier();
+    issue(kt + NS - 1);
+    const v4i* sbw = reinterpret_cast<const v4i*>(ring + (kt % NS) * STAGE_BYTES);
+    const v4i* pix = reinterpret_cast<const v4i*>(patch) + pp * CH;
+    const int sw_ = patch_swz(pp);
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const v4i fa = pix[(cblk * (BK / 16) + ks * 2 + fgrp) ^ sw_];
+      v4i fb[NI];
+#pragma unroll
+      for (int ni = 0; ni < NI; ++ni) fb[ni] = sbw[fb0[ks] + ni * 32 * CHW];
+#pragma unroll
+      for (int ni = 0; ni < NI; ++ni)
+        acc[0][ni] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fb[ni], fa, acc[0][ni], 0, 0, 0);
+    }
+    if (++cblk == blocks) {
+      cblk = 0;
+      ++tap;
+      const int kh = tap / 3, kw = tap - 3 * kh;
+      pp = pp0 + kh * RP + kw;
+    }
+  }
+  MXQ_STAMP(2);
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  if (blockIdx.x == 0 && tid == 0) epilogue_ranges(p.epi);
+  gemm_epilogue_lds<Cfg, kPatchBytes + RING_BYTES>(acc, p.epi, pre, m0, n0, p.M, p.O,
+                                                   static_cast<size_t>(p.O), lds);
+  MXQ_STAMP(3);
+}
+
+#ifdef MXQ_STAMPS
+extern "C" int mxq_dbg_read_stamps(long long* host, int count) {
+  return hipMemcpyFromSymbol(host, HIP_SYMBOL(mxq_dbg_stamps), sizeof(long long) * count) ==
+                 hipSuccess
+             ? 0
+             : -1;
+}
+#endif
+
+// Virtual rows the patch of a 128-pixel tile can span: the rows its pixels lie in, one
+// above, one below, and two halo rows for every image boundary inside the tile.
+inline int conv3x3_patch_rows(int OH, int OW) {
+  const int out_rows = (128 + OW - 2) / OW + 1;
+  const int crossings = (128 + OH * OW - 2) / (OH * OW);
+  return out_rows + 2 + 2 * crossings;
+}
+
+bool conv3x3_patch_ok(const ConvArgs& a) {
+  const long long data_bytes = static_cast<long long>(a.N) * a.H * a.W * a.C;
+  const int ch = a.C / 16;
+  return a.KH == 3 && a.KW == 3 && a.sh == 1 && a.sw == 1 && a.ph == 1 && a.pw == 1 &&
+         a.dh == 1 && a.dw == 1 && a.C % 128 == 0 && (ch & (ch - 1)) == 0 && a.O % 16 == 0 &&
+         aligned16(a.data) && aligned16(a.weight) && data_bytes < (1LL << 31) &&
+         static_cast<long long>(a.O) * a.K < (1LL << 31) &&
+         // (a patch row is whole load instructions of 1 KiB)
+         static_cast<long long>(conv3x3_patch_rows(a.OH, a.OW)) *
+                 (((a.W + 2) * ch + 63) / 64 * 1024) <=
+             kPatchBytes;
+}
+
+void launch_conv3x3_patch(hipStream_t s, const ConvArgs& a) {
+  const long tiles = static_cast<long>((a.M + 127) / 128) * ((a.O + 127) / 128);
+  hipLaunchKernelGGL(conv3x3_patch_kernel<2>, dim3(static_cast<unsigned>(tiles)), dim3(512), 0, s,
+                     a);
+  MXQ_LAUNCH_CHECK();
+}
+
 typedef GemmCfg<256, 256, 64, 2, 4> CfgL8;   // 8 waves, wave tile 128 x 64
 typedef GemmCfg<256, 128, 64, 4, 2> CfgW128; // 8 waves, wave tile 64 x 64
 typedef GemmCfg<256, 64, 64, 4, 1> CfgW64;   // 4 waves, wave tile 64 x 64
@@ -953,6 +1150,16 @@ void conv_nhwc(void* stream, const int8_t* data, const int8_t* weight, const int
     MXQ_CHECK(conv3x3_rows_ok(a), "shape does not qualify for the parked-weights 3x3 kernel");
     MXQ_CHECK(plan.splits <= 1 || force.splits == 0, "the 3x3 row kernel has no split-K form");
     launch_conv3x3_rows(s, a);
+    return;
+  }
+  // 62: the resident-patch 3 x 3 kernel; chosen where it was measured ahead of the tiled
+  // kernels (28 x 28 planes over 128 channels at batch 64: 15.4 against 16.6 us of kernel time)
+  const long patch_tiles = static_cast<long>((a.M + 127) / 128) * ((a.O + 127) / 128);
+  if (plan.cfg == 62 || (force.cfg == 0 && plan.splits <= 1 && conv3x3_patch_ok(a) &&
+                         patch_tiles >= num_cus())) {
+    MXQ_CHECK(conv3x3_patch_ok(a), "shape does not qualify for the resident-patch 3x3 kernel");
+    MXQ_CHECK(plan.splits <= 1 || force.splits == 0, "the patch kernel has no split-K form");
+    launch_conv3x3_patch(s, a);
     return;
   }
   const int cfg = plan.cfg, sp = plan.splits;

@@ -162,6 +162,44 @@ def test_conv3x3_parked_weights(capi, N, H, W, relu, use_bias, forced):
     assert (res["rmin"].item(), res["rmax"].item()) == (qmn, qmx)
 
 
+# the resident-patch 3 x 3 kernel (C a multiple of 128): whole planes smaller than a tile
+# (several images and their zero rows inside one patch), rows that straddle tiles, one
+# column, the last tile short, output channels off the tile, int32 and fused int8 outputs
+@pytest.mark.parametrize("N,C,H,W,O", [(2, 128, 28, 28, 128), (4, 128, 6, 14, 128),
+                                       (3, 128, 9, 6, 64), (3, 128, 28, 28, 144),
+                                       (40, 128, 6, 6, 32), (2, 128, 31, 29, 48),
+                                       (1, 128, 8, 20, 16)])
+@pytest.mark.parametrize("fused", [True, False])
+def test_conv3x3_resident_patch(capi, N, C, H, W, O, fused, cfg=62):
+    d = int8_uniform((N, C, H, W), seed=N + H + W)
+    w = int8_uniform((O, C, 3, 3), seed=H + 1, lo=-50, hi=50)
+    b = int8_uniform((O,), seed=W + 2)
+    ro, rmn, rmx = oracle.quantized_conv(d, w, b, -1.0, 1.0, -1.0, 1.0, -1.0, 1.0, (1, 1), (1, 1),
+                                         (1, 1))
+    fl = ro.astype(np.float64) * (float(rmx) / 2147483648.0)
+    R = float(np.percentile(np.abs(fl), 98.0)) or 1.0
+    res = run_conv_nchw(capi, d, w, b, 1.0, 1.0, 1.0, (1, 1), (1, 1), (1, 1),
+                        calib=(-R, 0.9 * R) if fused else None, relu=fused, force=(cfg, 1),
+                        want_int32=not fused)
+    assert (res["omin"].item(), res["omax"].item()) == (rmn, rmx)
+    if fused:
+        rq, qmn, qmx = oracle.requantize(ro, rmn, rmx, -R, 0.9 * R)
+        np.testing.assert_array_equal(res["out8_nchw"].cpu().numpy(), oracle.relu_i8(rq))
+    else:
+        np.testing.assert_array_equal(res["out32_nchw"].cpu().numpy(), ro)
+
+
+def test_conv3x3_resident_patch_refuses_other_shapes(capi):
+    import mxnet_amd
+    # C off 128; patches past their room (long rows; 1 x 1 planes: 128 images per tile)
+    for shape in [(1, 64, 8, 8), (1, 128, 8, 600), (2, 256, 14, 14), (3, 128, 1, 1)]:
+        d = int8_uniform(shape, seed=1)
+        w = int8_uniform((64, shape[1], 3, 3), seed=2)
+        with pytest.raises(mxnet_amd._lib.MXQError, match="resident-patch"):
+            run_conv_nchw(capi, d, w, None, 1.0, 1.0, 1.0, (1, 1), (1, 1), (1, 1),
+                          calib=(-1.0, 1.0), force=(62, 1), want_int32=False)
+
+
 def test_conv3x3_parked_weights_refuses_other_shapes(capi):
     import mxnet_amd
     d = int8_uniform((1, 32, 8, 8), seed=1)
