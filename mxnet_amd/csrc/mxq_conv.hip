@@ -691,6 +691,35 @@ void launch_cfg(hipStream_t s, const ConvArgs& a, bool aligned) {
 }
 
 // ---- layout adapters ------------------------------------------------------------
+// A second, small transpose that rides along in the launch of a large one: the weights of
+// a convolution ([O][C][taps] -> [O][taps][C]) next to its data.  A launch of its own costs
+// 4.6-5.9 us inside a network however little it moves (launch, then a cold round trip to
+// memory), which for four 3 x 3 layers was 20 us of a 520 us pass.  [B][R][S] -> [B][S][R]
+// with 16 | R and S small: a thread gathers 16 bytes S apart and stores them as one piece.
+struct SmallJob {
+  const uint8_t* in;
+  uint8_t* out;
+  int R, S;
+  unsigned pieces;   // B * S * R / 16; 0 = no job
+};
+
+__device__ __forceinline__ void small_transpose_job(const SmallJob& j, unsigned block,
+                                                    unsigned nblocks) {
+  typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+  const unsigned per_row = static_cast<unsigned>(j.R) >> 4;     // pieces per output row [b][s]
+  for (unsigned t = block * 256u + threadIdx.x; t < j.pieces; t += nblocks * 256u) {
+    const unsigned row = t / per_row, k = t - row * per_row;    // row = b * S + s
+    const unsigned b = row / static_cast<unsigned>(j.S), s = row - b * j.S;
+    const uint8_t* src = j.in + (static_cast<size_t>(b) * j.R + 16 * k) * j.S + s;
+    uint32_t w[4] = {0, 0, 0, 0};
+#pragma unroll
+    for (int i = 0; i < 16; ++i)
+      w[i >> 2] |= static_cast<uint32_t>(src[static_cast<size_t>(i) * j.S]) << (8 * (i & 3));
+    *reinterpret_cast<u4*>(j.out + static_cast<size_t>(row) * j.R + 16 * k) =
+        u4{w[0], w[1], w[2], w[3]};
+  }
+}
+
 // Batched transpose [B][R][S] -> [B][S][RP] through a padded LDS tile; reads are
 // contiguous along S, writes contiguous along R.  RP >= R: positions R..RP-1 of every
 // output row are written as zeros (channel padding).
@@ -722,9 +751,15 @@ __global__ __launch_bounds__(256) void transpose_kernel(const T* __restrict__ in
 // (a wave writes 1 KiB contiguous when the group covers all RP positions of its rows).
 __global__ __launch_bounds__(256) void transpose_i8_kernel(const uint8_t* __restrict__ in,
                                                            uint8_t* __restrict__ out, int R,
-                                                           int S, int RP) {
+                                                           int S, int RP, int B, SmallJob job) {
   constexpr int kPitch = 17;  // dwords per transposed row: 64 bytes + 4 of padding
   __shared__ uint32_t tile[128 * kPitch];
+  if (static_cast<int>(blockIdx.z) >= B) {   // the extra z slices carry the riding job
+    const unsigned per_z = gridDim.x * gridDim.y;
+    small_transpose_job(job, (blockIdx.z - B) * per_z + blockIdx.y * gridDim.x + blockIdx.x,
+                        (gridDim.z - B) * per_z);
+    return;
+  }
   const size_t b = blockIdx.z;
   const int r0 = blockIdx.y * 64, s0 = blockIdx.x * 128;
   const int t = threadIdx.x;
@@ -774,16 +809,21 @@ __global__ __launch_bounds__(256) void transpose_i8_kernel(const uint8_t* __rest
 // instructions instead of sixteen, and the output runs are whole 128-byte lines.
 struct WideOrder {
   unsigned tiles_s, tiles_r, total, per_xcd;
+  unsigned grid;   // work-groups of the tile grid
 };
 
 template <int PIECE>
 __global__ __launch_bounds__(256) void transpose_i8_wide_kernel(const uint8_t* __restrict__ in,
                                                                 uint8_t* __restrict__ out,
                                                                 int R, int S, int RP,
-                                                                WideOrder o) {
+                                                                WideOrder o, SmallJob job) {
   typedef uint32_t u4 __attribute__((ext_vector_type(4)));
   constexpr int kPitch = 33;  // dwords per transposed row: 128 bytes + 4 of padding
   __shared__ uint32_t tile[128 * kPitch];
+  if (blockIdx.x >= o.grid) {   // blocks past the tile grid carry the riding job
+    small_transpose_job(job, blockIdx.x - o.grid, gridDim.x - o.grid);
+    return;
+  }
   // the tile sequence runs along S first, then R, then the batch; with o.per_xcd != 0 the
   // round-robin of work-group ids over the 8 XCDs is undone, so that every XCD owns a
   // contiguous range of it and tiles that share input cache lines meet in one L2
@@ -852,6 +892,17 @@ __global__ __launch_bounds__(256) void copy16_kernel(const uint8_t* __restrict__
     reinterpret_cast<u4*>(out)[q] = reinterpret_cast<const u4*>(in)[q];
 }
 
+// Small tensors with a thin inner extent on their own (7 x 7 planes of up to 4 MiB, or a
+// weight tensor whose data took a kernel that carries no rider): the job body as a kernel,
+// up to two jobs per launch.
+__global__ __launch_bounds__(256) void small_transpose_kernel(SmallJob first, SmallJob second,
+                                                              unsigned first_blocks) {
+  if (blockIdx.x < first_blocks)
+    small_transpose_job(first, blockIdx.x, first_blocks);
+  else
+    small_transpose_job(second, blockIdx.x - first_blocks, gridDim.x - first_blocks);
+}
+
 // A thin extent (at most 64 bytes, e.g. 7 x 7 planes) beside a long one that is a multiple of
 // 128: see thin_transpose_tile.  One matrix per blockIdx.y.
 template <bool THIN_IN>
@@ -897,32 +948,50 @@ __global__ __launch_bounds__(256) void s2d_nhwc_kernel(const int8_t* __restrict_
 // work-group ids over the XCDs is undone (64 x 256 x 56 x 56: 22.6 -> 21.1 us, 64 x 512 x 28 x 28:
 // 14.3 -> 12.1 us).  Rows on the marks lose 10 % that way (64 x 64 planes: 25.6 -> 28.9 us) and
 // the way back to planes gains nothing reliably, so those keep the plain order.
+// work-groups a riding job gets: enough to be done when the carrier is
+inline unsigned job_blocks(const SmallJob& job) {
+  if (job.pieces == 0) return 0;
+  const unsigned want = (job.pieces + 255u) / 256u;
+  return want < 1024u ? want : 1024u;
+}
+
 template <int PIECE>
-void launch_wide(hipStream_t s, const void* in, void* out, int B, int R, int S, int RP) {
+void launch_wide(hipStream_t s, const void* in, void* out, int B, int R, int S, int RP,
+                 const SmallJob& job) {
   WideOrder o;
   o.tiles_s = static_cast<unsigned>((S + 127) / 128);
   o.tiles_r = static_cast<unsigned>((RP + 127) / 128);
   const unsigned long long total = 1ull * o.tiles_s * o.tiles_r * static_cast<unsigned>(B);
-  MXQ_CHECK(total < (1ull << 31) - 8, "transpose grid too large");
+  MXQ_CHECK(total < (1ull << 31) - 256, "transpose grid too large");
   o.total = static_cast<unsigned>(total);
   o.per_xcd = (S % 128 != 0) ? (o.total + 7u) / 8u : 0u;
-  const unsigned grid = o.per_xcd != 0 ? o.per_xcd * 8u : o.total;
-  hipLaunchKernelGGL(transpose_i8_wide_kernel<PIECE>, dim3(grid), dim3(256), 0, s,
-                     static_cast<const uint8_t*>(in), static_cast<uint8_t*>(out), R, S, RP, o);
+  o.grid = o.per_xcd != 0 ? o.per_xcd * 8u : o.total;
+  hipLaunchKernelGGL(transpose_i8_wide_kernel<PIECE>, dim3(o.grid + job_blocks(job)), dim3(256), 0,
+                     s, static_cast<const uint8_t*>(in), static_cast<uint8_t*>(out), R, S, RP, o,
+                     job);
   MXQ_LAUNCH_CHECK();
 }
 
+// [B][R][S] -> [B][S][RP].  `rider`, when given, is a small job the launch carries along if
+// its kernel can (then rider->pieces is cleared); the caller launches what is left.
 template <typename T>
-void launch_transpose(hipStream_t s, const void* in, void* out, int B, int R, int S, int RP) {
+void launch_transpose(hipStream_t s, const void* in, void* out, int B, int R, int S, int RP,
+                      SmallJob* rider = nullptr) {
   if (B == 0 || RP == 0 || S == 0) return;
   MXQ_CHECK(RP >= R, "padded extent below the extent");
+  SmallJob none = {nullptr, nullptr, 16, 1, 0};
+  SmallJob job = rider != nullptr ? *rider : none;
+  auto carried = [&]() {
+    if (rider != nullptr) rider->pieces = 0;
+  };
   // only the kernels that put batches and row tiles on grid.y / grid.z have their limit
   auto check_yz = [&]() {
-    MXQ_CHECK(B <= 65535 && (RP + 63) / 64 <= 65535, "transpose grid too large");
+    MXQ_CHECK(B < 65535 && (RP + 63) / 64 <= 65535, "transpose grid too large");
   };
   if (sizeof(T) == 1 && S % 16 == 0 && S >= 128 && RP >= 128 && RP % 4 == 0 && RP % 16 != 0 &&
       aligned16(in) && (reinterpret_cast<uintptr_t>(out) & 3u) == 0) {
-    launch_wide<4>(s, in, out, B, R, S, RP);
+    launch_wide<4>(s, in, out, B, R, S, RP, job);
+    carried();
     return;
   }
   if (sizeof(T) == 1 && S % 4 == 0 && RP % 16 == 0 &&
@@ -930,14 +999,32 @@ void launch_transpose(hipStream_t s, const void* in, void* out, int B, int R, in
     // (with fewer than 128 columns half of the wide tile's lanes would idle: 64 x 56 x 56 x 64
     // back to planes takes 7.8 us that way against 6.0 us)
     if (S % 16 == 0 && S >= 128 && RP >= 128 && aligned16(in)) {
-      launch_wide<16>(s, in, out, B, R, S, RP);
+      launch_wide<16>(s, in, out, B, R, S, RP, job);
+      carried();
       return;
     }
     check_yz();
-    dim3 grid128((S + 127) / 128, (RP + 63) / 64, B);
+    const unsigned per_z = static_cast<unsigned>((S + 127) / 128) * ((RP + 63) / 64);
+    const unsigned extra_z = (job_blocks(job) + per_z - 1) / per_z;
+    MXQ_CHECK(B + extra_z <= 65535u, "transpose grid too large");
+    dim3 grid128((S + 127) / 128, (RP + 63) / 64, B + extra_z);
     hipLaunchKernelGGL(transpose_i8_kernel, grid128, dim3(256), 0, s,
-                       static_cast<const uint8_t*>(in), static_cast<uint8_t*>(out), R, S, RP);
+                       static_cast<const uint8_t*>(in), static_cast<uint8_t*>(out), R, S, RP, B,
+                       job);
     MXQ_LAUNCH_CHECK();
+    carried();
+    return;
+  }
+  if (sizeof(T) == 1 && RP == R && R % 16 == 0 && S > 1 && S <= 64 && aligned16(out) &&
+      static_cast<long long>(B) * R * S <= (4LL << 20)) {
+    // a small tensor with a thin inner extent (3 x 3 weights, 7 x 7 planes)
+    SmallJob me = {static_cast<const uint8_t*>(in), static_cast<uint8_t*>(out), R, S,
+                   static_cast<unsigned>(static_cast<long long>(B) * S * (R / 16))};
+    const unsigned mine = (me.pieces + 255u) / 256u;
+    hipLaunchKernelGGL(small_transpose_kernel, dim3(mine + job_blocks(job)), dim3(256), 0, s, me,
+                       job, mine);
+    MXQ_LAUNCH_CHECK();
+    carried();
     return;
   }
   if (sizeof(T) == 1 && RP == R && aligned16(in) && aligned16(out)) {
@@ -1195,6 +1282,26 @@ void conv_nhwc(void* stream, const int8_t* data, const int8_t* weight, const int
 }
 
 }  // namespace
+
+// Data [N][C][H][W] -> [N][H][W][Cp] and weights [O][C][KH][KW] -> [O][KH][KW][Cp] for the
+// NCHW operator's adapter route, in one launch where the data's kernel can carry the weights.
+void nchw_to_nhwc_pair(hipStream_t s, const int8_t* data, int8_t* d_out, int N, int C, int H,
+                       int W, int Cp, const int8_t* weight, int8_t* w_out, int O, int KH, int KW) {
+  MXQ_CHECK(static_cast<long long>(H) * W < (1LL << 31), "image too large");
+  const int taps = KH * KW;
+  const long long wpieces = static_cast<long long>(O) * taps * (C / 16);
+  SmallJob job = {reinterpret_cast<const uint8_t*>(weight), reinterpret_cast<uint8_t*>(w_out), C,
+                  taps, 0};
+  const bool rides = w_out != nullptr && Cp == C && C % 16 == 0 && taps > 1 && taps <= 64 &&
+                     aligned16(w_out) && wpieces < (1LL << 31);
+  if (rides) job.pieces = static_cast<unsigned>(wpieces);
+  if (static_cast<long long>(N) * Cp * H * W != 0)
+    launch_transpose<int8_t>(s, data, d_out, N, C, H * W, Cp, &job);
+  if (w_out == nullptr) return;
+  if (rides && job.pieces == 0) return;   // carried
+  launch_transpose<int8_t>(s, weight, w_out, O, C, taps, Cp);
+}
+
 }  // namespace mxq
 
 using namespace mxq;

@@ -39,6 +39,11 @@
 #include "mxq_tiles.h"
 
 namespace mxq {
+
+// mxq_conv.hip: both operand transposes of the adapter route (w_out == nullptr: data only)
+void nchw_to_nhwc_pair(hipStream_t s, const int8_t* data, int8_t* d_out, int N, int C, int H,
+                       int W, int Cp, const int8_t* weight, int8_t* w_out, int O, int KH, int KW);
+
 namespace {
 
 // The activation operand as rows of one channel each.  GM == 0 (native): image n, channel
@@ -560,12 +565,11 @@ void launch_planes(hipStream_t s, PlaneArgs a, int gm) {
     hipLaunchKernelGGL((conv1x1_planes_kernel<Cfg, 2, kGatherBytes>), grid, block, 0, s, a);
   } else if (gm == kGatherPair2) {
     hipLaunchKernelGGL((conv1x1_planes_kernel<Cfg, 2, kGatherPair2>), grid, block, 0, s, a);
-  } else if (a.C <= 2 * Cfg::BK) {
-    // a reduction of up to two stages needs no deeper ring; a longer one is read from HBM
-    // once and wants several stages in flight per work-group
-    hipLaunchKernelGGL((conv1x1_planes_kernel<Cfg, 2, kNative>), grid, block, 0, s, a);
   } else {
-    hipLaunchKernelGGL((conv1x1_planes_kernel<Cfg, 4, kNative>), grid, block, 0, s, a);
+    // two ring stages whatever the reduction length: four (48 to 128 KiB of LDS) leave room
+    // for fewer work-groups per CU and measured level or behind on every ResNet-50 layer
+    // (512 -> 1024 / 2 at 28 x 28: 30.5 us with two stages, 34.9 with four)
+    hipLaunchKernelGGL((conv1x1_planes_kernel<Cfg, 2, kNative>), grid, block, 0, s, a);
   }
   MXQ_LAUNCH_CHECK();
 }
@@ -616,7 +620,7 @@ NchwPlan plan_nchw(int N, int C, int H, int W, int O, int KH, int KW, int sh, in
       return pl;
     }
     // The gathering loader works one stage ahead out of registers; the pre-pass costs a launch
-    // and a copy of what the layer reads but feeds the kernel's four-stage ring.  Measured
+    // and a copy of what the layer reads but feeds the kernel's direct-to-LDS ring.  Measured
     // on the ResNet-50 layers at batch 64: the loader wins while the weight matrix is small
     // (256 -> 128 / 2: 34 -> 28 us, 1024 -> 256 at 14 x 14: 24 -> 20 us), the ring once the
     // layer is a real GEMM (512 -> 1024 / 2 at 28 x 28: 38 us against 53 us).
@@ -806,12 +810,9 @@ void conv_nchw(void* stream, const int8_t* data, const int8_t* weight, const int
         omin, omax, split_ws, split_room));
     return;
   }
-  MXQ_FORWARD(mxq_nchw_to_nhwc_pad_i8(stream, data, d_nhwc, N, C, H, W, pl.vC));
-  const int8_t* wk = weight;
-  if (!pl.weight_in_place) {
-    MXQ_FORWARD(mxq_nchw_to_nhwc_pad_i8(stream, weight, w_ohwi, O, C, KH, KW, pl.vC));
-    wk = w_ohwi;
-  }
+  const int8_t* wk = pl.weight_in_place ? weight : w_ohwi;
+  nchw_to_nhwc_pair(s, data, d_nhwc, N, C, H, W, pl.vC, weight,
+                    pl.weight_in_place ? nullptr : w_ohwi, O, KH, KW);
   MXQ_FORWARD(mxq_quantized_conv_nhwc_out_nchw(
       stream, d_nhwc, wk, bias, N, H, W, pl.vC, O, KH, KW, sh, sw, ph, pw, dh, dw, min_data,
       max_data, min_weight, max_weight, min_bias, max_bias, out32, omin, omax, split_ws,
