@@ -188,12 +188,41 @@ __device__ __forceinline__ uint32_t pack_bytes(int a, int b, int c, int d) {
 // Four requantized outputs as one dword (first in byte 0).  (Converting the relu'd values as
 // unsigned and or-ing them without byte masks saves a quarter instruction per output and
 // measures the same: 19-layer stack 261.7 against 260.3 us.)
+// With the relu the four values are in [0, 127] and v_cvt_pk_u8_f32 can take the place of
+// the clamp's lower side, the truncating convert and the pack: it saturates at 0, writes
+// byte k of its destination, and rounds as the wave's float rounding mode says.  The mode
+// is switched to round-toward-zero for exactly the four converts (one asm statement, so
+// that no multiply or add of the requantization can be scheduled into the stretch) and
+// back: u = f * s + 0.5 itself is computed in round-to-nearest as before, only its
+// truncation changes hands.  6.25 VALU instructions per output instead of 7.
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"
+__device__ __forceinline__ uint32_t epi_requant_relu_pack(int a0, int a1, int a2, int a3,
+                                                          const EpiScalars& s) {
+  auto level = [&](int a) {
+    const float f = static_cast<float>(a) * s.in_scale;
+    const float u = f * s.qscale + 0.5f;
+    return (u < 127.0f) ? u : 127.0f;   // the reference's min(|f| * s + 0.5, 127)
+  };
+  const float u0 = level(a0), u1 = level(a1), u2 = level(a2), u3 = level(a3);
+  uint32_t w;
+  asm volatile(
+      "s_setreg_imm32_b32 hwreg(HW_REG_MODE, 0, 2), 3\n\t"
+      "v_cvt_pk_u8_f32 %0, %1, 0, 0\n\t"
+      "v_cvt_pk_u8_f32 %0, %2, 1, %0\n\t"
+      "v_cvt_pk_u8_f32 %0, %3, 2, %0\n\t"
+      "v_cvt_pk_u8_f32 %0, %4, 3, %0\n\t"
+      "s_setreg_imm32_b32 hwreg(HW_REG_MODE, 0, 2), 0"
+      : "=&v"(w)
+      : "v"(u0), "v"(u1), "v"(u2), "v"(u3));
+  return w;
+}
+#pragma clang diagnostic pop
+
 template <bool RELU>
 __device__ __forceinline__ uint32_t epi_requant_pack(int a0, int a1, int a2, int a3,
                                                      const EpiScalars& s) {
-  if (RELU)
-    return pack_bytes(epi_requant_relu(a0, s), epi_requant_relu(a1, s), epi_requant_relu(a2, s),
-                      epi_requant_relu(a3, s));
+  if (RELU) return epi_requant_relu_pack(a0, a1, a2, a3, s);
   return pack_bytes(epi_requant(a0, s, -127.0f), epi_requant(a1, s, -127.0f),
                     epi_requant(a2, s, -127.0f), epi_requant(a3, s, -127.0f));
 }
