@@ -9,13 +9,17 @@ default workload) are long enough for the clocks to settle: over the first ~100 
 idle period the same kernels run 5-15 % slower.  The default workload is the quantized fully-connected
 layer at M=K=N=4096 with the bias and the calibrated requantize-to-int8 fused in
 the epilogue; --workload selects the other headline kernels (the 64M-element
-quantize / requantize / dequantize casts, the 8192^3 FC).  One JSON line is
-printed.  `roofline` describes the workload's kernel (algorithmic bytes or ops
-per launch over the HIP-event-timed average launch); `other_kernels` lists the same
-figures for the other kernels and for the ResNet-50 conv stack and the BERT FC chain
-(many small launches: captured into a HIP graph), measured in the same run;
+quantize / requantize / dequantize casts, the 8192^3 FC, the ResNet-50 conv stacks).  One
+JSON line is printed.  `roofline` describes the workload's kernel (algorithmic bytes or ops
+per launch over the HIP-event-timed average launch; `traffic` is read from the rocprofv3
+summary under profiles/ that `traffic_source` names); `other_kernels` lists the same
+figures for the other kernels of the path and for the ResNet-50 conv stack and the BERT FC
+chain (many small launches: captured into a HIP graph), measured in the same run;
 `cpu_baseline` is the CPU oracle (the restatement of the reference's native CPU
-operator) timed on a bounded sample on this host.
+operator) timed on a bounded sample on this host.  The last key, `targets`, repeats the
+rows a reader looks for first (the casts, FC 8192^3, the two conv stacks) as
+[us per step, achieved, fraction of peak], so that a truncated tail of the line still
+holds them.
 """
 import argparse
 import ctypes
@@ -32,35 +36,61 @@ METRIC = "int8 FC TOPS (% MFMA peak) + quant/requant GB/s (% HBM peak), 1 GPU"
 HBM_PEAK_GBS = 8000.0    # MI355X HBM3E
 INT8_PEAK_TOPS = 5000.0  # MI355X dense int8 MFMA
 
-# HBM bytes per step of the workload's kernels from `rocprofv3 --pmc FETCH_SIZE` and
-# `--pmc WRITE_SIZE` runs (KiB per dispatch; FETCH_SIZE x 2.00 per the copy-kernel
-# calibration, profiles/copy_calibration_64M.md), with the summary under profiles/ each
-# figure was read from: `roofline.traffic` is that profile's figure, not a counter read in
-# this run (`roofline.traffic_source` names the file); a workload without an entry reports
-# null.
-_KIB = 1024.0
-MEASURED_TRAFFIC_BYTES = {
-    "fc4096": ((2.0 * 49277.4 + 16384.1) * _KIB, "profiles/fc_dma_kernel_4096.md"),
-    "quantize": ((2.0 * 131102.5 + 65536.1) * _KIB, "profiles/quantize_kernel_64M.md"),
-    "quantize_uncal": ((2.0 * (131093.7 + 131139.1) + 65536.1) * _KIB, "profiles/quantize_uncalibrated_64M.md"),
-    "requantize": ((2.0 * 131104.8 + 65536.1) * _KIB, "profiles/requantize_kernel_64M.md"),
-    "requantize_uncal": ((2.0 * (131089.2 + 131139.2) + 65536.1) * _KIB, "profiles/requantize_uncalibrated_64M.md"),
-    "dequantize": ((2.0 * 32782.0 + 262144.0) * _KIB, "profiles/dequantize_chunk_kernel_64M.md"),
-    "elemwise_add": ((2.0 * 65557.2 + 262144.1) * _KIB, "profiles/add32_chunk_kernel_64M.md"),
-    "elemwise_add_int8": ((2.0 * 65583.7 + 65536.1) * _KIB, "profiles/add_kernel_int8_64M.md"),
-    "concat": ((2.0 * 32890.0 + 65536.1) * _KIB, "profiles/concat_kernel_64M.md"),
-    "elemwise_mul_int8": ((2.0 * 65565.8 + 65536.1) * _KIB, "profiles/mul_kernel_int8_64M.md"),
-    "quantize_asym": ((2.0 * 131099.2 + 65536.1) * _KIB, "profiles/quantize_asym_kernel_64M.md"),
-    "batch_norm": ((2.0 * 32838.0 + 65536.1) * _KIB, "profiles/bn_rows_kernel_nchw_64M.md"),
-    "embedding": ((2.0 * 31709.6 + 65535.8) * _KIB, "profiles/embedding_kernel_bert_vocab.md"),
-    "transpose": ((2.0 * 32800.1 + 65548.3) * _KIB, "profiles/permute_elem_direct_kernel_attention_64M.md"),
-    "quantized_act": ((2.0 * 32791.8 + 65575.3) * _KIB, "profiles/relu_chunk_kernel_64M.md"),
-    "transpose_to_nhwc": ((2.0 * 32797.6 + 65541.4) * _KIB, "profiles/permute_tile16_kernel_to_nhwc_64M.md"),
-    "transpose_to_nchw": ((2.0 * 32797.6 + 65538.6) * _KIB, "profiles/permute_tile16_kernel_to_nchw_64M.md"),
-    "maxpool": ((2.0 * 100388.0 + 50177.2) * _KIB, "profiles/pool_lds_kernel_maxpool.md"),
-    "avgpool": ((2.0 * 200728.0 + 8192.1) * _KIB, "profiles/pool_lds_kernel_global_avgpool.md"),
-    "resnet50_convs": (521.8e6, "profiles/conv_stack_resnet50.md"),
+# `roofline.traffic`: HBM bytes per step of the workload's kernels, read at run time from the
+# rocprofv3 summary under profiles/ that holds the workload's `--pmc FETCH_SIZE` / `--pmc
+# WRITE_SIZE` runs (KiB per dispatch; FETCH_SIZE x 2.00 per the copy-kernel calibration,
+# profiles/copy_calibration_64M.md), so the figure cannot drift from the file it cites
+# (`roofline.traffic_source`).  It is that profile's figure, not a counter read in this run;
+# a workload without such a file reports null.
+TRAFFIC_PROFILES = {
+    "fc4096": "profiles/fc_dma_kernel_4096.md",
+    "fc8192": "profiles/fc_dma_kernel_8192.md",
+    "quantize": "profiles/quantize_kernel_64M.md",
+    "quantize_uncal": "profiles/quantize_uncalibrated_64M.md",
+    "requantize": "profiles/requantize_kernel_64M.md",
+    "requantize_uncal": "profiles/requantize_uncalibrated_64M.md",
+    "dequantize": "profiles/dequantize_chunk_kernel_64M.md",
+    "elemwise_add": "profiles/add32_chunk_kernel_64M.md",
+    "elemwise_add_int8": "profiles/add_kernel_int8_64M.md",
+    "concat": "profiles/concat_kernel_64M.md",
+    "quantized_act": "profiles/relu_chunk_kernel_64M.md",
+    "maxpool": "profiles/pool_lds_kernel_maxpool.md",
+    "avgpool": "profiles/pool_lds_kernel_global_avgpool.md",
+    "resnet50_convs": "profiles/conv_stack_resnet50.md",
+    "resnet50_convs_operator": "profiles/conv_stack_resnet50_operator_contract.md",
+    "elemwise_mul_int8": "profiles/mul_kernel_int8_64M.md",
+    "quantize_asym": "profiles/quantize_asym_kernel_64M.md",
+    "batch_norm": "profiles/bn_rows_kernel_nchw_64M.md",
+    "embedding": "profiles/embedding_kernel_bert_vocab.md",
+    "transpose": "profiles/permute_elem_direct_kernel_attention_64M.md",
+    "transpose_to_nhwc": "profiles/permute_tile16_kernel_to_nhwc_64M.md",
+    "transpose_to_nchw": "profiles/permute_tile16_kernel_to_nchw_64M.md",
 }
+
+
+def profile_traffic(key):
+    """(bytes per step, file) from the profile summary of workload `key`, or (None, None).
+    A summary of many launches per step states `traffic_bytes_per_step: N`; one of a single
+    launch (or of a two-launch step with one row per kernel and counter) is summed from its
+    counter table."""
+    import re
+    rel = TRAFFIC_PROFILES.get(key)
+    if rel is None or not os.path.exists(os.path.join(ROOT, rel)):
+        return None, None
+    text = open(os.path.join(ROOT, rel)).read()
+    m = re.search(r"traffic_bytes_per_step:\s*([0-9.eE+]+)", text)
+    if m:
+        return float(m.group(1)), rel
+    fetch = write = 0.0
+    rows = re.findall(r"^\| `[^`]*` \| (FETCH_SIZE|WRITE_SIZE) \| \d+ \| ([0-9.]+) \|", text, re.M)
+    for counter, kib in rows:
+        if counter == "FETCH_SIZE":
+            fetch += float(kib)
+        else:
+            write += float(kib)
+    if not rows:
+        return None, None
+    return (2.0 * fetch + write) * 1024.0, rel
 
 
 # What a default run measures besides the headline workload, in this order.  The operators
@@ -728,7 +758,8 @@ class ConvStackWorkload(GraphWorkload):
         self.kernel = "conv_dma_kernel / fc_dma_kernel (1x1)"
         self.bound = "mfma"
         self.name = "ResNet-50 v1 bottleneck conv stack (19 distinct layers), batch 64, " \
-                    "NHWC int8, fused relu + requantize"
+                    "NHWC int8, fused relu + requantize, naive per-layer calibration " \
+                    "(range = min/max of the layer's own fp32 output on a batch slice)"
         P = lambda t: ctypes.c_void_p(t.data_ptr())
         g = torch.Generator(device="cuda").manual_seed(4)
         N = 64
@@ -793,7 +824,8 @@ class ConvOperatorWorkload(GraphWorkload):
         self.kernel = "conv1x1_planes_kernel (NCHW 1x1) + adapters / conv_dma_kernel (3x3, small planes), int32 NCHW out"
         self.bound = "mfma"
         self.name = "ResNet-50 v1 bottleneck conv stack (19 distinct layers), batch 64, as the " \
-                    "operator sees it: NCHW int8 in, NCHW int32 out" + \
+                    "operator sees it: NCHW int8 in, NCHW int32 out (no requantize, so no " \
+                    "calibration)" + \
                     (" (every layer through the layout adapters)" if route == 1 else "")
         P = lambda t: ctypes.c_void_p(t.data_ptr())
         g = torch.Generator(device="cuda").manual_seed(4)
@@ -862,14 +894,17 @@ class ResNetChainWorkload(GraphWorkload):
         self.kernel = "conv / fc kernels, add_kernel, relu"
         self.bound = "mfma"
         self.name = "ResNet-50 v1 bottleneck body as a chain (52 convolutions + 16 residual " \
-                    "adds + relus), batch 64, NHWC int8, requantize fused"
+                    "adds + relus), batch 64, NHWC int8, requantize fused, naive per-layer " \
+                    "calibration (range = min/max of each layer's fp32 output on the chain's " \
+                    "own data)"
         if unfused:
             # the operator sequence of the graph the reference's pass emits: every convolution
             # writes int32, a _contrib_requantize node narrows it, relu is a node of its own
             self.kernel = "conv / fc kernels (int32 out), requantize, relu, add_kernel"
             self.name = "ResNet-50 v1 bottleneck body as the reference's graph runs it: " \
                         "quantized_conv (int32) -> requantize -> quantized_act per layer, " \
-                        "elemwise_add + act per block, batch 64, NHWC"
+                        "elemwise_add + act per block, batch 64, NHWC, naive per-layer " \
+                        "calibration"
         if fused_sum:
             self.kernel = "conv / fc kernels, the residual sum and its relu in the epilogue of " \
                           "each block's last 1x1 convolution"
@@ -1259,8 +1294,8 @@ def roofline_of(wl, event_s_per_launch, key=None):
         peak, unit = HBM_PEAK_GBS, "GB/s"
     return {"bound": wl.bound, "kernel": wl.kernel, "achieved": round(achieved, 1), "peak": peak,
             "unit": unit, "frac": round(achieved / peak, 4),
-            "traffic": MEASURED_TRAFFIC_BYTES.get(key, (None, None))[0],
-            "traffic_source": MEASURED_TRAFFIC_BYTES.get(key, (None, None))[1],
+            "traffic": profile_traffic(key)[0],
+            "traffic_source": profile_traffic(key)[1],
             "avg_launch_us": round(event_s_per_launch * 1e6, 2)}
 
 

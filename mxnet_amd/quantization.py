@@ -61,36 +61,34 @@ def _calibrate_quantized_sym(qsym, min_max_dict):
     return Symbol.fromjson(out.value.decode())
 
 
-def _quantize_params(qsym, params, min_max_dict):
-    """Parameters of the quantized symbol: `<name>_quantize` (int8 through the v1
-    quantize operator with the tensor's own min / max), `<name>_quantize_min/_max`,
-    untouched parameters of nodes that stayed float, and `<x>_min` / `<x>_max` scalars for
-    entries of `min_max_dict`."""
+def _own_range_int8(tensor):
+    """int8 values and the (min, max) scalars of a float parameter quantized over its own
+    range by the v1 quantize operator."""
     from . import contrib
-    quantized = {}
-    for name in qsym.list_arguments():
-        if name.endswith(("weight_quantize", "bias_quantize")):
-            original = name[:-len("_quantize")]
-            param = params[original]
-            param = (param if isinstance(param, torch.Tensor) else torch.as_tensor(param)).cuda()
-            val, vmin, vmax = contrib.quantize(param.to(torch.float32).contiguous(),
-                                               param.min().reshape(1).to(torch.float32),
-                                               param.max().reshape(1).to(torch.float32),
-                                               out_type="int8")
-            quantized[name] = val
-            quantized[name + "_min"] = vmin
-            quantized[name + "_max"] = vmax
-        elif name in params:
-            quantized[name] = params[name]
-        elif name.endswith("_min"):
-            output = name[:-len("_min")]
-            if output in min_max_dict:
-                quantized[name] = torch.tensor([min_max_dict[output][0]], dtype=torch.float32)
-        elif name.endswith("_max"):
-            output = name[:-len("_min")]
-            if output in min_max_dict:
-                quantized[name] = torch.tensor([min_max_dict[output][1]], dtype=torch.float32)
-    return quantized
+    t = tensor if isinstance(tensor, torch.Tensor) else torch.as_tensor(tensor)
+    t = t.cuda().to(torch.float32).contiguous()
+    bounds = [f().reshape(1).to(torch.float32) for f in (t.min, t.max)]
+    return contrib.quantize(t, bounds[0], bounds[1], out_type="int8")
+
+
+def _quantize_params(qsym, params, min_max_dict):
+    """Parameters of the quantized symbol, keyed by its argument names: `<p>_quantize`
+    (int8, the parameter's own range) with `<p>_quantize_min` / `_max` for weights and
+    biases, parameters of nodes that stayed float as they are, and one-element `<x>_min` /
+    `<x>_max` tensors for the entries of `min_max_dict`
+    (python/mxnet/contrib/quantization.py:85-123)."""
+    result = {}
+    for arg in qsym.list_arguments():
+        stem, _, tail = arg.rpartition("_")
+        if tail == "quantize" and stem.endswith(("weight", "bias")):
+            q, lo, hi = _own_range_int8(params[stem])
+            result.update({arg: q, arg + "_min": lo, arg + "_max": hi})
+        elif arg in params:
+            result[arg] = params[arg]
+        elif tail in ("min", "max") and stem in min_max_dict:
+            bound = min_max_dict[stem][1 if tail == "max" else 0]
+            result[arg] = torch.tensor([bound], dtype=torch.float32)
+    return result
 
 
 class CalibrationCollector:
@@ -147,9 +145,46 @@ def calibrate_entropy(hist, hist_edges, num_quantized_bins=255):
     return np.float32(th.value), np.float32(div.value)
 
 
+class _SymmetricHistogram:
+    """Counts of a tensor's values over [-th, th] in equal bins, growable by whole bins on
+    both sides so that what was counted keeps its bins when a later batch reaches further
+    out.  `lo` / `hi` are the extreme values seen."""
+
+    def __init__(self, counts, th, lo, hi):
+        self.counts, self.th, self.lo, self.hi = counts, th, lo, hi
+
+    @classmethod
+    def of(cls, arr, bins):
+        lo, hi = np.min(arr), np.max(arr)
+        th = max(abs(lo), abs(hi))
+        return cls(np.histogram(arr, bins=bins, range=(-th, th))[0], th, lo, hi)
+
+    @classmethod
+    def from_tuple(cls, t):
+        return cls(t[0], t[4], t[2], t[3])
+
+    def as_tuple(self):
+        edges = np.linspace(-self.th, self.th, len(self.counts) + 1)
+        return (self.counts, edges, self.lo, self.hi, self.th)
+
+    def absorb(self, arr, lo, hi, reach):
+        """Count one more batch (`reach` = max |value| of it)."""
+        if reach > self.th:
+            width = 2 * self.th / len(self.counts)
+            margin = int((reach - self.th) // width + 1)
+            self.counts = np.pad(self.counts, margin)
+            self.th = margin * width + self.th
+        batch = np.histogram(arr, bins=len(self.counts), range=(-self.th, self.th))[0]
+        self.counts = self.counts + batch
+        self.lo, self.hi = min(self.lo, lo), max(self.hi, hi)
+        return self
+
+
 class _LayerHistogramCollector(CalibrationCollector):
-    """calib_mode='entropy': symmetric histograms of every calibrated tensor, merged
-    across batches, then the KL-optimal threshold per tensor."""
+    """calib_mode='entropy': a symmetric histogram per calibrated tensor, grown over the
+    batches, then the KL-optimal threshold of each
+    (python/mxnet/contrib/quantization.py:269-361).  `hist_dict[name]` is the reference's
+    tuple (hist, edges, min, max, threshold)."""
 
     def __init__(self, quantized_dtype, num_bins=8001, include_layers=None, logger=None):
         super().__init__()
@@ -163,13 +198,13 @@ class _LayerHistogramCollector(CalibrationCollector):
         if name not in self.include_layers:
             return
         arr = _to_numpy(arr)
-        lo, hi = np.min(arr), np.max(arr)
-        th = max(abs(lo), abs(hi))
-        if name in self.hist_dict:
-            self.hist_dict[name] = self.combine_histogram(self.hist_dict[name], arr, lo, hi, th)
+        seen = self.hist_dict.get(name)
+        if seen is None:
+            self.hist_dict[name] = _SymmetricHistogram.of(arr, self.num_bins).as_tuple()
         else:
-            hist, edges = np.histogram(arr, bins=self.num_bins, range=(-th, th))
-            self.hist_dict[name] = (hist, edges, lo, hi, th)
+            lo, hi = np.min(arr), np.max(arr)
+            self.hist_dict[name] = self.combine_histogram(seen, arr, lo, hi,
+                                                          max(abs(lo), abs(hi)))
 
     def post_collect(self):
         return self.get_optimal_thresholds(self.hist_dict, self.quantized_dtype,
@@ -177,20 +212,8 @@ class _LayerHistogramCollector(CalibrationCollector):
 
     @staticmethod
     def combine_histogram(old_hist, arr, new_min, new_max, new_th):
-        (old_hist, old_edges, old_min, old_max, old_th) = old_hist
-        if new_th <= old_th:
-            hist, _ = np.histogram(arr, bins=len(old_hist), range=(-old_th, old_th))
-            return (old_hist + hist, old_edges, min(old_min, new_min), max(old_max, new_max),
-                    old_th)
-        # widen by whole bins of the old width on both sides so that old bins map 1:1
-        old_bins = len(old_hist)
-        old_step = 2 * old_th / old_bins
-        extra = int((new_th - old_th) // old_step + 1)
-        new_bins = extra * 2 + old_bins
-        new_th = extra * old_step + old_th
-        hist, edges = np.histogram(arr, bins=new_bins, range=(-new_th, new_th))
-        hist[extra:new_bins - extra] += old_hist
-        return (hist, edges, min(old_min, new_min), max(old_max, new_max), new_th)
+        return _SymmetricHistogram.from_tuple(old_hist).absorb(
+            arr, new_min, new_max, new_th).as_tuple()
 
     @staticmethod
     def get_optimal_threshold(hist_data, quantized_dtype, num_quantized_bins=255):

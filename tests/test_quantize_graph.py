@@ -346,6 +346,39 @@ def test_histogram_collector_merges_batches():
     assert m.post_collect() == {"x": (-2.0, 3.0)}
 
 
+def test_merged_histogram_equals_one_histogram_of_all_batches():
+    """Bins of width 1 with values on a quarter grid: every edge is exact in binary, so
+    growing by whole bins and counting batch by batch must give exactly the counts of one
+    histogram of everything over the final range (quantization.py:295-329 of the
+    reference)."""
+    rng = np.random.default_rng(3)
+    grid = lambda reach, n: (rng.integers(-4 * reach, 4 * reach, n) + 0.5) / 4.0
+    first = np.concatenate([grid(2, 50), [2.5]]).astype(np.float32)      # th 2.5, 5 bins
+    inside = grid(2, 30).astype(np.float32)
+    beyond = np.concatenate([grid(4, 40), [-4.25]]).astype(np.float32)   # reach 4.25
+    h = Q._LayerHistogramCollector("int8", num_bins=5, include_layers=["t"])
+    for batch in (first, inside, beyond):
+        h.collect("t", "op", batch)
+    hist, edges, lo, hi, th = h.hist_dict["t"]
+    # margin = floor((4.25 - 2.5) / 1) + 1 = 2 bins a side
+    assert th == 4.5 and len(hist) == 9
+    everything = np.concatenate([first, inside, beyond])
+    want, want_edges = np.histogram(everything, bins=9, range=(-4.5, 4.5))
+    # the first batch's own maximum (2.5) sat on the closed top edge of its histogram and
+    # keeps that bin; counted in one go it would open the next one
+    want[6] += 1
+    want[7] -= 1
+    np.testing.assert_array_equal(hist, want)
+    np.testing.assert_array_equal(edges, want_edges)
+    assert lo == everything.min() and hi == everything.max()
+    # the static form the reference's callers use gives the same tuple
+    t = Q._LayerHistogramCollector.combine_histogram(
+        (np.array([1, 2, 3]), np.linspace(-1.5, 1.5, 4), -1.25, 1.25, 1.5),
+        np.array([2.75, -0.25]), -0.25, 2.75, 2.75)
+    np.testing.assert_array_equal(t[0], [0, 0, 1, 3, 3, 0, 1])
+    assert t[2:] == (-1.25, 2.75, 3.5)
+
+
 def test_residual_add_and_concat_stay_int8():
     """elemwise_add (quantized_elemwise_add.cc:124-133, FNeedRequantize) and Concat
     (quantized_concat.cc:143-152): data inputs first, then one (min, max) pair per input in
