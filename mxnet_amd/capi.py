@@ -236,10 +236,6 @@ def quantized_conv_nchw(data, weight, bias, min_data, max_data, min_weight, max_
     geo = [N, C, H, W, O, KH, KW, stride[0], stride[1], pad[0], pad[1], dilate[0], dilate[1]]
     both_aligned = data.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0 and cfg != 1
     wsb = lib.mxq_quantized_conv_nchw_workspace(*geo, int(both_aligned))
-    if cfg is not None and KH == 1 and KW == 1:
-        # a pinned route may be one the query does not plan for: room for the largest
-        wsb = max(wsb, (C * ((N * ((OH * OW + 3) // 4 * 4) + 15) // 16 * 16) + 255) // 256 * 256,
-                  lib.mxq_quantized_conv_nchw_workspace(*geo, 0))
     ws = _workspace(wsb, dev) if wsb else None
     args = [_stream(), _ptr(data), _ptr(weight), _ptr(bias)] + geo + [
         _ptr(min_data), _ptr(max_data), _ptr(min_weight), _ptr(max_weight), _ptr(min_bias),

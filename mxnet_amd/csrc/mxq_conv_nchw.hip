@@ -31,7 +31,6 @@
 #include <hip/hip_runtime.h>
 
 #include <cmath>
-#include <cstdio>
 #include <cstdint>
 
 #include "../../include/mxq.h"
@@ -86,7 +85,7 @@ struct PlaneCfg {
   static_assert(BP % (32 * WP) == 0 && BO % (32 * WO) == 0, "wave tile");
   static_assert(A_SLOTS % (64 * NW) == 0 && B_SLOTS % (64 * NW) == 0, "loader");
   static_assert(CHP == 4 || CHP == 8 || CHP == 16, "pixel-chunk swizzle");
-  static_assert(CH == 4 || CH == 8 || CH == 16, "fragment addressing of the weight operand");
+  static_assert(CH == 4 || CH == 8, "fragment addressing of the weight operand");
   static_assert(kThreads % GROUPS == 0 && BK % TPG == 0 && TPG % 8 == 0,
                 "gathering loader: a thread's channels share their low three bits");
 };
@@ -118,16 +117,18 @@ constexpr int kGatherBytes = 3; // anything else: byte by byte
 constexpr int kGatherPair2 = 4; // sw == 2, 2 | OW, rows on dword marks: two dwords (two pixels
                                 // each, a pair never leaves its row) and a v_perm
 
-// Lab builds (-DMXQ_STAMPS) record the cycle counter of every work-group's first lane at four
-// points of the kernel; the product build compiles none of it.
+// Lab builds (-DMXQ_STAMPS) record, for every work-group's first lane, the shader clock and
+// the 100 MHz real-time counter at four points of the kernel (entry, first stage issued,
+// K loop done, last store issued); mxq_dbg_read_plane_stamps copies them out.  The product
+// build compiles none of it.
 #ifdef MXQ_STAMPS
 __device__ long long mxq_dbg_plane_stamps[8 * 16384];
-#define PLANE_STAMP(k)                                                                 \
-  do {                                                                                 \
-    if (threadIdx.x == 0 && blockIdx.x < 16384) {                                      \
-      mxq_dbg_plane_stamps[blockIdx.x * 8 + (k)] = __builtin_readcyclecounter();       \
+#define PLANE_STAMP(k)                                                                   \
+  do {                                                                                   \
+    if (threadIdx.x == 0 && blockIdx.x < 16384) {                                        \
+      mxq_dbg_plane_stamps[blockIdx.x * 8 + (k)] = __builtin_readcyclecounter();         \
       mxq_dbg_plane_stamps[blockIdx.x * 8 + 4 + (k)] = __builtin_amdgcn_s_memrealtime(); \
-    }                                                                                  \
+    }                                                                                    \
   } while (0)
 #else
 #define PLANE_STAMP(k)
@@ -442,349 +443,6 @@ __global__ __launch_bounds__(Cfg::kThreads, 2) void conv1x1_planes_kernel(PlaneA
   PLANE_STAMP(3);
 }
 
-// ---- activation-stationary form ----------------------------------------------------------
-// The same GEMM with the roles of the operands in time exchanged: a work-group fetches ALL
-// C channels of its BP pixels once (the slab [C][BP] stays in LDS for the life of the
-// group) and then walks output-channel tiles of 128, streaming only the weights, which
-// every group shares and the L2 holds.  What this buys over the kernel above, where every
-// (pixel tile, channel tile) pair is a work-group of its own that walks K in steps:
-//   * the activation is read from memory once, not once per channel tile, and with every
-//     load of the slab in flight together instead of one K step at a time (the K loop
-//     above spent 0.4 to 0.9 us per step waiting: 14 x 14 planes, 1024 -> 256, 16 steps);
-//   * a strided or odd-sized plane is gathered once per pixel tile, so the loader can
-//     afford the general form (below) and needs neither its pre-pass nor a workspace;
-//   * the stores of one channel tile drain while the next tile is multiplied.
-// Five waves: four multiply (wave w owns channels 32 w ... of the current channel tile
-// and all BP pixels, so a store instruction writes runs of 4 BP bytes) and never wait on
-// memory after the slab has landed; the fifth only issues the weights' direct-to-LDS
-// loads into a ring of NS stages and waits for them.  The split keeps the two kinds of
-// memory traffic on different wave counters: vmcnt retires loads in order among
-// themselves, but not against the stores of the epilogue, so a wave that did both could
-// not tell "my stage has landed" from "some of my stores have".
-//
-// The loader of a gathered slab: a thread owns four consecutive pixels (one LDS dword per
-// channel) of the matrix [C][N * P].  Consecutive output pixels are consecutive input
-// bytes (pixel stride 1) or every other byte (stride 2) within a row of RL pixels (an
-// output row; the whole plane when the layer reads whole planes), so the four pixels are
-// a first run of ka <= 4 pixels at the end of one row and, if ka < 4, the start of the
-// next row (of the same image or of the next one).  One unaligned 4- or 8-byte load per
-// run and a v_perm pick the bytes; rows of 4 | RL pixels never need the second run (TWO).
-#ifndef MXQ_STAT_NS
-#define MXQ_STAT_NS 3
-#endif
-constexpr int kStatBO = 128, kStatBK = 64, kStatNS = MXQ_STAT_NS;
-constexpr int kStatStage = kStatBO * kStatBK;       // bytes of a weight stage
-constexpr int kStatThreads = 320;
-
-// Work-group barrier of the stationary kernel: the wave's LDS traffic is done before it
-// arrives, and the compiler moves no memory access across it.
-__device__ __forceinline__ void stat_barrier() {
-  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-}
-
-enum StatMode { kStatDma = 0, kStatS1 = 1, kStatS1Two = 2, kStatS2 = 3, kStatS2Two = 4 };
-
-struct StatArgs {
-  const int8_t* data;
-  const int8_t* weight;  // [O][C]
-  int N, C, P, O;        // P = output pixels per image
-  int V;                 // N * P: columns of the activation matrix
-  int plane_in;          // input pixels per channel plane
-  int RL, rows;          // pixels per row and rows per image (RL * rows == P)
-  int row_pitch;         // input bytes from one row to the next
-  uint32_t data_bytes;
-  int tiles_p, o_groups, ot_per_group, tiles_o;
-  Epilogue epi;
-};
-
-// The work-group's LDS (slab, weight ring, staging rows of the four multiplying waves) is
-// dynamic, sized by the launcher from the layer's channel count: with a static array the
-// compiler knows that at most two groups fit a CU and pads the kernel's register count to
-// 129 "to match", after which the second group's waves no longer fit beside the first's
-// on the SIMD that holds two of each (measured: one group per CU until a wave exits).
-extern __shared__ __attribute__((aligned(16))) char stat_lds[];
-
-template <int BP, int MODE>
-__global__ __launch_bounds__(kStatThreads, 4) void conv1x1_stationary_kernel(StatArgs p) {
-  constexpr int BO = kStatBO, BK = kStatBK, NS = kStatNS, CH = BK / 16, CHP = BP / 16;
-  constexpr int MI = BP / 32, KS = BK / 32;
-  constexpr int LP = BP + 8;                 // staging row pitch in dwords
-  constexpr int CHB = BP == 128 ? 8 : 16;    // channels staged at a time
-  constexpr int LPR = BP / 4, RPI = 64 / LPR;
-  constexpr int RING = NS * kStatStage;
-  char* lds = stat_lds;
-  __shared__ __attribute__((aligned(16))) int sbias[2][BO];
-  const int tid = threadIdx.x, lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-
-  // group order: the channel groups of one pixel tile are neighbours in one XCD
-  const int total = p.tiles_p * p.o_groups;
-  const int lid = xcd_remap(blockIdx.x, total);
-  const int og = lid % p.o_groups, tp = lid / p.o_groups;
-  const int p0 = tp * BP;
-  const int ot0 = og * p.ot_per_group;
-  const int n_ot = (p.tiles_o - ot0 < p.ot_per_group) ? p.tiles_o - ot0 : p.ot_per_group;
-  const int KT = (p.C + BK - 1) / BK;
-  const int A_BYTES = KT * BK * BP;          // the slab; behind it the ring, then the staging rows
-  const int S = n_ot * KT;                   // weight stages of this group
-  const uint32_t lds0 = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(lds));
-  PLANE_STAMP(0);
-
-  if (wave == 4) {
-    // ---- the loading wave: weight stage s = (channel tile s / KT, K block s % KT)
-    const v4i wrsrc = make_rsrc(p.weight, static_cast<uint32_t>(p.O) * static_cast<uint32_t>(p.C));
-    constexpr int BI = kStatStage / 1024;    // wave instructions per stage
-    int wrow[BI];
-    uint32_t wk16[BI];
-#pragma unroll
-    for (int j = 0; j < BI; ++j) {
-      const int q = j * 64 + lane, r = q / CH;
-      wrow[j] = r;
-      wk16[j] = static_cast<uint32_t>(((q % CH) ^ swz<CH>(r)) * 16);
-    }
-    auto issue = [&](int s) {
-      if (s >= S) return;
-      const int t = s / KT, kt = s - t * KT;
-      const uint32_t sb = lds0 + A_BYTES + static_cast<uint32_t>(s % NS) * kStatStage;
-#pragma unroll
-      for (int j = 0; j < BI; ++j) {
-        const int o = (ot0 + t) * BO + wrow[j];
-        const uint32_t k0 = static_cast<uint32_t>(kt * BK) + wk16[j];
-        const uint32_t off = (o < p.O && k0 < static_cast<uint32_t>(p.C))
-                                 ? static_cast<uint32_t>(o) * static_cast<uint32_t>(p.C) + k0
-                                 : kOutOfRange;
-        dma_buffer(sb + j * 1024, off, wrsrc);
-      }
-    };
-#pragma unroll
-    for (int s = 0; s < NS - 1; ++s) issue(s);
-    stat_barrier();                          // the slab (the multiplying waves' work)
-    for (int s = 0; s < S; ++s) {
-      const int newest = (s + NS - 2) < (S - 1) ? (s + NS - 2) : (S - 1);
-      wait_ahead<BI, NS - 2>(newest - s);
-      stat_barrier();                        // stage s is there; stage s - 1 has been read
-      issue(s + NS - 1);
-    }
-    if (blockIdx.x == 0 && lane == 0) epilogue_ranges(p.epi);
-    return;
-  }
-
-  // ---- the multiplying waves: first the slab
-  const int ctid = tid;                      // 0 .. 255
-  if constexpr (MODE == kStatDma) {
-    // whole 16-byte chunks of channel rows; a chunk never leaves its image (16 | P)
-    const v4i arsrc = make_rsrc(p.data, p.data_bytes);
-    constexpr int RPW = 64 / CHP;            // channel rows per wave instruction
-    const int c_in = lane / CHP;
-    const int pc = (lane % CHP) ^ plane_swz<CHP>(c_in);
-    const int v = p0 + pc * 16;
-    uint32_t base = kOutOfRange;
-    if (v < p.V) {
-      const int img = v / p.P;
-      base = static_cast<uint32_t>(img) * static_cast<uint32_t>(p.C) * p.P + (v - img * p.P);
-    }
-    const int instrs = KT * BK / (4 * RPW);
-    for (int j = 0; j < instrs; ++j) {
-      const int c = (j * 4 + wave) * RPW + c_in;
-      const uint32_t off = (c < p.C && base != kOutOfRange)
-                               ? base + static_cast<uint32_t>(c) * p.P
-                               : kOutOfRange;
-      dma_buffer(lds0 + (j * 4 + wave) * 1024, off, arsrc);
-    }
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-  } else {
-    constexpr bool TWO = MODE == kStatS1Two || MODE == kStatS2Two;
-    constexpr bool S2 = MODE == kStatS2 || MODE == kStatS2Two;
-    constexpr int GROUPS = BP / 4, TPG = 256 / GROUPS;   // threads per pixel group
-    static_assert(TPG % 8 == 0, "a thread's channels share their low three bits");
-    const int grp = ctid % GROUPS, cs = ctid / GROUPS;
-    const int v = p0 + 4 * grp;
-    const int vv = v < p.V ? v : 0;          // columns past the end read pixel 0, never stored
-    const int img = vv / p.P, px = vv - img * p.P;
-    const int r = px / p.RL, col = px - r * p.RL;
-    const int ka = (p.RL - col) < 4 ? (p.RL - col) : 4;
-    const uint32_t img_bytes = static_cast<uint32_t>(p.C) * p.plane_in;
-    const uint32_t offA = img * img_bytes + r * p.row_pitch + col * (S2 ? 2 : 1);
-    uint32_t offB = offA, sel = 0x03020100u, maskA = 0x01010101u;
-    if (TWO) {
-      int r2 = r + 1, img2 = img;
-      if (r2 == p.rows) {
-        r2 = 0;
-        ++img2;
-      }
-      if (img2 < p.N) offB = img2 * img_bytes + r2 * p.row_pitch;
-      // byte j of the dword: j < ka from the first run, else byte j - ka of the second
-      sel = 0;
-      maskA = 0;
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        sel |= static_cast<uint32_t>(j < ka ? j : 4 + j - ka) << (8 * j);
-        maskA |= static_cast<uint32_t>(j < ka ? 1 : 0) << (8 * j);
-      }
-    }
-    const uint32_t maskB = 0x01010101u - maskA;
-    // A window that would run past the end of the tensor (the last rows of the last plane)
-    // is moved back to end with it, and the byte selectors move by as much: the bytes a run
-    // needs always lie inside the tensor, the window's other bytes need not.
-    const uint32_t last8 = p.data_bytes - 8, last4 = p.data_bytes - 4;
-    const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(
-        const_cast<int8_t*>(p.data), 0, static_cast<int>(p.data_bytes), 0x00020000);
-    char* slot = lds + cs * BP + ((((grp >> 2) ^ plane_swz<CHP>(cs))) << 4) + ((grp & 3) << 2);
-    typedef uint32_t u2 __attribute__((ext_vector_type(2)));
-    auto window8 = [&](uint32_t at) {   // the four even bytes from `at` on
-      const uint32_t from = at < last8 ? at : last8;
-      const u2 w = __builtin_amdgcn_raw_buffer_load_b64(rs, from, 0, 0);
-      return __builtin_amdgcn_perm(w.y, w.x, 0x06040200u + (at - from) * 0x01010101u);
-    };
-    constexpr int BATCH = (S2 && TWO) ? 8 : 16;   // loads in flight per thread (two 8-byte windows each there)
-    for (int c0 = cs; c0 < p.C; c0 += TPG * BATCH) {
-      uint32_t wd[BATCH];
-#pragma unroll
-      for (int i = 0; i < BATCH; ++i) {
-        int c = c0 + TPG * i;
-        c = c < p.C ? c : p.C - 1;
-        const uint32_t row = static_cast<uint32_t>(c) * p.plane_in;
-        if (S2) {
-          uint32_t w = window8(row + offA);
-          if (TWO) w = __builtin_amdgcn_perm(window8(row + offB), w, sel);
-          wd[i] = w;
-        } else if (TWO) {
-          const uint32_t atA = row + offA, atB = row + offB;
-          const uint32_t fromA = atA < last4 ? atA : last4, fromB = atB < last4 ? atB : last4;
-          const uint32_t wa = __builtin_amdgcn_raw_buffer_load_b32(rs, fromA, 0, 0);
-          const uint32_t wb = __builtin_amdgcn_raw_buffer_load_b32(rs, fromB, 0, 0);
-          wd[i] = __builtin_amdgcn_perm(wb, wa, sel + (atA - fromA) * maskA + (atB - fromB) * maskB);
-        } else {
-          wd[i] = __builtin_amdgcn_raw_buffer_load_b32(rs, row + offA, 0, 0);
-        }
-      }
-#pragma unroll
-      for (int i = 0; i < BATCH; ++i)
-        if (c0 + TPG * i < p.C)
-          *reinterpret_cast<uint32_t*>(slot + (c0 - cs + TPG * i) * BP) = wd[i];
-    }
-  }
-  const EpiScalars es = epi_scalars(p.epi);
-  stat_barrier();                            // the slab is in LDS
-  PLANE_STAMP(1);
-
-  // fragment addresses (see the kernel above): every wave reads the whole slab
-  const int G = lane >> 4, s16 = lane & 15;
-  const int crow = 16 * (G >> 1) + (s16 >> 1);
-  int a_frag[MI];
-#pragma unroll
-  for (int mi = 0; mi < MI; ++mi) {
-    const int pc = 2 * mi + (G & 1);
-    a_frag[mi] = crow * BP + ((pc ^ plane_swz<CHP>(crow)) << 4) + 8 * (s16 & 1);
-  }
-  const int frow = lane & 31, fgrp = lane >> 5;
-  const int rb = wave * 32 + frow;
-  int fb0[KS];
-#pragma unroll
-  for (int ks = 0; ks < KS; ++ks) fb0[ks] = rb * CH + ((ks * 2 + fgrp) ^ swz<CH>(rb));
-
-  // where this lane's four pixels of a staged row go
-  const int px4 = (lane % LPR) * 4, r0 = lane / LPR;
-  const bool wide = (p.P & 3) == 0 && (reinterpret_cast<uintptr_t>(p.epi.out32) & 15u) == 0;
-  int* t32 = reinterpret_cast<int*>(lds + A_BYTES + RING) + wave * (CHB * LP);
-  size_t wbase = 0;      // wide: offset of (image, channel 0, pixel) of the lane's four pixels
-  bool wok = false;
-  size_t nbase[MI];      // narrow: the same for the lane's pixel of MFMA tile mi
-  bool nok[MI];
-  if (wide) {
-    const int v = p0 + px4, img = v / p.P;
-    wok = v < p.V;
-    wbase = static_cast<size_t>(img) * p.O * p.P + (v - img * p.P);
-  } else {
-#pragma unroll
-    for (int mi = 0; mi < MI; ++mi) {
-      const int v = p0 + 32 * mi + frow, img = v / p.P;
-      nok[mi] = v < p.V;
-      nbase[mi] = static_cast<size_t>(img) * p.O * p.P + (v - img * p.P);
-    }
-  }
-
-  int s = 0;
-  for (int t = 0; t < n_ot; ++t) {
-    const int o0 = (ot0 + t) * BO;
-    if (ctid < BO) sbias[t & 1][ctid] = (o0 + ctid < p.O) ? epi_bias32(p.epi, es, o0 + ctid) : 0;
-    v16i acc[MI];
-#pragma unroll
-    for (int mi = 0; mi < MI; ++mi)
-#pragma unroll
-      for (int v = 0; v < 16; ++v) acc[mi][v] = 0;
-    for (int kt = 0; kt < KT; ++kt, ++s) {
-      stat_barrier();
-      const char* sa = lds + kt * BK * BP;
-      const v4i* sbw = reinterpret_cast<const v4i*>(lds + A_BYTES + (s % NS) * kStatStage);
-#pragma unroll
-      for (int ks = 0; ks < KS; ++ks) {
-        const v4i fb = sbw[fb0[ks]];
-#pragma unroll
-        for (int mi = 0; mi < MI; ++mi) {
-          const v2i lo = lds_read_tr8(sa + a_frag[mi] + (32 * ks) * BP);
-          const v2i hi = lds_read_tr8(sa + a_frag[mi] + (32 * ks + 8) * BP);
-          const v4i fa = v4i{lo.x, lo.y, hi.x, hi.y};
-          acc[mi] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fb, fa, acc[mi], 0, 0, 0);
-        }
-      }
-    }
-    if (t == 0) PLANE_STAMP(2);
-    // epilogue of channel tile t: lane = pixel, registers = channels 8 (v / 4) + 4 (lane / 32)
-    // + v % 4 of the wave's 32
-    const int* bias = sbias[t & 1] + wave * 32;
-    if (wide) {
-#pragma unroll
-      for (int part = 0; part < 32 / CHB; ++part) {
-#pragma unroll
-        for (int vq = 0; vq < 4; ++vq) {
-          if ((8 * vq) / CHB != part) continue;
-          const v4i b = *reinterpret_cast<const v4i*>(bias + 8 * vq + 4 * fgrp);
-#pragma unroll
-          for (int i = 0; i < 4; ++i)
-#pragma unroll
-            for (int mi = 0; mi < MI; ++mi)
-              t32[((8 * vq) % CHB + 4 * fgrp + i) * LP + 32 * mi + frow] =
-                  static_cast<int>(static_cast<uint32_t>(acc[mi][4 * vq + i]) +
-                                   static_cast<uint32_t>(b[i]));
-        }
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-        __builtin_amdgcn_wave_barrier();
-        v4i back[CHB / RPI];
-#pragma unroll
-        for (int it = 0; it < CHB / RPI; ++it)
-          back[it] = *reinterpret_cast<const v4i*>(t32 + (it * RPI + r0) * LP + px4);
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-        __builtin_amdgcn_wave_barrier();
-#pragma unroll
-        for (int it = 0; it < CHB / RPI; ++it) {
-          const int o = o0 + wave * 32 + part * CHB + it * RPI + r0;
-          if (wok && o < p.O)
-            *reinterpret_cast<v4i*>(p.epi.out32 + wbase + static_cast<size_t>(o) * p.P) = back[it];
-        }
-      }
-    } else {
-#pragma unroll
-      for (int vq = 0; vq < 4; ++vq) {
-        const v4i b = *reinterpret_cast<const v4i*>(bias + 8 * vq + 4 * fgrp);
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const int o = o0 + wave * 32 + 8 * vq + 4 * fgrp + i;
-          if (o < p.O) {
-            int32_t* plane = p.epi.out32 + static_cast<size_t>(o) * p.P;
-#pragma unroll
-            for (int mi = 0; mi < MI; ++mi)
-              if (nok[mi])
-                plane[nbase[mi]] = static_cast<int>(static_cast<uint32_t>(acc[mi][4 * vq + i]) +
-                                                    static_cast<uint32_t>(b[i]));
-          }
-        }
-      }
-    }
-  }
-  PLANE_STAMP(3);
-}
-
 // ---- pre-pass for gathered operands that would need byte loads --------------------------
 // out[c][n * pitch + oh * OW + ow] = in[n][c][oh * sh][ow * sw]: the pixels a 1 x 1
 // convolution without padding reads, as one row of `row_stride` bytes per channel over the
@@ -911,13 +569,6 @@ typedef PlaneCfg<64, 64, 64, 2, 2> PlaneS;     // 4 waves, wave tile 32 x 32
 typedef PlaneCfg<128, 256, 64, 2, 4> PlaneW;   // 8 waves, wave tile 64 x 64
 typedef PlaneCfg<256, 128, 64, 4, 2> PlaneH;   // 8 waves, wave tile 64 x 64
 typedef PlaneCfg<256, 256, 64, 2, 4> PlaneL;   // 8 waves, wave tile 128 x 64
-// longer stages for long reductions over few pixels
-typedef PlaneCfg<64, 64, 128, 2, 2> PlaneS2;
-typedef PlaneCfg<64, 64, 256, 2, 2> PlaneS4;
-typedef PlaneCfg<128, 128, 128, 2, 2> PlaneM2;
-typedef PlaneCfg<64, 128, 128, 2, 2> PlaneP64k2;
-typedef PlaneCfg<128, 64, 128, 2, 2> PlaneN64k2;
-typedef PlaneCfg<256, 128, 128, 4, 2> PlaneH2;
 
 template <class Cfg>
 void launch_planes(hipStream_t s, PlaneArgs a, int gm) {
@@ -945,99 +596,8 @@ void launch_planes(hipStream_t s, PlaneArgs a, int gm) {
   MXQ_LAUNCH_CHECK();
 }
 
-// ---- the stationary kernel's launcher ----------------------------------------------------
-struct StatGeometry {
-  int mode;        // StatMode
-  int RL, rows, row_pitch;
-};
-
-// Which loader reads the pixels of an unpadded 1 x 1 convolution, or false if none does.
-bool stat_geometry(int H, int W, int OH, int OW, int sh, int sw, bool data_aligned,
-                   StatGeometry* g) {
-  if (sw != 1 && sw != 2) return false;
-  const bool whole = sh == 1 && sw == 1;   // then OH == H, OW == W: planes are read as they lie
-  g->RL = whole ? OH * OW : OW;
-  g->rows = whole ? 1 : OH;
-  g->row_pitch = whole ? 0 : sh * W;
-  if (g->RL < 4) return false;             // four pixels may then span more than two rows
-  const bool two = g->RL % 4 != 0;
-  if (whole && data_aligned && (OH * OW) % 16 == 0)
-    g->mode = kStatDma;
-  else if (sw == 1)
-    g->mode = two ? kStatS1Two : kStatS1;
-  else
-    g->mode = two ? kStatS2Two : kStatS2;
-  return true;
-}
-
-// LDS of a group: slab + ring + staging rows (8 or 16 channels x (BP + 8) dwords per wave)
-inline size_t stat_lds_bytes(int cpad, int bp) {
-  const int chb = bp == 128 ? 8 : 16;
-  return static_cast<size_t>(cpad) * bp + kStatNS * kStatStage + 4 * chb * (bp + 8) * 4;
-}
-
-template <int BP, int MODE>
-void launch_stationary_kernel(hipStream_t s, const StatArgs& a, dim3 grid, size_t lds_bytes) {
-  // more than 64 KiB of dynamic LDS has to be allowed once per kernel (a host-side setting,
-  // not a stream operation)
-  static bool allowed = false;
-  if (!allowed) {
-    MXQ_HIP(hipFuncSetAttribute(
-        reinterpret_cast<const void*>(&conv1x1_stationary_kernel<BP, MODE>),
-        hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 2048));
-    allowed = true;
-  }
-  hipLaunchKernelGGL((conv1x1_stationary_kernel<BP, MODE>), grid, dim3(kStatThreads), lds_bytes, s,
-                     a);
-  MXQ_LAUNCH_CHECK();
-}
-
-template <int BP>
-void launch_stationary_mode(hipStream_t s, const StatArgs& a, int mode, dim3 grid, size_t lds) {
-  switch (mode) {
-    case kStatDma: launch_stationary_kernel<BP, kStatDma>(s, a, grid, lds); break;
-    case kStatS1: launch_stationary_kernel<BP, kStatS1>(s, a, grid, lds); break;
-    case kStatS1Two: launch_stationary_kernel<BP, kStatS1Two>(s, a, grid, lds); break;
-    case kStatS2: launch_stationary_kernel<BP, kStatS2>(s, a, grid, lds); break;
-    default: launch_stationary_kernel<BP, kStatS2Two>(s, a, grid, lds); break;
-  }
-}
-
-// Largest reduction the slab of BP pixels has room for.
-constexpr int kStatMaxSlab = 64 * 1024;
-inline int stat_padded_c(int C) { return (C + kStatBK - 1) / kStatBK * kStatBK; }
-
-// bp: 128 or 64 pixels per group, 0 = choose; o_groups: 0 = choose
-void launch_stationary(hipStream_t s, StatArgs a, int mode, int bp, int o_groups) {
-  const int cpad = stat_padded_c(a.C);
-  a.tiles_o = (a.O + kStatBO - 1) / kStatBO;
-  const long cus = num_cus();
-  if (bp == 0) bp = cpad * 128 <= 32 * 1024 ? 128 : 64;
-  MXQ_CHECK((bp == 128 || bp == 64) && cpad * bp <= kStatMaxSlab, "slab does not fit");
-  a.tiles_p = (a.V + bp - 1) / bp;
-  const int slots_per_cu = static_cast<int>((160 * 1024) / (stat_lds_bytes(cpad, bp) + 1024));
-  if (o_groups == 0) {
-    // enough groups to give every slot of the chip one, and no more: each extra channel
-    // group fetches the slab again
-    o_groups = 1;
-    while (o_groups < a.tiles_o && 1LL * a.tiles_p * o_groups < cus * slots_per_cu) o_groups *= 2;
-  }
-  if (o_groups > a.tiles_o) o_groups = a.tiles_o;
-  a.ot_per_group = (a.tiles_o + o_groups - 1) / o_groups;
-  a.o_groups = (a.tiles_o + a.ot_per_group - 1) / a.ot_per_group;
-  const long long total = 1LL * a.tiles_p * a.o_groups;
-  MXQ_CHECK(total < (1LL << 31), "grid too large");
-  const dim3 grid(static_cast<unsigned>(total));
-  const size_t lds = stat_lds_bytes(cpad, bp);
-  if (bp == 128)
-    launch_stationary_mode<128>(s, a, mode, grid, lds);
-  else
-    launch_stationary_mode<64>(s, a, mode, grid, lds);
-}
-
 // The route a convolution takes.
 enum class Route {
-  kStationary,    // unpadded 1 x 1 over at most 1024 channels: the activation-stationary kernel
   kPlanes,        // 1 x 1, unit stride, 16 | plane: the NCHW kernel on the operator's own tensors
   kPlanesGather,  // any other unpadded 1 x 1: the same kernel, its loader gathering the pixels
                   // the layer reads
@@ -1057,7 +617,6 @@ struct NchwPlan {
   int off_h, off_w, H2, W2, K2h, K2w, pad2_h, pad2_w;
   // NHWC view of the adapter routes
   int vC;
-  StatGeometry stat;       // kStationary
   int gather_mode;         // kPlanesGather: how the loader fetches a group's four pixels
   int pitch, row_stride;   // kPlanesPrepass: columns per image and bytes per channel row
   bool weight_in_place;    // 1 x 1 window over C % 16 == 0 channels: OIHW is OHWI already
@@ -1065,7 +624,7 @@ struct NchwPlan {
 };
 
 NchwPlan plan_nchw(int N, int C, int H, int W, int O, int KH, int KW, int sh, int sw, int ph,
-                   int pw, int dh, int dw, bool operands_aligned, bool stationary = true) {
+                   int pw, int dh, int dw, bool operands_aligned) {
   MXQ_CHECK(N >= 0 && C > 0 && H > 0 && W > 0 && O > 0 && KH > 0 && KW > 0, "bad shape");
   MXQ_CHECK(sh > 0 && sw > 0 && dh > 0 && dw > 0 && ph >= 0 && pw >= 0, "bad stride/dilate/pad");
   const int eh = dh * (KH - 1) + 1, ew = dw * (KW - 1) + 1;
@@ -1077,14 +636,6 @@ NchwPlan plan_nchw(int N, int C, int H, int W, int O, int KH, int KW, int sh, in
   const bool one = KH == 1 && KW == 1 && ph == 0 && pw == 0;
   const bool small = 1LL * N * C * P < (1LL << 31) && 1LL * O * C < (1LL << 31) &&
                      1LL * N * C * H * W < (1LL << 31);
-  // (the stationary kernel reads the data with unaligned loads unless it takes whole chunks;
-  // only its weights need the 16-byte marks, which `operands_aligned` promises)
-  if (stationary && one && operands_aligned && C % 16 == 0 && small &&
-      1LL * N * P + 128 < (1LL << 31) && stat_padded_c(C) * 64 <= kStatMaxSlab &&
-      stat_geometry(H, W, pl.OH, pl.OW, sh, sw, true, &pl.stat)) {
-    pl.route = Route::kStationary;
-    return pl;
-  }
   if (one && operands_aligned && C % 16 == 0 && small) {
     if (sh == 1 && sw == 1 && P % 16 == 0) {
       pl.route = Route::kPlanes;
@@ -1180,17 +731,13 @@ void conv_nchw(void* stream, const int8_t* data, const int8_t* weight, const int
                                         nullptr, nullptr, nullptr, 0, 0.f, 0.f, nullptr, 0));
     return;
   }
-  // cfg 1 pins the adapter route; 2 and 71 ... 89 the tiled NCHW kernel (2: its own choice of
-  // tile); 91 / 92 (+ 100 x channel groups) the stationary kernel with 128 / 64 pixels a group
+  // cfg 1 pins the adapter route; 71.. pin a tile of the NCHW kernel
   const bool aligned = aligned16(data) && aligned16(weight) && cfg != 1;
-  const int scfg = cfg % 100;
-  const bool want_stationary = cfg == 0 || scfg == 91 || scfg == 92;
-  NchwPlan pl = plan_nchw(N, C, H, W, O, KH, KW, sh, sw, ph, pw, dh, dw, aligned, want_stationary);
+  NchwPlan pl = plan_nchw(N, C, H, W, O, KH, KW, sh, sw, ph, pw, dh, dw, aligned);
   const bool planes_route = pl.route == Route::kPlanes || pl.route == Route::kPlanesGather ||
                             pl.route == Route::kPlanesPrepass;
-  MXQ_CHECK(cfg < 70 || planes_route || pl.route == Route::kStationary,
-            "shape does not qualify for the NCHW 1x1 kernels");
-  if (cfg == 2) cfg = 0;
+  MXQ_CHECK(cfg < 70 || planes_route,
+            "shape does not qualify for the NCHW 1x1 kernel");
   hipStream_t s = static_cast<hipStream_t>(stream);
   char* ws = static_cast<char*>(workspace);
   const size_t need = pl.d_bytes + pl.w_bytes;
@@ -1198,27 +745,6 @@ void conv_nchw(void* stream, const int8_t* data, const int8_t* weight, const int
             "workspace too small: " << workspace_bytes << " < " << need
                                     << " (see mxq_quantized_conv_nchw_workspace)");
 
-  if (pl.route == Route::kStationary) {
-    StatArgs a = {};
-    a.data = data;
-    a.weight = weight;
-    a.N = N; a.C = C; a.P = pl.OH * pl.OW; a.O = O;
-    a.V = N * a.P;
-    a.plane_in = H * W;
-    a.RL = pl.stat.RL; a.rows = pl.stat.rows; a.row_pitch = pl.stat.row_pitch;
-    a.data_bytes = static_cast<uint32_t>(N) * C * H * W;
-    Epilogue& e = a.epi;
-    e = Epilogue();
-    e.bias = bias;
-    e.min_data = min_data; e.max_data = max_data;
-    e.min_weight = min_weight; e.max_weight = max_weight;
-    e.min_bias = min_bias; e.max_bias = max_bias;
-    e.out32 = out32;
-    e.omin = omin; e.omax = omax;
-    launch_stationary(s, a, pl.stat.mode, scfg == 91 ? 128 : (scfg == 92 ? 64 : 0),
-                      cfg >= 100 ? cfg / 100 : 0);
-    return;
-  }
   if (planes_route) {
     PlaneArgs a = {};
     a.N = N; a.C = C; a.P = pl.OH * pl.OW; a.O = O;
@@ -1287,12 +813,6 @@ void conv_nchw(void* stream, const int8_t* data, const int8_t* weight, const int
       case 75: launch_planes<PlaneW>(s, a, gm); break;
       case 77: launch_planes<PlaneH>(s, a, gm); break;
       case 78: launch_planes<PlaneL>(s, a, gm); break;
-      case 81: launch_planes<PlaneS2>(s, a, gm); break;
-      case 82: launch_planes<PlaneS4>(s, a, gm); break;
-      case 83: launch_planes<PlaneM2>(s, a, gm); break;
-      case 84: launch_planes<PlaneP64k2>(s, a, gm); break;
-      case 85: launch_planes<PlaneN64k2>(s, a, gm); break;
-      case 86: launch_planes<PlaneH2>(s, a, gm); break;
       default: MXQ_CHECK(false, "unknown NCHW tile configuration " << pick);
     }
     return;
