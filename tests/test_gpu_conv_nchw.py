@@ -129,6 +129,17 @@ def test_conv_nchw_other_geometries(capi, case, use_bias):
     run(capi, case, use_bias)
 
 
+# 3 x 3 over 64 -> 64 channels with enough rows for every wave of the chip (N * OH >= 8 per
+# CU): behind the adapters the parked-weights kernel writes the int32 planes itself, one or
+# two output rows per item, rows longer than one MFMA tile, an odd last row
+@pytest.mark.parametrize("case", [(74, 64, 28, 8, 64, 3, 3, 1, 1, 1), (90, 64, 28, 8, 64, 3, 3, 1, 1, 1),
+                                  (100, 64, 21, 33, 64, 3, 3, 1, 1, 1),
+                                  (120, 64, 21, 33, 64, 3, 3, 1, 1, 1)])
+@pytest.mark.parametrize("use_bias", [False, True])
+def test_conv_nchw_3x3_64_channels_many_rows(capi, case, use_bias):
+    run(capi, case, use_bias)
+
+
 @pytest.mark.parametrize("case", [PLANE_CASES[0], PLANE_CASES[3], STRIDED_CASES[0]])
 def test_conv_nchw_routes_agree(capi, case):
     """The NCHW kernel and the adapter route (pinned through the test-only entry point)
