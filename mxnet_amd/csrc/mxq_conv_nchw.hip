@@ -63,6 +63,7 @@ struct PlaneArgs {
   int H, W, OW, sh, sw;         // gathered: input plane, output row length, strides
   uint32_t data_bytes;   // extent of the activation tensor
   int tiles_p, tiles_o;  // pixel tiles (per image if native, per matrix if gathered), channel tiles
+  int stream32;          // the int32 planes leave with non-temporal stores
   Epilogue epi;          // bias, input ranges, out32 ([N][O][P]), omin / omax
 };
 
@@ -350,8 +351,9 @@ __global__ __launch_bounds__(Cfg::kThreads, 2) void conv1x1_planes_kernel(PlaneA
     // store instruction writes runs of 4 * TP bytes of 256 / TP channel planes instead of two
     // runs of 128 bytes (measured on store-only kernels of this shape: 2.9 -> 4.8 TB/s for
     // 14 x 14 planes, 4.2 -> 5.0 for 28 x 28).  A group of four pixels never straddles two
-    // images because 4 | P.  The stores are plain ones: with the non-temporal hint that pays
-    // for the int8 tiles of the NHWC kernels, the 19 ResNet-50 layers through this entry
+    // images because 4 | P.  The stores are plain ones except for the very largest outputs
+    // (`stream32`, set by the launcher): with the non-temporal hint that pays for the int8
+    // tiles of the NHWC kernels on every layer, the 19 ResNet-50 layers through this entry
     // point took 517.8 us instead of 500.0 (same box, same command).
     constexpr int TP = Cfg::TP, LP = TP + 8;   // row pitch in dwords: lanes 32-63 write four
                                                // rows further down, 32 banks away
@@ -394,11 +396,21 @@ __global__ __launch_bounds__(Cfg::kThreads, 2) void conv1x1_planes_kernel(PlaneA
           back[it] = *reinterpret_cast<const v4i*>(t32 + (it * RPI + r0) * LP + px4);
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
         __builtin_amdgcn_wave_barrier();
+        if (p.stream32) {
 #pragma unroll
-        for (int it = 0; it < CHB / RPI; ++it) {
-          const int o = o0 + wo * Cfg::TO + ni * 32 + part * CHB + it * RPI + r0;
-          if (ok && o < p.O)
-            *reinterpret_cast<v4i*>(obase + static_cast<size_t>(o) * p.P) = back[it];
+          for (int it = 0; it < CHB / RPI; ++it) {
+            const int o = o0 + wo * Cfg::TO + ni * 32 + part * CHB + it * RPI + r0;
+            if (ok && o < p.O)
+              __builtin_nontemporal_store(
+                  back[it], reinterpret_cast<v4i*>(obase + static_cast<size_t>(o) * p.P));
+          }
+        } else {
+#pragma unroll
+          for (int it = 0; it < CHB / RPI; ++it) {
+            const int o = o0 + wo * Cfg::TO + ni * 32 + part * CHB + it * RPI + r0;
+            if (ok && o < p.O)
+              *reinterpret_cast<v4i*>(obase + static_cast<size_t>(o) * p.P) = back[it];
+          }
         }
       }
     }
@@ -777,6 +789,11 @@ void conv_nchw(void* stream, const int8_t* data, const int8_t* weight, const int
     e.min_bias = min_bias; e.max_bias = max_bias;
     e.out32 = out32;
     e.omin = omin; e.omax = omax;
+    // Non-temporal stores only for an output of large planes that no cache level will hold
+    // (56 x 56, 64 -> 256 at batch 64: 205 MB, the pass 2.5 us shorter); on every other
+    // ResNet-50 layer the hint measured level or behind inside the pass (+0.1 ... +10 us,
+    // worst on 14 x 14 and 28 x 28 planes)
+    a.stream32 = (a.P >= 2048 && 4LL * N * O * a.P >= (128LL << 20)) ? 1 : 0;
     int pick = cfg;
     if (pick < 70) {
       const long cus = num_cus();
