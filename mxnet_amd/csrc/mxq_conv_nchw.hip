@@ -511,7 +511,8 @@ __global__ __launch_bounds__(256) void gather_planes_kernel(GatherArgs a) {
       to[u] = a.out + static_cast<size_t>(c) * a.row_stride + static_cast<size_t>(n) * a.pitch +
               4 * dd;
       const int p4 = ok[u] ? 4 * dd : 0;
-      int oh = static_cast<int>(__umulhi(static_cast<uint32_t>(p4), a.ow_magic));
+      // (rows of one pixel: ceil(2^32 / 1) does not fit the magic's 32 bits)
+      int oh = a.OW == 1 ? p4 : static_cast<int>(__umulhi(static_cast<uint32_t>(p4), a.ow_magic));
       int ow = p4 - oh * a.OW;
       uint32_t bytes[4];
 #pragma unroll

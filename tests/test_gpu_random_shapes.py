@@ -146,3 +146,50 @@ def test_conv_random_geometry(capi, case):
     np.testing.assert_array_equal(capi.nhwc_to_nchw(res["out8"]).cpu().numpy(), rq)
     assert (res["omin"].item(), res["omax"].item()) == (rmn, rmx)
     assert (res["rmin"].item(), res["rmax"].item()) == (qmn, qmx)
+
+
+def conv_nchw_cases():
+    """Mostly unpadded 1 x 1 layers (the routes of the NCHW kernel: whole planes, the
+    gathering loaders, the pre-pass), planes of every residue mod 16, strides 1-3 alone and
+    mixed, batches large enough for pixel tiles to run across several images; a few padded
+    and 3 x 3 geometries for the adapters behind the same call."""
+    rng = np.random.default_rng(2024)
+    cases = []
+    while len(cases) < 56:
+        one = rng.random() < 0.8
+        N = int(rng.choice([1, 2, 3, 5, 17, 40]))
+        C = int(rng.choice([16, 32, 48, 64, 80, 128, 272, 512, 20]))
+        H = int(rng.integers(1, 30))
+        W = int(rng.integers(1, 30))
+        O = int(rng.choice([8, 24, 64, 72, 128, 136, 264]))
+        KH, KW = (1, 1) if one else (int(rng.choice([1, 3])), int(rng.choice([1, 3])))
+        sh, sw = int(rng.choice([1, 1, 2, 2, 3])), int(rng.choice([1, 1, 2, 2, 3]))
+        p = 0 if one else int(rng.integers(0, 2))
+        if H + 2 * p < KH or W + 2 * p < KW or N * C * H * W > (3 << 20):
+            continue
+        cases.append((N, C, H, W, O, KH, KW, sh, sw, p))
+    return cases
+
+
+@pytest.mark.parametrize("case", conv_nchw_cases())
+def test_conv_nchw_random_geometry(capi, case):
+    N, C, H, W, O, KH, KW, sh, sw, p = case
+    d = int8_uniform((N, C, H, W), seed=C + H * 3 + W)
+    w = int8_uniform((O, C, KH, KW), seed=O + KH + 11)
+    b = int8_uniform((O,), seed=O + 1) if (N + C + O + H) % 2 else None
+    ro, rmn, rmx = oracle.quantized_conv(d, w, b, -2.0, 2.0, -0.5, 0.5,
+                                         None if b is None else -1.0,
+                                         None if b is None else 1.0, (sh, sw), (p, p), (1, 1))
+    res = capi.quantized_conv_nchw(dev(d), dev(w), None if b is None else dev(b), f32(-2.0),
+                                   f32(2.0), f32(-0.5), f32(0.5),
+                                   None if b is None else f32(-1.0),
+                                   None if b is None else f32(1.0), stride=(sh, sw), pad=(p, p))
+    np.testing.assert_array_equal(res["out32"].cpu().numpy(), ro)
+    assert (res["omin"].item(), res["omax"].item()) == (rmn, rmx)
+    # the route through the layout adapters writes the same tensor
+    alt = capi.quantized_conv_nchw(dev(d), dev(w), None if b is None else dev(b), f32(-2.0),
+                                   f32(2.0), f32(-0.5), f32(0.5),
+                                   None if b is None else f32(-1.0),
+                                   None if b is None else f32(1.0), stride=(sh, sw), pad=(p, p),
+                                   cfg=1)
+    assert torch.equal(res["out32"], alt["out32"])
