@@ -134,3 +134,76 @@ def test_replays_follow_their_inputs():
         assert (fs[2].item(), fs[3].item()) == (smn, smx)
         # the program's own eager work between replays
         (x * 2.0).sum().item()
+
+
+def test_conv_nchw_replays_follow_their_inputs():
+    """mxq_quantized_conv_nchw under capture, one call per route that passes data between the
+    launches of a call: the NCHW kernel alone (whole planes), its gathering loader, the
+    pre-pass into the workspace, and the layout adapters (two operand copies in the
+    workspace).  Replayed on new data and new weights."""
+    import mxnet_amd
+    lib = mxnet_amd._lib.lib
+    # (N, C, H, W, O, K, stride, pad)
+    cases = [(3, 64, 8, 12, 72, 1, 1, 0),       # whole planes of 96 pixels
+             (3, 64, 16, 24, 72, 1, 2, 0),      # stride 2 over rows of 12: the loader gathers
+             (4, 1024, 14, 14, 512, 1, 2, 0),   # 14 -> 7: the pre-pass
+             (2, 32, 9, 11, 40, 3, 1, 1)]       # 3 x 3: the adapters
+    one = [torch.tensor([v], device="cuda") for v in (-1.0, 1.0)]
+    slots = []
+    for (N, C, H, W, O, K, s, p) in cases:
+        OH, OW = (H + 2 * p - K) // s + 1, (W + 2 * p - K) // s + 1
+        geo = (N, C, H, W, O, K, K, s, s, p, p, 1, 1)
+        nws = lib.mxq_quantized_conv_nchw_workspace(*geo, 1)
+        slots.append(dict(
+            geo=geo, d=torch.empty((N, C, H, W), dtype=torch.int8, device="cuda"),
+            w=torch.empty((O, C, K, K), dtype=torch.int8, device="cuda"),
+            b=torch.from_numpy(int8_uniform((O,), seed=O)).cuda(),
+            out=torch.empty((N, O, OH, OW), dtype=torch.int32, device="cuda"),
+            r=[scalar(), scalar()], nws=nws,
+            ws=torch.empty(max(nws, 16), dtype=torch.uint8, device="cuda")))
+    assert slots[0]["nws"] == 0 and slots[1]["nws"] == 0 and slots[2]["nws"] > 0 and slots[3]["nws"] > 0
+
+    def body():
+        st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+        for k in slots:
+            rc = lib.mxq_quantized_conv_nchw(st, P(k["d"]), P(k["w"]), P(k["b"]), *k["geo"],
+                                             P(one[0]), P(one[1]), P(one[0]), P(one[1]),
+                                             P(one[0]), P(one[1]), P(k["out"]), P(k["r"][0]),
+                                             P(k["r"][1]), P(k["ws"]) if k["nws"] else None,
+                                             k["nws"])
+            assert rc == 0, lib.mxq_last_error().decode()
+
+    def load(seed):
+        for i, k in enumerate(slots):
+            k["d_np"] = int8_uniform(tuple(k["d"].shape), seed=seed + 10 * i)
+            k["w_np"] = int8_uniform(tuple(k["w"].shape), seed=seed + 10 * i + 1)
+            k["d"].copy_(torch.from_numpy(k["d_np"]))
+            k["w"].copy_(torch.from_numpy(k["w_np"]))
+
+    def check():
+        torch.cuda.synchronize()
+        for k in slots:
+            g = k["geo"]
+            ro, rmn, rmx = oracle.quantized_conv(k["d_np"], k["w_np"], k["b"].cpu().numpy(), -1.0,
+                                                 1.0, -1.0, 1.0, -1.0, 1.0, (g[7], g[8]),
+                                                 (g[9], g[10]), (1, 1))
+            np.testing.assert_array_equal(k["out"].cpu().numpy(), ro)
+            assert (k["r"][0].item(), k["r"][1].item()) == (rmn, rmx)
+
+    load(1)
+    body()                       # eager: also the warm-up a capture needs
+    check()
+    graph = torch.cuda.CUDAGraph()
+    stream = torch.cuda.Stream()
+    with torch.cuda.stream(stream):
+        body()
+        torch.cuda.synchronize()
+        with torch.cuda.graph(graph, stream=stream):
+            body()
+    for seed in (100, 200, 300):
+        load(seed)
+        for k in slots:          # nothing left over from the last replay may pass as a result
+            k["out"].fill_(-1)
+        torch.cuda.synchronize()
+        graph.replay()
+        check()
