@@ -187,3 +187,43 @@ def test_conv_nchw_without_images(capi):
                                         0.5)
     assert tuple(res["out32"].shape) == (0, 32, 8, 8)
     assert (res["omin"].item(), res["omax"].item()) == (rmn, rmx)
+
+
+def test_conv_nchw_refuses_what_it_cannot_run(capi):
+    """Error behaviour of the entry point: a workspace smaller than the query's answer, a
+    missing range pointer, a window larger than the padded input; the output stays
+    untouched."""
+    import ctypes
+    import mxnet_amd
+    lib = mxnet_amd._lib.lib
+    P = lambda t: ctypes.c_void_p(t.data_ptr()) if t is not None else None
+    N, C, H, W, O = 2, 32, 9, 11, 40
+    d = dev(int8_uniform((N, C, H, W), seed=1))
+    w = dev(int8_uniform((O, C, 3, 3), seed=2))
+    out = torch.full((N, O, H, W), 7, dtype=torch.int32, device="cuda")
+    r = [f32(0.0), f32(0.0)]
+    one = [f32(-1.0), f32(1.0)]
+    geo = (N, C, H, W, O, 3, 3, 1, 1, 1, 1, 1, 1)
+    need = lib.mxq_quantized_conv_nchw_workspace(*geo, 1)
+    assert need > 0
+    ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+    st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+    def call(geo, ranges, ws_ptr, ws_bytes):
+        return lib.mxq_quantized_conv_nchw(st, P(d), P(w), None, *geo, *ranges, None, None, P(out),
+                                           P(r[0]), P(r[1]), ws_ptr, ws_bytes)
+
+    ok_ranges = (P(one[0]), P(one[1]), P(one[0]), P(one[1]))
+    assert call(geo, ok_ranges, P(ws), need - 16) != 0
+    assert b"workspace too small" in lib.mxq_last_error()
+    assert call(geo, ok_ranges, None, 0) != 0
+    assert call(geo, (None, P(one[1]), P(one[0]), P(one[1])), P(ws), need) != 0
+    assert b"range pointer" in lib.mxq_last_error()
+    big = (N, C, H, W, O, 13, 3, 1, 1, 1, 1, 1, 1)       # 13 rows over 9 + 2
+    assert call(big, ok_ranges, P(ws), need) != 0
+    assert b"kernel larger than padded input" in lib.mxq_last_error()
+    torch.cuda.synchronize()
+    assert bool((out == 7).all())
+    assert call(geo, ok_ranges, P(ws), need) == 0        # and the same call with its workspace runs
+    torch.cuda.synchronize()
+    assert not bool((out == 7).all())
