@@ -514,3 +514,38 @@ def test_fc_residual_sum_in_place(capi, M, K, N):
                                    P(rs), P(out[0]), P(out[1]), P(out[2]), P(out[3]), -R, R, -R,
                                    1.2 * R, 1, None, 0))
     np.testing.assert_array_equal(rs.cpu().numpy(), ref)
+
+
+# Exact ties and saturation in the fused requantize: ranges chosen so that every scale is a
+# power of two (data and weight range 127 -> one product level = 1.0; calibrated range 254 ->
+# requantize scale 0.5), accumulators that sweep the small integers of both signs.  Odd
+# accumulators land exactly on k + 0.5 (rounded away from zero by the reference,
+# quantization_utils.h:80-96), |acc| >= 255 saturates at 127, and with the relu every negative
+# value has to come out as 0 -- through the tiled kernels, the short-K streaming kernel and
+# the register-staged fallback.
+@pytest.mark.parametrize("M,K,N", [(256, 16, 64), (300, 64, 128), (512, 256, 256), (64, 20, 24)])
+@pytest.mark.parametrize("relu", [False, True])
+def test_fc_fused_requantize_on_exact_ties(capi, M, K, N, relu):
+    d = np.zeros((M, K), np.int8)
+    w = np.zeros((N, K), np.int8)
+    m, n = np.arange(M), np.arange(N)
+    d[:, 0] = (m * 37) % 256 - 128       # every residue within 256 rows, both signs within 8
+    d[:, 1] = (m * 7) % 5 - 2
+    d[:, 2] = 2
+    w[:, 0] = 1
+    w[:, 1] = (n % 64) - 32
+    w[:, 2] = 127 * (n % 3 - 1)
+    ro, rmn, rmx = oracle.quantized_fully_connected(d, w, None, -127.0, 127.0, -127.0, 127.0)
+    assert ro.min() < -300 and ro.max() > 300 and (ro % 2 != 0).sum() > ro.size // 4
+    rq, qmn, qmx = oracle.requantize(ro, rmn, rmx, -254.0, 254.0)
+    # the scale really is 0.5: the oracle's answer is round-half-away-from-zero of acc / 2
+    want = np.clip(np.sign(ro) * np.floor(np.abs(ro) / 2.0 + 0.5), -127, 127).astype(np.int8)
+    np.testing.assert_array_equal(rq, want)
+    if relu:
+        rq = oracle.relu_i8(rq)
+    for want_int32 in (True, False):
+        res = capi.quantized_fc(dev(d), dev(w), None, f32(-127.0), f32(127.0), f32(-127.0),
+                                f32(127.0), want_int32=want_int32, calib=(-254.0, 254.0),
+                                relu=relu)
+        np.testing.assert_array_equal(res["out8"].cpu().numpy(), rq)
+        assert (res["rmin"].item(), res["rmax"].item()) == (qmn, qmx)
