@@ -340,3 +340,36 @@ def test_conv_without_images_still_writes_its_range(capi):
                                         0.5, pad=(1, 1))
     assert tuple(res["out32"].shape) == (0, 8, 8, 32)
     assert (res["omin"].item(), res["omax"].item()) == (rmn, rmx)
+
+
+# Exact ties and saturation in the fused requantize of the convolution kernels (see the FC
+# test of the same name): power-of-two scales, a centre-tap-only 3 x 3 window so that the
+# accumulators sweep the small integers of both signs; the tiled kernel, the parked-weights
+# kernel and the resident-patch kernel, each with and without the relu.
+@pytest.mark.parametrize("C,O,force", [(64, 64, None), (64, 64, (61, 1)), (128, 128, (62, 1)),
+                                       (32, 48, None)])
+@pytest.mark.parametrize("relu", [False, True])
+def test_conv_fused_requantize_on_exact_ties(capi, C, O, force, relu):
+    N, H, W = 3, 12, 28
+    d = np.zeros((N, C, H, W), np.int8)
+    w = np.zeros((O, C, 3, 3), np.int8)
+    px = np.arange(N * H * W).reshape(N, H, W)
+    o = np.arange(O)
+    d[:, 0] = (px * 37) % 256 - 128
+    d[:, 1] = (px * 7) % 5 - 2
+    d[:, 2] = 2
+    w[:, 0, 1, 1] = 1
+    w[:, 1, 1, 1] = (o % 64) - 32
+    w[:, 2, 1, 1] = 127 * (o % 3 - 1)
+    ro, rmn, rmx = oracle.quantized_conv(d, w, None, -127.0, 127.0, -127.0, 127.0, None, None,
+                                         (1, 1), (1, 1), (1, 1))
+    assert ro.min() < -255 and ro.max() > 255 and (ro % 2 != 0).sum() > ro.size // 4
+    rq, qmn, qmx = oracle.requantize(ro, rmn, rmx, -254.0, 254.0)
+    want = np.clip(np.sign(ro) * np.floor(np.abs(ro) / 2.0 + 0.5), -127, 127).astype(np.int8)
+    np.testing.assert_array_equal(rq, want)
+    if relu:
+        rq = oracle.relu_i8(rq)
+    res = run_conv_nchw(capi, d, w, None, 127.0, 127.0, 1.0, (1, 1), (1, 1), (1, 1),
+                        calib=(-254.0, 254.0), relu=relu, force=force, want_int32=False)
+    np.testing.assert_array_equal(res["out8_nchw"].cpu().numpy(), rq)
+    assert (res["rmin"].item(), res["rmax"].item()) == (qmn, qmx)
