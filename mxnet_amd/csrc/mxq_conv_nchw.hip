@@ -86,7 +86,7 @@ struct PlaneCfg {
   static_assert(BP % (32 * WP) == 0 && BO % (32 * WO) == 0, "wave tile");
   static_assert(A_SLOTS % (64 * NW) == 0 && B_SLOTS % (64 * NW) == 0, "loader");
   static_assert(CHP == 4 || CHP == 8 || CHP == 16, "pixel-chunk swizzle");
-  static_assert(CH == 4 || CH == 8, "fragment addressing of the weight operand");
+  static_assert(CH == 4 || CH == 8 || CH == 16, "fragment addressing of the weight operand");
   static_assert(kThreads % GROUPS == 0 && BK % TPG == 0 && TPG % 8 == 0,
                 "gathering loader: a thread's channels share their low three bits");
 };
@@ -584,6 +584,10 @@ typedef PlaneCfg<64, 64, 64, 2, 2> PlaneS;     // 4 waves, wave tile 32 x 32
 typedef PlaneCfg<128, 256, 64, 2, 4> PlaneW;   // 8 waves, wave tile 64 x 64
 typedef PlaneCfg<256, 128, 64, 4, 2> PlaneH;   // 8 waves, wave tile 64 x 64
 typedef PlaneCfg<256, 256, 64, 2, 4> PlaneL;   // 8 waves, wave tile 128 x 64
+// 128-byte stages: half as many K steps.  Measured inside the ResNet-50 pass on every
+// gathered and every small-plane layer in five tile shapes: ahead only for the loader-gathered
+// 1024 -> 256 layer at 14 x 14 (-2.2 us), level or behind elsewhere (+0.3 ... +9.4 us).
+typedef PlaneCfg<64, 128, 128, 2, 2> PlaneP64k2;
 
 template <class Cfg>
 void launch_planes(hipStream_t s, PlaneArgs a, int gm) {
@@ -823,6 +827,8 @@ void conv_nchw(void* stream, const int8_t* data, const int8_t* weight, const int
         if (tiles(bp, bo) < cus) bp = 64;
         if (tiles(bp, bo) < cus) bo = 64;
         pick = bp == 128 ? 71 : (bo == 128 ? 73 : 74);
+        // a long reduction through the gathering loader: 128-byte stages halve its K steps
+        if (pick == 73 && gm == kGatherDword && C >= 1024) pick = 84;
       }
     }
     switch (pick) {
@@ -833,6 +839,7 @@ void conv_nchw(void* stream, const int8_t* data, const int8_t* weight, const int
       case 75: launch_planes<PlaneW>(s, a, gm); break;
       case 77: launch_planes<PlaneH>(s, a, gm); break;
       case 78: launch_planes<PlaneL>(s, a, gm); break;
+      case 84: launch_planes<PlaneP64k2>(s, a, gm); break;
       default: MXQ_CHECK(false, "unknown NCHW tile configuration " << pick);
     }
     return;
@@ -910,7 +917,7 @@ int mxq_dbg_read_plane_stamps(long long* host, int count) {
 
 #ifdef MXQ_TEST_HOOKS
 // Test-only twin (declared in tests/mxq_test_hooks.h): cfg 1 pins the route through the
-// layout adapters, 71 ... 78 a tile of the NCHW kernel, 0 leaves the choice to the launcher.
+// layout adapters, 71 ... 84 a tile of the NCHW kernel, 0 leaves the choice to the launcher.
 int mxq_test_quantized_conv_nchw(void* stream, const int8_t* data, const int8_t* weight,
                                  const int8_t* bias, int N, int C, int H, int W, int O, int KH,
                                  int KW, int stride_h, int stride_w, int pad_h, int pad_w,

@@ -65,7 +65,7 @@ int mxq_test_quantized_conv_nhwc(void* stream, const int8_t* data, const int8_t*
                                  size_t workspace_bytes, int cfg, int splits);
 
 /* mxq_quantized_conv_nchw with its route pinned: cfg 1 = through the layout adapters,
- * 71 ... 78 = a tile of the NCHW 1x1 kernel (mxq_conv_nchw.hip lists them), 0 = choose. */
+ * 71 ... 84 = a tile of the NCHW 1x1 kernel (mxq_conv_nchw.hip lists them), 0 = choose. */
 int mxq_test_quantized_conv_nchw(void* stream, const int8_t* data, const int8_t* weight,
                                  const int8_t* bias, int N, int C, int H, int W, int O, int KH,
                                  int KW, int stride_h, int stride_w, int pad_h, int pad_w,

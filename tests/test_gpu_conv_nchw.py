@@ -70,7 +70,7 @@ def test_conv_nchw_planes(capi, case, use_bias):
     assert res["workspace_bytes"] == 0  # nothing is copied for a unit-stride 1x1 layer
 
 
-@pytest.mark.parametrize("cfg", [71, 72, 73, 74, 75, 77, 78])
+@pytest.mark.parametrize("cfg", [71, 72, 73, 74, 75, 77, 78, 84])
 @pytest.mark.parametrize("case", [PLANE_CASES[2], PLANE_CASES[3], PLANE_CASES[5], PLANE_CASES[7],
                                   (3, 320, 7, 7, 200, 1, 1, 1, 0, 1),
                                   (2, 1024, 14, 14, 136, 1, 1, 1, 0, 1)])
