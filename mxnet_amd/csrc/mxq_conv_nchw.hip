@@ -18,16 +18,19 @@
 // writes two 128-byte runs of two channel planes: the int32 output goes to its NCHW place
 // straight from the accumulators.  No adapter launch, no second copy of any tensor.
 //
-// Strided 1 x 1 convolutions, and planes whose size is no multiple of 16 bytes (14 x 14,
-// 7 x 7), run in the same kernel with a gathering loader: a thread fetches the four pixels
-// of its LDS dword from wherever the stride puts them (one 8-byte load and a v_perm for
-// stride 2 over rows of 4 | OW pixels, the plane's own dwords for unit stride, bytes
-// otherwise) and the operand becomes the matrix [C][N * OH * OW] whose pixel tiles run
-// across image boundaries.  No workspace, no pre-pass: a strided layer reads only the
-// cache lines it uses.  Where that loader would have to fetch single bytes (odd rows, 7 x 7
-// planes) a pre-pass gathers the pixels into one row per channel in the caller's workspace
-// first and the kernel reads that with its 16-byte loads.  Everything else (3 x 3, padded
-// 1 x 1, C % 16 != 0) takes the NHWC kernels of mxq_conv.hip behind the layout adapters.
+// Unit-stride planes of 4 | P bytes that are no multiple of 16 (14 x 14) take the same direct
+// loads: 16 bytes from a dword mark, over columns padded to a multiple of 16 per image (a
+// plane's last piece runs into the next channel's first pixels; those columns are never
+// stored) and pixel tiles that run across image boundaries.  Strided 1 x 1 convolutions run
+// in the same kernel with a gathering loader: a thread fetches the four pixels of its LDS
+// dword from wherever the stride puts them (one 8-byte load and a v_perm for stride 2 over
+// rows of 4 | OW pixels, two dwords for 2 | OW, bytes otherwise) and the operand becomes the
+// matrix [C][N * OH * OW].  No workspace, no pre-pass: a strided layer reads only the cache
+// lines it uses.  Where that loader would have to fetch single bytes (odd rows, 7 x 7
+// planes), and for strided layers with a large weight matrix, a pre-pass gathers the pixels
+// into one row per channel in the caller's workspace first and the kernel reads that with
+// its 16-byte loads.  Everything else (3 x 3, padded 1 x 1, C % 16 != 0) takes the NHWC
+// kernels of mxq_conv.hip behind the layout adapters.
 #include <hip/hip_runtime.h>
 
 #include <cmath>
@@ -57,9 +60,13 @@ struct PlaneArgs {
   const int8_t* weight;  // [O][C]
   int N, C, P, O;        // P = output pixels per image
   int img_stride, row_stride;   // native
-  int pitch;             // native, 0: pixel tiles inside one image.  > 0: a pre-gathered
-                         // operand (gather_planes_kernel), one row per channel over the whole
-                         // batch with image n's P pixels at columns n * pitch ...; img_stride 0
+  int pitch;             // native, 0: pixel tiles inside one image.  > 0 (a multiple of 16):
+                         // pixel tiles over the columns of the whole batch, image n's P pixels
+                         // at columns n * pitch ... -- either a pre-gathered operand
+                         // (gather_planes_kernel: one row per channel, img_stride == pitch) or
+                         // the tensor itself read in 16-byte pieces from dword marks (planes of
+                         // 4 | P bytes: img_stride = C * P, row_stride = P; a plane's last piece
+                         // runs into the next channel's pixels, whose columns are never stored)
   int H, W, OW, sh, sw;         // gathered: input plane, output row length, strides
   uint32_t data_bytes;   // extent of the activation tensor
   int tiles_p, tiles_o;  // pixel tiles (per image if native, per matrix if gathered), channel tiles
@@ -112,7 +119,8 @@ __device__ __forceinline__ v2i lds_read_tr8(const char* p) {
 
 // How a gathered operand's four pixels of a group are fetched.
 constexpr int kNative = 0;      // not gathered: 16-byte direct-to-LDS loads
-constexpr int kGatherDword = 1; // unit stride, planes on dword marks: the plane's own dwords
+// (1 was a dword-gathering loader for unit-stride planes of 4 | P bytes; the direct loads read
+// those now)
 constexpr int kGatherPair = 2;  // sw == 2, 4 | OW, rows on 8-byte marks: 8 bytes and a v_perm
 constexpr int kGatherBytes = 3; // anything else: byte by byte
 constexpr int kGatherPair2 = 4; // sw == 2, 2 | OW, rows on dword marks: two dwords (two pixels
@@ -175,8 +183,16 @@ __global__ __launch_bounds__(Cfg::kThreads, 2) void conv1x1_planes_kernel(PlaneA
       const int q = (j * NW + wave) * 64 + lane;
       const int c = q / CHP, pc = (q % CHP) ^ plane_swz<CHP>(c);
       a_c[j] = c;
-      a_off[j] = static_cast<uint32_t>(n) * p.img_stride +
-                 static_cast<uint32_t>(c) * p.row_stride + p0 + pc * 16;
+      if (p.pitch != 0) {
+        // columns over the whole batch, `pitch` (a multiple of 16) per image: the chunk's image
+        const int v = p0 + pc * 16, img = v / p.pitch;
+        a_off[j] = img < p.N ? static_cast<uint32_t>(img) * p.img_stride + (v - img * p.pitch) +
+                                   static_cast<uint32_t>(c) * p.row_stride
+                             : kOutOfRange;
+      } else {
+        a_off[j] = static_cast<uint32_t>(n) * p.img_stride +
+                   static_cast<uint32_t>(c) * p.row_stride + p0 + pc * 16;
+      }
     }
   }
   RowIssuerBuffer<Cfg, BI> bi;
@@ -220,9 +236,7 @@ __global__ __launch_bounds__(Cfg::kThreads, 2) void conv1x1_planes_kernel(PlaneA
         int c = stage * BK + cs + TPG * i;
         c = c < p.C ? c : p.C - 1;   // the weights' zero K tail cancels whatever these rows hold
         const int8_t* row = p.data + static_cast<size_t>(c) * plane_in;
-        if (GM == kGatherDword) {
-          areg[i] = *reinterpret_cast<const uint32_t*>(row + goff[0]);
-        } else if (GM == kGatherPair) {
+        if (GM == kGatherPair) {
           typedef uint32_t u2 __attribute__((ext_vector_type(2)));
           const u2 w = *reinterpret_cast<const u2*>(row + goff[0]);
           areg[i] = __builtin_amdgcn_perm(w.y, w.x, 0x06040200u);
@@ -598,9 +612,7 @@ void launch_planes(hipStream_t s, PlaneArgs a, int gm) {
   const long long total = 1LL * (flat ? 1 : a.N) * a.tiles_p * a.tiles_o;
   MXQ_CHECK(total < (1LL << 31), "grid too large");
   const dim3 grid(static_cast<unsigned>(total)), block(Cfg::kThreads);
-  if (gm == kGatherDword) {
-    hipLaunchKernelGGL((conv1x1_planes_kernel<Cfg, 2, kGatherDword>), grid, block, 0, s, a);
-  } else if (gm == kGatherPair) {
+  if (gm == kGatherPair) {
     hipLaunchKernelGGL((conv1x1_planes_kernel<Cfg, 2, kGatherPair>), grid, block, 0, s, a);
   } else if (gm == kGatherBytes) {
     hipLaunchKernelGGL((conv1x1_planes_kernel<Cfg, 2, kGatherBytes>), grid, block, 0, s, a);
@@ -660,6 +672,14 @@ NchwPlan plan_nchw(int N, int C, int H, int W, int O, int KH, int KW, int sh, in
       pl.route = Route::kPlanes;
       return pl;
     }
+    // planes of 4 | P bytes (14 x 14): the same direct loads, 16 bytes from dword marks, over
+    // columns padded to a multiple of 16 per image
+    if (sh == 1 && sw == 1 && P % 4 == 0 &&
+        1LL * N * ((P + 15) / 16 * 16) < (1LL << 31)) {
+      pl.route = Route::kPlanes;
+      pl.pitch = static_cast<int>((P + 15) / 16 * 16);
+      return pl;
+    }
     // The gathering loader works one stage ahead out of registers; the pre-pass costs a launch
     // and a copy of what the layer reads but feeds the kernel's direct-to-LDS ring.  Measured
     // on the ResNet-50 layers at batch 64: the loader wins while the weight matrix is small
@@ -670,9 +690,7 @@ NchwPlan plan_nchw(int N, int C, int H, int W, int O, int KH, int KW, int sh, in
     const bool prepass_ok = P < kGatherMaxPlane && 1LL * C * row < (1LL << 31);
     const bool light = 1LL * O * C <= 256 * 1024 || !prepass_ok;
     int mode = kGatherBytes;
-    if (sh == 1 && sw == 1 && plane_in % 4 == 0)
-      mode = kGatherDword;
-    else if (sw == 2 && pl.OW % 4 == 0 && (sh * W) % 8 == 0 && plane_in % 8 == 0 && 2 * pl.OW <= W)
+    if (sw == 2 && pl.OW % 4 == 0 && (sh * W) % 8 == 0 && plane_in % 8 == 0 && 2 * pl.OW <= W)
       mode = kGatherPair;
     else if (sw == 2 && pl.OW % 2 == 0 && (sh * W) % 4 == 0 && plane_in % 4 == 0 && 2 * pl.OW <= W)
       mode = kGatherPair2;
@@ -778,13 +796,14 @@ void conv_nchw(void* stream, const int8_t* data, const int8_t* weight, const int
       launch_gather(s, data, reinterpret_cast<int8_t*>(ws), N, C, H, W, pl.OH, pl.OW, sh, sw,
                     pl.pitch, pl.row_stride);
       a.data = reinterpret_cast<const int8_t*>(ws);
-      a.img_stride = 0;
+      a.img_stride = pl.pitch;
       a.row_stride = pl.row_stride;
       a.pitch = pl.pitch;
       a.data_bytes = static_cast<uint32_t>(C) * pl.row_stride;
     } else {
       a.img_stride = C * a.P;
       a.row_stride = a.P;
+      a.pitch = pl.pitch;   // 0: whole 16-byte planes, tiles inside an image
     }
     Epilogue& e = a.epi;
     e = Epilogue();
@@ -827,8 +846,9 @@ void conv_nchw(void* stream, const int8_t* data, const int8_t* weight, const int
         if (tiles(bp, bo) < cus) bp = 64;
         if (tiles(bp, bo) < cus) bo = 64;
         pick = bp == 128 ? 71 : (bo == 128 ? 73 : 74);
-        // a long reduction through the gathering loader: 128-byte stages halve its K steps
-        if (pick == 73 && gm == kGatherDword && C >= 1024) pick = 84;
+        // a long reduction over 14 x 14 planes: 128-byte stages halve its K steps (-2.2 us
+        // inside the ResNet-50 pass)
+        if (pick == 73 && C >= 1024 && pl.route == Route::kPlanes && a.pitch != 0) pick = 84;
       }
     }
     switch (pick) {
