@@ -251,10 +251,9 @@ __global__ __launch_bounds__(Cfg::kThreads, NS <= 2 ? Cfg::kMinWaves : 1) void c
 // (2 x 2) MFMAs out of LDS, adds the bias, requantizes and stores the row; the int8 tile is
 // transposed through the patch row that has just become dead.  No barrier per K step,
 // every input row is fetched (R + 2) / R times instead of nine, and with two waves per SIMD
-// one wave's fetch and epilogue overlap the other's MFMAs.  Two output forms: int8 with the
-// fused requantize (what the quantized graph runs with a calibrated convolution), and the
-// operator's own int32 channel planes (PLANES32), stored from the accumulators; everything
-// else takes the tiled kernels.
+// one wave's fetch and epilogue overlap the other's MFMAs.  int8 output with the fused
+// requantize only (the form the quantized graph runs with a calibrated convolution);
+// everything else takes the tiled kernels.
 constexpr int kRowsC = 64;        // input channels = bytes per pixel
 constexpr int kRowsO = 64;        // output channels
 constexpr int kRowsPitch = 60;    // patch pixels per row
@@ -265,7 +264,7 @@ constexpr int kRowsWaves = 8;
 // pitch 64 bytes) over the banks for the column-wise writes and the row-wise reads alike
 __device__ __forceinline__ int tile_swz(int row) { return (row ^ (row >> 2)) & 3; }
 
-template <int R, bool PLANES32>
+template <int R>
 __global__ __launch_bounds__(64 * kRowsWaves, 1) void conv3x3_rows_kernel(ConvArgs p) {
   constexpr int CH = kRowsC / 16;                       // 16-byte chunks per pixel
   constexpr int kPatchPixels = (R + 2) * kRowsPitch;
@@ -376,28 +375,6 @@ __global__ __launch_bounds__(64 * kRowsWaves, 1) void conv3x3_rows_kernel(ConvAr
                 acc[mi][ni] =
                     __builtin_amdgcn_mfma_i32_32x32x32_i8(fb[ni], fa[mi], acc[mi][ni], 0, 0, 0);
           }
-      if constexpr (PLANES32) {
-        // the operator's own output: int32 channel planes [n][o][oh][ow].  A lane holds one
-        // pixel, its registers channels, so a store instruction writes up to 32 consecutive
-        // pixels of one row of two channel planes (planes of 56 x 56 take any store shape at
-        // the same rate)
-        int32_t* orow32 = p.epi.out32 + (static_cast<size_t>(n) * kRowsO * p.OH + oh0 + r) * p.OW;
-        const size_t plane = static_cast<size_t>(p.OH) * p.OW;
-#pragma unroll
-        for (int ni = 0; ni < 2; ++ni)
-#pragma unroll
-          for (int vq = 0; vq < 4; ++vq)
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-              const int o = ni * 32 + 8 * vq + 4 * lgrp + i;
-#pragma unroll
-              for (int mi = 0; mi < 2; ++mi) {
-                const int px = mi * 32 + lrow;
-                if (px < p.OW) orow32[o * plane + px] = acc[mi][ni][4 * vq + i];
-              }
-            }
-        continue;
-      }
       // patch row r is dead now (output row r + 1 starts at patch row r + 1): the int8 tile
       // of up to 58 pixels x 64 channels is transposed through it, 64 bytes per pixel
       char* stage = reinterpret_cast<char*>(patch + r * kRowsPitch * CH);
@@ -454,19 +431,12 @@ __global__ __launch_bounds__(64 * kRowsWaves, 1) void conv3x3_rows_kernel(ConvAr
   if (blockIdx.x == 0 && threadIdx.x == 0) epilogue_ranges(p.epi);
 }
 
-// the int32 form: channel planes only (the operator's NCHW output), nothing fused
-bool conv3x3_rows_planes32(const ConvArgs& a) {
-  return a.epi.out32 != nullptr && a.epi.out8 == nullptr && a.epi.outf == nullptr &&
-         a.epi.res == nullptr && a.epi.plane == a.OH * a.OW && a.epi.plane > 0;
-}
-
 bool conv3x3_rows_ok(const ConvArgs& a) {
   const long long data_bytes = static_cast<long long>(a.N) * a.H * a.W * a.C;
   return a.KH == 3 && a.KW == 3 && a.sh == 1 && a.sw == 1 && a.ph == 1 && a.pw == 1 &&
          a.dh == 1 && a.dw == 1 && a.C == kRowsC && a.O == kRowsO && a.W <= kRowsMaxW &&
-         aligned16(a.data) && aligned16(a.weight) && data_bytes < (1LL << 31) &&
-         ((a.epi.out32 == nullptr && a.epi.out8 != nullptr && aligned16(a.epi.out8)) ||
-          conv3x3_rows_planes32(a));
+         a.epi.out32 == nullptr && a.epi.out8 != nullptr && aligned16(a.data) &&
+         aligned16(a.weight) && aligned16(a.epi.out8) && data_bytes < (1LL << 31);
 }
 
 void launch_conv3x3_rows(hipStream_t s, const ConvArgs& a) {
@@ -478,18 +448,12 @@ void launch_conv3x3_rows(hipStream_t s, const ConvArgs& a) {
   const long items = two ? items2 : static_cast<long>(a.N) * a.OH;
   long grid = (items + kRowsWaves - 1) / kRowsWaves;
   if (grid > cus) grid = cus;
-  const dim3 g(static_cast<unsigned>(grid)), b(64 * kRowsWaves);
-  if (conv3x3_rows_planes32(a)) {
-    if (two)
-      hipLaunchKernelGGL((conv3x3_rows_kernel<2, true>), g, b, 0, s, a);
-    else
-      hipLaunchKernelGGL((conv3x3_rows_kernel<1, true>), g, b, 0, s, a);
-  } else {
-    if (two)
-      hipLaunchKernelGGL((conv3x3_rows_kernel<2, false>), g, b, 0, s, a);
-    else
-      hipLaunchKernelGGL((conv3x3_rows_kernel<1, false>), g, b, 0, s, a);
-  }
+  if (two)
+    hipLaunchKernelGGL(conv3x3_rows_kernel<2>, dim3(static_cast<unsigned>(grid)),
+                       dim3(64 * kRowsWaves), 0, s, a);
+  else
+    hipLaunchKernelGGL(conv3x3_rows_kernel<1>, dim3(static_cast<unsigned>(grid)),
+                       dim3(64 * kRowsWaves), 0, s, a);
   MXQ_LAUNCH_CHECK();
 }
 

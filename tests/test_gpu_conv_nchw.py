@@ -129,9 +129,9 @@ def test_conv_nchw_other_geometries(capi, case, use_bias):
     run(capi, case, use_bias)
 
 
-# 3 x 3 over 64 -> 64 channels with enough rows for every wave of the chip (N * OH >= 8 per
-# CU): behind the adapters the parked-weights kernel writes the int32 planes itself, one or
-# two output rows per item, rows longer than one MFMA tile, an odd last row
+# 3 x 3 over 64 -> 64 channels with many rows behind the adapters (more than 8192 output
+# pixels: int32 planes from the tiled kernel's many tiles), rows longer than one MFMA tile,
+# an odd last row
 @pytest.mark.parametrize("case", [(74, 64, 28, 8, 64, 3, 3, 1, 1, 1), (90, 64, 28, 8, 64, 3, 3, 1, 1, 1),
                                   (100, 64, 21, 33, 64, 3, 3, 1, 1, 1),
                                   (120, 64, 21, 33, 64, 3, 3, 1, 1, 1)])
